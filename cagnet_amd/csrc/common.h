@@ -1,0 +1,79 @@
+// Shared host/device helpers of libcagnet_amd (gfx950 only: 64-wide wavefronts).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+#include "../../include/cagnet_amd.h"
+
+namespace cg {
+
+constexpr int kWave = 64;
+
+// ---- error plumbing -----------------------------------------------------------------------
+void set_error(const char *fmt, ...);
+int hip_fail(hipError_t e, const char *what, const char *file, int line);
+
+#define CG_HIP(call)                                                        \
+  do {                                                                      \
+    hipError_t e_ = (call);                                                 \
+    if (e_ != hipSuccess) return cg::hip_fail(e_, #call, __FILE__, __LINE__); \
+  } while (0)
+
+#define CG_TRY(call)              \
+  do {                            \
+    int s_ = (call);              \
+    if (s_ != CG_OK) return s_;   \
+  } while (0)
+
+#define CG_FAIL(code, ...)        \
+  do {                            \
+    cg::set_error(__VA_ARGS__);   \
+    return (code);                \
+  } while (0)
+
+// Launch check: kernel launches report configuration errors through hipGetLastError.
+#define CG_LAUNCH_CHECK() CG_HIP(hipGetLastError())
+
+// ---- per (device, stream) grow-only scratch ------------------------------------------------
+// slot: independent buffers that must be alive at the same time use different slots.
+enum ScratchSlot { kSlotA = 0, kSlotB = 1, kSlotC = 2, kSlotD = 3, kNumSlots = 4 };
+int scratch_get(hipStream_t stream, int slot, size_t bytes, void **out);
+
+// ---- integer helpers ------------------------------------------------------------------------
+static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+static inline int bits_for(int32_t count) {  // number of bits needed to represent values in [0, count)
+  int b = 0;
+  uint32_t v = count > 1 ? (uint32_t)(count - 1) : 0u;
+  while (v) { ++b; v >>= 1; }
+  return b;
+}
+
+// ---- device-side scan / sort building blocks (scan.hip, sort.hip) ----------------------------
+// Exclusive prefix sum of d_in[0..count) into d_out (may alias d_in); if d_total != nullptr the
+// grand total is stored there.  Values and totals must fit uint32.
+int exclusive_scan_u32(const uint32_t *d_in, uint32_t *d_out, int64_t count, uint32_t *d_total, hipStream_t stream);
+
+// Stable LSD radix sort of `count` records (key_a, key_b, payload) by the low `bits` bits of
+// the array selected per pass: first all digits of key_b (minor key), then those of key_a
+// (major key).  Arrays are ping-ponged between buffer set 0 and 1; returns which set holds the
+// result in *result_set.  Either bit count may be 0 (that key is then not sorted on).
+struct SortBuffers {
+  int32_t *key_a[2];
+  int32_t *key_b[2];
+  int32_t *payload[2];
+};
+int radix_sort_pairs(SortBuffers &buf, int64_t count, int bits_a, int bits_b, int *result_set, hipStream_t stream);
+
+// coo2csr.hip
+int launch_rowptr(const int32_t *d_row, int64_t nnz, int32_t n, int32_t *d_rowptr, hipStream_t stream);
+int coo_check(const int32_t *d_row, const int32_t *d_col, int64_t nnz, int32_t n, int32_t m, int require_sorted,
+              hipStream_t stream);
+int coo2csr_general(const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz, int32_t n,
+                    int32_t m, int32_t *d_rowptr, int32_t *d_colind, float *d_values, int32_t *d_perm,
+                    hipStream_t stream);
+int csr_transpose(const int32_t *d_rowptr, const int32_t *d_colind, const float *d_values, int64_t nnz, int32_t n,
+                  int32_t m, int32_t *d_colptr, int32_t *d_rowind, float *d_values_t, int32_t *d_perm,
+                  hipStream_t stream);
+
+}  // namespace cg

@@ -1,0 +1,246 @@
+// COO -> CSR conversion, CSR transpose and input validation.
+//
+// Row compression replaces the cusparseXcoo2csr call of the reference operator
+// (sparse-extension/sparse_coo_tensor.cu:136-142).  The general path (unsorted input) and the
+// transpose are a stable radix sort followed by the same compression; the reference has neither
+// (its callers coalesce on the CPU, gcn_distr.py:546, and its backward assumes A == A^T,
+// gcn_distr.py:326).
+#include "common.h"
+
+namespace cg {
+
+constexpr int kThreads = 256;
+
+// One thread per boundary k in [0, nnz]: rows in (row[k-1], row[k]] start at position k.
+// Long runs of empty rows are filled by the whole wave instead of one lane.
+__global__ __launch_bounds__(kThreads) void rowptr_kernel(const int32_t *__restrict__ row, int64_t nnz, int32_t n,
+                                                          int32_t *__restrict__ rowptr) {
+  const int64_t k = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  const int lane = threadIdx.x & (kWave - 1);
+  int32_t lo = 1, hi = 0;
+  if (k <= nnz) {
+    int32_t prev = k == 0 ? -1 : row[k - 1];
+    int32_t cur = k == nnz ? n : row[k];
+    prev = prev < -1 ? -1 : (prev > n - 1 ? n - 1 : prev);  // clamp: bad input must not write outside rowptr
+    cur = cur < -1 ? -1 : (cur > n ? n : cur);
+    lo = prev + 1;
+    hi = cur;
+  }
+  const int32_t gap = hi - lo + 1;
+  if (gap > 0 && gap <= 8) {
+    for (int32_t i = lo; i <= hi; ++i) rowptr[i] = (int32_t)k;
+  }
+  uint64_t longs = __ballot(gap > 8);
+  while (longs) {
+    const int src = __builtin_ctzll(longs);
+    longs &= longs - 1;
+    const int32_t slo = __shfl(lo, src, kWave);
+    const int32_t shi = __shfl(hi, src, kWave);
+    const int32_t sk = (int32_t)__shfl((int32_t)k, src, kWave);
+    for (int32_t i = slo + lane; i <= shi; i += kWave) rowptr[i] = sk;
+  }
+}
+
+int launch_rowptr(const int32_t *d_row, int64_t nnz, int32_t n, int32_t *d_rowptr, hipStream_t stream) {
+  const int64_t blocks = ceil_div64(nnz + 1, kThreads);
+  rowptr_kernel<<<(unsigned)blocks, kThreads, 0, stream>>>(d_row, nnz, n, d_rowptr);
+  CG_LAUNCH_CHECK();
+  return CG_OK;
+}
+
+// flags: bit0 index out of range, bit1 rows descend, bit2 (row, col) not strictly ascending
+__global__ __launch_bounds__(kThreads) void coo_check_kernel(const int32_t *__restrict__ row,
+                                                             const int32_t *__restrict__ col, int64_t nnz, int32_t n,
+                                                             int32_t m, int *__restrict__ flags) {
+  const int64_t k = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  int f = 0;
+  if (k < nnz) {
+    const int32_t r = row[k];
+    const int32_t c = col ? col[k] : 0;
+    if (r < 0 || r >= n || c < 0 || c >= m) f |= 1;
+    if (k > 0) {
+      const int32_t pr = row[k - 1];
+      if (pr > r) f |= 2;
+      if (col && (pr > r || (pr == r && col[k - 1] >= c))) f |= 4;
+    }
+  }
+  if (f) atomicOr(flags, f);  // integer OR: order independent
+}
+
+__global__ __launch_bounds__(kThreads) void iota_kernel(int32_t *__restrict__ out, int64_t count) {
+  const int64_t k = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (k < count) out[k] = (int32_t)k;
+}
+
+__global__ __launch_bounds__(kThreads) void gather_f32_kernel(const float *__restrict__ src,
+                                                              const int32_t *__restrict__ perm,
+                                                              float *__restrict__ dst, int64_t count) {
+  const int64_t k = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (k < count) dst[k] = src[perm[k]];
+}
+
+// row index of every stored entry of a CSR matrix: one wave per row
+__global__ __launch_bounds__(kThreads) void csr_expand_rows_kernel(const int32_t *__restrict__ rowptr, int32_t n,
+                                                                   int32_t *__restrict__ row_out) {
+  const int64_t wave = ((int64_t)blockIdx.x * kThreads + threadIdx.x) / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  if (wave >= n) return;
+  const int32_t s = rowptr[wave], e = rowptr[wave + 1];
+  for (int32_t k = s + lane; k < e; k += kWave) row_out[k] = (int32_t)wave;
+}
+
+static int check_common(int64_t nnz, int32_t n, int32_t m) {
+  if (nnz < 0 || n < 0 || m < 0) CG_FAIL(CG_ERR_SIZE, "negative size: nnz=%lld n=%d m=%d", (long long)nnz, n, m);
+  if (nnz > 0x7fffffffLL - 1) CG_FAIL(CG_ERR_OVERFLOW, "nnz=%lld does not fit the int32 rowptr contract", (long long)nnz);
+  if (n == 0x7fffffff || m == 0x7fffffff) CG_FAIL(CG_ERR_OVERFLOW, "n + 1 overflows int32");
+  return CG_OK;
+}
+
+int coo_check(const int32_t *d_row, const int32_t *d_col, int64_t nnz, int32_t n, int32_t m, int require_sorted,
+              hipStream_t stream) {
+  if (nnz == 0) return CG_OK;
+  void *d_flags = nullptr;
+  CG_TRY(scratch_get(stream, kSlotD, sizeof(int), &d_flags));
+  CG_HIP(hipMemsetAsync(d_flags, 0, sizeof(int), stream));
+  coo_check_kernel<<<(unsigned)ceil_div64(nnz, kThreads), kThreads, 0, stream>>>(d_row, d_col, nnz, n, m,
+                                                                                 (int *)d_flags);
+  CG_LAUNCH_CHECK();
+  int flags = 0;
+  CG_HIP(hipMemcpyAsync(&flags, d_flags, sizeof(int), hipMemcpyDeviceToHost, stream));
+  CG_HIP(hipStreamSynchronize(stream));
+  if (flags & 1) CG_FAIL(CG_ERR_INDEX, "COO index outside [0,%d) x [0,%d)", n, m);
+  if (require_sorted >= 1 && (flags & 2)) CG_FAIL(CG_ERR_UNSORTED, "COO rows are not ascending");
+  if (require_sorted >= 2 && (flags & 4)) CG_FAIL(CG_ERR_UNSORTED, "COO (row, col) pairs are not strictly ascending");
+  return CG_OK;
+}
+
+struct DevFree {
+  void *p[8];
+  int count = 0;
+  ~DevFree() {
+    for (int i = 0; i < count; ++i)
+      if (p[i]) (void)hipFree(p[i]);
+  }
+  int alloc(void **out, size_t bytes) {
+    hipError_t e = hipMalloc(out, bytes ? bytes : 4);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      set_error("hipMalloc of %zu bytes failed: %s", bytes, hipGetErrorString(e));
+      return CG_ERR_ALLOC;
+    }
+    p[count++] = *out;
+    return CG_OK;
+  }
+};
+
+// Sort records (key_a major, key_b minor) carrying the input position; hand back the sorted
+// key arrays and the permutation in caller-owned outputs.
+int sort_coo(const int32_t *d_key_a, const int32_t *d_key_b, int64_t count, int bits_a, int bits_b,
+             int32_t *d_out_a, int32_t *d_out_b, int32_t *d_out_perm, hipStream_t stream) {
+  DevFree tmp;
+  SortBuffers buf;
+  const size_t bytes = (size_t)count * sizeof(int32_t);
+  for (int s = 0; s < 2; ++s) {
+    CG_TRY(tmp.alloc((void **)&buf.key_a[s], bytes));
+    CG_TRY(tmp.alloc((void **)&buf.key_b[s], bytes));
+    CG_TRY(tmp.alloc((void **)&buf.payload[s], bytes));
+  }
+  if (count > 0) {
+    CG_HIP(hipMemcpyAsync(buf.key_a[0], d_key_a, bytes, hipMemcpyDeviceToDevice, stream));
+    CG_HIP(hipMemcpyAsync(buf.key_b[0], d_key_b, bytes, hipMemcpyDeviceToDevice, stream));
+    iota_kernel<<<(unsigned)ceil_div64(count, kThreads), kThreads, 0, stream>>>(buf.payload[0], count);
+    CG_LAUNCH_CHECK();
+  }
+  int set = 0;
+  CG_TRY(radix_sort_pairs(buf, count, bits_a, bits_b, &set, stream));
+  if (count > 0) {
+    if (d_out_a) CG_HIP(hipMemcpyAsync(d_out_a, buf.key_a[set], bytes, hipMemcpyDeviceToDevice, stream));
+    if (d_out_b) CG_HIP(hipMemcpyAsync(d_out_b, buf.key_b[set], bytes, hipMemcpyDeviceToDevice, stream));
+    if (d_out_perm) CG_HIP(hipMemcpyAsync(d_out_perm, buf.payload[set], bytes, hipMemcpyDeviceToDevice, stream));
+  }
+  CG_HIP(hipStreamSynchronize(stream));  // the temporaries are freed when `tmp` goes out of scope
+  return CG_OK;
+}
+
+int coo2csr_general(const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz, int32_t n,
+                    int32_t m, int32_t *d_rowptr, int32_t *d_colind, float *d_values, int32_t *d_perm,
+                    hipStream_t stream) {
+  DevFree tmp;
+  int32_t *d_rows_sorted = nullptr, *d_perm_local = d_perm;
+  CG_TRY(tmp.alloc((void **)&d_rows_sorted, (size_t)nnz * sizeof(int32_t)));
+  if (!d_perm_local) CG_TRY(tmp.alloc((void **)&d_perm_local, (size_t)nnz * sizeof(int32_t)));
+  CG_TRY(sort_coo(d_row, d_col, nnz, bits_for(n), bits_for(m), d_rows_sorted, d_colind, d_perm_local, stream));
+  CG_TRY(launch_rowptr(d_rows_sorted, nnz, n, d_rowptr, stream));
+  if (d_val && d_values && nnz > 0) {
+    gather_f32_kernel<<<(unsigned)ceil_div64(nnz, kThreads), kThreads, 0, stream>>>(d_val, d_perm_local, d_values,
+                                                                                   nnz);
+    CG_LAUNCH_CHECK();
+  }
+  CG_HIP(hipStreamSynchronize(stream));
+  return CG_OK;
+}
+
+int csr_transpose(const int32_t *d_rowptr, const int32_t *d_colind, const float *d_values, int64_t nnz, int32_t n,
+                  int32_t m, int32_t *d_colptr, int32_t *d_rowind, float *d_values_t, int32_t *d_perm,
+                  hipStream_t stream) {
+  DevFree tmp;
+  int32_t *d_rows = nullptr, *d_cols_sorted = nullptr, *d_perm_local = d_perm;
+  CG_TRY(tmp.alloc((void **)&d_rows, (size_t)nnz * sizeof(int32_t)));
+  CG_TRY(tmp.alloc((void **)&d_cols_sorted, (size_t)nnz * sizeof(int32_t)));
+  if (!d_perm_local) CG_TRY(tmp.alloc((void **)&d_perm_local, (size_t)nnz * sizeof(int32_t)));
+  if (n > 0) {
+    csr_expand_rows_kernel<<<(unsigned)ceil_div64((int64_t)n * kWave, kThreads), kThreads, 0, stream>>>(d_rowptr, n,
+                                                                                                       d_rows);
+    CG_LAUNCH_CHECK();
+  }
+  // CSR order is (row, col) ascending, so a stable sort on col alone yields (col, row) order:
+  // major key = col (key_a), minor key = row with zero bits (already in place).
+  CG_TRY(sort_coo(d_colind, d_rows, nnz, bits_for(m), 0, d_cols_sorted, d_rowind, d_perm_local, stream));
+  CG_TRY(launch_rowptr(d_cols_sorted, nnz, m, d_colptr, stream));
+  if (d_values && d_values_t && nnz > 0) {
+    gather_f32_kernel<<<(unsigned)ceil_div64(nnz, kThreads), kThreads, 0, stream>>>(d_values, d_perm_local,
+                                                                                   d_values_t, nnz);
+    CG_LAUNCH_CHECK();
+  }
+  CG_HIP(hipStreamSynchronize(stream));
+  return CG_OK;
+}
+
+}  // namespace cg
+
+extern "C" {
+
+int cg_coo2csr_rowptr(const int32_t *d_row, int64_t nnz, int32_t n, int32_t *d_rowptr, cg_stream_t stream) {
+  CG_TRY(cg::check_common(nnz, n, 0));
+  if (!d_rowptr || (nnz > 0 && !d_row)) CG_FAIL(CG_ERR_NULL, "cg_coo2csr_rowptr: null pointer");
+  return cg::launch_rowptr(d_row, nnz, n, d_rowptr, (hipStream_t)stream);
+}
+
+int cg_coo_check(const int32_t *d_row, const int32_t *d_col, int64_t nnz, int32_t n, int32_t m, int require_sorted,
+                 cg_stream_t stream) {
+  CG_TRY(cg::check_common(nnz, n, m));
+  if (nnz > 0 && !d_row) CG_FAIL(CG_ERR_NULL, "cg_coo_check: null row pointer");
+  return cg::coo_check(d_row, d_col, nnz, n, m, require_sorted, (hipStream_t)stream);
+}
+
+int cg_coo2csr(const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz, int32_t n, int32_t m,
+               int32_t *d_rowptr, int32_t *d_colind, float *d_values, int32_t *d_perm, cg_stream_t stream) {
+  CG_TRY(cg::check_common(nnz, n, m));
+  if (!d_rowptr || (nnz > 0 && (!d_row || !d_col || !d_colind))) CG_FAIL(CG_ERR_NULL, "cg_coo2csr: null pointer");
+  if (d_val && !d_values) CG_FAIL(CG_ERR_NULL, "cg_coo2csr: values given but no output for them");
+  return cg::coo2csr_general(d_row, d_col, d_val, nnz, n, m, d_rowptr, d_colind, d_values, d_perm,
+                             (hipStream_t)stream);
+}
+
+int cg_csr_transpose(const int32_t *d_rowptr, const int32_t *d_colind, const float *d_values, int64_t nnz, int32_t n,
+                     int32_t m, int32_t *d_colptr, int32_t *d_rowind, float *d_values_t, int32_t *d_perm,
+                     cg_stream_t stream) {
+  CG_TRY(cg::check_common(nnz, n, m));
+  if (!d_rowptr || !d_colptr || (nnz > 0 && (!d_colind || !d_rowind)))
+    CG_FAIL(CG_ERR_NULL, "cg_csr_transpose: null pointer");
+  if (d_values && !d_values_t) CG_FAIL(CG_ERR_NULL, "cg_csr_transpose: values given but no output for them");
+  return cg::csr_transpose(d_rowptr, d_colind, d_values, nnz, n, m, d_colptr, d_rowind, d_values_t, d_perm,
+                           (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,246 @@
+// Device-wide primitives written for 64-wide wavefronts: exclusive scan (reduce-then-scan over
+// 2048-element tiles) and a stable LSD radix sort (8-bit digits, per-wave match ranking in LDS).
+// Both are integer-only and order-preserving, so results are run-to-run identical.
+#include "common.h"
+
+namespace cg {
+
+// ---------------------------------------------------------------------------------------------
+// scan
+// ---------------------------------------------------------------------------------------------
+constexpr int kScanThreads = 256;
+constexpr int kScanItems = 8;
+constexpr int kScanTile = kScanThreads * kScanItems;  // 2048
+
+__device__ inline uint32_t wave_inclusive_scan(uint32_t v, int lane) {
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    uint32_t t = __shfl_up(v, d, kWave);
+    if (lane >= d) v += t;
+  }
+  return v;
+}
+
+// Exclusive scan of one value per thread across a 256-thread block; *block_total gets the sum.
+__device__ inline uint32_t block_exclusive_scan(uint32_t v, uint32_t *block_total) {
+  __shared__ uint32_t wave_sum[kScanThreads / kWave];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  uint32_t incl = wave_inclusive_scan(v, lane);
+  if (lane == kWave - 1) wave_sum[wave] = incl;
+  __syncthreads();
+  uint32_t offset = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < kScanThreads / kWave; ++w) {
+    uint32_t s = wave_sum[w];
+    if (w < wave) offset += s;
+    total += s;
+  }
+  __syncthreads();
+  *block_total = total;
+  return offset + incl - v;
+}
+
+__global__ __launch_bounds__(kScanThreads) void scan_tile_sums_kernel(const uint32_t *__restrict__ in,
+                                                                      uint32_t *__restrict__ sums, int64_t count) {
+  const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
+  uint32_t s = 0;
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    int64_t idx = base + i;
+    if (idx < count) s += in[idx];
+  }
+  uint32_t total;
+  (void)block_exclusive_scan(s, &total);
+  if (threadIdx.x == 0) sums[blockIdx.x] = total;
+}
+
+// out[i] = offsets[tile] + exclusive prefix inside the tile.  in and out may alias: every thread
+// reads all of its own items before it writes them.
+__global__ __launch_bounds__(kScanThreads) void scan_tile_apply_kernel(const uint32_t *in, uint32_t *out,
+                                                                       const uint32_t *__restrict__ offsets,
+                                                                       int64_t count, uint32_t *total_out) {
+  const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
+  uint32_t item[kScanItems];
+  uint32_t s = 0;
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    int64_t idx = base + i;
+    item[i] = idx < count ? in[idx] : 0u;
+    s += item[i];
+  }
+  uint32_t total;
+  uint32_t run = block_exclusive_scan(s, &total);
+  run += offsets ? offsets[blockIdx.x] : 0u;
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    int64_t idx = base + i;
+    if (idx < count) out[idx] = run;
+    run += item[i];
+  }
+  if (total_out && blockIdx.x == gridDim.x - 1 && threadIdx.x == kScanThreads - 1) *total_out = run;
+}
+
+static int scan_level(const uint32_t *d_in, uint32_t *d_out, int64_t count, uint32_t *d_total, uint32_t *d_sums,
+                      hipStream_t stream) {
+  const int64_t tiles = ceil_div64(count, kScanTile);
+  if (tiles <= 1) {
+    scan_tile_apply_kernel<<<1, kScanThreads, 0, stream>>>(d_in, d_out, nullptr, count, d_total);
+    CG_LAUNCH_CHECK();
+    return CG_OK;
+  }
+  scan_tile_sums_kernel<<<(unsigned)tiles, kScanThreads, 0, stream>>>(d_in, d_sums, count);
+  CG_LAUNCH_CHECK();
+  // the tile sums are scanned in place; the next level's sums live right behind them
+  CG_TRY(scan_level(d_sums, d_sums, tiles, nullptr, d_sums + tiles, stream));
+  scan_tile_apply_kernel<<<(unsigned)tiles, kScanThreads, 0, stream>>>(d_in, d_out, d_sums, count, d_total);
+  CG_LAUNCH_CHECK();
+  return CG_OK;
+}
+
+int exclusive_scan_u32(const uint32_t *d_in, uint32_t *d_out, int64_t count, uint32_t *d_total, hipStream_t stream) {
+  if (count < 0) CG_FAIL(CG_ERR_SIZE, "scan: negative count");
+  if (count == 0) {
+    if (d_total) CG_HIP(hipMemsetAsync(d_total, 0, sizeof(uint32_t), stream));
+    return CG_OK;
+  }
+  if (ceil_div64(count, kScanTile) > 0x7fffffffLL) CG_FAIL(CG_ERR_OVERFLOW, "scan: too many tiles");
+  size_t sums = 0;
+  for (int64_t t = ceil_div64(count, kScanTile); t > 1; t = ceil_div64(t, kScanTile)) sums += (size_t)t;
+  sums += 1;
+  void *d_sums = nullptr;
+  CG_TRY(scratch_get(stream, kSlotD, sums * sizeof(uint32_t), &d_sums));
+  return scan_level(d_in, d_out, count, d_total, (uint32_t *)d_sums, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// radix sort
+// ---------------------------------------------------------------------------------------------
+constexpr int kSortThreads = 256;
+constexpr int kSortWaves = kSortThreads / kWave;         // 4
+constexpr int kSortRounds = 16;                          // keys per lane
+constexpr int kSortWaveTile = kSortRounds * kWave;       // 1024 consecutive keys per wave
+constexpr int kSortTile = kSortWaves * kSortWaveTile;    // 4096 keys per workgroup
+constexpr int kRadix = 256;
+
+// hist[digit * tiles + tile] = number of keys of this tile with that digit
+__global__ __launch_bounds__(kSortThreads) void radix_hist_kernel(const int32_t *__restrict__ key, int64_t count,
+                                                                  int shift, uint32_t *__restrict__ hist,
+                                                                  int64_t tiles) {
+  __shared__ uint32_t lh[kRadix];
+  lh[threadIdx.x] = 0;
+  __syncthreads();
+  const int64_t base = (int64_t)blockIdx.x * kSortTile;
+#pragma unroll
+  for (int i = 0; i < kSortTile / kSortThreads; ++i) {
+    int64_t idx = base + (int64_t)i * kSortThreads + threadIdx.x;
+    if (idx < count) {
+      uint32_t d = ((uint32_t)key[idx] >> shift) & (kRadix - 1);
+      atomicAdd(&lh[d], 1u);  // integer LDS atomic: the count does not depend on arrival order
+    }
+  }
+  __syncthreads();
+  hist[(int64_t)threadIdx.x * tiles + blockIdx.x] = lh[threadIdx.x];
+}
+
+// Stable scatter.  Wave w of a workgroup owns keys [tile + 1024 w, tile + 1024 (w+1)) and ranks
+// them 64 at a time: lanes holding equal digits find each other with 8 ballots, their rank is the
+// number of lower lanes in that peer set plus the wave's running count of the digit.
+__global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
+    const int32_t *__restrict__ key, int shift, const int32_t *__restrict__ in_a, const int32_t *__restrict__ in_b,
+    const int32_t *__restrict__ in_p, int32_t *__restrict__ out_a, int32_t *__restrict__ out_b,
+    int32_t *__restrict__ out_p, int64_t count, const uint32_t *__restrict__ scanned_hist, int64_t tiles) {
+  __shared__ uint32_t cnt[kSortWaves][kRadix];
+  for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) (&cnt[0][0])[i] = 0;
+  __syncthreads();
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const uint64_t lt_mask = (1ull << lane) - 1ull;
+  const int64_t base = (int64_t)blockIdx.x * kSortTile + (int64_t)wave * kSortWaveTile;
+
+  int32_t ra[kSortRounds], rb[kSortRounds], rp[kSortRounds];
+  uint32_t packed[kSortRounds];  // digit | local rank << 8
+
+#pragma unroll
+  for (int r = 0; r < kSortRounds; ++r) {
+    const int64_t idx = base + (int64_t)r * kWave + lane;
+    const bool valid = idx < count;
+    uint32_t d = 0;
+    if (valid) {
+      d = ((uint32_t)key[idx] >> shift) & (kRadix - 1);
+      ra[r] = in_a[idx];
+      rb[r] = in_b[idx];
+      rp[r] = in_p[idx];
+    }
+    uint64_t peers = __ballot(valid);
+#pragma unroll
+    for (int bit = 0; bit < 8; ++bit) {
+      const bool one = (d >> bit) & 1u;
+      const uint64_t bal = __ballot(one);
+      peers &= one ? bal : ~bal;
+    }
+    const uint32_t rank = (uint32_t)__popcll(peers & lt_mask);
+    uint32_t pre = 0;
+    if (valid) pre = cnt[wave][d];
+    // the peer set's lowest lane publishes the new running count; its value depends on `pre`, so
+    // the LDS read above completes before this write issues, and LDS serves a wave in order
+    if (valid && rank == 0) cnt[wave][d] = pre + (uint32_t)__popcll(peers);
+    packed[r] = d | ((pre + rank) << 8);
+  }
+  __syncthreads();
+
+  {  // thread t owns digit t: turn per-wave counts into per-wave output offsets
+    const int t = threadIdx.x;
+    uint32_t run = scanned_hist[(int64_t)t * tiles + blockIdx.x];
+#pragma unroll
+    for (int w = 0; w < kSortWaves; ++w) {
+      uint32_t c = cnt[w][t];
+      cnt[w][t] = run;
+      run += c;
+    }
+  }
+  __syncthreads();
+
+#pragma unroll
+  for (int r = 0; r < kSortRounds; ++r) {
+    const int64_t idx = base + (int64_t)r * kWave + lane;
+    if (idx < count) {
+      const uint32_t d = packed[r] & (kRadix - 1);
+      const uint32_t pos = cnt[wave][d] + (packed[r] >> 8);
+      out_a[pos] = ra[r];
+      out_b[pos] = rb[r];
+      out_p[pos] = rp[r];
+    }
+  }
+}
+
+int radix_sort_pairs(SortBuffers &buf, int64_t count, int bits_a, int bits_b, int *result_set, hipStream_t stream) {
+  int cur = 0;
+  *result_set = 0;
+  if (count <= 1) return CG_OK;
+  if (count > 0x7fffffffLL) CG_FAIL(CG_ERR_OVERFLOW, "radix sort: count %lld >= 2^31", (long long)count);
+  const int64_t tiles = ceil_div64(count, kSortTile);
+  void *d_hist = nullptr;
+  CG_TRY(scratch_get(stream, kSlotC, (size_t)tiles * kRadix * sizeof(uint32_t), &d_hist));
+  uint32_t *hist = (uint32_t *)d_hist;
+
+  for (int which = 0; which < 2; ++which) {  // 0: minor key (key_b), 1: major key (key_a)
+    const int bits = which == 0 ? bits_b : bits_a;
+    for (int shift = 0; shift < bits; shift += 8) {
+      const int32_t *key = which == 0 ? buf.key_b[cur] : buf.key_a[cur];
+      radix_hist_kernel<<<(unsigned)tiles, kSortThreads, 0, stream>>>(key, count, shift, hist, tiles);
+      CG_LAUNCH_CHECK();
+      CG_TRY(exclusive_scan_u32(hist, hist, tiles * kRadix, nullptr, stream));
+      radix_scatter_kernel<<<(unsigned)tiles, kSortThreads, 0, stream>>>(
+          key, shift, buf.key_a[cur], buf.key_b[cur], buf.payload[cur], buf.key_a[cur ^ 1], buf.key_b[cur ^ 1],
+          buf.payload[cur ^ 1], count, hist, tiles);
+      CG_LAUNCH_CHECK();
+      cur ^= 1;
+    }
+  }
+  *result_set = cur;
+  return CG_OK;
+}
+
+}  // namespace cg

@@ -1,0 +1,169 @@
+"""Host side of the per-rank GCN compute path: the stage loop, GCNFunc and train of the reference
+(gcn_distr.py:203-246, :248-339, :341-366) restated for one GPU on top of the C ABI.
+
+What changes against the reference, and why:
+  * the broadcasts are gone: the dense blocks the other ranks would have sent are already resident
+    (`ResidentBlocks`), so a stage is just `z_loc += A_k @ H_k`;
+  * sparse blocks are `CsrMatrix` handles (CSR, optional transpose and schedules built once)
+    instead of COO tensors that are cast and converted on every call (gcn_distr.py:238-240);
+  * ReLU is fused into the store of `(A H) W`; backward derives the mask from the saved output
+    instead of re-running the activation under autograd (gcn_distr.py:312-322);
+  * with one block that carries its transpose, backward multiplies by A^T; the reference always
+    reuses A and therefore needs a symmetric matrix (gcn_distr.py:326).
+Names and argument order follow the reference so that its drivers read the same.
+"""
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Sequence, Union
+
+import torch
+import torch.nn.functional as F
+
+from . import ops
+from .ops import CsrMatrix
+
+# the reference keeps these as module globals set from the command line (gcn_distr.py:57-58, :826-827)
+activations = True
+
+
+class ResidentBlocks:
+    """Stands where the reference passes a process group: the dense blocks that its broadcasts
+    would deliver (gcn_distr.py:230), already resident in HBM.  `forward[i]` is the H block and
+    `backward[i]` the gradient block of stage i; the entry of the calling rank itself is ignored
+    (its own tensor is used, as in the reference's `inputs.clone()` branch, gcn_distr.py:222-223)."""
+
+    def __init__(self, forward: Sequence[Optional[torch.Tensor]], backward: Sequence[Optional[torch.Tensor]]):
+        self.forward = list(forward)
+        self.backward = list(backward)
+
+
+def _stage_operand(i: int, rank: int, own: torch.Tensor, peers: Optional[Sequence[Optional[torch.Tensor]]]):
+    if i == rank or peers is None:
+        if i != rank:
+            raise ValueError(f"stage {i}: no resident block given and it is not the caller's own (rank {rank})")
+        return own
+    blk = peers[i]
+    if blk is None:
+        raise ValueError(f"stage {i}: resident block is missing")
+    if blk.shape[1] != own.shape[1]:
+        raise ValueError(f"stage {i}: resident block has width {blk.shape[1]}, expected {own.shape[1]}")
+    return blk
+
+
+def broad_func(node_count: int, am_partitions: Sequence[CsrMatrix], inputs: torch.Tensor, rank: int, size: int,
+               group: Optional[Sequence[Optional[torch.Tensor]]] = None, transpose: bool = False) -> torch.Tensor:
+    """z_loc = sum_i am_partitions[i] @ H_i, the stage loop of gcn_distr.py:203-246 without the
+    broadcasts.  `group` lists the resident H_i (None at index `rank`, where `inputs` is used).
+    The first stage writes (beta = 0), later stages accumulate (beta = 1), so no zero fill."""
+    if len(am_partitions) != size:
+        raise ValueError(f"{len(am_partitions)} sparse blocks for size {size}")
+    z_loc = None
+    for i in range(size):
+        h_i = _stage_operand(i, rank, inputs, group)
+        blk = am_partitions[i]
+        if z_loc is None:
+            z_loc = blk.spmm(h_i, transpose=transpose)
+        else:
+            blk.spmm(h_i, out=z_loc, beta=1.0, transpose=transpose)
+    return z_loc
+
+
+def outer_product2(inputs_t: torch.Tensor, ag: torch.Tensor, rank: int = 0, size: int = 1, group=None) -> torch.Tensor:
+    """grad_weight = H^T @ AG (gcn_distr.py:178-201 without the all-reduce).  Takes H^T like the
+    reference; the kernel reads H itself, so the transpose view is undone without a copy."""
+    return ops.dense_xtg(inputs_t.t(), ag)
+
+
+def _kind(func) -> str:
+    if func is F.relu or func is torch.relu or func == "relu":
+        return "relu"
+    if func is F.log_softmax or func is torch.log_softmax or func == "log_softmax":
+        return "log_softmax"
+    return "none"
+
+
+class GCNFunc(torch.autograd.Function):
+    """One GCN layer, `func((sum_i A_i @ H_i) @ W)`; same argument list as gcn_distr.py:250."""
+
+    @staticmethod
+    def forward(ctx, inputs, weight, adj_matrix, am_partitions, rank, size, group, func):
+        kind = _kind(func) if activations else "none"
+        node_count = adj_matrix if isinstance(adj_matrix, int) else adj_matrix.size(0)
+        peers_fwd = group.forward if isinstance(group, ResidentBlocks) else None
+        z = broad_func(node_count, am_partitions, inputs, rank, size, peers_fwd)
+        out = ops.dense_xw(z, weight, relu=(kind == "relu"))
+        del z
+        if kind == "log_softmax":
+            out = ops.log_softmax_fwd(out)
+        ctx.save_for_backward(inputs, weight, out)
+        ctx.am_partitions = am_partitions
+        ctx.rank, ctx.size, ctx.group, ctx.kind, ctx.node_count = rank, size, group, kind, node_count
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        inputs, weight, out = ctx.saved_tensors
+        kind = ctx.kind
+        if kind == "relu":
+            grad_output = ops.relu_bwd(grad_output, out)
+        elif kind == "log_softmax":
+            grad_output = ops.log_softmax_bwd(grad_output, out)
+        peers_bwd = ctx.group.backward if isinstance(ctx.group, ResidentBlocks) else None
+        blocks = ctx.am_partitions
+        use_t = ctx.size == 1 and blocks[0].has_transpose
+        # first backprop equation: A G (reference: same blocks, gcn_distr.py:326)
+        ag = broad_func(ctx.node_count, blocks, grad_output, ctx.rank, ctx.size, peers_bwd, transpose=use_t)
+        grad_input = ops.dense_gwt(ag, weight) if ctx.needs_input_grad[0] else None
+        # second backprop equation reuses A G (gcn_distr.py:337)
+        grad_weight = outer_product2(inputs.t(), ag) if ctx.needs_input_grad[1] else None
+        return grad_input, grad_weight, None, None, None, None, None, None
+
+
+class MaskedNLLLoss(torch.autograd.Function):
+    """F.nll_loss(outputs[mask], y[mask]) without materialising the gathered rows
+    (gcn_distr.py:356); an empty mask gives a zero loss with zero gradient, which is what the
+    reference's fake_loss branch produces (gcn_distr.py:359-362)."""
+
+    @staticmethod
+    def forward(ctx, outputs, y, mask):
+        loss, count = ops.nll_loss_fwd(outputs, y, mask)
+        ctx.save_for_backward(y, mask if mask is not None else torch.empty(0, device=y.device), count)
+        ctx.has_mask = mask is not None
+        ctx.shape = tuple(outputs.shape)
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_loss):
+        y, mask, count = ctx.saved_tensors
+        n, c = ctx.shape
+        g = ops.nll_loss_bwd(y, mask if ctx.has_mask else None, count, grad_loss.float().reshape(()), n, c)
+        return g, None, None
+
+
+def masked_nll_loss(outputs: torch.Tensor, y: torch.Tensor, mask: Optional[torch.Tensor]) -> torch.Tensor:
+    return MaskedNLLLoss.apply(outputs, y, mask)
+
+
+def train(inputs, weight1, weight2, adj_matrix, am_partitions, optimizer, data, rank=0, size=1, group=None):
+    """One epoch, gcn_distr.py:341-366.  `data` needs `.y` and `.train_mask`; `group` is None for a
+    whole graph on one GPU, or a pair (layer-1 ResidentBlocks, layer-2 ResidentBlocks)."""
+    g1, g2 = group if isinstance(group, (tuple, list)) else (group, group)
+    outputs = GCNFunc.apply(inputs, weight1, adj_matrix, am_partitions, rank, size, g1, F.relu)
+    outputs = GCNFunc.apply(outputs, weight2, adj_matrix, am_partitions, rank, size, g2, F.log_softmax)
+
+    optimizer.zero_grad()
+
+    node_count = adj_matrix if isinstance(adj_matrix, int) else adj_matrix.size(0)
+    n_per_proc = int(math.ceil(float(node_count) / size))
+    rank_train_mask = torch.split(data.train_mask.bool(), n_per_proc, dim=0)[rank]
+    datay_rank = torch.split(data.y, n_per_proc, dim=0)[rank]
+
+    loss = masked_nll_loss(outputs, datay_rank, rank_train_mask)
+    loss.backward()
+    optimizer.step()
+    train.last_loss = loss.detach()
+    return outputs
+
+
+train.last_loss = None

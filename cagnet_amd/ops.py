@@ -1,0 +1,382 @@
+"""Tensor-level wrappers over the C ABI: torch supplies device memory and the current stream,
+every computation happens in libcagnet_amd.so.
+
+Dense operands are fp32 CUDA(HIP) tensors, row-major with unit column stride (a row stride larger
+than the column count is passed on as the leading dimension).  Sparse indices are int32.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_int64, c_void_p
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import CG_CSR_SORTED, CG_CSR_TRANSPOSE, CG_CSR_VALIDATE, CagnetError, check, lib
+
+__all__ = [
+    "CagnetError", "CsrMatrix", "coo2csr_rowptr", "coo2csr", "csr_transpose", "coo_check", "spmm_coo",
+    "dense_xw", "dense_gwt", "dense_xtg", "relu_fwd", "relu_bwd", "log_softmax_fwd", "log_softmax_bwd",
+    "nll_loss_fwd", "nll_loss_bwd", "log_softmax_nll_bwd",
+]
+
+
+def _stream() -> c_void_p:
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: Optional[torch.Tensor]) -> c_void_p:
+    return c_void_p(t.data_ptr()) if t is not None and t.numel() > 0 else c_void_p(0)
+
+
+def _need(t: torch.Tensor, name: str, dtype: torch.dtype, dim: Optional[int] = None) -> torch.Tensor:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name}: expected a torch.Tensor, got {type(t).__name__}")
+    if not t.is_cuda:
+        raise ValueError(f"{name}: must live on the GPU (got device {t.device}); there is no CPU path")
+    if t.dtype != dtype:
+        raise TypeError(f"{name}: expected dtype {dtype}, got {t.dtype}")
+    if dim is not None and t.dim() != dim:
+        raise ValueError(f"{name}: expected {dim} dimensions, got {t.dim()}")
+    return t
+
+
+def _index(t: torch.Tensor, name: str) -> torch.Tensor:
+    t = _need(t, name, torch.int32, 1)
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def _values(t: torch.Tensor, name: str) -> torch.Tensor:
+    t = _need(t, name, torch.float32, 1)
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def _rowmajor(t: torch.Tensor, name: str) -> Tuple[torch.Tensor, int]:
+    """Return (tensor, leading dimension).  Copies only when the column stride is not 1."""
+    t = _need(t, name, torch.float32, 2)
+    rows, cols = t.shape
+    if cols > 0 and t.stride(1) != 1 or (rows > 1 and t.stride(0) < cols):
+        t = t.contiguous()
+    ld = t.stride(0) if rows > 1 else max(cols, 1)
+    return t, max(ld, cols, 1)
+
+
+def _out_rowmajor(t: torch.Tensor, name: str) -> int:
+    _need(t, name, torch.float32, 2)
+    rows, cols = t.shape
+    if (cols > 1 and t.stride(1) != 1) or (rows > 1 and t.stride(0) < cols):
+        raise ValueError(f"{name}: output must be row-major with unit column stride (strides {t.stride()})")
+    return max(t.stride(0) if rows > 1 else cols, cols, 1)
+
+
+# ------------------------------------------------------------------------------------------------
+# coo2csr family
+# ------------------------------------------------------------------------------------------------
+def coo2csr_rowptr(row: torch.Tensor, n: int) -> torch.Tensor:
+    """rowptr[n+1] of ascending int32 row indices (cusparseXcoo2csr of the reference,
+    sparse-extension/sparse_coo_tensor.cu:136-142)."""
+    row = _index(row, "row")
+    rowptr = torch.empty(n + 1, dtype=torch.int32, device=row.device)
+    check(lib.cg_coo2csr_rowptr(_ptr(row), row.numel(), n, _ptr(rowptr), _stream()), "cg_coo2csr_rowptr")
+    return rowptr
+
+
+def coo_check(row: torch.Tensor, col: torch.Tensor, n: int, m: int, require_sorted: int = 1) -> None:
+    row, col = _index(row, "row"), _index(col, "col")
+    if row.numel() != col.numel():
+        raise ValueError("row and col differ in length")
+    check(lib.cg_coo_check(_ptr(row), _ptr(col), row.numel(), n, m, require_sorted, _stream()), "cg_coo_check")
+
+
+def coo2csr(row: torch.Tensor, col: torch.Tensor, val: Optional[torch.Tensor], n: int, m: int,
+            return_perm: bool = False):
+    """COO in any order -> (rowptr, colind, values[, perm]) sorted by (row, col), stable."""
+    row, col = _index(row, "row"), _index(col, "col")
+    nnz = row.numel()
+    if col.numel() != nnz or (val is not None and val.numel() != nnz):
+        raise ValueError("row, col and val differ in length")
+    if val is not None:
+        val = _values(val, "val")
+    dev = row.device
+    rowptr = torch.empty(n + 1, dtype=torch.int32, device=dev)
+    colind = torch.empty(nnz, dtype=torch.int32, device=dev)
+    values = torch.empty(nnz, dtype=torch.float32, device=dev) if val is not None else None
+    perm = torch.empty(nnz, dtype=torch.int32, device=dev) if return_perm else None
+    check(lib.cg_coo2csr(_ptr(row), _ptr(col), _ptr(val), nnz, n, m, _ptr(rowptr), _ptr(colind), _ptr(values),
+                         _ptr(perm), _stream()), "cg_coo2csr")
+    return (rowptr, colind, values, perm) if return_perm else (rowptr, colind, values)
+
+
+def csr_transpose(rowptr: torch.Tensor, colind: torch.Tensor, values: Optional[torch.Tensor], n: int, m: int,
+                  return_perm: bool = False):
+    """CSR of A (n x m) -> CSR of A^T (m x n): (colptr, rowind, values_t[, perm])."""
+    rowptr, colind = _index(rowptr, "rowptr"), _index(colind, "colind")
+    if rowptr.numel() != n + 1:
+        raise ValueError(f"rowptr has {rowptr.numel()} entries, expected n + 1 = {n + 1}")
+    nnz = colind.numel()
+    if values is not None:
+        values = _values(values, "values")
+        if values.numel() != nnz:
+            raise ValueError("colind and values differ in length")
+    dev = rowptr.device
+    colptr = torch.empty(m + 1, dtype=torch.int32, device=dev)
+    rowind = torch.empty(nnz, dtype=torch.int32, device=dev)
+    values_t = torch.empty(nnz, dtype=torch.float32, device=dev) if values is not None else None
+    perm = torch.empty(nnz, dtype=torch.int32, device=dev) if return_perm else None
+    check(lib.cg_csr_transpose(_ptr(rowptr), _ptr(colind), _ptr(values), nnz, n, m, _ptr(colptr), _ptr(rowind),
+                               _ptr(values_t), _ptr(perm), _stream()), "cg_csr_transpose")
+    return (colptr, rowind, values_t, perm) if return_perm else (colptr, rowind, values_t)
+
+
+# ------------------------------------------------------------------------------------------------
+# SpMM
+# ------------------------------------------------------------------------------------------------
+def spmm_coo(row: torch.Tensor, col: torch.Tensor, val: torch.Tensor, n: int, m: int, B: torch.Tensor,
+             C: torch.Tensor, beta: float = 1.0) -> None:
+    """C[n,f] = beta*C + A*B with A as row-sorted COO; the one-shot form of the reference operator
+    (sparse-extension/sparse_coo_tensor.cu:113-240)."""
+    row, col, val = _index(row, "row"), _index(col, "col"), _values(val, "val")
+    if not (row.numel() == col.numel() == val.numel()):
+        raise ValueError("row, col and val differ in length")
+    B, ldb = _rowmajor(B, "B")
+    ldc = _out_rowmajor(C, "C")
+    if B.shape[0] != m or C.shape[0] != n or B.shape[1] != C.shape[1]:
+        raise ValueError(f"shape mismatch: A is {n}x{m}, B is {tuple(B.shape)}, C is {tuple(C.shape)}")
+    check(lib.cg_spmm_coo(_ptr(row), _ptr(col), _ptr(val), val.numel(), n, m, _ptr(B), ldb, _ptr(C), ldc,
+                          B.shape[1], float(beta), _stream()), "cg_spmm_coo")
+
+
+class _DeviceArray:
+    """Zero-copy view of handle-owned device memory for torch.as_tensor."""
+
+    def __init__(self, ptr: int, count: int, typestr: str):
+        self.__cuda_array_interface__ = {
+            "shape": (count,), "typestr": typestr, "data": (ptr, True), "version": 2, "strides": None,
+        }
+
+
+class CsrMatrix:
+    """Device-resident CSR of one sparse block (and optionally of its transpose) with cached
+    schedules: what the reference rebuilds inside every spmm_gpu call is built once here."""
+
+    def __init__(self, row: torch.Tensor, col: torch.Tensor, val: torch.Tensor, n: int, m: int, *,
+                 is_sorted: bool = True, transpose: bool = False, validate: bool = False):
+        row, col, val = _index(row, "row"), _index(col, "col"), _values(val, "val")
+        if not (row.numel() == col.numel() == val.numel()):
+            raise ValueError("row, col and val differ in length")
+        flags = (CG_CSR_SORTED if is_sorted else 0) | (CG_CSR_TRANSPOSE if transpose else 0) | (
+            CG_CSR_VALIDATE if validate else 0)
+        handle = c_void_p(0)
+        self._handle = None
+        self.device = row.device
+        with torch.cuda.device(self.device):
+            check(lib.cg_csr_create(ctypes.byref(handle), _ptr(row), _ptr(col), _ptr(val), val.numel(), n, m, flags,
+                                    _stream()), "cg_csr_create")
+        self._handle = handle
+        self.n, self.m, self.nnz = int(n), int(m), int(val.numel())
+        self.has_transpose = bool(transpose)
+
+    @classmethod
+    def from_torch_coo(cls, a: torch.Tensor, **kw) -> "CsrMatrix":
+        """From a coalesced torch.sparse_coo tensor (the type the reference keeps its blocks in,
+        gcn_distr.py:493-512, :546)."""
+        a = a.coalesce()
+        idx = a.indices()
+        return cls(idx[0].int(), idx[1].int(), a.values().float(), a.shape[0], a.shape[1], is_sorted=True, **kw)
+
+    def __del__(self):
+        h = getattr(self, "_handle", None)
+        if h is not None and lib is not None:
+            try:
+                lib.cg_csr_destroy(h)
+            except Exception:
+                pass
+            self._handle = None
+
+    @property
+    def shape(self) -> Tuple[int, int]:
+        return (self.n, self.m)
+
+    def info(self) -> dict:
+        buf = (c_int64 * 8)()
+        check(lib.cg_csr_info(self._handle, buf), "cg_csr_info")
+        return {"n": buf[0], "m": buf[1], "nnz": buf[2], "has_transpose": bool(buf[3]),
+                "max_row_degree": buf[4], "max_col_degree": buf[5]}
+
+    def arrays(self, transpose: bool = False):
+        """(rowptr, colind, values) of A, or of A^T, as tensors that alias the handle's memory."""
+        p = [c_void_p(0), c_void_p(0), c_void_p(0)]
+        check(lib.cg_csr_arrays(self._handle, int(transpose), ctypes.byref(p[0]), ctypes.byref(p[1]),
+                                ctypes.byref(p[2])), "cg_csr_arrays")
+        rows = self.m if transpose else self.n
+        out = [torch.as_tensor(_DeviceArray(p[0].value, rows + 1, "<i4"), device=self.device)]
+        if self.nnz > 0:
+            out.append(torch.as_tensor(_DeviceArray(p[1].value, self.nnz, "<i4"), device=self.device))
+            out.append(torch.as_tensor(_DeviceArray(p[2].value, self.nnz, "<f4"), device=self.device))
+        else:
+            out.append(torch.empty(0, dtype=torch.int32, device=self.device))
+            out.append(torch.empty(0, dtype=torch.float32, device=self.device))
+        return tuple(out)
+
+    def spmm(self, B: torch.Tensor, out: Optional[torch.Tensor] = None, beta: float = 0.0,
+             transpose: bool = False) -> torch.Tensor:
+        """out = beta*out + op(A)*B.  A fresh output is allocated (and beta forced to 0) if none is given."""
+        B, ldb = _rowmajor(B, "B")
+        rows, inner = (self.m, self.n) if transpose else (self.n, self.m)
+        if B.shape[0] != inner:
+            raise ValueError(f"B has {B.shape[0]} rows, the sparse operand has {inner} columns")
+        f = B.shape[1]
+        if out is None:
+            out = torch.empty(rows, f, dtype=torch.float32, device=B.device)
+            beta = 0.0
+        ldc = _out_rowmajor(out, "out")
+        if tuple(out.shape) != (rows, f):
+            raise ValueError(f"out has shape {tuple(out.shape)}, expected {(rows, f)}")
+        check(lib.cg_csr_spmm(self._handle, int(transpose), _ptr(B), ldb, _ptr(out), ldc, f, float(beta), _stream()),
+              "cg_csr_spmm")
+        return out
+
+
+# ------------------------------------------------------------------------------------------------
+# dense products
+# ------------------------------------------------------------------------------------------------
+def dense_xw(X: torch.Tensor, W: torch.Tensor, relu: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Z = X @ W (optionally ReLU fused into the store); torch.mm at gcn_distr.py:275."""
+    X, ldx = _rowmajor(X, "X")
+    W, ldw = _rowmajor(W, "W")
+    n, k = X.shape
+    if W.shape[0] != k:
+        raise ValueError(f"X is {tuple(X.shape)}, W is {tuple(W.shape)}")
+    fo = W.shape[1]
+    if out is None:
+        out = torch.empty(n, fo, dtype=torch.float32, device=X.device)
+    ldz = _out_rowmajor(out, "out")
+    check(lib.cg_dense_xw(_ptr(X), ldx, _ptr(W), ldw, _ptr(out), ldz, n, k, fo, int(relu), _stream()), "cg_dense_xw")
+    return out
+
+
+def dense_gwt(G: torch.Tensor, W: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """dX = G @ W.T; torch.mm(ag, weight.t()) at gcn_distr.py:330."""
+    G, ldg = _rowmajor(G, "G")
+    W, ldw = _rowmajor(W, "W")
+    n, fo = G.shape
+    k = W.shape[0]
+    if W.shape[1] != fo:
+        raise ValueError(f"G is {tuple(G.shape)}, W is {tuple(W.shape)}")
+    if out is None:
+        out = torch.empty(n, k, dtype=torch.float32, device=G.device)
+    lddx = _out_rowmajor(out, "out")
+    check(lib.cg_dense_gwt(_ptr(G), ldg, _ptr(W), ldw, _ptr(out), lddx, n, k, fo, _stream()), "cg_dense_gwt")
+    return out
+
+
+def dense_xtg(X: torch.Tensor, G: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """dW = X.T @ G; torch.mm(inputs.t(), ag) at gcn_distr.py:187."""
+    X, ldx = _rowmajor(X, "X")
+    G, ldg = _rowmajor(G, "G")
+    n, k = X.shape
+    if G.shape[0] != n:
+        raise ValueError(f"X is {tuple(X.shape)}, G is {tuple(G.shape)}")
+    fo = G.shape[1]
+    if out is None:
+        out = torch.empty(k, fo, dtype=torch.float32, device=X.device)
+    lddw = _out_rowmajor(out, "out")
+    check(lib.cg_dense_xtg(_ptr(X), ldx, _ptr(G), ldg, _ptr(out), lddw, n, k, fo, _stream()), "cg_dense_xtg")
+    return out
+
+
+# ------------------------------------------------------------------------------------------------
+# activations and loss
+# ------------------------------------------------------------------------------------------------
+def _flat(t: torch.Tensor, name: str) -> torch.Tensor:
+    t = _need(t, name, torch.float32)
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def relu_fwd(z: torch.Tensor) -> torch.Tensor:
+    z = _flat(z, "z")
+    h = torch.empty_like(z)
+    check(lib.cg_relu_fwd(_ptr(z), _ptr(h), z.numel(), _stream()), "cg_relu_fwd")
+    return h
+
+
+def relu_bwd(g: torch.Tensor, h: torch.Tensor) -> torch.Tensor:
+    g, h = _flat(g, "g"), _flat(h, "h")
+    if g.shape != h.shape:
+        raise ValueError("g and h differ in shape")
+    dz = torch.empty_like(g)
+    check(lib.cg_relu_bwd(_ptr(g), _ptr(h), _ptr(dz), g.numel(), _stream()), "cg_relu_bwd")
+    return dz
+
+
+def log_softmax_fwd(z: torch.Tensor) -> torch.Tensor:
+    z, ldz = _rowmajor(z, "z")
+    n, c = z.shape
+    out = torch.empty(n, c, dtype=torch.float32, device=z.device)
+    check(lib.cg_log_softmax_fwd(_ptr(z), ldz, _ptr(out), max(c, 1), n, c, _stream()), "cg_log_softmax_fwd")
+    return out
+
+
+def log_softmax_bwd(g: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    g, ldg = _rowmajor(g, "g")
+    out, ldo = _rowmajor(out, "out")
+    if g.shape != out.shape:
+        raise ValueError("g and out differ in shape")
+    n, c = g.shape
+    dz = torch.empty(n, c, dtype=torch.float32, device=g.device)
+    check(lib.cg_log_softmax_bwd(_ptr(g), ldg, _ptr(out), ldo, _ptr(dz), max(c, 1), n, c, _stream()),
+          "cg_log_softmax_bwd")
+    return dz
+
+
+def _labels(y: torch.Tensor, n: int) -> torch.Tensor:
+    y = _need(y, "y", torch.int64, 1)
+    if y.numel() != n:
+        raise ValueError(f"y has {y.numel()} labels for {n} rows")
+    return y if y.is_contiguous() else y.contiguous()
+
+
+def _mask(mask: Optional[torch.Tensor], n: int) -> Optional[torch.Tensor]:
+    if mask is None:
+        return None
+    if mask.dtype not in (torch.bool, torch.uint8) or not mask.is_cuda or mask.dim() != 1 or mask.numel() != n:
+        raise ValueError("mask must be a CUDA bool/uint8 vector with one entry per row")
+    return mask if mask.is_contiguous() else mask.contiguous()
+
+
+def nll_loss_fwd(logp: torch.Tensor, y: torch.Tensor, mask: Optional[torch.Tensor] = None):
+    """(loss, count): loss = -mean over masked rows of logp[i, y_i] as a 0-d tensor; count = |mask| (int64, 0-d)."""
+    logp, ld = _rowmajor(logp, "logp")
+    n, c = logp.shape
+    y, mask = _labels(y, n), _mask(mask, n)
+    loss = torch.empty((), dtype=torch.float32, device=logp.device)
+    count = torch.empty((), dtype=torch.int64, device=logp.device)
+    check(lib.cg_nll_loss_fwd(_ptr(logp), ld, _ptr(y), _ptr(mask), n, c, c_void_p(loss.data_ptr()),
+                              c_void_p(count.data_ptr()), _stream()), "cg_nll_loss_fwd")
+    return loss, count
+
+
+def nll_loss_bwd(y: torch.Tensor, mask: Optional[torch.Tensor], count: torch.Tensor, gscale: Optional[torch.Tensor],
+                 n: int, c: int) -> torch.Tensor:
+    y, mask = _labels(y, n), _mask(mask, n)
+    d = torch.empty(n, c, dtype=torch.float32, device=y.device)
+    gs = None if gscale is None else _need(gscale, "gscale", torch.float32).reshape(())
+    check(lib.cg_nll_loss_bwd(_ptr(y), _ptr(mask), c_void_p(count.data_ptr()),
+                              c_void_p(gs.data_ptr()) if gs is not None else c_void_p(0), _ptr(d), max(c, 1), n, c,
+                              _stream()), "cg_nll_loss_bwd")
+    return d
+
+
+def log_softmax_nll_bwd(logp: torch.Tensor, y: torch.Tensor, mask: Optional[torch.Tensor], count: torch.Tensor,
+                        gscale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """dz of mean-NLL(log_softmax(z)) given logp = log_softmax(z): gscale*mask/|mask|*(softmax - onehot)."""
+    logp, ld = _rowmajor(logp, "logp")
+    n, c = logp.shape
+    y, mask = _labels(y, n), _mask(mask, n)
+    dz = torch.empty(n, c, dtype=torch.float32, device=logp.device)
+    gs = None if gscale is None else _need(gscale, "gscale", torch.float32).reshape(())
+    check(lib.cg_log_softmax_nll_bwd(_ptr(logp), ld, _ptr(y), _ptr(mask), c_void_p(count.data_ptr()),
+                                     c_void_p(gs.data_ptr()) if gs is not None else c_void_p(0), _ptr(dz), max(c, 1),
+                                     n, c, _stream()), "cg_log_softmax_nll_bwd")
+    return dz

@@ -1,0 +1,53 @@
+"""The reference's native module, name for name.
+
+CAGNET's drivers do `from sparse_coo_tensor_cpp import sparse_coo_tensor_gpu, spmm_gpu`
+(gcn_distr.py:27, gcn_distr_15d.py:27, gcn_distr_2d.py:38, gcn_distr_3d.py:36); the module is
+registered at sparse-extension/sparse_coo_tensor.cu:242-245.  This module exports the same two
+names with the same positional signatures, plus `coo2csr`, which the reference only runs
+internally (sparse_coo_tensor.cu:136-142).
+
+Differences a caller can observe, all deliberate:
+  * errors raise (CagnetError) instead of being printed and ignored (sparse_coo_tensor.cu:20-30);
+  * B and C keep their storage and their row-major layout; the reference hands both back as
+    column-major strided views of fresh storage (sparse_coo_tensor.cu:166-168, :183-185, :233-239);
+  * the call is ordered on torch's current stream and does not synchronise the device.
+"""
+from __future__ import annotations
+
+from typing import Sequence
+
+import torch
+
+from . import ops
+
+__all__ = ["spmm_gpu", "sparse_coo_tensor_gpu", "coo2csr"]
+
+
+def spmm_gpu(A_rowindices: torch.Tensor, A_colindices: torch.Tensor, A_values: torch.Tensor, n: int, m: int,
+             B: torch.Tensor, C: torch.Tensor) -> None:
+    """C += A @ B.  A is n x m, given as row-sorted COO with int32 indices and fp32 values
+    (the callers pass `.indices()[k].int()` of a coalesced tensor, gcn_distr.py:238-240);
+    B is m x f and C is n x f, both fp32.  Returns None, like the reference."""
+    if C.dim() == 2 and C.numel() > 0 and C.stride(1) != 1:
+        # a transposed view, e.g. a C that an earlier reference-style call left column-major
+        tmp = C.contiguous()
+        ops.spmm_coo(A_rowindices, A_colindices, A_values, int(n), int(m), B, tmp, beta=1.0)
+        C.copy_(tmp)
+        return None
+    ops.spmm_coo(A_rowindices, A_colindices, A_values, int(n), int(m), B, C, beta=1.0)
+    return None
+
+
+def sparse_coo_tensor_gpu(indices: torch.Tensor, values: torch.Tensor, size: Sequence[int]) -> torch.Tensor:
+    """COO constructor that skips index validation (and its device synchronisation), like
+    sparse_coo_tensor_gpu at sparse-extension/sparse_coo_tensor.cu:43-54.  No kernel is involved."""
+    if indices.dim() != 2:
+        raise ValueError("indices must be 2-D (sparse_dim x nnz)")
+    return torch.sparse_coo_tensor(indices, values, tuple(size), check_invariants=False)
+
+
+def coo2csr(A_rowindices: torch.Tensor, A_colindices: torch.Tensor, A_values: torch.Tensor, n: int, m: int):
+    """(rowptr[n+1], colind[nnz], values[nnz]) in (row, col) order, from COO in any order.
+    The reference performs only the row compression, on sorted input, inside spmm_gpu
+    (cusparseXcoo2csr, sparse_coo_tensor.cu:137-142)."""
+    return ops.coo2csr(A_rowindices, A_colindices, A_values, int(n), int(m))

@@ -1,0 +1,174 @@
+/*
+ * cagnet_amd.h -- C ABI of libcagnet_amd.so: the per-rank GCN compute path of
+ * CAGNET (local coo2csr + accumulate-SpMM + H*W + ReLU / log_softmax+NLL,
+ * forward and backward) as hand-written gfx950 HIP kernels.
+ *
+ * Conventions
+ *   - Every pointer named d_* or documented "device" is a device pointer on the
+ *     current HIP device.  Dense matrices are fp32 row-major with an explicit
+ *     leading dimension in ELEMENTS (ld >= number of columns).  Sparse indices
+ *     are int32 (the reference's contract); dense offsets are 64-bit inside.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).  All
+ *     work is enqueued on it; no entry point synchronises the device unless its
+ *     comment says so.
+ *   - Every entry point returns a cg_status (0 = success).  cg_last_error()
+ *     returns a thread-local human-readable detail for the last failure.
+ *     (The reference prints cuSPARSE/CUDA errors and continues,
+ *     sparse-extension/sparse_coo_tensor.cu:20-30; a status code is strictly
+ *     stronger and needs no change at the call sites.)
+ *   - Summation orders are fixed by the schedule (no floating-point atomics):
+ *     two calls with the same arguments give bit-identical results.
+ *   - Library scratch memory is kept per (device, stream); calls that share a
+ *     stream are ordered by it.  Calls on different streams use different
+ *     scratch and may overlap.
+ */
+#ifndef CAGNET_AMD_H
+#define CAGNET_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CG_ABI_VERSION 1
+
+typedef void *cg_stream_t;       /* hipStream_t */
+typedef struct cg_csr cg_csr_t;  /* opaque: device-resident CSR (+ optional transpose) and its schedules */
+
+enum cg_status {
+  CG_OK = 0,
+  CG_ERR_NULL = 1,         /* a required pointer is NULL */
+  CG_ERR_SIZE = 2,         /* negative size, ld < columns, f <= 0, ... */
+  CG_ERR_OVERFLOW = 3,     /* nnz >= 2^31, n + 1 overflows int32, ... */
+  CG_ERR_UNSORTED = 4,     /* validation: rows not ascending on the sorted path */
+  CG_ERR_INDEX = 5,        /* validation: row >= n or col >= m or negative index */
+  CG_ERR_HIP = 6,          /* a HIP runtime call failed (detail in cg_last_error) */
+  CG_ERR_ALLOC = 7,        /* device or host allocation failed */
+  CG_ERR_UNSUPPORTED = 8,  /* argument combination not implemented */
+  CG_ERR_NO_TRANSPOSE = 9, /* transpose product asked of a handle built without CG_CSR_TRANSPOSE */
+  CG_ERR_ALIAS = 10        /* output aliases an input where that is not allowed */
+};
+
+/* flags of cg_csr_create */
+#define CG_CSR_SORTED 1u    /* trust: input is sorted by (row, col) (torch .coalesce() order) */
+#define CG_CSR_TRANSPOSE 2u /* also build the transpose (CSC of A = CSR of A^T) for A^T * G */
+#define CG_CSR_VALIDATE 4u  /* check index ranges (and sortedness if CG_CSR_SORTED); synchronises */
+
+int cg_abi_version(void);
+const char *cg_status_string(int status);
+const char *cg_last_error(void);
+
+/* ------------------------------------------------------------------------------------------
+ * coo2csr.  Replaces the cusparseXcoo2csr step that the reference runs inside every spmm_gpu
+ * call (sparse-extension/sparse_coo_tensor.cu:136-142): compress ascending int32 row indices
+ * into rowptr[n+1], base 0.  rowptr[i] = #{k : row[k] < i}.  d_row must be ascending; indices
+ * outside [0, n) are clamped into the table instead of faulting.  nnz == 0 is legal.
+ */
+int cg_coo2csr_rowptr(const int32_t *d_row, int64_t nnz, int32_t n, int32_t *d_rowptr, cg_stream_t stream);
+
+/* Validating companion (debug mode of the same boundary: the reference never checks its
+ * inputs, sparse_coo_tensor.cu:113-142).  Synchronises `stream`.  Returns CG_ERR_INDEX if any
+ * row is outside [0,n) or col outside [0,m); CG_ERR_UNSORTED if require_sorted and rows
+ * descend somewhere (or cols do not strictly ascend inside a row when require_sorted == 2). */
+int cg_coo_check(const int32_t *d_row, const int32_t *d_col, int64_t nnz, int32_t n, int32_t m,
+                 int require_sorted, cg_stream_t stream);
+
+/* General COO -> CSR for input in ANY order: stable LSD radix sort of (row, col) keys in LDS,
+ * then the row compression above.  Duplicates are kept (not summed), in input order.  Outputs:
+ * d_rowptr[n+1], d_colind[nnz], d_values[nnz] (may be NULL when d_val is NULL) and, when
+ * d_perm != NULL, d_perm[k] = input position of output entry k.  Result order equals
+ * scipy.sparse.coo_matrix(...).tocsr() with sorted indices / torch .coalesce() on
+ * duplicate-free input (what the reference's callers feed spmm_gpu: gcn_distr.py:546).
+ * Allocates temporaries and synchronises `stream` before returning. */
+int cg_coo2csr(const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz, int32_t n, int32_t m,
+               int32_t *d_rowptr, int32_t *d_colind, float *d_values, int32_t *d_perm, cg_stream_t stream);
+
+/* CSR of A (n x m) -> CSR of A^T (m x n) == CSC of A: the precomputed operand of the A^T*G
+ * backward product (the reference reuses A itself and so assumes symmetry, gcn_distr.py:326,
+ * gcn_distr_2d.py:683).  Stable radix sort by column, so rows ascend inside each column.
+ * d_perm (nullable): d_perm[k] = CSR position of transposed entry k.  Allocates temporaries
+ * and synchronises `stream`. */
+int cg_csr_transpose(const int32_t *d_rowptr, const int32_t *d_colind, const float *d_values, int64_t nnz,
+                     int32_t n, int32_t m, int32_t *d_colptr, int32_t *d_rowind, float *d_values_t,
+                     int32_t *d_perm, cg_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * spmm_gpu, one shot.  Same operands and meaning as the reference operator
+ *   spmm_gpu(A_rowindices, A_colindices, A_values, n, m, B, C)
+ * (sparse-extension/sparse_coo_tensor.cu:113-240, called at gcn_distr.py:238-240):
+ * C[n,f] = beta*C + A[n,m] * B[m,f] with A as row-sorted COO; the reference fixes beta = 1
+ * (sparse_coo_tensor.cu:149-150).  Stream ordered: no allocation after the scratch has grown
+ * to size, no device synchronisation, B and C stay row-major and keep their storage (the
+ * reference transposes both and replaces their storage, :166-168,:183-185,:234-239).
+ */
+int cg_spmm_coo(const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz, int32_t n, int32_t m,
+                const float *d_B, int64_t ldb, float *d_C, int64_t ldc, int32_t f, float beta, cg_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Cached handle: what the reference rebuilds on every call (index casts gcn_distr.py:238,
+ * coo2csr, workspace malloc/free, sparse_coo_tensor.cu:136-231) is built once here.
+ * cg_csr_create copies the operands (the caller may free its arrays afterwards), builds the CSR,
+ * the transpose if asked, and synchronises `stream`.
+ */
+int cg_csr_create(cg_csr_t **out, const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz,
+                  int32_t n, int32_t m, uint32_t flags, cg_stream_t stream);
+int cg_csr_destroy(cg_csr_t *h);
+
+/* C[rows,f] = beta*C + op(A) * B, op(A) = A (transpose == 0: rows = n, B is m x f) or A^T
+ * (transpose != 0: rows = m, B is n x f).  The first call for a given schedule class builds that
+ * schedule (degree bins, row segments) and synchronises once; later calls are stream ordered. */
+int cg_csr_spmm(cg_csr_t *h, int transpose, const float *d_B, int64_t ldb, float *d_C, int64_t ldc, int32_t f,
+                float beta, cg_stream_t stream);
+
+/* info[0..7] = { n, m, nnz, has_transpose, max row degree, max column degree (or -1), 0, 0 } */
+int cg_csr_info(const cg_csr_t *h, int64_t info[8]);
+/* Device pointers of the arrays the handle owns (transpose != 0: those of A^T). */
+int cg_csr_arrays(const cg_csr_t *h, int transpose, const int32_t **d_rowptr, const int32_t **d_colind,
+                  const float **d_values);
+
+/* ------------------------------------------------------------------------------------------
+ * Dense products of GCNFunc (torch.mm at gcn_distr.py:275, :330, :187).
+ *   cg_dense_xw : Z[n,fo]  = X[n,k] * W[k,fo]           (optionally fused ReLU: relu != 0)
+ *   cg_dense_gwt: dX[n,k]  = G[n,fo] * W[k,fo]^T
+ *   cg_dense_xtg: dW[k,fo] = X[n,k]^T * G[n,fo]         (split over n, fixed-order second pass)
+ */
+int cg_dense_xw(const float *d_X, int64_t ldx, const float *d_W, int64_t ldw, float *d_Z, int64_t ldz, int64_t n,
+                int32_t k, int32_t fo, int relu, cg_stream_t stream);
+int cg_dense_gwt(const float *d_G, int64_t ldg, const float *d_W, int64_t ldw, float *d_dX, int64_t lddx,
+                 int64_t n, int32_t k, int32_t fo, cg_stream_t stream);
+int cg_dense_xtg(const float *d_X, int64_t ldx, const float *d_G, int64_t ldg, float *d_dW, int64_t lddw,
+                 int64_t n, int32_t k, int32_t fo, cg_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Activations and loss of GCNFunc / train (gcn_distr.py:284-294, :312-322, :349-362).
+ *   relu_fwd        : h = max(z, 0)
+ *   relu_bwd        : dz = g * [h > 0]   (h is the ReLU OUTPUT; [h > 0] == [z > 0])
+ *   log_softmax_fwd : out[i,:] = z[i,:] - logsumexp(z[i,:])
+ *   log_softmax_bwd : dz[i,:] = g[i,:] - exp(out[i,:]) * sum_c g[i,c]
+ *   nll_loss_fwd    : *d_loss = -(1/|mask|) * sum_{i in mask} logp[i, y_i]; |mask| == 0 gives 0
+ *                     (the reference's fake_loss branch, gcn_distr.py:359-362)
+ *   nll_loss_bwd    : dlogp[i,c] = -gscale * mask_i / |mask| * [c == y_i]   (zero elsewhere)
+ *   log_softmax_nll_bwd : fused dz = gscale * mask_i/|mask| * (exp(logp[i,c]) - [c == y_i])
+ * y is int64 (torch labels); mask is one byte per row (torch.bool / uint8), NULL = all rows.
+ * A label outside [0, c) contributes nothing (torch would raise).  d_count receives |mask| as
+ * int64 (device).  Both reductions run in a fixed order.
+ */
+int cg_relu_fwd(const float *d_z, float *d_h, int64_t count, cg_stream_t stream);
+int cg_relu_bwd(const float *d_g, const float *d_h, float *d_dz, int64_t count, cg_stream_t stream);
+int cg_log_softmax_fwd(const float *d_z, int64_t ldz, float *d_out, int64_t ldo, int64_t n, int32_t c,
+                       cg_stream_t stream);
+int cg_log_softmax_bwd(const float *d_g, int64_t ldg, const float *d_out, int64_t ldo, float *d_dz, int64_t lddz,
+                       int64_t n, int32_t c, cg_stream_t stream);
+int cg_nll_loss_fwd(const float *d_logp, int64_t ld, const int64_t *d_y, const uint8_t *d_mask, int64_t n,
+                    int32_t c, float *d_loss, int64_t *d_count, cg_stream_t stream);
+int cg_nll_loss_bwd(const int64_t *d_y, const uint8_t *d_mask, const int64_t *d_count, const float *d_gscale,
+                    float *d_dlogp, int64_t ld, int64_t n, int32_t c, cg_stream_t stream);
+int cg_log_softmax_nll_bwd(const float *d_logp, int64_t ld, const int64_t *d_y, const uint8_t *d_mask,
+                           const int64_t *d_count, const float *d_gscale, float *d_dz, int64_t lddz, int64_t n,
+                           int32_t c, cg_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CAGNET_AMD_H */

@@ -1,0 +1,108 @@
+"""GPU parity of the dense products and of the activation / loss kernels through the C ABI."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from tests.util import REL_TOL, gemm_error
+
+pytestmark = pytest.mark.gpu
+
+
+def _rand(shape, seed):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed))
+
+
+SHAPES = [(1, 1, 1), (5, 3, 2), (1000, 602, 16), (777, 16, 41), (300, 128, 16), (4099, 300, 24), (513, 16, 602),
+          (130, 41, 16), (2000, 64, 100), (50, 700, 70)]
+
+
+@pytest.mark.parametrize("n,k,fo", SHAPES)
+def test_dense_xw(cuda, n, k, fo):
+    from cagnet_amd import ops
+    X, W = _rand((n, k), 1), _rand((k, fo), 2)
+    Z = ops.dense_xw(X.to(cuda), W.to(cuda))
+    assert gemm_error(Z, X, W) <= REL_TOL
+    Zr = ops.dense_xw(X.to(cuda), W.to(cuda), relu=True)
+    assert torch.equal(Zr, torch.relu(Z))   # same accumulation, only the store differs
+
+
+@pytest.mark.parametrize("n,k,fo", SHAPES)
+def test_dense_gwt(cuda, n, k, fo):
+    from cagnet_amd import ops
+    G, W = _rand((n, fo), 3), _rand((k, fo), 4)
+    dX = ops.dense_gwt(G.to(cuda), W.to(cuda))
+    assert gemm_error(dX, G, W.t()) <= REL_TOL
+
+
+@pytest.mark.parametrize("n,k,fo", SHAPES + [(100000, 602, 16), (200000, 16, 41)])
+def test_dense_xtg(cuda, n, k, fo):
+    from cagnet_amd import ops
+    X, G = _rand((n, k), 5), _rand((n, fo), 6)
+    dW = ops.dense_xtg(X.to(cuda), G.to(cuda))
+    assert gemm_error(dW, X.t(), G) <= REL_TOL
+    assert torch.equal(dW, ops.dense_xtg(X.to(cuda), G.to(cuda)))  # fixed slice order: bit identical
+
+
+def test_dense_strided_operands(cuda):
+    """Row stride larger than the width (a column slice of a wider matrix) is passed as ld."""
+    from cagnet_amd import ops
+    big = _rand((300, 700), 7).to(cuda)
+    X = big[:, 10:612]                      # 602 wide, ld 700, base not 16-byte aligned
+    W = _rand((602, 16), 8).to(cuda)
+    assert gemm_error(ops.dense_xw(X, W), X.cpu(), W.cpu()) <= REL_TOL
+
+
+@pytest.mark.parametrize("n,c", [(1, 1), (7, 8), (1000, 41), (333, 24), (50, 256), (4097, 16)])
+def test_log_softmax_and_relu(cuda, n, c):
+    from cagnet_amd import ops
+    z = (_rand((n, c), 9) * 5.0)
+    out = ops.log_softmax_fwd(z.to(cuda))
+    ref = F.log_softmax(z.double(), dim=1)
+    assert float((out.cpu().double() - ref).abs().max()) <= 1e-5 * max(1.0, float(ref.abs().max()))
+    g = _rand((n, c), 10)
+    dz = ops.log_softmax_bwd(g.to(cuda), out)
+    zr = z.double().requires_grad_(True)
+    (F.log_softmax(zr, dim=1) * g.double()).sum().backward()
+    scale = g.double().abs().sum(dim=1, keepdim=True)
+    assert float(((dz.cpu().double() - zr.grad).abs() / scale.clamp_min(1e-30)).max()) <= REL_TOL
+    h = ops.relu_fwd(z.to(cuda))
+    assert torch.equal(h.cpu(), torch.relu(z))
+    assert torch.equal(ops.relu_bwd(g.to(cuda), h).cpu(), g * (z > 0))
+
+
+@pytest.mark.parametrize("n,c,frac", [(1, 3, 1.0), (1000, 41, 0.66), (5000, 8, 1.0), (70000, 24, 0.3), (300, 5, 0.0)])
+def test_nll_loss_forward_backward(cuda, n, c, frac):
+    from cagnet_amd import ops
+    gen = torch.Generator().manual_seed(11)
+    logp = F.log_softmax(torch.randn(n, c, generator=gen), dim=1)
+    y = torch.randint(0, c, (n,), generator=gen)
+    mask = None if frac >= 1.0 else (torch.rand(n, generator=gen) < frac)
+    loss, count = ops.nll_loss_fwd(logp.to(cuda), y.to(cuda), None if mask is None else mask.to(cuda))
+    sel = slice(None) if mask is None else mask
+    expect_count = n if mask is None else int(mask.sum())
+    assert int(count) == expect_count
+    if expect_count == 0:
+        assert float(loss) == 0.0           # the reference's fake_loss branch (gcn_distr.py:359-362)
+    else:
+        ref = F.nll_loss(logp.double()[sel], y[sel])
+        assert abs(float(loss) - float(ref)) <= 1e-5 * max(1.0, abs(float(ref)))
+        assert float(loss) == float(ops.nll_loss_fwd(logp.to(cuda), y.to(cuda),
+                                                     None if mask is None else mask.to(cuda))[0])
+    # gradients: separate kernels and the fused one against autograd
+    gs = torch.tensor(0.5)
+    d = ops.nll_loss_bwd(y.to(cuda), None if mask is None else mask.to(cuda), count, gs.to(cuda), n, c)
+    lp = logp.double().requires_grad_(True)
+    if expect_count:
+        (F.nll_loss(lp[sel], y[sel]) * 0.5).backward()
+        assert float((d.cpu().double() - lp.grad).abs().max()) <= 1e-6
+    else:
+        assert torch.count_nonzero(d) == 0
+    z = torch.randn(n, c, generator=gen)
+    out = ops.log_softmax_fwd(z.to(cuda))
+    fused = ops.log_softmax_nll_bwd(out, y.to(cuda), None if mask is None else mask.to(cuda), count, gs.to(cuda))
+    two_step = ops.log_softmax_bwd(d, out)
+    assert float((fused - two_step).abs().max()) <= 1e-6
+    if expect_count:
+        zr = z.double().requires_grad_(True)
+        (F.nll_loss(F.log_softmax(zr, dim=1)[sel], y[sel]) * 0.5).backward()
+        assert float((fused.cpu().double() - zr.grad).abs().max()) <= 1e-6

@@ -1,0 +1,122 @@
+"""GPU parity of GCNFunc / train (one GPU, blocks resident) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from cagnet_amd import synth
+from oracle import gcn_oracle as orc
+from tests.util import LOSS_TOL, REL_TOL
+
+pytestmark = pytest.mark.gpu
+
+
+class _Data:
+    def __init__(self, y, mask):
+        self.y, self.train_mask = y, mask
+
+
+def _block(p, cuda, transpose=False):
+    from cagnet_amd import ops
+    return ops.CsrMatrix(p.row.int().to(cuda), p.col.int().to(cuda), p.val.to(cuda), p.n, p.n, transpose=transpose)
+
+
+def _close(got, ref64, what, tol=2e-4):
+    """Layer outputs and gradients chain several products; compare to the fp64 oracle relative to
+    the largest entry (the per-product 1e-5 bound is checked kernel by kernel elsewhere)."""
+    got = got.detach().cpu().double()
+    scale = max(float(ref64.abs().max()), 1e-30)
+    err = float((got - ref64).abs().max()) / scale
+    assert err <= tol, f"{what}: {err}"
+
+
+@pytest.mark.parametrize("transpose", [False, True])
+def test_forward_backward_matches_oracle(cuda, transpose):
+    from cagnet_amd import gcn
+    p = synth.make_problem(scale=11, n_edges=16384, features=128, hidden=16, classes=8, mask_fraction=0.66, seed=3)
+    A = orc.coo_tensor(p.row, p.col, p.val, p.n, p.n, torch.float64)
+    ref = orc.forward_backward(p.x, p.w1, p.w2, [A], p.y, p.train_mask, dtype=torch.float64)
+
+    blk = _block(p, cuda, transpose)
+    x = p.x.to(cuda).requires_grad_(True)
+    w1 = p.w1.to(cuda).requires_grad_(True)
+    w2 = p.w2.to(cuda).requires_grad_(True)
+    h = gcn.GCNFunc.apply(x, w1, p.n, [blk], 0, 1, None, F.relu)
+    out = gcn.GCNFunc.apply(h, w2, p.n, [blk], 0, 1, None, F.log_softmax)
+    loss = gcn.masked_nll_loss(out, p.y.to(cuda), p.train_mask.to(cuda))
+    loss.backward()
+    assert abs(float(loss) - float(ref["loss"])) <= LOSS_TOL
+    _close(h, ref["hidden"], "hidden")
+    _close(out, ref["outputs"], "outputs")
+    _close(w2.grad, ref["dw2"], "dw2")
+    _close(w1.grad, ref["dw1"], "dw1")
+    _close(x.grad, ref["dx"], "dx")
+
+
+def test_training_losses_match_oracle(cuda):
+    """100 epochs of SGD lr 0.01 on the R-MAT scale-12 plumbing configuration: per-epoch loss
+    within 1e-4 of the fp32 CPU oracle and of its fp64 twin."""
+    from cagnet_amd import gcn
+    p = synth.make_problem(scale=12, n_edges=32768, features=128, hidden=16, classes=8, mask_fraction=1.0, seed=0)
+    A = orc.coo_tensor(p.row, p.col, p.val, p.n, p.n, torch.float32)
+    ref32, _, _ = orc.train_epochs(p.x, p.w1, p.w2, [A], p.y, p.train_mask, epochs=100, dtype=torch.float32)
+    ref64, w1_64, w2_64 = orc.train_epochs(p.x, p.w1, p.w2, [A], p.y, p.train_mask, epochs=100, dtype=torch.float64)
+
+    blk = _block(p, cuda, transpose=True)
+    x = p.x.to(cuda)
+    w1 = p.w1.to(cuda).requires_grad_(True)
+    w2 = p.w2.to(cuda).requires_grad_(True)
+    opt = torch.optim.SGD([w1, w2], lr=0.01)
+    data = _Data(p.y.to(cuda), p.train_mask.to(cuda))
+    losses = []
+    for _ in range(100):
+        gcn.train(x, w1, w2, p.n, [blk], opt, data, 0, 1, None)
+        losses.append(float(gcn.train.last_loss))
+    assert max(abs(a - b) for a, b in zip(losses, ref64)) <= LOSS_TOL
+    assert max(abs(a - b) for a, b in zip(losses, ref32)) <= LOSS_TOL
+    assert losses[-1] < losses[0]
+    _close(w1, w1_64, "w1 after 100 epochs", 1e-3)
+    _close(w2, w2_64, "w2 after 100 epochs", 1e-3)
+
+
+def test_one_rank_share_of_2d_grid(cuda):
+    """One rank's share of the 4x4 2D algorithm (gcn_distr_2d.py:333-417) with the broadcast
+    operands resident: z = sum_k A(r,k) H_k over 4 stages, both layers, forward and backward."""
+    from cagnet_amd import gcn, ops
+    q, r = 4, 1
+    p = synth.make_problem(n=2003, target_nnz=60001, features=64, hidden=16, classes=7, mask_fraction=0.5, seed=5)
+    b = synth.block_bounds_2d(p.n, q)
+    assert b == orc.block_bounds_2d(p.n, q)
+    rows = b[r + 1] - b[r]
+    blocks_gpu, blocks_cpu = [], []
+    for k in range(q):
+        rr, cc, vv = synth.coo_block(p.row, p.col, p.val, b[r], b[r + 1], b[k], b[k + 1])
+        blocks_gpu.append(ops.CsrMatrix(rr.int().to(cuda), cc.int().to(cuda), vv.to(cuda), rows, b[k + 1] - b[k]))
+        blocks_cpu.append(orc.coo_tensor(rr, cc, vv, rows, b[k + 1] - b[k], torch.float64))
+    gen = torch.Generator().manual_seed(17)
+
+    def peers(width):
+        return [None if k == r else torch.randn(b[k + 1] - b[k], width, generator=gen) for k in range(q)]
+
+    # the forward peers of a layer have that layer's input width, the backward peers its output width
+    p1f, p1b, p2f, p2b = peers(64), peers(16), peers(16), peers(7)
+    x_r = p.x[b[r]:b[r + 1]]
+    y_r, m_r = p.y[b[r]:b[r + 1]], p.train_mask[b[r]:b[r + 1]]
+    ref = orc.forward_backward(x_r, p.w1, p.w2, blocks_cpu, y_r, m_r, dtype=torch.float64,
+                               peers1=(p1f, p1b), peers2=(p2f, p2b), rank=r)
+
+    dev = lambda lst: [None if t is None else t.to(cuda) for t in lst]
+    g1 = gcn.ResidentBlocks(dev(p1f), dev(p1b))
+    g2 = gcn.ResidentBlocks(dev(p2f), dev(p2b))
+    x = x_r.to(cuda).requires_grad_(True)
+    w1 = p.w1.to(cuda).requires_grad_(True)
+    w2 = p.w2.to(cuda).requires_grad_(True)
+    h = gcn.GCNFunc.apply(x, w1, rows, blocks_gpu, r, q, g1, F.relu)
+    out = gcn.GCNFunc.apply(h, w2, rows, blocks_gpu, r, q, g2, F.log_softmax)
+    loss = gcn.masked_nll_loss(out, y_r.to(cuda), m_r.to(cuda))
+    loss.backward()
+    assert abs(float(loss) - float(ref["loss"])) <= LOSS_TOL
+    _close(out, ref["outputs"], "outputs")
+    _close(w1.grad, ref["dw1"], "dw1")
+    _close(w2.grad, ref["dw2"], "dw2")
+    _close(x.grad, ref["dx"], "dx")

@@ -1,0 +1,247 @@
+"""GPU parity of coo2csr / transpose / SpMM through the C ABI against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from tests.util import REL_TOL, random_coo, small_graph, spmm_error
+from oracle import gcn_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _i32(t, dev):
+    return t.to(torch.int32).to(dev)
+
+
+@pytest.mark.parametrize("n,nnz_per_row,seed", [(1, 1, 0), (7, 2, 1), (1000, 5, 2), (5000, 40, 3), (100000, 3, 4)])
+def test_rowptr_sorted_bit_exact(cuda, n, nnz_per_row, seed):
+    from cagnet_amd import ops
+    row, col, val = random_coo(n, n, n * nnz_per_row, seed)
+    got = ops.coo2csr_rowptr(_i32(row, cuda), n).cpu().numpy()
+    assert np.array_equal(got, orc.coo2csr_rowptr(row.numpy(), n))
+
+
+def test_rowptr_empty_rows_and_empty_matrix(cuda):
+    from cagnet_amd import ops
+    # long runs of empty rows (wave-cooperative fill) and rows only at the far end
+    row = torch.tensor([3, 3, 500, 99998], dtype=torch.int32, device=cuda)
+    got = ops.coo2csr_rowptr(row, 100000).cpu().numpy()
+    assert np.array_equal(got, orc.coo2csr_rowptr(row.cpu().numpy(), 100000))
+    got = ops.coo2csr_rowptr(torch.empty(0, dtype=torch.int32, device=cuda), 1000).cpu().numpy()
+    assert np.array_equal(got, np.zeros(1001, dtype=np.int32))
+    got = ops.coo2csr_rowptr(torch.empty(0, dtype=torch.int32, device=cuda), 0).cpu().numpy()
+    assert np.array_equal(got, np.zeros(1, dtype=np.int32))
+
+
+@pytest.mark.parametrize("n,m,nnz,seed", [(1, 1, 1, 0), (13, 7, 40, 1), (300, 70000, 50000, 2), (70000, 300, 50000, 3),
+                                          (4096, 4096, 200000, 4), (1 << 17, 1 << 17, 600000, 5)])
+def test_coo2csr_unsorted_bit_exact(cuda, n, m, nnz, seed):
+    from cagnet_amd import ops
+    row, col, val = random_coo(n, m, nnz, seed, sort=False)
+    rp, ci, vv, perm = ops.coo2csr(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, m, return_perm=True)
+    erp, eci, evv, eperm = orc.coo2csr(row.numpy(), col.numpy(), val.numpy(), n, m)
+    assert np.array_equal(rp.cpu().numpy(), erp)
+    assert np.array_equal(ci.cpu().numpy(), eci)
+    assert np.array_equal(perm.cpu().numpy(), eperm)
+    assert np.array_equal(vv.cpu().numpy(), evv)  # values are moved, never recomputed: bit exact
+
+
+def test_coo2csr_duplicates_keep_input_order(cuda):
+    from cagnet_amd import ops
+    row = torch.tensor([2, 0, 2, 2, 0, 1], dtype=torch.int32)
+    col = torch.tensor([1, 3, 1, 0, 3, 2], dtype=torch.int32)
+    val = torch.arange(6, dtype=torch.float32)
+    rp, ci, vv, perm = ops.coo2csr(row.to(cuda), col.to(cuda), val.to(cuda), 3, 4, return_perm=True)
+    erp, eci, evv, eperm = orc.coo2csr(row.numpy(), col.numpy(), val.numpy(), 3, 4)
+    assert np.array_equal(perm.cpu().numpy(), eperm)
+    assert np.array_equal(vv.cpu().numpy(), evv)
+    assert np.array_equal(rp.cpu().numpy(), erp)
+
+
+@pytest.mark.parametrize("n,m,nnz,seed", [(13, 7, 40, 1), (300, 70000, 50000, 2), (70000, 300, 50000, 3),
+                                          (1 << 16, 1 << 16, 500000, 5)])
+def test_csr_transpose_bit_exact_and_involution(cuda, n, m, nnz, seed):
+    from cagnet_amd import ops
+    row, col, val = random_coo(n, m, nnz, seed)
+    rp, ci, vv, _ = orc.coo2csr(row.numpy(), col.numpy(), val.numpy(), n, m)
+    d = [torch.from_numpy(a).to(cuda) for a in (rp, ci, vv)]
+    cp, ri, vt, perm = ops.csr_transpose(d[0], d[1], d[2], n, m, return_perm=True)
+    ecp, eri, evt, eperm = orc.csr_transpose(rp, ci, vv, n, m)
+    assert np.array_equal(cp.cpu().numpy(), ecp)
+    assert np.array_equal(ri.cpu().numpy(), eri)
+    assert np.array_equal(vt.cpu().numpy(), evt)
+    assert np.array_equal(perm.cpu().numpy(), eperm)
+    # T(T(A)) == A
+    rp2, ci2, vv2 = ops.csr_transpose(cp, ri, vt, m, n)
+    assert np.array_equal(rp2.cpu().numpy(), rp)
+    assert np.array_equal(ci2.cpu().numpy(), ci)
+    assert np.array_equal(vv2.cpu().numpy(), vv)
+
+
+def test_coo_check_reports(cuda):
+    from cagnet_amd import ops
+    ok_r = torch.tensor([0, 0, 1, 2], dtype=torch.int32, device=cuda)
+    ok_c = torch.tensor([0, 2, 1, 0], dtype=torch.int32, device=cuda)
+    ops.coo_check(ok_r, ok_c, 3, 3, require_sorted=2)
+    with pytest.raises(ops.CagnetError, match="CG_ERR_INDEX"):
+        ops.coo_check(ok_r, ok_c, 2, 3)
+    with pytest.raises(ops.CagnetError, match="CG_ERR_INDEX"):
+        ops.coo_check(ok_r, torch.tensor([0, -1, 1, 0], dtype=torch.int32, device=cuda), 3, 3)
+    with pytest.raises(ops.CagnetError, match="CG_ERR_UNSORTED"):
+        ops.coo_check(torch.tensor([0, 2, 1, 2], dtype=torch.int32, device=cuda), ok_c, 3, 3)
+    with pytest.raises(ops.CagnetError, match="CG_ERR_UNSORTED"):
+        ops.coo_check(ok_r, torch.tensor([2, 0, 1, 0], dtype=torch.int32, device=cuda), 3, 3, require_sorted=2)
+
+
+WIDTHS = [1, 3, 16, 24, 41, 64, 100, 128, 300, 602, 1300]
+
+
+@pytest.mark.parametrize("f", WIDTHS)
+def test_spmm_handle_matches_oracle(cuda, f):
+    """Power-law graph (R-MAT scale 11, degrees from 1 to hundreds) at every width class."""
+    from cagnet_amd import ops
+    row, col, val, n = small_graph(11, 30000, seed=f)
+    B = torch.randn(n, f, generator=torch.Generator().manual_seed(f))
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n)
+    got = A.spmm(B.to(cuda))
+    assert spmm_error(got, row, col, val, n, n, B) <= REL_TOL
+    # accumulate form: C = C0 + A B (beta = 1), the reference operator's semantics
+    C0 = torch.randn(n, f, generator=torch.Generator().manual_seed(f + 1))
+    C = C0.to(cuda).clone()
+    A.spmm(B.to(cuda), out=C, beta=1.0)
+    assert spmm_error(C, row, col, val, n, n, B, C0) <= REL_TOL
+
+
+@pytest.mark.parametrize("f", [16, 41, 602])
+def test_spmm_gpu_one_shot_matches_oracle(cuda, f):
+    from cagnet_amd.sparse_coo_tensor_cpp import spmm_gpu
+    row, col, val, n = small_graph(10, 20000, seed=100 + f)
+    B = torch.randn(n, f, generator=torch.Generator().manual_seed(f))
+    C0 = torch.randn(n, f, generator=torch.Generator().manual_seed(f + 1))
+    C = C0.to(cuda).clone()
+    ret = spmm_gpu(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n, B.to(cuda), C)
+    assert ret is None
+    assert spmm_error(C, row, col, val, n, n, B, C0) <= REL_TOL
+    assert C.is_contiguous()
+
+
+@pytest.mark.parametrize("f", [16, 41, 128, 602])
+def test_spmm_split_rows(cuda, f):
+    """Rows longer than a segment (1024 to 4096 entries by width class) are split over several
+    wavefronts and recombined in order: a dense-ish rectangular block whose 40 rows hold ~9000
+    entries each exercises the partial-row path at every class."""
+    from cagnet_amd import ops
+    n, m = 40, 12000
+    row, col, val = random_coo(n, m, n * 9000, seed=f)
+    B = torch.randn(m, f, generator=torch.Generator().manual_seed(1))
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, m)
+    got = A.spmm(B.to(cuda))
+    assert spmm_error(got, row, col, val, n, m, B) <= REL_TOL
+    C0 = torch.randn(n, f, generator=torch.Generator().manual_seed(2))
+    C = C0.to(cuda).clone()
+    A.spmm(B.to(cuda), out=C, beta=1.0)
+    assert spmm_error(C, row, col, val, n, m, B, C0) <= REL_TOL
+
+
+def test_spmm_special_cases(cuda):
+    from cagnet_amd import ops
+    n, f = 257, 48
+    B = torch.randn(n, f, generator=torch.Generator().manual_seed(0)).to(cuda)
+    eye = torch.arange(n, dtype=torch.int32, device=cuda)
+    I = ops.CsrMatrix(eye, eye, torch.ones(n, device=cuda), n, n)
+    C0 = torch.randn(n, f, generator=torch.Generator().manual_seed(1)).to(cuda)
+    C = C0.clone()
+    I.spmm(B, out=C, beta=1.0)
+    assert torch.equal(C, C0 + B)            # A = I: C = C0 + B exactly
+    assert torch.equal(I.spmm(B), B)
+    # empty rows leave C untouched under beta = 1 and become zero under beta = 0
+    row = torch.tensor([5, 5, 200], dtype=torch.int32, device=cuda)
+    col = torch.tensor([0, 9, 256], dtype=torch.int32, device=cuda)
+    val = torch.tensor([1.0, 2.0, -1.0], device=cuda)
+    S = ops.CsrMatrix(row, col, val, n, n)
+    C = C0.clone()
+    S.spmm(B, out=C, beta=1.0)
+    expect = C0.clone()
+    expect[5] += B[0] + 2.0 * B[9]
+    expect[200] -= B[256]
+    assert torch.allclose(C, expect, rtol=0, atol=1e-6)
+    untouched = torch.ones(n, dtype=torch.bool)
+    untouched[[5, 200]] = False
+    assert torch.equal(C[untouched.to(cuda)], C0[untouched.to(cuda)])
+    Z = S.spmm(B)
+    assert torch.count_nonzero(Z[untouched.to(cuda)]) == 0
+    # all-empty matrix
+    E = ops.CsrMatrix(torch.empty(0, dtype=torch.int32, device=cuda), torch.empty(0, dtype=torch.int32, device=cuda),
+                      torch.empty(0, device=cuda), n, n)
+    assert torch.count_nonzero(E.spmm(B)) == 0
+
+
+def test_spmm_transpose_and_symmetry(cuda):
+    from cagnet_amd import ops
+    # rectangular, non-symmetric: A^T G against the oracle on the transposed triplets
+    n, m, f = 500, 1300, 41
+    row, col, val = random_coo(n, m, 20000, seed=9)
+    G = torch.randn(n, f, generator=torch.Generator().manual_seed(3))
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, m, transpose=True)
+    got = A.spmm(G.to(cuda), transpose=True)
+    order = np.lexsort((row.numpy(), col.numpy()))
+    assert spmm_error(got, col[order], row[order], val[order], m, n, G) <= REL_TOL
+    with pytest.raises(ops.CagnetError, match="CG_ERR_NO_TRANSPOSE"):
+        ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, m).spmm(G.to(cuda), transpose=True)
+    # symmetric normalised graph: A^T G == A G bit for bit (same rows, same order)
+    row, col, val, n = small_graph(10, 20000, seed=77)
+    S = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n, transpose=True)
+    G = torch.randn(n, 16, generator=torch.Generator().manual_seed(4)).to(cuda)
+    assert torch.equal(S.spmm(G), S.spmm(G, transpose=True))
+    a, t = S.arrays(False), S.arrays(True)
+    assert all(torch.equal(x, y) for x, y in zip(a, t))
+
+
+def test_spmm_deterministic_and_linear(cuda):
+    from cagnet_amd import ops
+    row, col, val, n = small_graph(12, 32768, seed=5)
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n)
+    g = torch.Generator().manual_seed(6)
+    B1, B2 = torch.randn(n, 602, generator=g).to(cuda), torch.randn(n, 602, generator=g).to(cuda)
+    r1 = A.spmm(B1)
+    assert torch.equal(r1, A.spmm(B1))       # fixed summation order: bit identical
+    lin = A.spmm(B1 + B2)
+    ref = r1 + A.spmm(B2)
+    scale = (A.spmm(B1.abs()) + A.spmm(B2.abs())).clamp_min(1e-30)
+    assert float(((lin - ref).abs() / scale).max()) <= 4e-6
+
+
+def test_stage_splitting_invariance(cuda):
+    """sum_k A[:, block k] H[block k] == A H: the local form of the 1D/2D stage loops."""
+    from cagnet_amd import ops, synth
+    row, col, val, n = small_graph(11, 30000, seed=8)
+    f = 64
+    H = torch.randn(n, f, generator=torch.Generator().manual_seed(7))
+    bounds = synth.block_bounds_2d(n, 4)
+    z = None
+    for k in range(4):
+        r, c, v = synth.coo_block(row, col, val, 0, n, bounds[k], bounds[k + 1])
+        blk = ops.CsrMatrix(_i32(r, cuda), _i32(c, cuda), v.to(cuda), n, bounds[k + 1] - bounds[k])
+        Hk = H[bounds[k]:bounds[k + 1]].to(cuda)
+        z = blk.spmm(Hk) if z is None else blk.spmm(Hk, out=z, beta=1.0)
+    assert spmm_error(z, row, col, val, n, n, H) <= REL_TOL
+
+
+def test_spmm_rejects_bad_arguments(cuda):
+    from cagnet_amd import ops
+    row, col, val, n = small_graph(8, 2000, seed=1)
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n)
+    with pytest.raises(ValueError):
+        A.spmm(torch.zeros(n + 1, 4, device=cuda))
+    with pytest.raises(ValueError):
+        A.spmm(torch.zeros(n, 4))             # CPU tensor: no CPU path
+    with pytest.raises(TypeError):
+        A.spmm(torch.zeros(n, 4, device=cuda, dtype=torch.float64))
+    with pytest.raises(ops.CagnetError, match="CG_ERR_INDEX"):
+        ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n - 1, n)
+    with pytest.raises(ops.CagnetError, match="CG_ERR_UNSORTED"):
+        ops.CsrMatrix(_i32(row.flip(0), cuda), _i32(col.flip(0), cuda), val.flip(0).to(cuda), n, n)
+    # the same unsorted triplets are fine on the general path
+    U = ops.CsrMatrix(_i32(row.flip(0), cuda), _i32(col.flip(0), cuda), val.flip(0).to(cuda), n, n, is_sorted=False)
+    B = torch.randn(n, 16, generator=torch.Generator().manual_seed(2)).to(cuda)
+    assert torch.equal(U.spmm(B), A.spmm(B))
