@@ -1,0 +1,241 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-rank GCN compute path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload reddit|rmat20|amazon|tiny]
+
+A step is one epoch of the 2-layer GCN (forward, loss, backward, Adam step: `train`,
+gcn_distr.py:341-366) over a seeded synthetic graph that is resident in HBM before the timed
+region starts.  The default workload is the Reddit-shaped configuration the headline metric is
+quoted on: 232,965 vertices, ~114.6 M stored entries, 602 features, hidden 16, 41 classes.
+
+One JSON line is printed:
+  value      SpMM GFLOP/s (2*nnz*f / kernel time) of the dominant launch, the f = 602 forward
+             SpMM, measured with HIP events on the launch stream inside the timed epochs
+  ms_per_step  epoch wall time
+  roofline   algorithmic bytes of that launch / its duration, against 8 TB/s
+  cpu_baseline  torch.sparse.mm on the host cores over a bounded row sample of the same product
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+WORKLOADS = {
+    # name: graph spec, features, hidden, classes, mask fraction
+    "reddit": dict(n=232_965, target_nnz=114_615_892, features=602, hidden=16, classes=41, mask=0.66,
+                   desc="Reddit-shaped 2-layer GCN: 232,965 vertices, ~114.6M nnz (R-MAT .57/.19/.19/.05, "
+                        "symmetrised, self-loops, GCN-normalised), 602 features, hidden 16, 41 classes, 66% mask"),
+    "amazon": dict(n=14_249_639, target_nnz=230_600_000, features=300, hidden=16, classes=24, mask=1.0,
+                   desc="Amazon-shaped 2-layer GCN: 14,249,639 vertices, ~230.6M nnz, 300 features, hidden 16, 24 classes"),
+    "rmat20": dict(scale=20, n_edges=16_777_216, features=128, hidden=16, classes=8, mask=1.0,
+                   desc="R-MAT scale 20 (1,048,576 vertices, 16,777,216 directed edges), 128 features, hidden 16"),
+    "tiny": dict(scale=12, n_edges=32_768, features=128, hidden=16, classes=8, mask=1.0,
+                 desc="R-MAT scale 12 plumbing configuration"),
+}
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs,
+# scaled by a copy kernel of known size; filled in from profiles/ once measured (None = not measured).
+MEASURED_TRAFFIC_BYTES = {"reddit": None}
+
+
+def spmm_alg_bytes(nnz: int, n: int, m: int, f: int, reads_c: bool) -> int:
+    """Compulsory traffic of one SpMM launch: col + val once, rowptr once, B once, C written once
+    (and read once when it accumulates)."""
+    return 8 * nnz + 4 * (n + 1) + 4 * m * f + 4 * n * f * (2 if reads_c else 1)
+
+
+def prof_read(lib, name: str):
+    ms, cnt = ctypes.c_double(0.0), ctypes.c_int64(0)
+    lib.cg_prof_read(name.encode(), ctypes.byref(ms), ctypes.byref(cnt))
+    return ms.value, cnt.value
+
+
+def cpu_baseline(prob, f: int, budget_s: float = 25.0):
+    """The oracle's SpMM (torch.sparse.mm on a coalesced COO tensor: the reference's tensor type,
+    gcn_distr.py:493-512, and the torch.sparse line it keeps beside spmm_gpu, gcn_distr_3d.py:478)
+    timed on the host cores over every 8th row of A times the full dense operand."""
+    import torch
+    from oracle import gcn_oracle as orc
+
+    stride = 8 if prob.nnz > 4_000_000 else 1
+    keep = (prob.row % stride) == 0
+    row = (prob.row[keep] // stride).cpu()
+    col = prob.col[keep].cpu()
+    val = prob.val[keep].cpu()
+    n_s = (prob.n + stride - 1) // stride
+    B = prob.x[:, :f].cpu().contiguous()
+    A = orc.coo_tensor(row, col, val, n_s, prob.n, torch.float32)
+    nnz_s = int(val.numel())
+    times = []
+    t_begin = time.perf_counter()
+    for rep in range(4):
+        t0 = time.perf_counter()
+        torch.sparse.mm(A, B)
+        dt = time.perf_counter() - t0
+        if rep > 0:
+            times.append(dt)
+        if time.perf_counter() - t_begin > budget_s and times:
+            break
+    times.sort()
+    t = times[len(times) // 2]
+    return {
+        "value": round(2.0 * nnz_s * f / t / 1e9, 3),
+        "unit": "GFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"torch.sparse.mm(COO fp32) of every {stride}th row of A ({n_s} x {prob.n}, {nnz_s} nnz) times the "
+                  f"full {prob.n} x {f} dense operand; median of {len(times)} after 1 warm-up; host has "
+                  f"{os.cpu_count()} logical CPUs",
+        "seconds_per_rep": round(t, 4),
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="reddit", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs the per-rank compute path on ONE GPU; --gpus {args.gpus} is not supported "
+              "(no collectives, no sharding). Run with --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from cagnet_amd import build as cg_build
+
+    if not cg_build.LIB_PATH.exists():
+        cg_build.build_library()
+    from cagnet_amd import _lib, gcn, ops, synth
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; cagnet_amd has no CPU path", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    spec = WORKLOADS[args.workload]
+
+    t0 = time.perf_counter()
+    prob = synth.make_problem(scale=spec.get("scale"), n_edges=spec.get("n_edges"), n=spec.get("n"),
+                              target_nnz=spec.get("target_nnz"), features=spec["features"], hidden=spec["hidden"],
+                              classes=spec["classes"], mask_fraction=spec["mask"], seed=args.seed, device=dev)
+    torch.cuda.synchronize()
+    t_gen = time.perf_counter() - t0
+    n, nnz, f_in, hidden, classes = prob.n, prob.nnz, spec["features"], spec["hidden"], spec["classes"]
+
+    t0 = time.perf_counter()
+    row32, col32 = prob.row.int(), prob.col.int()
+    blk = ops.CsrMatrix(row32, col32, prob.val, n, n, is_sorted=True, transpose=True)
+    torch.cuda.synchronize()
+    t_build = time.perf_counter() - t0
+    del row32, col32
+
+    class Data:
+        y = prob.y
+        train_mask = prob.train_mask
+
+    x = prob.x.requires_grad_(True)  # the reference asks for the input gradient too (gcn_distr.py:736)
+    w1 = prob.w1.clone().requires_grad_(True)
+    w2 = prob.w2.clone().requires_grad_(True)
+    opt = torch.optim.Adam([w1, w2], lr=0.01)
+
+    def step():
+        gcn.train(x, w1, w2, n, [blk], opt, Data, 0, 1, None)
+        x.grad = None
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.lib.cg_prof_enable(1)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    _lib.lib.cg_prof_enable(0)
+    ms_per_step = elapsed / args.steps * 1e3
+    loss = float(gcn.train.last_loss)
+
+    kernels = {}
+    widths = sorted({f_in, hidden, classes})
+    for f in widths:
+        for kname in ("spmm_rowseg", "spmm_reduce"):
+            ms, cnt = prof_read(_lib.lib, f"{kname}/f={f}")
+            if cnt:
+                kernels[f"{kname}/f={f}"] = {"launches": cnt, "avg_ms": ms / cnt}
+    for kname, ks in (("dense_xw", (f_in, hidden)), ("dense_gwt", (f_in, hidden)), ("dense_xtg", (f_in, hidden))):
+        for k in ks:
+            ms, cnt = prof_read(_lib.lib, f"{kname}/f={k}")
+            if cnt:
+                kernels[f"{kname}/k={k}"] = {"launches": cnt, "avg_ms": ms / cnt}
+
+    dom = kernels.get(f"spmm_rowseg/f={f_in}")
+    dom_ms = dom["avg_ms"] if dom else float("nan")
+    flops = 2.0 * nnz * f_in
+    gflops = flops / (dom_ms * 1e-3) / 1e9
+    alg_bytes = spmm_alg_bytes(nnz, n, n, f_in, reads_c=False)
+    achieved = alg_bytes / (dom_ms * 1e-3) / 1e9
+    gather_bytes = 8 * nnz + 4 * (n + 1) + 4 * nnz * f_in + 4 * n * f_in
+    spmm_total_ms = sum(v["avg_ms"] * v["launches"] for k, v in kernels.items() if k.startswith("spmm")) / args.steps
+    dense_total_ms = sum(v["avg_ms"] * v["launches"] for k, v in kernels.items() if k.startswith("dense")) / args.steps
+
+    out = {
+        "metric": "SpMM GFLOP/s (2*nnz*f) of the f=%d forward SpMM inside the 2-layer GCN epoch" % f_in,
+        "value": round(gflops, 2),
+        "unit": "GFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": spec["desc"], "name": args.workload, "n": n, "nnz": nnz, "features": f_in,
+                   "hidden": hidden, "classes": classes, "optimizer": "adam lr 0.01", "input_grad": True,
+                   "seeds": prob.seeds},
+        "epoch_ms": round(ms_per_step, 4),
+        "scomp_ms_per_epoch": round(spmm_total_ms, 4),
+        "dcomp_ms_per_epoch": round(dense_total_ms, 4),
+        "final_loss": loss,
+        "spmm_gbs_algorithmic": round(achieved, 2),
+        "spmm_gbs_gather_model": round(gather_bytes / (dom_ms * 1e-3) / 1e9, 2),
+        "spmm_time_lower_bound_ms": round(max(alg_bytes / 8e12, flops / 157.3e12) * 1e3, 4),
+        "kernels": {k: {"launches": v["launches"], "avg_ms": round(v["avg_ms"], 5)} for k, v in kernels.items()},
+        "setup_s": {"generate": round(t_gen, 2), "csr_and_transpose_build": round(t_build, 3)},
+        "roofline": {
+            "kernel": "spmm_rowseg_kernel f=%d (beta=0)" % f_in,
+            "bound": "hbm",
+            "achieved": round(achieved, 2),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 5),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "algorithmic_bytes": alg_bytes,
+            "avg_launch_ms": round(dom_ms, 5),
+        },
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(prob, f_in)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -60,6 +60,8 @@ _SIGNATURES = {
     "cg_nll_loss_fwd": [P, c_int64, P, P, c_int64, c_int32, P, P, P],
     "cg_nll_loss_bwd": [P, P, P, P, P, c_int64, c_int64, c_int32, P],
     "cg_log_softmax_nll_bwd": [P, c_int64, P, P, P, P, P, c_int64, c_int64, c_int32, P],
+    "cg_prof_enable": [c_int],
+    "cg_prof_read": [c_char_p, POINTER(ctypes.c_double), POINTER(c_int64)],
 }
 _RESTYPES = {"cg_status_string": c_char_p, "cg_last_error": c_char_p}
 
@@ -72,6 +74,11 @@ def _load() -> ctypes.CDLL:
             f"{LIB_PATH} is missing: build it with `python -m cagnet_amd.build` (hipcc, gfx950). "
             "cagnet_amd has no other backend."
         )
+    # One HIP runtime per process: torch ships its own libamdhip64.so.7, and the device pointers and
+    # streams handed to the library come from it.  Importing torch first makes the dynamic linker
+    # resolve the library's libamdhip64.so.7 dependency to that already loaded copy.
+    import torch  # noqa: F401
+
     lib = ctypes.CDLL(str(LIB_PATH))
     for name, argtypes in _SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError here means header and library disagree

@@ -40,6 +40,21 @@ int hip_fail(hipError_t e, const char *what, const char *file, int line);
 enum ScratchSlot { kSlotA = 0, kSlotB = 1, kSlotC = 2, kSlotD = 3, kNumSlots = 4 };
 int scratch_get(hipStream_t stream, int slot, size_t bytes, void **out);
 
+// ---- optional kernel timing with HIP events on the launch stream (runtime.hip) -------------------
+bool prof_on();
+void prof_begin(const char *name, int tag, hipStream_t stream);  // tag < 0: no "/f=" suffix
+void prof_end(hipStream_t stream);
+struct ProfScope {
+  hipStream_t s;
+  bool on;
+  ProfScope(const char *name, int tag, hipStream_t stream) : s(stream), on(prof_on()) {
+    if (on) prof_begin(name, tag, stream);
+  }
+  ~ProfScope() {
+    if (on) prof_end(s);
+  }
+};
+
 // ---- integer helpers ------------------------------------------------------------------------
 static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 static inline int bits_for(int32_t count) {  // number of bits needed to represent values in [0, count)

@@ -217,6 +217,7 @@ int cg_dense_xw(const float *d_X, int64_t ldx, const float *d_W, int64_t ldw, fl
   if (ldx < k || ldw < fo || ldz < fo) CG_FAIL(CG_ERR_SIZE, "cg_dense_xw: leading dimension too small");
   if (n == 0) return CG_OK;
   GemmArgs g{d_X, ldx, d_W, ldw, d_Z, ldz, n, fo, k, ceil_div64(k, kKT) * kKT, 1, relu ? 1 : 0};
+  ProfScope prof("dense_xw", k, (hipStream_t)stream);
   return launch_gemm<false, false>(g, (hipStream_t)stream);
 }
 
@@ -227,6 +228,7 @@ int cg_dense_gwt(const float *d_G, int64_t ldg, const float *d_W, int64_t ldw, f
   if (ldg < fo || ldw < fo || lddx < k) CG_FAIL(CG_ERR_SIZE, "cg_dense_gwt: leading dimension too small");
   if (n == 0) return CG_OK;
   GemmArgs g{d_G, ldg, d_W, ldw, d_dX, lddx, n, k, fo, ceil_div64(fo, kKT) * kKT, 1, 0};
+  ProfScope prof("dense_gwt", k, (hipStream_t)stream);
   return launch_gemm<false, true>(g, (hipStream_t)stream);
 }
 
@@ -244,6 +246,7 @@ int cg_dense_xtg(const float *d_X, int64_t ldx, const float *d_G, int64_t ldg, f
   if (kchunk < 4 * kKT) kchunk = 4 * kKT;
   splits = n > 0 ? ceil_div64(n, kchunk) : 1;
   GemmArgs g{d_X, ldx, d_G, ldg, d_dW, lddw, k, fo, n, kchunk, (int32_t)splits, 0};
+  ProfScope prof("dense_xtg", k, stream);
   if (splits <= 1) {
     g.splits = 1;
     g.kchunk = ceil_div64(n > 0 ? n : 1, kKT) * kKT;

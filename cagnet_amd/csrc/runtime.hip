@@ -1,8 +1,11 @@
 // Error reporting and the per (device, stream) scratch arena of libcagnet_amd.
 #include "common.h"
+#include <atomic>
 #include <map>
 #include <mutex>
+#include <string>
 #include <tuple>
+#include <vector>
 
 namespace cg {
 
@@ -57,9 +60,82 @@ int scratch_get(hipStream_t stream, int slot, size_t bytes, void **out) {
   return CG_OK;
 }
 
+// ---- event recorder ------------------------------------------------------------------------
+struct ProfRecord {
+  std::string name;
+  hipEvent_t start, stop;
+};
+static std::mutex g_prof_mu;
+static std::vector<ProfRecord> g_prof;
+static std::atomic<bool> g_prof_on{false};
+static thread_local int g_prof_open = -1;
+constexpr size_t kProfMaxRecords = 1 << 16;
+
+bool prof_on() { return g_prof_on.load(std::memory_order_relaxed); }
+
+void prof_begin(const char *name, int tag, hipStream_t stream) {
+  g_prof_open = -1;
+  ProfRecord r;
+  r.name = name;
+  if (tag >= 0) r.name += "/f=" + std::to_string(tag);
+  if (hipEventCreate(&r.start) != hipSuccess) return;
+  if (hipEventCreate(&r.stop) != hipSuccess) {
+    (void)hipEventDestroy(r.start);
+    return;
+  }
+  (void)hipEventRecord(r.start, stream);
+  std::lock_guard<std::mutex> lock(g_prof_mu);
+  if (g_prof.size() >= kProfMaxRecords) {  // full: drop this record rather than grow without bound
+    (void)hipEventDestroy(r.start);
+    (void)hipEventDestroy(r.stop);
+    return;
+  }
+  g_prof.push_back(r);
+  g_prof_open = (int)g_prof.size() - 1;
+}
+
+void prof_end(hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_prof_mu);
+  if (g_prof_open >= 0 && g_prof_open < (int)g_prof.size()) (void)hipEventRecord(g_prof[g_prof_open].stop, stream);
+  g_prof_open = -1;
+}
+
 }  // namespace cg
 
 extern "C" {
+
+int cg_prof_enable(int on) {
+  cg::g_prof_on.store(on != 0);
+  return CG_OK;
+}
+
+int cg_prof_read(const char *name, double *total_ms, int64_t *launches) {
+  using namespace cg;
+  if (!name || !total_ms || !launches) CG_FAIL(CG_ERR_NULL, "cg_prof_read: null pointer");
+  std::lock_guard<std::mutex> lock(g_prof_mu);
+  double total = 0.0;
+  int64_t count = 0;
+  std::vector<ProfRecord> keep;
+  for (auto &r : g_prof) {
+    if (r.name != name) {
+      keep.push_back(r);
+      continue;
+    }
+    float ms = 0.f;
+    if (hipEventSynchronize(r.stop) == hipSuccess && hipEventElapsedTime(&ms, r.start, r.stop) == hipSuccess) {
+      total += ms;
+      ++count;
+    } else {
+      (void)hipGetLastError();
+    }
+    (void)hipEventDestroy(r.start);
+    (void)hipEventDestroy(r.stop);
+  }
+  g_prof.swap(keep);
+  *total_ms = total;
+  *launches = count;
+  return CG_OK;
+}
 
 int cg_abi_version(void) { return CG_ABI_VERSION; }
 

@@ -512,8 +512,12 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
       CG_TRY(scratch_get(stream, kSlotA, (size_t)sc->nslots * ft * sizeof(float), &p));
       a.P = (float *)p;
     }
-    CG_TRY((launch_shape<true, false>(shape, a, stream)));
+    {
+      ProfScope prof("spmm_rowseg", f, stream);
+      CG_TRY((launch_shape<true, false>(shape, a, stream)));
+    }
     if (sc->nmulti > 0) {
+      ProfScope prof("spmm_reduce", f, stream);
       const int64_t threads = sc->nmulti * (int64_t)ft;
       spmm_reduce_kernel<<<(unsigned)ceil_div64(threads, kSpmmThreads), kSpmmThreads, 0, stream>>>(
           sc->multi_rows, sc->nmulti, s.rowptr, sc->pbase, sc->seg, a.P, Ct, ldc, ft, beta);

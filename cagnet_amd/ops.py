@@ -152,7 +152,7 @@ class _DeviceArray:
 
     def __init__(self, ptr: int, count: int, typestr: str):
         self.__cuda_array_interface__ = {
-            "shape": (count,), "typestr": typestr, "data": (ptr, True), "version": 2, "strides": None,
+            "shape": (count,), "typestr": typestr, "data": (ptr, False), "version": 2, "strides": None,
         }
 
 

@@ -168,6 +168,18 @@ int cg_log_softmax_nll_bwd(const float *d_logp, int64_t ld, const int64_t *d_y, 
                            const int64_t *d_count, const float *d_gscale, float *d_dz, int64_t lddz, int64_t n,
                            int32_t c, cg_stream_t stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Kernel timing (the reference brackets phases with wall clocks and device synchronisation,
+ * gcn_distr.py:66-94; here HIP events are recorded on the launch stream around single kernels).
+ * cg_prof_enable(1) starts recording, cg_prof_enable(0) stops.  cg_prof_read waits for the
+ * recorded events of `name`, returns their summed duration in milliseconds and their number, and
+ * forgets them.  Names: "spmm_rowseg" (the SpMM main kernel; one record per launch, tagged by f:
+ * "spmm_rowseg/f=602"), "spmm_reduce", "dense_xw", "dense_gwt", "dense_xtg".
+ * Recording is off by default and costs nothing then.
+ */
+int cg_prof_enable(int on);
+int cg_prof_read(const char *name, double *total_ms, int64_t *launches);
+
 #ifdef __cplusplus
 }
 #endif
