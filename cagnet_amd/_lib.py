@@ -61,6 +61,7 @@ _SIGNATURES = {
     "cg_nll_loss_bwd": [P, P, P, P, P, c_int64, c_int64, c_int32, P],
     "cg_log_softmax_nll_bwd": [P, c_int64, P, P, P, P, P, c_int64, c_int64, c_int32, P],
     "cg_prof_enable": [c_int],
+    "cg_tune_set": [c_char_p, c_int],
     "cg_prof_read": [c_char_p, POINTER(ctypes.c_double), POINTER(c_int64)],
 }
 _RESTYPES = {"cg_status_string": c_char_p, "cg_last_error": c_char_p}

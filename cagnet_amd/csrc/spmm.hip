@@ -17,6 +17,8 @@
 // with lane reads (readlane for G == 1, where the column index becomes a scalar base address).
 #include "common.h"
 #include <stdlib.h>
+#include <string.h>
+#include <atomic>
 #include <new>
 
 namespace cg {
@@ -41,6 +43,8 @@ struct SpmmArgs {
   float *P;                 // partial rows of split rows, row stride f
   int32_t f;
   float beta;
+  int32_t tiles;            // feature tiles (1, 2, 4 or 8); tile t is run by XCDs x with x % tiles == t
+  int32_t tile_slots;       // VEC-wide slots per tile (the last tile may hold fewer)
 };
 
 template <int VEC>
@@ -82,7 +86,18 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_rowseg_kernel(const SpmmArg
   static_assert(LPR == 64 || CHUNKS == 1, "several chunks only with a full-wave team");
   constexpr int G = kWave / LPR;
   const int lane = threadIdx.x & (kWave - 1);
-  const int64_t task = __builtin_amdgcn_readfirstlane((int)(((int64_t)blockIdx.x * kSpmmThreads + threadIdx.x) / kWave));
+  // Workgroups are dealt to the 8 XCDs round robin (workgroup w runs on XCD w % 8), and every XCD
+  // has its own L2.  With T feature tiles, XCD x only ever touches tile x % T of B, so its L2 holds
+  // a T times narrower slice of B's hot rows: the 8 L2s cache different data instead of 8 copies.
+  int tile = 0;
+  int64_t tb = blockIdx.x;
+  if (a.tiles > 1) {
+    const int x = blockIdx.x & 7;
+    const int per = 8 / a.tiles;  // XCDs that share a tile
+    tile = x % a.tiles;
+    tb = (int64_t)(blockIdx.x >> 3) * per + x / a.tiles;
+  }
+  const int64_t task = __builtin_amdgcn_readfirstlane((int)(tb * kWavesPerBlock + threadIdx.x / kWave));
   if (task >= a.ntasks) return;
 
   int32_t row, sidx, rs, re;
@@ -102,13 +117,16 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_rowseg_kernel(const SpmmArg
 
   const int g = lane / LPR;   // team
   const int j = lane % LPR;   // position inside the team
-  const int nslots = a.f / VEC;
+  const int slot0 = tile * a.tile_slots;
+  int nslots = a.f / VEC - slot0;  // slots of this tile
+  nslots = nslots < a.tile_slots ? nslots : a.tile_slots;
+  if (nslots <= 0) return;
   bool active[CHUNKS];
   int64_t boff[CHUNKS];  // lane's column offset per chunk; idle lanes re-read the chunk's first slot
 #pragma unroll
   for (int ch = 0; ch < CHUNKS; ++ch) {
     active[ch] = (ch * LPR + j) < nslots;
-    boff[ch] = (int64_t)(ch * LPR + (active[ch] ? j : 0)) * VEC;
+    boff[ch] = (int64_t)(slot0 + ch * LPR + (active[ch] ? j : 0)) * VEC;
   }
 
   float acc[CHUNKS][VEC];
@@ -212,28 +230,28 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_rowseg_kernel(const SpmmArg
   }
 
   if (single) {
-    float *crow = a.C + (int64_t)row * a.ldc + (int64_t)j * VEC;
+    float *crow = a.C + (int64_t)row * a.ldc;
 #pragma unroll
     for (int ch = 0; ch < CHUNKS; ++ch) {
       if (active[ch]) {
         float out[VEC];
         if (a.beta != 0.f) {
           float old[VEC];
-          load_vec<VEC>(crow + ch * (LPR * VEC), old);
+          load_vec<VEC>(crow + boff[ch], old);
 #pragma unroll
           for (int x = 0; x < VEC; ++x) out[x] = fmaf(a.beta, old[x], acc[ch][x]);
         } else {
 #pragma unroll
           for (int x = 0; x < VEC; ++x) out[x] = acc[ch][x];
         }
-        store_vec<VEC>(crow + ch * (LPR * VEC), out);
+        store_vec<VEC>(crow + boff[ch], out);
       }
     }
   } else {
-    float *prow = a.P + ((int64_t)a.pbase[row] + sidx) * a.f + (int64_t)j * VEC;
+    float *prow = a.P + ((int64_t)a.pbase[row] + sidx) * a.f;
 #pragma unroll
     for (int ch = 0; ch < CHUNKS; ++ch)
-      if (active[ch]) store_vec<VEC>(prow + ch * (LPR * VEC), acc[ch]);
+      if (active[ch]) store_vec<VEC>(prow + boff[ch], acc[ch]);
   }
 }
 
@@ -266,13 +284,16 @@ struct SpmmShape {
 
 constexpr int kMaxChunks = 5;
 
-// Widest vector the operands allow, then the smallest team that covers f.
-static SpmmShape pick_shape(int32_t f, const float *B, int64_t ldb, const float *C, int64_t ldc) {
+// Widest vector the operands allow.
+static int pick_vec(int32_t f, const float *B, int64_t ldb, const float *C, int64_t ldc) {
   const uintptr_t bits = (uintptr_t)B | (uintptr_t)C;
-  int vec = 1;
-  if (f % 4 == 0 && ldb % 4 == 0 && ldc % 4 == 0 && bits % 16 == 0) vec = 4;
-  else if (f % 2 == 0 && ldb % 2 == 0 && ldc % 2 == 0 && bits % 8 == 0) vec = 2;
-  const int slots = f / vec;
+  if (f % 4 == 0 && ldb % 4 == 0 && ldc % 4 == 0 && bits % 16 == 0) return 4;
+  if (f % 2 == 0 && ldb % 2 == 0 && ldc % 2 == 0 && bits % 8 == 0) return 2;
+  return 1;
+}
+
+// Smallest team that covers `slots` vector slots (one tile's worth).
+static SpmmShape pick_shape(int vec, int slots) {
   SpmmShape s{vec, 64, 1};
   if (slots <= 64) {
     int lpr = 4;
@@ -284,9 +305,24 @@ static SpmmShape pick_shape(int32_t f, const float *B, int64_t ldb, const float 
   return s;
 }
 
+// Tuning knobs (cg_tune_set): 0 = built-in choice.
+std::atomic<int> g_tune_seg{0}, g_tune_tiles{0};
+
+// Feature tiles per launch.  Wide outputs are split over the XCDs so that each L2 caches its own
+// column slice of B; narrow ones (a row of B is a cache line or two) stay whole.
+static int pick_tiles(int vec, int slots) {
+  const int t = g_tune_tiles.load(std::memory_order_relaxed);
+  if (t == 1 || t == 2 || t == 4 || t == 8) return slots >= t ? t : 1;
+  (void)vec;
+  return slots >= 256 ? 8 : 1;
+}
+
 template <bool TABLE, bool CLAMP>
 static int launch_shape(const SpmmShape &s, const SpmmArgs &a, hipStream_t stream) {
-  const unsigned grid = (unsigned)ceil_div64(a.ntasks, kWavesPerBlock);
+  int64_t blocks = ceil_div64(a.ntasks, kWavesPerBlock);
+  if (a.tiles > 1) blocks = ceil_div64(blocks, 8 / a.tiles) * 8;
+  if (blocks > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "SpMM grid too large");
+  const unsigned grid = (unsigned)blocks;
   if (grid == 0) return CG_OK;
 #define CG_CASE(V, L, CH)                                                                          \
   if (s.vec == V && s.lpr == L && s.chunks == CH) {                                                \
@@ -302,6 +338,22 @@ static int launch_shape(const SpmmShape &s, const SpmmArgs &a, hipStream_t strea
 #undef CG_CASE
   CG_FAIL(CG_ERR_UNSUPPORTED, "no SpMM kernel for vec=%d lpr=%d chunks=%d", s.vec, s.lpr, s.chunks);
 }
+
+// One launch covers at most tiles * 64 * kMaxChunks slots; wider outputs take several launches
+// over column ranges.  Fills the tiling fields of `a` for the range [f0, f0 + ft).
+struct SpmmPlan {
+  SpmmShape shape;
+  int tiles, tile_slots;
+};
+static SpmmPlan plan_range(int vec, int32_t ft) {
+  const int slots = ft / vec;
+  SpmmPlan p;
+  p.tiles = pick_tiles(vec, slots);
+  p.tile_slots = (slots + p.tiles - 1) / p.tiles;
+  p.shape = pick_shape(vec, p.tile_slots);
+  return p;
+}
+static int32_t range_cap(int vec) { return kWave * kMaxChunks * vec; }
 
 static int check_dense(const char *who, const float *B, int64_t ldb, float *C, int64_t ldc, int32_t f,
                        int64_t brows, int64_t crows) {
@@ -464,13 +516,10 @@ static int build_sched(CsrSide &s, int32_t seg, Sched **out, hipStream_t stream)
 }
 
 // Entries per task.  A team step consumes G entries per wave instruction, so narrow outputs get
-// longer segments for the same number of steps.  CG_SPMM_SEG overrides (tuning aid).
+// longer segments for the same number of steps.
 static int32_t pick_seg(const SpmmShape &s) {
-  static const int32_t env = [] {
-    const char *e = getenv("CG_SPMM_SEG");
-    return e ? (int32_t)atoi(e) : 0;
-  }();
-  if (env >= 64) return env;
+  const int t = g_tune_seg.load(std::memory_order_relaxed);
+  if (t >= 64) return t;
   const int g = kWave / s.lpr;
   if (g == 1) return 1024;
   if (g == 2) return 2048;
@@ -480,14 +529,19 @@ static int32_t pick_seg(const SpmmShape &s) {
 static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t ldc, int32_t f, float beta,
                      hipStream_t stream) {
   if (s.rows == 0) return CG_OK;
-  // wide outputs are processed in column tiles that one launch can cover
-  const SpmmShape probe = pick_shape(f, B, ldb, C, ldc);
-  const int32_t cap = kWave * kMaxChunks * probe.vec;
+  const int vec = pick_vec(f, B, ldb, C, ldc);
+  const int32_t cap = range_cap(vec) * 8;  // 8 tiles of kMaxChunks chunks
   for (int32_t f0 = 0; f0 < f; f0 += cap) {
     const int32_t ft = f - f0 < cap ? f - f0 : cap;
     const float *Bt = B + f0;
     float *Ct = C + f0;
-    const SpmmShape shape = pick_shape(ft, Bt, ldb, Ct, ldc);
+    SpmmPlan plan = plan_range(vec, ft);
+    if (plan.shape.chunks > kMaxChunks) {  // tiling was tuned down: fall back to 8 tiles
+      plan.tiles = 8;
+      plan.tile_slots = (ft / vec + 7) / 8;
+      plan.shape = pick_shape(vec, plan.tile_slots);
+    }
+    const SpmmShape shape = plan.shape;
     Sched *sc = nullptr;
     CG_TRY(build_sched(s, pick_seg(shape), &sc, stream));
     SpmmArgs a{};
@@ -506,6 +560,8 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
     a.ldc = ldc;
     a.f = ft;
     a.beta = beta;
+    a.tiles = plan.tiles;
+    a.tile_slots = plan.tile_slots;
     a.P = nullptr;
     if (sc->nslots > 0) {
       void *p = nullptr;
@@ -612,8 +668,8 @@ int cg_spmm_coo(const int32_t *d_row, const int32_t *d_col, const float *d_val, 
   // in-range spans, never an out-of-bounds read
   CG_HIP(hipMemsetAsync(d_rowptr, 0, (size_t)(n + 1) * sizeof(int32_t), stream));
   CG_TRY(launch_rowptr(d_row, nnz, n, (int32_t *)d_rowptr, stream));
-  const SpmmShape probe = pick_shape(f, d_B, ldb, d_C, ldc);
-  const int32_t cap = kWave * kMaxChunks * probe.vec;
+  const int vec = pick_vec(f, d_B, ldb, d_C, ldc);
+  const int32_t cap = range_cap(vec);
   for (int32_t f0 = 0; f0 < f; f0 += cap) {
     const int32_t ft = f - f0 < cap ? f - f0 : cap;
     SpmmArgs a{};
@@ -629,7 +685,9 @@ int cg_spmm_coo(const int32_t *d_row, const int32_t *d_col, const float *d_val, 
     a.ldc = ldc;
     a.f = ft;
     a.beta = beta;
-    CG_TRY((launch_shape<false, true>(pick_shape(ft, a.B, ldb, a.C, ldc), a, stream)));
+    a.tiles = 1;
+    a.tile_slots = ft / vec;
+    CG_TRY((launch_shape<false, true>(pick_shape(vec, ft / vec), a, stream)));
   }
   return CG_OK;
 }
@@ -674,6 +732,14 @@ int cg_csr_spmm(cg_csr_t *h, int transpose, const float *d_B, int64_t ldb, float
   CsrSide &s = transpose ? h->tr : h->fwd;
   CG_TRY(check_dense("cg_csr_spmm", d_B, ldb, d_C, ldc, f, s.cols, s.rows));
   return spmm_side(s, d_B, ldb, d_C, ldc, f, beta, (hipStream_t)stream);
+}
+
+int cg_tune_set(const char *key, int value) {
+  if (!key) CG_FAIL(CG_ERR_NULL, "cg_tune_set: key is NULL");
+  if (!strcmp(key, "spmm_seg")) cg::g_tune_seg.store(value);
+  else if (!strcmp(key, "spmm_tiles")) cg::g_tune_tiles.store(value);
+  else CG_FAIL(CG_ERR_UNSUPPORTED, "cg_tune_set: unknown key %s", key);
+  return CG_OK;
 }
 
 int cg_csr_info(const cg_csr_t *h, int64_t info[8]) {

@@ -178,6 +178,11 @@ int cg_log_softmax_nll_bwd(const float *d_logp, int64_t ld, const int64_t *d_y, 
  * Recording is off by default and costs nothing then.
  */
 int cg_prof_enable(int on);
+/* Tuning knobs, 0 = built-in choice.  "spmm_seg": stored entries per row segment (>= 64);
+ * "spmm_tiles": feature tiles of a wide SpMM launch (1, 2, 4 or 8; tile t runs on the XCDs x with
+ * x % tiles == t).  Results stay deterministic for a given setting; different settings change the
+ * summation order of split rows. */
+int cg_tune_set(const char *key, int value);
 int cg_prof_read(const char *name, double *total_ms, int64_t *launches);
 
 #ifdef __cplusplus

@@ -1,0 +1,67 @@
+"""Host-side logic that needs no GPU: the synthetic generator, the benchmark's accounting and
+its command line."""
+import hashlib
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import torch
+
+from cagnet_amd import synth
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+def _digest(*tensors):
+    h = hashlib.sha256()
+    for t in tensors:
+        h.update(np.ascontiguousarray(t.numpy()).tobytes())
+    return h.hexdigest()[:16]
+
+
+def test_rmat_graph_is_seeded_symmetric_and_self_looped():
+    row, col, n = synth.rmat_graph(10, 8192, 1)
+    row2, col2, _ = synth.rmat_graph(10, 8192, 1)
+    assert _digest(row, col) == _digest(row2, col2)
+    assert _digest(row, col) != _digest(*synth.rmat_graph(10, 8192, 2)[:2])
+    key = row * n + col
+    assert torch.all(key[1:] > key[:-1])                      # sorted by (row, col), duplicate free
+    assert torch.equal(torch.sort(col * n + row).values, key)  # symmetric pattern
+    assert int((row == col).sum()) == n                        # every self-loop present
+    deg = torch.bincount(row, minlength=n)
+    assert int(deg.max()) > 20 * int(deg.median())             # power-law: hubs far above the median
+
+
+def test_rmat_quadrant_probabilities():
+    src, dst = synth.rmat_edges(1, 400000, 3)
+    frac = [float(((src == s) & (dst == d)).float().mean()) for s, d in ((0, 0), (0, 1), (1, 0), (1, 1))]
+    assert all(abs(a - b) < 0.005 for a, b in zip(frac, synth.RMAT_ABCD))
+
+
+def test_target_nnz_is_met_exactly():
+    row, col = synth.rmat_graph_target_nnz(1000, 30001, 5)
+    assert row.numel() == 2 * ((30001 - 1000) // 2) + 1000 == 30000   # nnz = 2 * pairs + n: within one of the target
+    assert int(row.max()) < 1000 and int((row == col).sum()) == 1000
+
+
+def test_make_problem_shapes_and_seeds():
+    p = synth.make_problem(scale=8, n_edges=1024, features=12, hidden=16, classes=5, mask_fraction=0.66, seed=9)
+    assert p.x.shape == (256, 12) and p.w1.shape == (12, 16) and p.w2.shape == (16, 5)
+    assert p.y.min() >= 0 and p.y.max() < 5 and p.y.dtype == torch.int64
+    assert 0.5 < float(p.train_mask.float().mean()) < 0.8
+    bound = (6.0 / (12 + 16)) ** 0.5
+    assert float(p.w1.abs().max()) <= bound and float(p.w1.abs().max()) > 0.8 * bound
+    assert p.seeds == {"graph": 91, "x": 92, "y": 93, "mask": 94, "w1": 95, "w2": 96}
+
+
+def test_bench_accounting_and_gpu_count_guard():
+    sys.path.insert(0, str(ROOT))
+    import bench
+    # B_alg = 8 nnz + 4 (n+1) + 4 m f + 4 n f (1 + r)
+    assert bench.spmm_alg_bytes(10, 4, 5, 3, False) == 80 + 20 + 60 + 48
+    assert bench.spmm_alg_bytes(10, 4, 5, 3, True) == 80 + 20 + 60 + 96
+    reddit = bench.spmm_alg_bytes(114_615_891, 232_965, 232_965, 602, False)
+    assert abs(reddit - 2.04e9) < 0.01e9
+    proc = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert proc.returncode != 0 and "ONE GPU" in proc.stderr
