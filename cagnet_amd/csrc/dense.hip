@@ -172,15 +172,32 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_tile_kernel(const GemmArgs 
   }
 }
 
-// C[i] = sum over slices s of P[s][i], in slice order
+// C[i] = sum over slices z of P[z][i].  A workgroup owns 16 consecutive outputs; its 16 z-lanes
+// per output add slices z, z+16, ... in order and are then combined by a fixed xor butterfly, so
+// the order of additions depends only on the number of slices.
+constexpr int kSumOut = 16;
 __global__ __launch_bounds__(kGemmThreads) void gemm_slice_sum_kernel(const float *__restrict__ P, int64_t elems,
                                                                       int32_t splits, float *__restrict__ C,
                                                                       int64_t ldc, int32_t N) {
-  const int64_t idx = (int64_t)blockIdx.x * kGemmThreads + threadIdx.x;
-  if (idx >= elems) return;
+  const int e = threadIdx.x % kSumOut;
+  const int zl = threadIdx.x / kSumOut;  // 0..15; the 16 z-lanes of one output sit 16 lanes apart
+  const int64_t idx = (int64_t)blockIdx.x * kSumOut + e;
   float s = 0.f;
-  for (int32_t z = 0; z < splits; ++z) s += P[(int64_t)z * elems + idx];
-  C[(idx / N) * ldc + (idx % N)] = s;
+  if (idx < elems)
+    for (int32_t z = zl; z < splits; z += kGemmThreads / kSumOut) s += P[(int64_t)z * elems + idx];
+  // lanes of one wave: zl = 4*wave + lane/16 -> combine the 4 z-lanes inside the wave, then the 4 waves
+  s += __shfl_xor(s, 16, kWave);
+  s += __shfl_xor(s, 32, kWave);
+  __shared__ float part[kGemmThreads / kWave][kSumOut];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  if (lane < kSumOut) part[wave][lane] = s;
+  __syncthreads();
+  if (threadIdx.x < kSumOut && idx < elems) {
+    float t = part[0][e];
+#pragma unroll
+    for (int w = 1; w < kGemmThreads / kWave; ++w) t += part[w][e];
+    C[(idx / N) * ldc + (idx % N)] = t;
+  }
 }
 
 template <bool AT, bool BT>
@@ -242,6 +259,7 @@ int cg_dense_xtg(const float *d_X, int64_t ldx, const float *d_G, int64_t ldg, f
   const int bn = fo <= 16 ? 16 : (fo <= 32 ? 32 : 64);
   const int64_t tiles = ceil_div64(k, 4096 / bn) * ceil_div64(fo, bn);
   int64_t splits = ceil_div64(2048, tiles);
+  if (splits > 512) splits = 512;
   int64_t kchunk = ceil_div64(ceil_div64(n > 0 ? n : 1, splits), kKT) * kKT;
   if (kchunk < 4 * kKT) kchunk = 4 * kKT;
   splits = n > 0 ? ceil_div64(n, kchunk) : 1;
@@ -258,7 +276,7 @@ int cg_dense_xtg(const float *d_X, int64_t ldx, const float *d_G, int64_t ldg, f
   g.C = (float *)p;
   g.ldc = fo;
   CG_TRY((launch_gemm<true, false>(g, stream)));
-  gemm_slice_sum_kernel<<<(unsigned)ceil_div64(elems, kGemmThreads), kGemmThreads, 0, stream>>>(
+  gemm_slice_sum_kernel<<<(unsigned)ceil_div64(elems, kSumOut), kGemmThreads, 0, stream>>>(
       (const float *)p, elems, (int32_t)splits, d_dW, lddw, fo);
   CG_LAUNCH_CHECK();
   return CG_OK;

@@ -45,7 +45,14 @@ struct SpmmArgs {
   float beta;
   int32_t tiles;            // feature tiles (1, 2, 4 or 8); tile t is run by XCDs x with x % tiles == t
   int32_t tile_slots;       // VEC-wide slots per tile (the last tile may hold fewer)
+  int32_t groups;           // kModeHub: hot column groups (1, 2, 4 or 8); group g runs on XCDs x % groups == g
+  int64_t tstart[9];        // kModeHub: tasks of group g are [tstart[g], tstart[g+1])
 };
+
+// kModeRows: one task per row, no tables, column indices clamped (one-shot entry point)
+// kModeTable: tasks from the schedule tables of a handle
+// kModeHub:  tasks of the hot column groups of a hub plan, pinned to XCDs; every task writes a partial row
+enum { kModeRows = 0, kModeTable = 1, kModeHub = 2 };
 
 template <int VEC>
 struct VecT;
@@ -81,24 +88,38 @@ __device__ __forceinline__ void store_vec(float *p, const float (&r)[VEC]) {
   *reinterpret_cast<V *>(p) = t;
 }
 
-template <int VEC, int LPR, int CHUNKS, bool TABLE, bool CLAMP>
+template <int VEC, int LPR, int CHUNKS, int MODE>
 __global__ __launch_bounds__(kSpmmThreads) void spmm_rowseg_kernel(const SpmmArgs a) {
   static_assert(LPR == 64 || CHUNKS == 1, "several chunks only with a full-wave team");
   constexpr int G = kWave / LPR;
+  constexpr bool TABLE = MODE != kModeRows;
+  constexpr bool CLAMP = MODE == kModeRows;
+  constexpr bool HUB = MODE == kModeHub;
   const int lane = threadIdx.x & (kWave - 1);
   // Workgroups are dealt to the 8 XCDs round robin (workgroup w runs on XCD w % 8), and every XCD
   // has its own L2.  With T feature tiles, XCD x only ever touches tile x % T of B, so its L2 holds
   // a T times narrower slice of B's hot rows: the 8 L2s cache different data instead of 8 copies.
   int tile = 0;
   int64_t tb = blockIdx.x;
-  if (a.tiles > 1) {
+  int64_t task_lo = 0, task_hi = a.ntasks;
+  if (HUB) {
+    // Hot columns are dealt to `groups` groups; group g's rows of B are only ever read by the XCDs
+    // x with x % groups == g, so each L2 keeps its own share of the hot rows resident.
+    const int x = blockIdx.x & 7;
+    const int per = 8 / a.groups;
+    const int grp = x % a.groups;
+    tb = (int64_t)(blockIdx.x >> 3) * per + x / a.groups;
+    task_lo = a.tstart[grp];
+    task_hi = a.tstart[grp + 1];
+  } else if (a.tiles > 1) {
     const int x = blockIdx.x & 7;
     const int per = 8 / a.tiles;  // XCDs that share a tile
     tile = x % a.tiles;
     tb = (int64_t)(blockIdx.x >> 3) * per + x / a.tiles;
   }
-  const int64_t task = __builtin_amdgcn_readfirstlane((int)(tb * kWavesPerBlock + threadIdx.x / kWave));
-  if (task >= a.ntasks) return;
+  const int64_t task =
+      __builtin_amdgcn_readfirstlane((int)(task_lo + tb * kWavesPerBlock + threadIdx.x / kWave));
+  if (task >= task_hi) return;
 
   int32_t row, sidx, rs, re;
   if (TABLE) {
@@ -112,7 +133,7 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_rowseg_kernel(const SpmmArg
   re = a.rowptr[row + 1];
   const int32_t start = TABLE ? rs + sidx * a.seg : rs;
   const int32_t end = TABLE ? (start + a.seg < re ? start + a.seg : re) : re;
-  const bool single = TABLE ? (re - rs <= a.seg) : true;
+  const bool single = HUB ? false : (TABLE ? (re - rs <= a.seg) : true);
   if (single && start >= end && a.beta == 1.0f) return;  // empty row, C unchanged
 
   const int g = lane / LPR;   // team
@@ -248,7 +269,7 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_rowseg_kernel(const SpmmArg
       }
     }
   } else {
-    float *prow = a.P + ((int64_t)a.pbase[row] + sidx) * a.f;
+    float *prow = a.P + (HUB ? task : ((int64_t)a.pbase[row] + sidx)) * a.f;
 #pragma unroll
     for (int ch = 0; ch < CHUNKS; ++ch)
       if (active[ch]) store_vec<VEC>(prow + boff[ch], acc[ch]);
@@ -282,13 +303,18 @@ struct SpmmShape {
   int vec, lpr, chunks;
 };
 
-constexpr int kMaxChunks = 5;
+constexpr int kMaxChunks = 10;
+
+// Tuning knobs (cg_tune_set): 0 = built-in choice.
+std::atomic<int> g_tune_seg{0}, g_tune_tiles{0}, g_tune_vec{0};
 
 // Widest vector the operands allow.
 static int pick_vec(int32_t f, const float *B, int64_t ldb, const float *C, int64_t ldc) {
   const uintptr_t bits = (uintptr_t)B | (uintptr_t)C;
-  if (f % 4 == 0 && ldb % 4 == 0 && ldc % 4 == 0 && bits % 16 == 0) return 4;
-  if (f % 2 == 0 && ldb % 2 == 0 && ldc % 2 == 0 && bits % 8 == 0) return 2;
+  const int cap = g_tune_vec.load(std::memory_order_relaxed);
+  const int lim = (cap == 1 || cap == 2) ? cap : 4;
+  if (lim >= 4 && f % 4 == 0 && ldb % 4 == 0 && ldc % 4 == 0 && bits % 16 == 0) return 4;
+  if (lim >= 2 && f % 2 == 0 && ldb % 2 == 0 && ldc % 2 == 0 && bits % 8 == 0) return 2;
   return 1;
 }
 
@@ -305,9 +331,6 @@ static SpmmShape pick_shape(int vec, int slots) {
   return s;
 }
 
-// Tuning knobs (cg_tune_set): 0 = built-in choice.
-std::atomic<int> g_tune_seg{0}, g_tune_tiles{0};
-
 // Feature tiles per launch.  Wide outputs are split over the XCDs so that each L2 caches its own
 // column slice of B; narrow ones (a row of B is a cache line or two) stay whole.
 static int pick_tiles(int vec, int slots) {
@@ -317,22 +340,29 @@ static int pick_tiles(int vec, int slots) {
   return slots >= 256 ? 8 : 1;
 }
 
-template <bool TABLE, bool CLAMP>
+template <int MODE>
 static int launch_shape(const SpmmShape &s, const SpmmArgs &a, hipStream_t stream) {
   int64_t blocks = ceil_div64(a.ntasks, kWavesPerBlock);
-  if (a.tiles > 1) blocks = ceil_div64(blocks, 8 / a.tiles) * 8;
+  if (MODE == kModeHub) {
+    int64_t longest = 0;
+    for (int g = 0; g < a.groups; ++g) longest = longest > a.tstart[g + 1] - a.tstart[g] ? longest : a.tstart[g + 1] - a.tstart[g];
+    blocks = ceil_div64(ceil_div64(longest, kWavesPerBlock), 8 / a.groups) * 8;
+  } else if (a.tiles > 1) {
+    blocks = ceil_div64(blocks, 8 / a.tiles) * 8;
+  }
   if (blocks > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "SpMM grid too large");
   const unsigned grid = (unsigned)blocks;
   if (grid == 0) return CG_OK;
 #define CG_CASE(V, L, CH)                                                                          \
   if (s.vec == V && s.lpr == L && s.chunks == CH) {                                                \
-    spmm_rowseg_kernel<V, L, CH, TABLE, CLAMP><<<grid, kSpmmThreads, 0, stream>>>(a);              \
+    spmm_rowseg_kernel<V, L, CH, MODE><<<grid, kSpmmThreads, 0, stream>>>(a);                      \
     CG_LAUNCH_CHECK();                                                                             \
     return CG_OK;                                                                                  \
   }
 #define CG_CASES(V)                                                                                \
   CG_CASE(V, 4, 1) CG_CASE(V, 8, 1) CG_CASE(V, 16, 1) CG_CASE(V, 32, 1) CG_CASE(V, 64, 1)           \
-  CG_CASE(V, 64, 2) CG_CASE(V, 64, 3) CG_CASE(V, 64, 4) CG_CASE(V, 64, 5)
+  CG_CASE(V, 64, 2) CG_CASE(V, 64, 3) CG_CASE(V, 64, 4) CG_CASE(V, 64, 5) CG_CASE(V, 64, 6)           \
+  CG_CASE(V, 64, 7) CG_CASE(V, 64, 8) CG_CASE(V, 64, 9) CG_CASE(V, 64, 10)
   CG_CASES(1) CG_CASES(2) CG_CASES(4)
 #undef CG_CASES
 #undef CG_CASE
@@ -368,28 +398,35 @@ static int check_dense(const char *who, const float *B, int64_t ldb, float *C, i
 // ---------------------------------------------------------------------------------------------
 // schedules (row segments), built on the device
 // ---------------------------------------------------------------------------------------------
+// skip_empty: rows without entries get no task (hub plans); otherwise every row has at least one,
+// because a beta != 1 launch still has to scale the row of C.
+__device__ __forceinline__ uint32_t tasks_of(int32_t deg, int32_t seg, int skip_empty) {
+  if (deg <= 0) return skip_empty ? 0u : 1u;
+  return deg <= seg ? 1u : (uint32_t)((deg + seg - 1) / seg);
+}
+
 __global__ __launch_bounds__(kSpmmThreads) void sched_count_kernel(const int32_t *__restrict__ rowptr, int32_t n,
-                                                                   int32_t seg, uint32_t *__restrict__ ntask,
+                                                                   int32_t seg, int skip_empty,
+                                                                   uint32_t *__restrict__ ntask,
                                                                    uint32_t *__restrict__ nslot,
                                                                    uint32_t *__restrict__ nmulti) {
   const int64_t r = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (r >= n) return;
-  const int32_t deg = rowptr[r + 1] - rowptr[r];
-  const uint32_t t = deg <= seg ? 1u : (uint32_t)((deg + seg - 1) / seg);
+  const uint32_t t = tasks_of(rowptr[r + 1] - rowptr[r], seg, skip_empty);
   ntask[r] = t;
   nslot[r] = t > 1 ? t : 0u;
   nmulti[r] = t > 1 ? 1u : 0u;
 }
 
 __global__ __launch_bounds__(kSpmmThreads) void sched_fill_kernel(const int32_t *__restrict__ rowptr, int32_t n,
-                                                                  int32_t seg, const uint32_t *__restrict__ tbase,
+                                                                  int32_t seg, int skip_empty,
+                                                                  const uint32_t *__restrict__ tbase,
                                                                   const uint32_t *__restrict__ mbase,
                                                                   int32_t *__restrict__ task_row,
                                                                   int32_t *__restrict__ multi_rows) {
   const int64_t r = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (r >= n) return;
-  const int32_t deg = rowptr[r + 1] - rowptr[r];
-  const uint32_t t = deg <= seg ? 1u : (uint32_t)((deg + seg - 1) / seg);
+  const uint32_t t = tasks_of(rowptr[r + 1] - rowptr[r], seg, skip_empty);
   const uint32_t b = tbase[r];
   for (uint32_t i = 0; i < t; ++i) task_row[b + i] = (int32_t)r;
   if (t > 1) multi_rows[mbase[r]] = (int32_t)r;
@@ -421,25 +458,6 @@ struct Sched {
   }
 };
 
-struct CsrSide {
-  int32_t rows = 0, cols = 0;
-  int32_t *rowptr = nullptr, *colind = nullptr;
-  float *val = nullptr;
-  int32_t max_degree = 0;
-  static constexpr int kMaxSched = 4;
-  Sched sched[kMaxSched];
-  int nsched = 0;
-  void release() {
-    for (int i = 0; i < nsched; ++i) sched[i].release();
-    nsched = 0;
-    if (rowptr) (void)hipFree(rowptr);
-    if (colind) (void)hipFree(colind);
-    if (val) (void)hipFree(val);
-    rowptr = colind = nullptr;
-    val = nullptr;
-  }
-};
-
 static int dev_alloc(void **p, size_t bytes) {
   hipError_t e = hipMalloc(p, bytes ? bytes : 4);
   if (e != hipSuccess) {
@@ -451,21 +469,10 @@ static int dev_alloc(void **p, size_t bytes) {
   return CG_OK;
 }
 
-static int build_sched(CsrSide &s, int32_t seg, Sched **out, hipStream_t stream) {
-  for (int i = 0; i < s.nsched; ++i)
-    if (s.sched[i].seg == seg) {
-      *out = &s.sched[i];
-      return CG_OK;
-    }
-  if (s.nsched == CsrSide::kMaxSched) {  // recycle the oldest
-    CG_HIP(hipStreamSynchronize(stream));
-    s.sched[0].release();
-    for (int i = 1; i < s.nsched; ++i) s.sched[i - 1] = s.sched[i];
-    s.sched[--s.nsched] = Sched();
-  }
+// Task tables for the rows [0, n) described by rowptr.  Synchronises `stream`.
+static int make_sched(const int32_t *rowptr, int32_t n, int32_t seg, int skip_empty, Sched &out, hipStream_t stream) {
   Sched sc;
   sc.seg = seg;
-  const int32_t n = s.rows;
   const size_t nb = (size_t)(n + 1) * sizeof(uint32_t);
   uint32_t *d_mbase = nullptr;
   void *d_totals_v = nullptr;
@@ -479,11 +486,14 @@ static int build_sched(CsrSide &s, int32_t seg, Sched **out, hipStream_t stream)
     uint32_t totals[3] = {0, 0, 0};
     if (n > 0) {
       const unsigned grid = (unsigned)ceil_div64(n, kSpmmThreads);
-      sched_count_kernel<<<grid, kSpmmThreads, 0, stream>>>(s.rowptr, n, seg, (uint32_t *)sc.tbase,
+      sched_count_kernel<<<grid, kSpmmThreads, 0, stream>>>(rowptr, n, seg, skip_empty, (uint32_t *)sc.tbase,
                                                             (uint32_t *)sc.pbase, d_mbase);
       if (hipGetLastError() != hipSuccess) { st = CG_ERR_HIP; set_error("sched_count launch failed"); break; }
-      if ((st = exclusive_scan_u32((uint32_t *)sc.tbase, (uint32_t *)sc.tbase, n, d_totals + 0, stream)) != CG_OK) break;
-      if ((st = exclusive_scan_u32((uint32_t *)sc.pbase, (uint32_t *)sc.pbase, n, d_totals + 1, stream)) != CG_OK) break;
+      // scanning n + 1 entries puts the grand total behind the last row: tbase[n] == ntasks
+      if ((st = hipMemsetAsync((uint32_t *)sc.tbase + n, 0, 4, stream) == hipSuccess ? CG_OK : CG_ERR_HIP) != CG_OK) break;
+      if ((st = hipMemsetAsync((uint32_t *)sc.pbase + n, 0, 4, stream) == hipSuccess ? CG_OK : CG_ERR_HIP) != CG_OK) break;
+      if ((st = exclusive_scan_u32((uint32_t *)sc.tbase, (uint32_t *)sc.tbase, (int64_t)n + 1, d_totals + 0, stream)) != CG_OK) break;
+      if ((st = exclusive_scan_u32((uint32_t *)sc.pbase, (uint32_t *)sc.pbase, (int64_t)n + 1, d_totals + 1, stream)) != CG_OK) break;
       if ((st = exclusive_scan_u32(d_mbase, d_mbase, n, d_totals + 2, stream)) != CG_OK) break;
       if (hipMemcpyAsync(totals, d_totals, sizeof(totals), hipMemcpyDeviceToHost, stream) != hipSuccess ||
           hipStreamSynchronize(stream) != hipSuccess) {
@@ -499,8 +509,8 @@ static int build_sched(CsrSide &s, int32_t seg, Sched **out, hipStream_t stream)
     if ((st = dev_alloc((void **)&sc.multi_rows, (size_t)sc.nmulti * sizeof(int32_t))) != CG_OK) break;
     if (n > 0) {
       const unsigned grid = (unsigned)ceil_div64(n, kSpmmThreads);
-      sched_fill_kernel<<<grid, kSpmmThreads, 0, stream>>>(s.rowptr, n, seg, (const uint32_t *)sc.tbase, d_mbase,
-                                                           sc.task_row, sc.multi_rows);
+      sched_fill_kernel<<<grid, kSpmmThreads, 0, stream>>>(rowptr, n, seg, skip_empty, (const uint32_t *)sc.tbase,
+                                                           d_mbase, sc.task_row, sc.multi_rows);
       if (hipGetLastError() != hipSuccess) { st = CG_ERR_HIP; set_error("sched_fill launch failed"); break; }
       if (hipStreamSynchronize(stream) != hipSuccess) { st = CG_ERR_HIP; set_error("sched_fill failed"); break; }
     }
@@ -510,10 +520,79 @@ static int build_sched(CsrSide &s, int32_t seg, Sched **out, hipStream_t stream)
     sc.release();
     return st;
   }
-  s.sched[s.nsched] = sc;
-  *out = &s.sched[s.nsched++];
+  out = sc;
   return CG_OK;
 }
+
+// A small cache of schedules keyed by segment length.
+struct SchedCache {
+  static constexpr int kMax = 4;
+  Sched sched[kMax];
+  int count = 0;
+  void release() {
+    for (int i = 0; i < count; ++i) sched[i].release();
+    count = 0;
+  }
+  int get(const int32_t *rowptr, int32_t n, int32_t seg, Sched **out, hipStream_t stream) {
+    for (int i = 0; i < count; ++i)
+      if (sched[i].seg == seg) {
+        *out = &sched[i];
+        return CG_OK;
+      }
+    if (count == kMax) {  // recycle the oldest
+      CG_HIP(hipStreamSynchronize(stream));
+      sched[0].release();
+      for (int i = 1; i < count; ++i) sched[i - 1] = sched[i];
+      sched[--count] = Sched();
+    }
+    CG_TRY(make_sched(rowptr, n, seg, 0, sched[count], stream));
+    *out = &sched[count++];
+    return CG_OK;
+  }
+};
+
+// Hub plan: the stored entries regrouped by column class.  The `hot` most referenced columns
+// (= rows of B) are dealt round robin, by descending reference count, to `groups` groups; every
+// other column is cold.  Entries are kept as one CSR over (groups + 1) * rows virtual rows, virtual
+// row c * rows + r holding the entries of row r whose column has class c (cold = class `groups`).
+struct HubPlan {
+  int32_t hot = 0, groups = 0, seg = 0;
+  int32_t *vrowptr = nullptr, *colind = nullptr;
+  float *val = nullptr;
+  Sched hot_sched;        // over the virtual rows of the hot classes, empty rows skipped
+  SchedCache cold_sched;  // over the cold class
+  int64_t tstart[9] = {0};
+  bool valid = false;
+  void release() {
+    hot_sched.release();
+    cold_sched.release();
+    if (vrowptr) (void)hipFree(vrowptr);
+    if (colind) (void)hipFree(colind);
+    if (val) (void)hipFree(val);
+    vrowptr = colind = nullptr;
+    val = nullptr;
+    valid = false;
+  }
+};
+
+struct CsrSide {
+  int32_t rows = 0, cols = 0;
+  int64_t nnz = 0;
+  int32_t *rowptr = nullptr, *colind = nullptr;
+  float *val = nullptr;
+  int32_t max_degree = 0;
+  SchedCache sched;
+  HubPlan hub;
+  void release() {
+    sched.release();
+    hub.release();
+    if (rowptr) (void)hipFree(rowptr);
+    if (colind) (void)hipFree(colind);
+    if (val) (void)hipFree(val);
+    rowptr = colind = nullptr;
+    val = nullptr;
+  }
+};
 
 // Entries per task.  A team step consumes G entries per wave instruction, so narrow outputs get
 // longer segments for the same number of steps.
@@ -526,59 +605,345 @@ static int32_t pick_seg(const SpmmShape &s) {
   return 4096;
 }
 
+// ---------------------------------------------------------------------------------------------
+// hub plan construction
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kSpmmThreads) void col_count_kernel(const int32_t *__restrict__ colind, int64_t nnz,
+                                                                 uint32_t *__restrict__ count) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k < nnz) atomicAdd(&count[colind[k]], 1u);  // integer count: independent of arrival order
+}
+
+// sort key that orders columns by descending count (ties: ascending column, by stability)
+__global__ __launch_bounds__(kSpmmThreads) void col_key_kernel(const uint32_t *__restrict__ count, int32_t m,
+                                                               uint32_t maxcount, int32_t *__restrict__ key,
+                                                               int32_t *__restrict__ id) {
+  const int64_t j = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (j < m) {
+    key[j] = (int32_t)(maxcount - count[j]);
+    id[j] = (int32_t)j;
+  }
+}
+
+// class of every column from its rank: the first `hot` ranks go round robin to the groups
+__global__ __launch_bounds__(kSpmmThreads) void col_class_kernel(const int32_t *__restrict__ ranked_col, int32_t m,
+                                                                 int32_t hot, int32_t groups,
+                                                                 int32_t *__restrict__ cls) {
+  const int64_t rank = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (rank < m) cls[ranked_col[rank]] = rank < hot ? (int32_t)(rank % groups) : groups;
+}
+
+__global__ __launch_bounds__(kSpmmThreads) void entry_class_kernel(const int32_t *__restrict__ colind, int64_t nnz,
+                                                                   const int32_t *__restrict__ cls,
+                                                                   int32_t *__restrict__ out) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k < nnz) out[k] = cls[colind[k]];
+}
+
+__global__ __launch_bounds__(kSpmmThreads) void entry_finish_kernel(const int32_t *__restrict__ cls_sorted,
+                                                                    const int32_t *__restrict__ row_sorted,
+                                                                    const int32_t *__restrict__ pos, int64_t nnz,
+                                                                    int32_t rows, const int32_t *__restrict__ colind,
+                                                                    const float *__restrict__ val,
+                                                                    int32_t *__restrict__ vrow,
+                                                                    int32_t *__restrict__ colind2,
+                                                                    float *__restrict__ val2) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k < nnz) {
+    const int32_t p = pos[k];
+    vrow[k] = cls_sorted[k] * rows + row_sorted[k];
+    colind2[k] = colind[p];
+    val2[k] = val[p];
+  }
+}
+
+__global__ __launch_bounds__(kSpmmThreads) void hub_iota_kernel(int32_t *__restrict__ out, int64_t count) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k < count) out[k] = (int32_t)k;
+}
+
+__global__ __launch_bounds__(kSpmmThreads) void csr_rows_kernel(const int32_t *__restrict__ rowptr, int32_t n,
+                                                                int32_t *__restrict__ row_out) {
+  const int64_t wave = ((int64_t)blockIdx.x * kSpmmThreads + threadIdx.x) / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  if (wave >= n) return;
+  const int32_t s = rowptr[wave], e = rowptr[wave + 1];
+  for (int32_t k = s + lane; k < e; k += kWave) row_out[k] = (int32_t)wave;
+}
+
+struct TempFree {
+  void *p[16];
+  int count = 0;
+  ~TempFree() {
+    for (int i = 0; i < count; ++i)
+      if (p[i]) (void)hipFree(p[i]);
+  }
+  int alloc(void **out, size_t bytes) {
+    CG_TRY(dev_alloc(out, bytes));
+    p[count++] = *out;
+    return CG_OK;
+  }
+};
+
+static int build_hub(CsrSide &s, int32_t hot, int32_t groups, int32_t seg, hipStream_t stream) {
+  HubPlan &h = s.hub;
+  CG_HIP(hipStreamSynchronize(stream));
+  h.release();
+  const int64_t nnz = s.nnz;
+  const int32_t n = s.rows, m = s.cols;
+  const int64_t vrows = (int64_t)(groups + 1) * n;
+  if (vrows + 1 > 0x7fffffffLL) CG_FAIL(CG_ERR_OVERFLOW, "hub plan: %lld virtual rows exceed int32", (long long)vrows);
+  if (hot > m) hot = m;
+  TempFree tmp;
+  const unsigned gm = (unsigned)ceil_div64(m, kSpmmThreads), ge = (unsigned)ceil_div64(nnz, kSpmmThreads);
+
+  // 1. reference count of every column, and the columns ranked by it
+  uint32_t *count = nullptr;
+  int32_t *cls = nullptr;
+  CG_TRY(tmp.alloc((void **)&count, (size_t)m * 4));
+  CG_TRY(tmp.alloc((void **)&cls, (size_t)m * 4));
+  CG_HIP(hipMemsetAsync(count, 0, (size_t)m * 4, stream));
+  col_count_kernel<<<ge, kSpmmThreads, 0, stream>>>(s.colind, nnz, count);
+  CG_LAUNCH_CHECK();
+  {
+    SortBuffers buf;
+    for (int i = 0; i < 2; ++i) {
+      CG_TRY(tmp.alloc((void **)&buf.key_a[i], (size_t)m * 4));
+      CG_TRY(tmp.alloc((void **)&buf.payload[i], (size_t)m * 4));
+      CG_TRY(tmp.alloc((void **)&buf.key_b[i], (size_t)m * 4));  // no minor key: carried, never sorted on
+    }
+    // the largest possible count is the number of rows (duplicate-free) or nnz in general
+    const uint32_t maxcount = (uint32_t)(nnz < 0x7fffffffLL ? nnz : 0x7fffffffLL);
+    col_key_kernel<<<gm, kSpmmThreads, 0, stream>>>(count, m, maxcount, buf.key_a[0], buf.payload[0]);
+    CG_LAUNCH_CHECK();
+    CG_HIP(hipMemsetAsync(buf.key_b[0], 0, (size_t)m * 4, stream));
+    int set = 0;
+    CG_TRY(radix_sort_pairs(buf, m, bits_for((int32_t)(maxcount < 0x7ffffffeu ? maxcount + 1 : 0x7fffffff)), 0, &set,
+                            stream));
+    col_class_kernel<<<gm, kSpmmThreads, 0, stream>>>(buf.payload[set], m, hot, groups, cls);
+    CG_LAUNCH_CHECK();
+  }
+
+  // 2. stable regrouping of the entries by class: (row, col) order is kept inside a class
+  CG_TRY(dev_alloc((void **)&h.colind, (size_t)nnz * 4));
+  CG_TRY(dev_alloc((void **)&h.val, (size_t)nnz * 4));
+  CG_TRY(dev_alloc((void **)&h.vrowptr, (size_t)(vrows + 1) * 4));
+  int32_t *vrow = nullptr;
+  CG_TRY(tmp.alloc((void **)&vrow, (size_t)nnz * 4));
+  {
+    TempFree tmp2;
+    SortBuffers buf;
+    for (int i = 0; i < 2; ++i) {
+      CG_TRY(tmp2.alloc((void **)&buf.key_a[i], (size_t)nnz * 4));
+      CG_TRY(tmp2.alloc((void **)&buf.key_b[i], (size_t)nnz * 4));
+      CG_TRY(tmp2.alloc((void **)&buf.payload[i], (size_t)nnz * 4));
+    }
+    entry_class_kernel<<<ge, kSpmmThreads, 0, stream>>>(s.colind, nnz, cls, buf.key_a[0]);
+    CG_LAUNCH_CHECK();
+    if (n > 0) {
+      csr_rows_kernel<<<(unsigned)ceil_div64((int64_t)n * kWave, kSpmmThreads), kSpmmThreads, 0, stream>>>(
+          s.rowptr, n, buf.key_b[0]);
+      CG_LAUNCH_CHECK();
+    }
+    hub_iota_kernel<<<ge, kSpmmThreads, 0, stream>>>(buf.payload[0], nnz);  // position in the original CSR
+    CG_LAUNCH_CHECK();
+    int set = 0;
+    CG_TRY(radix_sort_pairs(buf, nnz, bits_for(groups + 1), 0, &set, stream));
+    entry_finish_kernel<<<ge, kSpmmThreads, 0, stream>>>(buf.key_a[set], buf.key_b[set], buf.payload[set], nnz, n,
+                                                         s.colind, s.val, vrow, h.colind, h.val);
+    CG_LAUNCH_CHECK();
+    CG_HIP(hipStreamSynchronize(stream));
+  }
+  CG_TRY(launch_rowptr(vrow, nnz, (int32_t)vrows, h.vrowptr, stream));
+
+  // 3. tasks of the hot classes (empty virtual rows get none); the cold class is scheduled on demand
+  CG_TRY(make_sched(h.vrowptr, groups * n, seg, 1, h.hot_sched, stream));
+  {
+    int32_t t[9];
+    for (int g = 0; g <= groups; ++g)
+      CG_HIP(hipMemcpyAsync(&t[g], h.hot_sched.tbase + (int64_t)g * n, 4, hipMemcpyDeviceToHost, stream));
+    CG_HIP(hipStreamSynchronize(stream));
+    for (int g = 0; g <= groups; ++g) h.tstart[g] = t[g];
+  }
+  h.hot = hot;
+  h.groups = groups;
+  h.seg = seg;
+  h.valid = true;
+  return CG_OK;
+}
+
+// C[r, :] += sum of the partial rows of r's hot tasks, in (group, segment) order.  One wavefront
+// per row: lane g fetches the task range of group g, then the lanes sweep the row's columns with
+// the partial rows of all tasks in flight together.
+__global__ __launch_bounds__(kSpmmThreads) void hub_reduce_kernel(const int32_t *__restrict__ tbase, int32_t n,
+                                                                  int32_t groups, const float *__restrict__ P,
+                                                                  float *__restrict__ C, int64_t ldc, int32_t f) {
+  const int64_t r = ((int64_t)blockIdx.x * kSpmmThreads + threadIdx.x) / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  if (r >= n) return;
+  int32_t t0 = 0, t1 = 0;
+  if (lane < groups) {
+    const int64_t v = (int64_t)lane * n + r;
+    t0 = tbase[v];
+    t1 = tbase[v + 1];
+  }
+  int32_t first[8], count[8];
+  int32_t total = 0;
+#pragma unroll
+  for (int g = 0; g < 8; ++g) {
+    first[g] = __builtin_amdgcn_readlane(t0, g);
+    count[g] = __builtin_amdgcn_readlane(t1, g) - first[g];
+    total += count[g];
+  }
+  if (total == 0) return;
+  float *crow = C + r * ldc;
+  for (int32_t c0 = 0; c0 < f; c0 += kWave) {
+    const int32_t col = c0 + lane;
+    if (col < f) {
+      float s = 0.f;
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+        const float *p = P + (int64_t)first[g] * f + col;
+        if (count[g] == 1) {
+          s += p[0];
+        } else {
+          for (int32_t t = 0; t < count[g]; ++t) s += p[(int64_t)t * f];
+        }
+      }
+      crow[col] += s;
+    }
+  }
+}
+
+std::atomic<int> g_tune_hub{0}, g_tune_hub_kb{0}, g_tune_hub_groups{0};
+
+static void fill_args(SpmmArgs &a, const int32_t *rowptr, const int32_t *colind, const float *val, const Sched *sc,
+                      int32_t cols, const float *B, int64_t ldb, float *C, int64_t ldc, int32_t f, float beta,
+                      const SpmmPlan &plan) {
+  a.rowptr = rowptr;
+  a.colind = colind;
+  a.val = val;
+  a.task_row = sc->task_row;
+  a.tbase = sc->tbase;
+  a.pbase = sc->pbase;
+  a.ntasks = sc->ntasks;
+  a.seg = sc->seg;
+  a.m = cols;
+  a.B = B;
+  a.ldb = ldb;
+  a.C = C;
+  a.ldc = ldc;
+  a.f = f;
+  a.beta = beta;
+  a.tiles = plan.tiles;
+  a.tile_slots = plan.tile_slots;
+  a.groups = 1;
+  a.P = nullptr;
+}
+
+// Plain handle path for one column range: row-segment tasks over (rowptr, colind, val).
+static int spmm_plain(const int32_t *rowptr, const int32_t *colind, const float *val, int32_t rows, int32_t cols,
+                      SchedCache &cache, int vec, const float *B, int64_t ldb, float *C, int64_t ldc, int32_t f,
+                      float beta, int prof_tag, hipStream_t stream) {
+  SpmmPlan plan = plan_range(vec, f);
+  if (plan.shape.chunks > kMaxChunks) {  // tiling was tuned down: fall back to 8 tiles
+    plan.tiles = 8;
+    plan.tile_slots = (f / vec + 7) / 8;
+    plan.shape = pick_shape(vec, plan.tile_slots);
+  }
+  Sched *sc = nullptr;
+  CG_TRY(cache.get(rowptr, rows, pick_seg(plan.shape), &sc, stream));
+  SpmmArgs a{};
+  fill_args(a, rowptr, colind, val, sc, cols, B, ldb, C, ldc, f, beta, plan);
+  if (sc->nslots > 0) {
+    void *p = nullptr;
+    CG_TRY(scratch_get(stream, kSlotA, (size_t)sc->nslots * f * sizeof(float), &p));
+    a.P = (float *)p;
+  }
+  {
+    ProfScope prof("spmm_rowseg", prof_tag, stream);
+    CG_TRY((launch_shape<kModeTable>(plan.shape, a, stream)));
+  }
+  if (sc->nmulti > 0) {
+    ProfScope prof("spmm_reduce", prof_tag, stream);
+    const int64_t threads = sc->nmulti * (int64_t)f;
+    spmm_reduce_kernel<<<(unsigned)ceil_div64(threads, kSpmmThreads), kSpmmThreads, 0, stream>>>(
+        sc->multi_rows, sc->nmulti, rowptr, sc->pbase, sc->seg, a.P, C, ldc, f, beta);
+    CG_LAUNCH_CHECK();
+  }
+  return CG_OK;
+}
+
+// Should a product of this width over this matrix go through a hub plan?  It pays when a row of B
+// is many cache lines (the gather dominates) and rows hold enough hot entries per group that the
+// partial rows they cost are small against the gathers they turn into L2 hits.
+static bool want_hub(const CsrSide &s, int32_t f) {
+  const int t = g_tune_hub.load(std::memory_order_relaxed);
+  if (t < 0) return false;
+  if (s.rows == 0 || s.nnz == 0) return false;
+  if (t > 0) return true;
+  return f >= 256 && s.nnz / s.rows >= 128;
+}
+
+static int spmm_hub(CsrSide &s, int vec, const float *B, int64_t ldb, float *C, int64_t ldc, int32_t f, float beta,
+                    hipStream_t stream) {
+  int groups = g_tune_hub_groups.load(std::memory_order_relaxed);
+  if (groups != 1 && groups != 2 && groups != 4 && groups != 8) groups = 8;
+  int kb = g_tune_hub_kb.load(std::memory_order_relaxed);
+  if (kb <= 0) kb = 8192;  // twice the 4 MB L2 of an XCD: measured optimum, LRU keeps the hottest half
+  int64_t per_group = (int64_t)kb * 1024 / ((int64_t)f * 4);
+  if (per_group < 1) per_group = 1;
+  int64_t hot = per_group * groups;
+  if (hot > s.cols) hot = s.cols;
+  // hot tasks always use full-wave teams on the whole width, one dword per lane and chunk: that is
+  // the fastest gather of L2-resident rows whose start is not 16-byte aligned
+  const int hot_vec = vec == 4 ? 4 : 1;
+  SpmmPlan hplan;
+  hplan.tiles = 1;
+  hplan.tile_slots = f / hot_vec;
+  hplan.shape = pick_shape(hot_vec, hplan.tile_slots);
+  const int32_t seg = pick_seg(hplan.shape);
+  if (!s.hub.valid || s.hub.hot != (int32_t)hot || s.hub.groups != groups || s.hub.seg != seg)
+    CG_TRY(build_hub(s, (int32_t)hot, groups, seg, stream));
+  HubPlan &h = s.hub;
+  const int32_t n = s.rows;
+  // 1. cold class straight into C
+  CG_TRY(spmm_plain(h.vrowptr + (int64_t)groups * n, h.colind, h.val, n, s.cols, h.cold_sched, vec, B, ldb, C, ldc, f,
+                    beta, f, stream));
+  // 2. hot classes: every task writes a partial row
+  const int64_t hot_tasks = h.hot_sched.ntasks;
+  if (hot_tasks == 0) return CG_OK;
+  void *p = nullptr;
+  CG_TRY(scratch_get(stream, kSlotC, (size_t)hot_tasks * f * sizeof(float), &p));
+  SpmmArgs a{};
+  fill_args(a, h.vrowptr, h.colind, h.val, &h.hot_sched, s.cols, B, ldb, C, ldc, f, 0.f, hplan);
+  a.P = (float *)p;
+  a.groups = groups;
+  for (int g = 0; g <= groups; ++g) a.tstart[g] = h.tstart[g];
+  {
+    ProfScope prof("spmm_hub_hot", f, stream);
+    CG_TRY((launch_shape<kModeHub>(hplan.shape, a, stream)));
+  }
+  // 3. fold the partial rows into C
+  {
+    ProfScope prof("spmm_hub_reduce", f, stream);
+    hub_reduce_kernel<<<(unsigned)ceil_div64((int64_t)n * kWave, kSpmmThreads), kSpmmThreads, 0, stream>>>(
+        h.hot_sched.tbase, n, groups, a.P, C, ldc, f);
+    CG_LAUNCH_CHECK();
+  }
+  return CG_OK;
+}
+
 static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t ldc, int32_t f, float beta,
                      hipStream_t stream) {
   if (s.rows == 0) return CG_OK;
   const int vec = pick_vec(f, B, ldb, C, ldc);
   const int32_t cap = range_cap(vec) * 8;  // 8 tiles of kMaxChunks chunks
+  if (f <= range_cap(vec == 4 ? 4 : 1) && want_hub(s, f)) return spmm_hub(s, vec, B, ldb, C, ldc, f, beta, stream);
   for (int32_t f0 = 0; f0 < f; f0 += cap) {
     const int32_t ft = f - f0 < cap ? f - f0 : cap;
-    const float *Bt = B + f0;
-    float *Ct = C + f0;
-    SpmmPlan plan = plan_range(vec, ft);
-    if (plan.shape.chunks > kMaxChunks) {  // tiling was tuned down: fall back to 8 tiles
-      plan.tiles = 8;
-      plan.tile_slots = (ft / vec + 7) / 8;
-      plan.shape = pick_shape(vec, plan.tile_slots);
-    }
-    const SpmmShape shape = plan.shape;
-    Sched *sc = nullptr;
-    CG_TRY(build_sched(s, pick_seg(shape), &sc, stream));
-    SpmmArgs a{};
-    a.rowptr = s.rowptr;
-    a.colind = s.colind;
-    a.val = s.val;
-    a.task_row = sc->task_row;
-    a.tbase = sc->tbase;
-    a.pbase = sc->pbase;
-    a.ntasks = sc->ntasks;
-    a.seg = sc->seg;
-    a.m = s.cols;
-    a.B = Bt;
-    a.ldb = ldb;
-    a.C = Ct;
-    a.ldc = ldc;
-    a.f = ft;
-    a.beta = beta;
-    a.tiles = plan.tiles;
-    a.tile_slots = plan.tile_slots;
-    a.P = nullptr;
-    if (sc->nslots > 0) {
-      void *p = nullptr;
-      CG_TRY(scratch_get(stream, kSlotA, (size_t)sc->nslots * ft * sizeof(float), &p));
-      a.P = (float *)p;
-    }
-    {
-      ProfScope prof("spmm_rowseg", f, stream);
-      CG_TRY((launch_shape<true, false>(shape, a, stream)));
-    }
-    if (sc->nmulti > 0) {
-      ProfScope prof("spmm_reduce", f, stream);
-      const int64_t threads = sc->nmulti * (int64_t)ft;
-      spmm_reduce_kernel<<<(unsigned)ceil_div64(threads, kSpmmThreads), kSpmmThreads, 0, stream>>>(
-          sc->multi_rows, sc->nmulti, s.rowptr, sc->pbase, sc->seg, a.P, Ct, ldc, ft, beta);
-      CG_LAUNCH_CHECK();
-    }
+    CG_TRY(spmm_plain(s.rowptr, s.colind, s.val, s.rows, s.cols, s.sched, vec, B + f0, ldb, C + f0, ldc, ft, beta, f,
+                      stream));
   }
   return CG_OK;
 }
@@ -597,6 +962,7 @@ namespace cg {
 static int side_alloc(CsrSide &s, int32_t rows, int32_t cols, int64_t nnz) {
   s.rows = rows;
   s.cols = cols;
+  s.nnz = nnz;
   CG_TRY(dev_alloc((void **)&s.rowptr, (size_t)(rows + 1) * sizeof(int32_t)));
   CG_TRY(dev_alloc((void **)&s.colind, (size_t)nnz * sizeof(int32_t)));
   CG_TRY(dev_alloc((void **)&s.val, (size_t)nnz * sizeof(float)));
@@ -687,7 +1053,7 @@ int cg_spmm_coo(const int32_t *d_row, const int32_t *d_col, const float *d_val, 
     a.beta = beta;
     a.tiles = 1;
     a.tile_slots = ft / vec;
-    CG_TRY((launch_shape<false, true>(pick_shape(vec, ft / vec), a, stream)));
+    CG_TRY((launch_shape<kModeRows>(pick_shape(vec, ft / vec), a, stream)));
   }
   return CG_OK;
 }
@@ -738,6 +1104,10 @@ int cg_tune_set(const char *key, int value) {
   if (!key) CG_FAIL(CG_ERR_NULL, "cg_tune_set: key is NULL");
   if (!strcmp(key, "spmm_seg")) cg::g_tune_seg.store(value);
   else if (!strcmp(key, "spmm_tiles")) cg::g_tune_tiles.store(value);
+  else if (!strcmp(key, "spmm_vec")) cg::g_tune_vec.store(value);
+  else if (!strcmp(key, "spmm_hub")) cg::g_tune_hub.store(value);
+  else if (!strcmp(key, "spmm_hub_kb")) cg::g_tune_hub_kb.store(value);
+  else if (!strcmp(key, "spmm_hub_groups")) cg::g_tune_hub_groups.store(value);
   else CG_FAIL(CG_ERR_UNSUPPORTED, "cg_tune_set: unknown key %s", key);
   return CG_OK;
 }

@@ -75,6 +75,12 @@ def outer_product2(inputs_t: torch.Tensor, ag: torch.Tensor, rank: int = 0, size
     return ops.dense_xtg(inputs_t.t(), ag)
 
 
+def _padded_width(c: int) -> int:
+    """Widths that are not a multiple of 4 (41 classes) are carried in buffers padded to the next
+    multiple of 4 with zero columns, so that the SpMM over them moves 16 bytes per lane."""
+    return (c + 3) // 4 * 4
+
+
 def _kind(func) -> str:
     if func is F.relu or func is torch.relu or func == "relu":
         return "relu"
@@ -112,8 +118,16 @@ class GCNFunc(torch.autograd.Function):
         peers_bwd = ctx.group.backward if isinstance(ctx.group, ResidentBlocks) else None
         blocks = ctx.am_partitions
         use_t = ctx.size == 1 and blocks[0].has_transpose
+        width = grad_output.shape[1]
+        padded = _padded_width(width)
+        if padded != width and peers_bwd is None:
+            wide = torch.zeros(grad_output.shape[0], padded, dtype=grad_output.dtype, device=grad_output.device)
+            wide[:, :width].copy_(grad_output)
+            grad_output = wide
         # first backprop equation: A G (reference: same blocks, gcn_distr.py:326)
         ag = broad_func(ctx.node_count, blocks, grad_output, ctx.rank, ctx.size, peers_bwd, transpose=use_t)
+        if padded != width and peers_bwd is None:
+            ag = ag[:, :width]  # a view: the dense products take the row stride as leading dimension
         grad_input = ops.dense_gwt(ag, weight) if ctx.needs_input_grad[0] else None
         # second backprop equation reuses A G (gcn_distr.py:337)
         grad_weight = outer_product2(inputs.t(), ag) if ctx.needs_input_grad[1] else None

@@ -245,3 +245,64 @@ def test_spmm_rejects_bad_arguments(cuda):
     U = ops.CsrMatrix(_i32(row.flip(0), cuda), _i32(col.flip(0), cuda), val.flip(0).to(cuda), n, n, is_sorted=False)
     B = torch.randn(n, 16, generator=torch.Generator().manual_seed(2)).to(cuda)
     assert torch.equal(U.spmm(B), A.spmm(B))
+
+
+@pytest.fixture
+def tune():
+    """Set schedule knobs for one test and put the built-in choices back afterwards."""
+    from cagnet_amd._lib import lib
+    touched = []
+
+    def set_knob(key, value):
+        assert lib.cg_tune_set(key.encode(), int(value)) == 0
+        touched.append(key)
+
+    yield set_knob
+    for key in touched:
+        lib.cg_tune_set(key.encode(), 0)
+
+
+@pytest.mark.parametrize("groups", [8, 2, 1])
+@pytest.mark.parametrize("f", [602, 256, 300])
+def test_spmm_hub_plan_matches_oracle(cuda, tune, f, groups):
+    """Hub plan forced on a small power-law graph: hot columns dealt to XCD groups, cold class
+    straight into C, hot partial rows folded in afterwards.  A 64 KB hot budget keeps only a few
+    dozen columns hot, so all three classes of entries (hot, cold, rows without hot entries) occur."""
+    from cagnet_amd import ops
+    row, col, val, n = small_graph(11, 60000, seed=300 + f)
+    B = torch.randn(n, f, generator=torch.Generator().manual_seed(f))
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n, transpose=True)
+    plain = A.spmm(B.to(cuda))
+    tune("spmm_hub", 1)
+    tune("spmm_hub_kb", 64)
+    tune("spmm_hub_groups", groups)
+    got = A.spmm(B.to(cuda))
+    assert spmm_error(got, row, col, val, n, n, B) <= REL_TOL
+    assert torch.equal(got, A.spmm(B.to(cuda)))                       # deterministic
+    scale = A.spmm(B.abs().to(cuda)).clamp_min(1e-30)
+    assert float(((got - plain).abs() / scale).max()) <= 4e-6          # same sum, different order
+    C0 = torch.randn(n, f, generator=torch.Generator().manual_seed(f + 1))
+    C = C0.to(cuda).clone()
+    A.spmm(B.to(cuda), out=C, beta=1.0)
+    assert spmm_error(C, row, col, val, n, n, B, C0) <= REL_TOL
+    assert torch.equal(A.spmm(B.to(cuda), transpose=True), got)        # symmetric graph, same plan on A^T
+
+
+def test_spmm_hub_plan_rectangular_and_all_hot(cuda, tune):
+    from cagnet_amd import ops
+    n, m, f = 700, 1500, 320
+    row, col, val = random_coo(n, m, 60000, seed=12)
+    B = torch.randn(m, f, generator=torch.Generator().manual_seed(5))
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, m)
+    tune("spmm_hub", 1)
+    tune("spmm_hub_kb", 16)
+    assert spmm_error(A.spmm(B.to(cuda)), row, col, val, n, m, B) <= REL_TOL
+    tune("spmm_hub_kb", 1 << 20)   # every column is hot: the cold class is empty
+    assert spmm_error(A.spmm(B.to(cuda)), row, col, val, n, m, B) <= REL_TOL
+    # long hot rows are split into segments as well
+    n, m = 24, 6000
+    row, col, val = random_coo(n, m, n * 5000, seed=13)
+    B = torch.randn(m, f, generator=torch.Generator().manual_seed(6))
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, m)
+    tune("spmm_hub_kb", 4096)
+    assert spmm_error(A.spmm(B.to(cuda)), row, col, val, n, m, B) <= REL_TOL
