@@ -172,7 +172,7 @@ def main() -> int:
     loss = float(gcn.train.last_loss)
 
     kernels = {}
-    widths = sorted({f_in, hidden, classes})
+    widths = sorted({f_in, hidden, classes, (classes + 3) // 4 * 4})  # backward carries 41 classes padded to 44
     for f in widths:
         for kname in ("spmm_rowseg", "spmm_reduce", "spmm_hub_hot", "spmm_hub_reduce"):
             ms, cnt = prof_read(_lib.lib, f"{kname}/f={f}")

@@ -306,7 +306,7 @@ struct SpmmShape {
 constexpr int kMaxChunks = 10;
 
 // Tuning knobs (cg_tune_set): 0 = built-in choice.
-std::atomic<int> g_tune_seg{0}, g_tune_tiles{0}, g_tune_vec{0};
+std::atomic<int> g_tune_seg{0}, g_tune_tiles{0}, g_tune_vec{0}, g_tune_stream{0}, g_tune_win{0};
 
 // Widest vector the operands allow.
 static int pick_vec(int32_t f, const float *B, int64_t ldb, const float *C, int64_t ldc) {
@@ -524,15 +524,546 @@ static int make_sched(const int32_t *rowptr, int32_t n, int32_t seg, int skip_em
   return CG_OK;
 }
 
+struct TempFree {
+  void *p[16];
+  int count = 0;
+  ~TempFree() {
+    for (int i = 0; i < count; ++i)
+      if (p[i]) (void)hipFree(p[i]);
+  }
+  int alloc(void **out, size_t bytes) {
+    CG_TRY(dev_alloc(out, bytes));
+    p[count++] = *out;
+    return CG_OK;
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
+// streaming over windows of tasks
+// ---------------------------------------------------------------------------------------------
+// Tasks are contiguous in the entry stream (task t covers [task_start[t], task_start[t+1])), so a
+// wavefront that takes a window of consecutive tasks reads one contiguous piece of (colind, val)
+// and never pays a task's start-up latency more than once per window.  Windows hold at most 64
+// tasks (their metadata lives in one register per lane) and start a new one every `S` entries.
+struct StreamTab {
+  int32_t S = 0, groups = 0;
+  bool hub = false;
+  int32_t *task_start = nullptr, *task_dst = nullptr, *wstart = nullptr;
+  int64_t nwin = 0;
+  int64_t win_first[9] = {0};
+  void release() {
+    if (task_start) (void)hipFree(task_start);
+    if (task_dst) (void)hipFree(task_dst);
+    if (wstart) (void)hipFree(wstart);
+    task_start = task_dst = wstart = nullptr;
+    S = 0;
+  }
+};
+
+// task_dst: row index (>= 0) when the task is the whole row and goes straight to C, else
+// -(partial slot + 1).  In a hub plan every task is partial and its slot is its own index.
+__global__ __launch_bounds__(kSpmmThreads) void stream_tasks_kernel(const int32_t *__restrict__ rowptr, int32_t nrows,
+                                                                    const int32_t *__restrict__ task_row,
+                                                                    const int32_t *__restrict__ tbase,
+                                                                    const int32_t *__restrict__ pbase, int32_t seg,
+                                                                    int64_t ntasks, int hub,
+                                                                    int32_t *__restrict__ task_start,
+                                                                    int32_t *__restrict__ task_dst) {
+  const int64_t t = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (t > ntasks) return;
+  if (t == ntasks) {
+    task_start[t] = rowptr[nrows];
+    return;
+  }
+  const int32_t row = task_row[t];
+  const int32_t sidx = (int32_t)t - tbase[row];
+  const int32_t rs = rowptr[row], re = rowptr[row + 1];
+  task_start[t] = rs + sidx * seg;
+  task_dst[t] = hub ? -((int32_t)t + 1) : ((re - rs <= seg) ? row : -(pbase[row] + sidx + 1));
+}
+
+// flags[t] = 1 where a window starts: every 64th task of a class ...
+__global__ __launch_bounds__(kSpmmThreads) void window_flag_tasks_kernel(int64_t t0, int64_t t1,
+                                                                         uint32_t *__restrict__ flags) {
+  const int64_t t = t0 + (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (t < t1) flags[t] = ((t - t0) & 63) == 0 ? 1u : 0u;
+}
+
+// ... and the first task that starts at or after every multiple of S entries of the class.
+__global__ __launch_bounds__(kSpmmThreads) void window_flag_entries_kernel(const int32_t *__restrict__ task_start,
+                                                                           int64_t t0, int64_t t1, int32_t S,
+                                                                           int64_t nbounds,
+                                                                           uint32_t *__restrict__ flags) {
+  const int64_t j = 1 + (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (j > nbounds) return;
+  const int64_t target = (int64_t)task_start[t0] + j * S;
+  int64_t lo = t0, hi = t1;  // first t in [t0, t1) with task_start[t] >= target
+  while (lo < hi) {
+    const int64_t mid = (lo + hi) >> 1;
+    if (task_start[mid] < target) lo = mid + 1;
+    else hi = mid;
+  }
+  if (lo < t1) flags[lo] = 1u;  // several j may land on the same task: they all store 1
+}
+
+__global__ __launch_bounds__(kSpmmThreads) void window_compact_kernel(const uint32_t *__restrict__ flags,
+                                                                      const uint32_t *__restrict__ index,
+                                                                      int64_t ntasks, int32_t *__restrict__ wstart,
+                                                                      uint32_t nwin) {
+  const int64_t t = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (t < ntasks && flags[t]) wstart[index[t]] = (int32_t)t;
+  if (t == ntasks) wstart[nwin] = (int32_t)ntasks;
+}
+
+// class_first[g] .. class_first[g+1]: tasks of class g (nclass == 1 for a plain schedule).
+static int build_stream(const Sched &sc, const int32_t *rowptr, int32_t nrows, bool hub, int nclass,
+                        const int64_t *class_first, int32_t S, StreamTab &out, hipStream_t stream) {
+  out.release();
+  const int64_t nt = sc.ntasks;
+  CG_TRY(dev_alloc((void **)&out.task_start, (size_t)(nt + 1) * 4));
+  CG_TRY(dev_alloc((void **)&out.task_dst, (size_t)(nt + 1) * 4));
+  stream_tasks_kernel<<<(unsigned)ceil_div64(nt + 1, kSpmmThreads), kSpmmThreads, 0, stream>>>(
+      rowptr, nrows, sc.task_row, sc.tbase, sc.pbase, sc.seg, nt, hub ? 1 : 0, out.task_start, out.task_dst);
+  CG_LAUNCH_CHECK();
+  out.S = S;
+  out.hub = hub;
+  out.groups = nclass;
+  out.nwin = 0;
+  for (int g = 0; g <= nclass; ++g) out.win_first[g] = 0;
+  if (nt == 0) {
+    CG_TRY(dev_alloc((void **)&out.wstart, 4));
+    CG_HIP(hipMemsetAsync(out.wstart, 0, 4, stream));
+    CG_HIP(hipStreamSynchronize(stream));
+    return CG_OK;
+  }
+  uint32_t *flags = nullptr, *index = nullptr;
+  TempFree tmp;
+  CG_TRY(tmp.alloc((void **)&flags, (size_t)(nt + 1) * 4));
+  CG_TRY(tmp.alloc((void **)&index, (size_t)(nt + 1) * 4));
+  // entry extents of the classes (host needs them to size the boundary launches)
+  int32_t ends[10];
+  for (int g = 0; g <= nclass; ++g)
+    CG_HIP(hipMemcpyAsync(&ends[g], out.task_start + class_first[g], 4, hipMemcpyDeviceToHost, stream));
+  CG_HIP(hipStreamSynchronize(stream));
+  for (int g = 0; g < nclass; ++g) {
+    const int64_t t0 = class_first[g], t1 = class_first[g + 1];
+    if (t1 <= t0) continue;
+    window_flag_tasks_kernel<<<(unsigned)ceil_div64(t1 - t0, kSpmmThreads), kSpmmThreads, 0, stream>>>(t0, t1, flags);
+    CG_LAUNCH_CHECK();
+    const int64_t nb = ((int64_t)ends[g + 1] - ends[g]) / S;
+    if (nb > 0) {
+      window_flag_entries_kernel<<<(unsigned)ceil_div64(nb, kSpmmThreads), kSpmmThreads, 0, stream>>>(
+          out.task_start, t0, t1, S, nb, flags);
+      CG_LAUNCH_CHECK();
+    }
+  }
+  void *d_total_v = nullptr;
+  CG_TRY(scratch_get(stream, kSlotB, 4, &d_total_v));
+  CG_TRY(exclusive_scan_u32(flags, index, nt, (uint32_t *)d_total_v, stream));
+  uint32_t nwin = 0;
+  CG_HIP(hipMemcpyAsync(&nwin, d_total_v, 4, hipMemcpyDeviceToHost, stream));
+  uint32_t firsts[10] = {0};
+  for (int g = 0; g < nclass; ++g)
+    if (class_first[g] < nt) CG_HIP(hipMemcpyAsync(&firsts[g], index + class_first[g], 4, hipMemcpyDeviceToHost, stream));
+  CG_HIP(hipStreamSynchronize(stream));
+  for (int g = 0; g < nclass; ++g) out.win_first[g] = class_first[g] < nt ? firsts[g] : nwin;
+  out.win_first[nclass] = nwin;
+  out.nwin = nwin;
+  CG_TRY(dev_alloc((void **)&out.wstart, (size_t)(nwin + 1) * 4));
+  window_compact_kernel<<<(unsigned)ceil_div64(nt + 1, kSpmmThreads), kSpmmThreads, 0, stream>>>(flags, index, nt,
+                                                                                                out.wstart, nwin);
+  CG_LAUNCH_CHECK();
+  CG_HIP(hipStreamSynchronize(stream));
+  return CG_OK;
+}
+
+struct StreamArgs {
+  const int32_t *task_start, *task_dst, *wstart;
+  const int32_t *colind;
+  const float *val;
+  int64_t win_first[9];
+  int32_t groups;  // 1: windows run anywhere; 2/4/8: windows of class g run on XCDs x % groups == g
+  const float *B;
+  int64_t ldb;
+  float *C;
+  int64_t ldc;
+  float *P;
+  int32_t f;
+  float beta;
+};
+
+// Full-wave teams (one stored entry per wave step, f covered by CHUNKS x 64 lanes x VEC floats).
+template <int VEC, int CHUNKS>
+__global__ __launch_bounds__(kSpmmThreads) void spmm_stream_wide_kernel(const StreamArgs a) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int x = blockIdx.x & 7;
+  const int per = 8 / a.groups;
+  const int grp = x % a.groups;
+  const int64_t lblock = (int64_t)(blockIdx.x >> 3) * per + x / a.groups;
+  const int64_t wl = lblock * kWavesPerBlock + threadIdx.x / kWave;
+  if (wl >= a.win_first[grp + 1] - a.win_first[grp]) return;
+  const int32_t w = __builtin_amdgcn_readfirstlane((int32_t)(a.win_first[grp] + wl));
+  const int32_t t0 = a.wstart[w], t1 = a.wstart[w + 1];
+  const int ntask = t1 - t0;  // 1..64
+  int32_t m_end = 0, m_dst = 0;
+  if (lane < ntask) {
+    m_end = a.task_start[t0 + lane + 1];
+    m_dst = a.task_dst[t0 + lane];
+  }
+  const int32_t e_begin = a.task_start[t0];
+  const int32_t e_end = __builtin_amdgcn_readlane(m_end, ntask - 1);
+
+  const int nslots = a.f / VEC;
+  bool active[CHUNKS];
+  int64_t boff[CHUNKS];
+#pragma unroll
+  for (int ch = 0; ch < CHUNKS; ++ch) {
+    active[ch] = (ch * kWave + lane) < nslots;
+    boff[ch] = (int64_t)(ch * kWave + (active[ch] ? lane : 0)) * VEC;
+  }
+  float acc[CHUNKS][VEC];
+#pragma unroll
+  for (int ch = 0; ch < CHUNKS; ++ch)
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[ch][v] = 0.f;
+
+  constexpr int U = 4;
+  int tk = 0;
+  int32_t tbeg = e_begin;
+  int32_t tend = __builtin_amdgcn_readlane(m_end, 0);
+
+  int32_t c_next = 0;
+  float v_next = 0.f;
+  if (e_begin + lane < e_end) {
+    c_next = a.colind[e_begin + lane];
+    v_next = a.val[e_begin + lane];
+  }
+  for (int32_t base = e_begin;; base += kWave) {
+    const int32_t c = c_next;
+    const float v = v_next;
+    const int32_t nb = base + kWave + lane;
+    c_next = 0;
+    v_next = 0.f;
+    if (nb < e_end) {
+      c_next = a.colind[nb];
+      v_next = a.val[nb];
+    }
+    int cnt = e_end - base;
+    cnt = cnt > kWave ? kWave : (cnt < 0 ? 0 : cnt);
+    int i = 0;
+    for (;;) {
+      while (tend == base + i) {  // the current task is complete (also true at once for an empty task)
+        const int32_t dst = __builtin_amdgcn_readlane(m_dst, tk);
+        if (dst >= 0) {
+          if (!(tend == tbeg && a.beta == 1.0f)) {  // an empty row leaves C alone when beta == 1
+            float *crow = a.C + (int64_t)dst * a.ldc;
+#pragma unroll
+            for (int ch = 0; ch < CHUNKS; ++ch) {
+              if (active[ch]) {
+                float out[VEC];
+                if (a.beta != 0.f) {
+                  float old[VEC];
+                  load_vec<VEC>(crow + boff[ch], old);
+#pragma unroll
+                  for (int q = 0; q < VEC; ++q) out[q] = fmaf(a.beta, old[q], acc[ch][q]);
+                } else {
+#pragma unroll
+                  for (int q = 0; q < VEC; ++q) out[q] = acc[ch][q];
+                }
+                store_vec<VEC>(crow + boff[ch], out);
+              }
+            }
+          }
+        } else {
+          float *prow = a.P + (int64_t)(-(dst + 1)) * a.f;
+#pragma unroll
+          for (int ch = 0; ch < CHUNKS; ++ch)
+            if (active[ch]) store_vec<VEC>(prow + boff[ch], acc[ch]);
+        }
+#pragma unroll
+        for (int ch = 0; ch < CHUNKS; ++ch)
+#pragma unroll
+          for (int q = 0; q < VEC; ++q) acc[ch][q] = 0.f;
+        if (++tk == ntask) return;
+        tbeg = tend;
+        tend = __builtin_amdgcn_readlane(m_end, tk);
+      }
+      if (i >= cnt) break;
+      int run = tend - base;
+      run = run < cnt ? run : cnt;
+      if (run <= i) return;  // cannot happen with monotone task starts; guarantees termination
+      for (; i + U <= run; i += U) {
+        float b[U][CHUNKS][VEC];
+        float vv[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int32_t cc = __builtin_amdgcn_readlane(c, i + u);
+          vv[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), i + u));
+          const float *brow = a.B + (int64_t)cc * a.ldb;
+#pragma unroll
+          for (int ch = 0; ch < CHUNKS; ++ch) load_vec<VEC>(brow + boff[ch], b[u][ch]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int ch = 0; ch < CHUNKS; ++ch)
+#pragma unroll
+            for (int q = 0; q < VEC; ++q) acc[ch][q] = fmaf(vv[u], b[u][ch][q], acc[ch][q]);
+      }
+      for (; i < run; ++i) {
+        const int32_t cc = __builtin_amdgcn_readlane(c, i);
+        const float vv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), i));
+        const float *brow = a.B + (int64_t)cc * a.ldb;
+        float b[CHUNKS][VEC];
+#pragma unroll
+        for (int ch = 0; ch < CHUNKS; ++ch) load_vec<VEC>(brow + boff[ch], b[ch]);
+#pragma unroll
+        for (int ch = 0; ch < CHUNKS; ++ch)
+#pragma unroll
+          for (int q = 0; q < VEC; ++q) acc[ch][q] = fmaf(vv, b[ch][q], acc[ch][q]);
+      }
+    }
+  }
+}
+
+static int launch_stream_wide(int vec, int chunks, const StreamArgs &a, hipStream_t stream) {
+  int64_t longest = 0;
+  for (int g = 0; g < a.groups; ++g) {
+    const int64_t len = a.win_first[g + 1] - a.win_first[g];
+    longest = longest > len ? longest : len;
+  }
+  const int64_t blocks = ceil_div64(ceil_div64(longest, kWavesPerBlock), 8 / a.groups) * 8;
+  if (blocks == 0) return CG_OK;
+  if (blocks > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "SpMM grid too large");
+  const unsigned grid = (unsigned)blocks;
+#define CG_CASE(V, CH)                                                              \
+  if (vec == V && chunks == CH) {                                                   \
+    spmm_stream_wide_kernel<V, CH><<<grid, kSpmmThreads, 0, stream>>>(a);           \
+    CG_LAUNCH_CHECK();                                                              \
+    return CG_OK;                                                                   \
+  }
+#define CG_CASES(V)                                                                                     \
+  CG_CASE(V, 1) CG_CASE(V, 2) CG_CASE(V, 3) CG_CASE(V, 4) CG_CASE(V, 5) CG_CASE(V, 6) CG_CASE(V, 7)     \
+  CG_CASE(V, 8) CG_CASE(V, 9) CG_CASE(V, 10)
+  CG_CASES(1) CG_CASES(2) CG_CASES(4)
+#undef CG_CASES
+#undef CG_CASE
+  CG_FAIL(CG_ERR_UNSUPPORTED, "no streaming SpMM kernel for vec=%d chunks=%d", vec, chunks);
+}
+
+// Teams of LPR < 64 lanes (f <= 64 * VEC floats): the window's entries and task table are staged
+// in LDS.  Long tasks (>= kLongFactor * G entries) are worked on by all G teams together (entries
+// dealt round robin, partial sums combined by the xor butterfly); the short ones are dealt to the
+// teams whole, G at a time, so rows of a few entries cost neither a butterfly nor an idle wave.
+constexpr int kNarrowLds = 1024;  // entries a window may hold (window length S plus one task, both <= 512)
+constexpr int kLongFactor = 4;
+
+template <int VEC, int LPR>
+__global__ __launch_bounds__(kSpmmThreads) void spmm_stream_narrow_kernel(const StreamArgs a) {
+  constexpr int G = kWave / LPR;
+  __shared__ int32_t s_col[kWavesPerBlock][kNarrowLds];
+  __shared__ float s_val[kWavesPerBlock][kNarrowLds];
+  __shared__ int32_t s_beg[kWavesPerBlock][kWave], s_end[kWavesPerBlock][kWave], s_dst[kWavesPerBlock][kWave];
+  __shared__ int32_t s_short[kWavesPerBlock][kWave];
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wv = threadIdx.x / kWave;
+  const int x = blockIdx.x & 7;
+  const int per = 8 / a.groups;
+  const int grp = x % a.groups;
+  const int64_t lblock = (int64_t)(blockIdx.x >> 3) * per + x / a.groups;
+  const int64_t wl = lblock * kWavesPerBlock + wv;
+  if (wl >= a.win_first[grp + 1] - a.win_first[grp]) return;
+  const int32_t w = __builtin_amdgcn_readfirstlane((int32_t)(a.win_first[grp] + wl));
+  const int32_t t0 = a.wstart[w], t1 = a.wstart[w + 1];
+  const int ntask = t1 - t0;  // 1..64
+  const bool valid = lane < ntask;
+  int32_t m_beg = 0, m_end = 0, m_dst = 0;
+  if (valid) {
+    m_beg = a.task_start[t0 + lane];
+    m_end = a.task_start[t0 + lane + 1];
+    m_dst = a.task_dst[t0 + lane];
+  }
+  const int32_t e_begin = __builtin_amdgcn_readlane(m_beg, 0);
+  const int32_t e_end = __builtin_amdgcn_readlane(m_end, ntask - 1);
+  const int32_t nent = e_end - e_begin;
+  if (nent > kNarrowLds) return;  // excluded by the schedule (S + seg <= kNarrowLds); keeps LDS writes in bounds
+
+  for (int32_t k = lane; k < nent; k += kWave) {
+    s_col[wv][k] = a.colind[e_begin + k];
+    s_val[wv][k] = a.val[e_begin + k];
+  }
+  const int32_t r_beg = m_beg - e_begin, r_end = m_end - e_begin;  // relative to the window
+  s_beg[wv][lane] = r_beg;
+  s_end[wv][lane] = r_end;
+  s_dst[wv][lane] = m_dst;
+  const int32_t len = r_end - r_beg;
+  const bool is_long = valid && len >= kLongFactor * G;
+  // an empty row that goes straight to C needs no work when beta == 1
+  const bool is_short = valid && !is_long && !(len == 0 && m_dst >= 0 && a.beta == 1.0f);
+
+  const int g = lane / LPR, j = lane % LPR;
+  const bool active = j * VEC < a.f;
+  const int64_t boff = active ? (int64_t)j * VEC : 0;
+  const int32_t *cw = s_col[wv];
+  const float *vw = s_val[wv];
+
+  const uint64_t short_mask = __ballot(is_short);
+  if (is_short) s_short[wv][__popcll(short_mask & ((1ull << lane) - 1ull))] = lane;
+  const int nshort = __popcll(short_mask);
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+  __builtin_amdgcn_wave_barrier();  // the staged window and tables are visible to every lane of the wave
+
+  // ---- long tasks: all teams together
+  uint64_t long_mask = __ballot(is_long);
+  while (long_mask) {
+    const int k = __builtin_ctzll(long_mask);
+    long_mask &= long_mask - 1;
+    const int32_t s = __builtin_amdgcn_readlane(r_beg, k);
+    const int32_t e = __builtin_amdgcn_readlane(r_end, k);
+    const int32_t d = __builtin_amdgcn_readlane(m_dst, k);
+    float acc[VEC];
+#pragma unroll
+    for (int q = 0; q < VEC; ++q) acc[q] = 0.f;
+    int32_t i = s + g;
+    for (; i + 3 * G < e; i += 4 * G) {
+      float b[4][VEC], vv[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int32_t cc = cw[i + u * G];
+        vv[u] = vw[i + u * G];
+        load_vec<VEC>(a.B + (int64_t)cc * a.ldb + boff, b[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int q = 0; q < VEC; ++q) acc[q] = fmaf(vv[u], b[u][q], acc[q]);
+    }
+    for (; i < e; i += G) {
+      float b[VEC];
+      const float vv = vw[i];
+      load_vec<VEC>(a.B + (int64_t)cw[i] * a.ldb + boff, b);
+#pragma unroll
+      for (int q = 0; q < VEC; ++q) acc[q] = fmaf(vv, b[q], acc[q]);
+    }
+#pragma unroll
+    for (int off = LPR; off < kWave; off <<= 1)
+#pragma unroll
+      for (int q = 0; q < VEC; ++q) acc[q] += __shfl_xor(acc[q], off, kWave);
+    if (g == 0 && active) {
+      if (d >= 0) {
+        float *crow = a.C + (int64_t)d * a.ldc + boff;
+        float out[VEC];
+        if (a.beta != 0.f) {
+          float old[VEC];
+          load_vec<VEC>(crow, old);
+#pragma unroll
+          for (int q = 0; q < VEC; ++q) out[q] = fmaf(a.beta, old[q], acc[q]);
+        } else {
+#pragma unroll
+          for (int q = 0; q < VEC; ++q) out[q] = acc[q];
+        }
+        store_vec<VEC>(crow, out);
+      } else {
+        store_vec<VEC>(a.P + (int64_t)(-(d + 1)) * a.f + boff, acc);
+      }
+    }
+  }
+
+  // ---- short tasks: one team each, G per round
+  for (int q0 = 0; q0 < nshort; q0 += G) {
+    const int my = q0 + g;
+    const bool has = my < nshort;
+    const int k = has ? s_short[wv][my] : 0;
+    const int32_t s = s_beg[wv][k];
+    const int32_t e = has ? s_end[wv][k] : s;
+    const int32_t d = s_dst[wv][k];
+    float acc[VEC];
+#pragma unroll
+    for (int q = 0; q < VEC; ++q) acc[q] = 0.f;
+    int32_t i = s;
+    for (; i + 3 < e; i += 4) {
+      float b[4][VEC], vv[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int32_t cc = cw[i + u];
+        vv[u] = vw[i + u];
+        load_vec<VEC>(a.B + (int64_t)cc * a.ldb + boff, b[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int q = 0; q < VEC; ++q) acc[q] = fmaf(vv[u], b[u][q], acc[q]);
+    }
+    for (; i < e; ++i) {
+      float b[VEC];
+      const float vv = vw[i];
+      load_vec<VEC>(a.B + (int64_t)cw[i] * a.ldb + boff, b);
+#pragma unroll
+      for (int q = 0; q < VEC; ++q) acc[q] = fmaf(vv, b[q], acc[q]);
+    }
+    if (has && active) {
+      if (d >= 0) {
+        float *crow = a.C + (int64_t)d * a.ldc + boff;
+        float out[VEC];
+        if (a.beta != 0.f) {
+          float old[VEC];
+          load_vec<VEC>(crow, old);
+#pragma unroll
+          for (int q = 0; q < VEC; ++q) out[q] = fmaf(a.beta, old[q], acc[q]);
+        } else {
+#pragma unroll
+          for (int q = 0; q < VEC; ++q) out[q] = acc[q];
+        }
+        store_vec<VEC>(crow, out);
+      } else {
+        store_vec<VEC>(a.P + (int64_t)(-(d + 1)) * a.f + boff, acc);
+      }
+    }
+  }
+}
+
+static int64_t stream_grid(const StreamArgs &a) {
+  int64_t longest = 0;
+  for (int g = 0; g < a.groups; ++g) {
+    const int64_t len = a.win_first[g + 1] - a.win_first[g];
+    longest = longest > len ? longest : len;
+  }
+  return ceil_div64(ceil_div64(longest, kWavesPerBlock), 8 / a.groups) * 8;
+}
+
+static int launch_stream_narrow(int vec, int lpr, const StreamArgs &a, hipStream_t stream) {
+  const int64_t blocks = stream_grid(a);
+  if (blocks == 0) return CG_OK;
+  if (blocks > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "SpMM grid too large");
+  const unsigned grid = (unsigned)blocks;
+#define CG_CASE(V, L)                                                               \
+  if (vec == V && lpr == L) {                                                       \
+    spmm_stream_narrow_kernel<V, L><<<grid, kSpmmThreads, 0, stream>>>(a);          \
+    CG_LAUNCH_CHECK();                                                              \
+    return CG_OK;                                                                   \
+  }
+#define CG_CASES(V) CG_CASE(V, 4) CG_CASE(V, 8) CG_CASE(V, 16) CG_CASE(V, 32)
+  CG_CASES(1) CG_CASES(2) CG_CASES(4)
+#undef CG_CASES
+#undef CG_CASE
+  CG_FAIL(CG_ERR_UNSUPPORTED, "no narrow streaming SpMM kernel for vec=%d lpr=%d", vec, lpr);
+}
+
 // A small cache of schedules keyed by segment length.
 struct SchedCache {
   static constexpr int kMax = 4;
   Sched sched[kMax];
+  StreamTab tab[kMax];  // window tables of sched[i], built on first use
   int count = 0;
   void release() {
-    for (int i = 0; i < count; ++i) sched[i].release();
+    for (int i = 0; i < count; ++i) {
+      sched[i].release();
+      tab[i].release();
+    }
     count = 0;
   }
+  StreamTab &tab_of(const Sched *s) { return tab[s - sched]; }
   int get(const int32_t *rowptr, int32_t n, int32_t seg, Sched **out, hipStream_t stream) {
     for (int i = 0; i < count; ++i)
       if (sched[i].seg == seg) {
@@ -542,8 +1073,13 @@ struct SchedCache {
     if (count == kMax) {  // recycle the oldest
       CG_HIP(hipStreamSynchronize(stream));
       sched[0].release();
-      for (int i = 1; i < count; ++i) sched[i - 1] = sched[i];
+      tab[0].release();
+      for (int i = 1; i < count; ++i) {
+        sched[i - 1] = sched[i];
+        tab[i - 1] = tab[i];
+      }
       sched[--count] = Sched();
+      tab[count] = StreamTab();
     }
     CG_TRY(make_sched(rowptr, n, seg, 0, sched[count], stream));
     *out = &sched[count++];
@@ -560,11 +1096,13 @@ struct HubPlan {
   int32_t *vrowptr = nullptr, *colind = nullptr;
   float *val = nullptr;
   Sched hot_sched;        // over the virtual rows of the hot classes, empty rows skipped
+  StreamTab hot_tab;      // its windows, one class per group
   SchedCache cold_sched;  // over the cold class
   int64_t tstart[9] = {0};
   bool valid = false;
   void release() {
     hot_sched.release();
+    hot_tab.release();
     cold_sched.release();
     if (vrowptr) (void)hipFree(vrowptr);
     if (colind) (void)hipFree(colind);
@@ -601,6 +1139,7 @@ static int32_t pick_seg(const SpmmShape &s) {
   if (t >= 64) return t;
   const int g = kWave / s.lpr;
   if (g == 1) return 1024;
+  if (g_tune_stream.load(std::memory_order_relaxed) >= 0) return 512;  // a window and one task fit the LDS stage
   if (g == 2) return 2048;
   return 4096;
 }
@@ -670,20 +1209,6 @@ __global__ __launch_bounds__(kSpmmThreads) void csr_rows_kernel(const int32_t *_
   const int32_t s = rowptr[wave], e = rowptr[wave + 1];
   for (int32_t k = s + lane; k < e; k += kWave) row_out[k] = (int32_t)wave;
 }
-
-struct TempFree {
-  void *p[16];
-  int count = 0;
-  ~TempFree() {
-    for (int i = 0; i < count; ++i)
-      if (p[i]) (void)hipFree(p[i]);
-  }
-  int alloc(void **out, size_t bytes) {
-    CG_TRY(dev_alloc(out, bytes));
-    p[count++] = *out;
-    return CG_OK;
-  }
-};
 
 static int build_hub(CsrSide &s, int32_t hot, int32_t groups, int32_t seg, hipStream_t stream) {
   HubPlan &h = s.hub;
@@ -817,6 +1342,12 @@ __global__ __launch_bounds__(kSpmmThreads) void hub_reduce_kernel(const int32_t 
 
 std::atomic<int> g_tune_hub{0}, g_tune_hub_kb{0}, g_tune_hub_groups{0};
 
+// stored entries after which a new window starts
+static int32_t window_entries() {
+  const int w = g_tune_win.load(std::memory_order_relaxed);
+  return w >= 64 ? w : 512;
+}
+
 static void fill_args(SpmmArgs &a, const int32_t *rowptr, const int32_t *colind, const float *val, const Sched *sc,
                       int32_t cols, const float *B, int64_t ldb, float *C, int64_t ldc, int32_t f, float beta,
                       const SpmmPlan &plan) {
@@ -860,7 +1391,36 @@ static int spmm_plain(const int32_t *rowptr, const int32_t *colind, const float 
     CG_TRY(scratch_get(stream, kSlotA, (size_t)sc->nslots * f * sizeof(float), &p));
     a.P = (float *)p;
   }
-  {
+  const bool narrow = plan.shape.lpr < kWave;
+  if (plan.tiles == 1 && g_tune_stream.load(std::memory_order_relaxed) >= 0 &&
+      (!narrow || (sc->seg <= 512 && window_entries() <= 512))) {
+    // stream windows of consecutive tasks
+    StreamTab &tab = cache.tab_of(sc);
+    const int32_t S = window_entries();
+    if (tab.S != S) {
+      const int64_t first[2] = {0, sc->ntasks};
+      CG_TRY(build_stream(*sc, rowptr, rows, false, 1, first, S, tab, stream));
+    }
+    StreamArgs sa{};
+    sa.task_start = tab.task_start;
+    sa.task_dst = tab.task_dst;
+    sa.wstart = tab.wstart;
+    sa.colind = colind;
+    sa.val = val;
+    sa.win_first[0] = 0;
+    sa.win_first[1] = tab.nwin;
+    sa.groups = 1;
+    sa.B = B;
+    sa.ldb = ldb;
+    sa.C = C;
+    sa.ldc = ldc;
+    sa.P = a.P;
+    sa.f = f;
+    sa.beta = beta;
+    ProfScope prof("spmm_rowseg", prof_tag, stream);
+    if (narrow) CG_TRY(launch_stream_narrow(vec, plan.shape.lpr, sa, stream));
+    else CG_TRY(launch_stream_wide(vec, plan.shape.chunks, sa, stream));
+  } else {
     ProfScope prof("spmm_rowseg", prof_tag, stream);
     CG_TRY((launch_shape<kModeTable>(plan.shape, a, stream)));
   }
@@ -882,7 +1442,7 @@ static bool want_hub(const CsrSide &s, int32_t f) {
   if (t < 0) return false;
   if (s.rows == 0 || s.nnz == 0) return false;
   if (t > 0) return true;
-  return f >= 256 && s.nnz / s.rows >= 128;
+  return f >= 128 && s.nnz / s.rows >= 128;
 }
 
 static int spmm_hub(CsrSide &s, int vec, const float *B, int64_t ldb, float *C, int64_t ldc, int32_t f, float beta,
@@ -897,7 +1457,7 @@ static int spmm_hub(CsrSide &s, int vec, const float *B, int64_t ldb, float *C, 
   if (hot > s.cols) hot = s.cols;
   // hot tasks always use full-wave teams on the whole width, one dword per lane and chunk: that is
   // the fastest gather of L2-resident rows whose start is not 16-byte aligned
-  const int hot_vec = vec == 4 ? 4 : 1;
+  const int hot_vec = (vec == 4 || f / vec <= kWave) ? vec : 1;
   SpmmPlan hplan;
   hplan.tiles = 1;
   hplan.tile_slots = f / hot_vec;
@@ -920,7 +1480,30 @@ static int spmm_hub(CsrSide &s, int vec, const float *B, int64_t ldb, float *C, 
   a.P = (float *)p;
   a.groups = groups;
   for (int g = 0; g <= groups; ++g) a.tstart[g] = h.tstart[g];
-  {
+  const bool hnarrow = hplan.shape.lpr < kWave;
+  if (g_tune_stream.load(std::memory_order_relaxed) >= 0 && (!hnarrow || (seg <= 512 && window_entries() <= 512))) {
+    const int32_t S = window_entries();
+    if (h.hot_tab.S != S || h.hot_tab.groups != groups)
+      CG_TRY(build_stream(h.hot_sched, h.vrowptr, groups * n, true, groups, h.tstart, S, h.hot_tab, stream));
+    StreamArgs sa{};
+    sa.task_start = h.hot_tab.task_start;
+    sa.task_dst = h.hot_tab.task_dst;
+    sa.wstart = h.hot_tab.wstart;
+    sa.colind = h.colind;
+    sa.val = h.val;
+    for (int g = 0; g <= groups; ++g) sa.win_first[g] = h.hot_tab.win_first[g];
+    sa.groups = groups;
+    sa.B = B;
+    sa.ldb = ldb;
+    sa.C = C;
+    sa.ldc = ldc;
+    sa.P = (float *)p;
+    sa.f = f;
+    sa.beta = 0.f;
+    ProfScope prof("spmm_hub_hot", f, stream);
+    if (hnarrow) CG_TRY(launch_stream_narrow(hot_vec, hplan.shape.lpr, sa, stream));
+    else CG_TRY(launch_stream_wide(hot_vec, hplan.shape.chunks, sa, stream));
+  } else {
     ProfScope prof("spmm_hub_hot", f, stream);
     CG_TRY((launch_shape<kModeHub>(hplan.shape, a, stream)));
   }
@@ -1106,6 +1689,8 @@ int cg_tune_set(const char *key, int value) {
   else if (!strcmp(key, "spmm_tiles")) cg::g_tune_tiles.store(value);
   else if (!strcmp(key, "spmm_vec")) cg::g_tune_vec.store(value);
   else if (!strcmp(key, "spmm_hub")) cg::g_tune_hub.store(value);
+  else if (!strcmp(key, "spmm_stream")) cg::g_tune_stream.store(value);
+  else if (!strcmp(key, "spmm_win")) cg::g_tune_win.store(value);
   else if (!strcmp(key, "spmm_hub_kb")) cg::g_tune_hub_kb.store(value);
   else if (!strcmp(key, "spmm_hub_groups")) cg::g_tune_hub_groups.store(value);
   else CG_FAIL(CG_ERR_UNSUPPORTED, "cg_tune_set: unknown key %s", key);
