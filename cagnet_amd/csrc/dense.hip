@@ -9,7 +9,20 @@
 //        every K-slice writes a partial product, a second kernel adds the slices in order.
 #include "common.h"
 
+#include <atomic>
+
 namespace cg {
+
+// dense_mfma.hip
+int xw_mfma(const float *X, int64_t ldx, const float *W, int64_t ldw, float *Z, int64_t ldz, int64_t n, int32_t k,
+            int32_t fo, int relu, hipStream_t stream);
+int xtg_mfma(const float *X, int64_t ldx, const float *G, int64_t ldg, float *P, int64_t n, int32_t k, int32_t fo,
+             int64_t rows_per_block, int64_t nblocks, hipStream_t stream);
+int gwt_mfma(const float *G, int64_t ldg, const float *W, int64_t ldw, float *dX, int64_t lddx, int64_t n, int32_t k,
+             int32_t fo, hipStream_t stream);
+
+// cg_tune_set("dense_mfma", -1) routes every product through the LDS-tiled vector kernel below
+std::atomic<int> g_tune_dense_mfma{0};
 
 constexpr int kGemmThreads = 256;
 constexpr int kKT = 16;  // K tile
@@ -235,6 +248,8 @@ int cg_dense_xw(const float *d_X, int64_t ldx, const float *d_W, int64_t ldw, fl
   if (n == 0) return CG_OK;
   GemmArgs g{d_X, ldx, d_W, ldw, d_Z, ldz, n, fo, k, ceil_div64(k, kKT) * kKT, 1, relu ? 1 : 0};
   ProfScope prof("dense_xw", k, (hipStream_t)stream);
+  if (fo <= 64 && g_tune_dense_mfma.load(std::memory_order_relaxed) >= 0)
+    return xw_mfma(d_X, ldx, d_W, ldw, d_Z, ldz, n, k, fo, relu ? 1 : 0, (hipStream_t)stream);
   return launch_gemm<false, false>(g, (hipStream_t)stream);
 }
 
@@ -246,6 +261,10 @@ int cg_dense_gwt(const float *d_G, int64_t ldg, const float *d_W, int64_t ldw, f
   if (n == 0) return CG_OK;
   GemmArgs g{d_G, ldg, d_W, ldw, d_dX, lddx, n, k, fo, ceil_div64(fo, kKT) * kKT, 1, 0};
   ProfScope prof("dense_gwt", k, (hipStream_t)stream);
+  // the matrix-core form pays when the result is narrow; a wide result is bound by its stores,
+  // which the vector kernel issues in longer contiguous runs
+  if (fo <= 64 && k <= 64 && g_tune_dense_mfma.load(std::memory_order_relaxed) >= 0)
+    return gwt_mfma(d_G, ldg, d_W, ldw, d_dX, lddx, n, k, fo, (hipStream_t)stream);
   return launch_gemm<false, true>(g, (hipStream_t)stream);
 }
 
@@ -255,6 +274,24 @@ int cg_dense_xtg(const float *d_X, int64_t ldx, const float *d_G, int64_t ldg, f
   hipStream_t stream = (hipStream_t)stream_;
   CG_TRY(check_gemm("cg_dense_xtg", d_X, d_G, d_dW, n, k, fo));
   if (ldx < k || ldg < fo || lddw < fo) CG_FAIL(CG_ERR_SIZE, "cg_dense_xtg: leading dimension too small");
+  if (fo <= 64 && n > 0 && g_tune_dense_mfma.load(std::memory_order_relaxed) >= 0) {
+    ProfScope prof("dense_xtg", k, stream);
+    // contiguous vertex ranges, enough wavefronts to keep ~16 per CU in flight
+    const int vecw = (ldx % 4 == 0 && ((uintptr_t)d_X) % 16 == 0 && k >= 4) ? 4 : ((ldx % 2 == 0 && ((uintptr_t)d_X) % 8 == 0 && k >= 2) ? 2 : 1);
+    const int64_t ywaves = ceil_div64(k, 16 * vecw);
+    int64_t nblocks = ceil_div64(8192, ywaves);
+    if (nblocks > 1024) nblocks = 1024;
+    int64_t rows_per_block = ceil_div64(ceil_div64(n, nblocks), 16) * 16;
+    nblocks = ceil_div64(n, rows_per_block);
+    const int64_t elems = (int64_t)k * fo;
+    void *p = nullptr;
+    CG_TRY(scratch_get(stream, kSlotA, (size_t)nblocks * elems * sizeof(float), &p));
+    CG_TRY(xtg_mfma(d_X, ldx, d_G, ldg, (float *)p, n, k, fo, rows_per_block, nblocks, stream));
+    gemm_slice_sum_kernel<<<(unsigned)ceil_div64(elems, kSumOut), kGemmThreads, 0, stream>>>(
+        (const float *)p, elems, (int32_t)nblocks, d_dW, lddw, fo);
+    CG_LAUNCH_CHECK();
+    return CG_OK;
+  }
   // slices over the vertex dimension: enough workgroups to fill 256 CUs several times over
   const int bn = fo <= 16 ? 16 : (fo <= 32 ? 32 : 64);
   const int64_t tiles = ceil_div64(k, 4096 / bn) * ceil_div64(fo, bn);

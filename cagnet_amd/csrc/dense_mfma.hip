@@ -1,0 +1,314 @@
+// Tall-skinny dense products of GCNFunc on the fp32 matrix cores (v_mfma_f32_16x16x4_f32: exact
+// fp32 multiply-add, 16x16 output tile per wavefront, 4 reduction steps per instruction).
+// One dimension of each product is the vertex count, the others are feature widths of 16..602, so
+// each kernel is one pass over a large operand; the matrix instruction is used because it turns a
+// 64-lane load straight into 1024 multiply-adds without staging the large operand in LDS.
+//
+// Register layout of the instruction (lane l of 64):
+//   A (16 x 4): lane holds A[l % 16][l / 16]        B (4 x 16): lane holds B[l / 16][l % 16]
+//   D (16 x 16) in 4 registers: register v of lane l holds D[4 * (l / 16) + v][l % 16]
+//
+//   xw_mfma  : Z[n, fo]   = X[n, k] * W[k, fo]  (+ReLU)   rows of X on the tile rows, W staged in LDS
+//   xtg_mfma : dW[k, fo]  = X[n, k]^T * G[n, fo]          columns of X on the tile rows, vertices reduced
+//   gwt_mfma : dX[n, k]   = G[n, fo] * W[k, fo]^T         computed as (W G^T) so a lane owns 4 consecutive
+//                                                         outputs of one row and stores them as one vector
+#include "common.h"
+
+namespace cg {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kMfmaThreads = 256;
+constexpr int kMfmaWaves = kMfmaThreads / kWave;
+
+__device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
+template <int VEC>
+__device__ __forceinline__ void load_k(const float *p, bool ok, float (&r)[VEC]) {
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) r[i] = 0.f;
+  if (!ok) return;
+  if (VEC == 4) {
+    const float4 t = *reinterpret_cast<const float4 *>(p);
+    r[0] = t.x; r[1 % VEC] = t.y; r[2 % VEC] = t.z; r[3 % VEC] = t.w;
+  } else if (VEC == 2) {
+    const float2 t = *reinterpret_cast<const float2 *>(p);
+    r[0] = t.x; r[1 % VEC] = t.y;
+  } else {
+    r[0] = p[0];
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Z = X W.  A wavefront owns 16 rows of X; lane (m, q) = (l % 16, l / 16) reads VEC consecutive
+// k-values of row m per step, which feed VEC instructions whose B operand comes from the W chunk
+// staged in LDS.  NT output tiles of 16 columns share every A value.
+// ---------------------------------------------------------------------------------------------
+constexpr int kXwChunk = 256;  // rows of W staged per pass (multiple of 16)
+
+template <int VEC, int NT>
+__global__ __launch_bounds__(kMfmaThreads) void xw_mfma_kernel(const float *__restrict__ X, int64_t ldx,
+                                                               const float *__restrict__ W, int64_t ldw,
+                                                               float *__restrict__ Z, int64_t ldz, int64_t n,
+                                                               int32_t k, int32_t fo, int relu) {
+  __shared__ float Ws[kXwChunk][16 * NT];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int m = lane & 15, q = lane >> 4;
+  const int64_t r0 = ((int64_t)blockIdx.x * kMfmaWaves + wave) * 16;
+  int64_t row = r0 + m;
+  if (row >= n) row = n - 1;  // clamp: the extra rows are computed and dropped
+  const float *xrow = X + row * ldx;
+
+  floatx4 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  for (int32_t c0 = 0; c0 < k; c0 += kXwChunk) {
+    const int32_t clen = k - c0 < kXwChunk ? k - c0 : kXwChunk;
+    __syncthreads();
+    // rows past the end of the chunk are read (as zeros) by the last load steps: stage them too
+    constexpr int kStepRows = 4 * VEC * 4;
+    const int32_t stage_rows = (clen + kStepRows - 1) / kStepRows * kStepRows < kXwChunk
+                                   ? (clen + kStepRows - 1) / kStepRows * kStepRows
+                                   : kXwChunk;
+    for (int idx = threadIdx.x; idx < stage_rows * 16 * NT; idx += kMfmaThreads) {
+      const int kk = idx / (16 * NT), c = idx % (16 * NT);
+      Ws[kk][c] = (kk < clen && c < fo) ? W[(int64_t)(c0 + kk) * ldw + c] : 0.f;
+    }
+    __syncthreads();
+    constexpr int STEP = 4 * VEC;  // k-values one load step covers
+    constexpr int U = 4;           // load steps in flight
+    for (int32_t kb = 0; kb < clen; kb += STEP * U) {
+      float x[U][VEC];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int32_t kk = kb + u * STEP + q * VEC;
+        load_k<VEC>(xrow + c0 + kk, kk + VEC <= clen, x[u]);
+        if (VEC > 1 && kk < clen && kk + VEC > clen) {  // ragged end of the row: element-wise
+#pragma unroll
+          for (int s = 0; s < VEC; ++s) x[u][s] = kk + s < clen ? xrow[c0 + kk + s] : 0.f;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int s = 0; s < VEC; ++s) {
+          const int32_t kk = kb + u * STEP + q * VEC + s;
+          if (kb + u * STEP < clen) {  // wave-uniform: skip steps past the chunk
+            const float *wrow = Ws[kk < kXwChunk ? kk : kXwChunk - 1];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) acc[t] = mfma16(x[u][s], wrow[t * 16 + m], acc[t]);
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int64_t orow = r0 + 4 * q + v;
+      const int32_t col = t * 16 + m;
+      if (orow < n && col < fo) {
+        float o = acc[t][v];
+        if (relu && o < 0.f) o = 0.f;
+        Z[orow * ldz + col] = o;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dW = X^T G.  A wavefront owns 16 * VEC columns of X and all fo columns of G; every step consumes
+// 4 vertices: lane (m, q) reads VEC consecutive columns of vertex row r + q, lane (j, q) of the B
+// side reads G[r + q][16 t + j].  Workgroups take contiguous vertex ranges and write partial
+// products that are added in order afterwards.
+// ---------------------------------------------------------------------------------------------
+template <int VEC, int NT>
+__global__ __launch_bounds__(kMfmaThreads) void xtg_mfma_kernel(const float *__restrict__ X, int64_t ldx,
+                                                                const float *__restrict__ G, int64_t ldg,
+                                                                float *__restrict__ P, int64_t n, int32_t k,
+                                                                int32_t fo, int64_t rows_per_block) {
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int m = lane & 15, q = lane >> 4;
+  const int32_t kt0 = (blockIdx.y * kMfmaWaves + wave) * 16 * VEC;  // first column of this wave
+  if (kt0 >= k) return;
+  const int32_t kcol = kt0 + m * VEC;
+  const bool full = kcol + VEC <= k;
+  const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
+  const int64_t r1 = r0 + rows_per_block < n ? r0 + rows_per_block : n;
+
+  floatx4 acc[VEC][NT];
+#pragma unroll
+  for (int s = 0; s < VEC; ++s)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[s][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  constexpr int U = 8;  // 4-vertex steps in flight
+  for (int64_t r = r0; r < r1; r += 4 * U) {
+    float x[U][VEC], g[U][NT];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t rr = r + u * 4 + q;
+      const bool live = rr < r1;
+      const float *xp = X + (live ? rr : r0) * ldx + kcol;
+      load_k<VEC>(xp, live && full, x[u]);
+      if (VEC > 1 && live && !full) {
+#pragma unroll
+        for (int s = 0; s < VEC; ++s) x[u][s] = kcol + s < k ? xp[s] : 0.f;
+      }
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const int32_t c = t * 16 + m;
+        g[u][t] = (live && c < fo) ? G[rr * ldg + c] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int s = 0; s < VEC; ++s)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[s][t] = mfma16(x[u][s], g[u][t], acc[s][t]);
+  }
+  float *out = P + (int64_t)blockIdx.x * k * fo;
+#pragma unroll
+  for (int s = 0; s < VEC; ++s)
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int32_t kc = kt0 + (4 * q + v) * VEC + s;  // tile row i = 4q + v holds column kt0 + i*VEC + s
+        const int32_t c = t * 16 + m;
+        if (kc < k && c < fo) out[(int64_t)kc * fo + c] = acc[s][t][v];
+      }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dX = G W^T, computed tile-wise as (W G^T): tile rows are 16 columns of dX (= rows of W), tile
+// columns are 16 vertices.  Register v of lane (j, q) then holds dX[r + j][kt + 4q + v], four
+// consecutive outputs of one row, stored as one vector.  The G values of the 16 vertices are kept
+// in registers across all column tiles.
+// ---------------------------------------------------------------------------------------------
+template <int KS>  // reduction steps: fo <= 4 * KS
+__global__ __launch_bounds__(kMfmaThreads) void gwt_mfma_kernel(const float *__restrict__ G, int64_t ldg,
+                                                                const float *__restrict__ W, int64_t ldw,
+                                                                float *__restrict__ dX, int64_t lddx, int64_t n,
+                                                                int32_t k, int32_t fo, int32_t tiles_per_wave) {
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int j = lane & 15, q = lane >> 4;
+  const int64_t r0 = ((int64_t)blockIdx.x * kMfmaWaves + wave) * 16;
+  if (r0 >= n) return;
+  int64_t grow = r0 + j;
+  const bool row_ok = grow < n;
+  if (!row_ok) grow = n - 1;
+  float g[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    const int32_t c = 4 * s + q;
+    g[s] = c < fo ? G[grow * ldg + c] : 0.f;
+  }
+  const int32_t ktiles = (k + 15) / 16;
+  const int32_t t_begin = blockIdx.y * tiles_per_wave;
+  const int32_t t_end = t_begin + tiles_per_wave < ktiles ? t_begin + tiles_per_wave : ktiles;
+  const bool st4 = (lddx % 4 == 0) && (((uintptr_t)dX) % 16 == 0);
+  const bool st2 = (lddx % 2 == 0) && (((uintptr_t)dX) % 8 == 0);
+  for (int32_t t = t_begin; t < t_end; ++t) {
+    const int32_t kt = t * 16;
+    const int32_t wr = kt + j < k ? kt + j : k - 1;  // A side: lane (m = j, q) reads W[kt + m][4 s + q]
+    floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const int32_t c = 4 * s + q;
+      const float w = c < fo ? W[(int64_t)wr * ldw + c] : 0.f;
+      acc = mfma16(w, g[s], acc);
+    }
+    if (row_ok) {
+      const int32_t c0 = kt + 4 * q;
+      float *dst = dX + (r0 + j) * lddx + c0;
+      if (c0 + 4 <= k && st4) {
+        *reinterpret_cast<float4 *>(dst) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+      } else if (c0 + 4 <= k && st2) {
+        *reinterpret_cast<float2 *>(dst) = make_float2(acc[0], acc[1]);
+        *reinterpret_cast<float2 *>(dst + 2) = make_float2(acc[2], acc[3]);
+      } else {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          if (c0 + v < k) dst[v] = acc[v];
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------------
+static int pick_kvec(const float *X, int64_t ldx, int32_t k) {
+  if (ldx % 4 == 0 && ((uintptr_t)X) % 16 == 0 && k >= 4) return 4;
+  if (ldx % 2 == 0 && ((uintptr_t)X) % 8 == 0 && k >= 2) return 2;
+  return 1;
+}
+
+int xw_mfma(const float *X, int64_t ldx, const float *W, int64_t ldw, float *Z, int64_t ldz, int64_t n, int32_t k,
+            int32_t fo, int relu, hipStream_t stream) {
+  const int nt = (fo + 15) / 16;
+  const int vec = pick_kvec(X, ldx, k);
+  const int64_t blocks = ceil_div64(n, 16 * kMfmaWaves);
+  if (blocks > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "cg_dense_xw: grid too large");
+  const unsigned grid = (unsigned)blocks;
+#define CG_CASE(V, T)                                                                                         \
+  if (vec == V && nt == T) {                                                                                  \
+    xw_mfma_kernel<V, T><<<grid, kMfmaThreads, 0, stream>>>(X, ldx, W, ldw, Z, ldz, n, k, fo, relu);          \
+    CG_LAUNCH_CHECK();                                                                                        \
+    return CG_OK;                                                                                             \
+  }
+#define CG_CASES(V) CG_CASE(V, 1) CG_CASE(V, 2) CG_CASE(V, 3) CG_CASE(V, 4)
+  CG_CASES(1) CG_CASES(2) CG_CASES(4)
+#undef CG_CASES
+#undef CG_CASE
+  CG_FAIL(CG_ERR_UNSUPPORTED, "cg_dense_xw: fo=%d has no matrix-core variant", fo);
+}
+
+int xtg_mfma(const float *X, int64_t ldx, const float *G, int64_t ldg, float *P, int64_t n, int32_t k, int32_t fo,
+             int64_t rows_per_block, int64_t nblocks, hipStream_t stream) {
+  const int nt = (fo + 15) / 16;
+  const int vec = pick_kvec(X, ldx, k);
+  const int64_t ywaves = ceil_div64(k, 16 * vec);
+  dim3 grid((unsigned)nblocks, (unsigned)ceil_div64(ywaves, kMfmaWaves));
+#define CG_CASE(V, T)                                                                                         \
+  if (vec == V && nt == T) {                                                                                  \
+    xtg_mfma_kernel<V, T><<<grid, kMfmaThreads, 0, stream>>>(X, ldx, G, ldg, P, n, k, fo, rows_per_block);    \
+    CG_LAUNCH_CHECK();                                                                                        \
+    return CG_OK;                                                                                             \
+  }
+#define CG_CASES(V) CG_CASE(V, 1) CG_CASE(V, 2) CG_CASE(V, 3) CG_CASE(V, 4)
+  CG_CASES(1) CG_CASES(2) CG_CASES(4)
+#undef CG_CASES
+#undef CG_CASE
+  CG_FAIL(CG_ERR_UNSUPPORTED, "cg_dense_xtg: fo=%d has no matrix-core variant", fo);
+}
+
+int gwt_mfma(const float *G, int64_t ldg, const float *W, int64_t ldw, float *dX, int64_t lddx, int64_t n, int32_t k,
+             int32_t fo, hipStream_t stream) {
+  const int ks = (fo + 3) / 4;
+  const int64_t xblocks = ceil_div64(n, 16 * kMfmaWaves);
+  if (xblocks > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "cg_dense_gwt: grid too large");
+  // few vertex tiles (small n): split the output columns over grid.y to fill the chip
+  const int32_t ktiles = (k + 15) / 16;
+  int32_t ysplit = 1;
+  if (xblocks < 1024) ysplit = (int32_t)(ceil_div64(1024, xblocks) < ktiles ? ceil_div64(1024, xblocks) : ktiles);
+  const int32_t tiles_per_wave = (ktiles + ysplit - 1) / ysplit;
+  dim3 grid((unsigned)xblocks, (unsigned)((ktiles + tiles_per_wave - 1) / tiles_per_wave));
+#define CG_CASE(S)                                                                                            \
+  if (ks <= S) {                                                                                              \
+    gwt_mfma_kernel<S><<<grid, kMfmaThreads, 0, stream>>>(G, ldg, W, ldw, dX, lddx, n, k, fo, tiles_per_wave); \
+    CG_LAUNCH_CHECK();                                                                                        \
+    return CG_OK;                                                                                             \
+  }
+  CG_CASE(2) CG_CASE(4) CG_CASE(8) CG_CASE(16)
+#undef CG_CASE
+  CG_FAIL(CG_ERR_UNSUPPORTED, "cg_dense_gwt: fo=%d has no matrix-core variant", fo);
+}
+
+}  // namespace cg

@@ -1533,6 +1533,10 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
 
 }  // namespace cg
 
+namespace cg {
+extern std::atomic<int> g_tune_dense_mfma;  // dense.hip
+}
+
 struct cg_csr {
   int device = 0;
   int32_t n = 0, m = 0;
@@ -1690,6 +1694,7 @@ int cg_tune_set(const char *key, int value) {
   else if (!strcmp(key, "spmm_vec")) cg::g_tune_vec.store(value);
   else if (!strcmp(key, "spmm_hub")) cg::g_tune_hub.store(value);
   else if (!strcmp(key, "spmm_stream")) cg::g_tune_stream.store(value);
+  else if (!strcmp(key, "dense_mfma")) cg::g_tune_dense_mfma.store(value);
   else if (!strcmp(key, "spmm_win")) cg::g_tune_win.store(value);
   else if (!strcmp(key, "spmm_hub_kb")) cg::g_tune_hub_kb.store(value);
   else if (!strcmp(key, "spmm_hub_groups")) cg::g_tune_hub_groups.store(value);

@@ -26,6 +26,12 @@ from .ops import CsrMatrix
 # the reference keeps these as module globals set from the command line (gcn_distr.py:57-58, :826-827)
 activations = True
 
+# Product order of a layer.  True (default) is the reference's: the SpMM runs first, at the input
+# width, Z = (A H) W (gcn_distr.py:271, :275).  False is an opt-in reordering, Z = A (H W): the
+# same mathematics with the SpMM at the output width (602 -> 16 for the first layer), different
+# rounding; backward is unchanged because it already multiplies A by the output-width gradient.
+spmm_first = True
+
 
 class ResidentBlocks:
     """Stands where the reference passes a process group: the dense blocks that its broadcasts
@@ -97,9 +103,14 @@ class GCNFunc(torch.autograd.Function):
         kind = _kind(func) if activations else "none"
         node_count = adj_matrix if isinstance(adj_matrix, int) else adj_matrix.size(0)
         peers_fwd = group.forward if isinstance(group, ResidentBlocks) else None
-        z = broad_func(node_count, am_partitions, inputs, rank, size, peers_fwd)
-        out = ops.dense_xw(z, weight, relu=(kind == "relu"))
-        del z
+        if spmm_first or size != 1:
+            z = broad_func(node_count, am_partitions, inputs, rank, size, peers_fwd)
+            out = ops.dense_xw(z, weight, relu=(kind == "relu"))
+            del z
+        else:
+            out = broad_func(node_count, am_partitions, ops.dense_xw(inputs, weight), rank, size, peers_fwd)
+            if kind == "relu":
+                out = ops.relu_fwd(out)
         if kind == "log_softmax":
             out = ops.log_softmax_fwd(out)
         ctx.save_for_backward(inputs, weight, out)

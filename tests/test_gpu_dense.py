@@ -106,3 +106,20 @@ def test_nll_loss_forward_backward(cuda, n, c, frac):
         zr = z.double().requires_grad_(True)
         (F.nll_loss(F.log_softmax(zr, dim=1)[sel], y[sel]) * 0.5).backward()
         assert float((fused.cpu().double() - zr.grad).abs().max()) <= 1e-6
+
+
+def test_dense_vector_fallback_path(cuda):
+    """The LDS-tiled vector kernel stays in the library for widths the matrix-core kernels do not
+    cover (fo > 64); forcing it for a covered shape must give the same products."""
+    from cagnet_amd import ops
+    from cagnet_amd._lib import lib
+    X, W, G = _rand((777, 300), 1), _rand((300, 24), 2), _rand((777, 24), 3)
+    try:
+        assert lib.cg_tune_set(b"dense_mfma", -1) == 0
+        assert gemm_error(ops.dense_xw(X.to(cuda), W.to(cuda)), X, W) <= REL_TOL
+        assert gemm_error(ops.dense_gwt(G.to(cuda), W.to(cuda)), G, W.t()) <= REL_TOL
+        assert gemm_error(ops.dense_xtg(X.to(cuda), G.to(cuda)), X.t(), G) <= REL_TOL
+    finally:
+        lib.cg_tune_set(b"dense_mfma", 0)
+    Wide = _rand((300, 100), 4)
+    assert gemm_error(ops.dense_xw(X.to(cuda), Wide.to(cuda)), X, Wide) <= REL_TOL   # fo = 100 > 64

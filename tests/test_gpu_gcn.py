@@ -120,3 +120,28 @@ def test_one_rank_share_of_2d_grid(cuda):
     _close(w1.grad, ref["dw1"], "dw1")
     _close(w2.grad, ref["dw2"], "dw2")
     _close(x.grad, ref["dx"], "dx")
+
+
+def test_reordered_forward_matches_reference_order(cuda):
+    """Opt-in product order Z = A (H W): same outputs and gradients as (A H) W up to rounding."""
+    from cagnet_amd import gcn
+    p = synth.make_problem(scale=10, n_edges=9000, features=96, hidden=16, classes=6, mask_fraction=0.7, seed=8)
+    A = orc.coo_tensor(p.row, p.col, p.val, p.n, p.n, torch.float64)
+    ref = orc.forward_backward(p.x, p.w1, p.w2, [A], p.y, p.train_mask, dtype=torch.float64)
+    blk = _block(p, cuda, True)
+    try:
+        gcn.spmm_first = False
+        x = p.x.to(cuda).requires_grad_(True)
+        w1 = p.w1.to(cuda).requires_grad_(True)
+        w2 = p.w2.to(cuda).requires_grad_(True)
+        h = gcn.GCNFunc.apply(x, w1, p.n, [blk], 0, 1, None, F.relu)
+        out = gcn.GCNFunc.apply(h, w2, p.n, [blk], 0, 1, None, F.log_softmax)
+        loss = gcn.masked_nll_loss(out, p.y.to(cuda), p.train_mask.to(cuda))
+        loss.backward()
+    finally:
+        gcn.spmm_first = True
+    assert abs(float(loss.detach()) - float(ref["loss"])) <= LOSS_TOL
+    _close(out, ref["outputs"], "outputs")
+    _close(w1.grad, ref["dw1"], "dw1")
+    _close(w2.grad, ref["dw2"], "dw2")
+    _close(x.grad, ref["dx"], "dx")
