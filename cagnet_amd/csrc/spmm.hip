@@ -550,7 +550,7 @@ struct StreamTab {
   bool hub = false;
   int32_t *task_start = nullptr, *task_dst = nullptr, *wstart = nullptr;
   int64_t nwin = 0;
-  int64_t win_first[9] = {0};
+  int64_t win_first[18] = {0};
   void release() {
     if (task_start) (void)hipFree(task_start);
     if (task_dst) (void)hipFree(task_dst);
@@ -641,7 +641,7 @@ static int build_stream(const Sched &sc, const int32_t *rowptr, int32_t nrows, b
   CG_TRY(tmp.alloc((void **)&flags, (size_t)(nt + 1) * 4));
   CG_TRY(tmp.alloc((void **)&index, (size_t)(nt + 1) * 4));
   // entry extents of the classes (host needs them to size the boundary launches)
-  int32_t ends[10];
+  int32_t ends[18];
   for (int g = 0; g <= nclass; ++g)
     CG_HIP(hipMemcpyAsync(&ends[g], out.task_start + class_first[g], 4, hipMemcpyDeviceToHost, stream));
   CG_HIP(hipStreamSynchronize(stream));
@@ -662,7 +662,7 @@ static int build_stream(const Sched &sc, const int32_t *rowptr, int32_t nrows, b
   CG_TRY(exclusive_scan_u32(flags, index, nt, (uint32_t *)d_total_v, stream));
   uint32_t nwin = 0;
   CG_HIP(hipMemcpyAsync(&nwin, d_total_v, 4, hipMemcpyDeviceToHost, stream));
-  uint32_t firsts[10] = {0};
+  uint32_t firsts[18] = {0};
   for (int g = 0; g < nclass; ++g)
     if (class_first[g] < nt) CG_HIP(hipMemcpyAsync(&firsts[g], index + class_first[g], 4, hipMemcpyDeviceToHost, stream));
   CG_HIP(hipStreamSynchronize(stream));
@@ -1087,18 +1087,22 @@ struct SchedCache {
   }
 };
 
-// Hub plan: the stored entries regrouped by column class.  The `hot` most referenced columns
-// (= rows of B) are dealt round robin, by descending reference count, to `groups` groups; every
-// other column is cold.  Entries are kept as one CSR over (groups + 1) * rows virtual rows, virtual
-// row c * rows + r holding the entries of row r whose column has class c (cold = class `groups`).
+// Hub plan: the stored entries regrouped by column class.  Columns (= rows of B) are ranked by
+// descending reference count; the first `hot` ranks form tier 0, the next `hot` tier 1, ...; inside
+// a tier the columns are dealt round robin to `groups` groups, and every column behind the last
+// tier is cold.  Class = tier * groups + group.  A tier is one launch in which XCD x only reads the
+// B rows of group x % groups, sized to stay resident in that XCD's L2.  Entries are kept as one CSR
+// over (classes + 1) * rows virtual rows, virtual row c * rows + r holding the entries of row r whose
+// column has class c (cold = class `classes`).
 struct HubPlan {
-  int32_t hot = 0, groups = 0, seg = 0;
+  int32_t hot = 0, groups = 0, tiers = 0, seg = 0;
+  int32_t classes() const { return groups * tiers; }
   int32_t *vrowptr = nullptr, *colind = nullptr;
   float *val = nullptr;
   Sched hot_sched;        // over the virtual rows of the hot classes, empty rows skipped
   StreamTab hot_tab;      // its windows, one class per group
   SchedCache cold_sched;  // over the cold class
-  int64_t tstart[9] = {0};
+  int64_t tstart[18] = {0};
   bool valid = false;
   void release() {
     hot_sched.release();
@@ -1164,12 +1168,14 @@ __global__ __launch_bounds__(kSpmmThreads) void col_key_kernel(const uint32_t *_
   }
 }
 
-// class of every column from its rank: the first `hot` ranks go round robin to the groups
+// class of every column from its rank: `hot` ranks per tier, dealt round robin to the groups
 __global__ __launch_bounds__(kSpmmThreads) void col_class_kernel(const int32_t *__restrict__ ranked_col, int32_t m,
-                                                                 int32_t hot, int32_t groups,
+                                                                 int32_t hot, int32_t groups, int32_t tiers,
                                                                  int32_t *__restrict__ cls) {
   const int64_t rank = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
-  if (rank < m) cls[ranked_col[rank]] = rank < hot ? (int32_t)(rank % groups) : groups;
+  if (rank >= m) return;
+  const int64_t tier = rank / hot;
+  cls[ranked_col[rank]] = tier < tiers ? (int32_t)(tier * groups + (rank % hot) % groups) : groups * tiers;
 }
 
 __global__ __launch_bounds__(kSpmmThreads) void entry_class_kernel(const int32_t *__restrict__ colind, int64_t nnz,
@@ -1210,15 +1216,16 @@ __global__ __launch_bounds__(kSpmmThreads) void csr_rows_kernel(const int32_t *_
   for (int32_t k = s + lane; k < e; k += kWave) row_out[k] = (int32_t)wave;
 }
 
-static int build_hub(CsrSide &s, int32_t hot, int32_t groups, int32_t seg, hipStream_t stream) {
+static int build_hub(CsrSide &s, int32_t hot, int32_t groups, int32_t tiers, int32_t seg, hipStream_t stream) {
   HubPlan &h = s.hub;
   CG_HIP(hipStreamSynchronize(stream));
   h.release();
   const int64_t nnz = s.nnz;
   const int32_t n = s.rows, m = s.cols;
-  const int64_t vrows = (int64_t)(groups + 1) * n;
+  const int32_t nclass = groups * tiers;
+  const int64_t vrows = (int64_t)(nclass + 1) * n;
+  if (hot < 1) hot = 1;
   if (vrows + 1 > 0x7fffffffLL) CG_FAIL(CG_ERR_OVERFLOW, "hub plan: %lld virtual rows exceed int32", (long long)vrows);
-  if (hot > m) hot = m;
   TempFree tmp;
   const unsigned gm = (unsigned)ceil_div64(m, kSpmmThreads), ge = (unsigned)ceil_div64(nnz, kSpmmThreads);
 
@@ -1245,7 +1252,7 @@ static int build_hub(CsrSide &s, int32_t hot, int32_t groups, int32_t seg, hipSt
     int set = 0;
     CG_TRY(radix_sort_pairs(buf, m, bits_for((int32_t)(maxcount < 0x7ffffffeu ? maxcount + 1 : 0x7fffffff)), 0, &set,
                             stream));
-    col_class_kernel<<<gm, kSpmmThreads, 0, stream>>>(buf.payload[set], m, hot, groups, cls);
+    col_class_kernel<<<gm, kSpmmThreads, 0, stream>>>(buf.payload[set], m, hot, groups, tiers, cls);
     CG_LAUNCH_CHECK();
   }
 
@@ -1273,7 +1280,7 @@ static int build_hub(CsrSide &s, int32_t hot, int32_t groups, int32_t seg, hipSt
     hub_iota_kernel<<<ge, kSpmmThreads, 0, stream>>>(buf.payload[0], nnz);  // position in the original CSR
     CG_LAUNCH_CHECK();
     int set = 0;
-    CG_TRY(radix_sort_pairs(buf, nnz, bits_for(groups + 1), 0, &set, stream));
+    CG_TRY(radix_sort_pairs(buf, nnz, bits_for(nclass + 1), 0, &set, stream));
     entry_finish_kernel<<<ge, kSpmmThreads, 0, stream>>>(buf.key_a[set], buf.key_b[set], buf.payload[set], nnz, n,
                                                          s.colind, s.val, vrow, h.colind, h.val);
     CG_LAUNCH_CHECK();
@@ -1282,16 +1289,17 @@ static int build_hub(CsrSide &s, int32_t hot, int32_t groups, int32_t seg, hipSt
   CG_TRY(launch_rowptr(vrow, nnz, (int32_t)vrows, h.vrowptr, stream));
 
   // 3. tasks of the hot classes (empty virtual rows get none); the cold class is scheduled on demand
-  CG_TRY(make_sched(h.vrowptr, groups * n, seg, 1, h.hot_sched, stream));
+  CG_TRY(make_sched(h.vrowptr, nclass * n, seg, 1, h.hot_sched, stream));
   {
-    int32_t t[9];
-    for (int g = 0; g <= groups; ++g)
+    int32_t t[18];
+    for (int g = 0; g <= nclass; ++g)
       CG_HIP(hipMemcpyAsync(&t[g], h.hot_sched.tbase + (int64_t)g * n, 4, hipMemcpyDeviceToHost, stream));
     CG_HIP(hipStreamSynchronize(stream));
-    for (int g = 0; g <= groups; ++g) h.tstart[g] = t[g];
+    for (int g = 0; g <= nclass; ++g) h.tstart[g] = t[g];
   }
   h.hot = hot;
   h.groups = groups;
+  h.tiers = tiers;
   h.seg = seg;
   h.valid = true;
   return CG_OK;
@@ -1300,22 +1308,23 @@ static int build_hub(CsrSide &s, int32_t hot, int32_t groups, int32_t seg, hipSt
 // C[r, :] += sum of the partial rows of r's hot tasks, in (group, segment) order.  One wavefront
 // per row: lane g fetches the task range of group g, then the lanes sweep the row's columns with
 // the partial rows of all tasks in flight together.
+template <int NC>  // classes the unrolled loops cover (nclass <= NC)
 __global__ __launch_bounds__(kSpmmThreads) void hub_reduce_kernel(const int32_t *__restrict__ tbase, int32_t n,
-                                                                  int32_t groups, const float *__restrict__ P,
+                                                                  int32_t nclass, const float *__restrict__ P,
                                                                   float *__restrict__ C, int64_t ldc, int32_t f) {
   const int64_t r = ((int64_t)blockIdx.x * kSpmmThreads + threadIdx.x) / kWave;
   const int lane = threadIdx.x & (kWave - 1);
   if (r >= n) return;
   int32_t t0 = 0, t1 = 0;
-  if (lane < groups) {
+  if (lane < nclass) {
     const int64_t v = (int64_t)lane * n + r;
     t0 = tbase[v];
     t1 = tbase[v + 1];
   }
-  int32_t first[8], count[8];
+  int32_t first[NC], count[NC];
   int32_t total = 0;
 #pragma unroll
-  for (int g = 0; g < 8; ++g) {
+  for (int g = 0; g < NC; ++g) {
     first[g] = __builtin_amdgcn_readlane(t0, g);
     count[g] = __builtin_amdgcn_readlane(t1, g) - first[g];
     total += count[g];
@@ -1327,7 +1336,7 @@ __global__ __launch_bounds__(kSpmmThreads) void hub_reduce_kernel(const int32_t 
     if (col < f) {
       float s = 0.f;
 #pragma unroll
-      for (int g = 0; g < 8; ++g) {
+      for (int g = 0; g < NC; ++g) {
         const float *p = P + (int64_t)first[g] * f + col;
         if (count[g] == 1) {
           s += p[0];
@@ -1340,7 +1349,7 @@ __global__ __launch_bounds__(kSpmmThreads) void hub_reduce_kernel(const int32_t 
   }
 }
 
-std::atomic<int> g_tune_hub{0}, g_tune_hub_kb{0}, g_tune_hub_groups{0};
+std::atomic<int> g_tune_hub{0}, g_tune_hub_kb{0}, g_tune_hub_groups{0}, g_tune_hub_tiers{0};
 
 // stored entries after which a new window starts
 static int32_t window_entries() {
@@ -1449,69 +1458,82 @@ static int spmm_hub(CsrSide &s, int vec, const float *B, int64_t ldb, float *C, 
                     hipStream_t stream) {
   int groups = g_tune_hub_groups.load(std::memory_order_relaxed);
   if (groups != 1 && groups != 2 && groups != 4 && groups != 8) groups = 8;
+  int tiers = g_tune_hub_tiers.load(std::memory_order_relaxed);
+  if (tiers < 1 || tiers * groups > 16) tiers = 1;
   int kb = g_tune_hub_kb.load(std::memory_order_relaxed);
-  if (kb <= 0) kb = 8192;  // twice the 4 MB L2 of an XCD: measured optimum, LRU keeps the hottest half
+  // one tier: twice the 4 MB L2 of an XCD is the measured optimum (LRU keeps the hottest half);
+  // several tiers: each is sized to stay resident
+  if (kb <= 0) kb = tiers == 1 ? 8192 : 3584;
   int64_t per_group = (int64_t)kb * 1024 / ((int64_t)f * 4);
   if (per_group < 1) per_group = 1;
-  int64_t hot = per_group * groups;
+  int64_t hot = per_group * groups;  // columns per tier
   if (hot > s.cols) hot = s.cols;
-  // hot tasks always use full-wave teams on the whole width, one dword per lane and chunk: that is
-  // the fastest gather of L2-resident rows whose start is not 16-byte aligned
+  // hot tasks use full-wave teams on the whole width with one dword per lane and chunk when the rows
+  // are not 16-byte aligned: that is the fastest gather of L2-resident rows
   const int hot_vec = (vec == 4 || f / vec <= kWave) ? vec : 1;
   SpmmPlan hplan;
   hplan.tiles = 1;
   hplan.tile_slots = f / hot_vec;
   hplan.shape = pick_shape(hot_vec, hplan.tile_slots);
   const int32_t seg = pick_seg(hplan.shape);
-  if (!s.hub.valid || s.hub.hot != (int32_t)hot || s.hub.groups != groups || s.hub.seg != seg)
-    CG_TRY(build_hub(s, (int32_t)hot, groups, seg, stream));
+  if (!s.hub.valid || s.hub.hot != (int32_t)hot || s.hub.groups != groups || s.hub.tiers != tiers || s.hub.seg != seg)
+    CG_TRY(build_hub(s, (int32_t)hot, groups, tiers, seg, stream));
   HubPlan &h = s.hub;
   const int32_t n = s.rows;
+  const int32_t nclass = h.classes();
   // 1. cold class straight into C
-  CG_TRY(spmm_plain(h.vrowptr + (int64_t)groups * n, h.colind, h.val, n, s.cols, h.cold_sched, vec, B, ldb, C, ldc, f,
+  CG_TRY(spmm_plain(h.vrowptr + (int64_t)nclass * n, h.colind, h.val, n, s.cols, h.cold_sched, vec, B, ldb, C, ldc, f,
                     beta, f, stream));
-  // 2. hot classes: every task writes a partial row
+  // 2. hot classes, one launch per tier: every task writes a partial row
   const int64_t hot_tasks = h.hot_sched.ntasks;
   if (hot_tasks == 0) return CG_OK;
   void *p = nullptr;
   CG_TRY(scratch_get(stream, kSlotC, (size_t)hot_tasks * f * sizeof(float), &p));
-  SpmmArgs a{};
-  fill_args(a, h.vrowptr, h.colind, h.val, &h.hot_sched, s.cols, B, ldb, C, ldc, f, 0.f, hplan);
-  a.P = (float *)p;
-  a.groups = groups;
-  for (int g = 0; g <= groups; ++g) a.tstart[g] = h.tstart[g];
   const bool hnarrow = hplan.shape.lpr < kWave;
-  if (g_tune_stream.load(std::memory_order_relaxed) >= 0 && (!hnarrow || (seg <= 512 && window_entries() <= 512))) {
+  const bool streaming =
+      g_tune_stream.load(std::memory_order_relaxed) >= 0 && (!hnarrow || (seg <= 512 && window_entries() <= 512));
+  if (streaming) {
     const int32_t S = window_entries();
-    if (h.hot_tab.S != S || h.hot_tab.groups != groups)
-      CG_TRY(build_stream(h.hot_sched, h.vrowptr, groups * n, true, groups, h.tstart, S, h.hot_tab, stream));
-    StreamArgs sa{};
-    sa.task_start = h.hot_tab.task_start;
-    sa.task_dst = h.hot_tab.task_dst;
-    sa.wstart = h.hot_tab.wstart;
-    sa.colind = h.colind;
-    sa.val = h.val;
-    for (int g = 0; g <= groups; ++g) sa.win_first[g] = h.hot_tab.win_first[g];
-    sa.groups = groups;
-    sa.B = B;
-    sa.ldb = ldb;
-    sa.C = C;
-    sa.ldc = ldc;
-    sa.P = (float *)p;
-    sa.f = f;
-    sa.beta = 0.f;
+    if (h.hot_tab.S != S || h.hot_tab.groups != nclass)
+      CG_TRY(build_stream(h.hot_sched, h.vrowptr, nclass * n, true, nclass, h.tstart, S, h.hot_tab, stream));
+  }
+  for (int t = 0; t < tiers; ++t) {
     ProfScope prof("spmm_hub_hot", f, stream);
-    if (hnarrow) CG_TRY(launch_stream_narrow(hot_vec, hplan.shape.lpr, sa, stream));
-    else CG_TRY(launch_stream_wide(hot_vec, hplan.shape.chunks, sa, stream));
-  } else {
-    ProfScope prof("spmm_hub_hot", f, stream);
-    CG_TRY((launch_shape<kModeHub>(hplan.shape, a, stream)));
+    if (streaming) {
+      StreamArgs sa{};
+      sa.task_start = h.hot_tab.task_start;
+      sa.task_dst = h.hot_tab.task_dst;
+      sa.wstart = h.hot_tab.wstart;
+      sa.colind = h.colind;
+      sa.val = h.val;
+      for (int g = 0; g <= groups; ++g) sa.win_first[g] = h.hot_tab.win_first[t * groups + g];
+      sa.groups = groups;
+      sa.B = B;
+      sa.ldb = ldb;
+      sa.C = C;
+      sa.ldc = ldc;
+      sa.P = (float *)p;
+      sa.f = f;
+      sa.beta = 0.f;
+      if (hnarrow) CG_TRY(launch_stream_narrow(hot_vec, hplan.shape.lpr, sa, stream));
+      else CG_TRY(launch_stream_wide(hot_vec, hplan.shape.chunks, sa, stream));
+    } else {
+      SpmmArgs a{};
+      fill_args(a, h.vrowptr, h.colind, h.val, &h.hot_sched, s.cols, B, ldb, C, ldc, f, 0.f, hplan);
+      a.P = (float *)p;
+      a.groups = groups;
+      for (int g = 0; g <= groups; ++g) a.tstart[g] = h.tstart[t * groups + g];
+      CG_TRY((launch_shape<kModeHub>(hplan.shape, a, stream)));
+    }
   }
   // 3. fold the partial rows into C
   {
     ProfScope prof("spmm_hub_reduce", f, stream);
-    hub_reduce_kernel<<<(unsigned)ceil_div64((int64_t)n * kWave, kSpmmThreads), kSpmmThreads, 0, stream>>>(
-        h.hot_sched.tbase, n, groups, a.P, C, ldc, f);
+    const unsigned rgrid = (unsigned)ceil_div64((int64_t)n * kWave, kSpmmThreads);
+    if (nclass <= 8)
+      hub_reduce_kernel<8><<<rgrid, kSpmmThreads, 0, stream>>>(h.hot_sched.tbase, n, nclass, (const float *)p, C, ldc, f);
+    else
+      hub_reduce_kernel<16><<<rgrid, kSpmmThreads, 0, stream>>>(h.hot_sched.tbase, n, nclass, (const float *)p, C, ldc, f);
     CG_LAUNCH_CHECK();
   }
   return CG_OK;
@@ -1698,6 +1720,7 @@ int cg_tune_set(const char *key, int value) {
   else if (!strcmp(key, "spmm_win")) cg::g_tune_win.store(value);
   else if (!strcmp(key, "spmm_hub_kb")) cg::g_tune_hub_kb.store(value);
   else if (!strcmp(key, "spmm_hub_groups")) cg::g_tune_hub_groups.store(value);
+  else if (!strcmp(key, "spmm_hub_tiers")) cg::g_tune_hub_tiers.store(value);
   else CG_FAIL(CG_ERR_UNSUPPORTED, "cg_tune_set: unknown key %s", key);
   return CG_OK;
 }

@@ -103,7 +103,7 @@ class GCNFunc(torch.autograd.Function):
         kind = _kind(func) if activations else "none"
         node_count = adj_matrix if isinstance(adj_matrix, int) else adj_matrix.size(0)
         peers_fwd = group.forward if isinstance(group, ResidentBlocks) else None
-        if spmm_first or size != 1:
+        if spmm_first or size != 1 or weight.shape[1] >= inputs.shape[1]:  # reordering only pays when the layer narrows
             z = broad_func(node_count, am_partitions, inputs, rank, size, peers_fwd)
             out = ops.dense_xw(z, weight, relu=(kind == "relu"))
             del z

@@ -262,9 +262,9 @@ def tune():
         lib.cg_tune_set(key.encode(), 0)
 
 
-@pytest.mark.parametrize("groups", [8, 2, 1])
+@pytest.mark.parametrize("groups,tiers", [(8, 1), (2, 1), (1, 1), (8, 2), (4, 3)])
 @pytest.mark.parametrize("f", [602, 256, 300])
-def test_spmm_hub_plan_matches_oracle(cuda, tune, f, groups):
+def test_spmm_hub_plan_matches_oracle(cuda, tune, f, groups, tiers):
     """Hub plan forced on a small power-law graph: hot columns dealt to XCD groups, cold class
     straight into C, hot partial rows folded in afterwards.  A 64 KB hot budget keeps only a few
     dozen columns hot, so all three classes of entries (hot, cold, rows without hot entries) occur."""
@@ -276,6 +276,7 @@ def test_spmm_hub_plan_matches_oracle(cuda, tune, f, groups):
     tune("spmm_hub", 1)
     tune("spmm_hub_kb", 64)
     tune("spmm_hub_groups", groups)
+    tune("spmm_hub_tiers", tiers)
     got = A.spmm(B.to(cuda))
     assert spmm_error(got, row, col, val, n, n, B) <= REL_TOL
     assert torch.equal(got, A.spmm(B.to(cuda)))                       # deterministic
