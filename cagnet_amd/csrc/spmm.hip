@@ -1,21 +1,10 @@
-// CSR SpMM  C[rows,f] = beta*C + A*B  for gfx950, and the cached handle around it.
+// Host side of the CSR SpMM: schedules, window tables, hub plans, the cached handle and the C ABI
+// entry points.  The device kernels are in spmm_kernels.h.
 //
-// Replaces cusparseSpMM(CSRMM_ALG1, alpha = 1, beta = 1) and everything the reference wraps
-// around it on every call (sparse-extension/sparse_coo_tensor.cu:136-231): B and C stay row-major,
-// nothing is transposed, and the CSR, its transpose and the schedules live in a handle.
-//
-// Work decomposition
-//   task    = a row segment: at most `seg` consecutive stored entries of one row.  One wavefront
-//             runs one task.  Rows of degree <= seg are one task and are written straight to C.
-//   team    = LPR lanes that together cover the f output columns (VEC floats per lane and chunk).
-//             A wavefront holds G = 64/LPR teams; team g takes entries g, g+G, ... of the task and
-//             the teams' partial rows are combined with a fixed xor butterfly (no atomics).
-//   split rows (degree > seg) write one partial row per task to a workspace; a second kernel adds
-//             a row's partials in segment order.  Summation order is a function of the matrix,
-//             f and seg only, so results are bit-identical from run to run.
-// (col, val) of 64 entries are fetched with one coalesced load per array and handed to the teams
-// with lane reads (readlane for G == 1, where the column index becomes a scalar base address).
-#include "common.h"
+// Replaces everything the reference wraps around cusparseSpMM on every call
+// (sparse-extension/sparse_coo_tensor.cu:136-231): B and C stay row-major, nothing is transposed,
+// and the CSR, its transpose, the schedules and the hub plan live in a handle.
+#include "spmm_kernels.h"
 #include <stdlib.h>
 #include <string.h>
 #include <atomic>
@@ -23,290 +12,20 @@
 
 namespace cg {
 
-constexpr int kSpmmThreads = 256;
-constexpr int kWavesPerBlock = kSpmmThreads / kWave;
+extern std::atomic<int> g_tune_dense_mfma;  // dense.hip
 
-struct SpmmArgs {
-  const int32_t *rowptr;
-  const int32_t *colind;
-  const float *val;
-  const int32_t *task_row;  // TABLE only
-  const int32_t *tbase;     // TABLE only: first task of each row
-  const int32_t *pbase;     // TABLE only: first partial slot of each split row
-  int64_t ntasks;
-  int32_t seg;
-  int32_t m;                // number of columns of A (rows of B), for CLAMP
-  const float *B;
-  int64_t ldb;
-  float *C;
-  int64_t ldc;
-  float *P;                 // partial rows of split rows, row stride f
-  int32_t f;
-  float beta;
-  int32_t tiles;            // feature tiles (1, 2, 4 or 8); tile t is run by XCDs x with x % tiles == t
-  int32_t tile_slots;       // VEC-wide slots per tile (the last tile may hold fewer)
-  int32_t groups;           // kModeHub: hot column groups (1, 2, 4 or 8); group g runs on XCDs x % groups == g
-  int64_t tstart[9];        // kModeHub: tasks of group g are [tstart[g], tstart[g+1])
-};
-
-// kModeRows: one task per row, no tables, column indices clamped (one-shot entry point)
-// kModeTable: tasks from the schedule tables of a handle
-// kModeHub:  tasks of the hot column groups of a hub plan, pinned to XCDs; every task writes a partial row
-enum { kModeRows = 0, kModeTable = 1, kModeHub = 2 };
-
-template <int VEC>
-struct VecT;
-template <>
-struct VecT<1> {
-  typedef float type;
-};
-template <>
-struct VecT<2> {
-  typedef float2 type;
-};
-template <>
-struct VecT<4> {
-  typedef float4 type;
-};
-
-template <int VEC>
-__device__ __forceinline__ void load_vec(const float *p, float (&r)[VEC]) {
-  typedef typename VecT<VEC>::type V;
-  const V t = *reinterpret_cast<const V *>(p);
-  const float *tp = reinterpret_cast<const float *>(&t);
-#pragma unroll
-  for (int i = 0; i < VEC; ++i) r[i] = tp[i];
-}
-
-template <int VEC>
-__device__ __forceinline__ void store_vec(float *p, const float (&r)[VEC]) {
-  typedef typename VecT<VEC>::type V;
-  V t;
-  float *tp = reinterpret_cast<float *>(&t);
-#pragma unroll
-  for (int i = 0; i < VEC; ++i) tp[i] = r[i];
-  *reinterpret_cast<V *>(p) = t;
-}
-
-template <int VEC, int LPR, int CHUNKS, int MODE>
-__global__ __launch_bounds__(kSpmmThreads) void spmm_rowseg_kernel(const SpmmArgs a) {
-  static_assert(LPR == 64 || CHUNKS == 1, "several chunks only with a full-wave team");
-  constexpr int G = kWave / LPR;
-  constexpr bool TABLE = MODE != kModeRows;
-  constexpr bool CLAMP = MODE == kModeRows;
-  constexpr bool HUB = MODE == kModeHub;
-  const int lane = threadIdx.x & (kWave - 1);
-  // Workgroups are dealt to the 8 XCDs round robin (workgroup w runs on XCD w % 8), and every XCD
-  // has its own L2.  With T feature tiles, XCD x only ever touches tile x % T of B, so its L2 holds
-  // a T times narrower slice of B's hot rows: the 8 L2s cache different data instead of 8 copies.
-  int tile = 0;
-  int64_t tb = blockIdx.x;
-  int64_t task_lo = 0, task_hi = a.ntasks;
-  if (HUB) {
-    // Hot columns are dealt to `groups` groups; group g's rows of B are only ever read by the XCDs
-    // x with x % groups == g, so each L2 keeps its own share of the hot rows resident.
-    const int x = blockIdx.x & 7;
-    const int per = 8 / a.groups;
-    const int grp = x % a.groups;
-    tb = (int64_t)(blockIdx.x >> 3) * per + x / a.groups;
-    task_lo = a.tstart[grp];
-    task_hi = a.tstart[grp + 1];
-  } else if (a.tiles > 1) {
-    const int x = blockIdx.x & 7;
-    const int per = 8 / a.tiles;  // XCDs that share a tile
-    tile = x % a.tiles;
-    tb = (int64_t)(blockIdx.x >> 3) * per + x / a.tiles;
-  }
-  const int64_t task =
-      __builtin_amdgcn_readfirstlane((int)(task_lo + tb * kWavesPerBlock + threadIdx.x / kWave));
-  if (task >= task_hi) return;
-
-  int32_t row, sidx, rs, re;
-  if (TABLE) {
-    row = a.task_row[task];
-    sidx = (int32_t)task - a.tbase[row];
-  } else {
-    row = (int32_t)task;
-    sidx = 0;
-  }
-  rs = a.rowptr[row];
-  re = a.rowptr[row + 1];
-  const int32_t start = TABLE ? rs + sidx * a.seg : rs;
-  const int32_t end = TABLE ? (start + a.seg < re ? start + a.seg : re) : re;
-  const bool single = HUB ? false : (TABLE ? (re - rs <= a.seg) : true);
-  if (single && start >= end && a.beta == 1.0f) return;  // empty row, C unchanged
-
-  const int g = lane / LPR;   // team
-  const int j = lane % LPR;   // position inside the team
-  const int slot0 = tile * a.tile_slots;
-  int nslots = a.f / VEC - slot0;  // slots of this tile
-  nslots = nslots < a.tile_slots ? nslots : a.tile_slots;
-  if (nslots <= 0) return;
-  bool active[CHUNKS];
-  int64_t boff[CHUNKS];  // lane's column offset per chunk; idle lanes re-read the chunk's first slot
-#pragma unroll
-  for (int ch = 0; ch < CHUNKS; ++ch) {
-    active[ch] = (ch * LPR + j) < nslots;
-    boff[ch] = (int64_t)(slot0 + ch * LPR + (active[ch] ? j : 0)) * VEC;
-  }
-
-  float acc[CHUNKS][VEC];
-#pragma unroll
-  for (int ch = 0; ch < CHUNKS; ++ch)
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) acc[ch][v] = 0.f;
-
-  constexpr int U = 4;  // entries per team in flight
-
-  // software pipeline: the next 64 (col, val) are in flight while the current 64 are consumed
-  int32_t c_next = 0;
-  float v_next = 0.f;
-  if (start + lane < end) {
-    c_next = a.colind[start + lane];
-    v_next = a.val[start + lane];
-  }
-  for (int32_t base = start; base < end; base += kWave) {
-    int32_t c = c_next;
-    const float v = v_next;
-    const int32_t nb = base + kWave + lane;
-    c_next = 0;
-    v_next = 0.f;
-    if (nb < end) {
-      c_next = a.colind[nb];
-      v_next = a.val[nb];
-    }
-    if (CLAMP) c = c < 0 ? 0 : (c >= a.m ? a.m - 1 : c);
-    const int cnt = (end - base) < kWave ? (end - base) : kWave;  // wave uniform
-
-    if (G == 1) {
-      int i = 0;
-      for (; i + U <= cnt; i += U) {
-        float b[U][CHUNKS][VEC];
-        float vv[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const int32_t cc = __builtin_amdgcn_readlane(c, i + u);
-          vv[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), i + u));
-          const float *brow = a.B + (int64_t)cc * a.ldb;
-#pragma unroll
-          for (int ch = 0; ch < CHUNKS; ++ch) load_vec<VEC>(brow + boff[ch], b[u][ch]);
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-          for (int ch = 0; ch < CHUNKS; ++ch)
-#pragma unroll
-            for (int x = 0; x < VEC; ++x) acc[ch][x] = fmaf(vv[u], b[u][ch][x], acc[ch][x]);
-      }
-      for (; i < cnt; ++i) {
-        const int32_t cc = __builtin_amdgcn_readlane(c, i);
-        const float vv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), i));
-        const float *brow = a.B + (int64_t)cc * a.ldb;
-        float b[CHUNKS][VEC];
-#pragma unroll
-        for (int ch = 0; ch < CHUNKS; ++ch) load_vec<VEC>(brow + boff[ch], b[ch]);
-#pragma unroll
-        for (int ch = 0; ch < CHUNKS; ++ch)
-#pragma unroll
-          for (int x = 0; x < VEC; ++x) acc[ch][x] = fmaf(vv, b[ch][x], acc[ch][x]);
-      }
-    } else {
-      int i = 0;
-      for (; i + U * G <= cnt; i += U * G) {
-        float b[U][VEC];
-        float vv[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const int src = i + u * G + g;
-          const int32_t cc = __shfl(c, src, kWave);
-          vv[u] = __shfl(v, src, kWave);
-          load_vec<VEC>(a.B + (int64_t)cc * a.ldb + boff[0], b[u]);
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-          for (int x = 0; x < VEC; ++x) acc[0][x] = fmaf(vv[u], b[u][x], acc[0][x]);
-      }
-      for (; i < cnt; i += G) {
-        const int src = i + g;
-        const int32_t cc = __shfl(c, src, kWave);  // lanes past cnt hold col 0, val 0
-        const float vv = __shfl(v, src, kWave);
-        if (src < cnt) {
-          float b[VEC];
-          load_vec<VEC>(a.B + (int64_t)cc * a.ldb + boff[0], b);
-#pragma unroll
-          for (int x = 0; x < VEC; ++x) acc[0][x] = fmaf(vv, b[x], acc[0][x]);
-        }
-      }
-    }
-  }
-
-  if (G > 1) {  // combine the teams: fixed butterfly, every lane ends with the full sum
-#pragma unroll
-    for (int off = LPR; off < kWave; off <<= 1) {
-#pragma unroll
-      for (int x = 0; x < VEC; ++x) acc[0][x] += __shfl_xor(acc[0][x], off, kWave);
-    }
-    if (g != 0) return;
-  }
-
-  if (single) {
-    float *crow = a.C + (int64_t)row * a.ldc;
-#pragma unroll
-    for (int ch = 0; ch < CHUNKS; ++ch) {
-      if (active[ch]) {
-        float out[VEC];
-        if (a.beta != 0.f) {
-          float old[VEC];
-          load_vec<VEC>(crow + boff[ch], old);
-#pragma unroll
-          for (int x = 0; x < VEC; ++x) out[x] = fmaf(a.beta, old[x], acc[ch][x]);
-        } else {
-#pragma unroll
-          for (int x = 0; x < VEC; ++x) out[x] = acc[ch][x];
-        }
-        store_vec<VEC>(crow + boff[ch], out);
-      }
-    }
-  } else {
-    float *prow = a.P + (HUB ? task : ((int64_t)a.pbase[row] + sidx)) * a.f;
-#pragma unroll
-    for (int ch = 0; ch < CHUNKS; ++ch)
-      if (active[ch]) store_vec<VEC>(prow + boff[ch], acc[ch]);
-  }
-}
-
-// C[row, :] = beta*C[row, :] + sum over the row's partial rows, in segment order.
-__global__ __launch_bounds__(kSpmmThreads) void spmm_reduce_kernel(const int32_t *__restrict__ multi_rows,
-                                                                   int64_t nmulti, const int32_t *__restrict__ rowptr,
-                                                                   const int32_t *__restrict__ pbase, int32_t seg,
-                                                                   const float *__restrict__ P, float *__restrict__ C,
-                                                                   int64_t ldc, int32_t f, float beta) {
-  const int64_t idx = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
-  const int64_t mr = idx / f;
-  const int32_t col = (int32_t)(idx % f);
-  if (mr >= nmulti) return;
-  const int32_t row = multi_rows[mr];
-  const int32_t deg = rowptr[row + 1] - rowptr[row];
-  const int32_t nseg = (deg + seg - 1) / seg;
-  const float *p = P + (int64_t)pbase[row] * f + col;
-  float s = 0.f;
-  for (int32_t i = 0; i < nseg; ++i) s += p[(int64_t)i * f];
-  float *c = C + (int64_t)row * ldc + col;
-  *c = beta != 0.f ? fmaf(beta, *c, s) : s;
-}
+// Tuning knobs (cg_tune_set): 0 = built-in choice.
+static std::atomic<int> g_tune_seg{0}, g_tune_vec{0}, g_tune_win{0};
+static std::atomic<int> g_tune_hub{0}, g_tune_hub_kb{0}, g_tune_hub_groups{0}, g_tune_hub_tiers{0};
 
 // ---------------------------------------------------------------------------------------------
-// kernel selection
+// kernel shape selection
 // ---------------------------------------------------------------------------------------------
 struct SpmmShape {
   int vec, lpr, chunks;
 };
 
-constexpr int kMaxChunks = 10;
-
-// Tuning knobs (cg_tune_set): 0 = built-in choice.
-std::atomic<int> g_tune_seg{0}, g_tune_tiles{0}, g_tune_vec{0}, g_tune_stream{0}, g_tune_win{0};
+constexpr int kMaxChunks = 10;  // full-wave teams cover up to 64 * kMaxChunks * VEC columns per launch
 
 // Widest vector the operands allow.
 static int pick_vec(int32_t f, const float *B, int64_t ldb, const float *C, int64_t ldc) {
@@ -318,7 +37,7 @@ static int pick_vec(int32_t f, const float *B, int64_t ldb, const float *C, int6
   return 1;
 }
 
-// Smallest team that covers `slots` vector slots (one tile's worth).
+// Smallest team that covers `slots` vector slots.
 static SpmmShape pick_shape(int vec, int slots) {
   SpmmShape s{vec, 64, 1};
   if (slots <= 64) {
@@ -331,59 +50,20 @@ static SpmmShape pick_shape(int vec, int slots) {
   return s;
 }
 
-// Feature tiles per launch.  Wide outputs are split over the XCDs so that each L2 caches its own
-// column slice of B; narrow ones (a row of B is a cache line or two) stay whole.
-static int pick_tiles(int vec, int slots) {
-  const int t = g_tune_tiles.load(std::memory_order_relaxed);
-  if (t == 1 || t == 2 || t == 4 || t == 8) return slots >= t ? t : 1;
-  (void)vec;
-  return slots >= 256 ? 8 : 1;
-}
-
-template <int MODE>
-static int launch_shape(const SpmmShape &s, const SpmmArgs &a, hipStream_t stream) {
-  int64_t blocks = ceil_div64(a.ntasks, kWavesPerBlock);
-  if (MODE == kModeHub) {
-    int64_t longest = 0;
-    for (int g = 0; g < a.groups; ++g) longest = longest > a.tstart[g + 1] - a.tstart[g] ? longest : a.tstart[g + 1] - a.tstart[g];
-    blocks = ceil_div64(ceil_div64(longest, kWavesPerBlock), 8 / a.groups) * 8;
-  } else if (a.tiles > 1) {
-    blocks = ceil_div64(blocks, 8 / a.tiles) * 8;
-  }
-  if (blocks > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "SpMM grid too large");
-  const unsigned grid = (unsigned)blocks;
-  if (grid == 0) return CG_OK;
-#define CG_CASE(V, L, CH)                                                                          \
-  if (s.vec == V && s.lpr == L && s.chunks == CH) {                                                \
-    spmm_rowseg_kernel<V, L, CH, MODE><<<grid, kSpmmThreads, 0, stream>>>(a);                      \
-    CG_LAUNCH_CHECK();                                                                             \
-    return CG_OK;                                                                                  \
-  }
-#define CG_CASES(V)                                                                                \
-  CG_CASE(V, 4, 1) CG_CASE(V, 8, 1) CG_CASE(V, 16, 1) CG_CASE(V, 32, 1) CG_CASE(V, 64, 1)           \
-  CG_CASE(V, 64, 2) CG_CASE(V, 64, 3) CG_CASE(V, 64, 4) CG_CASE(V, 64, 5) CG_CASE(V, 64, 6)           \
-  CG_CASE(V, 64, 7) CG_CASE(V, 64, 8) CG_CASE(V, 64, 9) CG_CASE(V, 64, 10)
-  CG_CASES(1) CG_CASES(2) CG_CASES(4)
-#undef CG_CASES
-#undef CG_CASE
-  CG_FAIL(CG_ERR_UNSUPPORTED, "no SpMM kernel for vec=%d lpr=%d chunks=%d", s.vec, s.lpr, s.chunks);
-}
-
-// One launch covers at most tiles * 64 * kMaxChunks slots; wider outputs take several launches
-// over column ranges.  Fills the tiling fields of `a` for the range [f0, f0 + ft).
-struct SpmmPlan {
-  SpmmShape shape;
-  int tiles, tile_slots;
-};
-static SpmmPlan plan_range(int vec, int32_t ft) {
-  const int slots = ft / vec;
-  SpmmPlan p;
-  p.tiles = pick_tiles(vec, slots);
-  p.tile_slots = (slots + p.tiles - 1) / p.tiles;
-  p.shape = pick_shape(vec, p.tile_slots);
-  return p;
-}
 static int32_t range_cap(int vec) { return kWave * kMaxChunks * vec; }
+
+// Entries per task.  Narrow teams stage a window plus one task in LDS, so their tasks are shorter.
+static int32_t pick_seg(const SpmmShape &s) {
+  const int t = g_tune_seg.load(std::memory_order_relaxed);
+  if (s.lpr == kWave) return t >= 64 ? t : 1024;
+  return (t >= 64 && t <= 512) ? t : 512;
+}
+
+// Stored entries after which a new window starts.
+static int32_t window_entries() {
+  const int w = g_tune_win.load(std::memory_order_relaxed);
+  return (w >= 64 && w <= 512) ? w : 512;
+}
 
 static int check_dense(const char *who, const float *B, int64_t ldb, float *C, int64_t ldc, int32_t f,
                        int64_t brows, int64_t crows) {
@@ -392,6 +72,61 @@ static int check_dense(const char *who, const float *B, int64_t ldb, float *C, i
                                   (long long)ldb, (long long)ldc, f);
   if ((!B && brows > 0) || (!C && crows > 0)) CG_FAIL(CG_ERR_NULL, "%s: null dense operand", who);
   if (B && C && (const float *)C == B) CG_FAIL(CG_ERR_ALIAS, "%s: C aliases B", who);
+  return CG_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// device memory for tables: owned allocations (handles) or a bump arena over a scratch buffer
+// (the one-shot entry point, which builds its tables anew on every call)
+// ---------------------------------------------------------------------------------------------
+static int dev_alloc(void **p, size_t bytes) {
+  hipError_t e = hipMalloc(p, bytes ? bytes : 4);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    *p = nullptr;
+    set_error("hipMalloc of %zu bytes failed: %s", bytes, hipGetErrorString(e));
+    return CG_ERR_ALLOC;
+  }
+  return CG_OK;
+}
+
+struct Alloc {
+  char *base = nullptr;  // arena mode when set
+  size_t cap = 0, off = 0;
+  bool arena() const { return base != nullptr; }
+  int get(void **p, size_t bytes) {
+    if (!base) return dev_alloc(p, bytes);
+    const size_t need = (bytes + 255) & ~(size_t)255;
+    if (off + need > cap) CG_FAIL(CG_ERR_ALLOC, "table arena too small (%zu + %zu > %zu)", off, need, cap);
+    *p = base + off;
+    off += need;
+    return CG_OK;
+  }
+};
+
+struct TempFree {
+  void *p[16];
+  int count = 0;
+  ~TempFree() {
+    for (int i = 0; i < count; ++i)
+      if (p[i]) (void)hipFree(p[i]);
+  }
+  int alloc(void **out, size_t bytes) {
+    CG_TRY(dev_alloc(out, bytes));
+    p[count++] = *out;
+    return CG_OK;
+  }
+};
+
+__global__ __launch_bounds__(kSpmmThreads) void fill_u32_kernel(uint32_t *__restrict__ p, int64_t count, uint32_t v) {
+  const int64_t i = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (i < count) p[i] = v;
+}
+
+static int fill_u32(uint32_t *p, int64_t count, uint32_t v, hipStream_t stream) {
+  if (count <= 0) return CG_OK;
+  fill_u32_kernel<<<(unsigned)ceil_div64(count, kSpmmThreads), kSpmmThreads, 0, stream>>>(p, count, v);
+  CG_LAUNCH_CHECK();
   return CG_OK;
 }
 
@@ -411,25 +146,33 @@ __global__ __launch_bounds__(kSpmmThreads) void sched_count_kernel(const int32_t
                                                                    uint32_t *__restrict__ nslot,
                                                                    uint32_t *__restrict__ nmulti) {
   const int64_t r = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
-  if (r >= n) return;
+  if (r > n) return;
+  if (r == n) {  // the scans run over n + 1 entries so that entry n receives the total
+    ntask[r] = nslot[r] = nmulti[r] = 0u;
+    return;
+  }
   const uint32_t t = tasks_of(rowptr[r + 1] - rowptr[r], seg, skip_empty);
   ntask[r] = t;
   nslot[r] = t > 1 ? t : 0u;
   nmulti[r] = t > 1 ? 1u : 0u;
 }
 
+// max_tasks / max_multi: capacities of the output tables (a malformed, unsorted row array could
+// otherwise describe more tasks than the arena of the one-shot entry point holds)
 __global__ __launch_bounds__(kSpmmThreads) void sched_fill_kernel(const int32_t *__restrict__ rowptr, int32_t n,
                                                                   int32_t seg, int skip_empty,
                                                                   const uint32_t *__restrict__ tbase,
                                                                   const uint32_t *__restrict__ mbase,
-                                                                  int32_t *__restrict__ task_row,
-                                                                  int32_t *__restrict__ multi_rows) {
+                                                                  int32_t *__restrict__ task_row, int64_t max_tasks,
+                                                                  int32_t *__restrict__ multi_rows,
+                                                                  int64_t max_multi) {
   const int64_t r = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (r >= n) return;
   const uint32_t t = tasks_of(rowptr[r + 1] - rowptr[r], seg, skip_empty);
   const uint32_t b = tbase[r];
-  for (uint32_t i = 0; i < t; ++i) task_row[b + i] = (int32_t)r;
-  if (t > 1) multi_rows[mbase[r]] = (int32_t)r;
+  for (uint32_t i = 0; i < t; ++i)
+    if ((int64_t)b + i < max_tasks) task_row[b + i] = (int32_t)r;
+  if (t > 1 && (int64_t)mbase[r] < max_multi) multi_rows[mbase[r]] = (int32_t)r;
 }
 
 __global__ __launch_bounds__(kSpmmThreads) void max_degree_kernel(const int32_t *__restrict__ rowptr, int32_t n,
@@ -447,75 +190,101 @@ __global__ __launch_bounds__(kSpmmThreads) void max_degree_kernel(const int32_t 
 
 struct Sched {
   int32_t seg = 0;
+  bool owned = true;  // false: tables live in an arena
+  // exact when built synchronously; upper bounds (table capacities) when built without a host
+  // round trip, in which case the exact values are only on the device (d_counts)
   int64_t ntasks = 0, nmulti = 0, nslots = 0;
   int32_t *task_row = nullptr, *tbase = nullptr, *pbase = nullptr, *multi_rows = nullptr;
+  uint32_t *d_counts = nullptr;  // {ntasks, nslots, nmulti} on the device (asynchronous builds only)
   void release() {
-    if (task_row) (void)hipFree(task_row);
-    if (tbase) (void)hipFree(tbase);
-    if (pbase) (void)hipFree(pbase);
-    if (multi_rows) (void)hipFree(multi_rows);
+    if (owned) {
+      if (task_row) (void)hipFree(task_row);
+      if (tbase) (void)hipFree(tbase);
+      if (pbase) (void)hipFree(pbase);
+      if (multi_rows) (void)hipFree(multi_rows);
+    }
     task_row = tbase = pbase = multi_rows = nullptr;
+    d_counts = nullptr;
   }
 };
 
-static int dev_alloc(void **p, size_t bytes) {
-  hipError_t e = hipMalloc(p, bytes ? bytes : 4);
-  if (e != hipSuccess) {
-    (void)hipGetLastError();
-    *p = nullptr;
-    set_error("hipMalloc of %zu bytes failed: %s", bytes, hipGetErrorString(e));
-    return CG_ERR_ALLOC;
-  }
-  return CG_OK;
-}
-
-// Task tables for the rows [0, n) described by rowptr.  Synchronises `stream`.
-static int make_sched(const int32_t *rowptr, int32_t n, int32_t seg, int skip_empty, Sched &out, hipStream_t stream) {
+// Task tables for the rows [0, n) described by rowptr.
+//   synchronous (async == false): exact table sizes, synchronises `stream`;
+//   asynchronous: tables sized by the bounds max_tasks / max_multi, nothing is read back.
+static int make_sched(const int32_t *rowptr, int32_t n, int32_t seg, int skip_empty, Sched &out, Alloc &mem,
+                      bool async, int64_t max_tasks, int64_t max_multi, hipStream_t stream) {
   Sched sc;
   sc.seg = seg;
+  sc.owned = !mem.arena();
   const size_t nb = (size_t)(n + 1) * sizeof(uint32_t);
-  uint32_t *d_mbase = nullptr;
-  void *d_totals_v = nullptr;
+  uint32_t *d_mbase = nullptr, *d_totals = nullptr;
+  TempFree tmp;
   int st = CG_OK;
   do {
-    if ((st = dev_alloc((void **)&sc.tbase, nb)) != CG_OK) break;
-    if ((st = dev_alloc((void **)&sc.pbase, nb)) != CG_OK) break;
-    if ((st = dev_alloc((void **)&d_mbase, nb)) != CG_OK) break;
-    if ((st = scratch_get(stream, kSlotB, 3 * sizeof(uint32_t), &d_totals_v)) != CG_OK) break;
-    uint32_t *d_totals = (uint32_t *)d_totals_v;
-    uint32_t totals[3] = {0, 0, 0};
-    if (n > 0) {
-      const unsigned grid = (unsigned)ceil_div64(n, kSpmmThreads);
-      sched_count_kernel<<<grid, kSpmmThreads, 0, stream>>>(rowptr, n, seg, skip_empty, (uint32_t *)sc.tbase,
-                                                            (uint32_t *)sc.pbase, d_mbase);
-      if (hipGetLastError() != hipSuccess) { st = CG_ERR_HIP; set_error("sched_count launch failed"); break; }
-      // scanning n + 1 entries puts the grand total behind the last row: tbase[n] == ntasks
-      if ((st = hipMemsetAsync((uint32_t *)sc.tbase + n, 0, 4, stream) == hipSuccess ? CG_OK : CG_ERR_HIP) != CG_OK) break;
-      if ((st = hipMemsetAsync((uint32_t *)sc.pbase + n, 0, 4, stream) == hipSuccess ? CG_OK : CG_ERR_HIP) != CG_OK) break;
-      if ((st = exclusive_scan_u32((uint32_t *)sc.tbase, (uint32_t *)sc.tbase, (int64_t)n + 1, d_totals + 0, stream)) != CG_OK) break;
-      if ((st = exclusive_scan_u32((uint32_t *)sc.pbase, (uint32_t *)sc.pbase, (int64_t)n + 1, d_totals + 1, stream)) != CG_OK) break;
-      if ((st = exclusive_scan_u32(d_mbase, d_mbase, n, d_totals + 2, stream)) != CG_OK) break;
+    if ((st = mem.get((void **)&sc.tbase, nb)) != CG_OK) break;
+    if ((st = mem.get((void **)&sc.pbase, nb)) != CG_OK) break;
+    if (mem.arena()) {
+      if ((st = mem.get((void **)&d_mbase, nb)) != CG_OK) break;
+      if ((st = mem.get((void **)&d_totals, 3 * sizeof(uint32_t))) != CG_OK) break;
+    } else {
+      if ((st = tmp.alloc((void **)&d_mbase, nb)) != CG_OK) break;
+      void *v = nullptr;
+      if ((st = scratch_get(stream, kSlotB, 3 * sizeof(uint32_t), &v)) != CG_OK) break;
+      d_totals = (uint32_t *)v;
+    }
+    const unsigned grid = (unsigned)ceil_div64((int64_t)n + 1, kSpmmThreads);
+    sched_count_kernel<<<grid, kSpmmThreads, 0, stream>>>(rowptr, n, seg, skip_empty, (uint32_t *)sc.tbase,
+                                                          (uint32_t *)sc.pbase, d_mbase);
+    if (hipGetLastError() != hipSuccess) {
+      st = CG_ERR_HIP;
+      set_error("sched_count launch failed");
+      break;
+    }
+    // scanning n + 1 entries leaves the grand total behind the last row: tbase[n] == ntasks
+    if ((st = exclusive_scan_u32((uint32_t *)sc.tbase, (uint32_t *)sc.tbase, (int64_t)n + 1, d_totals + 0, stream)) !=
+        CG_OK)
+      break;
+    if ((st = exclusive_scan_u32((uint32_t *)sc.pbase, (uint32_t *)sc.pbase, (int64_t)n + 1, d_totals + 1, stream)) !=
+        CG_OK)
+      break;
+    if ((st = exclusive_scan_u32(d_mbase, d_mbase, (int64_t)n + 1, d_totals + 2, stream)) != CG_OK) break;
+    if (async) {
+      sc.ntasks = max_tasks;
+      sc.nmulti = max_multi;
+      sc.nslots = 2 * max_multi;  // bound used for sizing only
+      sc.d_counts = d_totals;
+    } else {
+      uint32_t totals[3] = {0, 0, 0};
       if (hipMemcpyAsync(totals, d_totals, sizeof(totals), hipMemcpyDeviceToHost, stream) != hipSuccess ||
           hipStreamSynchronize(stream) != hipSuccess) {
         st = CG_ERR_HIP;
         set_error("schedule totals copy failed");
         break;
       }
+      sc.ntasks = totals[0];
+      sc.nslots = totals[1];
+      sc.nmulti = totals[2];
     }
-    sc.ntasks = totals[0];
-    sc.nslots = totals[1];
-    sc.nmulti = totals[2];
-    if ((st = dev_alloc((void **)&sc.task_row, (size_t)sc.ntasks * sizeof(int32_t))) != CG_OK) break;
-    if ((st = dev_alloc((void **)&sc.multi_rows, (size_t)sc.nmulti * sizeof(int32_t))) != CG_OK) break;
+    if ((st = mem.get((void **)&sc.task_row, (size_t)(sc.ntasks > 0 ? sc.ntasks : 1) * sizeof(int32_t))) != CG_OK)
+      break;
+    if ((st = mem.get((void **)&sc.multi_rows, (size_t)(sc.nmulti > 0 ? sc.nmulti : 1) * sizeof(int32_t))) != CG_OK)
+      break;
     if (n > 0) {
-      const unsigned grid = (unsigned)ceil_div64(n, kSpmmThreads);
-      sched_fill_kernel<<<grid, kSpmmThreads, 0, stream>>>(rowptr, n, seg, skip_empty, (const uint32_t *)sc.tbase,
-                                                           d_mbase, sc.task_row, sc.multi_rows);
-      if (hipGetLastError() != hipSuccess) { st = CG_ERR_HIP; set_error("sched_fill launch failed"); break; }
-      if (hipStreamSynchronize(stream) != hipSuccess) { st = CG_ERR_HIP; set_error("sched_fill failed"); break; }
+      sched_fill_kernel<<<(unsigned)ceil_div64(n, kSpmmThreads), kSpmmThreads, 0, stream>>>(
+          rowptr, n, seg, skip_empty, (const uint32_t *)sc.tbase, d_mbase, sc.task_row, sc.ntasks, sc.multi_rows,
+          sc.nmulti);
+      if (hipGetLastError() != hipSuccess) {
+        st = CG_ERR_HIP;
+        set_error("sched_fill launch failed");
+        break;
+      }
+    }
+    if (!async && hipStreamSynchronize(stream) != hipSuccess) {
+      st = CG_ERR_HIP;
+      set_error("sched_fill failed");
+      break;
     }
   } while (0);
-  if (d_mbase) (void)hipFree(d_mbase);
   if (st != CG_OK) {
     sc.release();
     return st;
@@ -524,51 +293,39 @@ static int make_sched(const int32_t *rowptr, int32_t n, int32_t seg, int skip_em
   return CG_OK;
 }
 
-struct TempFree {
-  void *p[16];
-  int count = 0;
-  ~TempFree() {
-    for (int i = 0; i < count; ++i)
-      if (p[i]) (void)hipFree(p[i]);
-  }
-  int alloc(void **out, size_t bytes) {
-    CG_TRY(dev_alloc(out, bytes));
-    p[count++] = *out;
-    return CG_OK;
-  }
-};
-
 // ---------------------------------------------------------------------------------------------
-// streaming over windows of tasks
+// window tables
 // ---------------------------------------------------------------------------------------------
-// Tasks are contiguous in the entry stream (task t covers [task_start[t], task_start[t+1])), so a
-// wavefront that takes a window of consecutive tasks reads one contiguous piece of (colind, val)
-// and never pays a task's start-up latency more than once per window.  Windows hold at most 64
-// tasks (their metadata lives in one register per lane) and start a new one every `S` entries.
 struct StreamTab {
   int32_t S = 0, groups = 0;
-  bool hub = false;
+  bool hub = false, owned = true;
   int32_t *task_start = nullptr, *task_dst = nullptr, *wstart = nullptr;
-  int64_t nwin = 0;
+  int64_t nwin = 0;            // exact, or the grid bound of an asynchronous build
+  uint32_t *d_nwin = nullptr;  // exact count on the device (asynchronous builds only)
   int64_t win_first[18] = {0};
   void release() {
-    if (task_start) (void)hipFree(task_start);
-    if (task_dst) (void)hipFree(task_dst);
-    if (wstart) (void)hipFree(wstart);
+    if (owned) {
+      if (task_start) (void)hipFree(task_start);
+      if (task_dst) (void)hipFree(task_dst);
+      if (wstart) (void)hipFree(wstart);
+    }
     task_start = task_dst = wstart = nullptr;
+    d_nwin = nullptr;
     S = 0;
   }
 };
 
+__device__ __forceinline__ int64_t count_of(int64_t host, const uint32_t *dev) { return dev ? (int64_t)*dev : host; }
+
 // task_dst: row index (>= 0) when the task is the whole row and goes straight to C, else
 // -(partial slot + 1).  In a hub plan every task is partial and its slot is its own index.
-__global__ __launch_bounds__(kSpmmThreads) void stream_tasks_kernel(const int32_t *__restrict__ rowptr, int32_t nrows,
-                                                                    const int32_t *__restrict__ task_row,
-                                                                    const int32_t *__restrict__ tbase,
-                                                                    const int32_t *__restrict__ pbase, int32_t seg,
-                                                                    int64_t ntasks, int hub,
-                                                                    int32_t *__restrict__ task_start,
-                                                                    int32_t *__restrict__ task_dst) {
+__global__ __launch_bounds__(kSpmmThreads) void stream_tasks_kernel(
+    const int32_t *__restrict__ rowptr, int32_t nrows, const int32_t *__restrict__ task_row,
+    const int32_t *__restrict__ tbase, const int32_t *__restrict__ pbase, int32_t seg, int64_t ntasks_host,
+    const uint32_t *__restrict__ d_ntasks, int64_t cap, int hub, int32_t *__restrict__ task_start,
+    int32_t *__restrict__ task_dst) {
+  int64_t ntasks = count_of(ntasks_host, d_ntasks);
+  if (ntasks > cap) ntasks = cap;
   const int64_t t = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (t > ntasks) return;
   if (t == ntasks) {
@@ -583,19 +340,25 @@ __global__ __launch_bounds__(kSpmmThreads) void stream_tasks_kernel(const int32_
 }
 
 // flags[t] = 1 where a window starts: every 64th task of a class ...
-__global__ __launch_bounds__(kSpmmThreads) void window_flag_tasks_kernel(int64_t t0, int64_t t1,
+__global__ __launch_bounds__(kSpmmThreads) void window_flag_tasks_kernel(int64_t t0, int64_t t1_host,
+                                                                         const uint32_t *__restrict__ d_t1,
                                                                          uint32_t *__restrict__ flags) {
+  int64_t t1 = count_of(t1_host, d_t1);
+  if (t1 > t1_host) t1 = t1_host;
   const int64_t t = t0 + (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (t < t1) flags[t] = ((t - t0) & 63) == 0 ? 1u : 0u;
 }
 
 // ... and the first task that starts at or after every multiple of S entries of the class.
 __global__ __launch_bounds__(kSpmmThreads) void window_flag_entries_kernel(const int32_t *__restrict__ task_start,
-                                                                           int64_t t0, int64_t t1, int32_t S,
-                                                                           int64_t nbounds,
+                                                                           int64_t t0, int64_t t1_host,
+                                                                           const uint32_t *__restrict__ d_t1,
+                                                                           int32_t S, int64_t nbounds,
                                                                            uint32_t *__restrict__ flags) {
+  int64_t t1 = count_of(t1_host, d_t1);
+  if (t1 > t1_host) t1 = t1_host;
   const int64_t j = 1 + (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
-  if (j > nbounds) return;
+  if (j > nbounds || t1 <= t0) return;
   const int64_t target = (int64_t)task_start[t0] + j * S;
   int64_t lo = t0, hi = t1;  // first t in [t0, t1) with task_start[t] >= target
   while (lo < hi) {
@@ -608,22 +371,34 @@ __global__ __launch_bounds__(kSpmmThreads) void window_flag_entries_kernel(const
 
 __global__ __launch_bounds__(kSpmmThreads) void window_compact_kernel(const uint32_t *__restrict__ flags,
                                                                       const uint32_t *__restrict__ index,
-                                                                      int64_t ntasks, int32_t *__restrict__ wstart,
-                                                                      uint32_t nwin) {
+                                                                      int64_t ntasks_host,
+                                                                      const uint32_t *__restrict__ d_ntasks,
+                                                                      int32_t *__restrict__ wstart,
+                                                                      uint32_t *__restrict__ d_nwin, int64_t wcap) {
+  int64_t ntasks = count_of(ntasks_host, d_ntasks);
+  if (ntasks > ntasks_host) ntasks = ntasks_host;
   const int64_t t = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
-  if (t < ntasks && flags[t]) wstart[index[t]] = (int32_t)t;
-  if (t == ntasks) wstart[nwin] = (int32_t)ntasks;
+  if (t < ntasks && flags[t] && (int64_t)index[t] < wcap) wstart[index[t]] = (int32_t)t;
+  if (t == ntasks) {
+    const int64_t nwin = (int64_t)index[ntasks] < wcap ? (int64_t)index[ntasks] : wcap;
+    wstart[nwin] = (int32_t)ntasks;
+    if (d_nwin) *d_nwin = (uint32_t)nwin;
+  }
 }
 
 // class_first[g] .. class_first[g+1]: tasks of class g (nclass == 1 for a plain schedule).
+// nnz: stored entries the tasks cover (bounds the window count of an asynchronous build).
 static int build_stream(const Sched &sc, const int32_t *rowptr, int32_t nrows, bool hub, int nclass,
-                        const int64_t *class_first, int32_t S, StreamTab &out, hipStream_t stream) {
+                        const int64_t *class_first, int32_t S, int64_t nnz, StreamTab &out, Alloc &mem, bool async,
+                        hipStream_t stream) {
   out.release();
-  const int64_t nt = sc.ntasks;
-  CG_TRY(dev_alloc((void **)&out.task_start, (size_t)(nt + 1) * 4));
-  CG_TRY(dev_alloc((void **)&out.task_dst, (size_t)(nt + 1) * 4));
+  out.owned = !mem.arena();
+  const int64_t nt = sc.ntasks;  // exact, or the capacity bound when async
+  const uint32_t *d_nt = async ? sc.d_counts + 0 : nullptr;
+  CG_TRY(mem.get((void **)&out.task_start, (size_t)(nt + 1) * 4));
+  CG_TRY(mem.get((void **)&out.task_dst, (size_t)(nt + 1) * 4));
   stream_tasks_kernel<<<(unsigned)ceil_div64(nt + 1, kSpmmThreads), kSpmmThreads, 0, stream>>>(
-      rowptr, nrows, sc.task_row, sc.tbase, sc.pbase, sc.seg, nt, hub ? 1 : 0, out.task_start, out.task_dst);
+      rowptr, nrows, sc.task_row, sc.tbase, sc.pbase, sc.seg, nt, d_nt, nt, hub ? 1 : 0, out.task_start, out.task_dst);
   CG_LAUNCH_CHECK();
   out.S = S;
   out.hub = hub;
@@ -631,16 +406,49 @@ static int build_stream(const Sched &sc, const int32_t *rowptr, int32_t nrows, b
   out.nwin = 0;
   for (int g = 0; g <= nclass; ++g) out.win_first[g] = 0;
   if (nt == 0) {
-    CG_TRY(dev_alloc((void **)&out.wstart, 4));
-    CG_HIP(hipMemsetAsync(out.wstart, 0, 4, stream));
-    CG_HIP(hipStreamSynchronize(stream));
+    CG_TRY(mem.get((void **)&out.wstart, 4));
+    CG_TRY(fill_u32((uint32_t *)out.wstart, 1, 0u, stream));
+    if (!async) CG_HIP(hipStreamSynchronize(stream));
     return CG_OK;
   }
-  uint32_t *flags = nullptr, *index = nullptr;
+  uint32_t *flags = nullptr, *index = nullptr, *d_total = nullptr;
   TempFree tmp;
-  CG_TRY(tmp.alloc((void **)&flags, (size_t)(nt + 1) * 4));
-  CG_TRY(tmp.alloc((void **)&index, (size_t)(nt + 1) * 4));
-  // entry extents of the classes (host needs them to size the boundary launches)
+  if (mem.arena()) {
+    CG_TRY(mem.get((void **)&flags, (size_t)(nt + 1) * 4));
+    CG_TRY(mem.get((void **)&index, (size_t)(nt + 1) * 4));
+    CG_TRY(mem.get((void **)&d_total, 4));
+  } else {
+    CG_TRY(tmp.alloc((void **)&flags, (size_t)(nt + 1) * 4));
+    CG_TRY(tmp.alloc((void **)&index, (size_t)(nt + 1) * 4));
+    void *v = nullptr;
+    CG_TRY(scratch_get(stream, kSlotB, 4, &v));
+    d_total = (uint32_t *)v;
+  }
+  // flags[nt] stays 0, so the scan over nt + 1 flags leaves the window count in index[ntasks]
+  CG_TRY(fill_u32(flags, nt + 1, 0u, stream));
+  if (async) {
+    // one class over all tasks; the exact task count stays on the device
+    window_flag_tasks_kernel<<<(unsigned)ceil_div64(nt, kSpmmThreads), kSpmmThreads, 0, stream>>>(0, nt, d_nt, flags);
+    CG_LAUNCH_CHECK();
+    const int64_t nb = nnz / S;
+    if (nb > 0) {
+      window_flag_entries_kernel<<<(unsigned)ceil_div64(nb, kSpmmThreads), kSpmmThreads, 0, stream>>>(
+          out.task_start, 0, nt, d_nt, S, nb, flags);
+      CG_LAUNCH_CHECK();
+    }
+    CG_TRY(exclusive_scan_u32(flags, index, nt + 1, nullptr, stream));
+    const int64_t wcap = ceil_div64(nt, 64) + nnz / S + 2;
+    CG_TRY(mem.get((void **)&out.wstart, (size_t)(wcap + 1) * 4));
+    window_compact_kernel<<<(unsigned)ceil_div64(nt + 1, kSpmmThreads), kSpmmThreads, 0, stream>>>(
+        flags, index, nt, d_nt, out.wstart, d_total, wcap);
+    CG_LAUNCH_CHECK();
+    out.nwin = wcap;
+    out.d_nwin = d_total;
+    out.win_first[0] = 0;
+    out.win_first[1] = wcap;
+    return CG_OK;
+  }
+  // entry extents of the classes (the host needs them to size the boundary launches)
   int32_t ends[18];
   for (int g = 0; g <= nclass; ++g)
     CG_HIP(hipMemcpyAsync(&ends[g], out.task_start + class_first[g], 4, hipMemcpyDeviceToHost, stream));
@@ -648,381 +456,37 @@ static int build_stream(const Sched &sc, const int32_t *rowptr, int32_t nrows, b
   for (int g = 0; g < nclass; ++g) {
     const int64_t t0 = class_first[g], t1 = class_first[g + 1];
     if (t1 <= t0) continue;
-    window_flag_tasks_kernel<<<(unsigned)ceil_div64(t1 - t0, kSpmmThreads), kSpmmThreads, 0, stream>>>(t0, t1, flags);
+    window_flag_tasks_kernel<<<(unsigned)ceil_div64(t1 - t0, kSpmmThreads), kSpmmThreads, 0, stream>>>(t0, t1, nullptr,
+                                                                                                     flags);
     CG_LAUNCH_CHECK();
     const int64_t nb = ((int64_t)ends[g + 1] - ends[g]) / S;
     if (nb > 0) {
       window_flag_entries_kernel<<<(unsigned)ceil_div64(nb, kSpmmThreads), kSpmmThreads, 0, stream>>>(
-          out.task_start, t0, t1, S, nb, flags);
+          out.task_start, t0, t1, nullptr, S, nb, flags);
       CG_LAUNCH_CHECK();
     }
   }
-  void *d_total_v = nullptr;
-  CG_TRY(scratch_get(stream, kSlotB, 4, &d_total_v));
-  CG_TRY(exclusive_scan_u32(flags, index, nt, (uint32_t *)d_total_v, stream));
+  CG_TRY(exclusive_scan_u32(flags, index, nt + 1, d_total, stream));
   uint32_t nwin = 0;
-  CG_HIP(hipMemcpyAsync(&nwin, d_total_v, 4, hipMemcpyDeviceToHost, stream));
+  CG_HIP(hipMemcpyAsync(&nwin, d_total, 4, hipMemcpyDeviceToHost, stream));
   uint32_t firsts[18] = {0};
   for (int g = 0; g < nclass; ++g)
-    if (class_first[g] < nt) CG_HIP(hipMemcpyAsync(&firsts[g], index + class_first[g], 4, hipMemcpyDeviceToHost, stream));
+    CG_HIP(hipMemcpyAsync(&firsts[g], index + class_first[g], 4, hipMemcpyDeviceToHost, stream));
   CG_HIP(hipStreamSynchronize(stream));
-  for (int g = 0; g < nclass; ++g) out.win_first[g] = class_first[g] < nt ? firsts[g] : nwin;
+  for (int g = 0; g < nclass; ++g) out.win_first[g] = firsts[g];
   out.win_first[nclass] = nwin;
   out.nwin = nwin;
-  CG_TRY(dev_alloc((void **)&out.wstart, (size_t)(nwin + 1) * 4));
-  window_compact_kernel<<<(unsigned)ceil_div64(nt + 1, kSpmmThreads), kSpmmThreads, 0, stream>>>(flags, index, nt,
-                                                                                                out.wstart, nwin);
+  CG_TRY(mem.get((void **)&out.wstart, (size_t)(nwin + 1) * 4));
+  window_compact_kernel<<<(unsigned)ceil_div64(nt + 1, kSpmmThreads), kSpmmThreads, 0, stream>>>(
+      flags, index, nt, nullptr, out.wstart, nullptr, (int64_t)nwin);
   CG_LAUNCH_CHECK();
   CG_HIP(hipStreamSynchronize(stream));
   return CG_OK;
 }
 
-struct StreamArgs {
-  const int32_t *task_start, *task_dst, *wstart;
-  const int32_t *colind;
-  const float *val;
-  int64_t win_first[9];
-  int32_t groups;  // 1: windows run anywhere; 2/4/8: windows of class g run on XCDs x % groups == g
-  const float *B;
-  int64_t ldb;
-  float *C;
-  int64_t ldc;
-  float *P;
-  int32_t f;
-  float beta;
-};
-
-// Full-wave teams (one stored entry per wave step, f covered by CHUNKS x 64 lanes x VEC floats).
-template <int VEC, int CHUNKS>
-__global__ __launch_bounds__(kSpmmThreads) void spmm_stream_wide_kernel(const StreamArgs a) {
-  const int lane = threadIdx.x & (kWave - 1);
-  const int x = blockIdx.x & 7;
-  const int per = 8 / a.groups;
-  const int grp = x % a.groups;
-  const int64_t lblock = (int64_t)(blockIdx.x >> 3) * per + x / a.groups;
-  const int64_t wl = lblock * kWavesPerBlock + threadIdx.x / kWave;
-  if (wl >= a.win_first[grp + 1] - a.win_first[grp]) return;
-  const int32_t w = __builtin_amdgcn_readfirstlane((int32_t)(a.win_first[grp] + wl));
-  const int32_t t0 = a.wstart[w], t1 = a.wstart[w + 1];
-  const int ntask = t1 - t0;  // 1..64
-  int32_t m_end = 0, m_dst = 0;
-  if (lane < ntask) {
-    m_end = a.task_start[t0 + lane + 1];
-    m_dst = a.task_dst[t0 + lane];
-  }
-  const int32_t e_begin = a.task_start[t0];
-  const int32_t e_end = __builtin_amdgcn_readlane(m_end, ntask - 1);
-
-  const int nslots = a.f / VEC;
-  bool active[CHUNKS];
-  int64_t boff[CHUNKS];
-#pragma unroll
-  for (int ch = 0; ch < CHUNKS; ++ch) {
-    active[ch] = (ch * kWave + lane) < nslots;
-    boff[ch] = (int64_t)(ch * kWave + (active[ch] ? lane : 0)) * VEC;
-  }
-  float acc[CHUNKS][VEC];
-#pragma unroll
-  for (int ch = 0; ch < CHUNKS; ++ch)
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) acc[ch][v] = 0.f;
-
-  constexpr int U = 4;
-  int tk = 0;
-  int32_t tbeg = e_begin;
-  int32_t tend = __builtin_amdgcn_readlane(m_end, 0);
-
-  int32_t c_next = 0;
-  float v_next = 0.f;
-  if (e_begin + lane < e_end) {
-    c_next = a.colind[e_begin + lane];
-    v_next = a.val[e_begin + lane];
-  }
-  for (int32_t base = e_begin;; base += kWave) {
-    const int32_t c = c_next;
-    const float v = v_next;
-    const int32_t nb = base + kWave + lane;
-    c_next = 0;
-    v_next = 0.f;
-    if (nb < e_end) {
-      c_next = a.colind[nb];
-      v_next = a.val[nb];
-    }
-    int cnt = e_end - base;
-    cnt = cnt > kWave ? kWave : (cnt < 0 ? 0 : cnt);
-    int i = 0;
-    for (;;) {
-      while (tend == base + i) {  // the current task is complete (also true at once for an empty task)
-        const int32_t dst = __builtin_amdgcn_readlane(m_dst, tk);
-        if (dst >= 0) {
-          if (!(tend == tbeg && a.beta == 1.0f)) {  // an empty row leaves C alone when beta == 1
-            float *crow = a.C + (int64_t)dst * a.ldc;
-#pragma unroll
-            for (int ch = 0; ch < CHUNKS; ++ch) {
-              if (active[ch]) {
-                float out[VEC];
-                if (a.beta != 0.f) {
-                  float old[VEC];
-                  load_vec<VEC>(crow + boff[ch], old);
-#pragma unroll
-                  for (int q = 0; q < VEC; ++q) out[q] = fmaf(a.beta, old[q], acc[ch][q]);
-                } else {
-#pragma unroll
-                  for (int q = 0; q < VEC; ++q) out[q] = acc[ch][q];
-                }
-                store_vec<VEC>(crow + boff[ch], out);
-              }
-            }
-          }
-        } else {
-          float *prow = a.P + (int64_t)(-(dst + 1)) * a.f;
-#pragma unroll
-          for (int ch = 0; ch < CHUNKS; ++ch)
-            if (active[ch]) store_vec<VEC>(prow + boff[ch], acc[ch]);
-        }
-#pragma unroll
-        for (int ch = 0; ch < CHUNKS; ++ch)
-#pragma unroll
-          for (int q = 0; q < VEC; ++q) acc[ch][q] = 0.f;
-        if (++tk == ntask) return;
-        tbeg = tend;
-        tend = __builtin_amdgcn_readlane(m_end, tk);
-      }
-      if (i >= cnt) break;
-      int run = tend - base;
-      run = run < cnt ? run : cnt;
-      if (run <= i) return;  // cannot happen with monotone task starts; guarantees termination
-      for (; i + U <= run; i += U) {
-        float b[U][CHUNKS][VEC];
-        float vv[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const int32_t cc = __builtin_amdgcn_readlane(c, i + u);
-          vv[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), i + u));
-          const float *brow = a.B + (int64_t)cc * a.ldb;
-#pragma unroll
-          for (int ch = 0; ch < CHUNKS; ++ch) load_vec<VEC>(brow + boff[ch], b[u][ch]);
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-          for (int ch = 0; ch < CHUNKS; ++ch)
-#pragma unroll
-            for (int q = 0; q < VEC; ++q) acc[ch][q] = fmaf(vv[u], b[u][ch][q], acc[ch][q]);
-      }
-      for (; i < run; ++i) {
-        const int32_t cc = __builtin_amdgcn_readlane(c, i);
-        const float vv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), i));
-        const float *brow = a.B + (int64_t)cc * a.ldb;
-        float b[CHUNKS][VEC];
-#pragma unroll
-        for (int ch = 0; ch < CHUNKS; ++ch) load_vec<VEC>(brow + boff[ch], b[ch]);
-#pragma unroll
-        for (int ch = 0; ch < CHUNKS; ++ch)
-#pragma unroll
-          for (int q = 0; q < VEC; ++q) acc[ch][q] = fmaf(vv, b[ch][q], acc[ch][q]);
-      }
-    }
-  }
-}
-
-static int launch_stream_wide(int vec, int chunks, const StreamArgs &a, hipStream_t stream) {
-  int64_t longest = 0;
-  for (int g = 0; g < a.groups; ++g) {
-    const int64_t len = a.win_first[g + 1] - a.win_first[g];
-    longest = longest > len ? longest : len;
-  }
-  const int64_t blocks = ceil_div64(ceil_div64(longest, kWavesPerBlock), 8 / a.groups) * 8;
-  if (blocks == 0) return CG_OK;
-  if (blocks > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "SpMM grid too large");
-  const unsigned grid = (unsigned)blocks;
-#define CG_CASE(V, CH)                                                              \
-  if (vec == V && chunks == CH) {                                                   \
-    spmm_stream_wide_kernel<V, CH><<<grid, kSpmmThreads, 0, stream>>>(a);           \
-    CG_LAUNCH_CHECK();                                                              \
-    return CG_OK;                                                                   \
-  }
-#define CG_CASES(V)                                                                                     \
-  CG_CASE(V, 1) CG_CASE(V, 2) CG_CASE(V, 3) CG_CASE(V, 4) CG_CASE(V, 5) CG_CASE(V, 6) CG_CASE(V, 7)     \
-  CG_CASE(V, 8) CG_CASE(V, 9) CG_CASE(V, 10)
-  CG_CASES(1) CG_CASES(2) CG_CASES(4)
-#undef CG_CASES
-#undef CG_CASE
-  CG_FAIL(CG_ERR_UNSUPPORTED, "no streaming SpMM kernel for vec=%d chunks=%d", vec, chunks);
-}
-
-// Teams of LPR < 64 lanes (f <= 64 * VEC floats): the window's entries and task table are staged
-// in LDS.  Long tasks (>= kLongFactor * G entries) are worked on by all G teams together (entries
-// dealt round robin, partial sums combined by the xor butterfly); the short ones are dealt to the
-// teams whole, G at a time, so rows of a few entries cost neither a butterfly nor an idle wave.
-constexpr int kNarrowLds = 1024;  // entries a window may hold (window length S plus one task, both <= 512)
-constexpr int kLongFactor = 4;
-
-template <int VEC, int LPR>
-__global__ __launch_bounds__(kSpmmThreads) void spmm_stream_narrow_kernel(const StreamArgs a) {
-  constexpr int G = kWave / LPR;
-  __shared__ int32_t s_col[kWavesPerBlock][kNarrowLds];
-  __shared__ float s_val[kWavesPerBlock][kNarrowLds];
-  __shared__ int32_t s_beg[kWavesPerBlock][kWave], s_end[kWavesPerBlock][kWave], s_dst[kWavesPerBlock][kWave];
-  __shared__ int32_t s_short[kWavesPerBlock][kWave];
-
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wv = threadIdx.x / kWave;
-  const int x = blockIdx.x & 7;
-  const int per = 8 / a.groups;
-  const int grp = x % a.groups;
-  const int64_t lblock = (int64_t)(blockIdx.x >> 3) * per + x / a.groups;
-  const int64_t wl = lblock * kWavesPerBlock + wv;
-  if (wl >= a.win_first[grp + 1] - a.win_first[grp]) return;
-  const int32_t w = __builtin_amdgcn_readfirstlane((int32_t)(a.win_first[grp] + wl));
-  const int32_t t0 = a.wstart[w], t1 = a.wstart[w + 1];
-  const int ntask = t1 - t0;  // 1..64
-  const bool valid = lane < ntask;
-  int32_t m_beg = 0, m_end = 0, m_dst = 0;
-  if (valid) {
-    m_beg = a.task_start[t0 + lane];
-    m_end = a.task_start[t0 + lane + 1];
-    m_dst = a.task_dst[t0 + lane];
-  }
-  const int32_t e_begin = __builtin_amdgcn_readlane(m_beg, 0);
-  const int32_t e_end = __builtin_amdgcn_readlane(m_end, ntask - 1);
-  const int32_t nent = e_end - e_begin;
-  if (nent > kNarrowLds) return;  // excluded by the schedule (S + seg <= kNarrowLds); keeps LDS writes in bounds
-
-  for (int32_t k = lane; k < nent; k += kWave) {
-    s_col[wv][k] = a.colind[e_begin + k];
-    s_val[wv][k] = a.val[e_begin + k];
-  }
-  const int32_t r_beg = m_beg - e_begin, r_end = m_end - e_begin;  // relative to the window
-  s_beg[wv][lane] = r_beg;
-  s_end[wv][lane] = r_end;
-  s_dst[wv][lane] = m_dst;
-  const int32_t len = r_end - r_beg;
-  const bool is_long = valid && len >= kLongFactor * G;
-  // an empty row that goes straight to C needs no work when beta == 1
-  const bool is_short = valid && !is_long && !(len == 0 && m_dst >= 0 && a.beta == 1.0f);
-
-  const int g = lane / LPR, j = lane % LPR;
-  const bool active = j * VEC < a.f;
-  const int64_t boff = active ? (int64_t)j * VEC : 0;
-  const int32_t *cw = s_col[wv];
-  const float *vw = s_val[wv];
-
-  const uint64_t short_mask = __ballot(is_short);
-  if (is_short) s_short[wv][__popcll(short_mask & ((1ull << lane) - 1ull))] = lane;
-  const int nshort = __popcll(short_mask);
-  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
-  __builtin_amdgcn_wave_barrier();  // the staged window and tables are visible to every lane of the wave
-
-  // ---- long tasks: all teams together
-  uint64_t long_mask = __ballot(is_long);
-  while (long_mask) {
-    const int k = __builtin_ctzll(long_mask);
-    long_mask &= long_mask - 1;
-    const int32_t s = __builtin_amdgcn_readlane(r_beg, k);
-    const int32_t e = __builtin_amdgcn_readlane(r_end, k);
-    const int32_t d = __builtin_amdgcn_readlane(m_dst, k);
-    float acc[VEC];
-#pragma unroll
-    for (int q = 0; q < VEC; ++q) acc[q] = 0.f;
-    int32_t i = s + g;
-    for (; i + 3 * G < e; i += 4 * G) {
-      float b[4][VEC], vv[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int32_t cc = cw[i + u * G];
-        vv[u] = vw[i + u * G];
-        load_vec<VEC>(a.B + (int64_t)cc * a.ldb + boff, b[u]);
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-#pragma unroll
-        for (int q = 0; q < VEC; ++q) acc[q] = fmaf(vv[u], b[u][q], acc[q]);
-    }
-    for (; i < e; i += G) {
-      float b[VEC];
-      const float vv = vw[i];
-      load_vec<VEC>(a.B + (int64_t)cw[i] * a.ldb + boff, b);
-#pragma unroll
-      for (int q = 0; q < VEC; ++q) acc[q] = fmaf(vv, b[q], acc[q]);
-    }
-#pragma unroll
-    for (int off = LPR; off < kWave; off <<= 1)
-#pragma unroll
-      for (int q = 0; q < VEC; ++q) acc[q] += __shfl_xor(acc[q], off, kWave);
-    if (g == 0 && active) {
-      if (d >= 0) {
-        float *crow = a.C + (int64_t)d * a.ldc + boff;
-        float out[VEC];
-        if (a.beta != 0.f) {
-          float old[VEC];
-          load_vec<VEC>(crow, old);
-#pragma unroll
-          for (int q = 0; q < VEC; ++q) out[q] = fmaf(a.beta, old[q], acc[q]);
-        } else {
-#pragma unroll
-          for (int q = 0; q < VEC; ++q) out[q] = acc[q];
-        }
-        store_vec<VEC>(crow, out);
-      } else {
-        store_vec<VEC>(a.P + (int64_t)(-(d + 1)) * a.f + boff, acc);
-      }
-    }
-  }
-
-  // ---- short tasks: one team each, G per round
-  for (int q0 = 0; q0 < nshort; q0 += G) {
-    const int my = q0 + g;
-    const bool has = my < nshort;
-    const int k = has ? s_short[wv][my] : 0;
-    const int32_t s = s_beg[wv][k];
-    const int32_t e = has ? s_end[wv][k] : s;
-    const int32_t d = s_dst[wv][k];
-    float acc[VEC];
-#pragma unroll
-    for (int q = 0; q < VEC; ++q) acc[q] = 0.f;
-    int32_t i = s;
-    for (; i + 3 < e; i += 4) {
-      float b[4][VEC], vv[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int32_t cc = cw[i + u];
-        vv[u] = vw[i + u];
-        load_vec<VEC>(a.B + (int64_t)cc * a.ldb + boff, b[u]);
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-#pragma unroll
-        for (int q = 0; q < VEC; ++q) acc[q] = fmaf(vv[u], b[u][q], acc[q]);
-    }
-    for (; i < e; ++i) {
-      float b[VEC];
-      const float vv = vw[i];
-      load_vec<VEC>(a.B + (int64_t)cw[i] * a.ldb + boff, b);
-#pragma unroll
-      for (int q = 0; q < VEC; ++q) acc[q] = fmaf(vv, b[q], acc[q]);
-    }
-    if (has && active) {
-      if (d >= 0) {
-        float *crow = a.C + (int64_t)d * a.ldc + boff;
-        float out[VEC];
-        if (a.beta != 0.f) {
-          float old[VEC];
-          load_vec<VEC>(crow, old);
-#pragma unroll
-          for (int q = 0; q < VEC; ++q) out[q] = fmaf(a.beta, old[q], acc[q]);
-        } else {
-#pragma unroll
-          for (int q = 0; q < VEC; ++q) out[q] = acc[q];
-        }
-        store_vec<VEC>(crow, out);
-      } else {
-        store_vec<VEC>(a.P + (int64_t)(-(d + 1)) * a.f + boff, acc);
-      }
-    }
-  }
-}
-
+// ---------------------------------------------------------------------------------------------
+// launches
+// ---------------------------------------------------------------------------------------------
 static int64_t stream_grid(const StreamArgs &a) {
   int64_t longest = 0;
   for (int g = 0; g < a.groups; ++g) {
@@ -1032,29 +496,42 @@ static int64_t stream_grid(const StreamArgs &a) {
   return ceil_div64(ceil_div64(longest, kWavesPerBlock), 8 / a.groups) * 8;
 }
 
-static int launch_stream_narrow(int vec, int lpr, const StreamArgs &a, hipStream_t stream) {
+static int launch_stream(const SpmmShape &s, const StreamArgs &a, hipStream_t stream) {
   const int64_t blocks = stream_grid(a);
   if (blocks == 0) return CG_OK;
   if (blocks > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "SpMM grid too large");
   const unsigned grid = (unsigned)blocks;
-#define CG_CASE(V, L)                                                               \
-  if (vec == V && lpr == L) {                                                       \
-    spmm_stream_narrow_kernel<V, L><<<grid, kSpmmThreads, 0, stream>>>(a);          \
-    CG_LAUNCH_CHECK();                                                              \
-    return CG_OK;                                                                   \
+#define CG_WIDE(V, CH)                                                    \
+  if (s.lpr == kWave && s.vec == V && s.chunks == CH) {                   \
+    spmm_stream_wide_kernel<V, CH><<<grid, kSpmmThreads, 0, stream>>>(a); \
+    CG_LAUNCH_CHECK();                                                    \
+    return CG_OK;                                                         \
   }
-#define CG_CASES(V) CG_CASE(V, 4) CG_CASE(V, 8) CG_CASE(V, 16) CG_CASE(V, 32)
+#define CG_NARROW(V, L)                                                    \
+  if (s.lpr == L && s.vec == V) {                                          \
+    spmm_stream_narrow_kernel<V, L><<<grid, kSpmmThreads, 0, stream>>>(a); \
+    CG_LAUNCH_CHECK();                                                     \
+    return CG_OK;                                                          \
+  }
+#define CG_CASES(V)                                                                                 \
+  CG_NARROW(V, 4) CG_NARROW(V, 8) CG_NARROW(V, 16) CG_NARROW(V, 32)                                 \
+  CG_WIDE(V, 1) CG_WIDE(V, 2) CG_WIDE(V, 3) CG_WIDE(V, 4) CG_WIDE(V, 5) CG_WIDE(V, 6) CG_WIDE(V, 7) \
+  CG_WIDE(V, 8) CG_WIDE(V, 9) CG_WIDE(V, 10)
   CG_CASES(1) CG_CASES(2) CG_CASES(4)
 #undef CG_CASES
-#undef CG_CASE
-  CG_FAIL(CG_ERR_UNSUPPORTED, "no narrow streaming SpMM kernel for vec=%d lpr=%d", vec, lpr);
+#undef CG_NARROW
+#undef CG_WIDE
+  CG_FAIL(CG_ERR_UNSUPPORTED, "no SpMM kernel for vec=%d lpr=%d chunks=%d", s.vec, s.lpr, s.chunks);
 }
 
-// A small cache of schedules keyed by segment length.
+// ---------------------------------------------------------------------------------------------
+// handle data
+// ---------------------------------------------------------------------------------------------
+// A small cache of schedules (and their window tables) keyed by segment length.
 struct SchedCache {
   static constexpr int kMax = 4;
   Sched sched[kMax];
-  StreamTab tab[kMax];  // window tables of sched[i], built on first use
+  StreamTab tab[kMax];
   int count = 0;
   void release() {
     for (int i = 0; i < count; ++i) {
@@ -1081,7 +558,8 @@ struct SchedCache {
       sched[--count] = Sched();
       tab[count] = StreamTab();
     }
-    CG_TRY(make_sched(rowptr, n, seg, 0, sched[count], stream));
+    Alloc owned;
+    CG_TRY(make_sched(rowptr, n, seg, 0, sched[count], owned, false, 0, 0, stream));
     *out = &sched[count++];
     return CG_OK;
   }
@@ -1091,16 +569,16 @@ struct SchedCache {
 // descending reference count; the first `hot` ranks form tier 0, the next `hot` tier 1, ...; inside
 // a tier the columns are dealt round robin to `groups` groups, and every column behind the last
 // tier is cold.  Class = tier * groups + group.  A tier is one launch in which XCD x only reads the
-// B rows of group x % groups, sized to stay resident in that XCD's L2.  Entries are kept as one CSR
-// over (classes + 1) * rows virtual rows, virtual row c * rows + r holding the entries of row r whose
-// column has class c (cold = class `classes`).
+// B rows of group x % groups, so each XCD's private L2 keeps its own share of the hot rows.
+// Entries are kept as one CSR over (classes + 1) * rows virtual rows, virtual row c * rows + r
+// holding the entries of row r whose column has class c (cold = class `classes`).
 struct HubPlan {
   int32_t hot = 0, groups = 0, tiers = 0, seg = 0;
   int32_t classes() const { return groups * tiers; }
   int32_t *vrowptr = nullptr, *colind = nullptr;
   float *val = nullptr;
   Sched hot_sched;        // over the virtual rows of the hot classes, empty rows skipped
-  StreamTab hot_tab;      // its windows, one class per group
+  StreamTab hot_tab;      // its windows, one class per (tier, group)
   SchedCache cold_sched;  // over the cold class
   int64_t tstart[18] = {0};
   bool valid = false;
@@ -1136,18 +614,6 @@ struct CsrSide {
   }
 };
 
-// Entries per task.  A team step consumes G entries per wave instruction, so narrow outputs get
-// longer segments for the same number of steps.
-static int32_t pick_seg(const SpmmShape &s) {
-  const int t = g_tune_seg.load(std::memory_order_relaxed);
-  if (t >= 64) return t;
-  const int g = kWave / s.lpr;
-  if (g == 1) return 1024;
-  if (g_tune_stream.load(std::memory_order_relaxed) >= 0) return 512;  // a window and one task fit the LDS stage
-  if (g == 2) return 2048;
-  return 4096;
-}
-
 // ---------------------------------------------------------------------------------------------
 // hub plan construction
 // ---------------------------------------------------------------------------------------------
@@ -1180,19 +646,19 @@ __global__ __launch_bounds__(kSpmmThreads) void col_class_kernel(const int32_t *
 
 __global__ __launch_bounds__(kSpmmThreads) void entry_class_kernel(const int32_t *__restrict__ colind, int64_t nnz,
                                                                    const int32_t *__restrict__ cls,
-                                                                   int32_t *__restrict__ out) {
+                                                                   int32_t *__restrict__ out,
+                                                                   int32_t *__restrict__ pos) {
   const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
-  if (k < nnz) out[k] = cls[colind[k]];
+  if (k < nnz) {
+    out[k] = cls[colind[k]];
+    pos[k] = (int32_t)k;  // position in the original CSR, carried through the sort
+  }
 }
 
-__global__ __launch_bounds__(kSpmmThreads) void entry_finish_kernel(const int32_t *__restrict__ cls_sorted,
-                                                                    const int32_t *__restrict__ row_sorted,
-                                                                    const int32_t *__restrict__ pos, int64_t nnz,
-                                                                    int32_t rows, const int32_t *__restrict__ colind,
-                                                                    const float *__restrict__ val,
-                                                                    int32_t *__restrict__ vrow,
-                                                                    int32_t *__restrict__ colind2,
-                                                                    float *__restrict__ val2) {
+__global__ __launch_bounds__(kSpmmThreads) void entry_finish_kernel(
+    const int32_t *__restrict__ cls_sorted, const int32_t *__restrict__ row_sorted, const int32_t *__restrict__ pos,
+    int64_t nnz, int32_t rows, const int32_t *__restrict__ colind, const float *__restrict__ val,
+    int32_t *__restrict__ vrow, int32_t *__restrict__ colind2, float *__restrict__ val2) {
   const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (k < nnz) {
     const int32_t p = pos[k];
@@ -1200,11 +666,6 @@ __global__ __launch_bounds__(kSpmmThreads) void entry_finish_kernel(const int32_
     colind2[k] = colind[p];
     val2[k] = val[p];
   }
-}
-
-__global__ __launch_bounds__(kSpmmThreads) void hub_iota_kernel(int32_t *__restrict__ out, int64_t count) {
-  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
-  if (k < count) out[k] = (int32_t)k;
 }
 
 __global__ __launch_bounds__(kSpmmThreads) void csr_rows_kernel(const int32_t *__restrict__ rowptr, int32_t n,
@@ -1234,7 +695,7 @@ static int build_hub(CsrSide &s, int32_t hot, int32_t groups, int32_t tiers, int
   int32_t *cls = nullptr;
   CG_TRY(tmp.alloc((void **)&count, (size_t)m * 4));
   CG_TRY(tmp.alloc((void **)&cls, (size_t)m * 4));
-  CG_HIP(hipMemsetAsync(count, 0, (size_t)m * 4, stream));
+  CG_TRY(fill_u32(count, m, 0u, stream));
   col_count_kernel<<<ge, kSpmmThreads, 0, stream>>>(s.colind, nnz, count);
   CG_LAUNCH_CHECK();
   {
@@ -1244,11 +705,10 @@ static int build_hub(CsrSide &s, int32_t hot, int32_t groups, int32_t tiers, int
       CG_TRY(tmp.alloc((void **)&buf.payload[i], (size_t)m * 4));
       CG_TRY(tmp.alloc((void **)&buf.key_b[i], (size_t)m * 4));  // no minor key: carried, never sorted on
     }
-    // the largest possible count is the number of rows (duplicate-free) or nnz in general
     const uint32_t maxcount = (uint32_t)(nnz < 0x7fffffffLL ? nnz : 0x7fffffffLL);
     col_key_kernel<<<gm, kSpmmThreads, 0, stream>>>(count, m, maxcount, buf.key_a[0], buf.payload[0]);
     CG_LAUNCH_CHECK();
-    CG_HIP(hipMemsetAsync(buf.key_b[0], 0, (size_t)m * 4, stream));
+    CG_TRY(fill_u32((uint32_t *)buf.key_b[0], m, 0u, stream));
     int set = 0;
     CG_TRY(radix_sort_pairs(buf, m, bits_for((int32_t)(maxcount < 0x7ffffffeu ? maxcount + 1 : 0x7fffffff)), 0, &set,
                             stream));
@@ -1270,15 +730,13 @@ static int build_hub(CsrSide &s, int32_t hot, int32_t groups, int32_t tiers, int
       CG_TRY(tmp2.alloc((void **)&buf.key_b[i], (size_t)nnz * 4));
       CG_TRY(tmp2.alloc((void **)&buf.payload[i], (size_t)nnz * 4));
     }
-    entry_class_kernel<<<ge, kSpmmThreads, 0, stream>>>(s.colind, nnz, cls, buf.key_a[0]);
+    entry_class_kernel<<<ge, kSpmmThreads, 0, stream>>>(s.colind, nnz, cls, buf.key_a[0], buf.payload[0]);
     CG_LAUNCH_CHECK();
     if (n > 0) {
       csr_rows_kernel<<<(unsigned)ceil_div64((int64_t)n * kWave, kSpmmThreads), kSpmmThreads, 0, stream>>>(
           s.rowptr, n, buf.key_b[0]);
       CG_LAUNCH_CHECK();
     }
-    hub_iota_kernel<<<ge, kSpmmThreads, 0, stream>>>(buf.payload[0], nnz);  // position in the original CSR
-    CG_LAUNCH_CHECK();
     int set = 0;
     CG_TRY(radix_sort_pairs(buf, nnz, bits_for(nclass + 1), 0, &set, stream));
     entry_finish_kernel<<<ge, kSpmmThreads, 0, stream>>>(buf.key_a[set], buf.key_b[set], buf.payload[set], nnz, n,
@@ -1289,7 +747,8 @@ static int build_hub(CsrSide &s, int32_t hot, int32_t groups, int32_t tiers, int
   CG_TRY(launch_rowptr(vrow, nnz, (int32_t)vrows, h.vrowptr, stream));
 
   // 3. tasks of the hot classes (empty virtual rows get none); the cold class is scheduled on demand
-  CG_TRY(make_sched(h.vrowptr, nclass * n, seg, 1, h.hot_sched, stream));
+  Alloc owned;
+  CG_TRY(make_sched(h.vrowptr, nclass * n, seg, 1, h.hot_sched, owned, false, 0, 0, stream));
   {
     int32_t t[18];
     for (int g = 0; g <= nclass; ++g)
@@ -1305,146 +764,67 @@ static int build_hub(CsrSide &s, int32_t hot, int32_t groups, int32_t tiers, int
   return CG_OK;
 }
 
-// C[r, :] += sum of the partial rows of r's hot tasks, in (group, segment) order.  One wavefront
-// per row: lane g fetches the task range of group g, then the lanes sweep the row's columns with
-// the partial rows of all tasks in flight together.
-template <int NC>  // classes the unrolled loops cover (nclass <= NC)
-__global__ __launch_bounds__(kSpmmThreads) void hub_reduce_kernel(const int32_t *__restrict__ tbase, int32_t n,
-                                                                  int32_t nclass, const float *__restrict__ P,
-                                                                  float *__restrict__ C, int64_t ldc, int32_t f) {
-  const int64_t r = ((int64_t)blockIdx.x * kSpmmThreads + threadIdx.x) / kWave;
-  const int lane = threadIdx.x & (kWave - 1);
-  if (r >= n) return;
-  int32_t t0 = 0, t1 = 0;
-  if (lane < nclass) {
-    const int64_t v = (int64_t)lane * n + r;
-    t0 = tbase[v];
-    t1 = tbase[v + 1];
-  }
-  int32_t first[NC], count[NC];
-  int32_t total = 0;
-#pragma unroll
-  for (int g = 0; g < NC; ++g) {
-    first[g] = __builtin_amdgcn_readlane(t0, g);
-    count[g] = __builtin_amdgcn_readlane(t1, g) - first[g];
-    total += count[g];
-  }
-  if (total == 0) return;
-  float *crow = C + r * ldc;
-  for (int32_t c0 = 0; c0 < f; c0 += kWave) {
-    const int32_t col = c0 + lane;
-    if (col < f) {
-      float s = 0.f;
-#pragma unroll
-      for (int g = 0; g < NC; ++g) {
-        const float *p = P + (int64_t)first[g] * f + col;
-        if (count[g] == 1) {
-          s += p[0];
-        } else {
-          for (int32_t t = 0; t < count[g]; ++t) s += p[(int64_t)t * f];
-        }
-      }
-      crow[col] += s;
-    }
-  }
-}
+// ---------------------------------------------------------------------------------------------
+// products
+// ---------------------------------------------------------------------------------------------
+struct DenseOps {
+  const float *B;
+  int64_t ldb;
+  float *C;
+  int64_t ldc;
+  int32_t f;
+  float beta;
+};
 
-std::atomic<int> g_tune_hub{0}, g_tune_hub_kb{0}, g_tune_hub_groups{0}, g_tune_hub_tiers{0};
-
-// stored entries after which a new window starts
-static int32_t window_entries() {
-  const int w = g_tune_win.load(std::memory_order_relaxed);
-  return w >= 64 ? w : 512;
-}
-
-static void fill_args(SpmmArgs &a, const int32_t *rowptr, const int32_t *colind, const float *val, const Sched *sc,
-                      int32_t cols, const float *B, int64_t ldb, float *C, int64_t ldc, int32_t f, float beta,
-                      const SpmmPlan &plan) {
-  a.rowptr = rowptr;
-  a.colind = colind;
-  a.val = val;
-  a.task_row = sc->task_row;
-  a.tbase = sc->tbase;
-  a.pbase = sc->pbase;
-  a.ntasks = sc->ntasks;
-  a.seg = sc->seg;
-  a.m = cols;
-  a.B = B;
-  a.ldb = ldb;
-  a.C = C;
-  a.ldc = ldc;
-  a.f = f;
-  a.beta = beta;
-  a.tiles = plan.tiles;
-  a.tile_slots = plan.tile_slots;
-  a.groups = 1;
-  a.P = nullptr;
-}
-
-// Plain handle path for one column range: row-segment tasks over (rowptr, colind, val).
-static int spmm_plain(const int32_t *rowptr, const int32_t *colind, const float *val, int32_t rows, int32_t cols,
-                      SchedCache &cache, int vec, const float *B, int64_t ldb, float *C, int64_t ldc, int32_t f,
-                      float beta, int prof_tag, hipStream_t stream) {
-  SpmmPlan plan = plan_range(vec, f);
-  if (plan.shape.chunks > kMaxChunks) {  // tiling was tuned down: fall back to 8 tiles
-    plan.tiles = 8;
-    plan.tile_slots = (f / vec + 7) / 8;
-    plan.shape = pick_shape(vec, plan.tile_slots);
-  }
+// Row-segment tasks over (rowptr, colind, val), for a column range one launch can cover.
+static int spmm_plain(const int32_t *rowptr, const int32_t *colind, const float *val, int32_t rows, int64_t nnz,
+                      SchedCache &cache, int vec, const DenseOps &d, int prof_tag, hipStream_t stream) {
+  const SpmmShape shape = pick_shape(vec, d.f / vec);
   Sched *sc = nullptr;
-  CG_TRY(cache.get(rowptr, rows, pick_seg(plan.shape), &sc, stream));
-  SpmmArgs a{};
-  fill_args(a, rowptr, colind, val, sc, cols, B, ldb, C, ldc, f, beta, plan);
+  CG_TRY(cache.get(rowptr, rows, pick_seg(shape), &sc, stream));
+  StreamTab &tab = cache.tab_of(sc);
+  const int32_t S = window_entries();
+  if (tab.S != S) {
+    const int64_t first[2] = {0, sc->ntasks};
+    Alloc owned;
+    CG_TRY(build_stream(*sc, rowptr, rows, false, 1, first, S, nnz, tab, owned, false, stream));
+  }
+  StreamArgs sa{};
+  sa.task_start = tab.task_start;
+  sa.task_dst = tab.task_dst;
+  sa.wstart = tab.wstart;
+  sa.colind = colind;
+  sa.val = val;
+  sa.win_first[0] = 0;
+  sa.win_first[1] = tab.nwin;
+  sa.groups = 1;
+  sa.B = d.B;
+  sa.ldb = d.ldb;
+  sa.C = d.C;
+  sa.ldc = d.ldc;
+  sa.f = d.f;
+  sa.beta = d.beta;
   if (sc->nslots > 0) {
     void *p = nullptr;
-    CG_TRY(scratch_get(stream, kSlotA, (size_t)sc->nslots * f * sizeof(float), &p));
-    a.P = (float *)p;
+    CG_TRY(scratch_get(stream, kSlotA, (size_t)sc->nslots * d.f * sizeof(float), &p));
+    sa.P = (float *)p;
   }
-  const bool narrow = plan.shape.lpr < kWave;
-  if (plan.tiles == 1 && g_tune_stream.load(std::memory_order_relaxed) >= 0 &&
-      (!narrow || (sc->seg <= 512 && window_entries() <= 512))) {
-    // stream windows of consecutive tasks
-    StreamTab &tab = cache.tab_of(sc);
-    const int32_t S = window_entries();
-    if (tab.S != S) {
-      const int64_t first[2] = {0, sc->ntasks};
-      CG_TRY(build_stream(*sc, rowptr, rows, false, 1, first, S, tab, stream));
-    }
-    StreamArgs sa{};
-    sa.task_start = tab.task_start;
-    sa.task_dst = tab.task_dst;
-    sa.wstart = tab.wstart;
-    sa.colind = colind;
-    sa.val = val;
-    sa.win_first[0] = 0;
-    sa.win_first[1] = tab.nwin;
-    sa.groups = 1;
-    sa.B = B;
-    sa.ldb = ldb;
-    sa.C = C;
-    sa.ldc = ldc;
-    sa.P = a.P;
-    sa.f = f;
-    sa.beta = beta;
+  {
     ProfScope prof("spmm_rowseg", prof_tag, stream);
-    if (narrow) CG_TRY(launch_stream_narrow(vec, plan.shape.lpr, sa, stream));
-    else CG_TRY(launch_stream_wide(vec, plan.shape.chunks, sa, stream));
-  } else {
-    ProfScope prof("spmm_rowseg", prof_tag, stream);
-    CG_TRY((launch_shape<kModeTable>(plan.shape, a, stream)));
+    CG_TRY(launch_stream(shape, sa, stream));
   }
   if (sc->nmulti > 0) {
     ProfScope prof("spmm_reduce", prof_tag, stream);
-    const int64_t threads = sc->nmulti * (int64_t)f;
+    const int64_t threads = sc->nmulti * (int64_t)d.f;
     spmm_reduce_kernel<<<(unsigned)ceil_div64(threads, kSpmmThreads), kSpmmThreads, 0, stream>>>(
-        sc->multi_rows, sc->nmulti, rowptr, sc->pbase, sc->seg, a.P, C, ldc, f, beta);
+        sc->multi_rows, sc->nmulti, nullptr, rowptr, sc->pbase, sc->seg, sa.P, d.C, d.ldc, d.f, d.beta, 0);
     CG_LAUNCH_CHECK();
   }
   return CG_OK;
 }
 
 // Should a product of this width over this matrix go through a hub plan?  It pays when a row of B
-// is many cache lines (the gather dominates) and rows hold enough hot entries per group that the
+// is several cache lines (the gather dominates) and rows hold enough hot entries per group that the
 // partial rows they cost are small against the gathers they turn into L2 hits.
 static bool want_hub(const CsrSide &s, int32_t f) {
   const int t = g_tune_hub.load(std::memory_order_relaxed);
@@ -1454,8 +834,8 @@ static bool want_hub(const CsrSide &s, int32_t f) {
   return f >= 128 && s.nnz / s.rows >= 128;
 }
 
-static int spmm_hub(CsrSide &s, int vec, const float *B, int64_t ldb, float *C, int64_t ldc, int32_t f, float beta,
-                    hipStream_t stream) {
+static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream) {
+  const int32_t f = d.f;
   int groups = g_tune_hub_groups.load(std::memory_order_relaxed);
   if (groups != 1 && groups != 2 && groups != 4 && groups != 8) groups = 8;
   int tiers = g_tune_hub_tiers.load(std::memory_order_relaxed);
@@ -1468,72 +848,58 @@ static int spmm_hub(CsrSide &s, int vec, const float *B, int64_t ldb, float *C, 
   if (per_group < 1) per_group = 1;
   int64_t hot = per_group * groups;  // columns per tier
   if (hot > s.cols) hot = s.cols;
-  // hot tasks use full-wave teams on the whole width with one dword per lane and chunk when the rows
-  // are not 16-byte aligned: that is the fastest gather of L2-resident rows
+  // hot tasks of a wide product use one dword per lane and chunk when the rows are not 16-byte
+  // aligned: that is the fastest gather of L2-resident rows
   const int hot_vec = (vec == 4 || f / vec <= kWave) ? vec : 1;
-  SpmmPlan hplan;
-  hplan.tiles = 1;
-  hplan.tile_slots = f / hot_vec;
-  hplan.shape = pick_shape(hot_vec, hplan.tile_slots);
-  const int32_t seg = pick_seg(hplan.shape);
+  const SpmmShape hshape = pick_shape(hot_vec, f / hot_vec);
+  const int32_t seg = pick_seg(hshape);
   if (!s.hub.valid || s.hub.hot != (int32_t)hot || s.hub.groups != groups || s.hub.tiers != tiers || s.hub.seg != seg)
     CG_TRY(build_hub(s, (int32_t)hot, groups, tiers, seg, stream));
   HubPlan &h = s.hub;
   const int32_t n = s.rows;
   const int32_t nclass = h.classes();
   // 1. cold class straight into C
-  CG_TRY(spmm_plain(h.vrowptr + (int64_t)nclass * n, h.colind, h.val, n, s.cols, h.cold_sched, vec, B, ldb, C, ldc, f,
-                    beta, f, stream));
+  CG_TRY(spmm_plain(h.vrowptr + (int64_t)nclass * n, h.colind, h.val, n, s.nnz, h.cold_sched, vec, d, f, stream));
   // 2. hot classes, one launch per tier: every task writes a partial row
   const int64_t hot_tasks = h.hot_sched.ntasks;
   if (hot_tasks == 0) return CG_OK;
   void *p = nullptr;
   CG_TRY(scratch_get(stream, kSlotC, (size_t)hot_tasks * f * sizeof(float), &p));
-  const bool hnarrow = hplan.shape.lpr < kWave;
-  const bool streaming =
-      g_tune_stream.load(std::memory_order_relaxed) >= 0 && (!hnarrow || (seg <= 512 && window_entries() <= 512));
-  if (streaming) {
-    const int32_t S = window_entries();
-    if (h.hot_tab.S != S || h.hot_tab.groups != nclass)
-      CG_TRY(build_stream(h.hot_sched, h.vrowptr, nclass * n, true, nclass, h.tstart, S, h.hot_tab, stream));
+  const int32_t S = window_entries();
+  if (h.hot_tab.S != S || h.hot_tab.groups != nclass) {
+    Alloc owned;
+    CG_TRY(build_stream(h.hot_sched, h.vrowptr, nclass * n, true, nclass, h.tstart, S, s.nnz, h.hot_tab, owned, false,
+                        stream));
   }
   for (int t = 0; t < tiers; ++t) {
+    StreamArgs sa{};
+    sa.task_start = h.hot_tab.task_start;
+    sa.task_dst = h.hot_tab.task_dst;
+    sa.wstart = h.hot_tab.wstart;
+    sa.colind = h.colind;
+    sa.val = h.val;
+    for (int g = 0; g <= groups; ++g) sa.win_first[g] = h.hot_tab.win_first[t * groups + g];
+    sa.groups = groups;
+    sa.B = d.B;
+    sa.ldb = d.ldb;
+    sa.C = d.C;
+    sa.ldc = d.ldc;
+    sa.P = (float *)p;
+    sa.f = f;
+    sa.beta = 0.f;
     ProfScope prof("spmm_hub_hot", f, stream);
-    if (streaming) {
-      StreamArgs sa{};
-      sa.task_start = h.hot_tab.task_start;
-      sa.task_dst = h.hot_tab.task_dst;
-      sa.wstart = h.hot_tab.wstart;
-      sa.colind = h.colind;
-      sa.val = h.val;
-      for (int g = 0; g <= groups; ++g) sa.win_first[g] = h.hot_tab.win_first[t * groups + g];
-      sa.groups = groups;
-      sa.B = B;
-      sa.ldb = ldb;
-      sa.C = C;
-      sa.ldc = ldc;
-      sa.P = (float *)p;
-      sa.f = f;
-      sa.beta = 0.f;
-      if (hnarrow) CG_TRY(launch_stream_narrow(hot_vec, hplan.shape.lpr, sa, stream));
-      else CG_TRY(launch_stream_wide(hot_vec, hplan.shape.chunks, sa, stream));
-    } else {
-      SpmmArgs a{};
-      fill_args(a, h.vrowptr, h.colind, h.val, &h.hot_sched, s.cols, B, ldb, C, ldc, f, 0.f, hplan);
-      a.P = (float *)p;
-      a.groups = groups;
-      for (int g = 0; g <= groups; ++g) a.tstart[g] = h.tstart[t * groups + g];
-      CG_TRY((launch_shape<kModeHub>(hplan.shape, a, stream)));
-    }
+    CG_TRY(launch_stream(hshape, sa, stream));
   }
   // 3. fold the partial rows into C
   {
     ProfScope prof("spmm_hub_reduce", f, stream);
     const unsigned rgrid = (unsigned)ceil_div64((int64_t)n * kWave, kSpmmThreads);
     if (nclass <= 8)
-      hub_reduce_kernel<8><<<rgrid, kSpmmThreads, 0, stream>>>(h.hot_sched.tbase, n, nclass, (const float *)p, C, ldc, f);
+      hub_reduce_kernel<8><<<rgrid, kSpmmThreads, 0, stream>>>(h.hot_sched.tbase, n, nclass, (const float *)p, d.C,
+                                                               d.ldc, f);
     else
-      hub_reduce_kernel<16><<<rgrid, kSpmmThreads, 0, stream>>>(h.hot_sched.tbase, n, nclass, (const float *)p, C, ldc, f);
+      hub_reduce_kernel<16><<<rgrid, kSpmmThreads, 0, stream>>>(h.hot_sched.tbase, n, nclass, (const float *)p, d.C,
+                                                                d.ldc, f);
     CG_LAUNCH_CHECK();
   }
   return CG_OK;
@@ -1543,21 +909,96 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
                      hipStream_t stream) {
   if (s.rows == 0) return CG_OK;
   const int vec = pick_vec(f, B, ldb, C, ldc);
-  const int32_t cap = range_cap(vec) * 8;  // 8 tiles of kMaxChunks chunks
-  if (f <= range_cap(vec == 4 ? 4 : 1) && want_hub(s, f)) return spmm_hub(s, vec, B, ldb, C, ldc, f, beta, stream);
+  const int32_t cap = range_cap(vec);
+  if (f <= range_cap(vec == 4 ? 4 : 1) && want_hub(s, f)) {
+    const DenseOps d{B, ldb, C, ldc, f, beta};
+    return spmm_hub(s, vec, d, stream);
+  }
+  for (int32_t f0 = 0; f0 < f; f0 += cap) {  // wider outputs take several launches over column ranges
+    const int32_t ft = f - f0 < cap ? f - f0 : cap;
+    const DenseOps d{B + f0, ldb, C + f0, ldc, ft, beta};
+    CG_TRY(spmm_plain(s.rowptr, s.colind, s.val, s.rows, s.nnz, s.sched, vec, d, f, stream));
+  }
+  return CG_OK;
+}
+
+// One-shot product from row-sorted COO: rowptr, schedule and window tables are rebuilt in a
+// scratch arena on every call, as device work on `stream` only (no allocation once the scratch
+// has grown, no host round trip: table sizes are bounds, the exact counts stay on the device).
+static int spmm_coo_oneshot(const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz, int32_t n,
+                            int32_t m, const float *B, int64_t ldb, float *C, int64_t ldc, int32_t f, float beta,
+                            hipStream_t stream) {
+  const int vec = pick_vec(f, B, ldb, C, ldc);
+  const int32_t cap = range_cap(vec);
+  const int32_t fmax = f < cap ? f : cap;
+  // every column range uses the tables of the first (widest) one; a narrower last range only
+  // means shorter teams over the same tasks, which is valid as long as the segment length fits
+  const SpmmShape shape0 = pick_shape(vec, fmax / vec);
+  int32_t seg = pick_seg(shape0);
+  if (f > cap && (f % cap) / vec <= kWave && seg > 512) seg = 512;  // the tail range runs narrow teams
+  const int32_t S = window_entries();
+  const int64_t max_multi = nnz / seg + 1;
+  const int64_t max_tasks = (int64_t)n + nnz / seg + 1;
+  const int64_t wcap = ceil_div64(max_tasks, 64) + nnz / S + 2;
+  // arena: rowptr, tbase/pbase/mbase, task_row, multi_rows, task_start/dst, flags/index, wstart
+  const size_t words = 4 * (size_t)(n + 1) + (size_t)max_tasks + (size_t)max_multi + 4 * (size_t)(max_tasks + 1) +
+                       (size_t)(wcap + 1) + 16;
+  const size_t arena_bytes = words * 4 + 32 * 256;
+  void *abase = nullptr;
+  CG_TRY(scratch_get(stream, kSlotB, arena_bytes, &abase));
+  Alloc mem;
+  mem.base = (char *)abase;
+  mem.cap = arena_bytes;
+  int32_t *rowptr = nullptr;
+  CG_TRY(mem.get((void **)&rowptr, (size_t)(n + 1) * 4));
+  // rows the compression never reaches (only possible for unsorted input) stay 0
+  CG_TRY(fill_u32((uint32_t *)rowptr, (int64_t)n + 1, 0u, stream));
+  CG_TRY(launch_rowptr(d_row, nnz, n, rowptr, stream));
+  Sched sc;
+  CG_TRY(make_sched(rowptr, n, seg, 0, sc, mem, true, max_tasks, max_multi, stream));
+  StreamTab tab;
+  const int64_t first[2] = {0, max_tasks};
+  CG_TRY(build_stream(sc, rowptr, n, false, 1, first, S, nnz, tab, mem, true, stream));
+  const int64_t pslots = 2 * max_multi;
+  void *p = nullptr;
+  CG_TRY(scratch_get(stream, kSlotA, (size_t)pslots * fmax * sizeof(float), &p));
   for (int32_t f0 = 0; f0 < f; f0 += cap) {
     const int32_t ft = f - f0 < cap ? f - f0 : cap;
-    CG_TRY(spmm_plain(s.rowptr, s.colind, s.val, s.rows, s.cols, s.sched, vec, B + f0, ldb, C + f0, ldc, ft, beta, f,
-                      stream));
+    const SpmmShape shape = pick_shape(vec, ft / vec);
+    StreamArgs sa{};
+    sa.task_start = tab.task_start;
+    sa.task_dst = tab.task_dst;
+    sa.wstart = tab.wstart;
+    sa.colind = d_col;
+    sa.val = d_val;
+    sa.win_first[0] = 0;
+    sa.win_first[1] = tab.nwin;
+    sa.groups = 1;
+    sa.clamp_m = m;
+    sa.p_cap = pslots;
+    sa.d_nwin = tab.d_nwin;
+    sa.B = B + f0;
+    sa.ldb = ldb;
+    sa.C = C + f0;
+    sa.ldc = ldc;
+    sa.P = (float *)p;
+    sa.f = ft;
+    sa.beta = beta;
+    {
+      ProfScope prof("spmm_rowseg", f, stream);
+      CG_TRY(launch_stream(shape, sa, stream));
+    }
+    ProfScope prof("spmm_reduce", f, stream);
+    const int64_t threads = max_multi * (int64_t)ft;
+    spmm_reduce_kernel<<<(unsigned)ceil_div64(threads, kSpmmThreads), kSpmmThreads, 0, stream>>>(
+        sc.multi_rows, max_multi, sc.d_counts + 2, rowptr, sc.pbase, seg, (const float *)p, C + f0, ldc, ft, beta,
+        pslots);
+    CG_LAUNCH_CHECK();
   }
   return CG_OK;
 }
 
 }  // namespace cg
-
-namespace cg {
-extern std::atomic<int> g_tune_dense_mfma;  // dense.hip
-}
 
 struct cg_csr {
   int device = 0;
@@ -1568,6 +1009,7 @@ struct cg_csr {
 };
 
 namespace cg {
+
 static int side_alloc(CsrSide &s, int32_t rows, int32_t cols, int64_t nnz) {
   s.rows = rows;
   s.cols = cols;
@@ -1581,7 +1023,7 @@ static int side_alloc(CsrSide &s, int32_t rows, int32_t cols, int64_t nnz) {
 static int side_max_degree(CsrSide &s, hipStream_t stream) {
   void *d = nullptr;
   CG_TRY(scratch_get(stream, kSlotB, sizeof(int), &d));
-  CG_HIP(hipMemsetAsync(d, 0, sizeof(int), stream));
+  CG_TRY(fill_u32((uint32_t *)d, 1, 0u, stream));
   if (s.rows > 0) {
     max_degree_kernel<<<(unsigned)ceil_div64(s.rows, kSpmmThreads), kSpmmThreads, 0, stream>>>(s.rowptr, s.rows,
                                                                                               (int *)d);
@@ -1623,6 +1065,7 @@ static int csr_create(cg_csr *h, const int32_t *d_row, const int32_t *d_col, con
   CG_HIP(hipStreamSynchronize(stream));
   return CG_OK;
 }
+
 }  // namespace cg
 
 extern "C" {
@@ -1632,39 +1075,13 @@ int cg_spmm_coo(const int32_t *d_row, const int32_t *d_col, const float *d_val, 
   using namespace cg;
   hipStream_t stream = (hipStream_t)stream_;
   if (nnz < 0 || n < 0 || m < 0) CG_FAIL(CG_ERR_SIZE, "cg_spmm_coo: negative size");
-  if (nnz > 0x7fffffffLL - 1 || n == 0x7fffffff) CG_FAIL(CG_ERR_OVERFLOW, "cg_spmm_coo: nnz=%lld n=%d exceed int32", (long long)nnz, n);
+  if (nnz > 0x7fffffffLL - 1 || n == 0x7fffffff)
+    CG_FAIL(CG_ERR_OVERFLOW, "cg_spmm_coo: nnz=%lld n=%d exceed int32", (long long)nnz, n);
   if (nnz > 0 && (!d_row || !d_col || !d_val)) CG_FAIL(CG_ERR_NULL, "cg_spmm_coo: null sparse operand");
   CG_TRY(check_dense("cg_spmm_coo", d_B, ldb, d_C, ldc, f, m, n));
   if (n == 0) return CG_OK;
   if (nnz > 0 && m == 0) CG_FAIL(CG_ERR_SIZE, "cg_spmm_coo: nnz > 0 with m == 0");
-  void *d_rowptr = nullptr;
-  CG_TRY(scratch_get(stream, kSlotB, (size_t)(n + 1) * sizeof(int32_t), &d_rowptr));
-  // rows the compression never reaches (only possible for unsorted input) stay 0 -> empty or
-  // in-range spans, never an out-of-bounds read
-  CG_HIP(hipMemsetAsync(d_rowptr, 0, (size_t)(n + 1) * sizeof(int32_t), stream));
-  CG_TRY(launch_rowptr(d_row, nnz, n, (int32_t *)d_rowptr, stream));
-  const int vec = pick_vec(f, d_B, ldb, d_C, ldc);
-  const int32_t cap = range_cap(vec);
-  for (int32_t f0 = 0; f0 < f; f0 += cap) {
-    const int32_t ft = f - f0 < cap ? f - f0 : cap;
-    SpmmArgs a{};
-    a.rowptr = (const int32_t *)d_rowptr;
-    a.colind = d_col;
-    a.val = d_val;
-    a.ntasks = n;
-    a.seg = 0;
-    a.m = m;
-    a.B = d_B + f0;
-    a.ldb = ldb;
-    a.C = d_C + f0;
-    a.ldc = ldc;
-    a.f = ft;
-    a.beta = beta;
-    a.tiles = 1;
-    a.tile_slots = ft / vec;
-    CG_TRY((launch_shape<kModeRows>(pick_shape(vec, ft / vec), a, stream)));
-  }
-  return CG_OK;
+  return spmm_coo_oneshot(d_row, d_col, d_val, nnz, n, m, d_B, ldb, d_C, ldc, f, beta, stream);
 }
 
 int cg_csr_create(cg_csr_t **out, const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz,
@@ -1712,15 +1129,13 @@ int cg_csr_spmm(cg_csr_t *h, int transpose, const float *d_B, int64_t ldb, float
 int cg_tune_set(const char *key, int value) {
   if (!key) CG_FAIL(CG_ERR_NULL, "cg_tune_set: key is NULL");
   if (!strcmp(key, "spmm_seg")) cg::g_tune_seg.store(value);
-  else if (!strcmp(key, "spmm_tiles")) cg::g_tune_tiles.store(value);
   else if (!strcmp(key, "spmm_vec")) cg::g_tune_vec.store(value);
-  else if (!strcmp(key, "spmm_hub")) cg::g_tune_hub.store(value);
-  else if (!strcmp(key, "spmm_stream")) cg::g_tune_stream.store(value);
-  else if (!strcmp(key, "dense_mfma")) cg::g_tune_dense_mfma.store(value);
   else if (!strcmp(key, "spmm_win")) cg::g_tune_win.store(value);
+  else if (!strcmp(key, "spmm_hub")) cg::g_tune_hub.store(value);
   else if (!strcmp(key, "spmm_hub_kb")) cg::g_tune_hub_kb.store(value);
   else if (!strcmp(key, "spmm_hub_groups")) cg::g_tune_hub_groups.store(value);
   else if (!strcmp(key, "spmm_hub_tiers")) cg::g_tune_hub_tiers.store(value);
+  else if (!strcmp(key, "dense_mfma")) cg::g_tune_dense_mfma.store(value);
   else CG_FAIL(CG_ERR_UNSUPPORTED, "cg_tune_set: unknown key %s", key);
   return CG_OK;
 }

@@ -1,0 +1,460 @@
+// Device kernels of the CSR SpMM  C[rows,f] = beta*C + A*B  for gfx950 (64-wide wavefronts).
+//
+// Replaces cusparseSpMM(CSRMM_ALG1, alpha = 1, beta = 1) of the reference operator
+// (sparse-extension/sparse_coo_tensor.cu:215-226) on row-major B and C, without atomics.
+//
+// Work decomposition
+//   task    = a row segment: at most `seg` consecutive stored entries of one row.  Rows of degree
+//             <= seg are one task and go straight to C; longer rows write one partial row per task
+//             that spmm_reduce_kernel adds in segment order.
+//   team    = LPR lanes that together cover the f output columns, VEC floats per lane and chunk.
+//             A wavefront holds G = 64 / LPR teams.
+//   window  = up to 64 consecutive tasks (a new window every S stored entries).  Tasks are
+//             contiguous in the entry stream, so the wavefront that takes a window reads one
+//             contiguous piece of (colind, val) and pays start-up latency once per window.
+// Summation order is a function of the matrix, f and the schedule only: results are bit-identical
+// from run to run.
+#pragma once
+#include "common.h"
+
+namespace cg {
+
+constexpr int kSpmmThreads = 256;
+constexpr int kWavesPerBlock = kSpmmThreads / kWave;
+
+template <int VEC>
+struct VecT;
+template <>
+struct VecT<1> {
+  typedef float type;
+};
+template <>
+struct VecT<2> {
+  typedef float2 type;
+};
+template <>
+struct VecT<4> {
+  typedef float4 type;
+};
+
+template <int VEC>
+__device__ __forceinline__ void load_vec(const float *p, float (&r)[VEC]) {
+  typedef typename VecT<VEC>::type V;
+  const V t = *reinterpret_cast<const V *>(p);
+  const float *tp = reinterpret_cast<const float *>(&t);
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) r[i] = tp[i];
+}
+
+template <int VEC>
+__device__ __forceinline__ void store_vec(float *p, const float (&r)[VEC]) {
+  typedef typename VecT<VEC>::type V;
+  V t;
+  float *tp = reinterpret_cast<float *>(&t);
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) tp[i] = r[i];
+  *reinterpret_cast<V *>(p) = t;
+}
+
+// C[row, :] = beta*C[row, :] + sum over the row's partial rows, in segment order.
+__global__ __launch_bounds__(kSpmmThreads) void spmm_reduce_kernel(const int32_t *__restrict__ multi_rows,
+                                                                   int64_t nmulti_host,
+                                                                   const uint32_t *__restrict__ d_nmulti,
+                                                                   const int32_t *__restrict__ rowptr,
+                                                                   const int32_t *__restrict__ pbase, int32_t seg,
+                                                                   const float *__restrict__ P, float *__restrict__ C,
+                                                                   int64_t ldc, int32_t f, float beta,
+                                                                   int64_t p_cap) {
+  const int64_t idx = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  const int64_t mr = idx / f;
+  const int32_t col = (int32_t)(idx % f);
+  int64_t nmulti = nmulti_host;  // capacity of multi_rows when the exact count is on the device
+  if (d_nmulti && (int64_t)*d_nmulti < nmulti) nmulti = (int64_t)*d_nmulti;
+  if (mr >= nmulti) return;
+  const int32_t row = multi_rows[mr];
+  const int32_t deg = rowptr[row + 1] - rowptr[row];
+  const int32_t nseg = (deg + seg - 1) / seg;
+  if (p_cap > 0 && (int64_t)pbase[row] + nseg > p_cap) return;  // only a malformed (unsorted) input gets here
+  const float *p = P + (int64_t)pbase[row] * f + col;
+  float s = 0.f;
+  for (int32_t i = 0; i < nseg; ++i) s += p[(int64_t)i * f];
+  float *c = C + (int64_t)row * ldc + col;
+  *c = beta != 0.f ? fmaf(beta, *c, s) : s;
+}
+
+struct StreamArgs {
+  const int32_t *task_start, *task_dst, *wstart;
+  const int32_t *colind;
+  const float *val;
+  int64_t win_first[9];
+  int32_t groups;  // 1: windows run anywhere; 2/4/8: windows of class g run on XCDs x % groups == g
+  int32_t clamp_m;   // > 0: column indices are clamped into [0, clamp_m) (entry point that does not validate)
+  int64_t p_cap;     // > 0: partial rows with a slot >= p_cap are dropped (same entry point: keeps a
+                     // malformed, unsorted input from writing outside the partial buffer)
+  const uint32_t *d_nwin;  // groups == 1 only: when set, the number of windows is read from the device
+                           // (tables built without a host round trip; the grid is an upper bound)
+  const float *B;
+  int64_t ldb;
+  float *C;
+  int64_t ldc;
+  float *P;
+  int32_t f;
+  float beta;
+};
+
+// Full-wave teams (one stored entry per wave step, f covered by CHUNKS x 64 lanes x VEC floats).
+template <int VEC, int CHUNKS>
+__global__ __launch_bounds__(kSpmmThreads) void spmm_stream_wide_kernel(const StreamArgs a) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int x = blockIdx.x & 7;
+  const int per = 8 / a.groups;
+  const int grp = x % a.groups;
+  const int64_t lblock = (int64_t)(blockIdx.x >> 3) * per + x / a.groups;
+  const int64_t wl = lblock * kWavesPerBlock + threadIdx.x / kWave;
+  const int64_t nwin_here = a.d_nwin ? (int64_t)*a.d_nwin : a.win_first[grp + 1] - a.win_first[grp];
+  if (wl >= nwin_here) return;
+  const int32_t w = __builtin_amdgcn_readfirstlane((int32_t)(a.win_first[grp] + wl));
+  const int32_t t0 = a.wstart[w], t1 = a.wstart[w + 1];
+  const int ntask = t1 - t0;  // 1..64
+  int32_t m_end = 0, m_dst = 0;
+  if (lane < ntask) {
+    m_end = a.task_start[t0 + lane + 1];
+    m_dst = a.task_dst[t0 + lane];
+  }
+  const int32_t e_begin = a.task_start[t0];
+  const int32_t e_end = __builtin_amdgcn_readlane(m_end, ntask - 1);
+
+  const int nslots = a.f / VEC;
+  bool active[CHUNKS];
+  int64_t boff[CHUNKS];
+#pragma unroll
+  for (int ch = 0; ch < CHUNKS; ++ch) {
+    active[ch] = (ch * kWave + lane) < nslots;
+    boff[ch] = (int64_t)(ch * kWave + (active[ch] ? lane : 0)) * VEC;
+  }
+  float acc[CHUNKS][VEC];
+#pragma unroll
+  for (int ch = 0; ch < CHUNKS; ++ch)
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[ch][v] = 0.f;
+
+  constexpr int U = 4;
+  int tk = 0;
+  int32_t tbeg = e_begin;
+  int32_t tend = __builtin_amdgcn_readlane(m_end, 0);
+
+  int32_t c_next = 0;
+  float v_next = 0.f;
+  if (e_begin + lane < e_end) {
+    c_next = a.colind[e_begin + lane];
+    v_next = a.val[e_begin + lane];
+  }
+  for (int32_t base = e_begin;; base += kWave) {
+    int32_t c = c_next;
+    const float v = v_next;
+    if (a.clamp_m > 0) c = c < 0 ? 0 : (c >= a.clamp_m ? a.clamp_m - 1 : c);
+    const int32_t nb = base + kWave + lane;
+    c_next = 0;
+    v_next = 0.f;
+    if (nb < e_end) {
+      c_next = a.colind[nb];
+      v_next = a.val[nb];
+    }
+    int cnt = e_end - base;
+    cnt = cnt > kWave ? kWave : (cnt < 0 ? 0 : cnt);
+    int i = 0;
+    for (;;) {
+      while (tend == base + i) {  // the current task is complete (also true at once for an empty task)
+        const int32_t dst = __builtin_amdgcn_readlane(m_dst, tk);
+        if (dst >= 0) {
+          if (!(tend == tbeg && a.beta == 1.0f)) {  // an empty row leaves C alone when beta == 1
+            float *crow = a.C + (int64_t)dst * a.ldc;
+#pragma unroll
+            for (int ch = 0; ch < CHUNKS; ++ch) {
+              if (active[ch]) {
+                float out[VEC];
+                if (a.beta != 0.f) {
+                  float old[VEC];
+                  load_vec<VEC>(crow + boff[ch], old);
+#pragma unroll
+                  for (int q = 0; q < VEC; ++q) out[q] = fmaf(a.beta, old[q], acc[ch][q]);
+                } else {
+#pragma unroll
+                  for (int q = 0; q < VEC; ++q) out[q] = acc[ch][q];
+                }
+                store_vec<VEC>(crow + boff[ch], out);
+              }
+            }
+          }
+        } else if (a.p_cap <= 0 || (int64_t)(-(dst + 1)) < a.p_cap) {
+          float *prow = a.P + (int64_t)(-(dst + 1)) * a.f;
+#pragma unroll
+          for (int ch = 0; ch < CHUNKS; ++ch)
+            if (active[ch]) store_vec<VEC>(prow + boff[ch], acc[ch]);
+        }
+#pragma unroll
+        for (int ch = 0; ch < CHUNKS; ++ch)
+#pragma unroll
+          for (int q = 0; q < VEC; ++q) acc[ch][q] = 0.f;
+        if (++tk == ntask) return;
+        tbeg = tend;
+        tend = __builtin_amdgcn_readlane(m_end, tk);
+      }
+      if (i >= cnt) break;
+      int run = tend - base;
+      run = run < cnt ? run : cnt;
+      if (run <= i) return;  // cannot happen with monotone task starts; guarantees termination
+      for (; i + U <= run; i += U) {
+        float b[U][CHUNKS][VEC];
+        float vv[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int32_t cc = __builtin_amdgcn_readlane(c, i + u);
+          vv[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), i + u));
+          const float *brow = a.B + (int64_t)cc * a.ldb;
+#pragma unroll
+          for (int ch = 0; ch < CHUNKS; ++ch) load_vec<VEC>(brow + boff[ch], b[u][ch]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int ch = 0; ch < CHUNKS; ++ch)
+#pragma unroll
+            for (int q = 0; q < VEC; ++q) acc[ch][q] = fmaf(vv[u], b[u][ch][q], acc[ch][q]);
+      }
+      for (; i < run; ++i) {
+        const int32_t cc = __builtin_amdgcn_readlane(c, i);
+        const float vv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), i));
+        const float *brow = a.B + (int64_t)cc * a.ldb;
+        float b[CHUNKS][VEC];
+#pragma unroll
+        for (int ch = 0; ch < CHUNKS; ++ch) load_vec<VEC>(brow + boff[ch], b[ch]);
+#pragma unroll
+        for (int ch = 0; ch < CHUNKS; ++ch)
+#pragma unroll
+          for (int q = 0; q < VEC; ++q) acc[ch][q] = fmaf(vv, b[ch][q], acc[ch][q]);
+      }
+    }
+  }
+}
+
+// Teams of LPR < 64 lanes (f <= 64 * VEC floats): the window's entries and task table are staged
+// in LDS.  Long tasks (>= kLongFactor * G entries) are worked on by all G teams together (entries
+// dealt round robin, partial sums combined by the xor butterfly); the short ones are dealt to the
+// teams whole, G at a time, so rows of a few entries cost neither a butterfly nor an idle wave.
+constexpr int kNarrowLds = 1024;  // entries a window may hold (window length S plus one task, both <= 512)
+constexpr int kLongFactor = 4;
+
+template <int VEC, int LPR>
+__global__ __launch_bounds__(kSpmmThreads) void spmm_stream_narrow_kernel(const StreamArgs a) {
+  constexpr int G = kWave / LPR;
+  __shared__ int32_t s_col[kWavesPerBlock][kNarrowLds];
+  __shared__ float s_val[kWavesPerBlock][kNarrowLds];
+  __shared__ int32_t s_beg[kWavesPerBlock][kWave], s_end[kWavesPerBlock][kWave], s_dst[kWavesPerBlock][kWave];
+  __shared__ int32_t s_short[kWavesPerBlock][kWave];
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wv = threadIdx.x / kWave;
+  const int x = blockIdx.x & 7;
+  const int per = 8 / a.groups;
+  const int grp = x % a.groups;
+  const int64_t lblock = (int64_t)(blockIdx.x >> 3) * per + x / a.groups;
+  const int64_t wl = lblock * kWavesPerBlock + wv;
+  const int64_t nwin_here = a.d_nwin ? (int64_t)*a.d_nwin : a.win_first[grp + 1] - a.win_first[grp];
+  if (wl >= nwin_here) return;
+  const int32_t w = __builtin_amdgcn_readfirstlane((int32_t)(a.win_first[grp] + wl));
+  const int32_t t0 = a.wstart[w], t1 = a.wstart[w + 1];
+  const int ntask = t1 - t0;  // 1..64
+  const bool valid = lane < ntask;
+  int32_t m_beg = 0, m_end = 0, m_dst = 0;
+  if (valid) {
+    m_beg = a.task_start[t0 + lane];
+    m_end = a.task_start[t0 + lane + 1];
+    m_dst = a.task_dst[t0 + lane];
+  }
+  const int32_t e_begin = __builtin_amdgcn_readlane(m_beg, 0);
+  const int32_t e_end = __builtin_amdgcn_readlane(m_end, ntask - 1);
+  const int32_t nent = e_end - e_begin;
+  if (nent > kNarrowLds) return;  // excluded by the schedule (S + seg <= kNarrowLds); keeps LDS writes in bounds
+
+  for (int32_t k = lane; k < nent; k += kWave) {
+    int32_t c = a.colind[e_begin + k];
+    if (a.clamp_m > 0) c = c < 0 ? 0 : (c >= a.clamp_m ? a.clamp_m - 1 : c);
+    s_col[wv][k] = c;
+    s_val[wv][k] = a.val[e_begin + k];
+  }
+  const int32_t r_beg = m_beg - e_begin, r_end = m_end - e_begin;  // relative to the window
+  s_beg[wv][lane] = r_beg;
+  s_end[wv][lane] = r_end;
+  s_dst[wv][lane] = m_dst;
+  const int32_t len = r_end - r_beg;
+  const bool is_long = valid && len >= kLongFactor * G;
+  // an empty row that goes straight to C needs no work when beta == 1
+  const bool is_short = valid && !is_long && !(len == 0 && m_dst >= 0 && a.beta == 1.0f);
+
+  const int g = lane / LPR, j = lane % LPR;
+  const bool active = j * VEC < a.f;
+  const int64_t boff = active ? (int64_t)j * VEC : 0;
+  const int32_t *cw = s_col[wv];
+  const float *vw = s_val[wv];
+
+  const uint64_t short_mask = __ballot(is_short);
+  if (is_short) s_short[wv][__popcll(short_mask & ((1ull << lane) - 1ull))] = lane;
+  const int nshort = __popcll(short_mask);
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+  __builtin_amdgcn_wave_barrier();  // the staged window and tables are visible to every lane of the wave
+
+  // ---- long tasks: all teams together
+  uint64_t long_mask = __ballot(is_long);
+  while (long_mask) {
+    const int k = __builtin_ctzll(long_mask);
+    long_mask &= long_mask - 1;
+    const int32_t s = __builtin_amdgcn_readlane(r_beg, k);
+    const int32_t e = __builtin_amdgcn_readlane(r_end, k);
+    const int32_t d = __builtin_amdgcn_readlane(m_dst, k);
+    float acc[VEC];
+#pragma unroll
+    for (int q = 0; q < VEC; ++q) acc[q] = 0.f;
+    int32_t i = s + g;
+    for (; i + 3 * G < e; i += 4 * G) {
+      float b[4][VEC], vv[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int32_t cc = cw[i + u * G];
+        vv[u] = vw[i + u * G];
+        load_vec<VEC>(a.B + (int64_t)cc * a.ldb + boff, b[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int q = 0; q < VEC; ++q) acc[q] = fmaf(vv[u], b[u][q], acc[q]);
+    }
+    for (; i < e; i += G) {
+      float b[VEC];
+      const float vv = vw[i];
+      load_vec<VEC>(a.B + (int64_t)cw[i] * a.ldb + boff, b);
+#pragma unroll
+      for (int q = 0; q < VEC; ++q) acc[q] = fmaf(vv, b[q], acc[q]);
+    }
+#pragma unroll
+    for (int off = LPR; off < kWave; off <<= 1)
+#pragma unroll
+      for (int q = 0; q < VEC; ++q) acc[q] += __shfl_xor(acc[q], off, kWave);
+    if (g == 0 && active) {
+      if (d >= 0) {
+        float *crow = a.C + (int64_t)d * a.ldc + boff;
+        float out[VEC];
+        if (a.beta != 0.f) {
+          float old[VEC];
+          load_vec<VEC>(crow, old);
+#pragma unroll
+          for (int q = 0; q < VEC; ++q) out[q] = fmaf(a.beta, old[q], acc[q]);
+        } else {
+#pragma unroll
+          for (int q = 0; q < VEC; ++q) out[q] = acc[q];
+        }
+        store_vec<VEC>(crow, out);
+      } else if (a.p_cap <= 0 || (int64_t)(-(d + 1)) < a.p_cap) {
+        store_vec<VEC>(a.P + (int64_t)(-(d + 1)) * a.f + boff, acc);
+      }
+    }
+  }
+
+  // ---- short tasks: one team each, G per round
+  for (int q0 = 0; q0 < nshort; q0 += G) {
+    const int my = q0 + g;
+    const bool has = my < nshort;
+    const int k = has ? s_short[wv][my] : 0;
+    const int32_t s = s_beg[wv][k];
+    const int32_t e = has ? s_end[wv][k] : s;
+    const int32_t d = s_dst[wv][k];
+    float acc[VEC];
+#pragma unroll
+    for (int q = 0; q < VEC; ++q) acc[q] = 0.f;
+    int32_t i = s;
+    for (; i + 3 < e; i += 4) {
+      float b[4][VEC], vv[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int32_t cc = cw[i + u];
+        vv[u] = vw[i + u];
+        load_vec<VEC>(a.B + (int64_t)cc * a.ldb + boff, b[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int q = 0; q < VEC; ++q) acc[q] = fmaf(vv[u], b[u][q], acc[q]);
+    }
+    for (; i < e; ++i) {
+      float b[VEC];
+      const float vv = vw[i];
+      load_vec<VEC>(a.B + (int64_t)cw[i] * a.ldb + boff, b);
+#pragma unroll
+      for (int q = 0; q < VEC; ++q) acc[q] = fmaf(vv, b[q], acc[q]);
+    }
+    if (has && active) {
+      if (d >= 0) {
+        float *crow = a.C + (int64_t)d * a.ldc + boff;
+        float out[VEC];
+        if (a.beta != 0.f) {
+          float old[VEC];
+          load_vec<VEC>(crow, old);
+#pragma unroll
+          for (int q = 0; q < VEC; ++q) out[q] = fmaf(a.beta, old[q], acc[q]);
+        } else {
+#pragma unroll
+          for (int q = 0; q < VEC; ++q) out[q] = acc[q];
+        }
+        store_vec<VEC>(crow, out);
+      } else if (a.p_cap <= 0 || (int64_t)(-(d + 1)) < a.p_cap) {
+        store_vec<VEC>(a.P + (int64_t)(-(d + 1)) * a.f + boff, acc);
+      }
+    }
+  }
+}
+
+// C[r, :] += sum of the partial rows of r's hot tasks, in (group, segment) order.  One wavefront
+// per row: lane g fetches the task range of group g, then the lanes sweep the row's columns with
+// the partial rows of all tasks in flight together.
+template <int NC>  // classes the unrolled loops cover (nclass <= NC)
+__global__ __launch_bounds__(kSpmmThreads) void hub_reduce_kernel(const int32_t *__restrict__ tbase, int32_t n,
+                                                                  int32_t nclass, const float *__restrict__ P,
+                                                                  float *__restrict__ C, int64_t ldc, int32_t f) {
+  const int64_t r = ((int64_t)blockIdx.x * kSpmmThreads + threadIdx.x) / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  if (r >= n) return;
+  int32_t t0 = 0, t1 = 0;
+  if (lane < nclass) {
+    const int64_t v = (int64_t)lane * n + r;
+    t0 = tbase[v];
+    t1 = tbase[v + 1];
+  }
+  int32_t first[NC], count[NC];
+  int32_t total = 0;
+#pragma unroll
+  for (int g = 0; g < NC; ++g) {
+    first[g] = __builtin_amdgcn_readlane(t0, g);
+    count[g] = __builtin_amdgcn_readlane(t1, g) - first[g];
+    total += count[g];
+  }
+  if (total == 0) return;
+  float *crow = C + r * ldc;
+  for (int32_t c0 = 0; c0 < f; c0 += kWave) {
+    const int32_t col = c0 + lane;
+    if (col < f) {
+      float s = 0.f;
+#pragma unroll
+      for (int g = 0; g < NC; ++g) {
+        const float *p = P + (int64_t)first[g] * f + col;
+        if (count[g] == 1) {
+          s += p[0];
+        } else {
+          for (int32_t t = 0; t < count[g]; ++t) s += p[(int64_t)t * f];
+        }
+      }
+      crow[col] += s;
+    }
+  }
+}
+
+}  // namespace cg

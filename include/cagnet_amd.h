@@ -178,10 +178,18 @@ int cg_log_softmax_nll_bwd(const float *d_logp, int64_t ld, const int64_t *d_y, 
  * Recording is off by default and costs nothing then.
  */
 int cg_prof_enable(int on);
-/* Tuning knobs, 0 = built-in choice.  "spmm_seg": stored entries per row segment (>= 64);
- * "spmm_tiles": feature tiles of a wide SpMM launch (1, 2, 4 or 8; tile t runs on the XCDs x with
- * x % tiles == t).  Results stay deterministic for a given setting; different settings change the
- * summation order of split rows. */
+/* Tuning knobs, 0 = built-in choice (no counterpart in the reference, which hands every choice to
+ * cuSPARSE).  Results stay deterministic for a given setting; different settings change the
+ * summation order of split rows.
+ *   "spmm_seg"        stored entries per row segment (>= 64; narrow teams cap it at 512)
+ *   "spmm_win"        stored entries after which a new window of tasks starts (64..512)
+ *   "spmm_vec"        cap on the floats a lane moves per access (1, 2; otherwise 4)
+ *   "spmm_hub"        hub plan: -1 never, 1 always, 0 by width and density
+ *   "spmm_hub_kb"     KiB of hot B rows per XCD group and tier
+ *   "spmm_hub_groups" XCD groups the hot columns are dealt to (1, 2, 4, 8)
+ *   "spmm_hub_tiers"  tiers of hot columns (groups * tiers <= 16)
+ *   "dense_mfma"      -1: dense products on the vector ALU tile kernel only
+ * An unknown key returns CG_ERR_UNSUPPORTED. */
 int cg_tune_set(const char *key, int value);
 int cg_prof_read(const char *name, double *total_ms, int64_t *launches);
 

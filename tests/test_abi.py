@@ -66,7 +66,7 @@ def test_status_codes_without_a_gpu():
     assert lib.cg_log_softmax_fwd(one, 3, one, 4, 10, 4, null) == E["size"]
     assert lib.cg_nll_loss_fwd(one, 4, one, null, 10, 4, null, one, null) == E["null"]
     assert lib.cg_tune_set(b"no_such_knob", 1) == E["unsupported"]
-    assert lib.cg_tune_set(b"spmm_tiles", 0) == 0
+    assert lib.cg_tune_set(b"spmm_seg", 0) == 0
     for code in range(0, 11):
         assert lib.cg_status_string(code) not in (None, b"unknown status")
     assert lib.cg_status_string(99) == b"unknown status"

@@ -125,6 +125,46 @@ def test_spmm_gpu_one_shot_matches_oracle(cuda, f):
     assert C.is_contiguous()
 
 
+@pytest.mark.parametrize("f", [16, 41, 602, 2600])
+def test_spmm_gpu_one_shot_split_rows_and_reuse(cuda, f):
+    """The one-shot operator rebuilds its tables in a reused arena on every call: long rows
+    (several segments), then a smaller matrix with empty rows on the same stream, then the first
+    again; every result is checked, and the repeat is bit-identical to the first."""
+    from cagnet_amd.sparse_coo_tensor_cpp import spmm_gpu
+    n, m = 40, 6000
+    row, col, val = random_coo(n, m, n * 3000, seed=f)
+    B = torch.randn(m, f, generator=torch.Generator().manual_seed(1))
+    C0 = torch.randn(n, f, generator=torch.Generator().manual_seed(2))
+    args = (_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, m, B.to(cuda))
+    C = C0.to(cuda).clone()
+    spmm_gpu(*args, C)
+    assert spmm_error(C, row, col, val, n, m, B, C0) <= REL_TOL
+    n2 = 300
+    r2, c2, v2 = random_coo(n2, n2, 900, seed=f + 1)
+    r2 = r2 // 3 * 3                       # two of every three rows are empty; still sorted
+    B2 = torch.randn(n2, f, generator=torch.Generator().manual_seed(3))
+    D0 = torch.randn(n2, f, generator=torch.Generator().manual_seed(4))
+    D = D0.to(cuda).clone()
+    spmm_gpu(_i32(r2, cuda), _i32(c2, cuda), v2.to(cuda), n2, n2, B2.to(cuda), D)
+    assert spmm_error(D, r2, c2, v2, n2, n2, B2, D0) <= REL_TOL
+    empty = torch.ones(n2, dtype=torch.bool)
+    empty[r2.long()] = False
+    assert torch.equal(D.cpu()[empty], D0[empty])      # beta = 1: rows without entries are untouched
+    C2 = C0.to(cuda).clone()
+    spmm_gpu(*args, C2)
+    assert torch.equal(C, C2)
+
+
+def test_spmm_gpu_one_shot_empty_inputs(cuda):
+    from cagnet_amd.sparse_coo_tensor_cpp import spmm_gpu
+    e32 = torch.empty(0, dtype=torch.int32, device=cuda)
+    B = torch.randn(9, 8, device=cuda)
+    C0 = torch.randn(5, 8, device=cuda)
+    C = C0.clone()
+    spmm_gpu(e32, e32, torch.empty(0, device=cuda), 5, 9, B, C)   # no stored entries: C is unchanged
+    assert torch.equal(C, C0)
+
+
 @pytest.mark.parametrize("f", [16, 41, 128, 602])
 def test_spmm_split_rows(cuda, f):
     """Rows longer than a segment (1024 to 4096 entries by width class) are split over several
