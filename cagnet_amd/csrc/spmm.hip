@@ -774,6 +774,10 @@ struct DenseOps {
   int64_t ldc;
   int32_t f;
   float beta;
+  // optional fold of another launch's partial rows into the rows written here (see StreamArgs)
+  const int32_t *fold_tbase = nullptr;
+  const float *fold_P = nullptr;
+  int32_t fold_classes = 0, fold_rows = 0;
 };
 
 // Row-segment tasks over (rowptr, colind, val), for a column range one launch can cover.
@@ -804,6 +808,11 @@ static int spmm_plain(const int32_t *rowptr, const int32_t *colind, const float 
   sa.ldc = d.ldc;
   sa.f = d.f;
   sa.beta = d.beta;
+  sa.fold_tbase = d.fold_tbase;
+  sa.fold_P = d.fold_P;
+  sa.fold_classes = d.fold_classes;
+  sa.fold_rows = d.fold_rows;
+  if (d.fold_tbase && shape.lpr != kWave) CG_FAIL(CG_ERR_UNSUPPORTED, "fold needs full-wave teams");
   if (sc->nslots > 0) {
     void *p = nullptr;
     CG_TRY(scratch_get(stream, kSlotA, (size_t)sc->nslots * d.f * sizeof(float), &p));
@@ -817,7 +826,8 @@ static int spmm_plain(const int32_t *rowptr, const int32_t *colind, const float 
     ProfScope prof("spmm_reduce", prof_tag, stream);
     const int64_t threads = sc->nmulti * (int64_t)d.f;
     spmm_reduce_kernel<<<(unsigned)ceil_div64(threads, kSpmmThreads), kSpmmThreads, 0, stream>>>(
-        sc->multi_rows, sc->nmulti, nullptr, rowptr, sc->pbase, sc->seg, sa.P, d.C, d.ldc, d.f, d.beta, 0);
+        sc->multi_rows, sc->nmulti, nullptr, rowptr, sc->pbase, sc->seg, sa.P, d.C, d.ldc, d.f, d.beta, 0, d.fold_tbase,
+        d.fold_P, d.fold_classes, d.fold_rows);
     CG_LAUNCH_CHECK();
   }
   return CG_OK;
@@ -858,40 +868,49 @@ static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream) 
   HubPlan &h = s.hub;
   const int32_t n = s.rows;
   const int32_t nclass = h.classes();
-  // 1. cold class straight into C
-  CG_TRY(spmm_plain(h.vrowptr + (int64_t)nclass * n, h.colind, h.val, n, s.nnz, h.cold_sched, vec, d, f, stream));
-  // 2. hot classes, one launch per tier: every task writes a partial row
+  // 1. hot classes, one launch per tier: every task writes a partial row
   const int64_t hot_tasks = h.hot_sched.ntasks;
-  if (hot_tasks == 0) return CG_OK;
   void *p = nullptr;
-  CG_TRY(scratch_get(stream, kSlotC, (size_t)hot_tasks * f * sizeof(float), &p));
-  const int32_t S = window_entries();
-  if (h.hot_tab.S != S || h.hot_tab.groups != nclass) {
-    Alloc owned;
-    CG_TRY(build_stream(h.hot_sched, h.vrowptr, nclass * n, true, nclass, h.tstart, S, s.nnz, h.hot_tab, owned, false,
-                        stream));
+  if (hot_tasks > 0) {
+    CG_TRY(scratch_get(stream, kSlotC, (size_t)hot_tasks * f * sizeof(float), &p));
+    const int32_t S = window_entries();
+    if (h.hot_tab.S != S || h.hot_tab.groups != nclass) {
+      Alloc owned;
+      CG_TRY(build_stream(h.hot_sched, h.vrowptr, nclass * n, true, nclass, h.tstart, S, s.nnz, h.hot_tab, owned, false,
+                          stream));
+    }
+    for (int t = 0; t < tiers; ++t) {
+      StreamArgs sa{};
+      sa.task_start = h.hot_tab.task_start;
+      sa.task_dst = h.hot_tab.task_dst;
+      sa.wstart = h.hot_tab.wstart;
+      sa.colind = h.colind;
+      sa.val = h.val;
+      for (int g = 0; g <= groups; ++g) sa.win_first[g] = h.hot_tab.win_first[t * groups + g];
+      sa.groups = groups;
+      sa.B = d.B;
+      sa.ldb = d.ldb;
+      sa.C = d.C;
+      sa.ldc = d.ldc;
+      sa.P = (float *)p;
+      sa.f = f;
+      sa.beta = 0.f;
+      ProfScope prof("spmm_hub_hot", f, stream);
+      CG_TRY(launch_stream(hshape, sa, stream));
+    }
   }
-  for (int t = 0; t < tiers; ++t) {
-    StreamArgs sa{};
-    sa.task_start = h.hot_tab.task_start;
-    sa.task_dst = h.hot_tab.task_dst;
-    sa.wstart = h.hot_tab.wstart;
-    sa.colind = h.colind;
-    sa.val = h.val;
-    for (int g = 0; g <= groups; ++g) sa.win_first[g] = h.hot_tab.win_first[t * groups + g];
-    sa.groups = groups;
-    sa.B = d.B;
-    sa.ldb = d.ldb;
-    sa.C = d.C;
-    sa.ldc = d.ldc;
-    sa.P = (float *)p;
-    sa.f = f;
-    sa.beta = 0.f;
-    ProfScope prof("spmm_hub_hot", f, stream);
-    CG_TRY(launch_stream(hshape, sa, stream));
+  // 2. cold class straight into C.  Full-wave teams add the hot partial rows of a row in the same
+  //    store; narrower teams leave that to a separate fold.
+  DenseOps cold = d;
+  const bool fused = hot_tasks > 0 && pick_shape(vec, f / vec).lpr == kWave;
+  if (fused) {
+    cold.fold_tbase = h.hot_sched.tbase;
+    cold.fold_P = (const float *)p;
+    cold.fold_classes = nclass;
+    cold.fold_rows = n;
   }
-  // 3. fold the partial rows into C
-  {
+  CG_TRY(spmm_plain(h.vrowptr + (int64_t)nclass * n, h.colind, h.val, n, s.nnz, h.cold_sched, vec, cold, f, stream));
+  if (hot_tasks > 0 && !fused) {
     ProfScope prof("spmm_hub_reduce", f, stream);
     const unsigned rgrid = (unsigned)ceil_div64((int64_t)n * kWave, kSpmmThreads);
     if (nclass <= 8)
@@ -992,7 +1011,7 @@ static int spmm_coo_oneshot(const int32_t *d_row, const int32_t *d_col, const fl
     const int64_t threads = max_multi * (int64_t)ft;
     spmm_reduce_kernel<<<(unsigned)ceil_div64(threads, kSpmmThreads), kSpmmThreads, 0, stream>>>(
         sc.multi_rows, max_multi, sc.d_counts + 2, rowptr, sc.pbase, seg, (const float *)p, C + f0, ldc, ft, beta,
-        pslots);
+        pslots, nullptr, nullptr, 0, 0);
     CG_LAUNCH_CHECK();
   }
   return CG_OK;

@@ -64,7 +64,10 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_reduce_kernel(const int32_t
                                                                    const int32_t *__restrict__ pbase, int32_t seg,
                                                                    const float *__restrict__ P, float *__restrict__ C,
                                                                    int64_t ldc, int32_t f, float beta,
-                                                                   int64_t p_cap) {
+                                                                   int64_t p_cap,
+                                                                   const int32_t *__restrict__ fold_tbase,
+                                                                   const float *__restrict__ fold_P,
+                                                                   int32_t fold_classes, int32_t fold_rows) {
   const int64_t idx = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   const int64_t mr = idx / f;
   const int32_t col = (int32_t)(idx % f);
@@ -78,6 +81,12 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_reduce_kernel(const int32_t
   const float *p = P + (int64_t)pbase[row] * f + col;
   float s = 0.f;
   for (int32_t i = 0; i < nseg; ++i) s += p[(int64_t)i * f];
+  if (fold_tbase) {  // same fold as in the main kernel, for rows that were split
+    for (int32_t cls = 0; cls < fold_classes; ++cls) {
+      const int32_t *tb = fold_tbase + (int64_t)cls * fold_rows + row;
+      for (int32_t t = tb[0]; t < tb[1]; ++t) s += fold_P[(int64_t)t * f + col];
+    }
+  }
   float *c = C + (int64_t)row * ldc + col;
   *c = beta != 0.f ? fmaf(beta, *c, s) : s;
 }
@@ -100,6 +109,12 @@ struct StreamArgs {
   float *P;
   int32_t f;
   float beta;
+  // Fold (wide teams, groups == 1): a row that goes straight to C also receives the partial rows
+  // fold_P[t] for t in [fold_tbase[c * fold_rows + row], fold_tbase[c * fold_rows + row + 1]) of
+  // every class c < fold_classes, added in (class, t) order after the row's own entries.
+  const int32_t *fold_tbase;
+  const float *fold_P;
+  int32_t fold_classes, fold_rows;
 };
 
 // Full-wave teams (one stored entry per wave step, f covered by CHUNKS x 64 lanes x VEC floats).
@@ -167,7 +182,26 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_stream_wide_kernel(const St
       while (tend == base + i) {  // the current task is complete (also true at once for an empty task)
         const int32_t dst = __builtin_amdgcn_readlane(m_dst, tk);
         if (dst >= 0) {
-          if (!(tend == tbeg && a.beta == 1.0f)) {  // an empty row leaves C alone when beta == 1
+          bool folded = false;
+          if (a.fold_tbase) {
+            for (int32_t cls = 0; cls < a.fold_classes; ++cls) {
+              const int32_t *tb = a.fold_tbase + (int64_t)cls * a.fold_rows + dst;
+              const int32_t p0 = __builtin_amdgcn_readfirstlane(tb[0]);
+              const int32_t p1 = __builtin_amdgcn_readfirstlane(tb[1]);
+              for (int32_t t = p0; t < p1; ++t) {
+                const float *prow = a.fold_P + (int64_t)t * a.f;
+                float pv[CHUNKS][VEC];
+#pragma unroll
+                for (int ch = 0; ch < CHUNKS; ++ch) load_vec<VEC>(prow + boff[ch], pv[ch]);
+#pragma unroll
+                for (int ch = 0; ch < CHUNKS; ++ch)
+#pragma unroll
+                  for (int q = 0; q < VEC; ++q) acc[ch][q] += pv[ch][q];
+                folded = true;
+              }
+            }
+          }
+          if (folded || !(tend == tbeg && a.beta == 1.0f)) {  // an empty row leaves C alone when beta == 1
             float *crow = a.C + (int64_t)dst * a.ldc;
 #pragma unroll
             for (int ch = 0; ch < CHUNKS; ++ch) {
