@@ -20,6 +20,10 @@ int xtg_mfma(const float *X, int64_t ldx, const float *G, int64_t ldg, float *P,
              int64_t rows_per_block, int64_t nblocks, hipStream_t stream);
 int gwt_mfma(const float *G, int64_t ldg, const float *W, int64_t ldw, float *dX, int64_t lddx, int64_t n, int32_t k,
              int32_t fo, hipStream_t stream);
+int xtg_vec(const float *X, int64_t ldx, int32_t k);
+// dense_rows.hip
+int gwt_rows(const float *G, int64_t ldg, const float *W, int64_t ldw, float *dX, int64_t lddx, int64_t n, int32_t k,
+             int32_t fo, hipStream_t stream);
 
 // cg_tune_set("dense_mfma", -1) routes every product through the LDS-tiled vector kernel below
 std::atomic<int> g_tune_dense_mfma{0};
@@ -265,6 +269,8 @@ int cg_dense_gwt(const float *d_G, int64_t ldg, const float *d_W, int64_t ldw, f
   // which the vector kernel issues in longer contiguous runs
   if (fo <= 64 && k <= 64 && g_tune_dense_mfma.load(std::memory_order_relaxed) >= 0)
     return gwt_mfma(d_G, ldg, d_W, ldw, d_dX, lddx, n, k, fo, (hipStream_t)stream);
+  if (fo <= 64 && k > 64 && g_tune_dense_mfma.load(std::memory_order_relaxed) >= 0)
+    return gwt_rows(d_G, ldg, d_W, ldw, d_dX, lddx, n, k, fo, (hipStream_t)stream);
   return launch_gemm<false, true>(g, (hipStream_t)stream);
 }
 
@@ -277,11 +283,11 @@ int cg_dense_xtg(const float *d_X, int64_t ldx, const float *d_G, int64_t ldg, f
   if (fo <= 64 && n > 0 && g_tune_dense_mfma.load(std::memory_order_relaxed) >= 0) {
     ProfScope prof("dense_xtg", k, stream);
     // contiguous vertex ranges, enough wavefronts to keep ~16 per CU in flight
-    const int vecw = (ldx % 4 == 0 && ((uintptr_t)d_X) % 16 == 0 && k >= 4) ? 4 : ((ldx % 2 == 0 && ((uintptr_t)d_X) % 8 == 0 && k >= 2) ? 2 : 1);
+    const int vecw = xtg_vec(d_X, ldx, k);
     const int64_t ywaves = ceil_div64(k, 16 * vecw);
     int64_t nblocks = ceil_div64(8192, ywaves);
-    if (nblocks > 1024) nblocks = 1024;
     int64_t rows_per_block = ceil_div64(ceil_div64(n, nblocks), 16) * 16;
+    if (rows_per_block < 256) rows_per_block = 256;  // the partial product a range writes stays small beside its reads
     nblocks = ceil_div64(n, rows_per_block);
     const int64_t elems = (int64_t)k * fo;
     void *p = nullptr;

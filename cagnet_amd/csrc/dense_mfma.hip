@@ -133,7 +133,7 @@ __global__ __launch_bounds__(kMfmaThreads) void xtg_mfma_kernel(const float *__r
                                                                 int32_t fo, int64_t rows_per_block) {
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int m = lane & 15, q = lane >> 4;
-  const int32_t kt0 = (blockIdx.y * kMfmaWaves + wave) * 16 * VEC;  // first column of this wave
+  const int32_t kt0 = (blockIdx.y * (blockDim.x / kWave) + wave) * 16 * VEC;  // first column of this wave
   if (kt0 >= k) return;
   const int32_t kcol = kt0 + m * VEC;
   const bool full = kcol + VEC <= k;
@@ -270,12 +270,23 @@ int xw_mfma(const float *X, int64_t ldx, const float *W, int64_t ldw, float *Z, 
   CG_FAIL(CG_ERR_UNSUPPORTED, "cg_dense_xw: fo=%d has no matrix-core variant", fo);
 }
 
+// Columns of X a lane reads per vertex: as wide as alignment allows, but no wider than keeps the 16
+// lanes of a tile row on live columns (k = 16 -> one column per lane).
+int xtg_vec(const float *X, int64_t ldx, int32_t k) {
+  int vec = pick_kvec(X, ldx, k);
+  while (vec > 1 && 16 * vec > k) vec >>= 1;
+  return vec;
+}
+
 int xtg_mfma(const float *X, int64_t ldx, const float *G, int64_t ldg, float *P, int64_t n, int32_t k, int32_t fo,
              int64_t rows_per_block, int64_t nblocks, hipStream_t stream) {
   const int nt = (fo + 15) / 16;
-  const int vec = pick_kvec(X, ldx, k);
+  const int vec = xtg_vec(X, ldx, k);
   const int64_t ywaves = ceil_div64(k, 16 * vec);
-  dim3 grid((unsigned)nblocks, (unsigned)ceil_div64(ywaves, kMfmaWaves));
+  // narrow X: fewer wavefronts per workgroup, so none of them is without columns
+  const int wpb = ywaves < kMfmaWaves ? (int)ywaves : kMfmaWaves;
+  dim3 grid((unsigned)nblocks, (unsigned)ceil_div64(ywaves, wpb));
+  const unsigned kMfmaThreads = (unsigned)(wpb * kWave);  // shadows the constant inside this function
 #define CG_CASE(V, T)                                                                                         \
   if (vec == V && nt == T) {                                                                                  \
     xtg_mfma_kernel<V, T><<<grid, kMfmaThreads, 0, stream>>>(X, ldx, G, ldg, P, n, k, fo, rows_per_block);    \
