@@ -9,12 +9,12 @@
 
 namespace cg {
 
-constexpr int kRowsThreads = 256;
+constexpr int kRowsMaxThreads = 1024;
 
-constexpr int kRowsLds = 8192;  // floats of G staged per workgroup
+constexpr int kRowsLds = 16384;  // floats of G staged per workgroup
 
 template <int FO, int VEC>
-__global__ __launch_bounds__(kRowsThreads) void gwt_rows_kernel(const float *__restrict__ G, int64_t ldg,
+__global__ __launch_bounds__(kRowsMaxThreads) void gwt_rows_kernel(const float *__restrict__ G, int64_t ldg,
                                                                 const float *__restrict__ W, int64_t ldw,
                                                                 float *__restrict__ dX, int64_t lddx, int64_t n,
                                                                 int32_t k, int32_t fo, int32_t tpr, int32_t nchunk,
@@ -24,12 +24,12 @@ __global__ __launch_bounds__(kRowsThreads) void gwt_rows_kernel(const float *__r
   __shared__ __attribute__((aligned(16))) float Gs[kRowsLds];
   const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
   const int32_t nrows = (int32_t)(r0 + rows_per_block < n ? rows_per_block : n - r0);
-  for (int32_t i = threadIdx.x; i < nrows * FO; i += kRowsThreads) {
+  for (int32_t i = threadIdx.x; i < nrows * FO; i += blockDim.x) {
     const int32_t row = i / FO, j = i % FO;
     Gs[i] = j < fo ? G[(r0 + row) * ldg + j] : 0.f;
   }
   __syncthreads();
-  const int rps = kRowsThreads / tpr;  // rows per step
+  const int rps = blockDim.x / tpr;  // rows per step
   const int rs = threadIdx.x / tpr, cv = threadIdx.x % tpr;
   if (rs >= rps) return;  // no barrier below
   for (int32_t chunk = 0; chunk < nchunk; ++chunk) {
@@ -83,10 +83,22 @@ int gwt_rows(const float *G, int64_t ldg, const float *W, int64_t ldw, float *dX
   if (lddx % 4 == 0 && ((uintptr_t)dX) % 16 == 0) vec = 4;
   else if (lddx % 2 == 0 && ((uintptr_t)dX) % 8 == 0) vec = 2;
   while (vec > 1 && vec * FO > 64) vec >>= 1;  // the weights of a thread's columns stay in registers
-  const int32_t cvs = (k + vec - 1) / vec;                              // column vectors of a row
-  const int32_t nchunk = (cvs + kRowsThreads - 1) / kRowsThreads;
-  const int32_t tpr = (cvs + nchunk - 1) / nchunk;                      // threads per row
-  const int rps = kRowsThreads / tpr;
+  const int32_t cvs = (k + vec - 1) / vec;  // column vectors of a row
+  // workgroup size: the one that leaves the fewest threads without a column
+  int threads = 256, nchunk = 1, tpr = 1;
+  double best = -1.0;
+  for (int t = 256; t <= kRowsMaxThreads; t *= 2) {
+    const int nc = (cvs + t - 1) / t;
+    const int per = (cvs + nc - 1) / nc;  // threads per row
+    const double used = (double)cvs / nc * (t / per) / t;
+    if (used > best + 0.02) {
+      best = used;
+      threads = t;
+      nchunk = nc;
+      tpr = per;
+    }
+  }
+  const int rps = threads / tpr;
   int32_t rows_per_block = rps * 128;  // amortises the weight loads of a workgroup
   if (rows_per_block > kRowsLds / FO) rows_per_block = kRowsLds / FO / rps * rps;
   if (rows_per_block < rps) rows_per_block = rps;
@@ -94,7 +106,7 @@ int gwt_rows(const float *G, int64_t ldg, const float *W, int64_t ldw, float *dX
   if (blocks > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "gwt_rows: grid too large");
 #define CG_CASE(F, V)                                                                                        \
   if (FO == F && vec == V) {                                                                                 \
-    gwt_rows_kernel<F, V><<<(unsigned)blocks, kRowsThreads, 0, stream>>>(G, ldg, W, ldw, dX, lddx, n, k, fo, \
+    gwt_rows_kernel<F, V><<<(unsigned)blocks, (unsigned)threads, 0, stream>>>(G, ldg, W, ldw, dX, lddx, n, k, fo, \
                                                                          tpr, nchunk, rows_per_block);          \
     CG_LAUNCH_CHECK();                                                                                       \
     return CG_OK;                                                                                            \
