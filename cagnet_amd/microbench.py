@@ -2,12 +2,15 @@
 
     python -m cagnet_amd.microbench spmm   [--graph rmat20|reddit] [--widths 16,64,128,602]
     python -m cagnet_amd.microbench grid2d [--grid 4] [--row 1]
+    python -m cagnet_amd.microbench prep   [--graph reddit]
 
 `spmm`   builds the CSR (sorted input, unsorted input, transpose) and times A @ H and A^T @ G at
          each width: GFLOP/s = 2 nnz f / t, algorithmic GB/s = (8 nnz + 4 (n+1) + 4 m f + 4 n f) / t.
 `grid2d` is one rank's share of the sqrt(P) x sqrt(P) 2D algorithm (gcn_distr_2d.py:333-417) on the
          Reddit-shaped graph: the sparse blocks A(r, 0..q-1) of process row r, each times a resident
          dense block, accumulated over q stages; forward and backward of both layers.
+`prep`   times the device-side input preparation on the graph's pattern: self-loop insertion,
+         D^-1/2 A D^-1/2 values, and the 16 block extractions of a 4 x 4 partition.
 One JSON object per line.  Timing: HIP events on the current stream, best of `--reps`.
 """
 from __future__ import annotations
@@ -144,6 +147,42 @@ def run_grid2d(args) -> None:
                       "stage_loop_algorithmic_gbs": round(alg / ms_stage / 1e6, 1)}), flush=True)
 
 
+def run_prep(args) -> None:
+    from . import ops, synth
+
+    dev = torch.device("cuda:0")
+    row, col, _, n = _graph(args.graph, dev)
+    r32, c32 = row.int(), col.int()
+    nnz = int(r32.numel())
+    del row, col
+
+    def wall(fn):
+        fn()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(args.reps):
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            best = min(best, (time.perf_counter() - t0) * 1e3)
+        return best
+
+    t_loops = wall(lambda: ops.add_self_loops(r32, c32, n))
+    t_norm = wall(lambda: ops.gcn_normalize(r32, c32, n))
+    val = ops.gcn_normalize(r32, c32, n)
+    b = synth.block_bounds_2d(n, 4)
+
+    def blocks():
+        for i in range(4):
+            for j in range(4):
+                ops.coo_block(r32, c32, val, b[i], b[i + 1], b[j], b[j + 1])
+
+    t_blocks = wall(blocks)
+    print(json.dumps({"what": "input preparation", "graph": args.graph, "n": n, "nnz": nnz,
+                      "add_self_loops_ms": round(t_loops, 3), "gcn_normalize_ms": round(t_norm, 3),
+                      "coo_block_4x4_all_16_ms": round(t_blocks, 3)}), flush=True)
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="cmd", required=True)
@@ -155,12 +194,17 @@ def main() -> int:
     g.add_argument("--grid", type=int, default=4)
     g.add_argument("--row", type=int, default=1)
     g.add_argument("--reps", type=int, default=5)
+    pr = sub.add_parser("prep")
+    pr.add_argument("--graph", default="reddit", choices=sorted(GRAPHS))
+    pr.add_argument("--reps", type=int, default=3)
     args = ap.parse_args()
     if not torch.cuda.is_available():
         print("microbench: no GPU visible; cagnet_amd has no CPU path", file=sys.stderr)
         return 2
     if args.cmd == "spmm":
         run_spmm(args)
+    elif args.cmd == "prep":
+        run_prep(args)
     else:
         run_grid2d(args)
     return 0

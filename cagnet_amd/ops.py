@@ -108,6 +108,60 @@ def coo2csr(row: torch.Tensor, col: torch.Tensor, val: Optional[torch.Tensor], n
     return (rowptr, colind, values, perm) if return_perm else (rowptr, colind, values)
 
 
+# ------------------------------------------------------------------------------------------------
+# input preparation (host code in the reference: gcn_distr.py:791, :412-470, :398-409)
+# ------------------------------------------------------------------------------------------------
+def add_self_loops(row: torch.Tensor, col: torch.Tensor, n: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Strictly ascending int32 COO pattern of an n x n matrix -> the same pattern with every
+    diagonal entry present exactly once (add_remaining_self_loops, gcn_distr.py:791)."""
+    row, col = _index(row, "row"), _index(col, "col")
+    if row.numel() != col.numel():
+        raise ValueError("row and col differ in length")
+    count = ctypes.c_int64(0)
+    check(lib.cg_add_self_loops(_ptr(row), _ptr(col), row.numel(), n, None, None, 0, ctypes.byref(count), _stream()),
+          "cg_add_self_loops")
+    out_row = torch.empty(count.value, dtype=torch.int32, device=row.device)
+    out_col = torch.empty(count.value, dtype=torch.int32, device=row.device)
+    check(lib.cg_add_self_loops(_ptr(row), _ptr(col), row.numel(), n, _ptr(out_row), _ptr(out_col), count.value,
+                                ctypes.byref(count), _stream()), "cg_add_self_loops")
+    return out_row, out_col
+
+
+def gcn_normalize(row: torch.Tensor, col: torch.Tensor, n: int, return_dinv: bool = False):
+    """fp32 values of D^-1/2 A D^-1/2 for a pattern that already holds its self-loops, in the
+    arithmetic of scale_elements (gcn_distr.py:439-468).  Bit-identical to the host computation."""
+    row, col = _index(row, "row"), _index(col, "col")
+    if row.numel() != col.numel():
+        raise ValueError("row and col differ in length")
+    val = torch.empty(row.numel(), dtype=torch.float32, device=row.device)
+    dinv = torch.empty(n, dtype=torch.float32, device=row.device) if return_dinv else None
+    check(lib.cg_gcn_normalize(_ptr(row), _ptr(col), row.numel(), n, _ptr(val), _ptr(dinv), _stream()),
+          "cg_gcn_normalize")
+    return (val, dinv) if return_dinv else val
+
+
+def coo_block(row: torch.Tensor, col: torch.Tensor, val: Optional[torch.Tensor], r0: int, r1: int, c0: int, c1: int):
+    """Entries inside [r0, r1) x [c0, c1) in input order, rebased to the block (split_coo,
+    gcn_distr.py:398-409): (row, col, val)."""
+    row, col = _index(row, "row"), _index(col, "col")
+    nnz = row.numel()
+    if col.numel() != nnz or (val is not None and val.numel() != nnz):
+        raise ValueError("row, col and val differ in length")
+    if val is not None:
+        val = _values(val, "val")
+    count = ctypes.c_int64(0)
+    check(lib.cg_coo_block(_ptr(row), _ptr(col), _ptr(val), nnz, r0, r1, c0, c1, None, None, None, 0,
+                           ctypes.byref(count), _stream()), "cg_coo_block")
+    dev = row.device
+    out_row = torch.empty(count.value, dtype=torch.int32, device=dev)
+    out_col = torch.empty(count.value, dtype=torch.int32, device=dev)
+    out_val = torch.empty(count.value, dtype=torch.float32, device=dev) if val is not None else None
+    if count.value:
+        check(lib.cg_coo_block(_ptr(row), _ptr(col), _ptr(val), nnz, r0, r1, c0, c1, _ptr(out_row), _ptr(out_col),
+                               _ptr(out_val), count.value, ctypes.byref(count), _stream()), "cg_coo_block")
+    return out_row, out_col, out_val
+
+
 def csr_transpose(rowptr: torch.Tensor, colind: torch.Tensor, values: Optional[torch.Tensor], n: int, m: int,
                   return_perm: bool = False):
     """CSR of A (n x m) -> CSR of A^T (m x n): (colptr, rowind, values_t[, perm])."""

@@ -169,6 +169,35 @@ int cg_log_softmax_nll_bwd(const float *d_logp, int64_t ld, const int64_t *d_y, 
                            int32_t c, cg_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Input preparation on the device.  The reference prepares its adjacency matrix on the host:
+ * add_remaining_self_loops (gcn_distr.py:791), scale_elements (gcn_distr.py:412-470) and
+ * split_coo (gcn_distr.py:398-409).  These three entry points do the same work on int32 COO
+ * arrays that are already in device memory.  All three allocate temporaries and synchronise
+ * `stream` before they return.
+ *
+ * cg_add_self_loops: (row, col) strictly ascending COO of an n x n pattern -> the same pattern
+ * with every diagonal entry present exactly once, still ascending.  *out_nnz receives the size of
+ * the result; with both outputs NULL the call only counts.  CG_ERR_SIZE if capacity is too small,
+ * CG_ERR_UNSORTED / CG_ERR_INDEX for input that is not strictly ascending or out of range. */
+int cg_add_self_loops(const int32_t *d_row, const int32_t *d_col, int64_t nnz, int32_t n, int32_t *d_out_row,
+                      int32_t *d_out_col, int64_t capacity, int64_t *out_nnz, cg_stream_t stream);
+
+/* cg_gcn_normalize: values of D^-1/2 A D^-1/2 for a pattern that already holds its self-loops, in
+ * the arithmetic of scale_elements: deg_i = stored entries of row i, dinv_i = fl32(deg_i^-1/2)
+ * with the power in fp64 (gcn_distr.py:440-448), val = fl32(dinv_row * fl32(1 * dinv_col))
+ * (gcn_distr.py:458-464).  Any entry order.  d_dinv (nullable, n floats) receives dinv. */
+int cg_gcn_normalize(const int32_t *d_row, const int32_t *d_col, int64_t nnz, int32_t n, float *d_val,
+                     float *d_dinv, cg_stream_t stream);
+
+/* cg_coo_block: the entries with r0 <= row < r1 and c0 <= col < c1, in input order, rebased to
+ * the block's origin (gcn_distr.py:404-406; the 2D variant gcn_distr_2d.py:1040-1047).  d_val
+ * and d_out_val may both be NULL (pattern only).  *out_nnz receives the block's size; with all
+ * outputs NULL the call only counts. */
+int cg_coo_block(const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz, int32_t r0, int32_t r1,
+                 int32_t c0, int32_t c1, int32_t *d_out_row, int32_t *d_out_col, float *d_out_val, int64_t capacity,
+                 int64_t *out_nnz, cg_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
  * Kernel timing (the reference brackets phases with wall clocks and device synchronisation,
  * gcn_distr.py:66-94; here HIP events are recorded on the launch stream around single kernels).
  * cg_prof_enable(1) starts recording, cg_prof_enable(0) stops.  cg_prof_read waits for the

@@ -16,7 +16,8 @@ the reference has no tests or golden vectors, so this is an independent restatem
                                                2D: gcn_distr_2d.py:333-417), broadcasts removed
   GCNFuncOracle    GCNFunc                     gcn_distr.py:248-339
   train_epoch      train                       gcn_distr.py:341-366
-  gcn_normalize    scale_elements              gcn_distr.py:412-470 (+ self-loops, :791)
+  gcn_normalize    scale_elements              gcn_distr.py:412-470
+  add_self_loops   add_remaining_self_loops    gcn_distr.py:791 (+ coalesce, :546)
   block_bounds_*   split_coo / partitions      gcn_distr.py:398-409, gcn_distr_2d.py:1032-1047, :1102
 
 How each function is pinned (tests/test_oracle.py): coo2csr/transpose against
@@ -24,8 +25,9 @@ scipy.sparse tocsr()/tocsc() and torch .coalesce()/.to_sparse_csr() and a lower_
 form; spmm against scipy CSR @ dense, a dense matmul and hand-computed special cases (identity,
 single row, empty rows); GCNFunc's hand-written backward against torch autograd over the same
 forward and torch.autograd.gradcheck in fp64; the loss against F.nll_loss on gathered rows; the
-normalisation against a dense D^-1/2 (A+I) D^-1/2 in fp64 and its symmetry; block bounds against
-brute-force enumeration.  No function of this oracle is "parity unpinned".
+normalisation against a dense D^-1/2 (A+I) D^-1/2 in fp64 and its symmetry; self-loops against
+scipy's (A - diag(A) + I) pattern; block bounds and block extraction against brute-force
+enumeration and scipy slicing.  No function of this oracle is "parity unpinned".
 
 Every routine takes `dtype` (torch.float32 for the reference's arithmetic, torch.float64 for the
 error yardstick both the GPU result and the fp32 CPU result are measured against).
@@ -226,6 +228,18 @@ def gcn_normalize(row: np.ndarray, col: np.ndarray, n: int) -> np.ndarray:
         dinv = np.power(deg, -0.5).astype(np.float32)
     right = (np.float32(1.0) * dinv[col]).astype(np.float32)
     return (dinv[row] * right).astype(np.float32)
+
+
+def add_self_loops(row: np.ndarray, col: np.ndarray, n: int):
+    """add_remaining_self_loops on an unweighted pattern (gcn_distr.py:791) followed by the
+    coalesce the reference applies to its adjacency matrix (gcn_distr.py:546): the off-diagonal
+    entries plus every (i, i) once, in (row, col) order."""
+    row, col = np.asarray(row, dtype=np.int64), np.asarray(col, dtype=np.int64)
+    off = row != col
+    r = np.concatenate([row[off], np.arange(n, dtype=np.int64)])
+    c = np.concatenate([col[off], np.arange(n, dtype=np.int64)])
+    order = np.lexsort((c, r))
+    return r[order], c[order]
 
 
 def block_bounds_1d(node_count: int, parts: int) -> List[int]:

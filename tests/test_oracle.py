@@ -253,3 +253,42 @@ def test_block_bounds_2d_reddit_grid():
     assert orc.block_bounds_2d(16, 4) == [0, 4, 8, 12, 16]
     r, c, v = orc.coo_block(np.array([0, 5, 5, 9]), np.array([1, 4, 8, 9]), np.array([1., 2., 3., 4.]), 4, 10, 4, 10)
     assert r.tolist() == [1, 1, 5] and c.tolist() == [0, 4, 5] and v.tolist() == [2., 3., 4.]
+
+
+@pytest.mark.parametrize("n,nnz,seed", [(1, 1, 0), (9, 30, 1), (300, 4000, 2), (2000, 3000, 3)])
+def test_add_self_loops_against_scipy(n, nnz, seed):
+    """The diagonal is present exactly once whether or not the input held it: scipy's pattern of
+    (A - diag(A)) + I, indices sorted."""
+    row, col, _ = random_coo(n, n, nnz, seed)
+    r, c = orc.add_self_loops(row.numpy(), col.numpy(), n)
+    a = sp.coo_matrix((np.ones(row.numel()), (row.numpy(), col.numpy())), shape=(n, n)).tocsr()
+    a.setdiag(0)
+    a.eliminate_zeros()
+    ref = (a + sp.identity(n, format="csr")).tocsr()
+    ref.sort_indices()
+    ref = ref.tocoo()
+    assert np.array_equal(r, ref.row) and np.array_equal(c, ref.col)
+    assert np.count_nonzero(r == c) == n
+
+
+def test_inverse_sqrt_degree_forms_agree_after_fp32_rounding():
+    """The device computes fl32(1 / sqrt(d)) with correctly rounded fp64 operations, the host
+    restatements fl32(d ** -0.5) through pow: both round to the same fp32 value for every degree a
+    graph of this size class can have (exhaustive over 1 .. 2^22)."""
+    d = np.arange(1, (1 << 22) + 1, dtype=np.float64)
+    a = (1.0 / np.sqrt(d)).astype(np.float32)
+    b = np.power(d, -0.5).astype(np.float32)
+    c = torch.from_numpy(d).pow(-0.5).to(torch.float32).numpy()
+    assert np.array_equal(a, b) and np.array_equal(a, c)
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_coo_block_against_scipy_slicing(seed):
+    n, m = 70, 90
+    row, col, val = random_coo(n, m, 900, seed)
+    r0, r1, c0, c1 = 13, 50, 30, 77
+    r, c, v = orc.coo_block(row.numpy(), col.numpy(), val.numpy(), r0, r1, c0, c1)
+    ref = sp.coo_matrix((val.numpy(), (row.numpy(), col.numpy())), shape=(n, m)).tocsr()[r0:r1, c0:c1].tocoo()
+    order = np.lexsort((ref.col, ref.row))
+    assert np.array_equal(r, ref.row[order]) and np.array_equal(c, ref.col[order])
+    assert np.array_equal(v, ref.data[order])
