@@ -82,6 +82,8 @@ int radix_sort_pairs(SortBuffers &buf, int64_t count, int bits_a, int bits_b, in
 
 // coo2csr.hip
 int launch_rowptr(const int32_t *d_row, int64_t nnz, int32_t n, int32_t *d_rowptr, hipStream_t stream);
+// row index of every stored entry of a CSR matrix
+int expand_rows(const int32_t *d_rowptr, int32_t n, int32_t *d_row, hipStream_t stream);
 int coo_check(const int32_t *d_row, const int32_t *d_col, int64_t nnz, int32_t n, int32_t m, int require_sorted,
               hipStream_t stream);
 int coo2csr_general(const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz, int32_t n,

@@ -89,6 +89,14 @@ __global__ __launch_bounds__(kThreads) void csr_expand_rows_kernel(const int32_t
   for (int32_t k = s + lane; k < e; k += kWave) row_out[k] = (int32_t)wave;
 }
 
+int expand_rows(const int32_t *d_rowptr, int32_t n, int32_t *d_row, hipStream_t stream) {
+  if (n <= 0) return CG_OK;
+  csr_expand_rows_kernel<<<(unsigned)ceil_div64((int64_t)n * kWave, kThreads), kThreads, 0, stream>>>(d_rowptr, n,
+                                                                                                     d_row);
+  CG_LAUNCH_CHECK();
+  return CG_OK;
+}
+
 static int check_common(int64_t nnz, int32_t n, int32_t m) {
   if (nnz < 0 || n < 0 || m < 0) CG_FAIL(CG_ERR_SIZE, "negative size: nnz=%lld n=%d m=%d", (long long)nnz, n, m);
   if (nnz > 0x7fffffffLL - 1) CG_FAIL(CG_ERR_OVERFLOW, "nnz=%lld does not fit the int32 rowptr contract", (long long)nnz);

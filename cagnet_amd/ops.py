@@ -248,6 +248,48 @@ class CsrMatrix:
                 pass
             self._handle = None
 
+    # ---- one byte string per block: files and transfers (the reference pickles int64 COO,
+    # gcn_distr.py:747, and sends indices as float32, gcn_distr_2d.py:369-374) ----------------------
+    def to_blob(self):
+        """The block as a numpy uint8 array: 128-byte header, int32 rowptr / colind, fp32 values."""
+        import numpy as np
+        size = c_int64(0)
+        check(lib.cg_csr_blob_size(self._handle, ctypes.byref(size)), "cg_csr_blob_size")
+        buf = np.empty(size.value, dtype=np.uint8)
+        with torch.cuda.device(self.device):
+            check(lib.cg_csr_blob_write(self._handle, c_void_p(buf.ctypes.data), size.value, _stream()),
+                  "cg_csr_blob_write")
+        return buf
+
+    @classmethod
+    def from_blob(cls, blob, device="cuda:0", transpose: bool = False) -> "CsrMatrix":
+        """Rebuild a block from `to_blob` bytes (numpy uint8 array, bytes or a memory map).  The
+        content is checked (header, checksum, rowptr, column range) before anything is launched on it."""
+        import numpy as np
+        buf = np.frombuffer(blob, dtype=np.uint8) if not isinstance(blob, np.ndarray) else blob
+        if buf.dtype != np.uint8 or buf.ndim != 1 or not buf.flags["C_CONTIGUOUS"]:
+            raise ValueError("blob must be a contiguous 1-D uint8 buffer")
+        self = cls.__new__(cls)
+        self._handle = None
+        self.device = torch.device(device)
+        handle = c_void_p(0)
+        with torch.cuda.device(self.device):
+            check(lib.cg_csr_blob_read(ctypes.byref(handle), c_void_p(buf.ctypes.data), buf.size,
+                                       CG_CSR_TRANSPOSE if transpose else 0, _stream()), "cg_csr_blob_read")
+        self._handle = handle
+        info = self.info()
+        self.n, self.m, self.nnz = int(info["n"]), int(info["m"]), int(info["nnz"])
+        self.has_transpose = bool(info["has_transpose"])
+        return self
+
+    def save(self, path) -> None:
+        self.to_blob().tofile(path)
+
+    @classmethod
+    def load(cls, path, device="cuda:0", transpose: bool = False) -> "CsrMatrix":
+        import numpy as np
+        return cls.from_blob(np.memmap(path, dtype=np.uint8, mode="r"), device=device, transpose=transpose)
+
     @property
     def shape(self) -> Tuple[int, int]:
         return (self.n, self.m)

@@ -169,6 +169,24 @@ int cg_log_softmax_nll_bwd(const float *d_logp, int64_t ld, const int64_t *d_y, 
                            int32_t c, cg_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
+ * A sparse block as one byte string in host memory, for files and for transfers between ranks.
+ * The reference loads its adjacency matrix from a pickled int64 COO tensor (gcn_distr.py:747)
+ * and sends blocks as three float32 arrays, indices included (gcn_distr_2d.py:369-374), which is
+ * lossy above 2^24.  The blob holds a 128-byte header (magic "CGNTCSR", version 1, flags, n, m,
+ * nnz, array offsets, total size, FNV-1a checksum of the payload) followed by int32 rowptr[n+1],
+ * int32 colind[nnz] and float values[nnz], each on a 64-byte boundary, little endian.
+ *
+ * cg_csr_blob_size: bytes a handle needs.  cg_csr_blob_write: fills host_buf (>= that size).
+ * cg_csr_blob_read: checks magic, version, sizes, offsets, checksum, rowptr monotonicity and the
+ * column range, then builds a handle; the transpose is rebuilt when the writer's handle had one
+ * or when `flags` holds CG_CSR_TRANSPOSE.  A malformed blob is rejected with CG_ERR_UNSUPPORTED
+ * (magic, version), CG_ERR_SIZE (truncated, inconsistent offsets), CG_ERR_INDEX (checksum, column
+ * range, rowptr ends) or CG_ERR_UNSORTED.  All three synchronise `stream`. */
+int cg_csr_blob_size(const cg_csr_t *h, int64_t *bytes);
+int cg_csr_blob_write(const cg_csr_t *h, void *host_buf, int64_t capacity, cg_stream_t stream);
+int cg_csr_blob_read(cg_csr_t **out, const void *host_buf, int64_t bytes, uint32_t flags, cg_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
  * Input preparation on the device.  The reference prepares its adjacency matrix on the host:
  * add_remaining_self_loops (gcn_distr.py:791), scale_elements (gcn_distr.py:412-470) and
  * split_coo (gcn_distr.py:398-409).  These three entry points do the same work on int32 COO

@@ -35,6 +35,7 @@ error yardstick both the GPU result and the fp32 CPU result are measured against
 from __future__ import annotations
 
 import math
+import struct
 from typing import List, Optional, Sequence, Tuple
 
 import numpy as np
@@ -259,6 +260,64 @@ def coo_block(row: np.ndarray, col: np.ndarray, val: np.ndarray, r0: int, r1: in
     row, col = np.asarray(row), np.asarray(col)
     keep = (row >= r0) & (row < r1) & (col >= c0) & (col < c1)
     return row[keep] - r0, col[keep] - c0, np.asarray(val)[keep]
+
+
+# ------------------------------------------------------------------------------------------------
+# byte format of a sparse block (replaces the pickled int64 COO of gcn_distr.py:747 and the float32
+# index payload of gcn_distr_2d.py:369-374); restated here from the format description alone
+# ------------------------------------------------------------------------------------------------
+BLOB_MAGIC = b"CGNTCSR\x00"
+BLOB_HEADER = 128
+
+
+def _blob_offsets(n: int, nnz: int):
+    up = lambda v: (v + 63) // 64 * 64
+    off_rowptr = BLOB_HEADER
+    off_colind = up(off_rowptr + 4 * (n + 1))
+    off_values = up(off_colind + 4 * nnz)
+    return off_rowptr, off_colind, off_values, up(off_values + 4 * nnz)
+
+
+def _fnv1a_words(payload: bytes) -> int:
+    h = 1469598103934665603
+    for (w,) in struct.iter_unpack("<Q", payload):
+        h = ((h ^ w) * 1099511628211) & 0xFFFFFFFFFFFFFFFF
+    return h
+
+
+def blob_write(rowptr: np.ndarray, colind: np.ndarray, values: np.ndarray, n: int, m: int, has_transpose: bool) -> bytes:
+    nnz = int(len(colind))
+    o_r, o_c, o_v, total = _blob_offsets(n, nnz)
+    buf = bytearray(total)
+    buf[o_r:o_r + 4 * (n + 1)] = np.asarray(rowptr, dtype="<i4").tobytes()
+    buf[o_c:o_c + 4 * nnz] = np.asarray(colind, dtype="<i4").tobytes()
+    buf[o_v:o_v + 4 * nnz] = np.asarray(values, dtype="<f4").tobytes()
+    head = struct.pack("<8sIIqqqQQQQQ", BLOB_MAGIC, 1, 1 if has_transpose else 0, n, m, nnz, o_r, o_c, o_v, total,
+                       _fnv1a_words(bytes(buf[BLOB_HEADER:])))
+    buf[:len(head)] = head
+    return bytes(buf)
+
+
+def blob_read(blob: bytes):
+    """(rowptr, colind, values, n, m, has_transpose); raises ValueError on a malformed blob."""
+    blob = bytes(blob)
+    if len(blob) < BLOB_HEADER:
+        raise ValueError("no header")
+    magic, version, flags, n, m, nnz, o_r, o_c, o_v, total, checksum = struct.unpack_from("<8sIIqqqQQQQQ", blob, 0)
+    if magic != BLOB_MAGIC or version != 1:
+        raise ValueError("bad magic or version")
+    if min(n, m, nnz) < 0 or (o_r, o_c, o_v, total) != _blob_offsets(n, nnz) or len(blob) < total:
+        raise ValueError("inconsistent sizes")
+    if _fnv1a_words(blob[BLOB_HEADER:total]) != checksum:
+        raise ValueError("checksum mismatch")
+    rowptr = np.frombuffer(blob, dtype="<i4", count=n + 1, offset=o_r)
+    colind = np.frombuffer(blob, dtype="<i4", count=nnz, offset=o_c)
+    values = np.frombuffer(blob, dtype="<f4", count=nnz, offset=o_v)
+    if rowptr[0] != 0 or rowptr[-1] != nnz or np.any(np.diff(rowptr) < 0):
+        raise ValueError("rowptr is not a monotone map onto [0, nnz]")
+    if nnz and (colind.min() < 0 or colind.max() >= m):
+        raise ValueError("column index out of range")
+    return rowptr, colind, values, n, m, bool(flags & 1)
 
 
 # ------------------------------------------------------------------------------------------------

@@ -347,3 +347,58 @@ def test_spmm_hub_plan_rectangular_and_all_hot(cuda, tune):
     A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, m)
     tune("spmm_hub_kb", 4096)
     assert spmm_error(A.spmm(B.to(cuda)), row, col, val, n, m, B) <= REL_TOL
+
+
+def test_blob_matches_format_restatement_and_roundtrips(cuda, tmp_path):
+    """The library's bytes equal the oracle's independent writer bit for bit; a blob written by
+    the oracle loads; a file round trip gives a handle whose products are bit-identical."""
+    from cagnet_amd import ops
+    row, col, val, n = small_graph(10, 20000, seed=21)
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n, transpose=True)
+    blob = A.to_blob()
+    rp, ci, vv, _ = orc.coo2csr(row.numpy(), col.numpy(), val.numpy(), n, n)
+    assert blob.tobytes() == orc.blob_write(rp, ci, vv, n, n, True)
+    parsed = orc.blob_read(blob.tobytes())
+    assert np.array_equal(parsed[1], ci) and parsed[5] is True
+    B = torch.randn(n, 48, generator=torch.Generator().manual_seed(3)).to(cuda)
+    A2 = ops.CsrMatrix.from_blob(orc.blob_write(rp, ci, vv, n, n, False))
+    assert not A2.has_transpose and torch.equal(A2.spmm(B), A.spmm(B))
+    path = tmp_path / "block.cgcsr"
+    A.save(path)
+    A3 = ops.CsrMatrix.load(path)
+    assert A3.has_transpose and A3.shape == (n, n) and A3.nnz == A.nnz
+    assert torch.equal(A3.spmm(B), A.spmm(B)) and torch.equal(A3.spmm(B, transpose=True), A.spmm(B, transpose=True))
+    assert all(torch.equal(x, y) for x, y in zip(A3.arrays(), A.arrays()))
+    # rectangular, empty rows at the end, and an empty block
+    r2, c2, v2 = random_coo(50, 3000, 700, 4)
+    R = ops.CsrMatrix(_i32(r2, cuda), _i32(c2, cuda), v2.to(cuda), 64, 3000)
+    R2 = ops.CsrMatrix.from_blob(R.to_blob(), transpose=True)
+    assert R2.has_transpose and all(torch.equal(x, y) for x, y in zip(R2.arrays(), R.arrays()))
+    e32 = torch.empty(0, dtype=torch.int32, device=cuda)
+    E = ops.CsrMatrix.from_blob(ops.CsrMatrix(e32, e32, torch.empty(0, device=cuda), 5, 7).to_blob())
+    assert E.nnz == 0 and E.shape == (5, 7)
+
+
+def test_blob_rejects_damage(cuda):
+    from cagnet_amd import ops
+    n, m = 40, 60
+    row, col, val = random_coo(n, m, 500, 8)
+    rp, ci, vv, _ = orc.coo2csr(row.numpy(), col.numpy(), val.numpy(), n, m)
+    good = orc.blob_write(rp, ci, vv, n, m, False)
+    ops.CsrMatrix.from_blob(good)
+    cases = {
+        "CG_ERR_UNSUPPORTED": b"X" + good[1:],
+        "CG_ERR_SIZE": good[:len(good) - 64],
+        "CG_ERR_INDEX": good[:200] + bytes([good[200] ^ 4]) + good[201:],
+    }
+    for err, blob in cases.items():
+        with pytest.raises(ops.CagnetError, match=err):
+            ops.CsrMatrix.from_blob(blob)
+    rp_bad = rp.copy(); rp_bad[3], rp_bad[4] = rp[4] + 1, rp[3]
+    with pytest.raises(ops.CagnetError, match="CG_ERR_UNSORTED"):
+        ops.CsrMatrix.from_blob(orc.blob_write(rp_bad, ci, vv, n, m, False))
+    ci_bad = ci.copy(); ci_bad[7] = m            # valid checksum, column outside the matrix
+    with pytest.raises(ops.CagnetError, match="CG_ERR_INDEX"):
+        ops.CsrMatrix.from_blob(orc.blob_write(rp, ci_bad, vv, n, m, False))
+    with pytest.raises(ops.CagnetError, match="CG_ERR_SIZE"):
+        ops.CsrMatrix.from_blob(good[:64])

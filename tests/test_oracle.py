@@ -292,3 +292,32 @@ def test_coo_block_against_scipy_slicing(seed):
     order = np.lexsort((ref.col, ref.row))
     assert np.array_equal(r, ref.row[order]) and np.array_equal(c, ref.col[order])
     assert np.array_equal(v, ref.data[order])
+
+
+def test_blob_roundtrip_layout_and_rejections():
+    """Header fields sit at the documented offsets, arrays on 64-byte boundaries, and every kind
+    of damage (magic, truncation, flipped payload bit, non-monotone rowptr, column out of range)
+    is refused."""
+    import struct
+    n, m = 37, 50
+    row, col, val = random_coo(n, m, 400, 5)
+    rp, ci, vv, _ = orc.coo2csr(row.numpy(), col.numpy(), val.numpy(), n, m)
+    blob = orc.blob_write(rp, ci, vv, n, m, True)
+    assert blob[:8] == b"CGNTCSR\x00" and struct.unpack_from("<II", blob, 8) == (1, 1)
+    assert struct.unpack_from("<qqq", blob, 16) == (n, m, 400)
+    o_r, o_c, o_v, total = struct.unpack_from("<QQQQ", blob, 40)
+    assert o_r == 128 and o_c % 64 == 0 and o_v % 64 == 0 and total == len(blob) and total % 64 == 0
+    assert np.array_equal(np.frombuffer(blob, "<i4", n + 1, o_r), rp)
+    got = orc.blob_read(blob)
+    assert np.array_equal(got[0], rp) and np.array_equal(got[1], ci) and np.array_equal(got[2], vv)
+    assert got[3:] == (n, m, True)
+    for bad in (b"X" + blob[1:], blob[:len(blob) - 64], blob[:o_v + 3] + bytes([blob[o_v + 3] ^ 1]) + blob[o_v + 4:]):
+        with pytest.raises(ValueError):
+            orc.blob_read(bad)
+    rp_bad = rp.copy(); rp_bad[3], rp_bad[4] = rp[4] + 1, rp[3]
+    ci_bad = ci.copy(); ci_bad[7] = m
+    for args in ((rp_bad, ci, vv), (rp, ci_bad, vv)):
+        with pytest.raises(ValueError):
+            orc.blob_read(orc.blob_write(*args, n, m, False))
+    empty = orc.blob_read(orc.blob_write(np.zeros(4, np.int32), np.zeros(0, np.int32), np.zeros(0, np.float32), 3, 9, False))
+    assert empty[3:] == (3, 9, False) and empty[1].size == 0
