@@ -18,8 +18,6 @@ int xw_mfma(const float *X, int64_t ldx, const float *W, int64_t ldw, float *Z, 
             int32_t fo, int relu, hipStream_t stream);
 int xtg_mfma(const float *X, int64_t ldx, const float *G, int64_t ldg, float *P, int64_t n, int32_t k, int32_t fo,
              int64_t rows_per_block, int64_t nblocks, hipStream_t stream);
-int gwt_mfma(const float *G, int64_t ldg, const float *W, int64_t ldw, float *dX, int64_t lddx, int64_t n, int32_t k,
-             int32_t fo, hipStream_t stream);
 int xtg_vec(const float *X, int64_t ldx, int32_t k);
 // dense_rows.hip
 int gwt_rows(const float *G, int64_t ldg, const float *W, int64_t ldw, float *dX, int64_t lddx, int64_t n, int32_t k,
@@ -265,10 +263,8 @@ int cg_dense_gwt(const float *d_G, int64_t ldg, const float *d_W, int64_t ldw, f
   if (n == 0) return CG_OK;
   GemmArgs g{d_G, ldg, d_W, ldw, d_dX, lddx, n, k, fo, ceil_div64(fo, kKT) * kKT, 1, 0};
   ProfScope prof("dense_gwt", k, (hipStream_t)stream);
-  // the matrix-core form pays when the result is narrow; a wide result is bound by its stores,
-  // which the vector kernel issues in longer contiguous runs
-  if (fo <= 64 && k <= 64 && g_tune_dense_mfma.load(std::memory_order_relaxed) >= 0)
-    return gwt_mfma(d_G, ldg, d_W, ldw, d_dX, lddx, n, k, fo, (hipStream_t)stream);
+  // wide result: bound by its stores, row-streaming kernel; narrow result: the LDS-tiled vector kernel
+  // (measured faster than a matrix-core form whose stores are 64-byte pieces)
   if (fo <= 64 && k > 64 && g_tune_dense_mfma.load(std::memory_order_relaxed) >= 0)
     return gwt_rows(d_G, ldg, d_W, ldw, d_dX, lddx, n, k, fo, (hipStream_t)stream);
   return launch_gemm<false, true>(g, (hipStream_t)stream);

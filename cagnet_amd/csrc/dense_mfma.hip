@@ -10,8 +10,7 @@
 //
 //   xw_mfma  : Z[n, fo]   = X[n, k] * W[k, fo]  (+ReLU)   rows of X on the tile rows, W staged in LDS
 //   xtg_mfma : dW[k, fo]  = X[n, k]^T * G[n, fo]          columns of X on the tile rows, vertices reduced
-//   gwt_mfma : dX[n, k]   = G[n, fo] * W[k, fo]^T         computed as (W G^T) so a lane owns 4 consecutive
-//                                                         outputs of one row and stores them as one vector
+// (dX = G W^T is bound by its stores and runs on the vector ALUs: dense_rows.hip, dense.hip.)
 #include "common.h"
 
 namespace cg {
@@ -46,65 +45,58 @@ __device__ __forceinline__ void load_k(const float *p, bool ok, float (&r)[VEC])
 // k-values of row m per step, which feed VEC instructions whose B operand comes from the W chunk
 // staged in LDS.  NT output tiles of 16 columns share every A value.
 // ---------------------------------------------------------------------------------------------
-constexpr int kXwChunk = 256;  // rows of W staged per pass (multiple of 16)
+constexpr int kXwChunk = 256;        // rows of W staged per pass when W does not fit LDS whole
+constexpr int kXwLdsBytes = 64 * 1024;
 
+// acc += X[rows of the wave, c0 .. c0+clen) * Ws, for the chunk of W staged in LDS (`cap` rows, zero padded)
 template <int VEC, int NT>
-__global__ __launch_bounds__(kMfmaThreads) void xw_mfma_kernel(const float *__restrict__ X, int64_t ldx,
-                                                               const float *__restrict__ W, int64_t ldw,
-                                                               float *__restrict__ Z, int64_t ldz, int64_t n,
-                                                               int32_t k, int32_t fo, int relu) {
-  __shared__ float Ws[kXwChunk][16 * NT];
-  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  const int m = lane & 15, q = lane >> 4;
-  const int64_t r0 = ((int64_t)blockIdx.x * kMfmaWaves + wave) * 16;
-  int64_t row = r0 + m;
-  if (row >= n) row = n - 1;  // clamp: the extra rows are computed and dropped
-  const float *xrow = X + row * ldx;
-
-  floatx4 acc[NT];
+__device__ __forceinline__ void xw_accumulate(const float *__restrict__ xrow, int32_t c0, int32_t clen,
+                                              const float *__restrict__ Ws, int32_t cap, int m, int q,
+                                              floatx4 (&acc)[NT]) {
+  constexpr int STEP = 4 * VEC;  // k-values one load step covers
+  constexpr int U = 4;           // load steps in flight
+  for (int32_t kb = 0; kb < clen; kb += STEP * U) {
+    float x[U][VEC];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-  for (int32_t c0 = 0; c0 < k; c0 += kXwChunk) {
-    const int32_t clen = k - c0 < kXwChunk ? k - c0 : kXwChunk;
-    __syncthreads();
-    // rows past the end of the chunk are read (as zeros) by the last load steps: stage them too
-    constexpr int kStepRows = 4 * VEC * 4;
-    const int32_t stage_rows = (clen + kStepRows - 1) / kStepRows * kStepRows < kXwChunk
-                                   ? (clen + kStepRows - 1) / kStepRows * kStepRows
-                                   : kXwChunk;
-    for (int idx = threadIdx.x; idx < stage_rows * 16 * NT; idx += kMfmaThreads) {
-      const int kk = idx / (16 * NT), c = idx % (16 * NT);
-      Ws[kk][c] = (kk < clen && c < fo) ? W[(int64_t)(c0 + kk) * ldw + c] : 0.f;
-    }
-    __syncthreads();
-    constexpr int STEP = 4 * VEC;  // k-values one load step covers
-    constexpr int U = 4;           // load steps in flight
-    for (int32_t kb = 0; kb < clen; kb += STEP * U) {
-      float x[U][VEC];
+    for (int u = 0; u < U; ++u) {
+      const int32_t kk = kb + u * STEP + q * VEC;
+      load_k<VEC>(xrow + c0 + kk, kk + VEC <= clen, x[u]);
+      if (VEC > 1 && kk < clen && kk + VEC > clen) {  // ragged end of the row: element-wise
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int32_t kk = kb + u * STEP + q * VEC;
-        load_k<VEC>(xrow + c0 + kk, kk + VEC <= clen, x[u]);
-        if (VEC > 1 && kk < clen && kk + VEC > clen) {  // ragged end of the row: element-wise
-#pragma unroll
-          for (int s = 0; s < VEC; ++s) x[u][s] = kk + s < clen ? xrow[c0 + kk + s] : 0.f;
-        }
+        for (int s = 0; s < VEC; ++s) x[u][s] = kk + s < clen ? xrow[c0 + kk + s] : 0.f;
       }
+    }
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
+    for (int u = 0; u < U; ++u) {
 #pragma unroll
-        for (int s = 0; s < VEC; ++s) {
-          const int32_t kk = kb + u * STEP + q * VEC + s;
-          if (kb + u * STEP < clen) {  // wave-uniform: skip steps past the chunk
-            const float *wrow = Ws[kk < kXwChunk ? kk : kXwChunk - 1];
+      for (int s = 0; s < VEC; ++s) {
+        const int32_t kk = kb + u * STEP + q * VEC + s;
+        if (kb + u * STEP < clen) {  // wave-uniform: skip steps past the chunk
+          const float *wrow = Ws + (size_t)(kk < cap ? kk : cap - 1) * (16 * NT);
 #pragma unroll
-            for (int t = 0; t < NT; ++t) acc[t] = mfma16(x[u][s], wrow[t * 16 + m], acc[t]);
-          }
+          for (int t = 0; t < NT; ++t) acc[t] = mfma16(x[u][s], wrow[t * 16 + m], acc[t]);
         }
       }
     }
   }
+}
+
+// rows past the end of the chunk are read (as zeros) by the last load steps: they are staged too
+template <int VEC, int NT>
+__device__ __forceinline__ void xw_stage(const float *__restrict__ W, int64_t ldw, int32_t c0, int32_t clen,
+                                         int32_t fo, float *__restrict__ Ws, int32_t cap) {
+  constexpr int kStepRows = 4 * VEC * 4;
+  int32_t stage_rows = (clen + kStepRows - 1) / kStepRows * kStepRows;
+  if (stage_rows > cap) stage_rows = cap;
+  for (int idx = threadIdx.x; idx < stage_rows * 16 * NT; idx += kMfmaThreads) {
+    const int kk = idx / (16 * NT), c = idx % (16 * NT);
+    Ws[idx] = (kk < clen && c < fo) ? W[(int64_t)(c0 + kk) * ldw + c] : 0.f;
+  }
+}
+
+template <int NT>
+__device__ __forceinline__ void xw_store(const floatx4 (&acc)[NT], float *__restrict__ Z, int64_t ldz, int64_t r0,
+                                         int64_t n, int32_t fo, int relu, int m, int q) {
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
 #pragma unroll
@@ -118,6 +110,48 @@ __global__ __launch_bounds__(kMfmaThreads) void xw_mfma_kernel(const float *__re
       }
     }
   }
+}
+
+// cap: rows of W the LDS buffer holds.  cap >= k: W is staged once and the workgroup then walks row
+// tiles (grid-stride) without another barrier; otherwise one row tile per workgroup, W in chunks.
+template <int VEC, int NT>
+__global__ __launch_bounds__(kMfmaThreads) void xw_mfma_kernel(const float *__restrict__ X, int64_t ldx,
+                                                               const float *__restrict__ W, int64_t ldw,
+                                                               float *__restrict__ Z, int64_t ldz, int64_t n,
+                                                               int32_t k, int32_t fo, int relu, int32_t cap) {
+  extern __shared__ float Ws[];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int m = lane & 15, q = lane >> 4;
+  const int64_t tiles = (n + 16 * kMfmaWaves - 1) / (16 * kMfmaWaves);
+  if (cap >= k) {
+    xw_stage<VEC, NT>(W, ldw, 0, k, fo, Ws, cap);
+    __syncthreads();
+    for (int64_t tb = blockIdx.x; tb < tiles; tb += gridDim.x) {
+      const int64_t r0 = (tb * kMfmaWaves + wave) * 16;
+      int64_t row = r0 + m;
+      if (row >= n) row = n - 1;  // clamp: the extra rows are computed and dropped
+      floatx4 acc[NT];
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+      xw_accumulate<VEC, NT>(X + row * ldx, 0, k, Ws, cap, m, q, acc);
+      xw_store<NT>(acc, Z, ldz, r0, n, fo, relu, m, q);
+    }
+    return;
+  }
+  const int64_t r0 = ((int64_t)blockIdx.x * kMfmaWaves + wave) * 16;
+  int64_t row = r0 + m;
+  if (row >= n) row = n - 1;
+  floatx4 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int32_t c0 = 0; c0 < k; c0 += cap) {
+    const int32_t clen = k - c0 < cap ? k - c0 : cap;
+    __syncthreads();
+    xw_stage<VEC, NT>(W, ldw, c0, clen, fo, Ws, cap);
+    __syncthreads();
+    xw_accumulate<VEC, NT>(X + row * ldx, c0, clen, Ws, cap, m, q, acc);
+  }
+  xw_store<NT>(acc, Z, ldz, r0, n, fo, relu, m, q);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -186,62 +220,6 @@ __global__ __launch_bounds__(kMfmaThreads) void xtg_mfma_kernel(const float *__r
 }
 
 // ---------------------------------------------------------------------------------------------
-// dX = G W^T, computed tile-wise as (W G^T): tile rows are 16 columns of dX (= rows of W), tile
-// columns are 16 vertices.  Register v of lane (j, q) then holds dX[r + j][kt + 4q + v], four
-// consecutive outputs of one row, stored as one vector.  The G values of the 16 vertices are kept
-// in registers across all column tiles.
-// ---------------------------------------------------------------------------------------------
-template <int KS>  // reduction steps: fo <= 4 * KS
-__global__ __launch_bounds__(kMfmaThreads) void gwt_mfma_kernel(const float *__restrict__ G, int64_t ldg,
-                                                                const float *__restrict__ W, int64_t ldw,
-                                                                float *__restrict__ dX, int64_t lddx, int64_t n,
-                                                                int32_t k, int32_t fo, int32_t tiles_per_wave) {
-  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  const int j = lane & 15, q = lane >> 4;
-  const int64_t r0 = ((int64_t)blockIdx.x * kMfmaWaves + wave) * 16;
-  if (r0 >= n) return;
-  int64_t grow = r0 + j;
-  const bool row_ok = grow < n;
-  if (!row_ok) grow = n - 1;
-  float g[KS];
-#pragma unroll
-  for (int s = 0; s < KS; ++s) {
-    const int32_t c = 4 * s + q;
-    g[s] = c < fo ? G[grow * ldg + c] : 0.f;
-  }
-  const int32_t ktiles = (k + 15) / 16;
-  const int32_t t_begin = blockIdx.y * tiles_per_wave;
-  const int32_t t_end = t_begin + tiles_per_wave < ktiles ? t_begin + tiles_per_wave : ktiles;
-  const bool st4 = (lddx % 4 == 0) && (((uintptr_t)dX) % 16 == 0);
-  const bool st2 = (lddx % 2 == 0) && (((uintptr_t)dX) % 8 == 0);
-  for (int32_t t = t_begin; t < t_end; ++t) {
-    const int32_t kt = t * 16;
-    const int32_t wr = kt + j < k ? kt + j : k - 1;  // A side: lane (m = j, q) reads W[kt + m][4 s + q]
-    floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const int32_t c = 4 * s + q;
-      const float w = c < fo ? W[(int64_t)wr * ldw + c] : 0.f;
-      acc = mfma16(w, g[s], acc);
-    }
-    if (row_ok) {
-      const int32_t c0 = kt + 4 * q;
-      float *dst = dX + (r0 + j) * lddx + c0;
-      if (c0 + 4 <= k && st4) {
-        *reinterpret_cast<float4 *>(dst) = make_float4(acc[0], acc[1], acc[2], acc[3]);
-      } else if (c0 + 4 <= k && st2) {
-        *reinterpret_cast<float2 *>(dst) = make_float2(acc[0], acc[1]);
-        *reinterpret_cast<float2 *>(dst + 2) = make_float2(acc[2], acc[3]);
-      } else {
-#pragma unroll
-        for (int v = 0; v < 4; ++v)
-          if (c0 + v < k) dst[v] = acc[v];
-      }
-    }
-  }
-}
-
-// ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
 static int pick_kvec(const float *X, int64_t ldx, int32_t k) {
@@ -254,12 +232,24 @@ int xw_mfma(const float *X, int64_t ldx, const float *W, int64_t ldw, float *Z, 
             int32_t fo, int relu, hipStream_t stream) {
   const int nt = (fo + 15) / 16;
   const int vec = pick_kvec(X, ldx, k);
-  const int64_t blocks = ceil_div64(n, 16 * kMfmaWaves);
-  if (blocks > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "cg_dense_xw: grid too large");
+  const int64_t tiles = ceil_div64(n, 16 * kMfmaWaves);
+  if (tiles > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "cg_dense_xw: grid too large");
+  // W whole in LDS when it fits (rows rounded up to what the last load steps touch)
+  const int step_rows = 4 * vec * 4;
+  const int64_t whole = ceil_div64(k, step_rows) * step_rows;
+  const size_t row_bytes = (size_t)16 * nt * sizeof(float);
+  int32_t cap = kXwChunk;
+  int64_t blocks = tiles;
+  if ((size_t)whole * row_bytes <= (size_t)kXwLdsBytes) {
+    cap = (int32_t)whole;
+    const int64_t resident = 256 * 8;  // workgroups that keep every CU busy; each walks several row tiles
+    if (blocks > resident) blocks = resident;
+  }
   const unsigned grid = (unsigned)blocks;
+  const size_t lds = (size_t)cap * row_bytes;
 #define CG_CASE(V, T)                                                                                         \
   if (vec == V && nt == T) {                                                                                  \
-    xw_mfma_kernel<V, T><<<grid, kMfmaThreads, 0, stream>>>(X, ldx, W, ldw, Z, ldz, n, k, fo, relu);          \
+    xw_mfma_kernel<V, T><<<grid, kMfmaThreads, lds, stream>>>(X, ldx, W, ldw, Z, ldz, n, k, fo, relu, cap);   \
     CG_LAUNCH_CHECK();                                                                                        \
     return CG_OK;                                                                                             \
   }
@@ -286,10 +276,10 @@ int xtg_mfma(const float *X, int64_t ldx, const float *G, int64_t ldg, float *P,
   // narrow X: fewer wavefronts per workgroup, so none of them is without columns
   const int wpb = ywaves < kMfmaWaves ? (int)ywaves : kMfmaWaves;
   dim3 grid((unsigned)nblocks, (unsigned)ceil_div64(ywaves, wpb));
-  const unsigned kMfmaThreads = (unsigned)(wpb * kWave);  // shadows the constant inside this function
+  const unsigned threads = (unsigned)(wpb * kWave);
 #define CG_CASE(V, T)                                                                                         \
   if (vec == V && nt == T) {                                                                                  \
-    xtg_mfma_kernel<V, T><<<grid, kMfmaThreads, 0, stream>>>(X, ldx, G, ldg, P, n, k, fo, rows_per_block);    \
+    xtg_mfma_kernel<V, T><<<grid, threads, 0, stream>>>(X, ldx, G, ldg, P, n, k, fo, rows_per_block);    \
     CG_LAUNCH_CHECK();                                                                                        \
     return CG_OK;                                                                                             \
   }
@@ -298,28 +288,6 @@ int xtg_mfma(const float *X, int64_t ldx, const float *G, int64_t ldg, float *P,
 #undef CG_CASES
 #undef CG_CASE
   CG_FAIL(CG_ERR_UNSUPPORTED, "cg_dense_xtg: fo=%d has no matrix-core variant", fo);
-}
-
-int gwt_mfma(const float *G, int64_t ldg, const float *W, int64_t ldw, float *dX, int64_t lddx, int64_t n, int32_t k,
-             int32_t fo, hipStream_t stream) {
-  const int ks = (fo + 3) / 4;
-  const int64_t xblocks = ceil_div64(n, 16 * kMfmaWaves);
-  if (xblocks > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "cg_dense_gwt: grid too large");
-  // few vertex tiles (small n): split the output columns over grid.y to fill the chip
-  const int32_t ktiles = (k + 15) / 16;
-  int32_t ysplit = 1;
-  if (xblocks < 1024) ysplit = (int32_t)(ceil_div64(1024, xblocks) < ktiles ? ceil_div64(1024, xblocks) : ktiles);
-  const int32_t tiles_per_wave = (ktiles + ysplit - 1) / ysplit;
-  dim3 grid((unsigned)xblocks, (unsigned)((ktiles + tiles_per_wave - 1) / tiles_per_wave));
-#define CG_CASE(S)                                                                                            \
-  if (ks <= S) {                                                                                              \
-    gwt_mfma_kernel<S><<<grid, kMfmaThreads, 0, stream>>>(G, ldg, W, ldw, dX, lddx, n, k, fo, tiles_per_wave); \
-    CG_LAUNCH_CHECK();                                                                                        \
-    return CG_OK;                                                                                             \
-  }
-  CG_CASE(2) CG_CASE(4) CG_CASE(8) CG_CASE(16)
-#undef CG_CASE
-  CG_FAIL(CG_ERR_UNSUPPORTED, "cg_dense_gwt: fo=%d has no matrix-core variant", fo);
 }
 
 }  // namespace cg
