@@ -279,6 +279,41 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_stream_wide_kernel(const St
 constexpr int kNarrowLds = 1024;  // entries a window may hold (window length S plus one task, both <= 512)
 constexpr int kLongFactor = 4;
 
+// acc += sum over u < U of val[i + u * stride] * B[col[i + u * stride], own columns]: U rows of B in flight
+template <int VEC, int U>
+__device__ __forceinline__ void narrow_gather(const int32_t *cw, const float *vw, int32_t i, int stride,
+                                              const float *__restrict__ B, int64_t ldb, int64_t boff,
+                                              float (&acc)[VEC]) {
+  float b[U][VEC], vv[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int32_t cc = cw[i + u * stride];
+    vv[u] = vw[i + u * stride];
+    load_vec<VEC>(B + (int64_t)cc * ldb + boff, b[u]);
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+#pragma unroll
+    for (int q = 0; q < VEC; ++q) acc[q] = fmaf(vv[u], b[u][q], acc[q]);
+}
+
+// entries i, i + stride, ... below e, in that order: blocks of 8, then 4, 2, 1
+template <int VEC>
+__device__ __forceinline__ void narrow_sweep(const int32_t *cw, const float *vw, int32_t i, int32_t e, int stride,
+                                             const float *__restrict__ B, int64_t ldb, int64_t boff,
+                                             float (&acc)[VEC]) {
+  for (; i + 7 * stride < e; i += 8 * stride) narrow_gather<VEC, 8>(cw, vw, i, stride, B, ldb, boff, acc);
+  if (i + 3 * stride < e) {
+    narrow_gather<VEC, 4>(cw, vw, i, stride, B, ldb, boff, acc);
+    i += 4 * stride;
+  }
+  if (i + stride < e) {
+    narrow_gather<VEC, 2>(cw, vw, i, stride, B, ldb, boff, acc);
+    i += 2 * stride;
+  }
+  if (i < e) narrow_gather<VEC, 1>(cw, vw, i, stride, B, ldb, boff, acc);
+}
+
 template <int VEC, int LPR>
 __global__ __launch_bounds__(kSpmmThreads) void spmm_stream_narrow_kernel(const StreamArgs a) {
   constexpr int G = kWave / LPR;
@@ -349,27 +384,7 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_stream_narrow_kernel(const 
     float acc[VEC];
 #pragma unroll
     for (int q = 0; q < VEC; ++q) acc[q] = 0.f;
-    int32_t i = s + g;
-    for (; i + 3 * G < e; i += 4 * G) {
-      float b[4][VEC], vv[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int32_t cc = cw[i + u * G];
-        vv[u] = vw[i + u * G];
-        load_vec<VEC>(a.B + (int64_t)cc * a.ldb + boff, b[u]);
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-#pragma unroll
-        for (int q = 0; q < VEC; ++q) acc[q] = fmaf(vv[u], b[u][q], acc[q]);
-    }
-    for (; i < e; i += G) {
-      float b[VEC];
-      const float vv = vw[i];
-      load_vec<VEC>(a.B + (int64_t)cw[i] * a.ldb + boff, b);
-#pragma unroll
-      for (int q = 0; q < VEC; ++q) acc[q] = fmaf(vv, b[q], acc[q]);
-    }
+    narrow_sweep<VEC>(cw, vw, s + g, e, G, a.B, a.ldb, boff, acc);
 #pragma unroll
     for (int off = LPR; off < kWave; off <<= 1)
 #pragma unroll
@@ -405,27 +420,7 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_stream_narrow_kernel(const 
     float acc[VEC];
 #pragma unroll
     for (int q = 0; q < VEC; ++q) acc[q] = 0.f;
-    int32_t i = s;
-    for (; i + 3 < e; i += 4) {
-      float b[4][VEC], vv[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int32_t cc = cw[i + u];
-        vv[u] = vw[i + u];
-        load_vec<VEC>(a.B + (int64_t)cc * a.ldb + boff, b[u]);
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-#pragma unroll
-        for (int q = 0; q < VEC; ++q) acc[q] = fmaf(vv[u], b[u][q], acc[q]);
-    }
-    for (; i < e; ++i) {
-      float b[VEC];
-      const float vv = vw[i];
-      load_vec<VEC>(a.B + (int64_t)cw[i] * a.ldb + boff, b);
-#pragma unroll
-      for (int q = 0; q < VEC; ++q) acc[q] = fmaf(vv, b[q], acc[q]);
-    }
+    narrow_sweep<VEC>(cw, vw, s, e, 1, a.B, a.ldb, boff, acc);
     if (has && active) {
       if (d >= 0) {
         float *crow = a.C + (int64_t)d * a.ldc + boff;
