@@ -32,6 +32,22 @@ def test_every_declaration_cites_the_reference_or_says_it_has_no_counterpart():
     assert "sparse-extension/sparse_coo_tensor.cu:113-240" in text     # spmm_gpu
     assert "sparse_coo_tensor.cu:136-142" in text                      # coo2csr
     assert "gcn_distr.py:275" in text and "gcn_distr.py:284-294" in text  # dense products, activations and loss
+    assert "gcn_distr.py:791" in text and "gcn_distr.py:412-470" in text and "gcn_distr.py:398-409" in text  # preparation
+    assert "gcn_distr.py:747" in text and "gcn_distr_2d.py:369-374" in text  # block format
+
+
+def test_header_is_plain_c_and_cplusplus(tmp_path):
+    """The boundary is a C ABI: the header must compile as C99 and as C++11 with nothing but <stdint.h>."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("gcc not available")
+    src = tmp_path / "use.c"
+    src.write_text('#include "cagnet_amd.h"\nint main(void) { return cg_abi_version() == CG_ABI_VERSION ? 0 : 1; }\n')
+    inc = str(HEADER.parent)
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-fsyntax-only", "-I", inc, str(src)],
+                   check=True)
+    subprocess.run(["g++", "-std=c++11", "-Wall", "-Werror", "-fsyntax-only", "-x", "c++", "-I", inc, str(src)], check=True)
 
 
 def test_status_codes_without_a_gpu():
@@ -65,6 +81,21 @@ def test_status_codes_without_a_gpu():
     assert lib.cg_relu_fwd(null, one, 5, null) == E["null"]
     assert lib.cg_log_softmax_fwd(one, 3, one, 4, 10, 4, null) == E["size"]
     assert lib.cg_nll_loss_fwd(one, 4, one, null, 10, 4, null, one, null) == E["null"]
+    count = ctypes.c_int64(-1)
+    assert lib.cg_add_self_loops(null, null, 5, 4, null, null, 0, ctypes.byref(count), null) == E["null"]
+    assert lib.cg_add_self_loops(one, one, 5, 4, null, null, 0, None, null) == E["null"]
+    assert lib.cg_add_self_loops(one, one, -1, 4, null, null, 0, ctypes.byref(count), null) == E["size"]
+    assert lib.cg_gcn_normalize(one, one, 1 << 31, 4, one, null, null) == E["overflow"]
+    assert lib.cg_gcn_normalize(one, null, 5, 4, one, null, null) == E["null"]
+    assert lib.cg_coo_block(one, one, null, 5, 3, 2, 0, 4, null, null, null, 0, ctypes.byref(count), null) == E["size"]
+    assert lib.cg_coo_block(one, one, null, 0, 0, 2, 0, 4, null, null, null, 0, ctypes.byref(count), null) == 0
+    assert count.value == 0
+    h2 = ctypes.c_void_p(0)
+    junk = (ctypes.c_uint8 * 256)()
+    assert lib.cg_csr_blob_read(ctypes.byref(h2), junk, 256, 0, null) == E["unsupported"]        # bad magic
+    assert lib.cg_csr_blob_read(ctypes.byref(h2), junk, 64, 0, null) == E["size"]                # no room for a header
+    assert lib.cg_csr_blob_read(ctypes.byref(h2), null, 256, 0, null) == E["null"]
+    assert lib.cg_csr_blob_size(null, ctypes.byref(count)) == E["null"]
     assert lib.cg_tune_set(b"no_such_knob", 1) == E["unsupported"]
     assert lib.cg_tune_set(b"spmm_seg", 0) == 0
     for code in range(0, 11):
