@@ -56,9 +56,32 @@ def training_case(name: str) -> None:
                         w2_after=w2.numpy())
 
 
+def prep_case(name: str) -> None:
+    """Raw pattern -> self-loops -> normalised values -> one block of a 3 x 3 partition -> blob."""
+    rng = np.random.default_rng(41)
+    n = 97
+    key = np.sort(rng.choice(n * n, size=700, replace=False))
+    row, col = (key // n).astype(np.int32), (key % n).astype(np.int32)      # holds a few of the 97 diagonal entries
+    lr, lc = orc.add_self_loops(row, col, n)
+    val = orc.gcn_normalize(lr, lc, n)
+    b = orc.block_bounds_2d(n, 3)
+    br, bc, bv = orc.coo_block(lr, lc, val, b[1], b[2], b[2], b[3])
+    rp, ci, vv, _ = orc.coo2csr(lr, lc, val, n, n)
+    blob = np.frombuffer(orc.blob_write(rp, ci, vv, n, n, True), dtype=np.uint8)
+    np.savez_compressed(OUT / f"{name}.npz", n=n, row=row, col=col, loops_row=lr.astype(np.int32),
+                        loops_col=lc.astype(np.int32), values=val, bounds=np.array(b), block_row=br.astype(np.int32),
+                        block_col=bc.astype(np.int32), block_val=bv, blob=blob)
+
+
 if __name__ == "__main__":
-    graph_case("graph_s6_f5", 6, 400, 5, 31)
-    graph_case("graph_s8_f41", 8, 2500, 41, 32)
-    training_case("train_s7")
+    only = set(sys.argv[1:])  # optional: names of the cases to (re)write; default all
+    cases = {"graph_s6_f5": lambda: graph_case("graph_s6_f5", 6, 400, 5, 31),
+             "graph_s8_f41": lambda: graph_case("graph_s8_f41", 8, 2500, 41, 32),
+             "train_s7": lambda: training_case("train_s7"),
+             "prep_n97": lambda: prep_case("prep_n97")}
+    for key, make in cases.items():
+        if not only or key in only:
+            make()
     for f in sorted(OUT.glob("*.npz")):
         print(f.name, f.stat().st_size, "bytes")
+    sys.exit(0)

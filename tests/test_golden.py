@@ -96,3 +96,40 @@ def test_gpu_matches_training_vectors(cuda):
         gcn.train(d("x"), w1, w2, n, [blk], opt, Data, 0, 1, None)
         losses.append(float(gcn.train.last_loss))
     assert np.max(np.abs(np.array(losses) - g["sgd_losses_f64"])) <= LOSS_TOL
+
+
+def test_oracle_reproduces_preparation_and_blob_vectors():
+    g = _load("prep_n97")
+    n = int(g["n"])
+    lr, lc = orc.add_self_loops(g["row"], g["col"], n)
+    assert np.array_equal(lr, g["loops_row"]) and np.array_equal(lc, g["loops_col"])
+    already = int(np.count_nonzero(g["row"] == g["col"]))
+    assert 0 < already < n and len(lr) == len(g["row"]) - already + n   # some diagonal entries were there, not all
+    val = orc.gcn_normalize(lr, lc, n)
+    assert np.array_equal(val, g["values"])
+    b = [int(v) for v in g["bounds"]]
+    br, bc, bv = orc.coo_block(lr, lc, val, b[1], b[2], b[2], b[3])
+    assert np.array_equal(br, g["block_row"]) and np.array_equal(bc, g["block_col"]) and np.array_equal(bv, g["block_val"])
+    rp, ci, vv, nn, mm, has_t = orc.blob_read(g["blob"].tobytes())
+    assert (nn, mm, has_t) == (n, n, True) and np.array_equal(vv, val)
+    assert np.array_equal(orc.csr_expand_rows(rp), lr) and np.array_equal(ci, lc)
+
+
+@pytest.mark.gpu
+def test_gpu_matches_preparation_and_blob_vectors(cuda):
+    from cagnet_amd import ops
+    g = _load("prep_n97")
+    n = int(g["n"])
+    d = lambda k: torch.from_numpy(g[k]).to(cuda)
+    lr, lc = ops.add_self_loops(d("row"), d("col"), n)
+    assert np.array_equal(lr.cpu().numpy(), g["loops_row"]) and np.array_equal(lc.cpu().numpy(), g["loops_col"])
+    val = ops.gcn_normalize(lr, lc, n)
+    assert np.array_equal(val.cpu().numpy(), g["values"])
+    b = [int(v) for v in g["bounds"]]
+    br, bc, bv = ops.coo_block(lr, lc, val, b[1], b[2], b[2], b[3])
+    assert np.array_equal(br.cpu().numpy(), g["block_row"]) and np.array_equal(bc.cpu().numpy(), g["block_col"])
+    assert np.array_equal(bv.cpu().numpy(), g["block_val"])
+    A = ops.CsrMatrix(lr, lc, val, n, n, transpose=True)
+    assert np.array_equal(A.to_blob(), g["blob"])
+    A2 = ops.CsrMatrix.from_blob(g["blob"])
+    assert all(torch.equal(x, y) for x, y in zip(A2.arrays(), A.arrays()))
