@@ -75,6 +75,52 @@ def broad_func(node_count: int, am_partitions: Sequence[CsrMatrix], inputs: torc
     return z_loc
 
 
+def stage_schedule_15d(rank: int, size: int, replication: int) -> List[tuple]:
+    """Stages of one rank in the 1.5D algorithm (gcn_distr_15d.py:194-208): a list of
+    (source rank q, block id).  The P/c block columns of a block row are dealt to the c replicas of
+    that row, P/c^2 consecutive ones each; the last replica also takes what is left over."""
+    if replication < 1 or size % replication != 0 or size // (replication ** 2) < 1:
+        raise ValueError(f"size {size} is not a multiple of replication {replication} squared blocks")
+    rank_col = rank % replication
+    per_replica = size // (replication ** 2)
+    stages = per_replica
+    if rank_col == replication - 1:
+        stages = (size // replication) - (replication - 1) * per_replica
+    out = []
+    for i in range(stages):
+        block = rank_col * per_replica + i
+        out.append((block * replication + rank_col, block))
+    return out
+
+
+def broad_func_15d(node_count: int, am_partitions: Sequence[CsrMatrix], inputs: torch.Tensor, rank: int, size: int,
+                   replication: int, group: Optional[Sequence[Optional[torch.Tensor]]] = None,
+                   replica_partials: Optional[Sequence[torch.Tensor]] = None, transpose: bool = False) -> torch.Tensor:
+    """This rank's share of the 1.5D stage loop (gcn_distr_15d.py:173-245) without the broadcasts:
+    z_loc = sum over its stages of am_partitions[block] @ H_block, where `am_partitions` are the
+    P/c blocks of the rank's block row and `group[block]` the resident H block of that stage (the
+    rank's own `inputs` when the stage's source is the rank itself).  The reference then sums
+    z_loc over the c replicas of the row with an all-reduce (:239); `replica_partials`, when given,
+    stands for the other replicas' results and is added in order."""
+    if len(am_partitions) != size // replication:
+        raise ValueError(f"{len(am_partitions)} sparse blocks for {size // replication} block columns")
+    z_loc = None
+    for q, block in stage_schedule_15d(rank, size, replication):
+        h = inputs if q == rank else (group[block] if group is not None else None)
+        if h is None:
+            raise ValueError(f"stage of block {block}: resident block is missing")
+        blk = am_partitions[block]
+        if z_loc is None:
+            z_loc = blk.spmm(h, transpose=transpose)
+        else:
+            blk.spmm(h, out=z_loc, beta=1.0, transpose=transpose)
+    if z_loc is None:
+        raise ValueError("rank has no stage")
+    for part in replica_partials or ():
+        z_loc = z_loc + part
+    return z_loc
+
+
 def outer_product2(inputs_t: torch.Tensor, ag: torch.Tensor, rank: int = 0, size: int = 1, group=None) -> torch.Tensor:
     """grad_weight = H^T @ AG (gcn_distr.py:178-201 without the all-reduce).  Takes H^T like the
     reference; the kernel reads H itself, so the transpose view is undone without a copy."""

@@ -12,6 +12,7 @@ the reference has no tests or golden vectors, so this is an independent restatem
   csr_transpose    (the A^T the reference never builds; it reuses A, gcn_distr.py:326)
   spmm             spmm_gpu, C += A B          sparse-extension/sparse_coo_tensor.cu:113-240
                    == the torch.sparse line the reference keeps commented, gcn_distr_3d.py:478
+  stage_schedule_15d  stages of a rank         gcn_distr_15d.py:194-208
   stage_loop       broad_func                  gcn_distr.py:203-246 (1.5D: gcn_distr_15d.py:197-234,
                                                2D: gcn_distr_2d.py:333-417), broadcasts removed
   GCNFuncOracle    GCNFunc                     gcn_distr.py:248-339
@@ -117,6 +118,21 @@ def stage_loop(blocks: Sequence[torch.Tensor], dense: Sequence[torch.Tensor], dt
     for a, h in zip(blocks, dense):
         z = z + torch.sparse.mm(a.to(dtype), h.to(dtype))
     return z
+
+
+def stage_schedule_15d(rank: int, size: int, replication: int):
+    """(source rank, block id) per stage of a rank in the 1.5D algorithm, restated from
+    gcn_distr_15d.py:194-208: stages = P // c^2, the last replica column takes the remainder
+    (:197-199); q = (rank_col * (P // c^2) + i) * c + rank_col (:204); block id = q // c (:208)."""
+    rank_col = rank % replication
+    stages = size // replication ** 2
+    if rank_col == replication - 1:
+        stages = size // replication - (replication - 1) * stages
+    sched = []
+    for i in range(stages):
+        q = (rank_col * (size // replication ** 2) + i) * replication + rank_col
+        sched.append((q, rank_col * (size // replication ** 2) + i))
+    return sched
 
 
 # ------------------------------------------------------------------------------------------------

@@ -122,6 +122,47 @@ def test_one_rank_share_of_2d_grid(cuda):
     _close(x.grad, ref["dx"], "dx")
 
 
+def test_one_rank_share_of_15d(cuda):
+    """The 1.5D stage loop (gcn_distr_15d.py:173-245) of the two replicas of one block row, P = 8,
+    c = 2: each replica multiplies its own two block columns; adding the other replica's partial
+    result (what the all-reduce would deliver) gives the whole block row of A H."""
+    from cagnet_amd import gcn, ops
+    size, c = 8, 2
+    p = synth.make_problem(n=1999, target_nnz=50001, features=48, hidden=16, classes=7, mask_fraction=0.5, seed=9)
+    b = synth.block_bounds_1d(p.n, size // c)                  # 4 block rows / columns of ceil(n / 4)
+    assert b == orc.block_bounds_1d(p.n, size // c)
+    row_id = 2
+    rows = b[row_id + 1] - b[row_id]
+    blocks_gpu, blocks_cpu, h_blocks = [], [], []
+    gen = torch.Generator().manual_seed(23)
+    H = torch.randn(p.n, 48, generator=gen)
+    for k in range(size // c):
+        rr, cc, vv = synth.coo_block(p.row, p.col, p.val, b[row_id], b[row_id + 1], b[k], b[k + 1])
+        blocks_gpu.append(ops.CsrMatrix(rr.int().to(cuda), cc.int().to(cuda), vv.to(cuda), rows, b[k + 1] - b[k]))
+        blocks_cpu.append(orc.coo_tensor(rr, cc, vv, rows, b[k + 1] - b[k], torch.float64))
+        h_blocks.append(H[b[k]:b[k + 1]])
+    partial = {}
+    for col in range(c):
+        rank = row_id * c + col
+        sched = gcn.stage_schedule_15d(rank, size, c)
+        own = [blk for q, blk in sched if q == rank]
+        inputs = h_blocks[own[0]].to(cuda) if own else torch.empty(0, 48, device=cuda)
+        group = [None if (own and k == own[0]) else h_blocks[k].to(cuda) for k in range(size // c)]
+        z = gcn.broad_func_15d(p.n, blocks_gpu, inputs, rank, size, c, group=group)
+        ref = orc.stage_loop([blocks_cpu[blk] for _, blk in sched], [h_blocks[blk] for _, blk in sched], torch.float64)
+        _close(z, ref, f"replica {col} partial")
+        partial[col] = z
+    rank = row_id * c + 1                                        # replica 1 (whose own block is a stage) receives replica 0's sum
+    sched = gcn.stage_schedule_15d(rank, size, c)
+    own = [blk for q, blk in sched if q == rank]
+    assert own == [row_id]
+    group = [None if k == own[0] else h_blocks[k].to(cuda) for k in range(size // c)]
+    z_row = gcn.broad_func_15d(p.n, blocks_gpu, h_blocks[own[0]].to(cuda), rank, size, c, group=group,
+                               replica_partials=[partial[0]])
+    whole = orc.stage_loop(blocks_cpu, h_blocks, torch.float64)
+    _close(z_row, whole, "block row after the replica sum")
+
+
 def test_reordered_forward_matches_reference_order(cuda):
     """Opt-in product order Z = A (H W): same outputs and gradients as (A H) W up to rounding."""
     from cagnet_amd import gcn

@@ -6,6 +6,7 @@ import sys
 from pathlib import Path
 
 import numpy as np
+import pytest
 import torch
 
 from cagnet_amd import synth
@@ -65,3 +66,24 @@ def test_bench_accounting_and_gpu_count_guard():
     assert abs(reddit - 2.04e9) < 0.01e9
     proc = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert proc.returncode != 0 and "ONE GPU" in proc.stderr
+
+
+@pytest.mark.parametrize("size,c", [(16, 2), (8, 2), (4, 1), (9, 3), (12, 2), (20, 2)])
+def test_stage_schedule_15d_covers_every_block_once(size, c):
+    """Over the c replicas of a block row the stages cover the P/c block columns exactly once, the
+    source of a stage sits in the stage's block row and the rank's replica column, and the host
+    schedule equals the oracle's restatement (gcn_distr_15d.py:194-208)."""
+    from cagnet_amd import gcn
+    from oracle import gcn_oracle as orc
+    for row in range(size // c):
+        seen = []
+        for col in range(c):
+            rank = row * c + col
+            sched = gcn.stage_schedule_15d(rank, size, c)
+            assert sched == orc.stage_schedule_15d(rank, size, c)
+            for q, block in sched:
+                assert q // c == block and q % c == col
+            seen += [b for _, b in sched]
+        assert sorted(seen) == list(range(size // c))
+    with pytest.raises(ValueError):
+        gcn.stage_schedule_15d(0, 6, 4)
