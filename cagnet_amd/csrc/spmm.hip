@@ -602,10 +602,15 @@ struct CsrSide {
   float *val = nullptr;
   int32_t max_degree = 0;
   SchedCache sched;
-  HubPlan hub;
+  // Hub plans depend on the product width (through the number of hot columns); a model with two
+  // wide layers alternates between two of them, so two are kept and the older one is replaced.
+  static constexpr int kHubPlans = 2;
+  HubPlan hub[kHubPlans];
+  uint64_t hub_used[kHubPlans] = {0, 0};
+  uint64_t hub_clock = 0;
   void release() {
     sched.release();
-    hub.release();
+    for (int i = 0; i < kHubPlans; ++i) hub[i].release();
     if (rowptr) (void)hipFree(rowptr);
     if (colind) (void)hipFree(colind);
     if (val) (void)hipFree(val);
@@ -677,8 +682,8 @@ __global__ __launch_bounds__(kSpmmThreads) void csr_rows_kernel(const int32_t *_
   for (int32_t k = s + lane; k < e; k += kWave) row_out[k] = (int32_t)wave;
 }
 
-static int build_hub(CsrSide &s, int32_t hot, int32_t groups, int32_t tiers, int32_t seg, hipStream_t stream) {
-  HubPlan &h = s.hub;
+static int build_hub(CsrSide &s, HubPlan &h, int32_t hot, int32_t groups, int32_t tiers, int32_t seg,
+                     hipStream_t stream) {
   CG_HIP(hipStreamSynchronize(stream));
   h.release();
   const int64_t nnz = s.nnz;
@@ -863,9 +868,24 @@ static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream) 
   const int hot_vec = (vec == 4 || f / vec <= kWave) ? vec : 1;
   const SpmmShape hshape = pick_shape(hot_vec, f / hot_vec);
   const int32_t seg = pick_seg(hshape);
-  if (!s.hub.valid || s.hub.hot != (int32_t)hot || s.hub.groups != groups || s.hub.tiers != tiers || s.hub.seg != seg)
-    CG_TRY(build_hub(s, (int32_t)hot, groups, tiers, seg, stream));
-  HubPlan &h = s.hub;
+  int slot = -1;
+  for (int i = 0; i < CsrSide::kHubPlans; ++i)
+    if (s.hub[i].valid && s.hub[i].hot == (int32_t)hot && s.hub[i].groups == groups && s.hub[i].tiers == tiers &&
+        s.hub[i].seg == seg)
+      slot = i;
+  if (slot < 0) {
+    slot = 0;
+    for (int i = 0; i < CsrSide::kHubPlans; ++i) {
+      if (!s.hub[i].valid) {
+        slot = i;
+        break;
+      }
+      if (s.hub_used[i] < s.hub_used[slot]) slot = i;
+    }
+    CG_TRY(build_hub(s, s.hub[slot], (int32_t)hot, groups, tiers, seg, stream));
+  }
+  s.hub_used[slot] = ++s.hub_clock;
+  HubPlan &h = s.hub[slot];
   const int32_t n = s.rows;
   const int32_t nclass = h.classes();
   // 1. hot classes, one launch per tier: every task writes a partial row

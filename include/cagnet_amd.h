@@ -98,9 +98,12 @@ int cg_csr_transpose(const int32_t *d_rowptr, const int32_t *d_colind, const flo
  *   spmm_gpu(A_rowindices, A_colindices, A_values, n, m, B, C)
  * (sparse-extension/sparse_coo_tensor.cu:113-240, called at gcn_distr.py:238-240):
  * C[n,f] = beta*C + A[n,m] * B[m,f] with A as row-sorted COO; the reference fixes beta = 1
- * (sparse_coo_tensor.cu:149-150).  Stream ordered: no allocation after the scratch has grown
- * to size, no device synchronisation, B and C stay row-major and keep their storage (the
- * reference transposes both and replaces their storage, :166-168,:183-185,:234-239).
+ * (sparse_coo_tensor.cu:149-150).  Like the reference it rebuilds everything from the COO arrays
+ * on every call (row compression, row-segment schedule), but as device work on `stream`: no
+ * allocation after the scratch has grown to size, no device synchronisation.  B and C stay
+ * row-major and keep their storage (the reference transposes both and replaces their storage,
+ * :166-168,:183-185,:234-239).  Rows must ascend; input that violates this gives wrong sums, as it
+ * does in the reference, but never an access outside the operands (indices are clamped).
  */
 int cg_spmm_coo(const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz, int32_t n, int32_t m,
                 const float *d_B, int64_t ldb, float *d_C, int64_t ldc, int32_t f, float beta, cg_stream_t stream);
@@ -116,8 +119,11 @@ int cg_csr_create(cg_csr_t **out, const int32_t *d_row, const int32_t *d_col, co
 int cg_csr_destroy(cg_csr_t *h);
 
 /* C[rows,f] = beta*C + op(A) * B, op(A) = A (transpose == 0: rows = n, B is m x f) or A^T
- * (transpose != 0: rows = m, B is n x f).  The first call for a given schedule class builds that
- * schedule (degree bins, row segments) and synchronises once; later calls are stream ordered. */
+ * (transpose != 0: rows = m, B is n x f).  The first call for a given width class builds its
+ * schedule (row segments, windows of tasks; for wide products over dense power-law matrices a
+ * plan that regroups the entries by column popularity) and synchronises once; later calls are
+ * stream ordered.  Results are bit-identical from call to call.  Scratch memory is kept per
+ * (device, stream); a handle may be used from one host thread at a time. */
 int cg_csr_spmm(cg_csr_t *h, int transpose, const float *d_B, int64_t ldb, float *d_C, int64_t ldc, int32_t f,
                 float beta, cg_stream_t stream);
 

@@ -349,6 +349,26 @@ def test_spmm_hub_plan_rectangular_and_all_hot(cuda, tune):
     assert spmm_error(A.spmm(B.to(cuda)), row, col, val, n, m, B) <= REL_TOL
 
 
+def test_spmm_hub_plans_of_several_widths_on_one_handle(cuda, tune):
+    """A handle keeps two hub plans (the hot-column count depends on the width); cycling through
+    three widths exercises reuse and replacement, and every product stays bit-identical to its
+    first evaluation."""
+    from cagnet_amd import ops
+    row, col, val, n = small_graph(11, 60000, seed=77)
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n)
+    tune("spmm_hub", 1)
+    tune("spmm_hub_kb", 64)
+    Bs = {f: torch.randn(n, f, generator=torch.Generator().manual_seed(f)) for f in (602, 256, 128)}
+    first = {}
+    for f in (602, 256, 602, 128, 256, 602, 128):
+        got = A.spmm(Bs[f].to(cuda))
+        if f not in first:
+            assert spmm_error(got, row, col, val, n, n, Bs[f]) <= REL_TOL
+            first[f] = got
+        else:
+            assert torch.equal(got, first[f])
+
+
 def test_blob_matches_format_restatement_and_roundtrips(cuda, tmp_path):
     """The library's bytes equal the oracle's independent writer bit for bit; a blob written by
     the oracle loads; a file round trip gives a handle whose products are bit-identical."""
