@@ -159,6 +159,10 @@ def main() -> int:
         gcn.train(x, w1, w2, n, [blk], opt, Data, 0, 1, None)
         x.grad = None
 
+    # The timed region runs the reference's operator sequence, one SpMM then one dense product per
+    # layer (gcn_distr.py:271-275), so that the headline kernel is exactly the f = f_in SpMM; the
+    # library's default, which folds the W product into that SpMM, is timed separately below.
+    gcn.fused_forward = False
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -171,6 +175,21 @@ def main() -> int:
     _lib.lib.cg_prof_enable(0)
     ms_per_step = elapsed / args.steps * 1e3
     loss = float(gcn.train.last_loss)
+
+    def timed_variant():
+        for _ in range(2):
+            step()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / args.steps * 1e3
+
+    # library default: the layer product Z = act((A H) W) is fused (no n x f intermediate) where rows are
+    # short enough for it to pay (the Amazon shape; on the Reddit shape this equals the headline)
+    gcn.fused_forward = True
+    fused_ms = timed_variant()
 
     # opt-in product order A (H W): same model, SpMM at the output width; reported beside the headline
     gcn.spmm_first = False
@@ -229,6 +248,7 @@ def main() -> int:
         "scomp_ms_per_epoch": round(spmm_total_ms, 4),
         "dcomp_ms_per_epoch": round(dense_total_ms, 4),
         "final_loss": loss,
+        "epoch_ms_default_fusion_policy": round(fused_ms, 4),
         "epoch_ms_opt_in_reordered_A_HW": round(reordered_ms, 4),
         "spmm_gbs_algorithmic": round(achieved, 2),
         "spmm_gbs_gather_model": round(gather_bytes / (dom_ms * 1e-3) / 1e9, 2),

@@ -496,14 +496,14 @@ static int64_t stream_grid(const StreamArgs &a) {
   return ceil_div64(ceil_div64(longest, kWavesPerBlock), 8 / a.groups) * 8;
 }
 
-static int launch_stream(const SpmmShape &s, const StreamArgs &a, hipStream_t stream) {
+static int launch_stream(const SpmmShape &s, const StreamArgs &a, hipStream_t stream, size_t wide_lds = 0) {
   const int64_t blocks = stream_grid(a);
   if (blocks == 0) return CG_OK;
   if (blocks > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "SpMM grid too large");
   const unsigned grid = (unsigned)blocks;
 #define CG_WIDE(V, CH)                                                    \
   if (s.lpr == kWave && s.vec == V && s.chunks == CH) {                   \
-    spmm_stream_wide_kernel<V, CH><<<grid, kSpmmThreads, 0, stream>>>(a); \
+    spmm_stream_wide_kernel<V, CH><<<grid, kSpmmThreads, wide_lds, stream>>>(a); \
     CG_LAUNCH_CHECK();                                                    \
     return CG_OK;                                                         \
   }
@@ -783,7 +783,20 @@ struct DenseOps {
   const int32_t *fold_tbase = nullptr;
   const float *fold_P = nullptr;
   int32_t fold_classes = 0, fold_rows = 0;
+  // optional epilogue: finished rows are multiplied by W (f x fo) into Z instead of being stored
+  // (see StreamArgs); C is then only read, and only when beta != 0
+  const float *epi_W = nullptr;
+  int64_t epi_ldw = 0;
+  float *epi_Z = nullptr;
+  int64_t epi_ldz = 0;
+  int32_t epi_fo = 0, epi_relu = 0;
 };
+
+constexpr size_t kEpiLdsBytes = 64 * 1024;
+static int32_t epi_pad(int32_t fo) { return fo <= 16 ? 16 : (fo <= 32 ? 32 : 64); }
+static size_t epi_lds_bytes(int32_t f, int32_t fo) {
+  return ((size_t)f * epi_pad(fo) + (size_t)kWavesPerBlock * f) * sizeof(float);
+}
 
 // Row-segment tasks over (rowptr, colind, val), for a column range one launch can cover.
 static int spmm_plain(const int32_t *rowptr, const int32_t *colind, const float *val, int32_t rows, int64_t nnz,
@@ -818,6 +831,18 @@ static int spmm_plain(const int32_t *rowptr, const int32_t *colind, const float 
   sa.fold_classes = d.fold_classes;
   sa.fold_rows = d.fold_rows;
   if (d.fold_tbase && shape.lpr != kWave) CG_FAIL(CG_ERR_UNSUPPORTED, "fold needs full-wave teams");
+  size_t lds = 0;
+  if (d.epi_W) {
+    if (shape.lpr != kWave) CG_FAIL(CG_ERR_UNSUPPORTED, "epilogue needs full-wave teams");
+    sa.epi_W = d.epi_W;
+    sa.epi_ldw = d.epi_ldw;
+    sa.epi_Z = d.epi_Z;
+    sa.epi_ldz = d.epi_ldz;
+    sa.epi_fo = d.epi_fo;
+    sa.epi_fop = epi_pad(d.epi_fo);
+    sa.epi_relu = d.epi_relu;
+    lds = epi_lds_bytes(d.f, d.epi_fo);
+  }
   if (sc->nslots > 0) {
     void *p = nullptr;
     CG_TRY(scratch_get(stream, kSlotA, (size_t)sc->nslots * d.f * sizeof(float), &p));
@@ -825,9 +850,35 @@ static int spmm_plain(const int32_t *rowptr, const int32_t *colind, const float 
   }
   {
     ProfScope prof("spmm_rowseg", prof_tag, stream);
-    CG_TRY(launch_stream(shape, sa, stream));
+    CG_TRY(launch_stream(shape, sa, stream, lds));
   }
-  if (sc->nmulti > 0) {
+  if (sc->nmulti > 0 && d.epi_W) {
+    ProfScope prof("spmm_reduce", prof_tag, stream);
+    ReduceEpiArgs ra{};
+    ra.multi_rows = sc->multi_rows;
+    ra.nmulti = sc->nmulti;
+    ra.rowptr = rowptr;
+    ra.pbase = sc->pbase;
+    ra.seg = sc->seg;
+    ra.P = sa.P;
+    ra.C = d.C;
+    ra.ldc = d.ldc;
+    ra.f = d.f;
+    ra.beta = d.beta;
+    ra.fold_tbase = d.fold_tbase;
+    ra.fold_P = d.fold_P;
+    ra.fold_classes = d.fold_classes;
+    ra.fold_rows = d.fold_rows;
+    ra.epi_W = sa.epi_W;
+    ra.epi_ldw = sa.epi_ldw;
+    ra.epi_Z = sa.epi_Z;
+    ra.epi_ldz = sa.epi_ldz;
+    ra.epi_fo = sa.epi_fo;
+    ra.epi_fop = sa.epi_fop;
+    ra.epi_relu = sa.epi_relu;
+    spmm_reduce_epi_kernel<<<(unsigned)ceil_div64(sc->nmulti, kWavesPerBlock), kSpmmThreads, lds, stream>>>(ra);
+    CG_LAUNCH_CHECK();
+  } else if (sc->nmulti > 0) {
     ProfScope prof("spmm_reduce", prof_tag, stream);
     const int64_t threads = sc->nmulti * (int64_t)d.f;
     spmm_reduce_kernel<<<(unsigned)ceil_div64(threads, kSpmmThreads), kSpmmThreads, 0, stream>>>(
@@ -944,19 +995,35 @@ static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream) 
   return CG_OK;
 }
 
+// epi (nullable): only its epilogue fields are read; the product then ends in Z = act(row * W)
+// instead of C, which needs full-wave teams, one column range and room for W in LDS.
+static bool epi_supported(int32_t f, int32_t fo, int vec) {
+  return fo >= 1 && fo <= 64 && f <= range_cap(vec) && pick_shape(vec, f / vec).lpr == kWave &&
+         epi_lds_bytes(f, fo) <= kEpiLdsBytes;
+}
+
 static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t ldc, int32_t f, float beta,
-                     hipStream_t stream) {
+                     hipStream_t stream, const DenseOps *epi = nullptr) {
   if (s.rows == 0) return CG_OK;
-  const int vec = pick_vec(f, B, ldb, C, ldc);
+  const int vec = pick_vec(f, B, ldb, C ? C : B, C ? ldc : ldb);
   const int32_t cap = range_cap(vec);
-  if (f <= range_cap(vec == 4 ? 4 : 1) && want_hub(s, f)) {
-    const DenseOps d{B, ldb, C, ldc, f, beta};
-    return spmm_hub(s, vec, d, stream);
+  DenseOps d{B, ldb, C, ldc, f, beta};
+  if (epi) {
+    if (!epi_supported(f, epi->epi_fo, vec))
+      CG_FAIL(CG_ERR_UNSUPPORTED, "fused product: f=%d fo=%d has no fused form", f, epi->epi_fo);
+    d.epi_W = epi->epi_W;
+    d.epi_ldw = epi->epi_ldw;
+    d.epi_Z = epi->epi_Z;
+    d.epi_ldz = epi->epi_ldz;
+    d.epi_fo = epi->epi_fo;
+    d.epi_relu = epi->epi_relu;
   }
+  if (f <= range_cap(vec == 4 ? 4 : 1) && want_hub(s, f)) return spmm_hub(s, vec, d, stream);
+  if (epi) return spmm_plain(s.rowptr, s.colind, s.val, s.rows, s.nnz, s.sched, vec, d, f, stream);
   for (int32_t f0 = 0; f0 < f; f0 += cap) {  // wider outputs take several launches over column ranges
     const int32_t ft = f - f0 < cap ? f - f0 : cap;
-    const DenseOps d{B + f0, ldb, C + f0, ldc, ft, beta};
-    CG_TRY(spmm_plain(s.rowptr, s.colind, s.val, s.rows, s.nnz, s.sched, vec, d, f, stream));
+    const DenseOps dr{B + f0, ldb, C + f0, ldc, ft, beta};
+    CG_TRY(spmm_plain(s.rowptr, s.colind, s.val, s.rows, s.nnz, s.sched, vec, dr, f, stream));
   }
   return CG_OK;
 }
@@ -1163,6 +1230,30 @@ int cg_csr_spmm(cg_csr_t *h, int transpose, const float *d_B, int64_t ldb, float
   CsrSide &s = transpose ? h->tr : h->fwd;
   CG_TRY(check_dense("cg_csr_spmm", d_B, ldb, d_C, ldc, f, s.cols, s.rows));
   return spmm_side(s, d_B, ldb, d_C, ldc, f, beta, (hipStream_t)stream);
+}
+
+int cg_csr_spmm_xw(cg_csr_t *h, int transpose, const float *d_B, int64_t ldb, const float *d_C, int64_t ldc, float beta,
+                   const float *d_W, int64_t ldw, float *d_Z, int64_t ldz, int32_t f, int32_t fo, int relu,
+                   cg_stream_t stream) {
+  using namespace cg;
+  if (!h) CG_FAIL(CG_ERR_NULL, "cg_csr_spmm_xw: handle is NULL");
+  if (transpose && !h->has_t) CG_FAIL(CG_ERR_NO_TRANSPOSE, "cg_csr_spmm_xw: handle was built without CG_CSR_TRANSPOSE");
+  CsrSide &s = transpose ? h->tr : h->fwd;
+  if (f <= 0 || fo <= 0) CG_FAIL(CG_ERR_SIZE, "cg_csr_spmm_xw: f=%d fo=%d must be positive", f, fo);
+  if (ldb < f || ldw < fo || ldz < fo) CG_FAIL(CG_ERR_SIZE, "cg_csr_spmm_xw: leading dimension too small");
+  if (beta != 0.f && (!d_C || ldc < f)) CG_FAIL(d_C ? CG_ERR_SIZE : CG_ERR_NULL, "cg_csr_spmm_xw: beta != 0 needs C");
+  if (!d_W || (!d_B && s.cols > 0) || (!d_Z && s.rows > 0)) CG_FAIL(CG_ERR_NULL, "cg_csr_spmm_xw: null dense operand");
+  if ((const float *)d_Z == d_B || (beta != 0.f && (const float *)d_Z == d_C))
+    CG_FAIL(CG_ERR_ALIAS, "cg_csr_spmm_xw: Z aliases an input");
+  DenseOps epi{};
+  epi.epi_W = d_W;
+  epi.epi_ldw = ldw;
+  epi.epi_Z = d_Z;
+  epi.epi_ldz = ldz;
+  epi.epi_fo = fo;
+  epi.epi_relu = relu ? 1 : 0;
+  // C is never written on this path
+  return spmm_side(s, d_B, ldb, beta != 0.f ? const_cast<float *>(d_C) : nullptr, ldc, f, beta, (hipStream_t)stream, &epi);
 }
 
 int cg_tune_set(const char *key, int value) {

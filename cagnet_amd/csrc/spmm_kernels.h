@@ -115,7 +115,92 @@ struct StreamArgs {
   const int32_t *fold_tbase;
   const float *fold_P;
   int32_t fold_classes, fold_rows;
+  // Epilogue (wide teams, groups == 1): a finished row r = beta*C[row] + (A B)[row] is not stored
+  // but multiplied by epi_W (f x epi_fo): epi_Z[row, :] = act(r * epi_W), the layer's (A H) W
+  // without the n x f intermediate.  epi_fop = epi_fo rounded up to 16, 32 or 64.
+  const float *epi_W;
+  int64_t epi_ldw;
+  float *epi_Z;
+  int64_t epi_ldz;
+  int32_t epi_fo, epi_fop, epi_relu;
 };
+
+// LDS of an epilogue launch: W as [f][fop] floats, then one row buffer of f floats per wave
+__device__ __forceinline__ void epi_stage_w(float *lds, const float *__restrict__ W, int64_t ldw, int32_t f, int32_t fo,
+                                            int32_t fop, int threads) {
+  for (int32_t idx = threadIdx.x; idx < f * fop; idx += threads) {
+    const int32_t k = idx / fop, j = idx % fop;
+    lds[idx] = j < fo ? W[(int64_t)k * ldw + j] : 0.f;
+  }
+}
+
+// z[j] = sum_k row[k] * Ws[k][j] by one wavefront: lane = (part, j), part strides over k, the parts
+// are then added by a fixed xor butterfly; lanes of part 0 store.
+__device__ __forceinline__ void epi_row(const float *row, const float *Ws, int32_t f, int32_t fop, int32_t fo, int lane,
+                                        float *zrow, int relu) {
+  const int j = lane & (fop - 1);
+  const int part = lane / fop, parts = kWave / fop;
+  float s0 = 0.f, s1 = 0.f;  // two chains, added at the end: k and k + parts alternate
+  int32_t k = part;
+  for (; k + parts < f; k += 2 * parts) {
+    s0 = fmaf(row[k], Ws[k * fop + j], s0);
+    s1 = fmaf(row[k + parts], Ws[(k + parts) * fop + j], s1);
+  }
+  if (k < f) s0 = fmaf(row[k], Ws[k * fop + j], s0);
+  float s = s0 + s1;
+  for (int off = fop; off < kWave; off <<= 1) s += __shfl_xor(s, off, kWave);
+  if (lane < fop && j < fo) zrow[j] = (relu && s < 0.f) ? 0.f : s;
+}
+
+// The same for a launch with an epilogue: one wavefront per split row rebuilds the row in LDS
+// (partials in segment order, then the folded partial rows) and sends it through W.
+struct ReduceEpiArgs {
+  const int32_t *multi_rows;
+  int64_t nmulti;
+  const int32_t *rowptr, *pbase;
+  int32_t seg;
+  const float *P;
+  const float *C;  // read only (beta != 0)
+  int64_t ldc;
+  int32_t f;
+  float beta;
+  const int32_t *fold_tbase;
+  const float *fold_P;
+  int32_t fold_classes, fold_rows;
+  const float *epi_W;
+  int64_t epi_ldw;
+  float *epi_Z;
+  int64_t epi_ldz;
+  int32_t epi_fo, epi_fop, epi_relu;
+};
+
+__global__ __launch_bounds__(kSpmmThreads) void spmm_reduce_epi_kernel(const ReduceEpiArgs a) {
+  extern __shared__ float epi_lds[];
+  epi_stage_w(epi_lds, a.epi_W, a.epi_ldw, a.f, a.epi_fo, a.epi_fop, kSpmmThreads);
+  __syncthreads();
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int64_t mr = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  if (mr >= a.nmulti) return;
+  const int32_t row = a.multi_rows[mr];
+  const int32_t deg = a.rowptr[row + 1] - a.rowptr[row];
+  const int32_t nseg = (deg + a.seg - 1) / a.seg;
+  float *rowbuf = epi_lds + (size_t)a.f * a.epi_fop + (size_t)wave * a.f;
+  for (int32_t col = lane; col < a.f; col += kWave) {
+    const float *p = a.P + (int64_t)a.pbase[row] * a.f + col;
+    float s = 0.f;
+    for (int32_t i = 0; i < nseg; ++i) s += p[(int64_t)i * a.f];
+    if (a.fold_tbase) {
+      for (int32_t cls = 0; cls < a.fold_classes; ++cls) {
+        const int32_t *tb = a.fold_tbase + (int64_t)cls * a.fold_rows + row;
+        for (int32_t t = tb[0]; t < tb[1]; ++t) s += a.fold_P[(int64_t)t * a.f + col];
+      }
+    }
+    rowbuf[col] = a.beta != 0.f ? fmaf(a.beta, a.C[(int64_t)row * a.ldc + col], s) : s;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  epi_row(rowbuf, epi_lds, a.f, a.epi_fop, a.epi_fo, lane, a.epi_Z + (int64_t)row * a.epi_ldz, a.epi_relu);
+}
 
 // Full-wave teams (one stored entry per wave step, f covered by CHUNKS x 64 lanes x VEC floats).
 template <int VEC, int CHUNKS>
@@ -127,7 +212,13 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_stream_wide_kernel(const St
   const int64_t lblock = (int64_t)(blockIdx.x >> 3) * per + x / a.groups;
   const int64_t wl = lblock * kWavesPerBlock + threadIdx.x / kWave;
   const int64_t nwin_here = a.d_nwin ? (int64_t)*a.d_nwin : a.win_first[grp + 1] - a.win_first[grp];
+  extern __shared__ float epi_lds[];
+  if (a.epi_W) {  // every wave of the workgroup stages W before any of them may leave
+    epi_stage_w(epi_lds, a.epi_W, a.epi_ldw, a.f, a.epi_fo, a.epi_fop, kSpmmThreads);
+    __syncthreads();
+  }
   if (wl >= nwin_here) return;
+  float *epi_rowbuf = epi_lds + (size_t)a.f * a.epi_fop + (size_t)(threadIdx.x / kWave) * a.f;
   const int32_t w = __builtin_amdgcn_readfirstlane((int32_t)(a.win_first[grp] + wl));
   const int32_t t0 = a.wstart[w], t1 = a.wstart[w + 1];
   const int ntask = t1 - t0;  // 1..64
@@ -201,7 +292,32 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_stream_wide_kernel(const St
               }
             }
           }
-          if (folded || !(tend == tbeg && a.beta == 1.0f)) {  // an empty row leaves C alone when beta == 1
+          if (a.epi_W) {
+            // the finished row goes to LDS and from there through W; C is only read (beta != 0)
+            const float *crow = a.C + (int64_t)dst * a.ldc;
+#pragma unroll
+            for (int ch = 0; ch < CHUNKS; ++ch) {
+              if (active[ch]) {
+                float out[VEC];
+                if (a.beta != 0.f) {
+                  float old[VEC];
+                  load_vec<VEC>(crow + boff[ch], old);
+#pragma unroll
+                  for (int q = 0; q < VEC; ++q) out[q] = fmaf(a.beta, old[q], acc[ch][q]);
+                } else {
+#pragma unroll
+                  for (int q = 0; q < VEC; ++q) out[q] = acc[ch][q];
+                }
+#pragma unroll
+                for (int q = 0; q < VEC; ++q) epi_rowbuf[boff[ch] + q] = out[q];
+              }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            epi_row(epi_rowbuf, epi_lds, a.f, a.epi_fop, a.epi_fo, lane, a.epi_Z + (int64_t)dst * a.epi_ldz, a.epi_relu);
+            __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+          } else if (folded || !(tend == tbeg && a.beta == 1.0f)) {  // an empty row leaves C alone when beta == 1
             float *crow = a.C + (int64_t)dst * a.ldc;
 #pragma unroll
             for (int ch = 0; ch < CHUNKS; ++ch) {

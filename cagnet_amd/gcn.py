@@ -33,6 +33,16 @@ activations = True
 spmm_first = True
 
 
+# Fuse the layer's two forward products, Z = act((sum_i A_i H_i) W), into the last stage's SpMM when
+# the width allows it: the n x f_in intermediate (gcn_distr.py:271) is then never written.  Same
+# product order as the reference; only the summation order inside the small W product differs.
+fused_forward = True
+# ... but only where it pays: the epilogue costs a fixed f_in * f_out multiply-adds per row, the
+# saving is one write and one read of the row.  Measured: Amazon shape (16 entries per row) epoch
+# 77.2 -> 72.9 ms, Reddit shape (492 entries per row) 24.7 -> 25.0 ms.
+fused_forward_max_row_entries = 64
+
+
 class ResidentBlocks:
     """Stands where the reference passes a process group: the dense blocks that its broadcasts
     would deliver (gcn_distr.py:230), already resident in HBM.  `forward[i]` is the H block and
@@ -150,9 +160,21 @@ class GCNFunc(torch.autograd.Function):
         node_count = adj_matrix if isinstance(adj_matrix, int) else adj_matrix.size(0)
         peers_fwd = group.forward if isinstance(group, ResidentBlocks) else None
         if spmm_first or size != 1 or weight.shape[1] >= inputs.shape[1]:  # reordering only pays when the layer narrows
-            z = broad_func(node_count, am_partitions, inputs, rank, size, peers_fwd)
-            out = ops.dense_xw(z, weight, relu=(kind == "relu"))
-            del z
+            out = None
+            last = am_partitions[size - 1]
+            short_rows = last.nnz <= fused_forward_max_row_entries * max(last.n, 1)
+            if fused_forward and short_rows and weight.shape[1] <= 64 and inputs.shape[1] >= 128:
+                # stages 0 .. size-2 accumulate as usual, the last one also applies W (and ReLU)
+                z = broad_func(node_count, am_partitions[:-1], inputs, rank, size - 1, peers_fwd) if size > 1 else None
+                h_last = _stage_operand(size - 1, rank, inputs, peers_fwd)
+                out = am_partitions[size - 1].spmm_xw(h_last, weight, relu=(kind == "relu"), acc=z)
+                if out is None and z is not None:      # no fused form for this width: finish the stage loop
+                    am_partitions[size - 1].spmm(h_last, out=z, beta=1.0)
+                    out = ops.dense_xw(z, weight, relu=(kind == "relu"))
+            if out is None:
+                z = broad_func(node_count, am_partitions, inputs, rank, size, peers_fwd)
+                out = ops.dense_xw(z, weight, relu=(kind == "relu"))
+                del z
         else:
             out = broad_func(node_count, am_partitions, ops.dense_xw(inputs, weight), rank, size, peers_fwd)
             if kind == "relu":

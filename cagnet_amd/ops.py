@@ -334,6 +334,31 @@ class CsrMatrix:
         return out
 
 
+    def spmm_xw(self, B: torch.Tensor, W: torch.Tensor, relu: bool = False, acc: Optional[torch.Tensor] = None,
+                transpose: bool = False) -> Optional[torch.Tensor]:
+        """Z = act((acc + op(A) @ B) @ W) in one pass, without the rows x f intermediate (the two
+        steps of GCNFunc.forward, gcn_distr.py:271-275).  `acc` is the sum of earlier stages (read
+        only).  Returns None when this width has no fused form; the caller then uses spmm + dense_xw."""
+        B, ldb = _rowmajor(B, "B")
+        W, ldw = _rowmajor(W, "W")
+        rows, inner = (self.m, self.n) if transpose else (self.n, self.m)
+        f, fo = B.shape[1], W.shape[1]
+        if B.shape[0] != inner or W.shape[0] != f:
+            raise ValueError(f"B is {tuple(B.shape)}, W is {tuple(W.shape)}, the sparse operand has {inner} columns")
+        ldc = 0
+        if acc is not None:
+            acc, ldc = _rowmajor(acc, "acc")
+            if tuple(acc.shape) != (rows, f):
+                raise ValueError(f"acc has shape {tuple(acc.shape)}, expected {(rows, f)}")
+        Z = torch.empty(rows, fo, dtype=torch.float32, device=B.device)
+        st = lib.cg_csr_spmm_xw(self._handle, int(transpose), _ptr(B), ldb, _ptr(acc), ldc, 1.0 if acc is not None else 0.0,
+                                _ptr(W), ldw, _ptr(Z), max(fo, 1), f, fo, int(relu), _stream())
+        if st == _lib.CG_ERR_UNSUPPORTED:
+            return None
+        check(st, "cg_csr_spmm_xw")
+        return Z
+
+
 # ------------------------------------------------------------------------------------------------
 # dense products
 # ------------------------------------------------------------------------------------------------

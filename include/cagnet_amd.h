@@ -127,6 +127,16 @@ int cg_csr_destroy(cg_csr_t *h);
 int cg_csr_spmm(cg_csr_t *h, int transpose, const float *d_B, int64_t ldb, float *d_C, int64_t ldc, int32_t f,
                 float beta, cg_stream_t stream);
 
+/* Fused layer product Z[rows,fo] = act((beta*C + op(A) * B) * W): the two steps of GCNFunc.forward,
+ * z = spmm(A, H) then torch.mm(z, weight) (gcn_distr.py:271-275), without writing the rows x f
+ * intermediate; relu != 0 applies max(., 0) (gcn_distr.py:284-288).  C is an input here (the sum of
+ * earlier stages, read when beta != 0, never written; NULL with beta == 0).  W is f x fo, fo <= 64.
+ * Returns CG_ERR_UNSUPPORTED, before any work, for widths that have no fused form (f below 128 or
+ * so, f * fo beyond the LDS budget): the caller then runs cg_csr_spmm and cg_dense_xw. */
+int cg_csr_spmm_xw(cg_csr_t *h, int transpose, const float *d_B, int64_t ldb, const float *d_C, int64_t ldc, float beta,
+                   const float *d_W, int64_t ldw, float *d_Z, int64_t ldz, int32_t f, int32_t fo, int relu,
+                   cg_stream_t stream);
+
 /* info[0..7] = { n, m, nnz, has_transpose, max row degree, max column degree (or -1), 0, 0 } */
 int cg_csr_info(const cg_csr_t *h, int64_t info[8]);
 /* Device pointers of the arrays the handle owns (transpose != 0: those of A^T). */

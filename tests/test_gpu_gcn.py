@@ -30,10 +30,15 @@ def _close(got, ref64, what, tol=2e-4):
     assert err <= tol, f"{what}: {err}"
 
 
+@pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("transpose", [False, True])
-def test_forward_backward_matches_oracle(cuda, transpose):
+def test_forward_backward_matches_oracle(cuda, monkeypatch, transpose, fused):
+    """Both forms of the layer product: SpMM with the W product folded in (rows are short here, so
+    the default takes it) and the reference's two separate kernels."""
     from cagnet_amd import gcn
+    monkeypatch.setattr(gcn, "fused_forward", fused)
     p = synth.make_problem(scale=11, n_edges=16384, features=128, hidden=16, classes=8, mask_fraction=0.66, seed=3)
+    assert p.row.numel() <= gcn.fused_forward_max_row_entries * p.n
     A = orc.coo_tensor(p.row, p.col, p.val, p.n, p.n, torch.float64)
     ref = orc.forward_backward(p.x, p.w1, p.w2, [A], p.y, p.train_mask, dtype=torch.float64)
 

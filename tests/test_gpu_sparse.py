@@ -369,6 +369,75 @@ def test_spmm_hub_plans_of_several_widths_on_one_handle(cuda, tune):
             assert torch.equal(got, first[f])
 
 
+def _xw_error(got, row, col, val, n, m, B, W, C0=None, relu=False):
+    """max |got - ref64| / (sum |a||b| (+|c0|)) |W|, ref64 = act((C0 + A B) W) in fp64."""
+    B64, W64 = B.double(), W.double()
+    C64 = torch.zeros(n, B.shape[1], dtype=torch.float64) if C0 is None else C0.double()
+    ab = orc.spmm(row, col, val, n, m, B64, C64, torch.float64)
+    ref = ab @ W64
+    if relu:
+        ref = ref.clamp_min(0.0)
+    mag = (orc.spmm_abs(row, col, val, n, m, B64) + C64.abs()) @ W64.abs()
+    return orc.max_rel_error(got, ref, mag)
+
+
+@pytest.mark.parametrize("hub", [-1, 1])
+@pytest.mark.parametrize("f,fo,relu", [(602, 16, True), (300, 24, False), (256, 7, True), (130, 41, False), (192, 64, False)])
+def test_spmm_xw_fused_layer_product(cuda, tune, f, fo, relu, hub):
+    """Z = act((acc + A B) W) in one pass against the fp64 oracle of the two separate products:
+    plain and hub-plan schedules, with and without an accumulated input, and on A^T."""
+    from cagnet_amd import ops
+    row, col, val, n = small_graph(11, 60000, seed=900 + f)
+    g = torch.Generator().manual_seed(f + fo)
+    B, W = torch.randn(n, f, generator=g), torch.randn(f, fo, generator=g)
+    C0 = torch.randn(n, f, generator=g)
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n, transpose=True)
+    tune("spmm_hub", hub)
+    tune("spmm_hub_kb", 64)
+    Z = A.spmm_xw(B.to(cuda), W.to(cuda), relu=relu)
+    assert Z is not None and tuple(Z.shape) == (n, fo)
+    assert _xw_error(Z, row, col, val, n, n, B, W, relu=relu) <= 2 * REL_TOL
+    assert torch.equal(Z, A.spmm_xw(B.to(cuda), W.to(cuda), relu=relu))          # deterministic
+    acc = C0.to(cuda)
+    keep = acc.clone()
+    Z2 = A.spmm_xw(B.to(cuda), W.to(cuda), relu=relu, acc=acc)
+    assert _xw_error(Z2, row, col, val, n, n, B, W, C0=C0, relu=relu) <= 2 * REL_TOL
+    assert torch.equal(acc, keep)                                                 # the accumulated input is only read
+    assert torch.equal(A.spmm_xw(B.to(cuda), W.to(cuda), relu=relu, transpose=True), Z)   # symmetric graph
+    # the separate kernels give the same numbers up to summation order
+    two = ops.dense_xw(A.spmm(B.to(cuda)), W.to(cuda), relu=relu)
+    scale = ops.dense_xw(A.spmm(B.abs().to(cuda)), W.abs().to(cuda)).clamp_min(1e-30)
+    assert float(((Z - two).abs() / scale).max()) <= 8e-6
+
+
+def test_spmm_xw_split_rows_and_unsupported_widths(cuda, tune):
+    from cagnet_amd import ops
+    # rows of ~4000 entries are split over several wavefronts: their epilogue runs in the reduce kernel
+    n, m, f, fo = 40, 9000, 320, 16
+    row, col, val = random_coo(n, m, n * 4000, seed=31)
+    g = torch.Generator().manual_seed(5)
+    B, W, C0 = torch.randn(m, f, generator=g), torch.randn(f, fo, generator=g), torch.randn(n, f, generator=g)
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, m)
+    for hub in (-1, 1):
+        tune("spmm_hub", hub)
+        tune("spmm_hub_kb", 256)
+        Z = A.spmm_xw(B.to(cuda), W.to(cuda), relu=True, acc=C0.to(cuda))
+        assert _xw_error(Z, row, col, val, n, m, B, W, C0=C0, relu=True) <= 2 * REL_TOL
+    tune("spmm_hub", 0)
+    # narrow products have no fused form: the wrapper says so instead of computing something else
+    assert A.spmm_xw(torch.randn(m, 64, device=cuda), torch.randn(64, 16, device=cuda)) is None
+    assert A.spmm_xw(torch.randn(m, 602, device=cuda), torch.randn(602, 64, device=cuda)) is None     # W beyond the LDS budget
+    with pytest.raises(ValueError):
+        A.spmm_xw(B.to(cuda), torch.randn(f + 1, fo, device=cuda))
+    # rows without entries: Z = act(acc W)
+    e32 = torch.empty(0, dtype=torch.int32, device=cuda)
+    E = ops.CsrMatrix(e32, e32, torch.empty(0, device=cuda), n, m)
+    Z = E.spmm_xw(B.to(cuda), W.to(cuda), acc=C0.to(cuda))
+    ref = C0.double() @ W.double()
+    assert float((Z.cpu().double() - ref).abs().max()) <= 1e-4 * float(ref.abs().max())
+    assert torch.count_nonzero(E.spmm_xw(B.to(cuda), W.to(cuda))) == 0
+
+
 def test_blob_matches_format_restatement_and_roundtrips(cuda, tmp_path):
     """The library's bytes equal the oracle's independent writer bit for bit; a blob written by
     the oracle loads; a file round trip gives a handle whose products are bit-identical."""
