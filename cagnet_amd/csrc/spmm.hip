@@ -794,8 +794,9 @@ struct DenseOps {
 
 constexpr size_t kEpiLdsBytes = 64 * 1024;
 static int32_t epi_pad(int32_t fo) { return fo <= 16 ? 16 : (fo <= 32 ? 32 : 64); }
-static size_t epi_lds_bytes(int32_t f, int32_t fo) {
-  return ((size_t)f * epi_pad(fo) + (size_t)kWavesPerBlock * f) * sizeof(float);
+static size_t epi_lds_bytes(int32_t f, int32_t fo) {  // W^T rows and one row buffer per wave, each fpad floats
+  const size_t fpad = (size_t)(f + 15) / 16 * 16 + 4;
+  return ((size_t)epi_pad(fo) + kWavesPerBlock) * fpad * sizeof(float);
 }
 
 // Row-segment tasks over (rowptr, colind, val), for a column range one launch can cover.

@@ -125,28 +125,43 @@ struct StreamArgs {
   int32_t epi_fo, epi_fop, epi_relu;
 };
 
-// LDS of an epilogue launch: W as [f][fop] floats, then one row buffer of f floats per wave
+// LDS of an epilogue launch: W transposed as [fop][fpad] floats, then one row buffer of fpad floats
+// per wave.  fpad = f rounded up to 16, plus 4 (keeps 16-byte alignment, spreads the rows of W^T
+// over the banks); everything past f is zero.
+__device__ __forceinline__ int32_t epi_fpad(int32_t f) { return (f + 15) / 16 * 16 + 4; }
+
 __device__ __forceinline__ void epi_stage_w(float *lds, const float *__restrict__ W, int64_t ldw, int32_t f, int32_t fo,
                                             int32_t fop, int threads) {
-  for (int32_t idx = threadIdx.x; idx < f * fop; idx += threads) {
-    const int32_t k = idx / fop, j = idx % fop;
-    lds[idx] = j < fo ? W[(int64_t)k * ldw + j] : 0.f;
+  const int32_t fpad = epi_fpad(f);
+  for (int32_t idx = threadIdx.x; idx < fpad * fop; idx += threads) {
+    const int32_t k = idx / fop, j = idx % fop;  // j fastest: coalesced reads of W
+    lds[j * fpad + k] = (k < f && j < fo) ? W[(int64_t)k * ldw + j] : 0.f;
   }
+  float *rows = lds + (size_t)fop * fpad;  // tails of the row buffers: read by the last steps, never written again
+  for (int32_t idx = threadIdx.x; idx < kWavesPerBlock * (fpad - f); idx += threads)
+    rows[(idx / (fpad - f)) * fpad + f + idx % (fpad - f)] = 0.f;
 }
 
-// z[j] = sum_k row[k] * Ws[k][j] by one wavefront: lane = (part, j), part strides over k, the parts
-// are then added by a fixed xor butterfly; lanes of part 0 store.
-__device__ __forceinline__ void epi_row(const float *row, const float *Ws, int32_t f, int32_t fop, int32_t fo, int lane,
+// z[j] = sum_k row[k] * W[k][j] by one wavefront: lane = (part, j); a part owns a contiguous range
+// of k and walks it four at a time (one 16-byte LDS read of the row, one of W^T); the parts are
+// then added by a fixed xor butterfly; lanes of part 0 store.
+__device__ __forceinline__ void epi_row(const float *row, const float *Wt, int32_t f, int32_t fop, int32_t fo, int lane,
                                         float *zrow, int relu) {
+  const int32_t fpad = epi_fpad(f);
   const int j = lane & (fop - 1);
   const int part = lane / fop, parts = kWave / fop;
-  float s0 = 0.f, s1 = 0.f;  // two chains, added at the end: k and k + parts alternate
-  int32_t k = part;
-  for (; k + parts < f; k += 2 * parts) {
-    s0 = fmaf(row[k], Ws[k * fop + j], s0);
-    s1 = fmaf(row[k + parts], Ws[(k + parts) * fop + j], s1);
+  const int32_t kper = ((f + parts - 1) / parts + 3) / 4 * 4;
+  const float *r = row + part * kper;
+  const float *w = Wt + (size_t)j * fpad + part * kper;
+  float s0 = 0.f, s1 = 0.f;
+  for (int32_t k = 0; k < kper; k += 4) {
+    const float4 x = *reinterpret_cast<const float4 *>(r + k);
+    const float4 y = *reinterpret_cast<const float4 *>(w + k);
+    s0 = fmaf(x.x, y.x, s0);
+    s1 = fmaf(x.y, y.y, s1);
+    s0 = fmaf(x.z, y.z, s0);
+    s1 = fmaf(x.w, y.w, s1);
   }
-  if (k < f) s0 = fmaf(row[k], Ws[k * fop + j], s0);
   float s = s0 + s1;
   for (int off = fop; off < kWave; off <<= 1) s += __shfl_xor(s, off, kWave);
   if (lane < fop && j < fo) zrow[j] = (relu && s < 0.f) ? 0.f : s;
@@ -184,7 +199,7 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_reduce_epi_kernel(const Red
   const int32_t row = a.multi_rows[mr];
   const int32_t deg = a.rowptr[row + 1] - a.rowptr[row];
   const int32_t nseg = (deg + a.seg - 1) / a.seg;
-  float *rowbuf = epi_lds + (size_t)a.f * a.epi_fop + (size_t)wave * a.f;
+  float *rowbuf = epi_lds + ((size_t)a.epi_fop + wave) * epi_fpad(a.f);
   for (int32_t col = lane; col < a.f; col += kWave) {
     const float *p = a.P + (int64_t)a.pbase[row] * a.f + col;
     float s = 0.f;
@@ -218,7 +233,7 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_stream_wide_kernel(const St
     __syncthreads();
   }
   if (wl >= nwin_here) return;
-  float *epi_rowbuf = epi_lds + (size_t)a.f * a.epi_fop + (size_t)(threadIdx.x / kWave) * a.f;
+  float *epi_rowbuf = epi_lds + ((size_t)a.epi_fop + threadIdx.x / kWave) * epi_fpad(a.f);
   const int32_t w = __builtin_amdgcn_readfirstlane((int32_t)(a.win_first[grp] + wl));
   const int32_t t0 = a.wstart[w], t1 = a.wstart[w + 1];
   const int ntask = t1 - t0;  // 1..64

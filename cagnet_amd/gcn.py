@@ -39,7 +39,7 @@ spmm_first = True
 fused_forward = True
 # ... but only where it pays: the epilogue costs a fixed f_in * f_out multiply-adds per row, the
 # saving is one write and one read of the row.  Measured: Amazon shape (16 entries per row) epoch
-# 77.2 -> 72.9 ms, Reddit shape (492 entries per row) 24.7 -> 25.0 ms.
+# 77.7 -> 71.4 ms, Reddit shape (492 entries per row) 24.3 -> 24.5 ms.
 fused_forward_max_row_entries = 64
 
 
