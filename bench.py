@@ -47,7 +47,7 @@ WORKLOADS = {
 # HBM bytes per launch of the dominant product (its four kernels together) from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE runs, reads scaled by 2.0 and writes by 1.0 as calibrated on a 1 GiB copy
 # kernel (profiles/spmm_f602_reddit_counters.txt): 142.25 GB read + 4.97 GB written.
-MEASURED_TRAFFIC_BYTES = {"reddit": 135.7e9}
+MEASURED_TRAFFIC_BYTES = {"reddit": 135.6e9}
 
 
 def spmm_alg_bytes(nnz: int, n: int, m: int, f: int, reads_c: bool) -> int:
