@@ -1,6 +1,6 @@
 """Stand-alone measurements of the sparse kernels on one MI355X.
 
-    python -m cagnet_amd.microbench spmm   [--graph rmat20|reddit] [--widths 16,64,128,602]
+    python -m cagnet_amd.microbench spmm   [--graph rmat20|reddit|amazon] [--widths 16,64,128,602]
     python -m cagnet_amd.microbench grid2d [--grid 4] [--row 1]
     python -m cagnet_amd.microbench prep   [--graph reddit]
 
@@ -27,6 +27,7 @@ GRAPHS = {
     "rmat20": dict(scale=20, n_edges=16_777_216),
     "reddit": dict(n=232_965, target_nnz=114_615_892),
     "rmat16": dict(scale=16, n_edges=1_048_576),
+    "amazon": dict(n=14_249_639, target_nnz=230_600_000),
 }
 
 
