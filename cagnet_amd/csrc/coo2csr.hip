@@ -51,7 +51,7 @@ int launch_rowptr(const int32_t *d_row, int64_t nnz, int32_t n, int32_t *d_rowpt
 // flags: bit0 index out of range, bit1 rows descend, bit2 (row, col) not strictly ascending
 __global__ __launch_bounds__(kThreads) void coo_check_kernel(const int32_t *__restrict__ row,
                                                              const int32_t *__restrict__ col, int64_t nnz, int32_t n,
-                                                             int32_t m, int *__restrict__ flags) {
+                                                             int32_t m, int care, int *__restrict__ flags) {
   const int64_t k = (int64_t)blockIdx.x * kThreads + threadIdx.x;
   int f = 0;
   if (k < nnz) {
@@ -64,7 +64,10 @@ __global__ __launch_bounds__(kThreads) void coo_check_kernel(const int32_t *__re
       if (col && (pr > r || (pr == r && col[k - 1] >= c))) f |= 4;
     }
   }
-  if (f) atomicOr(flags, f);  // integer OR: order independent
+  f &= care;  // only what the caller asked about (unsorted input is expected on the general path)
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) f |= __shfl_xor(f, off, kWave);
+  if (f && (threadIdx.x & (kWave - 1)) == 0) atomicOr(flags, f);  // one per wavefront; integer OR: order independent
 }
 
 __global__ __launch_bounds__(kThreads) void iota_kernel(int32_t *__restrict__ out, int64_t count) {
@@ -110,7 +113,8 @@ int coo_check(const int32_t *d_row, const int32_t *d_col, int64_t nnz, int32_t n
   void *d_flags = nullptr;
   CG_TRY(scratch_get(stream, kSlotD, sizeof(int), &d_flags));
   CG_HIP(hipMemsetAsync(d_flags, 0, sizeof(int), stream));
-  coo_check_kernel<<<(unsigned)ceil_div64(nnz, kThreads), kThreads, 0, stream>>>(d_row, d_col, nnz, n, m,
+  const int care = 1 | (require_sorted >= 1 ? 2 : 0) | (require_sorted >= 2 ? 4 : 0);
+  coo_check_kernel<<<(unsigned)ceil_div64(nnz, kThreads), kThreads, 0, stream>>>(d_row, d_col, nnz, n, m, care,
                                                                                  (int *)d_flags);
   CG_LAUNCH_CHECK();
   int flags = 0;
@@ -122,36 +126,48 @@ int coo_check(const int32_t *d_row, const int32_t *d_col, int64_t nnz, int32_t n
   return CG_OK;
 }
 
-struct DevFree {
-  void *p[8];
-  int count = 0;
-  ~DevFree() {
-    for (int i = 0; i < count; ++i)
-      if (p[i]) (void)hipFree(p[i]);
+// One device allocation carved into the temporaries of an operation (every hipMalloc / hipFree of a
+// few hundred MB costs milliseconds, more than the kernels that use it).
+struct DevArena {
+  char *base = nullptr;
+  size_t cap = 0, off = 0;
+  ~DevArena() {
+    if (base) (void)hipFree(base);
   }
-  int alloc(void **out, size_t bytes) {
-    hipError_t e = hipMalloc(out, bytes ? bytes : 4);
+  static size_t pad(size_t bytes) { return (bytes + 255) & ~(size_t)255; }
+  int reserve(size_t bytes) {
+    hipError_t e = hipMalloc((void **)&base, bytes ? bytes : 256);
     if (e != hipSuccess) {
       (void)hipGetLastError();
+      base = nullptr;
       set_error("hipMalloc of %zu bytes failed: %s", bytes, hipGetErrorString(e));
       return CG_ERR_ALLOC;
     }
-    p[count++] = *out;
+    cap = bytes;
+    return CG_OK;
+  }
+  int take(void **out, size_t bytes) {
+    const size_t need = pad(bytes);
+    if (off + need > cap) CG_FAIL(CG_ERR_ALLOC, "temporary arena too small (%zu + %zu > %zu)", off, need, cap);
+    *out = base + off;
+    off += need;
     return CG_OK;
   }
 };
 
+static size_t sort_coo_bytes(int64_t count) { return 6 * DevArena::pad((size_t)count * sizeof(int32_t)); }
+
 // Sort records (key_a major, key_b minor) carrying the input position; hand back the sorted
 // key arrays and the permutation in caller-owned outputs.
-int sort_coo(const int32_t *d_key_a, const int32_t *d_key_b, int64_t count, int bits_a, int bits_b,
-             int32_t *d_out_a, int32_t *d_out_b, int32_t *d_out_perm, hipStream_t stream) {
-  DevFree tmp;
+// `tmp` must have sort_coo_bytes(count) left.
+static int sort_coo(const int32_t *d_key_a, const int32_t *d_key_b, int64_t count, int bits_a, int bits_b,
+                    int32_t *d_out_a, int32_t *d_out_b, int32_t *d_out_perm, DevArena &tmp, hipStream_t stream) {
   SortBuffers buf;
   const size_t bytes = (size_t)count * sizeof(int32_t);
   for (int s = 0; s < 2; ++s) {
-    CG_TRY(tmp.alloc((void **)&buf.key_a[s], bytes));
-    CG_TRY(tmp.alloc((void **)&buf.key_b[s], bytes));
-    CG_TRY(tmp.alloc((void **)&buf.payload[s], bytes));
+    CG_TRY(tmp.take((void **)&buf.key_a[s], bytes));
+    CG_TRY(tmp.take((void **)&buf.key_b[s], bytes));
+    CG_TRY(tmp.take((void **)&buf.payload[s], bytes));
   }
   if (count > 0) {
     CG_HIP(hipMemcpyAsync(buf.key_a[0], d_key_a, bytes, hipMemcpyDeviceToDevice, stream));
@@ -166,18 +182,19 @@ int sort_coo(const int32_t *d_key_a, const int32_t *d_key_b, int64_t count, int 
     if (d_out_b) CG_HIP(hipMemcpyAsync(d_out_b, buf.key_b[set], bytes, hipMemcpyDeviceToDevice, stream));
     if (d_out_perm) CG_HIP(hipMemcpyAsync(d_out_perm, buf.payload[set], bytes, hipMemcpyDeviceToDevice, stream));
   }
-  CG_HIP(hipStreamSynchronize(stream));  // the temporaries are freed when `tmp` goes out of scope
-  return CG_OK;
+  return CG_OK;  // the caller synchronises before its arena goes away
 }
 
 int coo2csr_general(const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz, int32_t n,
                     int32_t m, int32_t *d_rowptr, int32_t *d_colind, float *d_values, int32_t *d_perm,
                     hipStream_t stream) {
-  DevFree tmp;
+  DevArena tmp;
+  const size_t ebytes = (size_t)nnz * sizeof(int32_t);
+  CG_TRY(tmp.reserve(sort_coo_bytes(nnz) + 2 * DevArena::pad(ebytes)));
   int32_t *d_rows_sorted = nullptr, *d_perm_local = d_perm;
-  CG_TRY(tmp.alloc((void **)&d_rows_sorted, (size_t)nnz * sizeof(int32_t)));
-  if (!d_perm_local) CG_TRY(tmp.alloc((void **)&d_perm_local, (size_t)nnz * sizeof(int32_t)));
-  CG_TRY(sort_coo(d_row, d_col, nnz, bits_for(n), bits_for(m), d_rows_sorted, d_colind, d_perm_local, stream));
+  CG_TRY(tmp.take((void **)&d_rows_sorted, ebytes));
+  if (!d_perm_local) CG_TRY(tmp.take((void **)&d_perm_local, ebytes));
+  CG_TRY(sort_coo(d_row, d_col, nnz, bits_for(n), bits_for(m), d_rows_sorted, d_colind, d_perm_local, tmp, stream));
   CG_TRY(launch_rowptr(d_rows_sorted, nnz, n, d_rowptr, stream));
   if (d_val && d_values && nnz > 0) {
     gather_f32_kernel<<<(unsigned)ceil_div64(nnz, kThreads), kThreads, 0, stream>>>(d_val, d_perm_local, d_values,
@@ -191,11 +208,13 @@ int coo2csr_general(const int32_t *d_row, const int32_t *d_col, const float *d_v
 int csr_transpose(const int32_t *d_rowptr, const int32_t *d_colind, const float *d_values, int64_t nnz, int32_t n,
                   int32_t m, int32_t *d_colptr, int32_t *d_rowind, float *d_values_t, int32_t *d_perm,
                   hipStream_t stream) {
-  DevFree tmp;
+  DevArena tmp;
+  const size_t ebytes = (size_t)nnz * sizeof(int32_t);
+  CG_TRY(tmp.reserve(sort_coo_bytes(nnz) + 3 * DevArena::pad(ebytes)));
   int32_t *d_rows = nullptr, *d_cols_sorted = nullptr, *d_perm_local = d_perm;
-  CG_TRY(tmp.alloc((void **)&d_rows, (size_t)nnz * sizeof(int32_t)));
-  CG_TRY(tmp.alloc((void **)&d_cols_sorted, (size_t)nnz * sizeof(int32_t)));
-  if (!d_perm_local) CG_TRY(tmp.alloc((void **)&d_perm_local, (size_t)nnz * sizeof(int32_t)));
+  CG_TRY(tmp.take((void **)&d_rows, ebytes));
+  CG_TRY(tmp.take((void **)&d_cols_sorted, ebytes));
+  if (!d_perm_local) CG_TRY(tmp.take((void **)&d_perm_local, ebytes));
   if (n > 0) {
     csr_expand_rows_kernel<<<(unsigned)ceil_div64((int64_t)n * kWave, kThreads), kThreads, 0, stream>>>(d_rowptr, n,
                                                                                                        d_rows);
@@ -203,7 +222,7 @@ int csr_transpose(const int32_t *d_rowptr, const int32_t *d_colind, const float 
   }
   // CSR order is (row, col) ascending, so a stable sort on col alone yields (col, row) order:
   // major key = col (key_a), minor key = row with zero bits (already in place).
-  CG_TRY(sort_coo(d_colind, d_rows, nnz, bits_for(m), 0, d_cols_sorted, d_rowind, d_perm_local, stream));
+  CG_TRY(sort_coo(d_colind, d_rows, nnz, bits_for(m), 0, d_cols_sorted, d_rowind, d_perm_local, tmp, stream));
   CG_TRY(launch_rowptr(d_cols_sorted, nnz, m, d_colptr, stream));
   if (d_values && d_values_t && nnz > 0) {
     gather_f32_kernel<<<(unsigned)ceil_div64(nnz, kThreads), kThreads, 0, stream>>>(d_values, d_perm_local,

@@ -145,22 +145,28 @@ __global__ __launch_bounds__(kSortThreads) void radix_hist_kernel(const int32_t 
 
 // Stable scatter.  Wave w of a workgroup owns keys [tile + 1024 w, tile + 1024 (w+1)) and ranks
 // them 64 at a time: lanes holding equal digits find each other with 8 ballots, their rank is the
-// number of lower lanes in that peer set plus the wave's running count of the digit.
+// number of lower lanes in that peer set plus the wave's running count of the digit.  The records
+// are then ordered by digit inside LDS and written out from there, so that the records of one
+// digit leave as one contiguous run instead of one 4-byte store each.
 __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
-    const int32_t *__restrict__ key, int shift, const int32_t *__restrict__ in_a, const int32_t *__restrict__ in_b,
+    int key_is_a, int shift, const int32_t *__restrict__ in_a, const int32_t *__restrict__ in_b,
     const int32_t *__restrict__ in_p, int32_t *__restrict__ out_a, int32_t *__restrict__ out_b,
     int32_t *__restrict__ out_p, int64_t count, const uint32_t *__restrict__ scanned_hist, int64_t tiles) {
   __shared__ uint32_t cnt[kSortWaves][kRadix];
+  __shared__ uint32_t goff[kRadix];        // global position of a record = goff[digit] + its position in the tile
+  __shared__ uint32_t wave_total[kSortWaves];
+  __shared__ int32_t sa[kSortTile], sb[kSortTile], sp[kSortTile];
   for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) (&cnt[0][0])[i] = 0;
   __syncthreads();
 
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const uint64_t lt_mask = (1ull << lane) - 1ull;
-  const int64_t base = (int64_t)blockIdx.x * kSortTile + (int64_t)wave * kSortWaveTile;
+  const int64_t tile_base = (int64_t)blockIdx.x * kSortTile;
+  const int64_t base = tile_base + (int64_t)wave * kSortWaveTile;
 
   int32_t ra[kSortRounds], rb[kSortRounds], rp[kSortRounds];
-  uint32_t packed[kSortRounds];  // digit | local rank << 8
+  uint32_t packed[kSortRounds];  // digit | rank among the wave's records of that digit << 8
 
 #pragma unroll
   for (int r = 0; r < kSortRounds; ++r) {
@@ -168,10 +174,10 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
     const bool valid = idx < count;
     uint32_t d = 0;
     if (valid) {
-      d = ((uint32_t)key[idx] >> shift) & (kRadix - 1);
       ra[r] = in_a[idx];
       rb[r] = in_b[idx];
       rp[r] = in_p[idx];
+      d = ((uint32_t)(key_is_a ? ra[r] : rb[r]) >> shift) & (kRadix - 1);
     }
     uint64_t peers = __ballot(valid);
 #pragma unroll
@@ -190,14 +196,30 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
   }
   __syncthreads();
 
-  {  // thread t owns digit t: turn per-wave counts into per-wave output offsets
+  {  // thread t owns digit t: exclusive scan of the tile's digit counts, then per-wave offsets
     const int t = threadIdx.x;
-    uint32_t run = scanned_hist[(int64_t)t * tiles + blockIdx.x];
+    uint32_t c[kSortWaves], total = 0;
 #pragma unroll
     for (int w = 0; w < kSortWaves; ++w) {
-      uint32_t c = cnt[w][t];
+      c[w] = cnt[w][t];
+      total += c[w];
+    }
+    uint32_t inc = total;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+      const uint32_t up = __shfl_up(inc, off, kWave);
+      if (lane >= off) inc += up;
+    }
+    if (lane == kWave - 1) wave_total[wave] = inc;
+    __syncthreads();
+    uint32_t excl = inc - total;
+    for (int w = 0; w < wave; ++w) excl += wave_total[w];
+    goff[t] = scanned_hist[(int64_t)t * tiles + blockIdx.x] - excl;  // modulo 2^32, undone by the addition below
+    uint32_t run = excl;
+#pragma unroll
+    for (int w = 0; w < kSortWaves; ++w) {
       cnt[w][t] = run;
-      run += c;
+      run += c[w];
     }
   }
   __syncthreads();
@@ -207,11 +229,23 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
     const int64_t idx = base + (int64_t)r * kWave + lane;
     if (idx < count) {
       const uint32_t d = packed[r] & (kRadix - 1);
-      const uint32_t pos = cnt[wave][d] + (packed[r] >> 8);
-      out_a[pos] = ra[r];
-      out_b[pos] = rb[r];
-      out_p[pos] = rp[r];
+      const uint32_t lpos = cnt[wave][d] + (packed[r] >> 8);
+      sa[lpos] = ra[r];
+      sb[lpos] = rb[r];
+      sp[lpos] = rp[r];
     }
+  }
+  __syncthreads();
+
+  const int64_t left = count - tile_base;
+  const int32_t here = (int32_t)(left < kSortTile ? left : kSortTile);
+  for (int32_t i = threadIdx.x; i < here; i += kSortThreads) {
+    const int32_t va = sa[i], vb = sb[i];
+    const uint32_t d = ((uint32_t)(key_is_a ? va : vb) >> shift) & (kRadix - 1);
+    const uint32_t pos = goff[d] + (uint32_t)i;
+    out_a[pos] = va;
+    out_b[pos] = vb;
+    out_p[pos] = sp[i];
   }
 }
 
@@ -233,7 +267,7 @@ int radix_sort_pairs(SortBuffers &buf, int64_t count, int bits_a, int bits_b, in
       CG_LAUNCH_CHECK();
       CG_TRY(exclusive_scan_u32(hist, hist, tiles * kRadix, nullptr, stream));
       radix_scatter_kernel<<<(unsigned)tiles, kSortThreads, 0, stream>>>(
-          key, shift, buf.key_a[cur], buf.key_b[cur], buf.payload[cur], buf.key_a[cur ^ 1], buf.key_b[cur ^ 1],
+          which, shift, buf.key_a[cur], buf.key_b[cur], buf.payload[cur], buf.key_a[cur ^ 1], buf.key_b[cur ^ 1],
           buf.payload[cur ^ 1], count, hist, tiles);
       CG_LAUNCH_CHECK();
       cur ^= 1;
