@@ -491,3 +491,43 @@ def test_blob_rejects_damage(cuda):
         ops.CsrMatrix.from_blob(orc.blob_write(rp, ci_bad, vv, n, m, False))
     with pytest.raises(ops.CagnetError, match="CG_ERR_SIZE"):
         ops.CsrMatrix.from_blob(good[:64])
+
+
+def test_dense_offsets_beyond_int32(cuda):
+    """Row-major operands with more than 2^31 elements (9.0 M rows x 256 floats = 9.2 GB each): a
+    few stored entries that touch the first and the last rows exercise the 64-bit addressing of the
+    gather, of the store and of the dense kernels without needing a large sparse matrix."""
+    from cagnet_amd import ops
+    n, f = 9_000_000, 256
+    assert n * f > 2 ** 31
+    gen = torch.Generator(device=cuda).manual_seed(3)
+    B = torch.randn(n, f, device=cuda, generator=gen)
+    rows = torch.tensor([0, 5, 4_500_000, n - 2, n - 1, n - 1], dtype=torch.int32, device=cuda)
+    cols = torch.tensor([n - 1, 7, n - 3, 0, n - 1, 11], dtype=torch.int32, device=cuda)
+    vals = torch.tensor([1.5, -2.0, 0.5, 3.0, -1.0, 2.0], device=cuda)
+    order = torch.argsort(rows.long() * n + cols.long())
+    rows, cols, vals = rows[order], cols[order], vals[order]
+    A = ops.CsrMatrix(rows, cols, vals, n, n)
+    C = A.spmm(B)
+    expect = {}
+    for r, c, v in zip(rows.tolist(), cols.tolist(), vals.tolist()):
+        expect[r] = expect.get(r, 0) + v * B[c].double()
+    for r, e in expect.items():
+        assert float((C[r].double() - e).abs().max()) <= 1e-5 * float(e.abs().max())
+    assert torch.count_nonzero(C[1]) == 0 and torch.count_nonzero(C[n - 3]) == 0
+    # dense products over the same tall operand: compare the last rows / the reduction with torch
+    W = torch.randn(f, 16, device=cuda, generator=gen)
+    Z = ops.dense_xw(B, W)
+    ref = B[n - 4:].double() @ W.double()
+    assert float((Z[n - 4:].double() - ref).abs().max()) <= 1e-4 * float(ref.abs().max())
+    G = torch.randn(n, 16, device=cuda, generator=gen)
+    dX = ops.dense_gwt(G, W, out=C)                   # reuses the 9.2 GB buffer
+    ref = G[n - 4:].double() @ W.double().t()
+    assert float((dX[n - 4:].double() - ref).abs().max()) <= 1e-4 * float(ref.abs().max())
+    G[: n - 1000] = 0                                  # X^T G then only sees the last 1000 rows
+    dW = ops.dense_xtg(B, G)
+    ref = B[n - 1000:].double().t() @ G[n - 1000:].double()
+    assert float((dW.double() - ref).abs().max()) <= 1e-4 * float(ref.abs().max())
+    del dX, C, G
+    H = ops.relu_fwd(B)                                # elementwise kernels index the same 2.3e9 elements
+    assert torch.equal(H[n - 1], B[n - 1].clamp_min(0)) and torch.equal(H[0], B[0].clamp_min(0))
