@@ -8,7 +8,8 @@
 //   A (16 x 4): lane holds A[l % 16][l / 16]        B (4 x 16): lane holds B[l / 16][l % 16]
 //   D (16 x 16) in 4 registers: register v of lane l holds D[4 * (l / 16) + v][l % 16]
 //
-//   xw_mfma  : Z[n, fo]   = X[n, k] * W[k, fo]  (+ReLU)   rows of X on the tile rows, W staged in LDS
+//   xw_mfma  : Z[n, fo]   = X[n, k] * W[k, fo]  (+ReLU)   computed as Z^T = W^T X^T: rows of X on the tile
+//                                                         columns, W staged in LDS
 //   xtg_mfma : dW[k, fo]  = X[n, k]^T * G[n, fo]          columns of X on the tile rows, vertices reduced
 // (dX = G W^T is bound by its stores and runs on the vector ALUs: dense_rows.hip, dense.hip.)
 #include "common.h"
@@ -24,11 +25,12 @@ __device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
 }
 
+// r = the VEC floats at p.  Loads are unconditional, from an address clamped into the operand, and
+// the values of dead lanes are zeroed where they are consumed (keep_k): with no branch around the
+// load and no use right behind it, the compiler counts outstanding loads exactly and loads issued
+// for a later step stay in flight across the multiplies of the current one.
 template <int VEC>
-__device__ __forceinline__ void load_k(const float *p, bool ok, float (&r)[VEC]) {
-#pragma unroll
-  for (int i = 0; i < VEC; ++i) r[i] = 0.f;
-  if (!ok) return;
+__device__ __forceinline__ void load_k(const float *p, float (&r)[VEC]) {
   if (VEC == 4) {
     const float4 t = *reinterpret_cast<const float4 *>(p);
     r[0] = t.x; r[1 % VEC] = t.y; r[2 % VEC] = t.z; r[3 % VEC] = t.w;
@@ -39,45 +41,75 @@ __device__ __forceinline__ void load_k(const float *p, bool ok, float (&r)[VEC])
     r[0] = p[0];
   }
 }
+__device__ __forceinline__ float keep_k(bool ok, float v) { return ok ? v : 0.f; }
 
 // ---------------------------------------------------------------------------------------------
 // Z = X W.  A wavefront owns 16 rows of X; lane (m, q) = (l % 16, l / 16) reads VEC consecutive
-// k-values of row m per step, which feed VEC instructions whose B operand comes from the W chunk
-// staged in LDS.  NT output tiles of 16 columns share every A value.
+// k-values of row m per step, which feed VEC instructions as the B operand (X^T); the A operand
+// (W^T) comes from the W chunk staged in LDS.  NT output tiles of 16 columns share every X value.
 // ---------------------------------------------------------------------------------------------
 constexpr int kXwChunk = 256;        // rows of W staged per pass when W does not fit LDS whole
 constexpr int kXwLdsBytes = 64 * 1024;
 
-// acc += X[rows of the wave, c0 .. c0+clen) * Ws, for the chunk of W staged in LDS (`cap` rows, zero padded)
+constexpr int kXwSteps = 4;  // load steps a wavefront keeps in flight
+
+// acc += X[row, c0 + kb .. c0 + kb + NS * STEP) * Ws for NS load steps.  Every load of X and every
+// LDS read of W is issued before the first multiply (the scheduling barrier keeps the compiler from
+// sinking them between the multiplies).  RAGGED: the last step crosses the end of the chunk; its
+// lanes past clen read a clamped address of X and contribute zeros.
+template <int VEC, int NT, int NS, bool RAGGED>
+__device__ __forceinline__ void xw_span(const float *__restrict__ xrow, int32_t c0, int32_t clen, int32_t kb,
+                                        const float *__restrict__ Ws, int m, int q, floatx4 (&acc)[NT]) {
+  constexpr int STEP = 4 * VEC;  // k-values one load step covers
+  float x[NS][VEC], w[NS][VEC][NT];
+#pragma unroll
+  for (int u = 0; u < NS; ++u) {
+    const int32_t kk = kb + u * STEP + q * VEC;
+    const bool live = !RAGGED || u < NS - 1 || kk < clen;  // VEC divides the chunk length: all or nothing
+    load_k<VEC>(xrow + c0 + (live ? kk : 0), x[u]);
+#pragma unroll
+    for (int s = 0; s < VEC; ++s)  // rows clen .. round_up(clen, span) of Ws exist and hold zeros
+#pragma unroll
+      for (int t = 0; t < NT; ++t) w[u][s][t] = Ws[(size_t)(kk + s) * (16 * NT) + t * 16 + m];
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int u = 0; u < NS; ++u) {
+    const bool live = !RAGGED || u < NS - 1 || kb + u * STEP + q * VEC < clen;
+#pragma unroll
+    for (int s = 0; s < VEC; ++s)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[t] = mfma16(w[u][s][t], keep_k(live, x[u][s]), acc[t]);
+  }
+}
+
+// acc += X[rows of the wave, c0 .. c0+clen) * Ws, for the chunk of W staged in LDS (zero padded to whole spans)
 template <int VEC, int NT>
 __device__ __forceinline__ void xw_accumulate(const float *__restrict__ xrow, int32_t c0, int32_t clen,
-                                              const float *__restrict__ Ws, int32_t cap, int m, int q,
-                                              floatx4 (&acc)[NT]) {
-  constexpr int STEP = 4 * VEC;  // k-values one load step covers
-  constexpr int U = 4;           // load steps in flight
-  for (int32_t kb = 0; kb < clen; kb += STEP * U) {
-    float x[U][VEC];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int32_t kk = kb + u * STEP + q * VEC;
-      load_k<VEC>(xrow + c0 + kk, kk + VEC <= clen, x[u]);
-      if (VEC > 1 && kk < clen && kk + VEC > clen) {  // ragged end of the row: element-wise
-#pragma unroll
-        for (int s = 0; s < VEC; ++s) x[u][s] = kk + s < clen ? xrow[c0 + kk + s] : 0.f;
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-#pragma unroll
-      for (int s = 0; s < VEC; ++s) {
-        const int32_t kk = kb + u * STEP + q * VEC + s;
-        if (kb + u * STEP < clen) {  // wave-uniform: skip steps past the chunk
-          const float *wrow = Ws + (size_t)(kk < cap ? kk : cap - 1) * (16 * NT);
-#pragma unroll
-          for (int t = 0; t < NT; ++t) acc[t] = mfma16(x[u][s], wrow[t * 16 + m], acc[t]);
-        }
-      }
-    }
+                                              const float *__restrict__ Ws, int m, int q, floatx4 (&acc)[NT]) {
+  constexpr int STEP = 4 * VEC, SPAN = STEP * kXwSteps;
+  int32_t kb = 0;
+  for (; kb + SPAN <= clen; kb += SPAN) xw_span<VEC, NT, kXwSteps, false>(xrow, c0, clen, kb, Ws, m, q, acc);
+  const int32_t left = clen - kb;  // < SPAN: up to kXwSteps - 1 whole steps and maybe a ragged one
+  static_assert(kXwSteps == 4, "the tail dispatch below lists the step counts of a 4-step span");
+  switch ((left + STEP - 1) / STEP) {  // wave-uniform
+    case 1:
+      if (left % STEP) xw_span<VEC, NT, 1, true>(xrow, c0, clen, kb, Ws, m, q, acc);
+      else xw_span<VEC, NT, 1, false>(xrow, c0, clen, kb, Ws, m, q, acc);
+      break;
+    case 2:
+      if (left % STEP) xw_span<VEC, NT, 2, true>(xrow, c0, clen, kb, Ws, m, q, acc);
+      else xw_span<VEC, NT, 2, false>(xrow, c0, clen, kb, Ws, m, q, acc);
+      break;
+    case 3:
+      if (left % STEP) xw_span<VEC, NT, 3, true>(xrow, c0, clen, kb, Ws, m, q, acc);
+      else xw_span<VEC, NT, 3, false>(xrow, c0, clen, kb, Ws, m, q, acc);
+      break;
+    case 4:  // left < SPAN: the fourth step is ragged
+      xw_span<VEC, NT, 4, true>(xrow, c0, clen, kb, Ws, m, q, acc);
+      break;
+    default:
+      break;
   }
 }
 
@@ -85,7 +117,7 @@ __device__ __forceinline__ void xw_accumulate(const float *__restrict__ xrow, in
 template <int VEC, int NT>
 __device__ __forceinline__ void xw_stage(const float *__restrict__ W, int64_t ldw, int32_t c0, int32_t clen,
                                          int32_t fo, float *__restrict__ Ws, int32_t cap) {
-  constexpr int kStepRows = 4 * VEC * 4;
+  constexpr int kStepRows = 4 * VEC * kXwSteps;
   int32_t stage_rows = (clen + kStepRows - 1) / kStepRows * kStepRows;
   if (stage_rows > cap) stage_rows = cap;
   for (int idx = threadIdx.x; idx < stage_rows * 16 * NT; idx += kMfmaThreads) {
@@ -94,20 +126,30 @@ __device__ __forceinline__ void xw_stage(const float *__restrict__ W, int64_t ld
   }
 }
 
+// The accumulators hold the transposed tile (W^T on the A side, X^T on the B side): register v of
+// lane (m, q) is Z[r0 + m][16 t + 4 q + v], so a lane stores four consecutive columns of one row and
+// a wavefront writes whole 64-byte row pieces (the whole 1 KB tile when ldz = 16).
 template <int NT>
 __device__ __forceinline__ void xw_store(const floatx4 (&acc)[NT], float *__restrict__ Z, int64_t ldz, int64_t r0,
                                          int64_t n, int32_t fo, int relu, int m, int q) {
+  const int64_t orow = r0 + m;
+  if (orow >= n) return;
+  const bool vec_ok = ldz % 4 == 0 && ((uintptr_t)Z) % 16 == 0;
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
+    const int32_t col = t * 16 + 4 * q;
+    floatx4 o = acc[t];
+    if (relu) {
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const int64_t orow = r0 + 4 * q + v;
-      const int32_t col = t * 16 + m;
-      if (orow < n && col < fo) {
-        float o = acc[t][v];
-        if (relu && o < 0.f) o = 0.f;
-        Z[orow * ldz + col] = o;
-      }
+      for (int v = 0; v < 4; ++v) o[v] = o[v] < 0.f ? 0.f : o[v];
+    }
+    float *dst = Z + orow * ldz + col;
+    if (vec_ok && col + 4 <= fo) {
+      *reinterpret_cast<floatx4 *>(dst) = o;
+    } else {
+#pragma unroll
+      for (int v = 0; v < 4; ++v)
+        if (col + v < fo) dst[v] = o[v];
     }
   }
 }
@@ -133,7 +175,7 @@ __global__ __launch_bounds__(kMfmaThreads) void xw_mfma_kernel(const float *__re
       floatx4 acc[NT];
 #pragma unroll
       for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-      xw_accumulate<VEC, NT>(X + row * ldx, 0, k, Ws, cap, m, q, acc);
+      xw_accumulate<VEC, NT>(X + row * ldx, 0, k, Ws, m, q, acc);
       xw_store<NT>(acc, Z, ldz, r0, n, fo, relu, m, q);
     }
     return;
@@ -149,7 +191,7 @@ __global__ __launch_bounds__(kMfmaThreads) void xw_mfma_kernel(const float *__re
     __syncthreads();
     xw_stage<VEC, NT>(W, ldw, c0, clen, fo, Ws, cap);
     __syncthreads();
-    xw_accumulate<VEC, NT>(X + row * ldx, c0, clen, Ws, cap, m, q, acc);
+    xw_accumulate<VEC, NT>(X + row * ldx, c0, clen, Ws, m, q, acc);
   }
   xw_store<NT>(acc, Z, ldz, r0, n, fo, relu, m, q);
 }
@@ -187,24 +229,23 @@ __global__ __launch_bounds__(kMfmaThreads) void xtg_mfma_kernel(const float *__r
     for (int u = 0; u < U; ++u) {
       const int64_t rr = r + u * 4 + q;
       const bool live = rr < r1;
-      const float *xp = X + (live ? rr : r0) * ldx + kcol;
-      load_k<VEC>(xp, live && full, x[u]);
-      if (VEC > 1 && live && !full) {
-#pragma unroll
-        for (int s = 0; s < VEC; ++s) x[u][s] = kcol + s < k ? xp[s] : 0.f;
-      }
+      // VEC divides k: a lane's columns are all inside or all outside
+      load_k<VEC>(X + (live ? rr : r0) * ldx + (full ? kcol : 0), x[u]);
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         const int32_t c = t * 16 + m;
-        g[u][t] = (live && c < fo) ? G[rr * ldg + c] : 0.f;
+        g[u][t] = G[(live ? rr : r0) * ldg + (c < fo ? c : 0)];
       }
     }
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int u = 0; u < U; ++u) {
+      const bool live = r + u * 4 + q < r1;
 #pragma unroll
       for (int s = 0; s < VEC; ++s)
 #pragma unroll
-        for (int t = 0; t < NT; ++t) acc[s][t] = mfma16(x[u][s], g[u][t], acc[s][t]);
+        for (int t = 0; t < NT; ++t)
+          acc[s][t] = mfma16(keep_k(live && full, x[u][s]), keep_k(live && t * 16 + m < fo, g[u][t]), acc[s][t]);
+    }
   }
   float *out = P + (int64_t)blockIdx.x * k * fo;
 #pragma unroll
@@ -222,9 +263,10 @@ __global__ __launch_bounds__(kMfmaThreads) void xtg_mfma_kernel(const float *__r
 // ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
+// widest aligned load that divides k, so no load straddles the end of a row
 static int pick_kvec(const float *X, int64_t ldx, int32_t k) {
-  if (ldx % 4 == 0 && ((uintptr_t)X) % 16 == 0 && k >= 4) return 4;
-  if (ldx % 2 == 0 && ((uintptr_t)X) % 8 == 0 && k >= 2) return 2;
+  if (ldx % 4 == 0 && ((uintptr_t)X) % 16 == 0 && k % 4 == 0) return 4;
+  if (ldx % 2 == 0 && ((uintptr_t)X) % 8 == 0 && k % 2 == 0) return 2;
   return 1;
 }
 
@@ -235,7 +277,7 @@ int xw_mfma(const float *X, int64_t ldx, const float *W, int64_t ldw, float *Z, 
   const int64_t tiles = ceil_div64(n, 16 * kMfmaWaves);
   if (tiles > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "cg_dense_xw: grid too large");
   // W whole in LDS when it fits (rows rounded up to what the last load steps touch)
-  const int step_rows = 4 * vec * 4;
+  const int step_rows = 4 * vec * kXwSteps;
   const int64_t whole = ceil_div64(k, step_rows) * step_rows;
   const size_t row_bytes = (size_t)16 * nt * sizeof(float);
   int32_t cap = kXwChunk;
