@@ -18,7 +18,8 @@ int xw_mfma(const float *X, int64_t ldx, const float *W, int64_t ldw, float *Z, 
             int32_t fo, int relu, hipStream_t stream);
 int xtg_mfma(const float *X, int64_t ldx, const float *G, int64_t ldg, float *P, int64_t n, int32_t k, int32_t fo,
              int64_t rows_per_block, int64_t nblocks, hipStream_t stream);
-int xtg_vec(const float *X, int64_t ldx, int32_t k);
+void xtg_plan(const float *X, int64_t ldx, int64_t n, int32_t k, int32_t fo, int64_t *nranges,
+              int64_t *rows_per_range);
 // dense_rows.hip
 int gwt_rows(const float *G, int64_t ldg, const float *W, int64_t ldw, float *dX, int64_t lddx, int64_t n, int32_t k,
              int32_t fo, hipStream_t stream);
@@ -278,13 +279,8 @@ int cg_dense_xtg(const float *d_X, int64_t ldx, const float *d_G, int64_t ldg, f
   if (ldx < k || ldg < fo || lddw < fo) CG_FAIL(CG_ERR_SIZE, "cg_dense_xtg: leading dimension too small");
   if (fo <= 64 && n > 0 && g_tune_dense_mfma.load(std::memory_order_relaxed) >= 0) {
     ProfScope prof("dense_xtg", k, stream);
-    // contiguous vertex ranges, enough wavefronts to keep ~16 per CU in flight
-    const int vecw = xtg_vec(d_X, ldx, k);
-    const int64_t ywaves = ceil_div64(k, 16 * vecw);
-    int64_t nblocks = ceil_div64(8192, ywaves);
-    int64_t rows_per_block = ceil_div64(ceil_div64(n, nblocks), 16) * 16;
-    if (rows_per_block < 256) rows_per_block = 256;  // the partial product a range writes stays small beside its reads
-    nblocks = ceil_div64(n, rows_per_block);
+    int64_t nblocks = 0, rows_per_block = 0;
+    xtg_plan(d_X, ldx, n, k, fo, &nblocks, &rows_per_block);
     const int64_t elems = (int64_t)k * fo;
     void *p = nullptr;
     CG_TRY(scratch_get(stream, kSlotA, (size_t)nblocks * elems * sizeof(float), &p));

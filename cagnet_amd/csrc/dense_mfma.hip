@@ -197,67 +197,96 @@ __global__ __launch_bounds__(kMfmaThreads) void xw_mfma_kernel(const float *__re
 }
 
 // ---------------------------------------------------------------------------------------------
-// dW = X^T G.  A wavefront owns 16 * VEC columns of X and all fo columns of G; every step consumes
-// 4 vertices: lane (m, q) reads VEC consecutive columns of vertex row r + q, lane (j, q) of the B
-// side reads G[r + q][16 t + j].  Workgroups take contiguous vertex ranges and write partial
-// products that are added in order afterwards.
+// dW = X^T G.  A wavefront owns CT adjacent column tiles of X (16 * VEC columns each: the whole
+// row when k <= CT * 16 * VEC) and all fo columns of G, and walks a contiguous range of vertices
+// 4 at a time: lane (m, q) reads VEC consecutive columns per tile of vertex row r + q, lane (j, q)
+// of the B side reads G[r + q][16 t + j].  A wavefront therefore reads whole contiguous pieces of
+// rows by itself -- rows split between wavefronts at boundaries that are not cache-line aligned
+// were measured a fifth slower -- and writes one partial product; the partial products of all
+// ranges are added in order afterwards.
 // ---------------------------------------------------------------------------------------------
-template <int VEC, int NT>
-__global__ __launch_bounds__(kMfmaThreads) void xtg_mfma_kernel(const float *__restrict__ X, int64_t ldx,
-                                                                const float *__restrict__ G, int64_t ldg,
-                                                                float *__restrict__ P, int64_t n, int32_t k,
-                                                                int32_t fo, int64_t rows_per_block) {
-  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  const int m = lane & 15, q = lane >> 4;
-  const int32_t kt0 = (blockIdx.y * (blockDim.x / kWave) + wave) * 16 * VEC;  // first column of this wave
-  if (kt0 >= k) return;
-  const int32_t kcol = kt0 + m * VEC;
-  const bool full = kcol + VEC <= k;
-  const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
-  const int64_t r1 = r0 + rows_per_block < n ? r0 + rows_per_block : n;
+template <int CT>
+struct XtgSteps {  // 4-vertex steps in flight: about 8 to 10 loads of X per lane
+  static constexpr int value = CT == 1 ? 8 : CT == 2 ? 4 : CT == 3 ? 3 : 2;
+};
 
-  floatx4 acc[VEC][NT];
-#pragma unroll
-  for (int s = 0; s < VEC; ++s)
-#pragma unroll
-    for (int t = 0; t < NT; ++t) acc[s][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+template <int VEC, int NT, int CT>
+__global__ __launch_bounds__(kWave) void xtg_mfma_kernel(const float *__restrict__ X, int64_t ldx,
+                                                         const float *__restrict__ G, int64_t ldg,
+                                                         float *__restrict__ P, int64_t n, int32_t k, int32_t fo,
+                                                         int64_t rows_per_range) {
+  constexpr int U = XtgSteps<CT>::value;
+  const int lane = threadIdx.x, m = lane & 15, q = lane >> 4;
+  const int32_t kt0 = blockIdx.y * (CT * 16 * VEC);  // first column of this wavefront
+  const int64_t r0 = (int64_t)blockIdx.x * rows_per_range;
+  const int64_t r1 = r0 + rows_per_range < n ? r0 + rows_per_range : n;
 
-  constexpr int U = 8;  // 4-vertex steps in flight
+  // VEC divides k: the columns of a lane are all inside or all outside
+  int32_t xoff[CT];
+  bool xlive[CT];
+  int32_t goff[NT];
+  bool glive[NT];
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+    const int32_t col = kt0 + c * 16 * VEC + m * VEC;
+    xlive[c] = col + VEC <= k;
+    xoff[c] = xlive[c] ? col : 0;
+  }
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    glive[t] = t * 16 + m < fo;
+    goff[t] = glive[t] ? t * 16 + m : 0;
+  }
+
+  floatx4 acc[CT][VEC][NT];
+#pragma unroll
+  for (int c = 0; c < CT; ++c)
+#pragma unroll
+    for (int s = 0; s < VEC; ++s)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[c][s][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
   for (int64_t r = r0; r < r1; r += 4 * U) {
-    float x[U][VEC], g[U][NT];
+    float x[U][CT][VEC], g[U][NT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int64_t rr = r + u * 4 + q;
-      const bool live = rr < r1;
-      // VEC divides k: a lane's columns are all inside or all outside
-      load_k<VEC>(X + (live ? rr : r0) * ldx + (full ? kcol : 0), x[u]);
+      const int64_t row = rr < r1 ? rr : r0;  // clamped, dropped below
 #pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        const int32_t c = t * 16 + m;
-        g[u][t] = G[(live ? rr : r0) * ldg + (c < fo ? c : 0)];
-      }
+      for (int c = 0; c < CT; ++c) load_k<VEC>(X + row * ldx + xoff[c], x[u][c]);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) g[u][t] = G[row * ldg + goff[t]];
     }
+    __builtin_amdgcn_sched_barrier(0);  // every load of the round is issued before its first multiply
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const bool live = r + u * 4 + q < r1;
 #pragma unroll
-      for (int s = 0; s < VEC; ++s)
+      for (int t = 0; t < NT; ++t) g[u][t] = keep_k(live && glive[t], g[u][t]);
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
-          acc[s][t] = mfma16(keep_k(live && full, x[u][s]), keep_k(live && t * 16 + m < fo, g[u][t]), acc[s][t]);
+      for (int c = 0; c < CT; ++c)
+#pragma unroll
+        for (int s = 0; s < VEC; ++s) {
+          const float xv = keep_k(live && xlive[c], x[u][c][s]);
+#pragma unroll
+          for (int t = 0; t < NT; ++t) acc[c][s][t] = mfma16(xv, g[u][t], acc[c][s][t]);
+        }
     }
   }
   float *out = P + (int64_t)blockIdx.x * k * fo;
 #pragma unroll
-  for (int s = 0; s < VEC; ++s)
+  for (int c = 0; c < CT; ++c)
 #pragma unroll
-    for (int t = 0; t < NT; ++t)
+    for (int s = 0; s < VEC; ++s)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const int32_t kc = kt0 + (4 * q + v) * VEC + s;  // tile row i = 4q + v holds column kt0 + i*VEC + s
-        const int32_t c = t * 16 + m;
-        if (kc < k && c < fo) out[(int64_t)kc * fo + c] = acc[s][t][v];
-      }
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          // tile row i = 4q + v of tile c holds column kt0 + 16 c VEC + i VEC + s
+          const int32_t kc = kt0 + c * 16 * VEC + (4 * q + v) * VEC + s;
+          const int32_t col = t * 16 + m;
+          if (kc < k && col < fo) out[(int64_t)kc * fo + col] = acc[c][s][t][v];
+        }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -304,28 +333,51 @@ int xw_mfma(const float *X, int64_t ldx, const float *W, int64_t ldw, float *Z, 
 
 // Columns of X a lane reads per vertex: as wide as alignment allows, but no wider than keeps the 16
 // lanes of a tile row on live columns (k = 16 -> one column per lane).
-int xtg_vec(const float *X, int64_t ldx, int32_t k) {
+static int xtg_vec(const float *X, int64_t ldx, int32_t k) {
   int vec = pick_kvec(X, ldx, k);
   while (vec > 1 && 16 * vec > k) vec >>= 1;
   return vec;
 }
 
+// column tiles one wavefront owns: bounded by the accumulator registers (CT * VEC * NT tiles of 4)
+static int xtg_tiles_per_wave(int32_t k, int vec, int nt, int64_t *groups) {
+  const int64_t tiles = ceil_div64(k, 16 * vec);
+  const int cap = nt == 1 ? 5 : (nt == 2 ? 3 : 2);
+  *groups = ceil_div64(tiles, cap);
+  return (int)ceil_div64(tiles, *groups);
+}
+
+// Vertex ranges of X^T G: one wavefront per (range, column group).  About 4096 wavefronts in all
+// (several per SIMD in flight, with slack so the last ones do not run alone), ranges of at least
+// 256 vertices so the partial product a range writes stays small beside what it reads.
+void xtg_plan(const float *X, int64_t ldx, int64_t n, int32_t k, int32_t fo, int64_t *nranges,
+              int64_t *rows_per_range) {
+  int64_t groups = 1;
+  xtg_tiles_per_wave(k, xtg_vec(X, ldx, k), (fo + 15) / 16, &groups);
+  int64_t ranges = ceil_div64(4096, groups);
+  int64_t rows = ceil_div64(ceil_div64(n, ranges), 16) * 16;
+  if (rows < 256) rows = 256;
+  *rows_per_range = rows;
+  *nranges = ceil_div64(n, rows);
+}
+
 int xtg_mfma(const float *X, int64_t ldx, const float *G, int64_t ldg, float *P, int64_t n, int32_t k, int32_t fo,
-             int64_t rows_per_block, int64_t nblocks, hipStream_t stream) {
+             int64_t rows_per_range, int64_t nranges, hipStream_t stream) {
   const int nt = (fo + 15) / 16;
   const int vec = xtg_vec(X, ldx, k);
-  const int64_t ywaves = ceil_div64(k, 16 * vec);
-  // narrow X: fewer wavefronts per workgroup, so none of them is without columns
-  const int wpb = ywaves < kMfmaWaves ? (int)ywaves : kMfmaWaves;
-  dim3 grid((unsigned)nblocks, (unsigned)ceil_div64(ywaves, wpb));
-  const unsigned threads = (unsigned)(wpb * kWave);
-#define CG_CASE(V, T)                                                                                         \
-  if (vec == V && nt == T) {                                                                                  \
-    xtg_mfma_kernel<V, T><<<grid, threads, 0, stream>>>(X, ldx, G, ldg, P, n, k, fo, rows_per_block);    \
+  int64_t groups = 1;
+  const int ct = xtg_tiles_per_wave(k, vec, nt, &groups);
+  if (nranges > 0x7fffffffLL || groups > 65535) CG_FAIL(CG_ERR_SIZE, "cg_dense_xtg: grid too large");
+  dim3 grid((unsigned)nranges, (unsigned)groups);
+#define CG_CASE(V, T, C)                                                                                      \
+  if (vec == V && nt == T && ct == C) {                                                                       \
+    xtg_mfma_kernel<V, T, C><<<grid, kWave, 0, stream>>>(X, ldx, G, ldg, P, n, k, fo, rows_per_range);        \
     CG_LAUNCH_CHECK();                                                                                        \
     return CG_OK;                                                                                             \
   }
-#define CG_CASES(V) CG_CASE(V, 1) CG_CASE(V, 2) CG_CASE(V, 3) CG_CASE(V, 4)
+#define CG_CASES(V)                                                                                           \
+  CG_CASE(V, 1, 1) CG_CASE(V, 1, 2) CG_CASE(V, 1, 3) CG_CASE(V, 1, 4) CG_CASE(V, 1, 5) CG_CASE(V, 2, 1)       \
+  CG_CASE(V, 2, 2) CG_CASE(V, 2, 3) CG_CASE(V, 3, 1) CG_CASE(V, 3, 2) CG_CASE(V, 4, 1) CG_CASE(V, 4, 2)
   CG_CASES(1) CG_CASES(2) CG_CASES(4)
 #undef CG_CASES
 #undef CG_CASE
