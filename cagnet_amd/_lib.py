@@ -46,6 +46,9 @@ _SIGNATURES = {
     "cg_coo2csr": [P, P, P, c_int64, c_int32, c_int32, P, P, P, P, P],
     "cg_csr_transpose": [P, P, P, c_int64, c_int32, c_int32, P, P, P, P, P],
     "cg_spmm_coo": [P, P, P, c_int64, c_int32, c_int32, P, c_int64, P, c_int64, c_int32, c_float, P],
+    "cg_spmm_coo_cached": [P, P, P, c_int64, c_int32, c_int32, P, c_int64, P, c_int64, c_int32, c_float, P],
+    "cg_coo_cache_clear": [],
+    "cg_coo_cache_info": [POINTER(c_int64)],
     "cg_csr_create": [POINTER(c_void_p), P, P, P, c_int64, c_int32, c_int32, c_uint32, P],
     "cg_csr_destroy": [P],
     "cg_csr_spmm": [P, c_int, P, c_int64, P, c_int64, c_int32, c_float, P],

@@ -187,9 +187,11 @@ def csr_transpose(rowptr: torch.Tensor, colind: torch.Tensor, values: Optional[t
 # SpMM
 # ------------------------------------------------------------------------------------------------
 def spmm_coo(row: torch.Tensor, col: torch.Tensor, val: torch.Tensor, n: int, m: int, B: torch.Tensor,
-             C: torch.Tensor, beta: float = 1.0) -> None:
+             C: torch.Tensor, beta: float = 1.0, cached: bool = False) -> None:
     """C[n,f] = beta*C + A*B with A as row-sorted COO; the one-shot form of the reference operator
-    (sparse-extension/sparse_coo_tensor.cu:113-240)."""
+    (sparse-extension/sparse_coo_tensor.cu:113-240).  cached=True recognises a block it has seen
+    before by a digest of its arrays and reuses the CSR, schedules and plans built then (one stream
+    synchronisation per call); cached=False rebuilds them as asynchronous device work."""
     row, col, val = _index(row, "row"), _index(col, "col"), _values(val, "val")
     if not (row.numel() == col.numel() == val.numel()):
         raise ValueError("row, col and val differ in length")
@@ -197,8 +199,21 @@ def spmm_coo(row: torch.Tensor, col: torch.Tensor, val: torch.Tensor, n: int, m:
     ldc = _out_rowmajor(C, "C")
     if B.shape[0] != m or C.shape[0] != n or B.shape[1] != C.shape[1]:
         raise ValueError(f"shape mismatch: A is {n}x{m}, B is {tuple(B.shape)}, C is {tuple(C.shape)}")
-    check(lib.cg_spmm_coo(_ptr(row), _ptr(col), _ptr(val), val.numel(), n, m, _ptr(B), ldb, _ptr(C), ldc,
-                          B.shape[1], float(beta), _stream()), "cg_spmm_coo")
+    fn, name = (lib.cg_spmm_coo_cached, "cg_spmm_coo_cached") if cached else (lib.cg_spmm_coo, "cg_spmm_coo")
+    check(fn(_ptr(row), _ptr(col), _ptr(val), val.numel(), n, m, _ptr(B), ldb, _ptr(C), ldc, B.shape[1],
+             float(beta), _stream()), name)
+
+
+def coo_cache_info() -> dict:
+    """Blocks spmm_coo(cached=True) keeps, and its hits / misses / evictions so far."""
+    info = (ctypes.c_int64 * 4)()
+    check(lib.cg_coo_cache_info(info), "cg_coo_cache_info")
+    return {"blocks": info[0], "hits": info[1], "misses": info[2], "evictions": info[3]}
+
+
+def coo_cache_clear() -> None:
+    """Drop every block spmm_coo(cached=True) keeps."""
+    check(lib.cg_coo_cache_clear(), "cg_coo_cache_clear")
 
 
 class _DeviceArray:

@@ -10,7 +10,14 @@ Differences a caller can observe, all deliberate:
   * errors raise (CagnetError) instead of being printed and ignored (sparse_coo_tensor.cu:20-30);
   * B and C keep their storage and their row-major layout; the reference hands both back as
     column-major strided views of fresh storage (sparse_coo_tensor.cu:166-168, :183-185, :233-239);
-  * the call is ordered on torch's current stream and does not synchronise the device.
+  * the call is ordered on torch's current stream; with `cache_blocks` (the default) it
+    synchronises that stream once per call to read back a 16-byte digest, without it not at all
+    (the reference synchronises the whole device on every call, sparse_coo_tensor.cu:231).
+
+`cache_blocks`: the reference's callers pass the same block at every stage of every epoch, as
+fresh `.int()` temporaries.  When True, spmm_gpu recognises a block by a digest of its arrays and
+reuses the CSR, schedules and plans built when it first saw it (cg_spmm_coo_cached); when False
+every call rebuilds them on the device (cg_spmm_coo).
 """
 from __future__ import annotations
 
@@ -20,7 +27,9 @@ import torch
 
 from . import ops
 
-__all__ = ["spmm_gpu", "sparse_coo_tensor_gpu", "coo2csr"]
+__all__ = ["spmm_gpu", "sparse_coo_tensor_gpu", "coo2csr", "cache_blocks"]
+
+cache_blocks = True
 
 
 def spmm_gpu(A_rowindices: torch.Tensor, A_colindices: torch.Tensor, A_values: torch.Tensor, n: int, m: int,
@@ -31,10 +40,10 @@ def spmm_gpu(A_rowindices: torch.Tensor, A_colindices: torch.Tensor, A_values: t
     if C.dim() == 2 and C.numel() > 0 and C.stride(1) != 1:
         # a transposed view, e.g. a C that an earlier reference-style call left column-major
         tmp = C.contiguous()
-        ops.spmm_coo(A_rowindices, A_colindices, A_values, int(n), int(m), B, tmp, beta=1.0)
+        ops.spmm_coo(A_rowindices, A_colindices, A_values, int(n), int(m), B, tmp, beta=1.0, cached=cache_blocks)
         C.copy_(tmp)
         return None
-    ops.spmm_coo(A_rowindices, A_colindices, A_values, int(n), int(m), B, C, beta=1.0)
+    ops.spmm_coo(A_rowindices, A_colindices, A_values, int(n), int(m), B, C, beta=1.0, cached=cache_blocks)
     return None
 
 

@@ -108,6 +108,30 @@ int cg_csr_transpose(const int32_t *d_rowptr, const int32_t *d_colind, const flo
 int cg_spmm_coo(const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz, int32_t n, int32_t m,
                 const float *d_B, int64_t ldb, float *d_C, int64_t ldc, int32_t f, float beta, cg_stream_t stream);
 
+/* Same product and checks as cg_spmm_coo, for the way the reference's callers use spmm_gpu: the same
+ * block at every stage of every epoch, through fresh `.indices()[k].int()` temporaries
+ * (gcn_distr.py:238-240), so neither addresses nor tensor identities tell whether a block was seen
+ * before.  Products that cg_csr_spmm would run with a column-popularity plan (wide, over a dense
+ * power-law block: the plan is far too costly to build per call) are handled here; every other
+ * product is passed to cg_spmm_coo, which rebuilds its plain schedule for less than a digest costs.
+ * A handled call computes a 128-bit digest of (row, col, val) on the device (one pass over
+ * 12 nnz bytes) and reads it back, which synchronises `stream` once; a block whose digest, nnz, n
+ * and m were seen before on this device reuses the handle built at its first sighting (a private
+ * copy of the arrays as CSR, the schedules and the column-popularity plans of cg_csr_spmm), and the
+ * result is bit-identical to cg_csr_spmm on such a handle.  A first sighting builds the handle
+ * as cg_csr_create(CG_CSR_SORTED) does: index ranges and row order are checked and reported
+ * (CG_ERR_INDEX, CG_ERR_UNSORTED).  Two different blocks with equal digests (probability about
+ * 2^-128 per pair) would be taken for one another.  The least recently used block is dropped
+ * beyond cg_tune_set("coo_cache_blocks", k) blocks (default 8; negative: keep none and behave as
+ * cg_spmm_coo).  Thread safe; products on one block are serialised. */
+int cg_spmm_coo_cached(const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz, int32_t n,
+                       int32_t m, const float *d_B, int64_t ldb, float *d_C, int64_t ldc, int32_t f, float beta,
+                       cg_stream_t stream);
+/* Drops every block cg_spmm_coo_cached keeps (device memory is freed once queued products finish). */
+int cg_coo_cache_clear(void);
+/* info = {blocks kept, hits, misses, evictions} since the library was loaded. */
+int cg_coo_cache_info(int64_t info[4]);
+
 /* ------------------------------------------------------------------------------------------
  * Cached handle: what the reference rebuilds on every call (index casts gcn_distr.py:238,
  * coo2csr, workspace malloc/free, sparse_coo_tensor.cu:136-231) is built once here.
@@ -252,6 +276,7 @@ int cg_prof_enable(int on);
  *   "spmm_hub_groups" XCD groups the hot columns are dealt to (1, 2, 4, 8)
  *   "spmm_hub_tiers"  tiers of hot columns (groups * tiers <= 16)
  *   "dense_mfma"      -1: dense products on the vector ALU tile kernel only
+ *   "coo_cache_blocks" blocks cg_spmm_coo_cached keeps (0: 8; negative: none)
  * An unknown key returns CG_ERR_UNSUPPORTED. */
 int cg_tune_set(const char *key, int value);
 int cg_prof_read(const char *name, double *total_ms, int64_t *launches);

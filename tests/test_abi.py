@@ -61,6 +61,14 @@ def test_status_codes_without_a_gpu():
     assert lib.cg_spmm_coo(one, one, one, 5, 4, 4, one, 3, one, 4, 4, 1.0, null) == E["size"]      # ldb < f
     assert lib.cg_spmm_coo(one, one, one, 5, 4, 4, one, 4, one, 4, 0, 1.0, null) == E["size"]      # f == 0
     assert lib.cg_spmm_coo(one, one, one, 5, 4, 4, one, 4, one, 4, 4, 1.0, null) == 10             # C aliases B
+    # the block-cache form checks the same things before it touches the device
+    assert lib.cg_spmm_coo_cached(null, null, null, -1, 4, 4, one, 4, one, 4, 4, 1.0, null) == E["size"]
+    assert lib.cg_spmm_coo_cached(null, null, null, 1 << 31, 4, 4, one, 4, one, 4, 4, 1.0, null) == E["overflow"]
+    assert lib.cg_spmm_coo_cached(null, null, null, 5, 4, 4, one, 4, one, 4, 4, 1.0, null) == E["null"]
+    assert lib.cg_spmm_coo_cached(one, one, one, 5, 4, 4, one, 3, one, 4, 4, 1.0, null) == E["size"]
+    assert lib.cg_coo_cache_info(None) == E["null"]
+    assert lib.cg_coo_cache_clear() == 0
+    assert lib.cg_spmm_coo_cached(one, one, one, 5, 4, 4, one, 4, one, 4, 4, 1.0, null) == 10
     assert b"alias" in lib.cg_last_error()
     h = ctypes.c_void_p(0)
     assert lib.cg_csr_create(ctypes.byref(h), null, null, null, 3, 4, 4, 1, null) == E["null"]

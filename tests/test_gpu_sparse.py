@@ -112,9 +112,18 @@ def test_spmm_handle_matches_oracle(cuda, f):
     assert spmm_error(C, row, col, val, n, n, B, C0) <= REL_TOL
 
 
+@pytest.fixture(params=[False, True], ids=["rebuild", "cached"])
+def spmm_gpu(request, monkeypatch):
+    """The drop-in operator in both of its modes: tables rebuilt on every call (cg_spmm_coo) and
+    blocks recognised by digest (cg_spmm_coo_cached)."""
+    from cagnet_amd import ops, sparse_coo_tensor_cpp as mod
+    monkeypatch.setattr(mod, "cache_blocks", request.param)
+    yield mod.spmm_gpu
+    ops.coo_cache_clear()
+
+
 @pytest.mark.parametrize("f", [16, 41, 602])
-def test_spmm_gpu_one_shot_matches_oracle(cuda, f):
-    from cagnet_amd.sparse_coo_tensor_cpp import spmm_gpu
+def test_spmm_gpu_one_shot_matches_oracle(cuda, spmm_gpu, f):
     row, col, val, n = small_graph(10, 20000, seed=100 + f)
     B = torch.randn(n, f, generator=torch.Generator().manual_seed(f))
     C0 = torch.randn(n, f, generator=torch.Generator().manual_seed(f + 1))
@@ -126,11 +135,11 @@ def test_spmm_gpu_one_shot_matches_oracle(cuda, f):
 
 
 @pytest.mark.parametrize("f", [16, 41, 602, 2600])
-def test_spmm_gpu_one_shot_split_rows_and_reuse(cuda, f):
-    """The one-shot operator rebuilds its tables in a reused arena on every call: long rows
-    (several segments), then a smaller matrix with empty rows on the same stream, then the first
-    again; every result is checked, and the repeat is bit-identical to the first."""
-    from cagnet_amd.sparse_coo_tensor_cpp import spmm_gpu
+def test_spmm_gpu_one_shot_split_rows_and_reuse(cuda, spmm_gpu, f):
+    """The one-shot operator rebuilds its tables in a reused arena on every call (or finds the
+    block again by its digest): long rows (several segments), then a smaller matrix with empty
+    rows on the same stream, then the first again; every result is checked, and the repeat is
+    bit-identical to the first."""
     n, m = 40, 6000
     row, col, val = random_coo(n, m, n * 3000, seed=f)
     B = torch.randn(m, f, generator=torch.Generator().manual_seed(1))
@@ -155,14 +164,87 @@ def test_spmm_gpu_one_shot_split_rows_and_reuse(cuda, f):
     assert torch.equal(C, C2)
 
 
-def test_spmm_gpu_one_shot_empty_inputs(cuda):
-    from cagnet_amd.sparse_coo_tensor_cpp import spmm_gpu
+def test_spmm_gpu_one_shot_empty_inputs(cuda, spmm_gpu):
     e32 = torch.empty(0, dtype=torch.int32, device=cuda)
     B = torch.randn(9, 8, device=cuda)
     C0 = torch.randn(5, 8, device=cuda)
     C = C0.clone()
     spmm_gpu(e32, e32, torch.empty(0, device=cuda), 5, 9, B, C)   # no stored entries: C is unchanged
     assert torch.equal(C, C0)
+
+
+def test_spmm_gpu_block_cache(cuda, tune):
+    """cg_spmm_coo_cached: a block is recognised by content, not by address or tensor identity; a
+    changed value is a different block; the result is the handle's, bit for bit; the least recently
+    used block is dropped beyond the capacity; unsorted rows are reported at the first sighting."""
+    from cagnet_amd import ops
+    tune("spmm_hub", 1)     # every product takes a column-popularity plan, so every block is kept
+    ops.coo_cache_clear()
+    base = ops.coo_cache_info()
+    n, f = 3000, 602
+    row, col, val = random_coo(n, n, 90000, seed=11)
+    B = torch.randn(n, f, generator=torch.Generator().manual_seed(12))
+    C0 = torch.randn(n, f, generator=torch.Generator().manual_seed(13))
+    Bd = B.to(cuda)
+    r, c, v = _i32(row, cuda), _i32(col, cuda), val.to(cuda)
+
+    def product(r, c, v):
+        C = C0.to(cuda).clone()
+        ops.spmm_coo(r, c, v, n, n, Bd, C, beta=1.0, cached=True)
+        return C
+
+    first = product(r, c, v)
+    assert spmm_error(first, row, col, val, n, n, B, C0) <= REL_TOL
+    again = product(r.clone(), c.clone(), v.clone())           # same content at other addresses
+    assert torch.equal(first, again)
+    pad = torch.zeros(r.numel() + 1, dtype=torch.int32, device=cuda)
+    pad[1:] = r                                                 # 4-byte aligned only: the scalar digest agrees
+    assert torch.equal(first, product(pad[1:], c, v))
+    assert ops.coo_cache_info()["hits"] - base["hits"] == 2
+    base["hits"] += 1
+    info = ops.coo_cache_info()
+    assert (info["blocks"], info["hits"] - base["hits"], info["misses"] - base["misses"]) == (1, 1, 1)
+    handle = ops.CsrMatrix(r, c, v, n, n)
+    assert torch.equal(first, handle.spmm(Bd, out=C0.to(cuda).clone(), beta=1.0))
+
+    v2 = v.clone()
+    v2[12345] += 1.0                                            # one value changed in place: another block
+    val2 = v2.cpu()
+    changed = product(r, c, v2)
+    assert spmm_error(changed, row, col, val2, n, n, B, C0) <= REL_TOL
+    assert not torch.equal(changed, first)
+    assert ops.coo_cache_info()["blocks"] == 2
+    swapped = c.clone()
+    swapped[[0, 1]] = swapped[[1, 0]]                           # same multiset of entries, other order
+    if not torch.equal(swapped, c):
+        product(r, swapped, v)
+        assert ops.coo_cache_info()["blocks"] == 3
+
+    tune("coo_cache_blocks", 2)
+    ops.coo_cache_clear()
+    blocks = []
+    for seed in (21, 22, 23):
+        rr, cc, vv = random_coo(500, 500, 4000, seed=seed)
+        blocks.append((_i32(rr, cuda), _i32(cc, cuda), vv.to(cuda), rr, cc, vv))
+    Bs = torch.randn(500, 16, generator=torch.Generator().manual_seed(1))
+    before = ops.coo_cache_info()
+    for k in (0, 1, 2, 0):                                       # 0 is evicted by 2 and rebuilt
+        rr, cc, vv, hr, hc, hv = blocks[k]
+        C = torch.zeros(500, 16, device=cuda)
+        ops.spmm_coo(rr, cc, vv, 500, 500, Bs.to(cuda), C, beta=0.0, cached=True)
+        assert spmm_error(C, hr, hc, hv, 500, 500, Bs, None) <= REL_TOL
+    after = ops.coo_cache_info()
+    assert after["blocks"] == 2
+    assert after["misses"] - before["misses"] == 4 and after["hits"] == before["hits"]
+    assert after["evictions"] - before["evictions"] == 2
+
+    bad = torch.tensor([5, 3, 7], dtype=torch.int32, device=cuda)  # rows descend
+    ones = torch.ones(3, device=cuda)
+    with pytest.raises(ops.CagnetError):
+        ops.spmm_coo(bad, bad, ones, 10, 10, torch.zeros(10, 4, device=cuda), torch.zeros(10, 4, device=cuda),
+                     cached=True)
+    ops.coo_cache_clear()
+    assert ops.coo_cache_info()["blocks"] == 0
 
 
 @pytest.mark.parametrize("f", [16, 41, 128, 602])
