@@ -19,7 +19,7 @@ extern std::atomic<int> g_tune_dense_mfma;  // dense.hip
 
 // Tuning knobs (cg_tune_set): 0 = built-in choice.
 static std::atomic<int> g_tune_seg{0}, g_tune_vec{0}, g_tune_win{0};
-static std::atomic<int> g_tune_hub{0}, g_tune_hub_kb{0}, g_tune_hub_groups{0}, g_tune_hub_tiers{0};
+static std::atomic<int> g_tune_hub{0}, g_tune_hub_kb{0}, g_tune_hub_groups{0}, g_tune_hub_tiers{0}, g_tune_hub_row{0};
 static std::atomic<int> g_tune_coo_cache{0};  // blocks cg_spmm_coo_cached keeps: 0 = 8, negative = none
 
 // ---------------------------------------------------------------------------------------------
@@ -577,7 +577,7 @@ struct SchedCache {
 // Entries are kept as one CSR over (classes + 1) * rows virtual rows, virtual row c * rows + r
 // holding the entries of row r whose column has class c (cold = class `classes`).
 struct HubPlan {
-  int32_t hot = 0, groups = 0, tiers = 0, seg = 0;
+  int32_t hot = 0, groups = 0, tiers = 0, seg = 0, min_degree = 0;
   int32_t classes() const { return groups * tiers; }
   int32_t *vrowptr = nullptr, *colind = nullptr;
   float *val = nullptr;
@@ -626,10 +626,15 @@ struct CsrSide {
 // ---------------------------------------------------------------------------------------------
 // hub plan construction
 // ---------------------------------------------------------------------------------------------
+// only entries of rows with at least min_degree entries can be hot, so only they are counted
 __global__ __launch_bounds__(kSpmmThreads) void col_count_kernel(const int32_t *__restrict__ colind, int64_t nnz,
+                                                                 const int32_t *__restrict__ rowptr,
+                                                                 const int32_t *__restrict__ erow, int32_t min_degree,
                                                                  uint32_t *__restrict__ count) {
   const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
-  if (k < nnz) atomicAdd(&count[colind[k]], 1u);  // integer count: independent of arrival order
+  if (k >= nnz) return;
+  const int32_t r = erow[k];
+  if (rowptr[r + 1] - rowptr[r] >= min_degree) atomicAdd(&count[colind[k]], 1u);  // integer count: order independent
 }
 
 // sort key that orders columns by descending count (ties: ascending column, by stability)
@@ -653,13 +658,20 @@ __global__ __launch_bounds__(kSpmmThreads) void col_class_kernel(const int32_t *
   cls[ranked_col[rank]] = tier < tiers ? (int32_t)(tier * groups + (rank % hot) % groups) : groups * tiers;
 }
 
+// class of an entry: that of its column when its row is long enough, else cold.  A hot entry costs
+// its row a partial row per class (written, then read again by the fold), which only pays when
+// the row has many entries to spread over the classes.
 __global__ __launch_bounds__(kSpmmThreads) void entry_class_kernel(const int32_t *__restrict__ colind, int64_t nnz,
                                                                    const int32_t *__restrict__ cls,
+                                                                   const int32_t *__restrict__ rowptr,
+                                                                   const int32_t *__restrict__ erow,
+                                                                   int32_t min_degree, int32_t cold,
                                                                    int32_t *__restrict__ out,
                                                                    int32_t *__restrict__ pos) {
   const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (k < nnz) {
-    out[k] = cls[colind[k]];
+    const int32_t r = erow[k];
+    out[k] = rowptr[r + 1] - rowptr[r] >= min_degree ? cls[colind[k]] : cold;
     pos[k] = (int32_t)k;  // position in the original CSR, carried through the sort
   }
 }
@@ -687,7 +699,7 @@ __global__ __launch_bounds__(kSpmmThreads) void csr_rows_kernel(const int32_t *_
 }
 
 static int build_hub(CsrSide &s, HubPlan &h, int32_t hot, int32_t groups, int32_t tiers, int32_t seg,
-                     hipStream_t stream) {
+                     int32_t min_degree, hipStream_t stream) {
   CG_HIP(hipStreamSynchronize(stream));
   h.release();
   const int64_t nnz = s.nnz;
@@ -699,13 +711,19 @@ static int build_hub(CsrSide &s, HubPlan &h, int32_t hot, int32_t groups, int32_
   TempFree tmp;
   const unsigned gm = (unsigned)ceil_div64(m, kSpmmThreads), ge = (unsigned)ceil_div64(nnz, kSpmmThreads);
 
-  // 1. reference count of every column, and the columns ranked by it
+  // 1. reference count of every column (over the rows that may have hot entries), and the columns
+  //    ranked by it
   uint32_t *count = nullptr;
-  int32_t *cls = nullptr;
+  int32_t *cls = nullptr, *erow = nullptr;
   CG_TRY(tmp.alloc((void **)&count, (size_t)m * 4));
   CG_TRY(tmp.alloc((void **)&cls, (size_t)m * 4));
+  CG_TRY(tmp.alloc((void **)&erow, (size_t)nnz * 4));
   CG_TRY(fill_u32(count, m, 0u, stream));
-  col_count_kernel<<<ge, kSpmmThreads, 0, stream>>>(s.colind, nnz, count);
+  if (n > 0) {
+    csr_rows_kernel<<<(unsigned)ceil_div64((int64_t)n * kWave, kSpmmThreads), kSpmmThreads, 0, stream>>>(s.rowptr, n, erow);
+    CG_LAUNCH_CHECK();
+  }
+  col_count_kernel<<<ge, kSpmmThreads, 0, stream>>>(s.colind, nnz, s.rowptr, erow, min_degree, count);
   CG_LAUNCH_CHECK();
   {
     SortBuffers buf;
@@ -739,13 +757,10 @@ static int build_hub(CsrSide &s, HubPlan &h, int32_t hot, int32_t groups, int32_
       CG_TRY(tmp2.alloc((void **)&buf.key_b[i], (size_t)nnz * 4));
       CG_TRY(tmp2.alloc((void **)&buf.payload[i], (size_t)nnz * 4));
     }
-    entry_class_kernel<<<ge, kSpmmThreads, 0, stream>>>(s.colind, nnz, cls, buf.key_a[0], buf.payload[0]);
+    entry_class_kernel<<<ge, kSpmmThreads, 0, stream>>>(s.colind, nnz, cls, s.rowptr, erow, min_degree, nclass,
+                                                        buf.key_a[0], buf.payload[0]);
     CG_LAUNCH_CHECK();
-    if (n > 0) {
-      csr_rows_kernel<<<(unsigned)ceil_div64((int64_t)n * kWave, kSpmmThreads), kSpmmThreads, 0, stream>>>(
-          s.rowptr, n, buf.key_b[0]);
-      CG_LAUNCH_CHECK();
-    }
+    CG_HIP(hipMemcpyAsync(buf.key_b[0], erow, (size_t)nnz * 4, hipMemcpyDeviceToDevice, stream));
     int set = 0;
     CG_TRY(radix_sort_pairs(buf, nnz, bits_for(nclass + 1), 0, &set, stream));
     entry_finish_kernel<<<ge, kSpmmThreads, 0, stream>>>(buf.key_a[set], buf.key_b[set], buf.payload[set], nnz, n,
@@ -769,6 +784,7 @@ static int build_hub(CsrSide &s, HubPlan &h, int32_t hot, int32_t groups, int32_
   h.groups = groups;
   h.tiers = tiers;
   h.seg = seg;
+  h.min_degree = min_degree;
   h.valid = true;
   return CG_OK;
 }
@@ -897,6 +913,8 @@ static int spmm_plain(const int32_t *rowptr, const int32_t *colind, const float 
 // Should a product of this width over this matrix go through a hub plan?  It pays when a row of B
 // is two cache lines or more (the gather dominates) and rows hold enough hot entries per group that the
 // partial rows they cost are small against the gathers they turn into L2 hits.
+constexpr int32_t kHubRowDegree = 32;  // rows shorter than this keep all their entries in the cold class
+
 static bool want_hub(int32_t rows, int64_t nnz, int32_t f) {
   const int t = g_tune_hub.load(std::memory_order_relaxed);
   if (t < 0) return false;
@@ -925,10 +943,12 @@ static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream) 
   const int hot_vec = (vec == 4 || f / vec <= kWave) ? vec : 1;
   const SpmmShape hshape = pick_shape(hot_vec, f / hot_vec);
   const int32_t seg = pick_seg(hshape);
+  int32_t min_degree = g_tune_hub_row.load(std::memory_order_relaxed);
+  if (min_degree <= 0) min_degree = kHubRowDegree;
   int slot = -1;
   for (int i = 0; i < CsrSide::kHubPlans; ++i)
     if (s.hub[i].valid && s.hub[i].hot == (int32_t)hot && s.hub[i].groups == groups && s.hub[i].tiers == tiers &&
-        s.hub[i].seg == seg)
+        s.hub[i].seg == seg && s.hub[i].min_degree == min_degree)
       slot = i;
   if (slot < 0) {
     slot = 0;
@@ -939,7 +959,7 @@ static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream) 
       }
       if (s.hub_used[i] < s.hub_used[slot]) slot = i;
     }
-    CG_TRY(build_hub(s, s.hub[slot], (int32_t)hot, groups, tiers, seg, stream));
+    CG_TRY(build_hub(s, s.hub[slot], (int32_t)hot, groups, tiers, seg, min_degree, stream));
   }
   s.hub_used[slot] = ++s.hub_clock;
   HubPlan &h = s.hub[slot];
@@ -1460,6 +1480,7 @@ int cg_tune_set(const char *key, int value) {
   else if (!strcmp(key, "spmm_hub_kb")) cg::g_tune_hub_kb.store(value);
   else if (!strcmp(key, "spmm_hub_groups")) cg::g_tune_hub_groups.store(value);
   else if (!strcmp(key, "spmm_hub_tiers")) cg::g_tune_hub_tiers.store(value);
+  else if (!strcmp(key, "spmm_hub_row")) cg::g_tune_hub_row.store(value);
   else if (!strcmp(key, "dense_mfma")) cg::g_tune_dense_mfma.store(value);
   else if (!strcmp(key, "coo_cache_blocks")) cg::g_tune_coo_cache.store(value);
   else CG_FAIL(CG_ERR_UNSUPPORTED, "cg_tune_set: unknown key %s", key);

@@ -431,6 +431,33 @@ def test_spmm_hub_plan_rectangular_and_all_hot(cuda, tune):
     assert spmm_error(A.spmm(B.to(cuda)), row, col, val, n, m, B) <= REL_TOL
 
 
+@pytest.mark.parametrize("min_degree", [1, 40, 10 ** 6])
+def test_spmm_hub_plan_short_rows_stay_cold(cuda, tune, min_degree):
+    """Only rows with at least `spmm_hub_row` entries get hot entries (and partial rows); the
+    others keep everything in the cold class.  Rows of 0..4 and of ~120 entries, thresholds below
+    all, between the two kinds, and above all (no hot task at all)."""
+    from cagnet_amd import ops
+    n, m, f = 900, 1200, 300
+    gen = torch.Generator().manual_seed(31)
+    dense = torch.rand(n, m, generator=gen)
+    keep = torch.where(torch.arange(n).unsqueeze(1) % 3 == 0, dense < 0.1, dense < 0.002)   # long rows, short rows
+    keep[5] = False                                                                        # and an empty one
+    row, col = keep.nonzero(as_tuple=True)
+    val = torch.randn(row.numel(), generator=gen)
+    B = torch.randn(m, f, generator=gen)
+    C0 = torch.randn(n, f, generator=gen)
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, m)
+    tune("spmm_hub", 1)
+    tune("spmm_hub_kb", 64)
+    tune("spmm_hub_row", min_degree)
+    got = A.spmm(B.to(cuda))
+    assert spmm_error(got, row, col, val, n, m, B) <= REL_TOL
+    assert torch.equal(got[5], torch.zeros(f, device=cuda))
+    C = C0.to(cuda).clone()
+    A.spmm(B.to(cuda), out=C, beta=1.0)
+    assert spmm_error(C, row, col, val, n, m, B, C0) <= REL_TOL
+
+
 def test_spmm_hub_plans_of_several_widths_on_one_handle(cuda, tune):
     """A handle keeps two hub plans (the hot-column count depends on the width); cycling through
     three widths exercises reuse and replacement, and every product stays bit-identical to its
