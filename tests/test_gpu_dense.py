@@ -52,7 +52,8 @@ def test_dense_strided_operands(cuda):
     assert gemm_error(ops.dense_xw(X, W), X.cpu(), W.cpu()) <= REL_TOL
 
 
-@pytest.mark.parametrize("n,c", [(1, 1), (7, 8), (1000, 41), (333, 24), (50, 256), (4097, 16)])
+@pytest.mark.parametrize("n,c", [(1, 1), (7, 8), (1000, 41), (333, 24), (50, 256), (4097, 16), (257, 4), (129, 64),
+                                 (1001, 40), (70001, 24)])
 def test_log_softmax_and_relu(cuda, n, c):
     from cagnet_amd import ops
     z = (_rand((n, c), 9) * 5.0)
@@ -70,7 +71,8 @@ def test_log_softmax_and_relu(cuda, n, c):
     assert torch.equal(ops.relu_bwd(g.to(cuda), h).cpu(), g * (z > 0))
 
 
-@pytest.mark.parametrize("n,c,frac", [(1, 3, 1.0), (1000, 41, 0.66), (5000, 8, 1.0), (70000, 24, 0.3), (300, 5, 0.0)])
+@pytest.mark.parametrize("n,c,frac", [(1, 3, 1.0), (1000, 41, 0.66), (5000, 8, 1.0), (70000, 24, 0.3), (300, 5, 0.0),
+                                      (513, 4, 0.5), (999, 64, 1.0), (2000, 40, 0.7), (300, 16, 0.0)])
 def test_nll_loss_forward_backward(cuda, n, c, frac):
     from cagnet_amd import ops
     gen = torch.Generator().manual_seed(11)
@@ -106,6 +108,30 @@ def test_nll_loss_forward_backward(cuda, n, c, frac):
         zr = z.double().requires_grad_(True)
         (F.nll_loss(F.log_softmax(zr, dim=1)[sel], y[sel]) * 0.5).backward()
         assert float((fused.cpu().double() - zr.grad).abs().max()) <= 1e-6
+
+
+def test_rowwise_kernels_on_views(cuda):
+    """Rows inside a wider buffer: a 16-byte aligned view (leading dimension 32, 24 columns) takes the
+    16-byte form, a view shifted by one float the element form; both must agree with torch."""
+    from cagnet_amd import ops
+    big = (_rand((500, 32), 21) * 3.0).to(cuda)
+    g_big = _rand((500, 32), 22).to(cuda)
+    for lo in (0, 1, 4):
+        z, g = big[:, lo:lo + 24], g_big[:, lo:lo + 24]
+        out = ops.log_softmax_fwd(z)
+        ref = F.log_softmax(z.double(), dim=1)
+        assert float((out.double() - ref).abs().max()) <= 1e-5 * max(1.0, float(ref.abs().max()))
+        dz = ops.log_softmax_bwd(g, out)
+        expect = g.double() - torch.exp(ref) * g.double().sum(dim=1, keepdim=True)
+        scale = g.double().abs().sum(dim=1, keepdim=True)
+        assert float(((dz.double() - expect).abs() / scale).max()) <= REL_TOL
+    # ReLU on an unaligned flat range with a tail that is not a multiple of 4
+    flat = _rand((1, 4099), 23).to(cuda).reshape(-1)
+    for lo in (0, 1):
+        v = flat[lo:lo + 4001]
+        h = ops.relu_fwd(v.reshape(1, -1))
+        assert torch.equal(h.reshape(-1), torch.relu(v))
+        assert torch.equal(ops.relu_bwd(v.reshape(1, -1) * 2, h).reshape(-1), 2 * v * (v > 0))
 
 
 def test_dense_vector_fallback_path(cuda):
