@@ -11,8 +11,6 @@
 // accumulators (64-byte pieces of 16 rows per instruction) and a vector-ALU form (one thread per
 // 4 columns, weights in registers) were both measured slower: the first stalls on the matrix-core
 // results and writes partial lines, the second is bound by its multiply-adds.
-#include <atomic>
-
 #include "common.h"
 
 namespace cg {
@@ -189,12 +187,9 @@ int gwt_rows(const float *G, int64_t ldg, const float *W, int64_t ldw, float *dX
   dim3 grid((unsigned)blocks, (unsigned)chunks);
 #define CG_CASE(F, GV, SV)                                                                                    \
   if (fb == F && gvec == GV && svec == SV) {                                                                  \
-    static std::atomic<bool> raised{false}; /* more than 64 KB of dynamic LDS must be asked for, once */         \
-    if (lds > 64 * 1024 && !raised.load(std::memory_order_acquire)) {                                          \
+    if (lds > 64 * 1024) /* more than 64 KB of dynamic LDS must be asked for (per device, so on every launch) */ \
       CG_HIP(hipFuncSetAttribute((const void *)gwt_mfma_kernel<F, GV, SV>,                                     \
                                  hipFuncAttributeMaxDynamicSharedMemorySize, kGwtLdsBytes));                   \
-      raised.store(true, std::memory_order_release);                                                           \
-    }                                                                                                         \
     gwt_mfma_kernel<F, GV, SV><<<grid, kGwtThreads, lds, stream>>>(G, ldg, W, ldw, dX, lddx, n, k, fo, kc);   \
     CG_LAUNCH_CHECK();                                                                                        \
     return CG_OK;                                                                                             \
