@@ -48,7 +48,7 @@ WORKLOADS = {
 # FETCH_SIZE / WRITE_SIZE runs, reads scaled by 2.0 and writes by 1.0 as calibrated on a 1 GiB copy
 # kernel: profiles/spmm_f602_reddit_counters.txt (131.3 GB read + 4.3 GB written) and
 # profiles/spmm_amazon_counters.txt (291.6 GB read + 17.6 GB written, f = 300).
-MEASURED_TRAFFIC_BYTES = {"reddit": 135.6e9, "amazon": 309.2e9}
+MEASURED_TRAFFIC_BYTES = {"reddit": 134.7e9, "amazon": 309.2e9}
 
 
 def spmm_alg_bytes(nnz: int, n: int, m: int, f: int, reads_c: bool) -> int:
