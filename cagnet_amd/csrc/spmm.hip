@@ -1270,7 +1270,9 @@ struct CooCacheEntry {
 };
 
 static std::mutex g_coo_cache_mu;
-static std::vector<std::shared_ptr<CooCacheEntry>> g_coo_cache;
+// Never destroyed: at process exit the kept blocks are left to the driver, like the scratch buffers;
+// freeing device memory from a static destructor would race the teardown of the HIP runtime.
+static std::vector<std::shared_ptr<CooCacheEntry>> &g_coo_cache = *new std::vector<std::shared_ptr<CooCacheEntry>>();
 static uint64_t g_coo_cache_tick = 0;
 static int64_t g_coo_cache_hits = 0, g_coo_cache_misses = 0, g_coo_cache_evictions = 0;
 

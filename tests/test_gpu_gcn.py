@@ -191,3 +191,51 @@ def test_reordered_forward_matches_reference_order(cuda):
     _close(w1.grad, ref["dw1"], "dw1")
     _close(w2.grad, ref["dw2"], "dw2")
     _close(x.grad, ref["dx"], "dx")
+
+
+def test_forward_backward_replays_in_a_hip_graph(cuda):
+    """After warm-up the library neither allocates, synchronises nor records memset nodes, so the
+    launches of a whole forward + backward pass can be captured into a HIP graph.  Every replay,
+    with eager work and synchronisations between the replays, must reproduce the eager results
+    bit for bit."""
+    from cagnet_amd import ops
+    p = synth.make_problem(scale=13, n_edges=150000, features=128, hidden=16, classes=8, mask_fraction=0.7, seed=3,
+                           device=cuda)
+    blk = ops.CsrMatrix(p.row.int(), p.col.int(), p.val, p.n, p.n, transpose=True)
+    one = torch.ones((), device=cuda)
+
+    def fwd_bwd():
+        z1 = ops.dense_xw(blk.spmm(p.x), p.w1)
+        h = ops.relu_fwd(z1)
+        out = ops.log_softmax_fwd(ops.dense_xw(blk.spmm(h), p.w2))
+        loss, count = ops.nll_loss_fwd(out, p.y, p.train_mask)
+        ag2 = blk.spmm(ops.log_softmax_nll_bwd(out, p.y, p.train_mask, count, one), transpose=True)
+        dw2 = ops.dense_xtg(h, ag2)
+        ag1 = blk.spmm(ops.relu_bwd(ops.dense_gwt(ag2, p.w2), h), transpose=True)
+        return loss, ops.dense_xtg(p.x, ag1), dw2
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):                      # scratch of this stream grows, schedules are built
+            fwd_bwd()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        outs = fwd_bwd()
+    torch.cuda.synchronize()
+    for _ in range(3):
+        for t in outs:
+            t.zero_()
+        eager = fwd_bwd()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(outs, eager):
+            assert torch.equal(got, want)
+    A = orc.coo_tensor(p.row.cpu(), p.col.cpu(), p.val.cpu(), p.n, p.n, torch.float64)
+    ref = orc.forward_backward(p.x.cpu(), p.w1.cpu(), p.w2.cpu(), [A], p.y.cpu(), p.train_mask.cpu(), dtype=torch.float64)
+    assert abs(float(outs[0]) - float(ref["loss"])) <= LOSS_TOL
+    _close(outs[1], ref["dw1"], "dw1 from the graph")
+    _close(outs[2], ref["dw2"], "dw2 from the graph")
