@@ -181,9 +181,11 @@ __global__ __launch_bounds__(kSpmmThreads) void sched_fill_kernel(const int32_t 
 
 __global__ __launch_bounds__(kSpmmThreads) void max_degree_kernel(const int32_t *__restrict__ rowptr, int32_t n,
                                                                   int *__restrict__ out) {
-  const int64_t r = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
-  int32_t deg = 0;
-  if (r < n) deg = rowptr[r + 1] - rowptr[r];
+  int32_t deg = 0;  // grid-stride: a few thousand atomics on the one word, not one per 64 rows
+  for (int64_t r = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x; r < n; r += (int64_t)gridDim.x * kSpmmThreads) {
+    const int32_t d = rowptr[r + 1] - rowptr[r];
+    deg = d > deg ? d : deg;
+  }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     int32_t o = __shfl_xor(deg, off, kWave);
@@ -1157,8 +1159,9 @@ static int side_max_degree(CsrSide &s, hipStream_t stream) {
   CG_TRY(scratch_get(stream, kSlotB, sizeof(int), &d));
   CG_TRY(fill_u32((uint32_t *)d, 1, 0u, stream));
   if (s.rows > 0) {
-    max_degree_kernel<<<(unsigned)ceil_div64(s.rows, kSpmmThreads), kSpmmThreads, 0, stream>>>(s.rowptr, s.rows,
-                                                                                              (int *)d);
+    int64_t blocks = ceil_div64(s.rows, kSpmmThreads);
+    if (blocks > 2048) blocks = 2048;
+    max_degree_kernel<<<(unsigned)blocks, kSpmmThreads, 0, stream>>>(s.rowptr, s.rows, (int *)d);
     CG_LAUNCH_CHECK();
   }
   int v = 0;
