@@ -13,7 +13,11 @@ def _rand(shape, seed):
 
 
 SHAPES = [(1, 1, 1), (5, 3, 2), (1000, 602, 16), (777, 16, 41), (300, 128, 16), (4099, 300, 24), (513, 16, 602),
-          (130, 41, 16), (2000, 64, 100), (50, 700, 70)]
+          (130, 41, 16), (2000, 64, 100), (50, 700, 70),
+          # span tails of X W (whole steps only, whole + ragged, a single ragged step), row counts off the 16-row tiles,
+          # every column-tile count of X^T G, column chunks and all three store widths of G W^T
+          (33, 48, 16), (17, 52, 33), (64, 20, 5), (9, 4, 64), (1500, 320, 48), (700, 1024, 64), (600, 603, 20),
+          (250, 1000, 64), (4100, 65, 8), (1000, 256, 1)]
 
 
 @pytest.mark.parametrize("n,k,fo", SHAPES)
