@@ -264,8 +264,8 @@ int cg_dense_gwt(const float *d_G, int64_t ldg, const float *d_W, int64_t ldw, f
   if (n == 0) return CG_OK;
   GemmArgs g{d_G, ldg, d_W, ldw, d_dX, lddx, n, k, fo, ceil_div64(fo, kKT) * kKT, 1, 0};
   ProfScope prof("dense_gwt", k, (hipStream_t)stream);
-  // wide result: bound by its stores, row-streaming kernel; narrow result: the LDS-tiled vector kernel
-  // (measured faster than a matrix-core form whose stores are 64-byte pieces)
+  // wide result: bound by its stores, matrix-core tiles through an LDS row buffer (dense_rows.hip);
+  // narrow result: the LDS-tiled vector kernel (the matrix-core form measured the same there)
   if (fo <= 64 && k > 64 && g_tune_dense_mfma.load(std::memory_order_relaxed) >= 0)
     return gwt_rows(d_G, ldg, d_W, ldw, d_dX, lddx, n, k, fo, (hipStream_t)stream);
   return launch_gemm<false, true>(g, (hipStream_t)stream);

@@ -11,7 +11,8 @@
 //   xw_mfma  : Z[n, fo]   = X[n, k] * W[k, fo]  (+ReLU)   computed as Z^T = W^T X^T: rows of X on the tile
 //                                                         columns, W staged in LDS
 //   xtg_mfma : dW[k, fo]  = X[n, k]^T * G[n, fo]          columns of X on the tile rows, vertices reduced
-// (dX = G W^T is bound by its stores and runs on the vector ALUs: dense_rows.hip, dense.hip.)
+// (dX = G W^T is bound by its stores: dense_rows.hip for wide results, the vector kernel of dense.hip
+// for narrow ones.)
 #include "common.h"
 
 namespace cg {
