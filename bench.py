@@ -287,6 +287,12 @@ def main() -> int:
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
             "algorithmic_bytes": alg_bytes,
             "avg_launch_ms": round(dom_ms, 5),
+            # the same launch priced on the HBM-side bytes rocprofv3 counted for it (profiles/), not a substitute
+            # for `achieved`: how close the kernel runs to the memory system given the traffic it causes
+            "traffic_gbs": (round(MEASURED_TRAFFIC_BYTES[args.workload] / (dom_ms * 1e-3) / 1e9, 1)
+                            if args.workload in MEASURED_TRAFFIC_BYTES else None),
+            "traffic_frac_of_peak": (round(MEASURED_TRAFFIC_BYTES[args.workload] / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+                                     if args.workload in MEASURED_TRAFFIC_BYTES else None),
         },
     }
     if not args.no_cpu_baseline:
