@@ -1,5 +1,5 @@
 // Device-wide primitives written for 64-wide wavefronts: exclusive scan (reduce-then-scan over
-// 2048-element tiles) and a stable LSD radix sort (8-bit digits, per-wave match ranking in LDS).
+// 2048-element tiles) and a stable LSD radix sort (digits of up to 8 bits, balanced over the passes; per-wave match ranking in LDS).
 // Both are integer-only and order-preserving, so results are run-to-run identical.
 #include "common.h"
 
@@ -125,7 +125,7 @@ constexpr int kRadix = 256;
 
 // hist[digit * tiles + tile] = number of keys of this tile with that digit
 __global__ __launch_bounds__(kSortThreads) void radix_hist_kernel(const int32_t *__restrict__ key, int64_t count,
-                                                                  int shift, uint32_t *__restrict__ hist,
+                                                                  int shift, int dbits, uint32_t *__restrict__ hist,
                                                                   int64_t tiles) {
   __shared__ uint32_t lh[kRadix];
   lh[threadIdx.x] = 0;
@@ -135,12 +135,12 @@ __global__ __launch_bounds__(kSortThreads) void radix_hist_kernel(const int32_t 
   for (int i = 0; i < kSortTile / kSortThreads; ++i) {
     int64_t idx = base + (int64_t)i * kSortThreads + threadIdx.x;
     if (idx < count) {
-      uint32_t d = ((uint32_t)key[idx] >> shift) & (kRadix - 1);
+      uint32_t d = ((uint32_t)key[idx] >> shift) & ((1u << dbits) - 1u);
       atomicAdd(&lh[d], 1u);  // integer LDS atomic: the count does not depend on arrival order
     }
   }
   __syncthreads();
-  hist[(int64_t)threadIdx.x * tiles + blockIdx.x] = lh[threadIdx.x];
+  if ((int)threadIdx.x < (1 << dbits)) hist[(int64_t)threadIdx.x * tiles + blockIdx.x] = lh[threadIdx.x];
 }
 
 // Stable scatter.  Wave w of a workgroup owns keys [tile + 1024 w, tile + 1024 (w+1)) and ranks
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_hist_kernel(const int32_t 
 // are then ordered by digit inside LDS and written out from there, so that the records of one
 // digit leave as one contiguous run instead of one 4-byte store each.
 __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
-    int key_is_a, int shift, const int32_t *__restrict__ in_a, const int32_t *__restrict__ in_b,
+    int key_is_a, int shift, int dbits, const int32_t *__restrict__ in_a, const int32_t *__restrict__ in_b,
     const int32_t *__restrict__ in_p, int32_t *__restrict__ out_a, int32_t *__restrict__ out_b,
     int32_t *__restrict__ out_p, int64_t count, const uint32_t *__restrict__ scanned_hist, int64_t tiles) {
   __shared__ uint32_t cnt[kSortWaves][kRadix];
@@ -164,6 +164,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
   const uint64_t lt_mask = (1ull << lane) - 1ull;
   const int64_t tile_base = (int64_t)blockIdx.x * kSortTile;
   const int64_t base = tile_base + (int64_t)wave * kSortWaveTile;
+  const uint32_t dmask = (1u << dbits) - 1u;
 
   int32_t ra[kSortRounds], rb[kSortRounds], rp[kSortRounds];
   uint32_t packed[kSortRounds];  // digit | rank among the wave's records of that digit << 8
@@ -177,14 +178,16 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
       ra[r] = in_a[idx];
       rb[r] = in_b[idx];
       rp[r] = in_p[idx];
-      d = ((uint32_t)(key_is_a ? ra[r] : rb[r]) >> shift) & (kRadix - 1);
+      d = ((uint32_t)(key_is_a ? ra[r] : rb[r]) >> shift) & dmask;
     }
     uint64_t peers = __ballot(valid);
 #pragma unroll
     for (int bit = 0; bit < 8; ++bit) {
-      const bool one = (d >> bit) & 1u;
-      const uint64_t bal = __ballot(one);
-      peers &= one ? bal : ~bal;
+      if (bit < dbits) {  // wave-uniform
+        const bool one = (d >> bit) & 1u;
+        const uint64_t bal = __ballot(one);
+        peers &= one ? bal : ~bal;
+      }
     }
     const uint32_t rank = (uint32_t)__popcll(peers & lt_mask);
     uint32_t pre = 0;
@@ -214,7 +217,8 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
     __syncthreads();
     uint32_t excl = inc - total;
     for (int w = 0; w < wave; ++w) excl += wave_total[w];
-    goff[t] = scanned_hist[(int64_t)t * tiles + blockIdx.x] - excl;  // modulo 2^32, undone by the addition below
+    // modulo 2^32, undone by the addition below; digits beyond the pass's range have no records
+    goff[t] = t <= (int)dmask ? scanned_hist[(int64_t)t * tiles + blockIdx.x] - excl : 0u;
     uint32_t run = excl;
 #pragma unroll
     for (int w = 0; w < kSortWaves; ++w) {
@@ -241,7 +245,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
   const int32_t here = (int32_t)(left < kSortTile ? left : kSortTile);
   for (int32_t i = threadIdx.x; i < here; i += kSortThreads) {
     const int32_t va = sa[i], vb = sb[i];
-    const uint32_t d = ((uint32_t)(key_is_a ? va : vb) >> shift) & (kRadix - 1);
+    const uint32_t d = ((uint32_t)(key_is_a ? va : vb) >> shift) & dmask;
     const uint32_t pos = goff[d] + (uint32_t)i;
     out_a[pos] = va;
     out_b[pos] = vb;
@@ -261,13 +265,18 @@ int radix_sort_pairs(SortBuffers &buf, int64_t count, int bits_a, int bits_b, in
 
   for (int which = 0; which < 2; ++which) {  // 0: minor key (key_b), 1: major key (key_a)
     const int bits = which == 0 ? bits_b : bits_a;
-    for (int shift = 0; shift < bits; shift += 8) {
+    if (bits <= 0) continue;
+    // balanced digits: the fewest 8-bit passes, each as narrow as that allows (18 bits: 3 x 6), so the
+    // records of one digit leave a tile as longer runs
+    const int passes = (bits + 7) / 8;
+    const int dbits = (bits + passes - 1) / passes;
+    for (int shift = 0; shift < bits; shift += dbits) {
       const int32_t *key = which == 0 ? buf.key_b[cur] : buf.key_a[cur];
-      radix_hist_kernel<<<(unsigned)tiles, kSortThreads, 0, stream>>>(key, count, shift, hist, tiles);
+      radix_hist_kernel<<<(unsigned)tiles, kSortThreads, 0, stream>>>(key, count, shift, dbits, hist, tiles);
       CG_LAUNCH_CHECK();
-      CG_TRY(exclusive_scan_u32(hist, hist, tiles * kRadix, nullptr, stream));
+      CG_TRY(exclusive_scan_u32(hist, hist, tiles << dbits, nullptr, stream));
       radix_scatter_kernel<<<(unsigned)tiles, kSortThreads, 0, stream>>>(
-          which, shift, buf.key_a[cur], buf.key_b[cur], buf.payload[cur], buf.key_a[cur ^ 1], buf.key_b[cur ^ 1],
+          which, shift, dbits, buf.key_a[cur], buf.key_b[cur], buf.payload[cur], buf.key_a[cur ^ 1], buf.key_b[cur ^ 1],
           buf.payload[cur ^ 1], count, hist, tiles);
       CG_LAUNCH_CHECK();
       cur ^= 1;
