@@ -1,5 +1,6 @@
 // Device-wide primitives written for 64-wide wavefronts: exclusive scan (reduce-then-scan over
-// 2048-element tiles) and a stable LSD radix sort (digits of up to 8 bits, balanced over the passes; per-wave match ranking in LDS).
+// 2048-element tiles) and a stable LSD radix sort (digits of up to 8 bits, balanced over the
+// passes; per-wave match ranking in LDS).
 // Both are integer-only and order-preserving, so results are run-to-run identical.
 #include "common.h"
 
