@@ -31,6 +31,11 @@ __global__ __launch_bounds__(kPrepThreads) void prep_degree_kernel(const int32_t
   }
 }
 
+__global__ __launch_bounds__(kPrepThreads) void fill_zero_u32_kernel(uint32_t *__restrict__ p, int64_t count) {
+  const int64_t i = (int64_t)blockIdx.x * kPrepThreads + threadIdx.x;
+  if (i < count) p[i] = 0u;
+}
+
 // dinv[i] = fl32(deg_i ^ -1/2), the power taken in fp64 (gcn_distr.py:440-448); deg == 0 gives +inf
 // like the reference's pow.  The fp64 square root and division are correctly rounded.
 __global__ __launch_bounds__(kPrepThreads) void prep_dinv_kernel(const uint32_t *__restrict__ deg, int32_t n,
@@ -54,111 +59,137 @@ __global__ __launch_bounds__(kPrepThreads) void prep_scale_kernel(const int32_t 
 
 // ---- self-loops ---------------------------------------------------------------------------------
 // Row i of the result = row i of the input without its diagonal entry, plus (i, i), columns
-// ascending.  One wavefront per row.  count[i] = entries of output row i.
-__global__ __launch_bounds__(kPrepThreads) void loops_count_kernel(const int32_t *__restrict__ rowptr,
-                                                                   const int32_t *__restrict__ col, int32_t n,
-                                                                   uint32_t *__restrict__ count) {
-  const int64_t r = ((int64_t)blockIdx.x * kPrepThreads + threadIdx.x) / kWave;
-  const int lane = threadIdx.x & (kWave - 1);
+// ascending.  Per row (one thread, binary search in the ascending columns): below[i] = entries left
+// of the diagonal, diag[i] = 1 if the input holds (i, i); count[i] = entries of output row i.
+__global__ __launch_bounds__(kPrepThreads) void loops_rows_kernel(const int32_t *__restrict__ rowptr,
+                                                                  const int32_t *__restrict__ col, int32_t n,
+                                                                  uint32_t *__restrict__ count,
+                                                                  int32_t *__restrict__ below,
+                                                                  uint8_t *__restrict__ diag) {
+  const int64_t r = (int64_t)blockIdx.x * kPrepThreads + threadIdx.x;
   if (r > n) return;
   if (r == n) {  // the scan runs over n + 1 entries so that entry n receives the total
-    if (lane == 0) count[r] = 0u;
+    count[r] = 0u;
     return;
   }
   const int32_t s = rowptr[r], e = rowptr[r + 1];
-  uint32_t diag = 0;
-  for (int32_t k = s + lane; k < e; k += kWave) diag += col[k] == (int32_t)r ? 1u : 0u;
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) diag += __shfl_xor(diag, off, kWave);
-  if (lane == 0) count[r] = (uint32_t)(e - s) - diag + 1u;
+  int32_t lo = s, hi = e;  // first position whose column is >= r
+  while (lo < hi) {
+    const int32_t mid = lo + (hi - lo) / 2;
+    if (col[mid] < (int32_t)r) lo = mid + 1;
+    else hi = mid;
+  }
+  const bool has = lo < e && col[lo] == (int32_t)r;
+  below[r] = lo - s;
+  diag[r] = has ? 1 : 0;
+  count[r] = (uint32_t)(e - s) - (has ? 1u : 0u) + 1u;
 }
 
-__global__ __launch_bounds__(kPrepThreads) void loops_fill_kernel(const int32_t *__restrict__ rowptr,
-                                                                  const int32_t *__restrict__ col, int32_t n,
-                                                                  const uint32_t *__restrict__ obase,
+// One thread per input entry: entries left of the diagonal keep their rank in the row, the others
+// move by one for the inserted diagonal (and back by one if the input's own diagonal entry, which
+// is dropped here, preceded them).
+__global__ __launch_bounds__(kPrepThreads) void loops_entries_kernel(
+    const int32_t *__restrict__ row, const int32_t *__restrict__ col, int64_t nnz, const int32_t *__restrict__ rowptr,
+    const uint32_t *__restrict__ obase, const uint8_t *__restrict__ diag, int32_t *__restrict__ out_row,
+    int32_t *__restrict__ out_col) {
+  for (int64_t k = (int64_t)blockIdx.x * kPrepThreads + threadIdx.x; k < nnz; k += (int64_t)gridDim.x * kPrepThreads) {
+    const int32_t r = row[k], c = col[k];
+    if (c == r) continue;
+    int64_t pos = (int64_t)obase[r] + (k - rowptr[r]);
+    if (c > r) pos += 1 - (int64_t)diag[r];
+    out_row[pos] = r;
+    out_col[pos] = c;
+  }
+}
+
+__global__ __launch_bounds__(kPrepThreads) void loops_diag_kernel(const uint32_t *__restrict__ obase,
+                                                                  const int32_t *__restrict__ below, int32_t n,
                                                                   int32_t *__restrict__ out_row,
                                                                   int32_t *__restrict__ out_col) {
-  const int64_t r = ((int64_t)blockIdx.x * kPrepThreads + threadIdx.x) / kWave;
-  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t r = (int64_t)blockIdx.x * kPrepThreads + threadIdx.x;
   if (r >= n) return;
-  const int32_t s = rowptr[r], e = rowptr[r + 1];
-  const int64_t o = obase[r];
-  // entries below the diagonal keep their rank, the diagonal follows them, the rest moves by one
-  // (or stays, when the row already held a diagonal entry that is dropped here)
-  uint32_t below = 0;
-  for (int32_t k = s + lane; k < e; k += kWave) below += col[k] < (int32_t)r ? 1u : 0u;
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) below += __shfl_xor(below, off, kWave);
-  if (lane == 0) {
-    out_row[o + below] = (int32_t)r;
-    out_col[o + below] = (int32_t)r;
-  }
-  // ranks among the entries above the diagonal: columns ascend, so the input position gives them
-  uint32_t skipped = 0;  // diagonal entries of the input met so far
-  for (int32_t base = s; base < e; base += kWave) {
-    const int32_t k = base + lane;
-    const int32_t c = k < e ? col[k] : -1;
-    const bool is_diag = k < e && c == (int32_t)r;
-    const uint64_t dmask = __ballot(is_diag);
-    const uint32_t before = skipped + (uint32_t)__popcll(dmask & ((1ull << lane) - 1ull));
-    if (k < e && !is_diag) {
-      const int64_t pos = c < (int32_t)r ? (int64_t)(k - s) - before : (int64_t)(k - s) - before + 1;
-      out_row[o + pos] = (int32_t)r;
-      out_col[o + pos] = c;
-    }
-    skipped += (uint32_t)__popcll(dmask);
-  }
+  const int64_t pos = (int64_t)obase[r] + below[r];
+  out_row[pos] = (int32_t)r;
+  out_col[pos] = (int32_t)r;
 }
 
 // ---- block extraction ---------------------------------------------------------------------------
-__global__ __launch_bounds__(kPrepThreads) void block_flag_kernel(const int32_t *__restrict__ row,
-                                                                  const int32_t *__restrict__ col, int64_t nnz,
-                                                                  int32_t r0, int32_t r1, int32_t c0, int32_t c1,
-                                                                  uint32_t *__restrict__ flag) {
-  const int64_t k = (int64_t)blockIdx.x * kPrepThreads + threadIdx.x;
-  if (k > nnz) return;
-  if (k == nnz) {
-    flag[k] = 0u;
+// Order-preserving compaction in tiles of kBlockTile entries: a count per tile, an exclusive scan of
+// the tile counts, then every tile ranks its own matches (wave ballots, running counts) and writes
+// them behind its base.  Wave w of a workgroup owns entries [tile + 1024 w, tile + 1024 (w + 1)).
+constexpr int kBlockRounds = 16;
+constexpr int kBlockWaveTile = kBlockRounds * kWave;
+constexpr int kBlockTile = (kPrepThreads / kWave) * kBlockWaveTile;  // 4096
+
+__device__ __forceinline__ bool in_block(int32_t r, int32_t c, int32_t r0, int32_t r1, int32_t c0, int32_t c1) {
+  return r >= r0 && r < r1 && c >= c0 && c < c1;
+}
+
+__global__ __launch_bounds__(kPrepThreads) void block_count_kernel(const int32_t *__restrict__ row,
+                                                                   const int32_t *__restrict__ col, int64_t nnz,
+                                                                   int32_t r0, int32_t r1, int32_t c0, int32_t c1,
+                                                                   int64_t tiles, uint32_t *__restrict__ tile_count) {
+  __shared__ uint32_t wsum[kPrepThreads / kWave];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  if ((int64_t)blockIdx.x == tiles) {  // the scan runs over tiles + 1 entries so that the last receives the total
+    if (threadIdx.x == 0) tile_count[tiles] = 0u;
     return;
   }
-  const int32_t r = row[k], c = col[k];
-  flag[k] = (r >= r0 && r < r1 && c >= c0 && c < c1) ? 1u : 0u;
+  const int64_t base = (int64_t)blockIdx.x * kBlockTile + (int64_t)wave * kBlockWaveTile;
+  uint32_t cnt = 0;
+#pragma unroll
+  for (int i = 0; i < kBlockRounds; ++i) {
+    const int64_t k = base + (int64_t)i * kWave + lane;
+    const bool hit = k < nnz && in_block(row[k < nnz ? k : 0], col[k < nnz ? k : 0], r0, r1, c0, c1);
+    cnt += (uint32_t)__popcll(__ballot(hit));
+  }
+  if (lane == 0) wsum[wave] = cnt;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t t = 0;
+    for (int w = 0; w < kPrepThreads / kWave; ++w) t += wsum[w];
+    tile_count[blockIdx.x] = t;
+  }
 }
 
-__global__ __launch_bounds__(kPrepThreads) void block_scatter_kernel(
+__global__ __launch_bounds__(kPrepThreads) void block_compact_kernel(
     const int32_t *__restrict__ row, const int32_t *__restrict__ col, const float *__restrict__ val, int64_t nnz,
-    int32_t r0, int32_t r1, int32_t c0, int32_t c1, const uint32_t *__restrict__ pos, int64_t capacity,
+    int32_t r0, int32_t r1, int32_t c0, int32_t c1, const uint32_t *__restrict__ tile_base, int64_t capacity,
     int32_t *__restrict__ out_row, int32_t *__restrict__ out_col, float *__restrict__ out_val) {
-  const int64_t k = (int64_t)blockIdx.x * kPrepThreads + threadIdx.x;
-  if (k >= nnz) return;
-  const int32_t r = row[k], c = col[k];
-  if (!(r >= r0 && r < r1 && c >= c0 && c < c1)) return;
-  const int64_t o = pos[k];
-  if (o >= capacity) return;
-  out_row[o] = r - r0;  // rebased like split_coo (gcn_distr.py:406)
-  out_col[o] = c - c0;
-  if (val) out_val[o] = val[k];
-}
-
-struct PrepTemp {
-  void *p[4] = {nullptr, nullptr, nullptr, nullptr};
-  int count = 0;
-  ~PrepTemp() {
-    for (int i = 0; i < count; ++i)
-      if (p[i]) (void)hipFree(p[i]);
+  __shared__ uint32_t wsum[kPrepThreads / kWave];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const uint64_t lower = (1ull << lane) - 1ull;
+  const int64_t base = (int64_t)blockIdx.x * kBlockTile + (int64_t)wave * kBlockWaveTile;
+  int32_t rr[kBlockRounds], cc[kBlockRounds];
+  uint32_t rank[kBlockRounds];  // rank of a match among the wave's matches; ~0u: not in the block
+  uint32_t cnt = 0;
+#pragma unroll
+  for (int i = 0; i < kBlockRounds; ++i) {
+    const int64_t k = base + (int64_t)i * kWave + lane;
+    const int64_t kc = k < nnz ? k : 0;
+    rr[i] = row[kc];
+    cc[i] = col[kc];
+    const bool hit = k < nnz && in_block(rr[i], cc[i], r0, r1, c0, c1);
+    const uint64_t bal = __ballot(hit);
+    rank[i] = hit ? cnt + (uint32_t)__popcll(bal & lower) : ~0u;
+    cnt += (uint32_t)__popcll(bal);
   }
-  int alloc(void **out, size_t bytes) {
-    hipError_t e = hipMalloc(out, bytes ? bytes : 4);
-    if (e != hipSuccess) {
-      (void)hipGetLastError();
-      *out = nullptr;
-      set_error("hipMalloc of %zu bytes failed: %s", bytes, hipGetErrorString(e));
-      return CG_ERR_ALLOC;
+  if (lane == 0) wsum[wave] = cnt;
+  __syncthreads();
+  int64_t o = tile_base[blockIdx.x];
+  for (int w = 0; w < wave; ++w) o += wsum[w];
+#pragma unroll
+  for (int i = 0; i < kBlockRounds; ++i) {
+    if (rank[i] != ~0u) {
+      const int64_t pos = o + rank[i];
+      if (pos < capacity) {
+        out_row[pos] = rr[i] - r0;  // rebased like split_coo (gcn_distr.py:406)
+        out_col[pos] = cc[i] - c0;
+        if (val) out_val[pos] = val[base + (int64_t)i * kWave + lane];
+      }
     }
-    p[count++] = *out;
-    return CG_OK;
   }
-};
+}
 
 static unsigned grid_for(int64_t count) { return (unsigned)ceil_div64(count > 0 ? count : 1, kPrepThreads); }
 
@@ -174,19 +205,19 @@ int cg_gcn_normalize(const int32_t *d_row, const int32_t *d_col, int64_t nnz, in
   if (nnz > 0x7fffffffLL - 1) CG_FAIL(CG_ERR_OVERFLOW, "cg_gcn_normalize: nnz=%lld exceeds int32", (long long)nnz);
   if (nnz > 0 && (!d_row || !d_col || !d_val)) CG_FAIL(CG_ERR_NULL, "cg_gcn_normalize: null operand");
   if (n == 0 || nnz == 0) return CG_OK;
-  PrepTemp tmp;
-  uint32_t *deg = nullptr;
-  float *dinv = d_dinv;
-  CG_TRY(tmp.alloc((void **)&deg, (size_t)n * sizeof(uint32_t)));
-  if (!dinv) CG_TRY(tmp.alloc((void **)&dinv, (size_t)n * sizeof(float)));
-  CG_HIP(hipMemsetAsync(deg, 0, (size_t)n * sizeof(uint32_t), stream));
+  // degrees and their inverse roots live in the stream's scratch: no allocation, no synchronisation
+  void *p = nullptr;
+  CG_TRY(scratch_get(stream, kSlotB, (size_t)n * (sizeof(uint32_t) + sizeof(float)), &p));
+  uint32_t *deg = (uint32_t *)p;
+  float *dinv = d_dinv ? d_dinv : (float *)(deg + n);
+  fill_zero_u32_kernel<<<grid_for(n), kPrepThreads, 0, stream>>>(deg, n);
+  CG_LAUNCH_CHECK();
   prep_degree_kernel<<<grid_for(nnz), kPrepThreads, 0, stream>>>(d_row, nnz, n, deg);
   CG_LAUNCH_CHECK();
   prep_dinv_kernel<<<grid_for(n), kPrepThreads, 0, stream>>>(deg, n, dinv);
   CG_LAUNCH_CHECK();
   prep_scale_kernel<<<grid_for(nnz), kPrepThreads, 0, stream>>>(d_row, d_col, nnz, n, dinv, d_val);
   CG_LAUNCH_CHECK();
-  CG_HIP(hipStreamSynchronize(stream));  // the temporaries are freed on return
   return CG_OK;
 }
 
@@ -205,15 +236,14 @@ int cg_add_self_loops(const int32_t *d_row, const int32_t *d_col, int64_t nnz, i
     return CG_OK;
   }
   CG_TRY(coo_check(d_row, d_col, nnz, n, n, 2, stream));  // the ranks below rely on (row, col) order
-  PrepTemp tmp;
-  int32_t *rowptr = nullptr;
-  uint32_t *obase = nullptr, *d_total = nullptr;
-  CG_TRY(tmp.alloc((void **)&rowptr, (size_t)(n + 1) * sizeof(int32_t)));
-  CG_TRY(tmp.alloc((void **)&obase, (size_t)(n + 2) * sizeof(uint32_t)));
-  d_total = obase + n + 1;
+  // per-row tables in the stream's scratch: rowptr[n+1], below[n], obase[n+2], diag[n]
+  void *p = nullptr;
+  CG_TRY(scratch_get(stream, kSlotB, (size_t)(3 * (int64_t)n + 3) * sizeof(int32_t) + (size_t)n, &p));
+  int32_t *rowptr = (int32_t *)p, *below = rowptr + n + 1;
+  uint32_t *obase = (uint32_t *)(below + n), *d_total = obase + n + 1;
+  uint8_t *diag = (uint8_t *)(obase + n + 2);
   CG_TRY(launch_rowptr(d_row, nnz, n, rowptr, stream));
-  const unsigned wgrid = grid_for(((int64_t)n + 1) * kWave);
-  loops_count_kernel<<<wgrid, kPrepThreads, 0, stream>>>(rowptr, d_col, n, obase);
+  loops_rows_kernel<<<grid_for((int64_t)n + 1), kPrepThreads, 0, stream>>>(rowptr, d_col, n, obase, below, diag);
   CG_LAUNCH_CHECK();
   CG_TRY(exclusive_scan_u32(obase, obase, (int64_t)n + 1, d_total, stream));
   uint32_t total = 0;
@@ -224,7 +254,14 @@ int cg_add_self_loops(const int32_t *d_row, const int32_t *d_col, int64_t nnz, i
   if ((int64_t)total > capacity)
     CG_FAIL(CG_ERR_SIZE, "cg_add_self_loops: result has %u entries, capacity is %lld", total, (long long)capacity);
   if (!d_out_row || !d_out_col) CG_FAIL(CG_ERR_NULL, "cg_add_self_loops: null output");
-  loops_fill_kernel<<<wgrid, kPrepThreads, 0, stream>>>(rowptr, d_col, n, obase, d_out_row, d_out_col);
+  if (nnz > 0) {
+    int64_t blocks = ceil_div64(nnz, kPrepThreads);
+    if (blocks > 256 * 64) blocks = 256 * 64;
+    loops_entries_kernel<<<(unsigned)blocks, kPrepThreads, 0, stream>>>(d_row, d_col, nnz, rowptr, obase, diag,
+                                                                        d_out_row, d_out_col);
+    CG_LAUNCH_CHECK();
+  }
+  loops_diag_kernel<<<grid_for(n), kPrepThreads, 0, stream>>>(obase, below, n, d_out_row, d_out_col);
   CG_LAUNCH_CHECK();
   CG_HIP(hipStreamSynchronize(stream));
   return CG_OK;
@@ -242,13 +279,15 @@ int cg_coo_block(const int32_t *d_row, const int32_t *d_col, const float *d_val,
   if (nnz > 0 && (!d_row || !d_col)) CG_FAIL(CG_ERR_NULL, "cg_coo_block: null operand");
   *out_nnz = 0;
   if (nnz == 0) return CG_OK;
-  PrepTemp tmp;
-  uint32_t *flag = nullptr;
-  CG_TRY(tmp.alloc((void **)&flag, (size_t)(nnz + 2) * sizeof(uint32_t)));
-  uint32_t *d_total = flag + nnz + 1;
-  block_flag_kernel<<<grid_for(nnz + 1), kPrepThreads, 0, stream>>>(d_row, d_col, nnz, r0, r1, c0, c1, flag);
+  // tile counts live in the stream's scratch: the call allocates nothing
+  const int64_t tiles = ceil_div64(nnz, kBlockTile);
+  void *p = nullptr;
+  CG_TRY(scratch_get(stream, kSlotB, (size_t)(tiles + 2) * sizeof(uint32_t), &p));
+  uint32_t *tile_count = (uint32_t *)p, *d_total = tile_count + tiles + 1;
+  block_count_kernel<<<(unsigned)(tiles + 1), kPrepThreads, 0, stream>>>(d_row, d_col, nnz, r0, r1, c0, c1, tiles,
+                                                                      tile_count);
   CG_LAUNCH_CHECK();
-  CG_TRY(exclusive_scan_u32(flag, flag, nnz + 1, d_total, stream));
+  CG_TRY(exclusive_scan_u32(tile_count, tile_count, tiles + 1, d_total, stream));
   uint32_t total = 0;
   CG_HIP(hipMemcpyAsync(&total, d_total, sizeof(total), hipMemcpyDeviceToHost, stream));
   CG_HIP(hipStreamSynchronize(stream));
@@ -257,8 +296,9 @@ int cg_coo_block(const int32_t *d_row, const int32_t *d_col, const float *d_val,
   if ((int64_t)total > capacity)
     CG_FAIL(CG_ERR_SIZE, "cg_coo_block: block has %u entries, capacity is %lld", total, (long long)capacity);
   if (!d_out_row || !d_out_col || (d_val && !d_out_val)) CG_FAIL(CG_ERR_NULL, "cg_coo_block: null output");
-  block_scatter_kernel<<<grid_for(nnz), kPrepThreads, 0, stream>>>(d_row, d_col, d_val, nnz, r0, r1, c0, c1, flag,
-                                                                  capacity, d_out_row, d_out_col, d_out_val);
+  block_compact_kernel<<<(unsigned)tiles, kPrepThreads, 0, stream>>>(d_row, d_col, d_val, nnz, r0, r1, c0, c1,
+                                                                    tile_count, capacity, d_out_row, d_out_col,
+                                                                    d_out_val);
   CG_LAUNCH_CHECK();
   CG_HIP(hipStreamSynchronize(stream));
   return CG_OK;

@@ -230,8 +230,9 @@ int cg_csr_blob_read(cg_csr_t **out, const void *host_buf, int64_t bytes, uint32
  * Input preparation on the device.  The reference prepares its adjacency matrix on the host:
  * add_remaining_self_loops (gcn_distr.py:791), scale_elements (gcn_distr.py:412-470) and
  * split_coo (gcn_distr.py:398-409).  These three entry points do the same work on int32 COO
- * arrays that are already in device memory.  All three allocate temporaries and synchronise
- * `stream` before they return.
+ * arrays that are already in device memory.  Temporaries come from the scratch memory the library
+ * keeps per (device, stream).  cg_add_self_loops and cg_coo_block return a count, so they
+ * synchronise `stream`; cg_gcn_normalize is stream ordered and does not.
  *
  * cg_add_self_loops: (row, col) strictly ascending COO of an n x n pattern -> the same pattern
  * with every diagonal entry present exactly once, still ascending.  *out_nnz receives the size of
