@@ -12,6 +12,7 @@ from tests.util import REL_TOL
 
 pytestmark = pytest.mark.gpu
 
+
 @pytest.fixture(autouse=True)
 def _release_device_memory():
     """These tests hold tens of GB; hand the cached blocks back so later tests and the library's own
