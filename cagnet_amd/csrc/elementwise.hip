@@ -356,6 +356,7 @@ int cg_relu_fwd(const float *d_z, float *d_h, int64_t count, cg_stream_t stream)
   if (count < 0) CG_FAIL(CG_ERR_SIZE, "cg_relu_fwd: negative count");
   if (count == 0) return CG_OK;
   if (!d_z || !d_h) CG_FAIL(CG_ERR_NULL, "cg_relu_fwd: null pointer");
+  ProfScope prof("relu_fwd", -1, (hipStream_t)stream);
   if (aligned16(d_z, d_h))
     relu_fwd_vec_kernel<<<vec_grid(count / 4), kEwThreads, 0, (hipStream_t)stream>>>(d_z, d_h, count);
   else
@@ -369,6 +370,7 @@ int cg_relu_bwd(const float *d_g, const float *d_h, float *d_dz, int64_t count, 
   if (count < 0) CG_FAIL(CG_ERR_SIZE, "cg_relu_bwd: negative count");
   if (count == 0) return CG_OK;
   if (!d_g || !d_h || !d_dz) CG_FAIL(CG_ERR_NULL, "cg_relu_bwd: null pointer");
+  ProfScope prof("relu_bwd", -1, (hipStream_t)stream);
   if (aligned16(d_g, d_h, d_dz))
     relu_bwd_vec_kernel<<<vec_grid(count / 4), kEwThreads, 0, (hipStream_t)stream>>>(d_g, d_h, d_dz, count);
   else
@@ -386,6 +388,7 @@ int cg_log_softmax_fwd(const float *d_z, int64_t ldz, float *d_out, int64_t ldo,
   if (!d_z || !d_out) CG_FAIL(CG_ERR_NULL, "cg_log_softmax_fwd: null pointer");
   if (ldz < c || ldo < c) CG_FAIL(CG_ERR_SIZE, "cg_log_softmax_fwd: leading dimension smaller than c");
   hipStream_t s = (hipStream_t)stream;
+  ProfScope prof("log_softmax_fwd", c, s);
   switch (vec_team(c, ldz, ldo, 4, d_z, d_out, nullptr)) {
 #define CG_CASE(T)                                                                                        \
   case T:                                                                                                 \
@@ -408,6 +411,7 @@ int cg_log_softmax_bwd(const float *d_g, int64_t ldg, const float *d_out, int64_
   if (!d_g || !d_out || !d_dz) CG_FAIL(CG_ERR_NULL, "cg_log_softmax_bwd: null pointer");
   if (ldg < c || ldo < c || lddz < c) CG_FAIL(CG_ERR_SIZE, "cg_log_softmax_bwd: leading dimension smaller than c");
   hipStream_t s = (hipStream_t)stream;
+  ProfScope prof("log_softmax_bwd", c, s);
   switch (vec_team(c, ldg, ldo, lddz, d_g, d_out, d_dz)) {
 #define CG_CASE(T)                                                                                              \
   case T:                                                                                                       \
@@ -436,6 +440,7 @@ int cg_nll_loss_fwd(const float *d_logp, int64_t ld, const int64_t *d_y, const u
   CG_TRY(scratch_get(stream, kSlotB, (size_t)(parts + 1) * (sizeof(float) + sizeof(int64_t)) + 16, &p));
   int64_t *pcnt = (int64_t *)p;                 // 8-byte aligned part first
   float *psum = (float *)(pcnt + parts + 1);
+  ProfScope prof("nll_fwd", c, stream);
   if (parts > 0) {
     nll_partial_kernel<<<(unsigned)parts, kEwThreads, 0, stream>>>(d_logp, ld, d_y, d_mask, n, c, psum, pcnt);
     CG_LAUNCH_CHECK();
@@ -453,6 +458,7 @@ int cg_nll_loss_bwd(const int64_t *d_y, const uint8_t *d_mask, const int64_t *d_
   if (!d_y || !d_count || !d_dlogp) CG_FAIL(CG_ERR_NULL, "cg_nll_loss_bwd: null pointer");
   if (ld < c) CG_FAIL(CG_ERR_SIZE, "cg_nll_loss_bwd: leading dimension smaller than c");
   hipStream_t s = (hipStream_t)stream;
+  ProfScope prof("nll_bwd", c, s);
   switch (vec_team(c, ld, 4, 4, d_dlogp, nullptr, nullptr)) {
 #define CG_CASE(T)                                                                                                \
   case T:                                                                                                         \
@@ -478,6 +484,7 @@ int cg_log_softmax_nll_bwd(const float *d_logp, int64_t ld, const int64_t *d_y, 
   if (!d_logp || !d_y || !d_count || !d_dz) CG_FAIL(CG_ERR_NULL, "cg_log_softmax_nll_bwd: null pointer");
   if (ld < c || lddz < c) CG_FAIL(CG_ERR_SIZE, "cg_log_softmax_nll_bwd: leading dimension smaller than c");
   hipStream_t s = (hipStream_t)stream;
+  ProfScope prof("log_softmax_nll_bwd", c, s);
   switch (vec_team(c, ld, lddz, 4, d_logp, d_dz, nullptr)) {
 #define CG_CASE(T)                                                                                               \
   case T:                                                                                                        \
