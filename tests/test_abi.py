@@ -106,6 +106,8 @@ def test_status_codes_without_a_gpu():
     assert lib.cg_csr_blob_size(null, ctypes.byref(count)) == E["null"]
     assert lib.cg_tune_set(b"no_such_knob", 1) == E["unsupported"]
     assert lib.cg_tune_set(b"spmm_seg", 0) == 0
+    for key in (b"spmm_hub_row", b"coo_cache_blocks", b"dense_mfma"):
+        assert lib.cg_tune_set(key, 0) == 0
     for code in range(0, 11):
         assert lib.cg_status_string(code) not in (None, b"unknown status")
     assert lib.cg_status_string(99) == b"unknown status"
@@ -127,3 +129,5 @@ def test_python_surface_rejects_cpu_tensors_and_wrong_types():
     assert t.is_sparse and t.shape == (2, 2) and float(t.to_dense()[0, 1]) == 1.0
     import sparse_coo_tensor_cpp as shim  # the reference's module name resolves from the repo root
     assert shim.spmm_gpu is spmm_gpu
+    from cagnet_amd import sparse_coo_tensor_cpp as mod
+    assert mod.cache_blocks is True      # blocks seen before are recognised by default
