@@ -29,6 +29,9 @@ struct SpmmShape {
   int vec, lpr, chunks;
 };
 
+constexpr int kMaxHubClasses = 64;  // column classes of a hub plan (XCD groups x tiers)
+constexpr int kHubAutoTiers = 6;    // most tiers the automatic choice takes
+constexpr double kHubTierEntriesPerPair = 2.4;  // entries per (class, row) pair below which a tier no longer pays
 constexpr int kMaxChunks = 10;  // full-wave teams cover up to 64 * kMaxChunks * VEC columns per launch
 
 // Widest vector the operands allow.
@@ -308,7 +311,7 @@ struct StreamTab {
   int32_t *task_start = nullptr, *task_dst = nullptr, *wstart = nullptr;
   int64_t nwin = 0;            // exact, or the grid bound of an asynchronous build
   uint32_t *d_nwin = nullptr;  // exact count on the device (asynchronous builds only)
-  int64_t win_first[18] = {0};
+  int64_t win_first[kMaxHubClasses + 2] = {0};
   void release() {
     if (owned) {
       if (task_start) (void)hipFree(task_start);
@@ -455,7 +458,7 @@ static int build_stream(const Sched &sc, const int32_t *rowptr, int32_t nrows, b
     return CG_OK;
   }
   // entry extents of the classes (the host needs them to size the boundary launches)
-  int32_t ends[18];
+  int32_t ends[kMaxHubClasses + 2];
   for (int g = 0; g <= nclass; ++g)
     CG_HIP(hipMemcpyAsync(&ends[g], out.task_start + class_first[g], 4, hipMemcpyDeviceToHost, stream));
   CG_HIP(hipStreamSynchronize(stream));
@@ -475,7 +478,7 @@ static int build_stream(const Sched &sc, const int32_t *rowptr, int32_t nrows, b
   CG_TRY(exclusive_scan_u32(flags, index, nt + 1, d_total, stream));
   uint32_t nwin = 0;
   CG_HIP(hipMemcpyAsync(&nwin, d_total, 4, hipMemcpyDeviceToHost, stream));
-  uint32_t firsts[18] = {0};
+  uint32_t firsts[kMaxHubClasses + 2] = {0};
   for (int g = 0; g < nclass; ++g)
     CG_HIP(hipMemcpyAsync(&firsts[g], index + class_first[g], 4, hipMemcpyDeviceToHost, stream));
   CG_HIP(hipStreamSynchronize(stream));
@@ -580,13 +583,14 @@ struct SchedCache {
 // holding the entries of row r whose column has class c (cold = class `classes`).
 struct HubPlan {
   int32_t hot = 0, groups = 0, tiers = 0, seg = 0, min_degree = 0;
+  int32_t req_hot = 0, req_tiers = 0, req_single = 0;  // what was asked for (tiers 0: chosen from the column counts)
   int32_t classes() const { return groups * tiers; }
   int32_t *vrowptr = nullptr, *colind = nullptr;
   float *val = nullptr;
   Sched hot_sched;        // over the virtual rows of the hot classes, empty rows skipped
   StreamTab hot_tab;      // its windows, one class per (tier, group)
   SchedCache cold_sched;  // over the cold class
-  int64_t tstart[18] = {0};
+  int64_t tstart[kMaxHubClasses + 2] = {0};
   bool valid = false;
   void release() {
     hot_sched.release();
@@ -650,6 +654,28 @@ __global__ __launch_bounds__(kSpmmThreads) void col_key_kernel(const uint32_t *_
   }
 }
 
+// sums[t] = entries whose column has rank [t * hot, (t + 1) * hot): one workgroup per tier.  The keys
+// are maxcount - count in ascending order.
+__global__ __launch_bounds__(kSpmmThreads) void tier_sum_kernel(const int32_t *__restrict__ sorted_key, int32_t m,
+                                                                uint32_t maxcount, int32_t hot,
+                                                                unsigned long long *__restrict__ sums) {
+  __shared__ unsigned long long part[kSpmmThreads / kWave];
+  const int64_t lo = (int64_t)blockIdx.x * hot;
+  int64_t hi = lo + hot;
+  if (hi > m) hi = m;
+  unsigned long long v = 0;
+  for (int64_t r = lo + threadIdx.x; r < hi; r += kSpmmThreads) v += (unsigned long long)(maxcount - (uint32_t)sorted_key[r]);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  if ((threadIdx.x & (kWave - 1)) == 0) part[threadIdx.x / kWave] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned long long t = 0;
+    for (int w = 0; w < kSpmmThreads / kWave; ++w) t += part[w];
+    sums[blockIdx.x] = t;
+  }
+}
+
 // class of every column from its rank: `hot` ranks per tier, dealt round robin to the groups
 __global__ __launch_bounds__(kSpmmThreads) void col_class_kernel(const int32_t *__restrict__ ranked_col, int32_t m,
                                                                  int32_t hot, int32_t groups, int32_t tiers,
@@ -700,16 +726,20 @@ __global__ __launch_bounds__(kSpmmThreads) void csr_rows_kernel(const int32_t *_
   for (int32_t k = s + lane; k < e; k += kWave) row_out[k] = (int32_t)wave;
 }
 
-static int build_hub(CsrSide &s, HubPlan &h, int32_t hot, int32_t groups, int32_t tiers, int32_t seg,
-                     int32_t min_degree, hipStream_t stream) {
+// tiers == 0: the number of tiers is chosen from the column counts (tiers of `hot` columns each); if
+// one tier comes out, it holds `hot_single` columns.
+static int build_hub(CsrSide &s, HubPlan &h, int32_t hot, int32_t hot_single, int32_t groups, int32_t tiers,
+                     int32_t seg, int32_t min_degree, hipStream_t stream) {
   CG_HIP(hipStreamSynchronize(stream));
   h.release();
+  h.req_hot = hot;
+  h.req_tiers = tiers;
+  h.req_single = hot_single;
   const int64_t nnz = s.nnz;
   const int32_t n = s.rows, m = s.cols;
-  const int32_t nclass = groups * tiers;
-  const int64_t vrows = (int64_t)(nclass + 1) * n;
   if (hot < 1) hot = 1;
-  if (vrows + 1 > 0x7fffffffLL) CG_FAIL(CG_ERR_OVERFLOW, "hub plan: %lld virtual rows exceed int32", (long long)vrows);
+  if (hot_single < 1) hot_single = 1;
+  if ((int64_t)(kMaxHubClasses + 1) * n + 1 > 0x7fffffffLL && tiers == 0) tiers = 1;  // keep the virtual rows in int32
   TempFree tmp;
   const unsigned gm = (unsigned)ceil_div64(m, kSpmmThreads), ge = (unsigned)ceil_div64(nnz, kSpmmThreads);
 
@@ -741,9 +771,27 @@ static int build_hub(CsrSide &s, HubPlan &h, int32_t hot, int32_t groups, int32_
     int set = 0;
     CG_TRY(radix_sort_pairs(buf, m, bits_for((int32_t)(maxcount < 0x7ffffffeu ? maxcount + 1 : 0x7fffffff)), 0, &set,
                             stream));
+    if (tiers == 0) {
+      // A further tier serves its entries from L2 instead of HBM but costs every (class, row) pair it
+      // touches a partial row, written and read again: it pays while it holds well over two
+      // entries per pair it can have (measured break-even 2.4: f = 602 takes 4 tiers, 300 two, 128 one).
+      const int max_tiers = kMaxHubClasses / groups < kHubAutoTiers ? kMaxHubClasses / groups : kHubAutoTiers;
+      unsigned long long *d_sums = nullptr, sums[kHubAutoTiers] = {0};
+      CG_TRY(tmp.alloc((void **)&d_sums, sizeof(sums)));
+      tier_sum_kernel<<<max_tiers, kSpmmThreads, 0, stream>>>(buf.key_a[set], m, maxcount, hot, d_sums);
+      CG_LAUNCH_CHECK();
+      CG_HIP(hipMemcpyAsync(sums, d_sums, sizeof(unsigned long long) * max_tiers, hipMemcpyDeviceToHost, stream));
+      CG_HIP(hipStreamSynchronize(stream));
+      tiers = 1;
+      while (tiers < max_tiers && (double)sums[tiers] >= kHubTierEntriesPerPair * (double)groups * (double)n) ++tiers;
+      if (tiers == 1) hot = hot_single;
+    }
     col_class_kernel<<<gm, kSpmmThreads, 0, stream>>>(buf.payload[set], m, hot, groups, tiers, cls);
     CG_LAUNCH_CHECK();
   }
+  const int32_t nclass = groups * tiers;
+  const int64_t vrows = (int64_t)(nclass + 1) * n;
+  if (vrows + 1 > 0x7fffffffLL) CG_FAIL(CG_ERR_OVERFLOW, "hub plan: %lld virtual rows exceed int32", (long long)vrows);
 
   // 2. stable regrouping of the entries by class: (row, col) order is kept inside a class
   CG_TRY(dev_alloc((void **)&h.colind, (size_t)nnz * 4));
@@ -776,7 +824,7 @@ static int build_hub(CsrSide &s, HubPlan &h, int32_t hot, int32_t groups, int32_
   Alloc owned;
   CG_TRY(make_sched(h.vrowptr, nclass * n, seg, 1, h.hot_sched, owned, false, 0, 0, stream));
   {
-    int32_t t[18];
+    int32_t t[kMaxHubClasses + 2];
     for (int g = 0; g <= nclass; ++g)
       CG_HIP(hipMemcpyAsync(&t[g], h.hot_sched.tbase + (int64_t)g * n, 4, hipMemcpyDeviceToHost, stream));
     CG_HIP(hipStreamSynchronize(stream));
@@ -915,7 +963,7 @@ static int spmm_plain(const int32_t *rowptr, const int32_t *colind, const float 
 // Should a product of this width over this matrix go through a hub plan?  It pays when a row of B
 // is two cache lines or more (the gather dominates) and rows hold enough hot entries per group that the
 // partial rows they cost are small against the gathers they turn into L2 hits.
-constexpr int32_t kHubRowDegree = 32;  // rows shorter than this keep all their entries in the cold class
+constexpr int32_t kHubRowDegree = 64;  // rows shorter than this keep all their entries in the cold class
 
 static bool want_hub(int32_t rows, int64_t nnz, int32_t f) {
   const int t = g_tune_hub.load(std::memory_order_relaxed);
@@ -930,16 +978,21 @@ static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream) 
   const int32_t f = d.f;
   int groups = g_tune_hub_groups.load(std::memory_order_relaxed);
   if (groups != 1 && groups != 2 && groups != 4 && groups != 8) groups = 8;
+  // Hot columns per tier = the rows of B that fit `kb` KiB per XCD group.  One tier: twice the 4 MB
+  // L2 of an XCD is the measured optimum (LRU keeps the hotter half).  Several tiers: each is sized
+  // to stay resident (measured optimum 5 to 6 MiB); how many there are is decided from the column
+  // counts when the plan is built, unless a number is forced.
   int tiers = g_tune_hub_tiers.load(std::memory_order_relaxed);
-  if (tiers < 1 || tiers * groups > 16) tiers = 1;
-  int kb = g_tune_hub_kb.load(std::memory_order_relaxed);
-  // one tier: twice the 4 MB L2 of an XCD is the measured optimum (LRU keeps the hottest half);
-  // several tiers: each is sized to stay resident
-  if (kb <= 0) kb = tiers == 1 ? 8192 : 3584;
-  int64_t per_group = (int64_t)kb * 1024 / ((int64_t)f * 4);
-  if (per_group < 1) per_group = 1;
-  int64_t hot = per_group * groups;  // columns per tier
-  if (hot > s.cols) hot = s.cols;
+  if (tiers < 0 || tiers * groups > kMaxHubClasses) tiers = 0;
+  const int kb_forced = g_tune_hub_kb.load(std::memory_order_relaxed);
+  auto columns_for = [&](int kb) {
+    int64_t per_group = (int64_t)kb * 1024 / ((int64_t)f * 4);
+    if (per_group < 1) per_group = 1;
+    const int64_t c = per_group * groups;
+    return c > s.cols ? (int64_t)s.cols : c;
+  };
+  const int64_t hot = columns_for(kb_forced > 0 ? kb_forced : (tiers == 1 ? 8192 : 5632));  // per tier
+  const int64_t hot_single = columns_for(kb_forced > 0 ? kb_forced : 8192);
   // hot tasks of a wide product use one dword per lane and chunk when the rows are not 16-byte
   // aligned: that is the fastest gather of L2-resident rows
   const int hot_vec = (vec == 4 || f / vec <= kWave) ? vec : 1;
@@ -949,8 +1002,9 @@ static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream) 
   if (min_degree <= 0) min_degree = kHubRowDegree;
   int slot = -1;
   for (int i = 0; i < CsrSide::kHubPlans; ++i)
-    if (s.hub[i].valid && s.hub[i].hot == (int32_t)hot && s.hub[i].groups == groups && s.hub[i].tiers == tiers &&
-        s.hub[i].seg == seg && s.hub[i].min_degree == min_degree)
+    if (s.hub[i].valid && s.hub[i].req_hot == (int32_t)hot && s.hub[i].req_single == (int32_t)hot_single &&
+        s.hub[i].req_tiers == tiers && s.hub[i].groups == groups && s.hub[i].seg == seg &&
+        s.hub[i].min_degree == min_degree)
       slot = i;
   if (slot < 0) {
     slot = 0;
@@ -961,7 +1015,7 @@ static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream) 
       }
       if (s.hub_used[i] < s.hub_used[slot]) slot = i;
     }
-    CG_TRY(build_hub(s, s.hub[slot], (int32_t)hot, groups, tiers, seg, min_degree, stream));
+    CG_TRY(build_hub(s, s.hub[slot], (int32_t)hot, (int32_t)hot_single, groups, tiers, seg, min_degree, stream));
   }
   s.hub_used[slot] = ++s.hub_clock;
   HubPlan &h = s.hub[slot];
@@ -978,7 +1032,8 @@ static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream) 
       CG_TRY(build_stream(h.hot_sched, h.vrowptr, nclass * n, true, nclass, h.tstart, S, s.nnz, h.hot_tab, owned, false,
                           stream));
     }
-    for (int t = 0; t < tiers; ++t) {
+    ProfScope prof("spmm_hub_hot", f, stream);  // all tiers of a product are timed as one
+    for (int t = 0; t < h.tiers; ++t) {
       StreamArgs sa{};
       sa.task_start = h.hot_tab.task_start;
       sa.task_dst = h.hot_tab.task_dst;
@@ -994,7 +1049,6 @@ static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream) 
       sa.P = (float *)p;
       sa.f = f;
       sa.beta = 0.f;
-      ProfScope prof("spmm_hub_hot", f, stream);
       CG_TRY(launch_stream(hshape, sa, stream));
     }
   }
@@ -1015,8 +1069,14 @@ static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream) 
     if (nclass <= 8)
       hub_reduce_kernel<8><<<rgrid, kSpmmThreads, 0, stream>>>(h.hot_sched.tbase, n, nclass, (const float *)p, d.C,
                                                                d.ldc, f);
-    else
+    else if (nclass <= 16)
       hub_reduce_kernel<16><<<rgrid, kSpmmThreads, 0, stream>>>(h.hot_sched.tbase, n, nclass, (const float *)p, d.C,
+                                                                d.ldc, f);
+    else if (nclass <= 32)
+      hub_reduce_kernel<32><<<rgrid, kSpmmThreads, 0, stream>>>(h.hot_sched.tbase, n, nclass, (const float *)p, d.C,
+                                                                d.ldc, f);
+    else
+      hub_reduce_kernel<64><<<rgrid, kSpmmThreads, 0, stream>>>(h.hot_sched.tbase, n, nclass, (const float *)p, d.C,
                                                                 d.ldc, f);
     CG_LAUNCH_CHECK();
   }

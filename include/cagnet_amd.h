@@ -275,8 +275,8 @@ int cg_prof_enable(int on);
  *   "spmm_hub"        hub plan: -1 never, 1 always, 0 by width and density
  *   "spmm_hub_kb"     KiB of hot B rows per XCD group and tier
  *   "spmm_hub_groups" XCD groups the hot columns are dealt to (1, 2, 4, 8)
- *   "spmm_hub_tiers"  tiers of hot columns (groups * tiers <= 16)
- *   "spmm_hub_row"    rows with fewer entries keep all of them in the cold class (0: 32)
+ *   "spmm_hub_tiers"  tiers of hot columns (0: chosen from the column counts; groups * tiers <= 64)
+ *   "spmm_hub_row"    rows with fewer entries keep all of them in the cold class (0: 64)
  *   "dense_mfma"      -1: dense products on the vector ALU tile kernel only
  *   "coo_cache_blocks" blocks cg_spmm_coo_cached keeps (0: 8; negative: none)
  * An unknown key returns CG_ERR_UNSUPPORTED. */
