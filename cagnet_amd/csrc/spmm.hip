@@ -1388,7 +1388,7 @@ int cg_spmm_coo_cached(const int32_t *d_row, const int32_t *d_col, const float *
   const int capacity = coo_cache_capacity();
   // Keeping a block pays through the column-popularity plan, which is too costly to build per call;
   // the plain schedule is rebuilt on the device for less than the digest costs (measured on 114.6 M
-  // entries: rebuild + 0.26 ms, digest and read-back + 0.57 ms; with a plan 34.6 -> 20.2 ms).
+  // entries: rebuild + 0.26 ms, digest and read-back + 0.57 ms; with a plan 34.4 -> 18.6 ms).
   if (nnz <= 0 || n <= 0 || m <= 0 || capacity == 0 || !want_hub(n, nnz, f))
     return cg_spmm_coo(d_row, d_col, d_val, nnz, n, m, d_B, ldb, d_C, ldc, f, beta, stream_);
   if (nnz > 0x7fffffffLL - 1 || n == 0x7fffffff || m == 0x7fffffff)
