@@ -32,6 +32,7 @@ struct SpmmShape {
 constexpr int kMaxHubClasses = 64;  // column classes of a hub plan (XCD groups x tiers)
 constexpr int kHubAutoTiers = 6;    // most tiers the automatic choice takes
 constexpr double kHubTierEntriesPerPair = 2.4;  // entries per (class, row) pair below which a tier no longer pays
+constexpr double kHubMinHotFraction = 0.35;     // share of the entries the first tier must hold for a plan to pay
 constexpr int kMaxChunks = 10;  // full-wave teams cover up to 64 * kMaxChunks * VEC columns per launch
 
 // Widest vector the operands allow.
@@ -584,9 +585,11 @@ struct SchedCache {
 struct HubPlan {
   int32_t hot = 0, groups = 0, tiers = 0, seg = 0, min_degree = 0;
   int32_t req_hot = 0, req_tiers = 0, req_single = 0;  // what was asked for (tiers 0: chosen from the column counts)
+  bool declined = false;  // the column counts said a plan does not pay: the plain schedule is used
   int32_t classes() const { return groups * tiers; }
   int32_t *vrowptr = nullptr, *colind = nullptr;
   float *val = nullptr;
+  uint8_t *row_hot = nullptr;  // 1 for rows long enough to have hot entries
   Sched hot_sched;        // over the virtual rows of the hot classes, empty rows skipped
   StreamTab hot_tab;      // its windows, one class per (tier, group)
   SchedCache cold_sched;  // over the cold class
@@ -599,9 +602,12 @@ struct HubPlan {
     if (vrowptr) (void)hipFree(vrowptr);
     if (colind) (void)hipFree(colind);
     if (val) (void)hipFree(val);
+    if (row_hot) (void)hipFree(row_hot);
     vrowptr = colind = nullptr;
     val = nullptr;
+    row_hot = nullptr;
     valid = false;
+    declined = false;
   }
 };
 
@@ -641,6 +647,12 @@ __global__ __launch_bounds__(kSpmmThreads) void col_count_kernel(const int32_t *
   if (k >= nnz) return;
   const int32_t r = erow[k];
   if (rowptr[r + 1] - rowptr[r] >= min_degree) atomicAdd(&count[colind[k]], 1u);  // integer count: order independent
+}
+
+__global__ __launch_bounds__(kSpmmThreads) void row_hot_kernel(const int32_t *__restrict__ rowptr, int32_t n,
+                                                               int32_t min_degree, uint8_t *__restrict__ out) {
+  const int64_t r = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (r < n) out[r] = rowptr[r + 1] - rowptr[r] >= min_degree ? 1 : 0;
 }
 
 // sort key that orders columns by descending count (ties: ascending column, by stability)
@@ -728,8 +740,10 @@ __global__ __launch_bounds__(kSpmmThreads) void csr_rows_kernel(const int32_t *_
 
 // tiers == 0: the number of tiers is chosen from the column counts (tiers of `hot` columns each); if
 // one tier comes out, it holds `hot_single` columns.
+// may_decline: leave the plan empty (h.declined) when the first tier would hold less than
+// kHubMinHotFraction of the entries.
 static int build_hub(CsrSide &s, HubPlan &h, int32_t hot, int32_t hot_single, int32_t groups, int32_t tiers,
-                     int32_t seg, int32_t min_degree, hipStream_t stream) {
+                     int32_t seg, int32_t min_degree, bool may_decline, hipStream_t stream) {
   CG_HIP(hipStreamSynchronize(stream));
   h.release();
   h.req_hot = hot;
@@ -771,10 +785,7 @@ static int build_hub(CsrSide &s, HubPlan &h, int32_t hot, int32_t hot_single, in
     int set = 0;
     CG_TRY(radix_sort_pairs(buf, m, bits_for((int32_t)(maxcount < 0x7ffffffeu ? maxcount + 1 : 0x7fffffff)), 0, &set,
                             stream));
-    if (tiers == 0) {
-      // A further tier serves its entries from L2 instead of HBM but costs every (class, row) pair it
-      // touches a partial row, written and read again: it pays while it holds well over two
-      // entries per pair it can have (measured break-even 2.4: f = 602 takes 4 tiers, 300 two, 128 one).
+    if (tiers == 0 || may_decline) {
       const int max_tiers = kMaxHubClasses / groups < kHubAutoTiers ? kMaxHubClasses / groups : kHubAutoTiers;
       unsigned long long *d_sums = nullptr, sums[kHubAutoTiers] = {0};
       CG_TRY(tmp.alloc((void **)&d_sums, sizeof(sums)));
@@ -782,9 +793,24 @@ static int build_hub(CsrSide &s, HubPlan &h, int32_t hot, int32_t hot_single, in
       CG_LAUNCH_CHECK();
       CG_HIP(hipMemcpyAsync(sums, d_sums, sizeof(unsigned long long) * max_tiers, hipMemcpyDeviceToHost, stream));
       CG_HIP(hipStreamSynchronize(stream));
-      tiers = 1;
-      while (tiers < max_tiers && (double)sums[tiers] >= kHubTierEntriesPerPair * (double)groups * (double)n) ++tiers;
-      if (tiers == 1) hot = hot_single;
+      // Measured over R-MAT graphs of 16 to 492 entries per row and blocks of them: with 45 % or more
+      // of the entries in the first tier the plan gains 20 to 37 %, with 25 to 29 % it gains 1 to 4 %.
+      if (may_decline && (double)sums[0] < kHubMinHotFraction * (double)nnz) {
+        h.declined = true;
+        h.groups = groups;
+        h.seg = seg;
+        h.min_degree = min_degree;
+        h.valid = true;
+        return CG_OK;
+      }
+      if (tiers == 0) {
+        // A further tier serves its entries from L2 instead of HBM but costs every (class, row) pair it
+        // touches a partial row, written and read again: it pays while it holds well over two
+        // entries per pair it can have (measured break-even 2.4: f = 602 takes 3 tiers, 300 two, 128 one).
+        tiers = 1;
+        while (tiers < max_tiers && (double)sums[tiers] >= kHubTierEntriesPerPair * (double)groups * (double)n) ++tiers;
+        if (tiers == 1) hot = hot_single;
+      }
     }
     col_class_kernel<<<gm, kSpmmThreads, 0, stream>>>(buf.payload[set], m, hot, groups, tiers, cls);
     CG_LAUNCH_CHECK();
@@ -794,6 +820,11 @@ static int build_hub(CsrSide &s, HubPlan &h, int32_t hot, int32_t hot_single, in
   if (vrows + 1 > 0x7fffffffLL) CG_FAIL(CG_ERR_OVERFLOW, "hub plan: %lld virtual rows exceed int32", (long long)vrows);
 
   // 2. stable regrouping of the entries by class: (row, col) order is kept inside a class
+  CG_TRY(dev_alloc((void **)&h.row_hot, (size_t)(n > 0 ? n : 1)));
+  if (n > 0) {
+    row_hot_kernel<<<(unsigned)ceil_div64(n, kSpmmThreads), kSpmmThreads, 0, stream>>>(s.rowptr, n, min_degree, h.row_hot);
+    CG_LAUNCH_CHECK();
+  }
   CG_TRY(dev_alloc((void **)&h.colind, (size_t)nnz * 4));
   CG_TRY(dev_alloc((void **)&h.val, (size_t)nnz * 4));
   CG_TRY(dev_alloc((void **)&h.vrowptr, (size_t)(vrows + 1) * 4));
@@ -852,6 +883,7 @@ struct DenseOps {
   // optional fold of another launch's partial rows into the rows written here (see StreamArgs)
   const int32_t *fold_tbase = nullptr;
   const float *fold_P = nullptr;
+  const uint8_t *fold_any = nullptr;
   int32_t fold_classes = 0, fold_rows = 0;
   // optional epilogue: finished rows are multiplied by W (f x fo) into Z instead of being stored
   // (see StreamArgs); C is then only read, and only when beta != 0
@@ -899,6 +931,7 @@ static int spmm_plain(const int32_t *rowptr, const int32_t *colind, const float 
   sa.beta = d.beta;
   sa.fold_tbase = d.fold_tbase;
   sa.fold_P = d.fold_P;
+  sa.fold_any = d.fold_any;
   sa.fold_classes = d.fold_classes;
   sa.fold_rows = d.fold_rows;
   if (d.fold_tbase && shape.lpr != kWave) CG_FAIL(CG_ERR_UNSUPPORTED, "fold needs full-wave teams");
@@ -965,16 +998,22 @@ static int spmm_plain(const int32_t *rowptr, const int32_t *colind, const float 
 // partial rows they cost are small against the gathers they turn into L2 hits.
 constexpr int32_t kHubRowDegree = 64;  // rows shorter than this keep all their entries in the cold class
 
+// Cheap test before any plan is built: wide rows of B, enough work for the extra launches to
+// disappear in it (products under about 3e9 multiply-adds measured slower with a plan), and not
+// a matrix of near-empty rows.  Whether the hot columns carry enough of the entries is decided
+// from the column counts when the plan is built (build_hub may decline).
 static bool want_hub(int32_t rows, int64_t nnz, int32_t f) {
   const int t = g_tune_hub.load(std::memory_order_relaxed);
   if (t < 0) return false;
   if (rows == 0 || nnz == 0) return false;
   if (t > 0) return true;
-  return f >= 64 && nnz / rows >= 128;  // measured on 492 entries per row: f = 44 even, f = 64 -28 %, f = 128 -53 %
+  return f >= 64 && nnz / rows >= 8 && (double)nnz * f >= 3e9;
 }
 static bool want_hub(const CsrSide &s, int32_t f) { return want_hub(s.rows, s.nnz, f); }
 
-static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream) {
+// *declined: the plan was found not to pay for this matrix and width; nothing was computed.
+static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream, bool *declined) {
+  *declined = false;
   const int32_t f = d.f;
   int groups = g_tune_hub_groups.load(std::memory_order_relaxed);
   if (groups != 1 && groups != 2 && groups != 4 && groups != 8) groups = 8;
@@ -1000,11 +1039,12 @@ static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream) 
   const int32_t seg = pick_seg(hshape);
   int32_t min_degree = g_tune_hub_row.load(std::memory_order_relaxed);
   if (min_degree <= 0) min_degree = kHubRowDegree;
+  const bool may_decline = g_tune_hub.load(std::memory_order_relaxed) == 0;
   int slot = -1;
   for (int i = 0; i < CsrSide::kHubPlans; ++i)
     if (s.hub[i].valid && s.hub[i].req_hot == (int32_t)hot && s.hub[i].req_single == (int32_t)hot_single &&
         s.hub[i].req_tiers == tiers && s.hub[i].groups == groups && s.hub[i].seg == seg &&
-        s.hub[i].min_degree == min_degree)
+        s.hub[i].min_degree == min_degree && (may_decline || !s.hub[i].declined))
       slot = i;
   if (slot < 0) {
     slot = 0;
@@ -1015,10 +1055,15 @@ static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream) 
       }
       if (s.hub_used[i] < s.hub_used[slot]) slot = i;
     }
-    CG_TRY(build_hub(s, s.hub[slot], (int32_t)hot, (int32_t)hot_single, groups, tiers, seg, min_degree, stream));
+    CG_TRY(build_hub(s, s.hub[slot], (int32_t)hot, (int32_t)hot_single, groups, tiers, seg, min_degree, may_decline,
+                     stream));
   }
   s.hub_used[slot] = ++s.hub_clock;
   HubPlan &h = s.hub[slot];
+  if (h.declined) {
+    *declined = true;
+    return CG_OK;
+  }
   const int32_t n = s.rows;
   const int32_t nclass = h.classes();
   // 1. hot classes, one launch per tier: every task writes a partial row
@@ -1059,6 +1104,7 @@ static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream) 
   if (fused) {
     cold.fold_tbase = h.hot_sched.tbase;
     cold.fold_P = (const float *)p;
+    cold.fold_any = h.row_hot;
     cold.fold_classes = nclass;
     cold.fold_rows = n;
   }
@@ -1106,7 +1152,11 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
     d.epi_fo = epi->epi_fo;
     d.epi_relu = epi->epi_relu;
   }
-  if (f <= range_cap(vec == 4 ? 4 : 1) && want_hub(s, f)) return spmm_hub(s, vec, d, stream);
+  if (f <= range_cap(vec == 4 ? 4 : 1) && want_hub(s, f)) {
+    bool declined = false;
+    CG_TRY(spmm_hub(s, vec, d, stream, &declined));
+    if (!declined) return CG_OK;
+  }
   if (epi) return spmm_plain(s.rowptr, s.colind, s.val, s.rows, s.nnz, s.sched, vec, d, f, stream);
   for (int32_t f0 = 0; f0 < f; f0 += cap) {  // wider outputs take several launches over column ranges
     const int32_t ft = f - f0 < cap ? f - f0 : cap;

@@ -112,8 +112,11 @@ struct StreamArgs {
   // Fold (wide teams, groups == 1): a row that goes straight to C also receives the partial rows
   // fold_P[t] for t in [fold_tbase[c * fold_rows + row], fold_tbase[c * fold_rows + row + 1]) of
   // every class c < fold_classes, added in (class, t) order after the row's own entries.
+  // fold_any (nullable): one byte per row, 0 for rows that have no partial rows at all, so that
+  // the many short rows of a low-degree matrix do not pay the per-class look-ups.
   const int32_t *fold_tbase;
   const float *fold_P;
+  const uint8_t *fold_any;
   int32_t fold_classes, fold_rows;
   // Epilogue (wide teams, groups == 1): a finished row r = beta*C[row] + (A B)[row] is not stored
   // but multiplied by epi_W (f x epi_fo): epi_Z[row, :] = act(r * epi_W), the layer's (A H) W
@@ -289,7 +292,7 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_stream_wide_kernel(const St
         const int32_t dst = __builtin_amdgcn_readlane(m_dst, tk);
         if (dst >= 0) {
           bool folded = false;
-          if (a.fold_tbase) {
+          if (a.fold_tbase && (!a.fold_any || a.fold_any[dst])) {
             for (int32_t cls = 0; cls < a.fold_classes; ++cls) {
               const int32_t *tb = a.fold_tbase + (int64_t)cls * a.fold_rows + dst;
               const int32_t p0 = __builtin_amdgcn_readfirstlane(tb[0]);
