@@ -1610,8 +1610,16 @@ int cg_csr_info(const cg_csr_t *h, int64_t info[8]) {
   info[3] = h->has_t ? 1 : 0;
   info[4] = h->fwd.max_degree;
   info[5] = h->has_t ? h->tr.max_degree : -1;
-  info[6] = 0;
-  info[7] = 0;
+  // the plan the last wide product of a side looked up: tiers taken, -1 declined, 0 none so far
+  auto last_plan = [](const cg::CsrSide &s) -> int64_t {
+    int best = -1;
+    for (int i = 0; i < cg::CsrSide::kHubPlans; ++i)
+      if (s.hub[i].valid && (best < 0 || s.hub_used[i] > s.hub_used[best])) best = i;
+    if (best < 0) return 0;
+    return s.hub[best].declined ? -1 : s.hub[best].tiers;
+  };
+  info[6] = last_plan(h->fwd);
+  info[7] = h->has_t ? last_plan(h->tr) : 0;
   return CG_OK;
 }
 

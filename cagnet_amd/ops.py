@@ -313,7 +313,9 @@ class CsrMatrix:
         buf = (c_int64 * 8)()
         check(lib.cg_csr_info(self._handle, buf), "cg_csr_info")
         return {"n": buf[0], "m": buf[1], "nnz": buf[2], "has_transpose": bool(buf[3]),
-                "max_row_degree": buf[4], "max_col_degree": buf[5]}
+                "max_row_degree": buf[4], "max_col_degree": buf[5],
+                # column-popularity plan the last wide product looked up: tiers, -1 declined, 0 none
+                "plan_tiers": buf[6], "plan_tiers_transpose": buf[7]}
 
     def arrays(self, transpose: bool = False):
         """(rowptr, colind, values) of A, or of A^T, as tensors that alias the handle's memory."""

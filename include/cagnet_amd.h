@@ -161,7 +161,9 @@ int cg_csr_spmm_xw(cg_csr_t *h, int transpose, const float *d_B, int64_t ldb, co
                    const float *d_W, int64_t ldw, float *d_Z, int64_t ldz, int32_t f, int32_t fo, int relu,
                    cg_stream_t stream);
 
-/* info[0..7] = { n, m, nnz, has_transpose, max row degree, max column degree (or -1), 0, 0 } */
+/* info[0..7] = { n, m, nnz, has_transpose, max row degree, max column degree (or -1),
+ *                column-popularity plan last looked up by a wide product of A, of A^T:
+ *                tiers in use, -1 when the column counts declined it, 0 when none was considered } */
 int cg_csr_info(const cg_csr_t *h, int64_t info[8]);
 /* Device pointers of the arrays the handle owns (transpose != 0: those of A^T). */
 int cg_csr_arrays(const cg_csr_t *h, int transpose, const int32_t **d_rowptr, const int32_t **d_colind,

@@ -458,6 +458,39 @@ def test_spmm_hub_plan_short_rows_stay_cold(cuda, tune, min_degree):
     assert spmm_error(C, row, col, val, n, m, B, C0) <= REL_TOL
 
 
+def test_spmm_hub_plan_is_declined_when_columns_are_not_skewed(cuda):
+    """Built-in choice at a size where a plan is considered (>= 3e9 multiply-adds): with uniformly
+    spread columns the first tier would hold a tenth of the entries, the plan is declined and the
+    plain schedule computes the product; with power-law columns of the same size it is taken.  Both
+    must match the oracle and repeat bit for bit."""
+    from cagnet_amd import ops
+    n, f = 100_000, 602
+    gen = torch.Generator().manual_seed(41)
+    B = torch.randn(n, f, generator=gen)
+    Bd = B.to(cuda)
+    per_row = 96                                                       # rows long enough to have hot entries
+    row = torch.arange(n).repeat_interleave(per_row)
+    sample = torch.randint(0, n, (3000,), generator=gen)               # rows checked against the oracle
+    for skewed in (False, True):
+        u = torch.rand(n * per_row, generator=gen)
+        col = ((u ** 6) * n).long() if skewed else (u * n).long()      # u^6: a few columns take most entries
+        key = torch.unique(row * n + col)                              # (row, col) ascending, duplicates dropped
+        r, c = key // n, key % n
+        v = torch.rand(key.numel(), generator=gen) + 0.5
+        A = ops.CsrMatrix(_i32(r, cuda), _i32(c, cuda), v.to(cuda), n, n)
+        got = A.spmm(Bd)
+        assert torch.equal(got, A.spmm(Bd))
+        assert key.numel() * f >= 3e9                                  # large enough for a plan to be considered
+        tiers = A.info()["plan_tiers"]
+        assert (tiers >= 1) if skewed else (tiers == -1), tiers
+        keep = torch.isin(r, sample)
+        ref_rows = torch.unique(r[keep])
+        remap = torch.full((n,), -1, dtype=torch.long)
+        remap[ref_rows] = torch.arange(ref_rows.numel())
+        err = spmm_error(got[ref_rows.to(cuda)], remap[r[keep]], c[keep], v[keep], ref_rows.numel(), n, B)
+        assert err <= REL_TOL, (skewed, err)
+
+
 def test_spmm_hub_plans_of_several_widths_on_one_handle(cuda, tune):
     """A handle keeps two hub plans (the hot-column count depends on the width); cycling through
     three widths exercises reuse and replacement, and every product stays bit-identical to its
