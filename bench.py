@@ -46,7 +46,7 @@ WORKLOADS = {
 
 # HBM bytes per launch of the dominant product (all of its kernels together) from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE runs, reads scaled by 2.0 and writes by 1.0 as calibrated on a 1 GiB copy
-# kernel: profiles/spmm_f602_reddit_counters.txt (131.3 GB read + 4.3 GB written) and
+# kernel: profiles/spmm_f602_reddit_counters.txt (89.3 GB read + 6.0 GB written) and
 # profiles/spmm_amazon_counters.txt (291.6 GB read + 17.6 GB written, f = 300).
 MEASURED_TRAFFIC_BYTES = {"reddit": 95.3e9, "amazon": 309.2e9}
 
