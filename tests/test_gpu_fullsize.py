@@ -194,3 +194,76 @@ def test_amazon_shape_products(cuda):
     _check_product(A, row, col, val, G, seed=2)                          # narrow teams
     _check_product(A, row, col, val, torch.randn(n, spec["classes"], device=cuda, generator=gen), transpose=True, seed=3)
     _check_dense(X, W, G)
+
+
+def test_rmat20_shape_products(cuda):
+    """Configuration 2 (R-MAT scale 20: 1,048,576 vertices, 16,777,216 directed edges): A H and A^T G
+    at the four widths, with the transpose built by the library from entries given in arbitrary order."""
+    from cagnet_amd import ops
+    row, col, n = synth.rmat_graph(20, 16_777_216, 1, cuda)
+    val = synth.gcn_normalize(row, col, n)
+    nnz = row.numel()
+    perm = torch.randperm(nnz, device=cuda, generator=torch.Generator(device=cuda).manual_seed(2))
+    A = ops.CsrMatrix(row.int()[perm], col.int()[perm], val[perm], n, n, is_sorted=False, transpose=True)
+    del perm
+    rowptr, colind, values = A.arrays()
+    _structure(rowptr, colind, n, nnz)
+    assert torch.equal(colind, col.int()) and torch.equal(values, val)   # any order in, the (row, col) order out
+    tp, ti, tv = A.arrays(transpose=True)
+    assert torch.equal(tp, rowptr) and torch.equal(ti, colind) and torch.equal(tv, values)  # symmetric bit for bit
+    del rowptr, colind, values, tp, ti, tv
+    gen = torch.Generator(device=cuda).manual_seed(19)
+    for f in (16, 64, 128, 602):
+        B = torch.randn(n, f, device=cuda, generator=gen)
+        C = _check_product(A, row, col, val, B, seed=f)
+        # the graph is symmetric, so the product with the stored transpose sums the same terms in the same order
+        assert torch.equal(A.spmm(B, transpose=True), C)
+        del B, C
+
+
+def test_reddit_shape_grid_row_of_blocks(cuda):
+    """Configuration 4: the four sparse blocks A(r, 0..3) of the last process row of the 4 x 4 grid
+    (58,242 rows; block columns of 58,241 | 58,241 | 58,241 | 58,242), cut by the library, each times
+    its 602-wide block of H and accumulated over the four stages through the reference's operator
+    (gcn_distr_2d.py:333-417) -- against the same rows of the whole product."""
+    from cagnet_amd import ops
+    from cagnet_amd.sparse_coo_tensor_cpp import spmm_gpu
+    spec = REDDIT
+    n, f, q = spec["n"], spec["f"], 4
+    row, col, val = _graph(spec, cuda)
+    r32, c32 = row.int(), col.int()
+    b = synth.block_bounds_2d(n, q)
+    assert [b[k + 1] - b[k] for k in range(q)] == [58_241, 58_241, 58_241, 58_242]
+    r = q - 1
+    rows = b[r + 1] - b[r]
+    H = torch.randn(n, f, device=cuda, generator=torch.Generator(device=cuda).manual_seed(23))
+    z = torch.zeros(rows, f, device=cuda)
+    mag = torch.zeros(rows, f, device=cuda)
+    total = 0
+    for k in range(q):
+        br, bc, bv = ops.coo_block(r32, c32, val, b[r], b[r + 1], b[k], b[k + 1])
+        inside = (row >= b[r]) & (row < b[r + 1]) & (col >= b[k]) & (col < b[k + 1])       # split_coo, gcn_distr.py:398-409
+        assert torch.equal(br.long(), row[inside] - b[r]) and torch.equal(bc.long(), col[inside] - b[k])
+        assert torch.equal(bv, val[inside])
+        total += br.numel()
+        Hk = H[b[k]:b[k + 1]].contiguous()
+        for pass_ in range(2):                                                           # second pass: a block seen before
+            zk = torch.zeros(rows, f, device=cuda)
+            spmm_gpu(br, bc, bv, rows, b[k + 1] - b[k], Hk, zk)
+            if pass_ == 0:
+                first = zk
+        assert torch.equal(first, zk)
+        spmm_gpu(br, bc, bv, rows, b[k + 1] - b[k], Hk, z)                                # accumulates over the stages
+        spmm_gpu(br, bc, bv, rows, b[k + 1] - b[k], Hk.abs(), mag)
+        del br, bc, bv, inside, Hk, zk, first
+    assert total == int(((row >= b[r]) & (row < b[r + 1])).sum())
+    A = ops.CsrMatrix(r32, c32, val, n, n, is_sorted=True)
+    whole = A.spmm(H)[b[r]:b[r + 1]]
+    assert float(((z - whole).abs() / mag.clamp_min(1e-30)).max()) <= 4 * REL_TOL
+    # rows recomputed in fp64 from the COO arrays
+    rowptr = torch.searchsorted(row, torch.arange(n + 1, device=cuda))
+    for i in torch.randint(b[r], b[r + 1], (32,), generator=torch.Generator().manual_seed(29)).tolist():
+        s, e = int(rowptr[i]), int(rowptr[i + 1])
+        a, hb = val[s:e].double(), H[col[s:e]].double()
+        err = ((z[i - b[r]].double() - a @ hb).abs() / (a.abs() @ hb.abs()).clamp_min(1e-30)).max()
+        assert float(err) <= REL_TOL, f"row {i}: {float(err)}"
