@@ -80,6 +80,18 @@ struct SortBuffers {
 };
 int radix_sort_pairs(SortBuffers &buf, int64_t count, int bits_a, int bits_b, int *result_set, hipStream_t stream);
 
+// The same sort from caller-owned inputs to caller-owned outputs: the first pass reads `in_*`, the
+// last writes `out_*`, the passes between ping-pong through `tmp` (both sets are needed from three
+// passes on).  in_p == nullptr: the payload is the record's position in the input (the result is
+// the sorting permutation).  payload == false: none is carried.  Outputs that are nullptr are
+// dropped.  The inputs are never written.
+struct SortIo {
+  const int32_t *in_a, *in_b, *in_p;
+  int32_t *out_a, *out_b, *out_p;
+  bool payload;
+};
+int radix_sort_records(const SortIo &io, SortBuffers &tmp, int64_t count, int bits_a, int bits_b, hipStream_t stream);
+
 // coo2csr.hip
 int launch_rowptr(const int32_t *d_row, int64_t nnz, int32_t n, int32_t *d_rowptr, hipStream_t stream);
 // row index of every stored entry of a CSR matrix

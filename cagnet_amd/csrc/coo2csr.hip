@@ -70,11 +70,6 @@ __global__ __launch_bounds__(kThreads) void coo_check_kernel(const int32_t *__re
   if (f && (threadIdx.x & (kWave - 1)) == 0) atomicOr(flags, f);  // one per wavefront; integer OR: order independent
 }
 
-__global__ __launch_bounds__(kThreads) void iota_kernel(int32_t *__restrict__ out, int64_t count) {
-  const int64_t k = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-  if (k < count) out[k] = (int32_t)k;
-}
-
 __global__ __launch_bounds__(kThreads) void gather_f32_kernel(const float *__restrict__ src,
                                                               const int32_t *__restrict__ perm,
                                                               float *__restrict__ dst, int64_t count) {
@@ -157,11 +152,14 @@ struct DevArena {
 
 static size_t sort_coo_bytes(int64_t count) { return 6 * DevArena::pad((size_t)count * sizeof(int32_t)); }
 
-// Sort records (key_a major, key_b minor) carrying the input position; hand back the sorted
-// key arrays and the permutation in caller-owned outputs.
-// `tmp` must have sort_coo_bytes(count) left.
-static int sort_coo(const int32_t *d_key_a, const int32_t *d_key_b, int64_t count, int bits_a, int bits_b,
-                    int32_t *d_out_a, int32_t *d_out_b, int32_t *d_out_perm, DevArena &tmp, hipStream_t stream) {
+// Sort records (key_a major, key_b minor) from the caller's arrays into the caller's outputs.
+// payload == nullptr with want_perm: the records carry their input position, d_out_p receives the
+// sorting permutation.  payload != nullptr: its 32-bit words travel with the records (values need no
+// gather by permutation afterwards).  Neither: the keys travel alone.
+// `tmp` must have sort_coo_bytes(count) left; the caller synchronises before its arena goes away.
+static int sort_coo(const int32_t *d_key_a, const int32_t *d_key_b, const int32_t *d_payload, bool want_perm,
+                    int64_t count, int bits_a, int bits_b, int32_t *d_out_a, int32_t *d_out_b, int32_t *d_out_p,
+                    DevArena &tmp, hipStream_t stream) {
   SortBuffers buf;
   const size_t bytes = (size_t)count * sizeof(int32_t);
   for (int s = 0; s < 2; ++s) {
@@ -169,36 +167,39 @@ static int sort_coo(const int32_t *d_key_a, const int32_t *d_key_b, int64_t coun
     CG_TRY(tmp.take((void **)&buf.key_b[s], bytes));
     CG_TRY(tmp.take((void **)&buf.payload[s], bytes));
   }
-  if (count > 0) {
-    CG_HIP(hipMemcpyAsync(buf.key_a[0], d_key_a, bytes, hipMemcpyDeviceToDevice, stream));
-    CG_HIP(hipMemcpyAsync(buf.key_b[0], d_key_b, bytes, hipMemcpyDeviceToDevice, stream));
-    iota_kernel<<<(unsigned)ceil_div64(count, kThreads), kThreads, 0, stream>>>(buf.payload[0], count);
-    CG_LAUNCH_CHECK();
-  }
-  int set = 0;
-  CG_TRY(radix_sort_pairs(buf, count, bits_a, bits_b, &set, stream));
-  if (count > 0) {
-    if (d_out_a) CG_HIP(hipMemcpyAsync(d_out_a, buf.key_a[set], bytes, hipMemcpyDeviceToDevice, stream));
-    if (d_out_b) CG_HIP(hipMemcpyAsync(d_out_b, buf.key_b[set], bytes, hipMemcpyDeviceToDevice, stream));
-    if (d_out_perm) CG_HIP(hipMemcpyAsync(d_out_perm, buf.payload[set], bytes, hipMemcpyDeviceToDevice, stream));
-  }
-  return CG_OK;  // the caller synchronises before its arena goes away
+  const SortIo io{d_key_a, d_key_b, d_payload, d_out_a, d_out_b, d_out_p, d_payload != nullptr || want_perm};
+  return radix_sort_records(io, buf, count, bits_a, bits_b, stream);
 }
+
+// Values ride along as the payload unless the caller wants the permutation, in which case they are
+// gathered by it afterwards.
+struct ValuePlan {
+  const int32_t *payload;
+  int32_t *out_p;
+  bool want_perm, gather;
+  ValuePlan(const float *d_val, float *d_val_out, int32_t *d_perm) {
+    const bool values = d_val && d_val_out;
+    want_perm = d_perm != nullptr;
+    gather = values && want_perm;
+    payload = values && !want_perm ? reinterpret_cast<const int32_t *>(d_val) : nullptr;
+    out_p = want_perm ? d_perm : (values ? reinterpret_cast<int32_t *>(d_val_out) : nullptr);
+  }
+};
 
 int coo2csr_general(const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz, int32_t n,
                     int32_t m, int32_t *d_rowptr, int32_t *d_colind, float *d_values, int32_t *d_perm,
                     hipStream_t stream) {
   DevArena tmp;
   const size_t ebytes = (size_t)nnz * sizeof(int32_t);
-  CG_TRY(tmp.reserve(sort_coo_bytes(nnz) + 2 * DevArena::pad(ebytes)));
-  int32_t *d_rows_sorted = nullptr, *d_perm_local = d_perm;
+  CG_TRY(tmp.reserve(sort_coo_bytes(nnz) + DevArena::pad(ebytes)));
+  int32_t *d_rows_sorted = nullptr;
   CG_TRY(tmp.take((void **)&d_rows_sorted, ebytes));
-  if (!d_perm_local) CG_TRY(tmp.take((void **)&d_perm_local, ebytes));
-  CG_TRY(sort_coo(d_row, d_col, nnz, bits_for(n), bits_for(m), d_rows_sorted, d_colind, d_perm_local, tmp, stream));
+  const ValuePlan vp(d_val, d_values, d_perm);
+  CG_TRY(sort_coo(d_row, d_col, vp.payload, vp.want_perm, nnz, bits_for(n), bits_for(m), d_rows_sorted, d_colind,
+                  vp.out_p, tmp, stream));
   CG_TRY(launch_rowptr(d_rows_sorted, nnz, n, d_rowptr, stream));
-  if (d_val && d_values && nnz > 0) {
-    gather_f32_kernel<<<(unsigned)ceil_div64(nnz, kThreads), kThreads, 0, stream>>>(d_val, d_perm_local, d_values,
-                                                                                   nnz);
+  if (vp.gather && nnz > 0) {
+    gather_f32_kernel<<<(unsigned)ceil_div64(nnz, kThreads), kThreads, 0, stream>>>(d_val, d_perm, d_values, nnz);
     CG_LAUNCH_CHECK();
   }
   CG_HIP(hipStreamSynchronize(stream));
@@ -210,11 +211,10 @@ int csr_transpose(const int32_t *d_rowptr, const int32_t *d_colind, const float 
                   hipStream_t stream) {
   DevArena tmp;
   const size_t ebytes = (size_t)nnz * sizeof(int32_t);
-  CG_TRY(tmp.reserve(sort_coo_bytes(nnz) + 3 * DevArena::pad(ebytes)));
-  int32_t *d_rows = nullptr, *d_cols_sorted = nullptr, *d_perm_local = d_perm;
+  CG_TRY(tmp.reserve(sort_coo_bytes(nnz) + 2 * DevArena::pad(ebytes)));
+  int32_t *d_rows = nullptr, *d_cols_sorted = nullptr;
   CG_TRY(tmp.take((void **)&d_rows, ebytes));
   CG_TRY(tmp.take((void **)&d_cols_sorted, ebytes));
-  if (!d_perm_local) CG_TRY(tmp.take((void **)&d_perm_local, ebytes));
   if (n > 0) {
     csr_expand_rows_kernel<<<(unsigned)ceil_div64((int64_t)n * kWave, kThreads), kThreads, 0, stream>>>(d_rowptr, n,
                                                                                                        d_rows);
@@ -222,11 +222,12 @@ int csr_transpose(const int32_t *d_rowptr, const int32_t *d_colind, const float 
   }
   // CSR order is (row, col) ascending, so a stable sort on col alone yields (col, row) order:
   // major key = col (key_a), minor key = row with zero bits (already in place).
-  CG_TRY(sort_coo(d_colind, d_rows, nnz, bits_for(m), 0, d_cols_sorted, d_rowind, d_perm_local, tmp, stream));
+  const ValuePlan vp(d_values, d_values_t, d_perm);
+  CG_TRY(sort_coo(d_colind, d_rows, vp.payload, vp.want_perm, nnz, bits_for(m), 0, d_cols_sorted, d_rowind, vp.out_p, tmp,
+                  stream));
   CG_TRY(launch_rowptr(d_cols_sorted, nnz, m, d_colptr, stream));
-  if (d_values && d_values_t && nnz > 0) {
-    gather_f32_kernel<<<(unsigned)ceil_div64(nnz, kThreads), kThreads, 0, stream>>>(d_values, d_perm_local,
-                                                                                   d_values_t, nnz);
+  if (vp.gather && nnz > 0) {
+    gather_f32_kernel<<<(unsigned)ceil_div64(nnz, kThreads), kThreads, 0, stream>>>(d_values, d_perm, d_values_t, nnz);
     CG_LAUNCH_CHECK();
   }
   CG_HIP(hipStreamSynchronize(stream));

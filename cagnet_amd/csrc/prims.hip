@@ -149,6 +149,8 @@ __global__ __launch_bounds__(kSortThreads) void radix_hist_kernel(const int32_t 
 // number of lower lanes in that peer set plus the wave's running count of the digit.  The records
 // are then ordered by digit inside LDS and written out from there, so that the records of one
 // digit leave as one contiguous run instead of one 4-byte store each.
+// in_p == nullptr: the payload of a record is its position in the input.  Outputs that are nullptr
+// are not written.
 __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
     int key_is_a, int shift, int dbits, const int32_t *__restrict__ in_a, const int32_t *__restrict__ in_b,
     const int32_t *__restrict__ in_p, int32_t *__restrict__ out_a, int32_t *__restrict__ out_b,
@@ -163,7 +165,8 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const uint64_t lt_mask = (1ull << lane) - 1ull;
-  const int64_t tile_base = (int64_t)blockIdx.x * kSortTile;
+  const int64_t tile = blockIdx.x;
+  const int64_t tile_base = tile * kSortTile;
   const int64_t base = tile_base + (int64_t)wave * kSortWaveTile;
   const uint32_t dmask = (1u << dbits) - 1u;
 
@@ -178,7 +181,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
     if (valid) {
       ra[r] = in_a[idx];
       rb[r] = in_b[idx];
-      rp[r] = in_p[idx];
+      rp[r] = in_p ? in_p[idx] : (int32_t)idx;
       d = ((uint32_t)(key_is_a ? ra[r] : rb[r]) >> shift) & dmask;
     }
     uint64_t peers = __ballot(valid);
@@ -219,7 +222,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
     uint32_t excl = inc - total;
     for (int w = 0; w < wave; ++w) excl += wave_total[w];
     // modulo 2^32, undone by the addition below; digits beyond the pass's range have no records
-    goff[t] = t <= (int)dmask ? scanned_hist[(int64_t)t * tiles + blockIdx.x] - excl : 0u;
+    goff[t] = t <= (int)dmask ? scanned_hist[(int64_t)t * tiles + tile] - excl : 0u;
     uint32_t run = excl;
 #pragma unroll
     for (int w = 0; w < kSortWaves; ++w) {
@@ -248,42 +251,104 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
     const int32_t va = sa[i], vb = sb[i];
     const uint32_t d = ((uint32_t)(key_is_a ? va : vb) >> shift) & dmask;
     const uint32_t pos = goff[d] + (uint32_t)i;
-    out_a[pos] = va;
-    out_b[pos] = vb;
-    out_p[pos] = sp[i];
+    if (out_a) out_a[pos] = va;
+    if (out_b) out_b[pos] = vb;
+    if (out_p) out_p[pos] = sp[i];
   }
+}
+
+struct SortPass {
+  int which, shift, dbits;  // which 0: digit of key_b (minor key), 1: of key_a (major key)
+};
+
+// Balanced digits: the fewest 8-bit passes, each as narrow as that allows (18 bits: 3 x 6), so the
+// records of one digit leave a tile as longer runs.
+static int plan_passes(int bits_a, int bits_b, SortPass out[16]) {
+  int count = 0;
+  for (int which = 0; which < 2; ++which) {
+    const int bits = which == 0 ? bits_b : bits_a;
+    if (bits <= 0) continue;
+    const int passes = (bits + 7) / 8;
+    const int dbits = (bits + passes - 1) / passes;
+    for (int shift = 0; shift < bits; shift += dbits) out[count++] = SortPass{which, shift, dbits};
+  }
+  return count;
+}
+
+static int sort_pass(const SortPass &ps, const int32_t *in_a, const int32_t *in_b, const int32_t *in_p, int32_t *out_a,
+                     int32_t *out_b, int32_t *out_p, int64_t count, uint32_t *hist, int64_t tiles, hipStream_t stream) {
+  radix_hist_kernel<<<(unsigned)tiles, kSortThreads, 0, stream>>>(ps.which == 0 ? in_b : in_a, count, ps.shift, ps.dbits,
+                                                                  hist, tiles);
+  CG_LAUNCH_CHECK();
+  CG_TRY(exclusive_scan_u32(hist, hist, tiles << ps.dbits, nullptr, stream));
+  radix_scatter_kernel<<<(unsigned)tiles, kSortThreads, 0, stream>>>(ps.which, ps.shift, ps.dbits, in_a, in_b, in_p, out_a,
+                                                                     out_b, out_p, count, hist, tiles);
+  CG_LAUNCH_CHECK();
+  return CG_OK;
+}
+
+static int sort_hist(int64_t count, uint32_t **hist, int64_t *tiles, hipStream_t stream) {
+  if (count > 0x7fffffffLL) CG_FAIL(CG_ERR_OVERFLOW, "radix sort: count %lld >= 2^31", (long long)count);
+  *tiles = ceil_div64(count, kSortTile);
+  void *d_hist = nullptr;
+  CG_TRY(scratch_get(stream, kSlotC, (size_t)*tiles * kRadix * sizeof(uint32_t), &d_hist));
+  *hist = (uint32_t *)d_hist;
+  return CG_OK;
 }
 
 int radix_sort_pairs(SortBuffers &buf, int64_t count, int bits_a, int bits_b, int *result_set, hipStream_t stream) {
   int cur = 0;
   *result_set = 0;
   if (count <= 1) return CG_OK;
-  if (count > 0x7fffffffLL) CG_FAIL(CG_ERR_OVERFLOW, "radix sort: count %lld >= 2^31", (long long)count);
-  const int64_t tiles = ceil_div64(count, kSortTile);
-  void *d_hist = nullptr;
-  CG_TRY(scratch_get(stream, kSlotC, (size_t)tiles * kRadix * sizeof(uint32_t), &d_hist));
-  uint32_t *hist = (uint32_t *)d_hist;
-
-  for (int which = 0; which < 2; ++which) {  // 0: minor key (key_b), 1: major key (key_a)
-    const int bits = which == 0 ? bits_b : bits_a;
-    if (bits <= 0) continue;
-    // balanced digits: the fewest 8-bit passes, each as narrow as that allows (18 bits: 3 x 6), so the
-    // records of one digit leave a tile as longer runs
-    const int passes = (bits + 7) / 8;
-    const int dbits = (bits + passes - 1) / passes;
-    for (int shift = 0; shift < bits; shift += dbits) {
-      const int32_t *key = which == 0 ? buf.key_b[cur] : buf.key_a[cur];
-      radix_hist_kernel<<<(unsigned)tiles, kSortThreads, 0, stream>>>(key, count, shift, dbits, hist, tiles);
-      CG_LAUNCH_CHECK();
-      CG_TRY(exclusive_scan_u32(hist, hist, tiles << dbits, nullptr, stream));
-      radix_scatter_kernel<<<(unsigned)tiles, kSortThreads, 0, stream>>>(
-          which, shift, dbits, buf.key_a[cur], buf.key_b[cur], buf.payload[cur], buf.key_a[cur ^ 1], buf.key_b[cur ^ 1],
-          buf.payload[cur ^ 1], count, hist, tiles);
-      CG_LAUNCH_CHECK();
-      cur ^= 1;
-    }
+  uint32_t *hist = nullptr;
+  int64_t tiles = 0;
+  CG_TRY(sort_hist(count, &hist, &tiles, stream));
+  SortPass passes[16];
+  const int np = plan_passes(bits_a, bits_b, passes);
+  for (int i = 0; i < np; ++i) {
+    CG_TRY(sort_pass(passes[i], buf.key_a[cur], buf.key_b[cur], buf.payload[cur], buf.key_a[cur ^ 1], buf.key_b[cur ^ 1],
+                     buf.payload[cur ^ 1], count, hist, tiles, stream));
+    cur ^= 1;
   }
   *result_set = cur;
+  return CG_OK;
+}
+
+int radix_sort_records(const SortIo &io, SortBuffers &tmp, int64_t count, int bits_a, int bits_b, hipStream_t stream) {
+  if (count <= 0) return CG_OK;
+  uint32_t *hist = nullptr;
+  int64_t tiles = 0;
+  CG_TRY(sort_hist(count, &hist, &tiles, stream));
+  SortPass passes[16];
+  int np = plan_passes(bits_a, bits_b, passes);
+  if (np == 0) passes[np++] = SortPass{1, 0, 0};  // nothing to sort on: one pass with a single digit copies the records
+  if (np == 1) {
+    // a single pass would write the outputs while other tiles still read the inputs: when they overlap,
+    // a copying pass through `tmp` comes first
+    const size_t bytes = (size_t)count * sizeof(int32_t);
+    const int32_t *ins[3] = {io.in_a, io.in_b, io.in_p};
+    const int32_t *outs[3] = {io.out_a, io.out_b, io.payload ? io.out_p : nullptr};
+    bool overlap = false;
+    for (const int32_t *i : ins)
+      for (const int32_t *o : outs)
+        if (i && o && (const char *)i < (const char *)o + bytes && (const char *)o < (const char *)i + bytes) overlap = true;
+    if (overlap) {
+      passes[1] = passes[0];
+      passes[0] = SortPass{1, 0, 0};
+      np = 2;
+    }
+  }
+  for (int i = 0; i < np; ++i) {
+    const bool first = i == 0, last = i == np - 1;
+    const int from = (i - 1) & 1, to = i & 1;
+    const int32_t *in_a = first ? io.in_a : tmp.key_a[from];
+    const int32_t *in_b = first ? io.in_b : tmp.key_b[from];
+    const int32_t *in_p = first ? io.in_p : (io.payload ? tmp.payload[from] : nullptr);
+    int32_t *out_a = last ? io.out_a : tmp.key_a[to];
+    int32_t *out_b = last ? io.out_b : tmp.key_b[to];
+    int32_t *out_p = !io.payload ? nullptr : (last ? io.out_p : tmp.payload[to]);
+    CG_TRY(sort_pass(passes[i], in_a, in_b, in_p, out_a, out_b, out_p, count, hist, tiles, stream));
+  }
   return CG_OK;
 }
 

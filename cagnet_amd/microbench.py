@@ -67,10 +67,15 @@ def run_spmm(args) -> None:
     torch.cuda.synchronize()
 
     def build(**kw):
-        t0 = time.perf_counter()
-        a = ops.CsrMatrix(**kw)
-        torch.cuda.synchronize()
-        return a, (time.perf_counter() - t0) * 1e3
+        best, a = float("inf"), None
+        for _ in range(3):
+            del a
+            torch.cuda.synchronize()  # the arguments may still be in the making (permuted copies)
+            t0 = time.perf_counter()
+            a = ops.CsrMatrix(**kw)
+            torch.cuda.synchronize()
+            best = min(best, (time.perf_counter() - t0) * 1e3)
+        return a, best
 
     build(row=r32, col=c32, val=val, n=n, m=n)  # first call also grows the scratch buffers
     _, t_sorted = build(row=r32, col=c32, val=val, n=n, m=n)

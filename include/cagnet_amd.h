@@ -80,6 +80,8 @@ int cg_coo_check(const int32_t *d_row, const int32_t *d_col, int64_t nnz, int32_
  * d_perm != NULL, d_perm[k] = input position of output entry k.  Result order equals
  * scipy.sparse.coo_matrix(...).tocsr() with sorted indices / torch .coalesce() on
  * duplicate-free input (what the reference's callers feed spmm_gpu: gcn_distr.py:546).
+ * d_colind may be d_col and d_values may be d_val (conversion in place; the inputs are otherwise
+ * left untouched); with d_perm the values are gathered by it, so d_values must then differ from d_val.
  * Allocates temporaries and synchronises `stream` before returning. */
 int cg_coo2csr(const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz, int32_t n, int32_t m,
                int32_t *d_rowptr, int32_t *d_colind, float *d_values, int32_t *d_perm, cg_stream_t stream);
@@ -87,8 +89,8 @@ int cg_coo2csr(const int32_t *d_row, const int32_t *d_col, const float *d_val, i
 /* CSR of A (n x m) -> CSR of A^T (m x n) == CSC of A: the precomputed operand of the A^T*G
  * backward product (the reference reuses A itself and so assumes symmetry, gcn_distr.py:326,
  * gcn_distr_2d.py:683).  Stable radix sort by column, so rows ascend inside each column.
- * d_perm (nullable): d_perm[k] = CSR position of transposed entry k.  Allocates temporaries
- * and synchronises `stream`. */
+ * d_perm (nullable): d_perm[k] = CSR position of transposed entry k.  d_rowind may be d_colind
+ * and, without d_perm, d_values_t may be d_values.  Allocates temporaries and synchronises `stream`. */
 int cg_csr_transpose(const int32_t *d_rowptr, const int32_t *d_colind, const float *d_values, int64_t nnz,
                      int32_t n, int32_t m, int32_t *d_colptr, int32_t *d_rowind, float *d_values_t,
                      int32_t *d_perm, cg_stream_t stream);

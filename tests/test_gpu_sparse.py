@@ -78,6 +78,43 @@ def test_csr_transpose_bit_exact_and_involution(cuda, n, m, nnz, seed):
     assert np.array_equal(vv2.cpu().numpy(), vv)
 
 
+@pytest.mark.parametrize("n,m,nnz,seed", [(1, 1, 1, 0), (13, 7, 40, 1), (200, 200, 20000, 6), (300, 70000, 50000, 2),
+                                          (1 << 17, 1 << 17, 600000, 5)])
+def test_conversions_without_permutation_and_in_place(cuda, n, m, nnz, seed):
+    """Without a permutation output the values travel with the records; without values the keys travel
+    alone; and outputs may be the input arrays themselves (a single-pass sort then goes through a copy)."""
+    from cagnet_amd import ops
+    from cagnet_amd._lib import lib
+    from cagnet_amd.ops import _ptr, _stream, check
+    row, col, val = random_coo(n, m, nnz, seed, sort=False)
+    erp, eci, evv, _ = orc.coo2csr(row.numpy(), col.numpy(), val.numpy(), n, m)
+    r, c, v = _i32(row, cuda), _i32(col, cuda), val.to(cuda)
+    rp, ci, vv = ops.coo2csr(r, c, v, n, m)
+    assert np.array_equal(rp.cpu().numpy(), erp) and np.array_equal(ci.cpu().numpy(), eci)
+    assert np.array_equal(vv.cpu().numpy(), evv)
+    rp0, ci0, none = ops.coo2csr(r, c, None, n, m)
+    assert none is None and torch.equal(rp0, rp) and torch.equal(ci0, ci)
+    assert torch.equal(r, _i32(row, cuda)) and torch.equal(c, _i32(col, cuda)) and torch.equal(v, val.to(cuda))  # inputs intact
+    # in place: colind and values land in the arrays that held col and val
+    c2, v2 = c.clone(), v.clone()
+    rp2 = torch.empty(n + 1, dtype=torch.int32, device=cuda)
+    check(lib.cg_coo2csr(_ptr(r), _ptr(c2), _ptr(v2), r.numel(), n, m, _ptr(rp2), _ptr(c2), _ptr(v2), None, _stream()),
+          "cg_coo2csr")
+    assert torch.equal(rp2, rp) and torch.equal(c2, ci) and torch.equal(v2, vv)
+    # transpose, the same three ways
+    ecp, eri, evt, _ = orc.csr_transpose(erp, eci, evv, n, m)
+    cp, ri, vt = ops.csr_transpose(rp, ci, vv, n, m)
+    assert np.array_equal(cp.cpu().numpy(), ecp) and np.array_equal(ri.cpu().numpy(), eri)
+    assert np.array_equal(vt.cpu().numpy(), evt)
+    cp0, ri0, none = ops.csr_transpose(rp, ci, None, n, m)
+    assert none is None and torch.equal(cp0, cp) and torch.equal(ri0, ri)
+    ci3, vv3 = ci.clone(), vv.clone()
+    cp3 = torch.empty(m + 1, dtype=torch.int32, device=cuda)
+    check(lib.cg_csr_transpose(_ptr(rp), _ptr(ci3), _ptr(vv3), ci3.numel(), n, m, _ptr(cp3), _ptr(ci3), _ptr(vv3), None,
+                               _stream()), "cg_csr_transpose")
+    assert torch.equal(cp3, cp) and torch.equal(ci3, ri) and torch.equal(vv3, vt)
+
+
 def test_coo_check_reports(cuda):
     from cagnet_amd import ops
     ok_r = torch.tensor([0, 0, 1, 2], dtype=torch.int32, device=cuda)
