@@ -123,6 +123,7 @@ constexpr int kSortRounds = 16;                          // keys per lane
 constexpr int kSortWaveTile = kSortRounds * kWave;       // 1024 consecutive keys per wave
 constexpr int kSortTile = kSortWaves * kSortWaveTile;    // 4096 keys per workgroup
 constexpr int kRadix = 256;
+constexpr int kXcds = 8;
 
 // hist[digit * tiles + tile] = number of keys of this tile with that digit
 __global__ __launch_bounds__(kSortThreads) void radix_hist_kernel(const int32_t *__restrict__ key, int64_t count,
@@ -132,13 +133,18 @@ __global__ __launch_bounds__(kSortThreads) void radix_hist_kernel(const int32_t 
   lh[threadIdx.x] = 0;
   __syncthreads();
   const int64_t base = (int64_t)blockIdx.x * kSortTile;
+  // every load is issued before the first count (unconditional, clamped index: a load behind a branch
+  // would make each of the 16 steps wait for its own round trip)
+  uint32_t k[kSortTile / kSortThreads];
 #pragma unroll
   for (int i = 0; i < kSortTile / kSortThreads; ++i) {
-    int64_t idx = base + (int64_t)i * kSortThreads + threadIdx.x;
-    if (idx < count) {
-      uint32_t d = ((uint32_t)key[idx] >> shift) & ((1u << dbits) - 1u);
-      atomicAdd(&lh[d], 1u);  // integer LDS atomic: the count does not depend on arrival order
-    }
+    const int64_t idx = base + (int64_t)i * kSortThreads + threadIdx.x;
+    k[i] = (uint32_t)key[idx < count ? idx : count - 1];
+  }
+#pragma unroll
+  for (int i = 0; i < kSortTile / kSortThreads; ++i) {
+    const int64_t idx = base + (int64_t)i * kSortThreads + threadIdx.x;
+    if (idx < count) atomicAdd(&lh[(k[i] >> shift) & ((1u << dbits) - 1u)], 1u);  // integer LDS atomic: order independent
   }
   __syncthreads();
   if ((int)threadIdx.x < (1 << dbits)) hist[(int64_t)threadIdx.x * tiles + blockIdx.x] = lh[threadIdx.x];
@@ -165,7 +171,9 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const uint64_t lt_mask = (1ull << lane) - 1ull;
-  const int64_t tile = blockIdx.x;
+  const int64_t per_xcd = (tiles + kXcds - 1) / kXcds;
+  const int64_t tile = (int64_t)(blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
+  if (tile >= tiles) return;  // whole workgroup
   const int64_t tile_base = tile * kSortTile;
   const int64_t base = tile_base + (int64_t)wave * kSortWaveTile;
   const uint32_t dmask = (1u << dbits) - 1u;
@@ -173,17 +181,34 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
   int32_t ra[kSortRounds], rb[kSortRounds], rp[kSortRounds];
   uint32_t packed[kSortRounds];  // digit | rank among the wave's records of that digit << 8
 
+  // All loads of the tile are issued before the first record is ranked: keys first, payload last.
+  // They are unconditional (index clamped to the last record, dead lanes are masked where the value
+  // is used), because a load behind a branch makes the compiler wait for all outstanding loads and
+  // each of the 16 rounds would then pay a full memory round trip.
+  const int64_t last = count - 1;
+  const int32_t *__restrict__ src_p = in_p ? in_p : in_a;  // no payload array: the position is the payload
+#pragma unroll
+  for (int r = 0; r < kSortRounds; ++r) {
+    const int64_t idx = base + (int64_t)r * kWave + lane;
+    const int64_t cidx = idx < last ? idx : last;
+    ra[r] = in_a[cidx];
+    rb[r] = in_b[cidx];
+  }
+#pragma unroll
+  for (int r = 0; r < kSortRounds; ++r) {
+    const int64_t idx = base + (int64_t)r * kWave + lane;
+    const int64_t cidx = idx < last ? idx : last;
+    const int32_t v = src_p[cidx];
+    rp[r] = in_p ? v : (int32_t)idx;
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
 #pragma unroll
   for (int r = 0; r < kSortRounds; ++r) {
     const int64_t idx = base + (int64_t)r * kWave + lane;
     const bool valid = idx < count;
     uint32_t d = 0;
-    if (valid) {
-      ra[r] = in_a[idx];
-      rb[r] = in_b[idx];
-      rp[r] = in_p ? in_p[idx] : (int32_t)idx;
-      d = ((uint32_t)(key_is_a ? ra[r] : rb[r]) >> shift) & dmask;
-    }
+    if (valid) d = ((uint32_t)(key_is_a ? ra[r] : rb[r]) >> shift) & dmask;
     uint64_t peers = __ballot(valid);
 #pragma unroll
     for (int bit = 0; bit < 8; ++bit) {
@@ -281,7 +306,8 @@ static int sort_pass(const SortPass &ps, const int32_t *in_a, const int32_t *in_
                                                                   hist, tiles);
   CG_LAUNCH_CHECK();
   CG_TRY(exclusive_scan_u32(hist, hist, tiles << ps.dbits, nullptr, stream));
-  radix_scatter_kernel<<<(unsigned)tiles, kSortThreads, 0, stream>>>(ps.which, ps.shift, ps.dbits, in_a, in_b, in_p, out_a,
+  const int64_t grid = (tiles + kXcds - 1) / kXcds * kXcds;
+  radix_scatter_kernel<<<(unsigned)grid, kSortThreads, 0, stream>>>(ps.which, ps.shift, ps.dbits, in_a, in_b, in_p, out_a,
                                                                      out_b, out_p, count, hist, tiles);
   CG_LAUNCH_CHECK();
   return CG_OK;
