@@ -56,6 +56,22 @@ __device__ __forceinline__ void store_vec(float *p, const float (&r)[VEC]) {
   *reinterpret_cast<V *>(p) = t;
 }
 
+// p[0] + p[f] + ... + p[(nseg - 1) f] in that order.  The longest rows of a power-law graph have
+// hundreds of segments and one lane adds them all: the loads go out eight at a time.
+__device__ __forceinline__ float sum_segments(const float *__restrict__ p, int32_t nseg, int32_t f) {
+  float s = 0.f;
+  int32_t i = 0;
+  for (; i + 8 <= nseg; i += 8) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = p[(int64_t)(i + u) * f];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s += v[u];
+  }
+  for (; i < nseg; ++i) s += p[(int64_t)i * f];
+  return s;
+}
+
 // C[row, :] = beta*C[row, :] + sum over the row's partial rows, in segment order.
 __global__ __launch_bounds__(kSpmmThreads) void spmm_reduce_kernel(const int32_t *__restrict__ multi_rows,
                                                                    int64_t nmulti_host,
@@ -79,8 +95,7 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_reduce_kernel(const int32_t
   const int32_t nseg = (deg + seg - 1) / seg;
   if (p_cap > 0 && (int64_t)pbase[row] + nseg > p_cap) return;  // only a malformed (unsorted) input gets here
   const float *p = P + (int64_t)pbase[row] * f + col;
-  float s = 0.f;
-  for (int32_t i = 0; i < nseg; ++i) s += p[(int64_t)i * f];
+  float s = sum_segments(p, nseg, f);
   if (fold_tbase) {  // same fold as in the main kernel, for rows that were split
     for (int32_t cls = 0; cls < fold_classes; ++cls) {
       const int32_t *tb = fold_tbase + (int64_t)cls * fold_rows + row;
@@ -205,8 +220,7 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_reduce_epi_kernel(const Red
   float *rowbuf = epi_lds + ((size_t)a.epi_fop + wave) * epi_fpad(a.f);
   for (int32_t col = lane; col < a.f; col += kWave) {
     const float *p = a.P + (int64_t)a.pbase[row] * a.f + col;
-    float s = 0.f;
-    for (int32_t i = 0; i < nseg; ++i) s += p[(int64_t)i * a.f];
+    float s = sum_segments(p, nseg, a.f);
     if (a.fold_tbase) {
       for (int32_t cls = 0; cls < a.fold_classes; ++cls) {
         const int32_t *tb = a.fold_tbase + (int64_t)cls * a.fold_rows + row;
@@ -605,14 +619,19 @@ __global__ __launch_bounds__(kSpmmThreads) void hub_reduce_kernel(const int32_t 
   for (int32_t c0 = 0; c0 < f; c0 += kWave) {
     const int32_t col = c0 + lane;
     if (col < f) {
+      // the first partial row of every class is loaded before anything is added (classes without one
+      // read slot 0, which exists because total > 0, and are skipped in the sum); classes with more
+      // than one partial row (rows split into segments) add the rest in order
+      float v[NC];
+#pragma unroll
+      for (int g = 0; g < NC; ++g) v[g] = P[(int64_t)(count[g] > 0 ? first[g] : 0) * f + col];
       float s = 0.f;
 #pragma unroll
       for (int g = 0; g < NC; ++g) {
-        const float *p = P + (int64_t)first[g] * f + col;
-        if (count[g] == 1) {
-          s += p[0];
-        } else {
-          for (int32_t t = 0; t < count[g]; ++t) s += p[(int64_t)t * f];
+        if (count[g] > 0) s += v[g];
+        if (count[g] > 1) {
+          const float *p = P + (int64_t)first[g] * f + col;
+          for (int32_t t = 1; t < count[g]; ++t) s += p[(int64_t)t * f];
         }
       }
       crow[col] += s;
