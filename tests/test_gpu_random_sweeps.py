@@ -1,0 +1,192 @@
+"""Seeded random sweeps over shapes, strides and schedule knobs.  torch on the same device is the
+independent party: fp64 dense products for the floating-point kernels (bound: REL_TOL of the
+magnitude sum), sort / searchsorted / boolean masks for the integer kernels (bit-exact).  Every input is
+valid; the sweeps look for shape and knob combinations the hand-written cases do not name."""
+import random
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from cagnet_amd import synth
+from tests.util import REL_TOL
+
+pytestmark = pytest.mark.gpu
+
+SPMM_KNOBS = [b"spmm_seg", b"spmm_win", b"spmm_vec", b"spmm_hub", b"spmm_hub_kb", b"spmm_hub_groups",
+              b"spmm_hub_tiers", b"spmm_hub_row"]
+
+
+@pytest.fixture
+def knobs_restored():
+    from cagnet_amd._lib import lib
+    yield lib
+    for key in SPMM_KNOBS + [b"dense_mfma"]:
+        lib.cg_tune_set(key, 0)
+
+
+def _rel(got, ref, mag):
+    return float(((got.double() - ref).abs() / mag.clamp_min(1e-30)).max()) if ref.numel() else 0.0
+
+
+def _strided(rows, cols, extra, gen, dev):
+    return torch.randn(rows, cols + extra, device=dev, generator=gen)[:, :cols]
+
+
+@pytest.mark.parametrize("seed", [11, 12])
+def test_spmm_schedules_random(cuda, knobs_restored, seed):
+    """Handle, one-shot and digest-cached products over random patterns (empty, sparse, nearly dense,
+    with full rows and full columns), widths of every kernel family, both sides, accumulate forms,
+    padded leading dimensions and random schedule knobs (segment and window lengths, vector cap,
+    hub plans with 1 to 8 tiers over 1 to 8 groups and several row thresholds)."""
+    from cagnet_amd import ops
+    lib = knobs_restored
+    rng = random.Random(seed)
+    for case in range(120):
+        n = rng.choice([1, 7, 63, 64, 65, 300, 1000, 4097])
+        m = rng.choice([1, 5, 64, 129, 1000, 3001])
+        dens = rng.choice([0.0, 0.002, 0.02, 0.2, 0.9])
+        f = rng.choice([1, 2, 3, 4, 8, 16, 24, 41, 44, 64, 100, 128, 130, 256, 300, 301, 602, 640, 644, 1300, 2562])
+        g = torch.Generator().manual_seed(rng.randrange(1 << 30))
+        mask = torch.rand(n, m, generator=g) < dens
+        if rng.random() < 0.5 and n > 2:
+            mask[rng.randrange(n)] = True
+            mask[:, rng.randrange(m)] = True
+        dense = torch.where(mask, torch.randn(n, m, generator=g), torch.zeros(()))
+        idx = mask.nonzero()
+        row, col, val = idx[:, 0].int().to(cuda), idx[:, 1].int().to(cuda), dense[mask].to(cuda)
+        values = [rng.choice([0, 64, 100, 512, 1024, 4096]), rng.choice([0, 64, 200, 512]), rng.choice([0, 1, 2]),
+                  rng.choice([-1, 0, 1, 1, 1]), rng.choice([0, 1, 4, 64]), rng.choice([0, 1, 2, 4, 8]),
+                  rng.choice([0, 1, 2, 3, 6, 8]), rng.choice([0, 1, 8, 64, 1000])]
+        for key, v in zip(SPMM_KNOBS, values):
+            assert lib.cg_tune_set(key, v) == 0
+        tr = rng.random() < 0.4
+        beta = rng.choice([0.0, 1.0, 1.0, -0.5])
+        extra_b, extra_c = rng.choice([0, 0, 1, 4]), rng.choice([0, 0, 2, 4])
+        what = f"seed {seed} case {case}: n={n} m={m} nnz={val.numel()} f={f} tr={tr} beta={beta} ld+{extra_b}/{extra_c} knobs={values}"
+        gen = torch.Generator(device=cuda).manual_seed(case)
+        B = _strided(n if tr else m, f, extra_b, gen, cuda)
+        C0 = torch.randn(m if tr else n, f, device=cuda, generator=gen)
+        A = ops.CsrMatrix(row, col, val, n, m, is_sorted=True, transpose=tr)
+        outs = []
+        for _ in range(2):
+            C = torch.empty(C0.shape[0], f + extra_c, device=cuda)[:, :f].copy_(C0)
+            A.spmm(B, out=C, beta=beta, transpose=tr)
+            outs.append(C)
+        A64 = dense.double().to(cuda)
+        A64 = A64.t() if tr else A64
+        ref = beta * C0.double() + A64 @ B.double()
+        mag = abs(beta) * C0.double().abs() + A64.abs() @ B.double().abs()
+        assert _rel(outs[0], ref, mag) <= REL_TOL, what
+        assert torch.equal(outs[0], outs[1]), what
+        if not tr and val.numel() > 0:
+            ref1 = C0.double() + A64 @ B.double()
+            mag1 = C0.double().abs() + A64.abs() @ B.double().abs()
+            for cached in (False, True):
+                C = C0.clone()
+                ops.spmm_coo(row, col, val, n, m, B.contiguous(), C, cached=cached)
+                assert _rel(C, ref1, mag1) <= REL_TOL, f"{what} one-shot cached={cached}"
+        del A
+    ops.coo_cache_clear()
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_dense_and_rowwise_random(cuda, knobs_restored, seed):
+    """The three dense products (both kernel families) on strided operands and outputs, and the
+    row-wise kernels, over random n, k and output widths from 1 to 100."""
+    from cagnet_amd import ops
+    lib = knobs_restored
+    rng = random.Random(seed)
+    for case in range(150):
+        n = rng.choice([1, 2, 15, 16, 17, 63, 64, 65, 255, 1000, 4099, 70001])
+        k = rng.choice([1, 2, 3, 4, 7, 16, 31, 64, 65, 100, 128, 300, 301, 302, 320, 322, 602, 640, 700, 1026])
+        fo = rng.choice([1, 2, 3, 7, 8, 16, 17, 24, 32, 41, 44, 64, 65, 100])
+        ex = [rng.choice([0, 0, 1, 2, 4]) for _ in range(6)]
+        assert lib.cg_tune_set(b"dense_mfma", rng.choice([0, 0, 0, -1])) == 0
+        relu = rng.random() < 0.5
+        what = f"seed {seed} case {case}: n={n} k={k} fo={fo} extras={ex} relu={relu}"
+        gen = torch.Generator(device=cuda).manual_seed(case)
+        X, W, G = _strided(n, k, ex[0], gen, cuda), _strided(k, fo, ex[1], gen, cuda), _strided(n, fo, ex[2], gen, cuda)
+        Xd, Wd, Gd = X.double(), W.double(), G.double()
+        Z = torch.empty(n, fo + ex[3], device=cuda)[:, :fo]
+        ops.dense_xw(X, W, relu=relu, out=Z)
+        ref = (Xd @ Wd).clamp_min(0) if relu else Xd @ Wd
+        assert _rel(Z, ref, Xd.abs() @ Wd.abs()) <= REL_TOL, what + " xw"
+        dX = torch.empty(n, k + ex[4], device=cuda)[:, :k]
+        ops.dense_gwt(G, W, out=dX)
+        assert _rel(dX, Gd @ Wd.t(), Gd.abs() @ Wd.abs().t()) <= REL_TOL, what + " gwt"
+        dW = [torch.empty(k, fo + ex[5], device=cuda)[:, :fo] for _ in range(2)]
+        for out in dW:
+            ops.dense_xtg(X, G, out=out)
+        assert _rel(dW[0], Xd.t() @ Gd, Xd.abs().t() @ Gd.abs()) <= REL_TOL, what + " xtg"
+        assert torch.equal(dW[0], dW[1]), what + " xtg repeat"
+        Zc = G.contiguous()
+        lp = ops.log_softmax_fwd(Zc)
+        assert float((lp.double() - F.log_softmax(Zc.double(), dim=1)).abs().max()) <= 2e-6 * max(1.0, float(Zc.abs().max())), what
+        go = torch.randn(n, fo, device=cuda, generator=gen)
+        gi = ops.log_softmax_bwd(go, lp)
+        p = torch.exp(lp.double())
+        refg = go.double() - p * go.double().sum(dim=1, keepdim=True)
+        magg = go.double().abs() + p * go.double().abs().sum(dim=1, keepdim=True)
+        assert _rel(gi, refg, magg) <= REL_TOL, what + " log_softmax_bwd"
+        h = ops.relu_fwd(Zc)
+        assert torch.equal(h, Zc.clamp_min(0)), what
+        assert torch.equal(ops.relu_bwd(go, h), go * (h > 0)), what
+        y = torch.randint(0, fo, (n,), device=cuda, generator=gen)
+        mask = torch.rand(n, device=cuda, generator=gen) < 0.6
+        loss, count = ops.nll_loss_fwd(lp, y, mask)
+        cnt = int(mask.sum())
+        assert int(count) == cnt, what
+        refl = float(-(lp.double()[mask, y[mask]]).sum() / cnt) if cnt else 0.0
+        assert abs(float(loss) - refl) <= 1e-5 * max(1.0, abs(refl)), what + " nll"
+
+
+@pytest.mark.parametrize("seed", [31])
+def test_conversions_and_preparation_random(cuda, seed):
+    """COO in arbitrary order -> CSR, transposes (with and without the permutation), block extraction,
+    self-loops and normalisation, bit for bit against sort / searchsorted / masks."""
+    from cagnet_amd import ops
+    rng = random.Random(seed)
+    for case in range(150):
+        n = rng.choice([1, 2, 5, 64, 255, 256, 257, 1000, 65536, 70001, 300000])
+        m = rng.choice([1, 3, 64, 255, 256, 257, 4097, 65537, 262145]) if rng.random() < 0.5 else n
+        cap = n * m
+        nnz = min(cap, rng.choice([0, 1, 5, 1000, 4096, 4097, 100000, 1500000]))
+        gen = torch.Generator(device=cuda).manual_seed(case * 7 + 1)
+        if cap <= 4_000_000:
+            key = torch.randperm(cap, device=cuda, generator=gen)[:nnz]
+        else:
+            key = torch.unique(torch.randint(0, cap, (nnz,), device=cuda, generator=gen))
+            key = key[torch.randperm(key.numel(), device=cuda, generator=gen)]
+        nnz = key.numel()
+        row, col = (key // m).int(), (key % m).int()
+        val = torch.randn(nnz, device=cuda, generator=gen)
+        what = f"seed {seed} case {case}: n={n} m={m} nnz={nnz}"
+        order = torch.sort(key, stable=True).indices
+        srow, scol, sval = row[order], col[order], val[order]
+        want_rp = torch.searchsorted(srow.long(), torch.arange(n + 1, device=cuda)).int()
+        rp, ci, vv, perm = ops.coo2csr(row, col, val, n, m, return_perm=True)
+        assert torch.equal(rp, want_rp) and torch.equal(ci, scol) and torch.equal(vv, sval), what
+        assert torch.equal(perm.long(), order), what
+        rp, ci, vv = ops.coo2csr(row, col, val, n, m)
+        assert torch.equal(rp, want_rp) and torch.equal(ci, scol) and torch.equal(vv, sval), what
+        assert torch.equal(ops.coo2csr_rowptr(srow, n), want_rp), what
+        torder = torch.sort(scol.long() * n + srow.long(), stable=True).indices
+        want_cp = torch.searchsorted(scol[torder].long(), torch.arange(m + 1, device=cuda)).int()
+        cp, ri, vt, tperm = ops.csr_transpose(rp, ci, vv, n, m, return_perm=True)
+        assert torch.equal(cp, want_cp) and torch.equal(ri, srow[torder]) and torch.equal(vt, sval[torder]), what
+        assert torch.equal(tperm.long(), torder), what
+        cp, ri, vt = ops.csr_transpose(rp, ci, vv, n, m)
+        assert torch.equal(cp, want_cp) and torch.equal(ri, srow[torder]) and torch.equal(vt, sval[torder]), what
+        r0, r1 = sorted((rng.randrange(n + 1), rng.randrange(n + 1)))
+        c0, c1 = sorted((rng.randrange(m + 1), rng.randrange(m + 1)))
+        br, bc, bv = ops.coo_block(srow, scol, sval, r0, r1, c0, c1)
+        inside = (srow >= r0) & (srow < r1) & (scol >= c0) & (scol < c1)
+        assert torch.equal(br, srow[inside] - r0) and torch.equal(bc, scol[inside] - c0), what
+        assert torch.equal(bv, sval[inside]), what
+        if n == m:
+            lr, lc = ops.add_self_loops(srow, scol, n)
+            diag = torch.arange(n, device=cuda)
+            allk = torch.unique(torch.cat([srow.long() * n + scol.long(), diag * n + diag]))
+            assert torch.equal(lr.long(), allk // n) and torch.equal(lc.long(), allk % n), what
+            assert torch.equal(ops.gcn_normalize(lr, lc, n), synth.gcn_normalize(lr.long(), lc.long(), n)), what
