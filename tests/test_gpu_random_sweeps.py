@@ -190,3 +190,54 @@ def test_conversions_and_preparation_random(cuda, seed):
             allk = torch.unique(torch.cat([srow.long() * n + scol.long(), diag * n + diag]))
             assert torch.equal(lr.long(), allk // n) and torch.equal(lc.long(), allk % n), what
             assert torch.equal(ops.gcn_normalize(lr, lc, n), synth.gcn_normalize(lr.long(), lc.long(), n)), what
+
+
+@pytest.mark.parametrize("seed", [41])
+def test_fused_layer_product_random(cuda, knobs_restored, seed):
+    """Z = act((acc + op(A) B) W) in one pass, over random patterns, widths with and without a fused
+    form (those must answer None, not compute), sides, accumulators and schedule knobs."""
+    from cagnet_amd import ops
+    lib = knobs_restored
+    rng = random.Random(seed)
+    fused = 0
+    for case in range(200):
+        n = rng.choice([1, 7, 64, 65, 300, 1000, 4097])
+        m = rng.choice([1, 5, 64, 129, 1000, 3001])
+        dens = rng.choice([0.0, 0.002, 0.02, 0.2, 0.9])
+        f = rng.choice([16, 64, 100, 128, 130, 256, 257, 300, 301, 512, 602, 640, 644, 1000, 1300])
+        fo = rng.choice([1, 2, 7, 8, 16, 17, 24, 32, 41, 64, 65])
+        g = torch.Generator().manual_seed(rng.randrange(1 << 30))
+        mask = torch.rand(n, m, generator=g) < dens
+        if rng.random() < 0.5 and n > 2:
+            mask[rng.randrange(n)] = True
+            mask[:, rng.randrange(m)] = True
+        dense = torch.where(mask, torch.randn(n, m, generator=g), torch.zeros(()))
+        idx = mask.nonzero()
+        row, col, val = idx[:, 0].int().to(cuda), idx[:, 1].int().to(cuda), dense[mask].to(cuda)
+        values = [rng.choice([0, 64, 100, 512, 1024]), rng.choice([0, 64, 200, 512]), rng.choice([0, 1, 2]),
+                  rng.choice([-1, 0, 1, 1]), rng.choice([0, 1, 4, 64]), rng.choice([0, 1, 2, 4, 8]),
+                  rng.choice([0, 1, 2, 3, 6]), rng.choice([0, 1, 8, 64])]
+        for key, v in zip(SPMM_KNOBS, values):
+            assert lib.cg_tune_set(key, v) == 0
+        tr, relu, use_acc = rng.random() < 0.3, rng.random() < 0.5, rng.random() < 0.4
+        what = f"seed {seed} case {case}: n={n} m={m} nnz={val.numel()} f={f} fo={fo} tr={tr} relu={relu} acc={use_acc} knobs={values}"
+        gen = torch.Generator(device=cuda).manual_seed(case)
+        rows_b, rows_c = (n, m) if tr else (m, n)
+        B = _strided(rows_b, f, rng.choice([0, 0, 4]), gen, cuda)
+        W = _strided(f, fo, rng.choice([0, 0, 3]), gen, cuda)
+        acc = torch.randn(rows_c, f, device=cuda, generator=gen) if use_acc else None
+        A = ops.CsrMatrix(row, col, val, n, m, is_sorted=True, transpose=tr)
+        Z = A.spmm_xw(B, W, relu=relu, acc=acc, transpose=tr)
+        if Z is None:
+            continue
+        fused += 1
+        assert torch.equal(Z, A.spmm_xw(B, W, relu=relu, acc=acc, transpose=tr)), what
+        A64 = dense.double().to(cuda)
+        A64 = A64.t() if tr else A64
+        inner = A64 @ B.double() + (acc.double() if use_acc else 0)
+        inner_mag = A64.abs() @ B.double().abs() + (acc.double().abs() if use_acc else 0)
+        ref = inner @ W.double()
+        ref = ref.clamp_min(0) if relu else ref
+        # two roundings in a row (the row of A B, then its product with W): twice the bound of one
+        assert _rel(Z, ref, inner_mag @ W.double().abs()) <= 2 * REL_TOL, what
+    assert fused >= 60
