@@ -260,3 +260,45 @@ def train(inputs, weight1, weight2, adj_matrix, am_partitions, optimizer, data, 
 
 
 train.last_loss = None
+
+
+class GraphedTrain:
+    """`train` captured once into a HIP graph and replayed: one launch per epoch instead of some
+    forty.  On graphs of a few thousand vertices an epoch is bound by launches and host work, not
+    by kernels (4,096 vertices: 0.69 ms per eager epoch); on the large configurations it changes
+    nothing measurable.  The reference has no counterpart (its epoch synchronises the device in
+    every spmm_gpu call, sparse_coo_tensor.cu:229-231).
+
+    The library's scratch buffers are cached per stream, so warm-up, capture and replay all use
+    one private stream.  The constructor runs `warmup` ordinary epochs there (they train: weights
+    and optimizer state advance) and then records one more epoch without executing it; `step()`
+    replays it.  Every tensor the epoch reads (`inputs`, the weights, `data.y`, `data.train_mask`)
+    is read from the same memory on every replay: update them in place.  Optimizers that keep
+    scalars on the host must be built for capture (`torch.optim.Adam(..., capturable=True)`)."""
+
+    def __init__(self, inputs, weight1, weight2, adj_matrix, am_partitions, optimizer, data, rank=0, size=1,
+                 group=None, warmup: int = 3):
+        if warmup < 1:
+            raise ValueError("at least one warm-up epoch is needed: it builds the schedules and grows the scratch")
+        args = (inputs, weight1, weight2, adj_matrix, am_partitions, optimizer, data, rank, size, group)
+        self.stream = torch.cuda.Stream(device=weight1.device)
+        self.stream.wait_stream(torch.cuda.current_stream(weight1.device))
+        with torch.cuda.stream(self.stream):
+            for _ in range(warmup):
+                train(*args)
+                inputs.grad = None
+        torch.cuda.current_stream(weight1.device).wait_stream(self.stream)
+        torch.cuda.synchronize(weight1.device)
+        optimizer.zero_grad(set_to_none=True)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph, stream=self.stream):
+            self.outputs = train(*args)
+            self.loss = train.last_loss
+        self.epochs_run = warmup
+
+    def step(self) -> torch.Tensor:
+        """One more epoch.  Returns the epoch's outputs (the same tensor every time; `self.loss`
+        likewise holds the epoch's loss after the replay has run)."""
+        self.graph.replay()
+        self.epochs_run += 1
+        return self.outputs

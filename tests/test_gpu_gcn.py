@@ -239,3 +239,51 @@ def test_forward_backward_replays_in_a_hip_graph(cuda):
     assert abs(float(outs[0]) - float(ref["loss"])) <= LOSS_TOL
     _close(outs[1], ref["dw1"], "dw1 from the graph")
     _close(outs[2], ref["dw2"], "dw2 from the graph")
+
+
+@pytest.mark.parametrize("optimizer", ["sgd", "adam"])
+def test_graphed_train_matches_eager_epochs(cuda, optimizer):
+    """`GraphedTrain` (warm-up epochs, then one captured epoch replayed) against the same number of
+    eager epochs of `train` on a twin model: the loss of every epoch and the weights after it must
+    agree bit for bit, with eager work and synchronisations between the replays."""
+    from cagnet_amd import gcn, ops
+    p = synth.make_problem(scale=12, n_edges=32768, features=128, hidden=16, classes=8, mask_fraction=0.7, seed=9,
+                           device=cuda)
+    blk = ops.CsrMatrix(p.row.int(), p.col.int(), p.val, p.n, p.n, transpose=True)
+
+    class Data:
+        y = p.y
+        train_mask = p.train_mask
+
+    def model():
+        w1, w2 = p.w1.clone().requires_grad_(True), p.w2.clone().requires_grad_(True)
+        x = p.x.clone().requires_grad_(True)
+        opt = (torch.optim.SGD([w1, w2], lr=0.01) if optimizer == "sgd"
+               else torch.optim.Adam([w1, w2], lr=0.01, capturable=True))
+        return x, w1, w2, opt
+
+    xe, w1e, w2e, opte = model()
+    xg, w1g, w2g, optg = model()
+    warm = 2
+    graphed = gcn.GraphedTrain(xg, w1g, w2g, p.n, [blk], optg, Data, warmup=warm)
+    for _ in range(warm):
+        gcn.train(xe, w1e, w2e, p.n, [blk], opte, Data)
+        xe.grad = None
+    torch.cuda.synchronize()
+    assert torch.equal(w1e, w1g) and torch.equal(w2e, w2g)
+    losses = []
+    for epoch in range(5):
+        out_e = gcn.train(xe, w1e, w2e, p.n, [blk], opte, Data)          # eager work between the replays
+        loss_e = float(gcn.train.last_loss)
+        dx_e = xe.grad.clone()
+        xe.grad = None
+        torch.cuda.synchronize()
+        out_g = graphed.step()
+        torch.cuda.synchronize()
+        assert float(graphed.loss) == loss_e, f"epoch {epoch}"
+        assert torch.equal(out_g, out_e), f"epoch {epoch}"
+        assert torch.equal(w1g, w1e) and torch.equal(w2g, w2e), f"epoch {epoch}"
+        assert torch.equal(xg.grad, dx_e), f"epoch {epoch}"
+        losses.append(loss_e)
+    assert losses[-1] < losses[0]
+    assert graphed.epochs_run == warm + 5
