@@ -265,13 +265,14 @@ int cg_coo_block(const int32_t *d_row, const int32_t *d_col, const float *d_val,
  * gcn_distr.py:66-94; here HIP events are recorded on the launch stream around single kernels).
  * cg_prof_enable(1) starts recording, cg_prof_enable(0) stops.  cg_prof_read waits for the
  * recorded events of `name`, returns their summed duration in milliseconds and their number, and
- * forgets them.  Names, the SpMM ones tagged by the product's width ("spmm_rowseg/f=602") and the
- * dense ones by the reduction length ("dense_xw/k=602"): "spmm_rowseg" (the main kernel of a
+ * forgets them.  A record's name ends in "/f=<number>": the width of an SpMM product
+ * ("spmm_rowseg/f=602"), the reduction length k of a dense product ("dense_xw/f=602"), the number
+ * of classes of a row-wise kernel.  Names: "spmm_rowseg" (the main kernel of a
  * product, or the cold class of a hub plan), "spmm_hub_hot" (all hot tiers of a hub plan as one
  * record), "spmm_reduce" (rows split into segments), "spmm_hub_reduce" (partial rows of a hub plan
  * with narrow teams), "dense_xw", "dense_gwt", "dense_xtg" (partial products and their sum),
- * "relu_fwd", "relu_bwd" (no tag), "log_softmax_fwd", "log_softmax_bwd", "nll_fwd", "nll_bwd",
- * "log_softmax_nll_bwd" (tagged "/f=" by the number of classes).
+ * "relu_fwd", "relu_bwd" (no suffix), "log_softmax_fwd", "log_softmax_bwd", "nll_fwd", "nll_bwd",
+ * "log_softmax_nll_bwd".
  * Recording is off by default and costs nothing then.
  */
 int cg_prof_enable(int on);
