@@ -241,3 +241,42 @@ def test_fused_layer_product_random(cuda, knobs_restored, seed):
         # two roundings in a row (the row of A B, then its product with W): twice the bound of one
         assert _rel(Z, ref, inner_mag @ W.double().abs()) <= 2 * REL_TOL, what
     assert fused >= 60
+
+
+@pytest.mark.parametrize("seed", [51])
+def test_two_layer_forward_backward_random(cuda, monkeypatch, seed):
+    """GCNFunc twice + masked NLL + backward over random graph sizes and densities, feature, hidden and
+    class widths, mask fractions (including an empty mask), product orders, fusion and with or without a
+    stored transpose, against the fp64 CPU oracle of the same pass."""
+    from cagnet_amd import gcn, ops
+    from oracle import gcn_oracle as orc
+    from tests.util import LOSS_TOL
+    rng = random.Random(seed)
+
+    def rel(got, ref64):
+        return float((got.detach().cpu().double() - ref64).abs().max()) / max(float(ref64.abs().max()), 1e-30)
+
+    for case in range(40):
+        n = rng.choice([33, 100, 257, 1000, 3000])
+        nnz = max(n, min(n * n // 2, rng.choice([n, 4 * n, 20 * n, 100 * n])))
+        f = rng.choice([1, 3, 16, 64, 100, 128, 300, 301, 602])
+        hidden = rng.choice([1, 4, 16, 17, 32, 64])
+        classes = rng.choice([2, 7, 8, 24, 41, 64])
+        frac = rng.choice([0.0, 0.3, 0.66, 1.0])
+        fused, first, tr = rng.random() < 0.5, rng.random() < 0.7, rng.random() < 0.5
+        monkeypatch.setattr(gcn, "fused_forward", fused)
+        monkeypatch.setattr(gcn, "spmm_first", first)
+        what = f"seed {seed} case {case}: n={n} nnz~{nnz} f={f} hidden={hidden} classes={classes} mask={frac} fused={fused} spmm_first={first} transpose={tr}"
+        p = synth.make_problem(n=n, target_nnz=nnz, features=f, hidden=hidden, classes=classes, mask_fraction=frac, seed=case)
+        A = orc.coo_tensor(p.row, p.col, p.val, p.n, p.n, torch.float64)
+        ref = orc.forward_backward(p.x, p.w1, p.w2, [A], p.y, p.train_mask, dtype=torch.float64)
+        blk = ops.CsrMatrix(p.row.int().to(cuda), p.col.int().to(cuda), p.val.to(cuda), p.n, p.n, transpose=tr)
+        x, w1, w2 = (t.to(cuda).requires_grad_(True) for t in (p.x, p.w1, p.w2))
+        h = gcn.GCNFunc.apply(x, w1, p.n, [blk], 0, 1, None, F.relu)
+        out = gcn.GCNFunc.apply(h, w2, p.n, [blk], 0, 1, None, F.log_softmax)
+        loss = gcn.masked_nll_loss(out, p.y.to(cuda), p.train_mask.to(cuda))
+        loss.backward()
+        assert abs(float(loss.detach()) - float(ref["loss"])) <= LOSS_TOL, what
+        for name, got, want in (("hidden", h, ref["hidden"]), ("outputs", out, ref["outputs"]), ("dw1", w1.grad, ref["dw1"]),
+                                ("dw2", w2.grad, ref["dw2"]), ("dx", x.grad, ref["dx"])):
+            assert rel(got, want) <= 2e-4, f"{what}: {name}"   # several chained products: relative to the largest entry
