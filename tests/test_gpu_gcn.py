@@ -287,3 +287,33 @@ def test_graphed_train_matches_eager_epochs(cuda, optimizer):
         losses.append(loss_e)
     assert losses[-1] < losses[0]
     assert graphed.epochs_run == warm + 5
+
+
+def test_activations_off_is_the_plain_linear_model(cuda, monkeypatch):
+    """The reference runs with its activations switched off unless asked otherwise (module global,
+    gcn_distr.py:57, :284-294): GCNFunc then returns Z itself for every `func`, and backward passes the
+    gradient through unchanged.  Checked against autograd over the dense fp64 composition."""
+    from cagnet_amd import gcn
+    monkeypatch.setattr(gcn, "activations", False)
+    p = synth.make_problem(scale=10, n_edges=6000, features=64, hidden=16, classes=8, mask_fraction=0.5, seed=4)
+    blk = _block(p, cuda, transpose=True)
+    x = p.x.to(cuda).requires_grad_(True)
+    w1 = p.w1.to(cuda).requires_grad_(True)
+    w2 = p.w2.to(cuda).requires_grad_(True)
+    h = gcn.GCNFunc.apply(x, w1, p.n, [blk], 0, 1, None, F.relu)
+    out = gcn.GCNFunc.apply(h, w2, p.n, [blk], 0, 1, None, F.log_softmax)
+    loss = gcn.masked_nll_loss(out, p.y.to(cuda), p.train_mask.to(cuda))
+    loss.backward()
+
+    A = torch.sparse_coo_tensor(torch.stack([p.row, p.col]), p.val.double(), (p.n, p.n)).to_dense()
+    xr, w1r, w2r = (t.double().requires_grad_(True) for t in (p.x, p.w1, p.w2))
+    hr = A @ xr @ w1r
+    outr = A @ hr @ w2r
+    lossr = F.nll_loss(outr[p.train_mask], p.y[p.train_mask])
+    lossr.backward()
+    assert abs(float(loss.detach()) - float(lossr.detach())) <= LOSS_TOL
+    _close(h, hr.detach(), "hidden")
+    _close(out, outr.detach(), "outputs")
+    _close(w1.grad, w1r.grad, "dw1")
+    _close(w2.grad, w2r.grad, "dw2")
+    _close(x.grad, xr.grad, "dx")
