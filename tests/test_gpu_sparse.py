@@ -386,6 +386,29 @@ def test_stage_splitting_invariance(cuda):
     assert spmm_error(z, row, col, val, n, n, H) <= REL_TOL
 
 
+def test_from_torch_coo_takes_the_reference_block_type(cuda):
+    """The reference keeps its blocks as torch.sparse_coo tensors, transposed and coalesced on the
+    device (gcn_distr.py:493-512, :543-546); a handle is built straight from one, duplicates summed by
+    the coalescing as torch does."""
+    from cagnet_amd import ops
+    n, m, f = 300, 200, 24
+    row, col, val = random_coo(n, m, 4000, 17, sort=False)
+    idx = torch.stack([torch.cat([row, row[:50]]), torch.cat([col, col[:50]])])          # 50 duplicates
+    vals = torch.cat([val, val[:50]])
+    blk = torch.sparse_coo_tensor(idx, vals, (n, m)).to(cuda)
+    A = ops.CsrMatrix.from_torch_coo(blk.t(), transpose=True)                          # the drivers hold A^T
+    assert A.shape == (m, n) and A.nnz == row.numel()
+    B = torch.randn(n, f, device=cuda)
+    dense = blk.to_dense().double()
+    got = A.spmm(B)
+    mag = dense.abs().t() @ B.double().abs()
+    assert float(((got.double() - dense.t() @ B.double()).abs() / mag.clamp_min(1e-30)).max()) <= REL_TOL
+    G = torch.randn(m, f, device=cuda)
+    back = A.spmm(G, transpose=True)
+    mag = dense.abs() @ G.double().abs()
+    assert float(((back.double() - dense @ G.double()).abs() / mag.clamp_min(1e-30)).max()) <= REL_TOL
+
+
 def test_spmm_rejects_bad_arguments(cuda):
     from cagnet_amd import ops
     row, col, val, n = small_graph(8, 2000, seed=1)
