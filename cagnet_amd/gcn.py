@@ -238,12 +238,41 @@ def masked_nll_loss(outputs: torch.Tensor, y: torch.Tensor, mask: Optional[torch
     return MaskedNLLLoss.apply(outputs, y, mask)
 
 
+# `train` ends in log_softmax followed by the masked NLL (gcn_distr.py:344, :356).  With this flag
+# their backward passes are one kernel, dZ = (softmax(Z) - onehot(y)) * mask / |mask|, instead of the
+# NLL gradient (an n x classes array that is zero except for one entry per row) written out and read
+# again by the log_softmax gradient.  Amazon shape: 1.27 -> 0.55 ms per epoch.
+fused_loss = True
+
+
+class LogSoftmaxNLLLoss(torch.autograd.Function):
+    """(log_softmax(z, dim=1), masked mean NLL of it): the last activation of `train` and its loss as
+    one autograd node.  The log-probabilities are returned because `train` returns them; gradients
+    flow through the loss only."""
+
+    @staticmethod
+    def forward(ctx, z, y, mask):
+        logp = ops.log_softmax_fwd(z)
+        loss, count = ops.nll_loss_fwd(logp, y, mask)
+        ctx.save_for_backward(logp, y, mask if mask is not None else torch.empty(0, device=y.device), count)
+        ctx.has_mask = mask is not None
+        ctx.mark_non_differentiable(logp)
+        return logp, loss
+
+    @staticmethod
+    def backward(ctx, _grad_logp, grad_loss):
+        logp, y, mask, count = ctx.saved_tensors
+        dz = ops.log_softmax_nll_bwd(logp, y, mask if ctx.has_mask else None, count, grad_loss.float().reshape(()))
+        return dz, None, None
+
+
 def train(inputs, weight1, weight2, adj_matrix, am_partitions, optimizer, data, rank=0, size=1, group=None):
     """One epoch, gcn_distr.py:341-366.  `data` needs `.y` and `.train_mask`; `group` is None for a
     whole graph on one GPU, or a pair (layer-1 ResidentBlocks, layer-2 ResidentBlocks)."""
     g1, g2 = group if isinstance(group, (tuple, list)) else (group, group)
     outputs = GCNFunc.apply(inputs, weight1, adj_matrix, am_partitions, rank, size, g1, F.relu)
-    outputs = GCNFunc.apply(outputs, weight2, adj_matrix, am_partitions, rank, size, g2, F.log_softmax)
+    fuse = fused_loss and activations
+    outputs = GCNFunc.apply(outputs, weight2, adj_matrix, am_partitions, rank, size, g2, None if fuse else F.log_softmax)
 
     optimizer.zero_grad()
 
@@ -252,7 +281,10 @@ def train(inputs, weight1, weight2, adj_matrix, am_partitions, optimizer, data, 
     rank_train_mask = torch.split(data.train_mask.bool(), n_per_proc, dim=0)[rank]
     datay_rank = torch.split(data.y, n_per_proc, dim=0)[rank]
 
-    loss = masked_nll_loss(outputs, datay_rank, rank_train_mask)
+    if fuse:
+        outputs, loss = LogSoftmaxNLLLoss.apply(outputs, datay_rank, rank_train_mask)
+    else:
+        loss = masked_nll_loss(outputs, datay_rank, rank_train_mask)
     loss.backward()
     optimizer.step()
     train.last_loss = loss.detach()

@@ -58,10 +58,13 @@ def test_forward_backward_matches_oracle(cuda, monkeypatch, transpose, fused):
     _close(x.grad, ref["dx"], "dx")
 
 
-def test_training_losses_match_oracle(cuda):
+@pytest.mark.parametrize("fused_loss", [True, False])
+def test_training_losses_match_oracle(cuda, monkeypatch, fused_loss):
     """100 epochs of SGD lr 0.01 on the R-MAT scale-12 plumbing configuration: per-epoch loss
-    within 1e-4 of the fp32 CPU oracle and of its fp64 twin."""
+    within 1e-4 of the fp32 CPU oracle and of its fp64 twin, with the last log_softmax and the
+    loss as one autograd node (the default) and as the reference's two."""
     from cagnet_amd import gcn
+    monkeypatch.setattr(gcn, "fused_loss", fused_loss)
     p = synth.make_problem(scale=12, n_edges=32768, features=128, hidden=16, classes=8, mask_fraction=1.0, seed=0)
     A = orc.coo_tensor(p.row, p.col, p.val, p.n, p.n, torch.float32)
     ref32, _, _ = orc.train_epochs(p.x, p.w1, p.w2, [A], p.y, p.train_mask, epochs=100, dtype=torch.float32)
