@@ -65,6 +65,7 @@ _SIGNATURES = {
     "cg_nll_loss_fwd": [P, c_int64, P, P, c_int64, c_int32, P, P, P],
     "cg_nll_loss_bwd": [P, P, P, P, P, c_int64, c_int64, c_int32, P],
     "cg_log_softmax_nll_bwd": [P, c_int64, P, P, P, P, P, c_int64, c_int64, c_int32, P],
+    "cg_log_softmax_nll_fwd": [P, c_int64, P, P, P, c_int64, c_int64, c_int32, P, P, P],
     "cg_csr_blob_size": [P, POINTER(c_int64)],
     "cg_csr_blob_write": [P, P, c_int64, P],
     "cg_csr_blob_read": [POINTER(c_void_p), P, c_int64, c_uint32, P],

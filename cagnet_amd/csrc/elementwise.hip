@@ -86,9 +86,15 @@ __device__ __forceinline__ float team_sum(float v) {
   return v;
 }
 
+// LOSS: the lane that holds the label's column also writes the row's contribution to the masked NLL,
+// rowloss[row] = -out[row, y[row]] (0 for rows outside the mask or with a label outside [0, c)),
+// so that the loss needs no second pass over the n x c array.
+template <bool LOSS>
 __global__ __launch_bounds__(kEwThreads) void log_softmax_fwd_kernel(const float *__restrict__ z, int64_t ldz,
                                                                      float *__restrict__ out, int64_t ldo, int64_t n,
-                                                                     int32_t c) {
+                                                                     int32_t c, const int64_t *__restrict__ y,
+                                                                     const uint8_t *__restrict__ mask,
+                                                                     float *__restrict__ rowloss) {
   const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + threadIdx.x / kTeam;
   const int j = threadIdx.x % kTeam;
   const bool live = row < n;
@@ -105,6 +111,12 @@ __global__ __launch_bounds__(kEwThreads) void log_softmax_fwd_kernel(const float
   if (live) {
     float *orow = out + row * ldo;
     for (int32_t k = j; k < c; k += kTeam) orow[k] = zr[k] - lse;
+    if (LOSS) {
+      const int64_t label = y[row];
+      const bool counted = (!mask || mask[row]) && label >= 0 && label < c;
+      const int writer = counted ? (int)(label % kTeam) : 0;
+      if (j == writer) rowloss[row] = counted ? -(zr[label] - lse) : 0.f;
+    }
   }
 }
 
@@ -158,23 +170,42 @@ __device__ __forceinline__ RowWalk row_walk() {
   return RowWalk{gw * (kWave / T), nw * (kWave / T), lane / T, lane % T};
 }
 
-template <int T>
+template <int T, bool LOSS>
 __global__ __launch_bounds__(kEwThreads) void log_softmax_fwd_vec_kernel(const float *__restrict__ z, int64_t ldz,
                                                                          float *__restrict__ out, int64_t ldo,
-                                                                         int64_t n, int32_t c) {
+                                                                         int64_t n, int32_t c,
+                                                                         const int64_t *__restrict__ y,
+                                                                         const uint8_t *__restrict__ mask,
+                                                                         float *__restrict__ rowloss) {
   const RowWalk w = row_walk<T>();
   const bool col_live = 4 * w.j < c;
   const int32_t col = col_live ? 4 * w.j : 0;
   for (int64_t r0 = w.first; r0 < n; r0 += w.step) {
     const int64_t row = r0 + w.sub;
     const bool live = row < n && col_live;
-    const float4 v = *reinterpret_cast<const float4 *>(z + (row < n ? row : n - 1) * ldz + col);
+    const int64_t rc = row < n ? row : n - 1;
+    const float4 v = *reinterpret_cast<const float4 *>(z + rc * ldz + col);
+    int64_t label = 0;
+    bool counted = false;
+    if (LOSS) {  // every lane of the team reads the same two words (unconditional, clamped row)
+      label = y[rc];
+      counted = (!mask || mask[rc]) && label >= 0 && label < c;
+    }
     float mx = live ? fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w)) : -INFINITY;
     mx = vteam_max<T>(mx);
     float s = live ? (expf(v.x - mx) + expf(v.y - mx)) + (expf(v.z - mx) + expf(v.w - mx)) : 0.f;
     s = vteam_sum<T>(s);
     const float lse = mx + logf(s);
-    if (live) *reinterpret_cast<float4 *>(out + row * ldo + col) = make_float4(v.x - lse, v.y - lse, v.z - lse, v.w - lse);
+    const float4 o = make_float4(v.x - lse, v.y - lse, v.z - lse, v.w - lse);
+    if (live) *reinterpret_cast<float4 *>(out + row * ldo + col) = o;
+    if (LOSS && row < n) {
+      const int writer = counted ? (int)(label >> 2) : 0;  // the lane whose piece holds the label (its columns are live)
+      if (w.j == writer) {
+        const int q = (int)(label & 3);
+        const float at = q == 0 ? o.x : (q == 1 ? o.y : (q == 2 ? o.z : o.w));
+        rowloss[row] = counted ? -at : 0.f;
+      }
+    }
   }
 }
 
@@ -289,6 +320,44 @@ __global__ __launch_bounds__(kEwThreads) void nll_partial_kernel(const float *__
 }
 
 // pass 2: one workgroup; thread t adds partials t, t+256, ... in order, then a fixed tree
+// The same partial sums from the per-row contributions a fused forward pass left behind: same rows
+// per workgroup and the same order of additions as nll_partial_kernel, so the loss is the same float.
+__global__ __launch_bounds__(kEwThreads) void nll_rows_partial_kernel(const float *__restrict__ rowloss,
+                                                                      const uint8_t *__restrict__ mask, int64_t n,
+                                                                      float *__restrict__ psum,
+                                                                      int64_t *__restrict__ pcnt) {
+  __shared__ float ssum[kEwThreads / kWave];
+  __shared__ int scnt[kEwThreads / kWave];
+  const int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x;
+  float v = 0.f;
+  int cnt = 0;
+  if (i < n && (!mask || mask[i])) {
+    cnt = 1;
+    v = rowloss[i];
+  }
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    v += __shfl_xor(v, off, kWave);
+    cnt += __shfl_xor(cnt, off, kWave);
+  }
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  if (lane == 0) {
+    ssum[wave] = v;
+    scnt[wave] = cnt;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float s = 0.f;
+    int64_t k = 0;
+    for (int w = 0; w < kEwThreads / kWave; ++w) {
+      s += ssum[w];
+      k += scnt[w];
+    }
+    psum[blockIdx.x] = s;
+    pcnt[blockIdx.x] = k;
+  }
+}
+
 __global__ __launch_bounds__(kEwThreads) void nll_final_kernel(const float *__restrict__ psum,
                                                                const int64_t *__restrict__ pcnt, int64_t nparts,
                                                                float *__restrict__ loss, int64_t *__restrict__ count) {
@@ -392,12 +461,14 @@ int cg_log_softmax_fwd(const float *d_z, int64_t ldz, float *d_out, int64_t ldo,
   switch (vec_team(c, ldz, ldo, 4, d_z, d_out, nullptr)) {
 #define CG_CASE(T)                                                                                        \
   case T:                                                                                                 \
-    log_softmax_fwd_vec_kernel<T><<<row_grid(n, T), kEwThreads, 0, s>>>(d_z, ldz, d_out, ldo, n, c);      \
+    log_softmax_fwd_vec_kernel<T, false><<<row_grid(n, T), kEwThreads, 0, s>>>(d_z, ldz, d_out, ldo, n, c, nullptr, \
+                                                                               nullptr, nullptr);        \
     break;
     CG_CASE(1) CG_CASE(2) CG_CASE(4) CG_CASE(8) CG_CASE(16)
 #undef CG_CASE
     default:
-      log_softmax_fwd_kernel<<<(unsigned)ceil_div64(n, kRowsPerBlock), kEwThreads, 0, s>>>(d_z, ldz, d_out, ldo, n, c);
+      log_softmax_fwd_kernel<false><<<(unsigned)ceil_div64(n, kRowsPerBlock), kEwThreads, 0, s>>>(d_z, ldz, d_out, ldo, n,
+                                                                                                  c, nullptr, nullptr, nullptr);
   }
   CG_LAUNCH_CHECK();
   return CG_OK;
@@ -446,6 +517,47 @@ int cg_nll_loss_fwd(const float *d_logp, int64_t ld, const int64_t *d_y, const u
     CG_LAUNCH_CHECK();
   }
   nll_final_kernel<<<1, kEwThreads, 0, stream>>>(psum, pcnt, parts, d_loss, d_count);
+  CG_LAUNCH_CHECK();
+  return CG_OK;
+}
+
+int cg_log_softmax_nll_fwd(const float *d_z, int64_t ldz, const int64_t *d_y, const uint8_t *d_mask, float *d_out,
+                           int64_t ldo, int64_t n, int32_t c, float *d_loss, int64_t *d_count, cg_stream_t stream_) {
+  using namespace cg;
+  hipStream_t s = (hipStream_t)stream_;
+  CG_TRY(check_rows("cg_log_softmax_nll_fwd", n, c));
+  if (!d_loss || !d_count) CG_FAIL(CG_ERR_NULL, "cg_log_softmax_nll_fwd: null output");
+  if (n > 0 && (!d_z || !d_out || !d_y)) CG_FAIL(CG_ERR_NULL, "cg_log_softmax_nll_fwd: null pointer");
+  if (ldz < c || ldo < c) CG_FAIL(CG_ERR_SIZE, "cg_log_softmax_nll_fwd: leading dimension smaller than c");
+  const int64_t parts = ceil_div64(n, kEwThreads);
+  void *p = nullptr;
+  const size_t head = (size_t)(parts + 1) * (sizeof(float) + sizeof(int64_t)) + 16;
+  CG_TRY(scratch_get(s, kSlotB, head + (size_t)(n > 0 ? n : 1) * sizeof(float), &p));
+  int64_t *pcnt = (int64_t *)p;  // 8-byte aligned part first
+  float *psum = (float *)(pcnt + parts + 1);
+  float *rowloss = (float *)((char *)p + (head & ~(size_t)15));
+  if (n > 0) {
+    ProfScope prof("log_softmax_fwd", c, s);
+    switch (vec_team(c, ldz, ldo, 4, d_z, d_out, nullptr)) {
+#define CG_CASE(T)                                                                                                 \
+  case T:                                                                                                          \
+    log_softmax_fwd_vec_kernel<T, true><<<row_grid(n, T), kEwThreads, 0, s>>>(d_z, ldz, d_out, ldo, n, c, d_y, d_mask, \
+                                                                              rowloss);                            \
+    break;
+      CG_CASE(1) CG_CASE(2) CG_CASE(4) CG_CASE(8) CG_CASE(16)
+#undef CG_CASE
+      default:
+        log_softmax_fwd_kernel<true><<<(unsigned)ceil_div64(n, kRowsPerBlock), kEwThreads, 0, s>>>(d_z, ldz, d_out, ldo, n, c,
+                                                                                                   d_y, d_mask, rowloss);
+    }
+    CG_LAUNCH_CHECK();
+  }
+  ProfScope prof("nll_fwd", c, s);
+  if (parts > 0) {
+    nll_rows_partial_kernel<<<(unsigned)parts, kEwThreads, 0, s>>>(rowloss, d_mask, n, psum, pcnt);
+    CG_LAUNCH_CHECK();
+  }
+  nll_final_kernel<<<1, kEwThreads, 0, s>>>(psum, pcnt, parts, d_loss, d_count);
   CG_LAUNCH_CHECK();
   return CG_OK;
 }

@@ -241,7 +241,8 @@ def masked_nll_loss(outputs: torch.Tensor, y: torch.Tensor, mask: Optional[torch
 # `train` ends in log_softmax followed by the masked NLL (gcn_distr.py:344, :356).  With this flag
 # their backward passes are one kernel, dZ = (softmax(Z) - onehot(y)) * mask / |mask|, instead of the
 # NLL gradient (an n x classes array that is zero except for one entry per row) written out and read
-# again by the log_softmax gradient.  Amazon shape: 1.27 -> 0.55 ms per epoch.
+# again by the log_softmax gradient; forward likewise takes the loss from the log_softmax pass
+# instead of reading the log-probabilities again.
 fused_loss = True
 
 
@@ -252,8 +253,7 @@ class LogSoftmaxNLLLoss(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, z, y, mask):
-        logp = ops.log_softmax_fwd(z)
-        loss, count = ops.nll_loss_fwd(logp, y, mask)
+        logp, loss, count = ops.log_softmax_nll_fwd(z, y, mask)
         ctx.save_for_backward(logp, y, mask if mask is not None else torch.empty(0, device=y.device), count)
         ctx.has_mask = mask is not None
         ctx.mark_non_differentiable(logp)

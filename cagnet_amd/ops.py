@@ -495,6 +495,21 @@ def nll_loss_fwd(logp: torch.Tensor, y: torch.Tensor, mask: Optional[torch.Tenso
     return loss, count
 
 
+def log_softmax_nll_fwd(z: torch.Tensor, y: torch.Tensor, mask: Optional[torch.Tensor] = None):
+    """(logp, loss, count) = log_softmax_fwd followed by nll_loss_fwd, in one pass over z; the loss is
+    the same float the two separate calls give."""
+    z, ldz = _rowmajor(z, "z")
+    n, c = z.shape
+    y, mask = _labels(y, n), _mask(mask, n)
+    logp = torch.empty(n, c, dtype=torch.float32, device=z.device)
+    loss = torch.empty((), dtype=torch.float32, device=z.device)
+    count = torch.empty((), dtype=torch.int64, device=z.device)
+    check(lib.cg_log_softmax_nll_fwd(_ptr(z), ldz, _ptr(y), _ptr(mask), _ptr(logp), max(c, 1), n, c,
+                                     c_void_p(loss.data_ptr()), c_void_p(count.data_ptr()), _stream()),
+          "cg_log_softmax_nll_fwd")
+    return logp, loss, count
+
+
 def nll_loss_bwd(y: torch.Tensor, mask: Optional[torch.Tensor], count: torch.Tensor, gscale: Optional[torch.Tensor],
                  n: int, c: int) -> torch.Tensor:
     y, mask = _labels(y, n), _mask(mask, n)

@@ -194,6 +194,9 @@ int cg_dense_xtg(const float *d_X, int64_t ldx, const float *d_G, int64_t ldg, f
  *                     (the reference's fake_loss branch, gcn_distr.py:359-362)
  *   nll_loss_bwd    : dlogp[i,c] = -gscale * mask_i / |mask| * [c == y_i]   (zero elsewhere)
  *   log_softmax_nll_bwd : fused dz = gscale * mask_i/|mask| * (exp(logp[i,c]) - [c == y_i])
+ *   log_softmax_nll_fwd : log_softmax_fwd and nll_loss_fwd in one pass over z (the reference's
+ *                         train ends in exactly this pair, gcn_distr.py:344 and :356); the loss is
+ *                         the same float nll_loss_fwd returns for the log-probabilities written
  * y is int64 (torch labels); mask is one byte per row (torch.bool / uint8), NULL = all rows.
  * A label outside [0, c) contributes nothing (torch would raise).  d_count receives |mask| as
  * int64 (device).  Both reductions run in a fixed order.
@@ -211,6 +214,8 @@ int cg_nll_loss_bwd(const int64_t *d_y, const uint8_t *d_mask, const int64_t *d_
 int cg_log_softmax_nll_bwd(const float *d_logp, int64_t ld, const int64_t *d_y, const uint8_t *d_mask,
                            const int64_t *d_count, const float *d_gscale, float *d_dz, int64_t lddz, int64_t n,
                            int32_t c, cg_stream_t stream);
+int cg_log_softmax_nll_fwd(const float *d_z, int64_t ldz, const int64_t *d_y, const uint8_t *d_mask, float *d_out,
+                           int64_t ldo, int64_t n, int32_t c, float *d_loss, int64_t *d_count, cg_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * A sparse block as one byte string in host memory, for files and for transfers between ranks.

@@ -112,6 +112,17 @@ def test_nll_loss_forward_backward(cuda, n, c, frac):
         zr = z.double().requires_grad_(True)
         (F.nll_loss(F.log_softmax(zr, dim=1)[sel], y[sel]) * 0.5).backward()
         assert float((fused.cpu().double() - zr.grad).abs().max()) <= 1e-6
+    # forward fused as well: the same log-probabilities, count and (bit for bit) loss as the two calls
+    m = None if mask is None else mask.to(cuda)
+    logp2, loss2, count2 = ops.log_softmax_nll_fwd(z.to(cuda), y.to(cuda), m)
+    loss1, count1 = ops.nll_loss_fwd(out, y.to(cuda), m)
+    assert torch.equal(logp2, out) and int(count2) == int(count1) == expect_count
+    assert float(loss2) == float(loss1)
+    y_bad = y.clone()
+    y_bad[0] = c + 3                           # a label outside [0, c) contributes nothing but is counted
+    l2 = ops.log_softmax_nll_fwd(z.to(cuda), y_bad.to(cuda), m)
+    l1 = ops.nll_loss_fwd(out, y_bad.to(cuda), m)
+    assert float(l2[1]) == float(l1[0]) and int(l2[2]) == int(l1[1])
 
 
 def test_rowwise_kernels_on_views(cuda):
