@@ -320,3 +320,37 @@ def test_activations_off_is_the_plain_linear_model(cuda, monkeypatch):
     _close(w1.grad, w1r.grad, "dw1")
     _close(w2.grad, w2r.grad, "dw2")
     _close(x.grad, xr.grad, "dx")
+
+
+@pytest.mark.parametrize("classes,features,scale,edges", [(8, 128, 12, 32768), (41, 64, 11, 16384)])
+def test_adam_epochs_with_reference_init_match_oracle(cuda, classes, features, scale, edges):
+    """The reference's own set-up of a run (gcn_distr.py:550-562): torch.manual_seed(0), weights
+    torch.rand(features, 16) and torch.rand(16, classes), Adam lr 0.01.  60 epochs of `train`: the loss of
+    every epoch within 1e-4 of the fp32 CPU oracle and of its fp64 twin, and the weights after them."""
+    from cagnet_amd import gcn
+    p = synth.make_problem(scale=scale, n_edges=edges, features=features, hidden=16, classes=classes,
+                           mask_fraction=0.66, seed=0)
+    torch.manual_seed(0)
+    w1_0 = torch.rand(features, 16)
+    w2_0 = torch.rand(16, classes)
+    A = orc.coo_tensor(p.row, p.col, p.val, p.n, p.n, torch.float32)
+    epochs = 60
+    ref32, _, _ = orc.train_epochs(p.x, w1_0, w2_0, [A], p.y, p.train_mask, epochs=epochs, optimizer="adam",
+                                   dtype=torch.float32)
+    ref64, w1_64, w2_64 = orc.train_epochs(p.x, w1_0, w2_0, [A], p.y, p.train_mask, epochs=epochs, optimizer="adam",
+                                           dtype=torch.float64)
+    blk = _block(p, cuda, transpose=True)
+    x = p.x.to(cuda)
+    w1 = w1_0.to(cuda).requires_grad_(True)
+    w2 = w2_0.to(cuda).requires_grad_(True)
+    opt = torch.optim.Adam([w1, w2], lr=0.01)
+    data = _Data(p.y.to(cuda), p.train_mask.to(cuda))
+    losses = []
+    for _ in range(epochs):
+        gcn.train(x, w1, w2, p.n, [blk], opt, data, 0, 1, None)
+        losses.append(float(gcn.train.last_loss))
+    assert max(abs(a - b) for a, b in zip(losses, ref64)) <= LOSS_TOL
+    assert max(abs(a - b) for a, b in zip(losses, ref32)) <= LOSS_TOL
+    assert losses[-1] < losses[0]
+    _close(w1, w1_64, "w1 after 60 Adam epochs", 1e-3)
+    _close(w2, w2_64, "w2 after 60 Adam epochs", 1e-3)

@@ -733,3 +733,82 @@ def test_dense_offsets_beyond_int32(cuda):
     del dX, C, G
     H = ops.relu_fwd(B)                                # elementwise kernels index the same 2.3e9 elements
     assert torch.equal(H[n - 1], B[n - 1].clamp_min(0)) and torch.equal(H[0], B[0].clamp_min(0))
+
+
+def test_sparse_coo_tensor_gpu_on_device_tensors(cuda):
+    """sparse_coo_tensor_gpu (sparse-extension/sparse_coo_tensor.cu:43-54) on device int64 indices, the
+    way the 2D driver calls it (gcn_distr_2d.py:385-389): the result equals torch.sparse_coo_tensor's,
+    shares the storage of its arguments (no copy, no validation pass), and feeds a handle."""
+    from cagnet_amd import ops
+    from cagnet_amd.sparse_coo_tensor_cpp import sparse_coo_tensor_gpu
+    n, m, f = 211, 157, 20
+    row, col, val = random_coo(n, m, 3000, 31)
+    idx = torch.stack([row, col]).to(cuda)
+    v = val.to(cuda)
+    t = sparse_coo_tensor_gpu(idx, v, (n, m))
+    assert t.is_sparse and t.device.type == "cuda" and tuple(t.shape) == (n, m)
+    assert t._indices().dtype == torch.int64 and t._values().dtype == torch.float32
+    assert t._indices().data_ptr() == idx.data_ptr() and t._values().data_ptr() == v.data_ptr()
+    ref = torch.sparse_coo_tensor(idx, v, (n, m))
+    assert torch.equal(t.to_dense(), ref.to_dense())
+    assert t.sparse_dim() == 2 and t.dense_dim() == 0           # sparse_dim = indices.size(0), dense_dim = values.dim() - 1
+    B = torch.randn(m, f, device=cuda)
+    A = ops.CsrMatrix.from_torch_coo(t)
+    assert spmm_error(A.spmm(B), row, col, val, n, m, B.cpu()) <= REL_TOL
+    # an index that torch's validating constructor would reject passes unchecked, like the reference's
+    bad = idx.clone()
+    bad[0, 0] = n + 5
+    assert sparse_coo_tensor_gpu(bad, v, (n, m))._nnz() == v.numel()
+    # values with a dense dimension: dense_dim = values.dim() - 1
+    tv = sparse_coo_tensor_gpu(idx, torch.randn(v.numel(), 3, device=cuda), (n, m, 3))
+    assert tv.sparse_dim() == 2 and tv.dense_dim() == 1
+
+
+def test_spmm_from_two_host_threads_on_two_streams(cuda, tune):
+    """The digest-cached drop-in and the handle product called concurrently from two host threads,
+    each on a stream of its own and on a matrix of its own: both results against the oracle.  (One
+    handle serves one host thread at a time; the block cache is what two threads may share.)"""
+    import threading
+    from cagnet_amd import ops
+    f = 96
+    cases = []
+    for seed in (41, 42):
+        row, col, val, n = small_graph(11, 40000, seed=seed)
+        B = torch.randn(n, f, generator=torch.Generator().manual_seed(seed))
+        cases.append((row, col, val, n, B))
+    results, errors = [None, None], []
+
+    def work(k):
+        try:
+            row, col, val, n, B = cases[k]
+            stream = torch.cuda.Stream(device=cuda)
+            with torch.cuda.stream(stream):
+                r32, c32, v, Bd = _i32(row, cuda), _i32(col, cuda), val.to(cuda), B.to(cuda)
+                handle = ops.CsrMatrix(r32, c32, v, n, n)
+                outs = []
+                for _ in range(6):
+                    C = torch.zeros(n, f, device=cuda)
+                    ops.spmm_coo(r32, c32, v, n, n, Bd, C, beta=1.0, cached=True)
+                    outs.append(C)
+                    outs.append(handle.spmm(Bd))
+                stream.synchronize()
+            results[k] = outs
+        except Exception as e:  # noqa: BLE001  (reported by the main thread)
+            errors.append(e)
+
+    tune("spmm_hub", 1)                          # the cached entry point only keeps blocks that take a plan
+    try:
+        threads = [threading.Thread(target=work, args=(k,)) for k in range(2)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+    finally:
+        ops.coo_cache_clear()
+    assert not errors, errors
+    for k in range(2):
+        row, col, val, n, B = cases[k]
+        for C in results[k]:
+            assert spmm_error(C, row, col, val, n, n, B) <= REL_TOL
+        assert all(torch.equal(results[k][0], C) for C in results[k][2::2])      # cached form: bit-identical repeats
+        assert all(torch.equal(results[k][1], C) for C in results[k][3::2])      # handle form likewise
