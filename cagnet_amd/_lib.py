@@ -63,6 +63,7 @@ _SIGNATURES = {
     "cg_log_softmax_fwd": [P, c_int64, P, c_int64, c_int64, c_int32, P],
     "cg_log_softmax_bwd": [P, c_int64, P, c_int64, P, c_int64, c_int64, c_int32, P],
     "cg_nll_loss_fwd": [P, c_int64, P, P, c_int64, c_int32, P, P, P],
+    "cg_nll_loss_fwd_static": [P, c_int64, P, P, c_int64, c_int32, P, P, P],
     "cg_nll_loss_bwd": [P, P, P, P, P, c_int64, c_int64, c_int32, P],
     "cg_log_softmax_nll_bwd": [P, c_int64, P, P, P, P, P, c_int64, c_int64, c_int32, P],
     "cg_log_softmax_nll_fwd": [P, c_int64, P, P, P, c_int64, c_int64, c_int32, P, P, P],

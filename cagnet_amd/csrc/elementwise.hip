@@ -9,6 +9,7 @@
 // element per lane and step.  ReLU moves 16 bytes per lane when the operands are aligned.  The loss
 // reduction is two fixed-order passes (per workgroup, then one workgroup over the partial sums).
 #include "common.h"
+#include <mutex>
 
 namespace cg {
 
@@ -410,6 +411,35 @@ __global__ __launch_bounds__(kEwThreads) void nll_bwd_kernel(const float *__rest
   }
 }
 
+// ---- partial sums of cg_nll_loss_fwd_static: device memory that exists from load to exit --------------------
+// Room for the per-workgroup partial sums of kStaticNllMaxRows rows: (parts + 1) int64 counts, then
+// (parts + 1) float sums, laid out as in cg_nll_loss_fwd.  About 768 KiB per device.
+constexpr int64_t kStaticNllMaxRows = (int64_t)1 << 24;
+constexpr int64_t kStaticNllMaxParts = kStaticNllMaxRows / kEwThreads;
+constexpr size_t kStaticNllBytes = (size_t)(kStaticNllMaxParts + 1) * (sizeof(int64_t) + sizeof(float)) + 16;
+static __device__ __align__(256) unsigned char scratch[kStaticNllBytes];
+
+// In host code `scratch` is only a name to look the array up by; the address the kernels may use is
+// the one hipGetSymbolAddress returns, and every device holds its own copy at its own address.
+constexpr int kStaticMaxDevices = 64;
+static std::mutex g_static_mu;
+static void *g_static_ptr[kStaticMaxDevices] = {nullptr};
+
+static int static_scratch(void **out) {
+  int dev = 0;
+  CG_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kStaticMaxDevices) CG_FAIL(CG_ERR_UNSUPPORTED, "device ordinal %d beyond %d", dev, kStaticMaxDevices);
+  std::lock_guard<std::mutex> lock(g_static_mu);
+  if (!g_static_ptr[dev]) {
+    void *p = nullptr;
+    CG_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) CG_FAIL(CG_ERR_HIP, "hipGetSymbolAddress returned a null address for the static scratch array");
+    g_static_ptr[dev] = p;
+  }
+  *out = g_static_ptr[dev];
+  return CG_OK;
+}
+
 static int check_rows(const char *who, int64_t n, int32_t c) {
   if (n < 0 || c <= 0) CG_FAIL(CG_ERR_SIZE, "%s: bad sizes n=%lld c=%d", who, (long long)n, c);
   if (ceil_div64(n, kRowsPerBlock) > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "%s: too many rows", who);
@@ -512,6 +542,32 @@ int cg_nll_loss_fwd(const float *d_logp, int64_t ld, const int64_t *d_y, const u
   int64_t *pcnt = (int64_t *)p;                 // 8-byte aligned part first
   float *psum = (float *)(pcnt + parts + 1);
   ProfScope prof("nll_fwd", c, stream);
+  if (parts > 0) {
+    nll_partial_kernel<<<(unsigned)parts, kEwThreads, 0, stream>>>(d_logp, ld, d_y, d_mask, n, c, psum, pcnt);
+    CG_LAUNCH_CHECK();
+  }
+  nll_final_kernel<<<1, kEwThreads, 0, stream>>>(psum, pcnt, parts, d_loss, d_count);
+  CG_LAUNCH_CHECK();
+  return CG_OK;
+}
+
+int cg_nll_loss_fwd_static(const float *d_logp, int64_t ld, const int64_t *d_y, const uint8_t *d_mask, int64_t n,
+                           int32_t c, float *d_loss, int64_t *d_count, cg_stream_t stream_) {
+  using namespace cg;
+  hipStream_t stream = (hipStream_t)stream_;
+  CG_TRY(check_rows("cg_nll_loss_fwd_static", n, c));
+  if (n > kStaticNllMaxRows)
+    CG_FAIL(CG_ERR_SIZE, "cg_nll_loss_fwd_static: n=%lld exceeds the %lld rows the static scratch holds partial sums for",
+            (long long)n, (long long)kStaticNllMaxRows);
+  if (!d_loss || !d_count) CG_FAIL(CG_ERR_NULL, "cg_nll_loss_fwd_static: null output");
+  if (n > 0 && (!d_logp || !d_y)) CG_FAIL(CG_ERR_NULL, "cg_nll_loss_fwd_static: null input");
+  if (ld < c) CG_FAIL(CG_ERR_SIZE, "cg_nll_loss_fwd_static: leading dimension smaller than c");
+  void *p = nullptr;
+  CG_TRY(static_scratch(&p));
+  const int64_t parts = ceil_div64(n, kEwThreads);
+  int64_t *pcnt = (int64_t *)p;  // same layout as cg_nll_loss_fwd: the 8-byte aligned part first
+  float *psum = (float *)(pcnt + parts + 1);
+  // Nothing has to start at zero: the first pass writes every partial sum the second one reads.
   if (parts > 0) {
     nll_partial_kernel<<<(unsigned)parts, kEwThreads, 0, stream>>>(d_logp, ld, d_y, d_mask, n, c, psum, pcnt);
     CG_LAUNCH_CHECK();

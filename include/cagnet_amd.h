@@ -209,6 +209,16 @@ int cg_log_softmax_bwd(const float *d_g, int64_t ldg, const float *d_out, int64_
                        int64_t n, int32_t c, cg_stream_t stream);
 int cg_nll_loss_fwd(const float *d_logp, int64_t ld, const int64_t *d_y, const uint8_t *d_mask, int64_t n,
                     int32_t c, float *d_loss, int64_t *d_count, cg_stream_t stream);
+/* cg_nll_loss_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same
+ * kernels, same order of additions and therefore the same float as cg_nll_loss_fwd, but the
+ * per-workgroup partial sums live in a device array that is part of the library image (about 768 KiB
+ * on every GPU the library runs on, held until the process ends) instead of the grow-only scratch:
+ * the call allocates and frees nothing.  n may be at most 16,777,216 rows (CG_ERR_SIZE beyond).
+ * The first call on a device looks the array's address up (once; make that call outside a capture).
+ * All calls on one GPU share the array: calls that overlap on one GPU, on any streams, race. */
+int cg_nll_loss_fwd_static(const float *d_logp, int64_t ld, const int64_t *d_y, const uint8_t *d_mask, int64_t n,
+                           int32_t c, float *d_loss, int64_t *d_count, cg_stream_t stream);
 int cg_nll_loss_bwd(const int64_t *d_y, const uint8_t *d_mask, const int64_t *d_count, const float *d_gscale,
                     float *d_dlogp, int64_t ld, int64_t n, int32_t c, cg_stream_t stream);
 int cg_log_softmax_nll_bwd(const float *d_logp, int64_t ld, const int64_t *d_y, const uint8_t *d_mask,
