@@ -250,7 +250,7 @@ def main() -> int:
     kernels = {}
     widths = sorted({f_in, hidden, classes, (classes + 3) // 4 * 4})  # backward carries 41 classes padded to 44
     for f in widths:
-        for kname in ("spmm_rowseg", "spmm_reduce", "spmm_hub_hot", "spmm_hub_reduce"):
+        for kname in ("spmm_panel", "spmm_rowseg", "spmm_reduce", "spmm_hub_hot", "spmm_hub_reduce"):
             ms, cnt = prof_read(_lib.lib, f"{kname}/f={f}")
             if cnt:
                 kernels[f"{kname}/f={f}"] = {"launches": cnt, "avg_ms": ms / cnt}

@@ -54,6 +54,7 @@ _SIGNATURES = {
     "cg_csr_spmm": [P, c_int, P, c_int64, P, c_int64, c_int32, c_float, P],
     "cg_csr_spmm_xw": [P, c_int, P, c_int64, P, c_int64, c_float, P, c_int64, P, c_int64, c_int32, c_int32, c_int, P],
     "cg_csr_info": [P, POINTER(c_int64)],
+    "cg_csr_panel_info": [P, c_int, POINTER(c_int64)],
     "cg_csr_arrays": [P, c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p)],
     "cg_dense_xw": [P, c_int64, P, c_int64, P, c_int64, c_int64, c_int32, c_int32, c_int, P],
     "cg_dense_gwt": [P, c_int64, P, c_int64, P, c_int64, c_int64, c_int32, c_int32, P],

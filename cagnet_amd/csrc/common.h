@@ -37,7 +37,7 @@ int hip_fail(hipError_t e, const char *what, const char *file, int line);
 
 // ---- per (device, stream) grow-only scratch ------------------------------------------------
 // slot: independent buffers that must be alive at the same time use different slots.
-enum ScratchSlot { kSlotA = 0, kSlotB = 1, kSlotC = 2, kSlotD = 3, kNumSlots = 4 };
+enum ScratchSlot { kSlotA = 0, kSlotB = 1, kSlotC = 2, kSlotD = 3, kSlotE = 4, kNumSlots = 5 };
 int scratch_get(hipStream_t stream, int slot, size_t bytes, void **out);
 
 // ---- optional kernel timing with HIP events on the launch stream (runtime.hip) -------------------

@@ -6,7 +6,7 @@
 // Replaces everything the reference wraps around cusparseSpMM on every call
 // (sparse-extension/sparse_coo_tensor.cu:136-231): B and C stay row-major, nothing is transposed,
 // and the CSR, its transpose, the schedules and the hub plan live in a handle.
-#include "spmm_hub.h"
+#include "spmm_panel_build.h"
 #include <stdlib.h>
 #include <string.h>
 #include <atomic>
@@ -34,6 +34,9 @@ struct DenseOps {
   const float *fold_P = nullptr;
   const uint8_t *fold_any = nullptr;
   int32_t fold_classes = 0, fold_rows = 0;
+  // optional direct fold: one more partial row per row, fold_D[fold_dslot[row] * f ...] (panel plan)
+  const float *fold_D = nullptr;
+  const int32_t *fold_dslot = nullptr;
   // optional epilogue: finished rows are multiplied by W (f x fo) into Z instead of being stored
   // (see StreamArgs); C is then only read, and only when beta != 0
   const float *epi_W = nullptr;
@@ -83,7 +86,9 @@ static int spmm_plain(const int32_t *rowptr, const int32_t *colind, const float 
   sa.fold_any = d.fold_any;
   sa.fold_classes = d.fold_classes;
   sa.fold_rows = d.fold_rows;
-  if (d.fold_tbase && shape.lpr != kWave) CG_FAIL(CG_ERR_UNSUPPORTED, "fold needs full-wave teams");
+  sa.fold_D = d.fold_D;
+  sa.fold_dslot = d.fold_dslot;
+  if ((d.fold_tbase || d.fold_dslot) && shape.lpr != kWave) CG_FAIL(CG_ERR_UNSUPPORTED, "fold needs full-wave teams");
   size_t lds = 0;
   if (d.epi_W) {
     if (shape.lpr != kWave) CG_FAIL(CG_ERR_UNSUPPORTED, "epilogue needs full-wave teams");
@@ -136,7 +141,7 @@ static int spmm_plain(const int32_t *rowptr, const int32_t *colind, const float 
     const int64_t threads = sc->nmulti * (int64_t)d.f;
     spmm_reduce_kernel<<<(unsigned)ceil_div64(threads, kSpmmThreads), kSpmmThreads, 0, stream>>>(
         sc->multi_rows, sc->nmulti, nullptr, rowptr, sc->pbase, sc->seg, sa.P, d.C, d.ldc, d.f, d.beta, 0, d.fold_tbase,
-        d.fold_P, d.fold_classes, d.fold_rows);
+        d.fold_P, d.fold_classes, d.fold_rows, d.fold_D, d.fold_dslot);
     CG_LAUNCH_CHECK();
   }
   return CG_OK;
@@ -295,12 +300,19 @@ static bool epi_supported(int32_t f, int32_t fo, int vec) {
          epi_lds_bytes(f, fo) <= kEpiLdsBytes;
 }
 
+// fold (nullable): only its direct-fold fields are read (the partial rows of a panel plan, added to the rows
+// this product finishes).  allow_panel: false for the rest matrix of a panel plan.
 static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t ldc, int32_t f, float beta,
-                     hipStream_t stream, const DenseOps *epi = nullptr) {
+                     hipStream_t stream, const DenseOps *epi = nullptr, const DenseOps *fold = nullptr,
+                     bool allow_panel = true) {
   if (s.rows == 0) return CG_OK;
   const int vec = pick_vec(f, B, ldb, C ? C : B, C ? ldc : ldb);
   const int32_t cap = range_cap(vec);
   DenseOps d{B, ldb, C, ldc, f, beta};
+  if (fold) {
+    d.fold_D = fold->fold_D;
+    d.fold_dslot = fold->fold_dslot;
+  }
   if (epi) {
     if (!epi_supported(f, epi->epi_fo, vec))
       CG_FAIL(CG_ERR_UNSUPPORTED, "fused product: f=%d fo=%d has no fused form", f, epi->epi_fo);
@@ -311,12 +323,35 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
     d.epi_fo = epi->epi_fo;
     d.epi_relu = epi->epi_relu;
   }
+  // Panel plan: the entries of dense (row panel, column block) tiles are multiplied out of LDS into
+  // partial rows; the row-wise kernels then run over the other entries and add those rows in.
+  if (!epi && allow_panel && f <= cap && want_panel(s, f)) {
+    int32_t emin = g_tune_panel_emin.load(std::memory_order_relaxed);
+    if (emin <= 0) emin = kPanelDefaultEmin;
+    int32_t cols = g_tune_panel_cols.load(std::memory_order_relaxed);
+    if (cols <= 0) cols = kPanelDefaultCols;
+    int32_t unit = g_tune_panel_unit.load(std::memory_order_relaxed);
+    if (unit <= 0) unit = kPanelDefaultUnit;
+    const bool may_decline = g_tune_panel.load(std::memory_order_relaxed) == 0;
+    PanelPlan &pp = s.panel;
+    if (!pp.valid || pp.emin != emin || pp.hot_cols != cols || pp.unit_entries != unit || (pp.declined && !may_decline))
+      CG_TRY(build_panel(s, pp, emin, cols, unit, may_decline, stream));
+    if (!pp.declined) {
+      float *P = nullptr;
+      CG_TRY(launch_panel(pp, B, ldb, f, &P, stream));
+      DenseOps fd{};
+      fd.fold_D = P;
+      fd.fold_dslot = pp.dslot;
+      return spmm_side(*pp.rest, B, ldb, C, ldc, f, beta, stream, nullptr, &fd, false);
+    }
+  }
   if (f <= range_cap(vec == 4 ? 4 : 1) && want_hub(s, f)) {
     bool declined = false;
     CG_TRY(spmm_hub(s, vec, d, stream, &declined));
     if (!declined) return CG_OK;
   }
-  if (epi) return spmm_plain(s.rowptr, s.colind, s.val, s.rows, s.nnz, s.sched, vec, d, f, stream);
+  if (epi || f <= cap) return spmm_plain(s.rowptr, s.colind, s.val, s.rows, s.nnz, s.sched, vec, d, f, stream);
+  if (d.fold_dslot) CG_FAIL(CG_ERR_UNSUPPORTED, "direct fold needs a width one launch covers");
   for (int32_t f0 = 0; f0 < f; f0 += cap) {  // wider outputs take several launches over column ranges
     const int32_t ft = f - f0 < cap ? f - f0 : cap;
     const DenseOps dr{B + f0, ldb, C + f0, ldc, ft, beta};
@@ -395,7 +430,7 @@ static int spmm_coo_oneshot(const int32_t *d_row, const int32_t *d_col, const fl
     const int64_t threads = max_multi * (int64_t)ft;
     spmm_reduce_kernel<<<(unsigned)ceil_div64(threads, kSpmmThreads), kSpmmThreads, 0, stream>>>(
         sc.multi_rows, max_multi, sc.d_counts + 2, rowptr, sc.pbase, seg, (const float *)p, C + f0, ldc, ft, beta,
-        pslots, nullptr, nullptr, 0, 0);
+        pslots, nullptr, nullptr, 0, 0, nullptr, nullptr);
     CG_LAUNCH_CHECK();
   }
   return CG_OK;
@@ -755,6 +790,10 @@ int cg_tune_set(const char *key, int value) {
   else if (!strcmp(key, "spmm_hub_groups")) cg::g_tune_hub_groups.store(value);
   else if (!strcmp(key, "spmm_hub_tiers")) cg::g_tune_hub_tiers.store(value);
   else if (!strcmp(key, "spmm_hub_row")) cg::g_tune_hub_row.store(value);
+  else if (!strcmp(key, "spmm_panel")) cg::g_tune_panel.store(value);
+  else if (!strcmp(key, "spmm_panel_emin")) cg::g_tune_panel_emin.store(value);
+  else if (!strcmp(key, "spmm_panel_cols")) cg::g_tune_panel_cols.store(value);
+  else if (!strcmp(key, "spmm_panel_unit")) cg::g_tune_panel_unit.store(value);
   else if (!strcmp(key, "dense_mfma")) cg::g_tune_dense_mfma.store(value);
   else if (!strcmp(key, "coo_cache_blocks")) cg::g_tune_coo_cache.store(value);
   else CG_FAIL(CG_ERR_UNSUPPORTED, "cg_tune_set: unknown key %s", key);
@@ -770,7 +809,9 @@ int cg_csr_info(const cg_csr_t *h, int64_t info[8]) {
   info[4] = h->fwd.max_degree;
   info[5] = h->has_t ? h->tr.max_degree : -1;
   // the plan the last wide product of a side looked up: tiers taken, -1 declined, 0 none so far
-  auto last_plan = [](const cg::CsrSide &s) -> int64_t {
+  auto last_plan = [](const cg::CsrSide &side) -> int64_t {
+    // with a panel plan in use the row-wise kernels, and so the hub plans, work on its rest matrix
+    const cg::CsrSide &s = (side.panel.valid && !side.panel.declined && side.panel.rest) ? *side.panel.rest : side;
     int best = -1;
     for (int i = 0; i < cg::CsrSide::kHubPlans; ++i)
       if (s.hub[i].valid && (best < 0 || s.hub_used[i] > s.hub_used[best])) best = i;
@@ -779,6 +820,22 @@ int cg_csr_info(const cg_csr_t *h, int64_t info[8]) {
   };
   info[6] = last_plan(h->fwd);
   info[7] = h->has_t ? last_plan(h->tr) : 0;
+  return CG_OK;
+}
+
+int cg_csr_panel_info(const cg_csr_t *h, int transpose, int64_t info[8]) {
+  if (!h || !info) CG_FAIL(CG_ERR_NULL, "cg_csr_panel_info: null pointer");
+  if (transpose && !h->has_t) CG_FAIL(CG_ERR_NO_TRANSPOSE, "cg_csr_panel_info: handle was built without CG_CSR_TRANSPOSE");
+  const cg::PanelPlan &pp = (transpose ? h->tr : h->fwd).panel;
+  const bool used = pp.valid && !pp.declined;
+  info[0] = !pp.valid ? 0 : (pp.declined ? -1 : 1);
+  info[1] = used ? pp.covered : 0;
+  info[2] = used ? pp.ntiles : 0;
+  info[3] = used ? pp.nunits : 0;
+  info[4] = used ? pp.nsplit : 0;
+  info[5] = used && pp.rest ? pp.rest->nnz : 0;
+  info[6] = pp.valid ? pp.emin : 0;
+  info[7] = pp.valid ? pp.hot_cols : 0;
   return CG_OK;
 }
 

@@ -2,7 +2,7 @@
 // construction of hub plans: columns ranked by reference count, dealt to tiers and XCD groups, the
 // entries regrouped by class.  Included by spmm.hip only, after spmm_tables.h.
 #pragma once
-#include "spmm_tables.h"
+#include "spmm_panel.h"
 
 namespace cg {
 
@@ -96,7 +96,9 @@ struct CsrSide {
   HubPlan hub[kHubPlans];
   uint64_t hub_used[kHubPlans] = {0, 0};
   uint64_t hub_clock = 0;
+  PanelPlan panel;  // plan of the wide products that multiply the dense part out of LDS (spmm_panel.h)
   void release() {
+    panel.release();
     sched.release();
     for (int i = 0; i < kHubPlans; ++i) hub[i].release();
     if (rowptr) (void)hipFree(rowptr);
@@ -106,6 +108,22 @@ struct CsrSide {
     val = nullptr;
   }
 };
+
+inline void PanelPlan::release() {
+  void *owned[] = {unit_tile, unit_order, tile_kb, tile_wptr, ent, qcol, dslot, split};
+  for (void *p : owned)
+    if (p) (void)hipFree(p);
+  unit_tile = unit_order = tile_kb = tile_wptr = qcol = dslot = split = nullptr;
+  ent = nullptr;
+  if (rest) {
+    rest->release();
+    delete rest;
+    rest = nullptr;
+  }
+  valid = declined = false;
+  covered = 0;
+  ntiles = nunits = nsplit = 0;
+}
 
 // ---------------------------------------------------------------------------------------------
 // hub plan construction

@@ -83,7 +83,9 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_reduce_kernel(const int32_t
                                                                    int64_t p_cap,
                                                                    const int32_t *__restrict__ fold_tbase,
                                                                    const float *__restrict__ fold_P,
-                                                                   int32_t fold_classes, int32_t fold_rows) {
+                                                                   int32_t fold_classes, int32_t fold_rows,
+                                                                   const float *__restrict__ fold_D,
+                                                                   const int32_t *__restrict__ fold_dslot) {
   const int64_t idx = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   const int64_t mr = idx / f;
   const int32_t col = (int32_t)(idx % f);
@@ -101,6 +103,10 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_reduce_kernel(const int32_t
       const int32_t *tb = fold_tbase + (int64_t)cls * fold_rows + row;
       for (int32_t t = tb[0]; t < tb[1]; ++t) s += fold_P[(int64_t)t * f + col];
     }
+  }
+  if (fold_dslot) {
+    const int32_t ds = fold_dslot[row];
+    if (ds >= 0) s += fold_D[(int64_t)ds * f + col];
   }
   float *c = C + (int64_t)row * ldc + col;
   *c = beta != 0.f ? fmaf(beta, *c, s) : s;
@@ -133,6 +139,10 @@ struct StreamArgs {
   const float *fold_P;
   const uint8_t *fold_any;
   int32_t fold_classes, fold_rows;
+  // Direct fold (wide teams, groups == 1): row r also receives the one partial row
+  // fold_D[fold_dslot[r] * f ...] when fold_dslot[r] >= 0 (the panel plan's share of the row), added last.
+  const float *fold_D;
+  const int32_t *fold_dslot;
   // Epilogue (wide teams, groups == 1): a finished row r = beta*C[row] + (A B)[row] is not stored
   // but multiplied by epi_W (f x epi_fo): epi_Z[row, :] = act(r * epi_W), the layer's (A H) W
   // without the n x f intermediate.  epi_fop = epi_fo rounded up to 16, 32 or 64.
@@ -322,6 +332,20 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_stream_wide_kernel(const St
                   for (int q = 0; q < VEC; ++q) acc[ch][q] += pv[ch][q];
                 folded = true;
               }
+            }
+          }
+          if (a.fold_dslot) {
+            const int32_t ds = __builtin_amdgcn_readfirstlane(a.fold_dslot[dst]);
+            if (ds >= 0) {
+              const float *prow = a.fold_D + (int64_t)ds * a.f;
+              float pv[CHUNKS][VEC];
+#pragma unroll
+              for (int ch = 0; ch < CHUNKS; ++ch) load_vec<VEC>(prow + boff[ch], pv[ch]);
+#pragma unroll
+              for (int ch = 0; ch < CHUNKS; ++ch)
+#pragma unroll
+                for (int q = 0; q < VEC; ++q) acc[ch][q] += pv[ch][q];
+              folded = true;
             }
           }
           if (a.epi_W) {

@@ -1,0 +1,339 @@
+// Panel plan of the wide CSR SpMM: the dense part of a power-law matrix is multiplied out of LDS.
+//
+// A row-wise SpMM gathers one row of B per stored entry (2408 bytes at f = 602); on a matrix with a
+// few hundred entries per row nearly all of that traffic is re-reading rows of B that other rows of A
+// also use.  Here rows and columns are ranked by their entry counts, rows are taken in panels of 128
+// consecutive ranks and columns in blocks of 32 consecutive ranks.  A (panel, block) tile that holds
+// enough entries is "active": its 32 rows of B are copied into LDS once (global -> LDS directly, no
+// registers in between) and all of the tile's entries read them from there, at LDS bandwidth instead
+// of through the vector memory path.  A workgroup of 16 waves owns a unit = a run of active tiles of one
+// panel; wave w holds the accumulators of the 8 rows {w, w + 16, ...} of the panel in registers for the
+// whole unit and writes them out once as partial rows.  Entries of tiles that are not active stay in a
+// second CSR matrix (the "rest") that the row-wise kernels multiply; their finished rows add the
+// partial rows in.  Replaces nothing in the reference beyond cusparseSpMM itself
+// (sparse-extension/sparse_coo_tensor.cu:215-226); sums are in a fixed order, no atomics on floats.
+#pragma once
+#include "spmm_tables.h"
+#include <algorithm>
+#include <vector>
+
+namespace cg {
+
+constexpr int kPanelRows = 128;   // rows of a panel
+constexpr int kPanelWaves = 16;   // waves of a workgroup; wave w owns rows w, w + 16, ... of the panel
+constexpr int kPanelSlots = kPanelRows / kPanelWaves;  // rows per wave
+constexpr int kPanelCols = 32;    // columns of a block = rows of B staged per tile
+constexpr int kPanelThreads = kPanelWaves * kWave;
+constexpr int32_t kPanelMinF = 258, kPanelMaxF = 636;  // widths the kernel is instantiated for (even)
+
+static std::atomic<int> g_tune_panel{0}, g_tune_panel_emin{0}, g_tune_panel_cols{0}, g_tune_panel_unit{0};
+
+struct CsrSide;
+
+struct PanelPlan {
+  bool valid = false, declined = false;
+  int32_t emin = 0, hot_cols = 0, unit_entries = 0;  // what the plan was built with
+  int64_t covered = 0;      // entries the panel kernel multiplies
+  int32_t ntiles = 0, nunits = 0, nsplit = 0;
+  int32_t *unit_tile = nullptr;    // [nunits + 1] tiles of a unit (units never span panels)
+  int32_t *unit_order = nullptr;   // [nunits] launch order: heaviest unit first
+  int32_t *tile_kb = nullptr;      // [ntiles] column block of a tile
+  int32_t *tile_wptr = nullptr;    // [ntiles * 16 + 1] records of (tile, wave)
+  uint2 *ent = nullptr;            // [covered] {column in block | slot << 8, value bits}, by (tile, wave, slot)
+  int32_t *qcol = nullptr;         // [hot_cols] column (row of B) of every ranked hot column
+  int32_t *dslot = nullptr;        // [rows] partial row of a row of A: unit * 128 + position, or -1
+  int32_t *split = nullptr;        // [2 * nsplit] (first unit, units) of panels that have several units
+  CsrSide *rest = nullptr;         // entries outside active tiles, same rows and columns
+  void release();
+};
+
+// -------------------------------------------------------------------------------------------------
+// the product kernel
+// -------------------------------------------------------------------------------------------------
+// One 16-byte (or 4-byte) piece per lane from global memory straight into LDS at lds_addr + lane * size.
+// The compiler does not see these loads: it would otherwise wait for them before every LDS read (it
+// cannot tell the two LDS buffers apart); the kernel waits for them itself before the barrier.
+__device__ __forceinline__ void panel_copy16(uint32_t lds_addr, const float *src) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(src) : "memory");
+}
+__device__ __forceinline__ void panel_copy4(uint32_t lds_addr, const float *src) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_addr), "v"(src) : "memory");
+}
+
+template <int CHUNKS>
+__global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
+    const int32_t *__restrict__ unit_tile, const int32_t *__restrict__ unit_order, const int32_t *__restrict__ tile_kb,
+    const int32_t *__restrict__ tile_wptr, const uint2 *__restrict__ ent, const int32_t *__restrict__ qcol,
+    const float *__restrict__ B, int64_t ldb, float *__restrict__ P, int32_t f) {
+  extern __shared__ __align__(16) char panel_lds[];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int unit = unit_order[blockIdx.x];
+  const int t0 = unit_tile[unit], t1 = unit_tile[unit + 1];
+  const int npair = f >> 1;
+  const int rs = (f * 4 + 15) & ~15;  // bytes of a staged row: 16-byte aligned for the direct copies
+  const int bufsz = kPanelCols * rs;
+  constexpr int RPW = kPanelCols / kPanelWaves;  // rows of B a wave stages per tile
+  float2 acc[kPanelSlots][CHUNKS];
+#pragma unroll
+  for (int s = 0; s < kPanelSlots; ++s)
+#pragma unroll
+    for (int ch = 0; ch < CHUNKS; ++ch) acc[s][ch] = make_float2(0.f, 0.f);
+
+  const int nq = f >> 2;     // whole 16-byte pieces of a row of B
+  const int tail0 = nq * 4;  // first float of the 4-byte pieces behind them
+  auto stage_row = [&](int t, int r, int buf) {
+    const int kb = tile_kb[t];
+    const int row = wave + r * kPanelWaves;
+    const int q = qcol[kb * kPanelCols + row];
+    const float *src = B + (int64_t)q * ldb;
+    const uint32_t dst = (uint32_t)(uintptr_t)(panel_lds + buf * bufsz + row * rs);
+    for (int p0 = 0; p0 < nq; p0 += kWave) {
+      const int p = p0 + lane;
+      if (p < nq) panel_copy16(dst + p0 * 16, src + 4 * p);
+    }
+    for (int c0 = tail0; c0 < f; c0 += kWave) {
+      const int c = c0 + lane;
+      if (c < f) panel_copy4(dst + c0 * 4, src + c);
+    }
+  };
+  // records of a (tile, wave), first 64 of them: one per lane, loaded a tile ahead
+  auto rec_load = [&](int t, uint2 &r, int &b0, int &b1) {
+    b0 = tile_wptr[t * kPanelWaves + wave];
+    b1 = tile_wptr[t * kPanelWaves + wave + 1];
+    int idx = b0 + lane;
+    idx = idx < b1 ? idx : (b1 > b0 ? b1 - 1 : 0);  // unconditional, clamped
+    r = ent[idx];
+  };
+  uint2 rec = make_uint2(0u, 0u);
+  int e0 = 0, e1 = 0;
+  if (t1 > t0) {
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) stage_row(t0, r, 0);
+    rec_load(t0, rec, e0, e1);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  for (int t = t0; t < t1; ++t) {
+    const int buf = (t - t0) & 1;
+    const int tn = t + 1 < t1 ? t + 1 : t;  // the last tile stages itself again: no branch around the copies
+    const char *lbase = panel_lds + buf * bufsz + lane * 8;
+    // The records of this tile arrived before the last barrier.  Touching them here puts the compiler's
+    // wait for them ahead of the copies it cannot see, so that nothing below waits for those.
+    asm volatile("" ::"v"(rec.x), "v"(rec.y));
+    uint2 recn;
+    int e0n, e1n;
+    rec_load(tn, recn, e0n, e1n);
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) stage_row(tn, r, buf ^ 1);
+
+    // records are sorted by slot: the lanes' ballots give the length of every slot's run, and a run
+    // adds into that slot's registers (static register indices)
+    auto process = [&](const uint2 r, int cnt) {
+      const uint32_t myslot = (r.x >> 8) & 0x7u;
+      int i = 0;
+#pragma unroll
+      for (int s = 0; s < kPanelSlots; ++s) {
+        const int c = __builtin_popcountll(__ballot(lane < cnt && myslot == (uint32_t)s));
+        const int end = i + c;
+        for (; i < end; ++i) {
+          const uint32_t x = __builtin_amdgcn_readlane(r.x, i);
+          const float v = __uint_as_float(__builtin_amdgcn_readlane(r.y, i));
+          const char *src = lbase + (x & 0xffu) * rs;
+          float2 b[CHUNKS];
+#pragma unroll
+          for (int ch = 0; ch < CHUNKS; ++ch) b[ch] = *reinterpret_cast<const float2 *>(src + ch * 512);
+#pragma unroll
+          for (int ch = 0; ch < CHUNKS; ++ch) {
+            acc[s][ch].x = fmaf(v, b[ch].x, acc[s][ch].x);
+            acc[s][ch].y = fmaf(v, b[ch].y, acc[s][ch].y);
+          }
+        }
+      }
+    };
+    {
+      const int cnt = e1 - e0;
+      process(rec, cnt > kWave ? kWave : cnt);
+    }
+    for (int base = e0 + kWave; base < e1; base += kWave) {  // further records of a dense tile, fetched on demand
+      int idx = base + lane;
+      idx = idx < e1 ? idx : e1 - 1;
+      const uint2 r2 = ent[idx];
+      const int cnt = e1 - base;
+      process(r2, cnt > kWave ? kWave : cnt);
+    }
+    rec = recn;
+    e0 = e0n;
+    e1 = e1n;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+  // P[unit][slot * 16 + wave][:]: position in the block = rank of the row inside its panel
+#pragma unroll
+  for (int s = 0; s < kPanelSlots; ++s) {
+    float *prow = P + ((int64_t)unit * kPanelRows + s * kPanelWaves + wave) * f;
+#pragma unroll
+    for (int ch = 0; ch < CHUNKS; ++ch) {
+      const int p = lane + kWave * ch;
+      if (p < npair) *reinterpret_cast<float2 *>(prow + 2 * p) = acc[s][ch];
+    }
+  }
+}
+
+// Panels with several units: the blocks of the later units are added to the first one's, in unit order.
+__global__ __launch_bounds__(kSpmmThreads) void panel_reduce_kernel(const int32_t *__restrict__ split, float *__restrict__ P,
+                                                                    int32_t f) {
+  const int32_t first = split[2 * blockIdx.y], count = split[2 * blockIdx.y + 1];
+  const int64_t block = (int64_t)kPanelRows * f;
+  const int64_t idx = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (idx >= block) return;
+  float *p = P + (int64_t)first * block + idx;
+  float s = p[0];
+  int32_t u = 1;
+  for (; u + 4 <= count; u += 4) {
+    float v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = p[(int64_t)(u + k) * block];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) s += v[k];
+  }
+  for (; u < count; ++u) s += p[(int64_t)u * block];
+  p[0] = s;
+}
+
+// -------------------------------------------------------------------------------------------------
+// plan construction kernels
+// -------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kSpmmThreads) void panel_degree_key_kernel(const int32_t *__restrict__ rowptr, int32_t n,
+                                                                        int32_t maxdeg, int32_t *__restrict__ key,
+                                                                        int32_t *__restrict__ id) {
+  const int64_t r = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (r < n) {
+    key[r] = maxdeg - (rowptr[r + 1] - rowptr[r]);  // ascending key = descending degree, ties by row (stable sort)
+    id[r] = (int32_t)r;
+  }
+}
+
+__global__ __launch_bounds__(kSpmmThreads) void panel_col_count_kernel(const int32_t *__restrict__ colind, int64_t nnz,
+                                                                       uint32_t *__restrict__ count) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k < nnz) atomicAdd(&count[colind[k]], 1u);  // integer count: order independent
+}
+
+__global__ __launch_bounds__(kSpmmThreads) void panel_count_key_kernel(const uint32_t *__restrict__ count, int32_t m,
+                                                                       uint32_t maxcount, int32_t *__restrict__ key,
+                                                                       int32_t *__restrict__ id) {
+  const int64_t j = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (j < m) {
+    key[j] = (int32_t)(maxcount - count[j]);
+    id[j] = (int32_t)j;
+  }
+}
+
+// rank_of[ranked[k]] = k
+__global__ __launch_bounds__(kSpmmThreads) void panel_invert_kernel(const int32_t *__restrict__ ranked, int32_t count,
+                                                                    int32_t *__restrict__ rank_of) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k < count) rank_of[ranked[k]] = (int32_t)k;
+}
+
+// tile of an entry: (row rank / 128) * nkb + column rank / 32 when both ranks are inside the ranked
+// area (the first prows row ranks, the first hot column ranks), else -1
+__device__ __forceinline__ int64_t panel_tile_of(int32_t rrank, int32_t crank, int32_t prows, int32_t hot, int32_t nkb) {
+  if (rrank >= prows || crank >= hot) return -1;
+  return (int64_t)(rrank / kPanelRows) * nkb + crank / kPanelCols;
+}
+
+__global__ __launch_bounds__(kSpmmThreads) void panel_tile_count_kernel(
+    const int32_t *__restrict__ erow, const int32_t *__restrict__ colind, int64_t nnz, const int32_t *__restrict__ row_rank,
+    const int32_t *__restrict__ col_rank, int32_t prows, int32_t hot, int32_t nkb, uint32_t *__restrict__ tcount) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k >= nnz) return;
+  const int64_t t = panel_tile_of(row_rank[erow[k]], col_rank[colind[k]], prows, hot, nkb);
+  if (t >= 0) atomicAdd(&tcount[t], 1u);
+}
+
+// flag[t] = 1 and kept[t] = tcount[t] for tiles with at least emin entries, else 0 (both arrays are then scanned)
+__global__ __launch_bounds__(kSpmmThreads) void panel_tile_select_kernel(const uint32_t *__restrict__ tcount, int64_t tiles,
+                                                                         uint32_t emin, uint32_t *__restrict__ flag,
+                                                                         uint32_t *__restrict__ kept) {
+  const int64_t t = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (t > tiles) return;
+  const bool on = t < tiles && tcount[t] >= emin;  // entry `tiles` is the slot the scans leave their totals in
+  flag[t] = on ? 1u : 0u;
+  kept[t] = on ? tcount[t] : 0u;
+}
+
+// compact tables of the active tiles
+__global__ __launch_bounds__(kSpmmThreads) void panel_tile_tables_kernel(const uint32_t *__restrict__ tcount,
+                                                                         const uint32_t *__restrict__ tindex, int64_t tiles,
+                                                                         uint32_t emin, int32_t nkb,
+                                                                         int32_t *__restrict__ tile_kb,
+                                                                         int32_t *__restrict__ tile_panel) {
+  const int64_t t = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (t >= tiles || tcount[t] < emin) return;
+  tile_kb[tindex[t]] = (int32_t)(t % nkb);
+  tile_panel[tindex[t]] = (int32_t)(t / nkb);
+}
+
+// sort keys: covered entries get (active tile * 16 + wave) as major and the slot as minor key, all others the
+// sentinel `ntiles * 16`, which a stable sort leaves behind the covered ones in their (row, col) order
+__global__ __launch_bounds__(kSpmmThreads) void panel_entry_key_kernel(
+    const int32_t *__restrict__ erow, const int32_t *__restrict__ colind, int64_t nnz, const int32_t *__restrict__ row_rank,
+    const int32_t *__restrict__ col_rank, int32_t prows, int32_t hot, int32_t nkb, const uint32_t *__restrict__ tcount,
+    const uint32_t *__restrict__ tindex, uint32_t emin, int32_t sentinel, int32_t *__restrict__ key,
+    int32_t *__restrict__ slot, int32_t *__restrict__ pos) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k >= nnz) return;
+  const int32_t rr = row_rank[erow[k]];
+  const int64_t t = panel_tile_of(rr, col_rank[colind[k]], prows, hot, nkb);
+  int32_t ky = sentinel, sl = 0;
+  if (t >= 0 && tcount[t] >= emin) {
+    const int32_t p = rr % kPanelRows;
+    ky = (int32_t)tindex[t] * kPanelWaves + p % kPanelWaves;
+    sl = p / kPanelWaves;
+  }
+  key[k] = ky;
+  slot[k] = sl;
+  pos[k] = (int32_t)k;
+}
+
+// after the sort: records of the covered entries, and the arrays of the rest
+__global__ __launch_bounds__(kSpmmThreads) void panel_entry_finish_kernel(
+    const int32_t *__restrict__ slot_sorted, const int32_t *__restrict__ pos, int64_t nnz, int64_t covered,
+    const int32_t *__restrict__ erow, const int32_t *__restrict__ colind, const float *__restrict__ val,
+    const int32_t *__restrict__ col_rank, uint2 *__restrict__ ent, int32_t *__restrict__ rest_row,
+    int32_t *__restrict__ rest_col, float *__restrict__ rest_val) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k >= nnz) return;
+  const int32_t p = pos[k];
+  if (k < covered) {
+    ent[k] = make_uint2((uint32_t)(col_rank[colind[p]] % kPanelCols) | ((uint32_t)slot_sorted[k] << 8), __float_as_uint(val[p]));
+  } else {
+    rest_row[k - covered] = erow[p];
+    rest_col[k - covered] = colind[p];
+    rest_val[k - covered] = val[p];
+  }
+}
+
+__global__ __launch_bounds__(kSpmmThreads) void panel_dslot_kernel(const int32_t *__restrict__ row_rank, int32_t n,
+                                                                   const int32_t *__restrict__ panel_unit, int32_t npanels,
+                                                                   int32_t *__restrict__ dslot) {
+  const int64_t r = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (r >= n) return;
+  const int32_t rr = row_rank[r];
+  const int32_t panel = rr / kPanelRows;
+  const int32_t u = panel < npanels ? panel_unit[panel] : -1;
+  dslot[r] = u < 0 ? -1 : u * kPanelRows + rr % kPanelRows;
+}
+
+__global__ __launch_bounds__(kSpmmThreads) void panel_expand_rows_kernel(const int32_t *__restrict__ rowptr, int32_t n,
+                                                                         int32_t *__restrict__ row_out) {
+  const int64_t wave = ((int64_t)blockIdx.x * kSpmmThreads + threadIdx.x) / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  if (wave >= n) return;
+  const int32_t s = rowptr[wave], e = rowptr[wave + 1];
+  for (int32_t k = s + lane; k < e; k += kWave) row_out[k] = (int32_t)wave;
+}
+
+}  // namespace cg

@@ -167,6 +167,12 @@ int cg_csr_spmm_xw(cg_csr_t *h, int transpose, const float *d_B, int64_t ldb, co
  *                column-popularity plan last looked up by a wide product of A, of A^T:
  *                tiers in use, -1 when the column counts declined it, 0 when none was considered } */
 int cg_csr_info(const cg_csr_t *h, int64_t info[8]);
+/* Panel plan a wide product of A (transpose != 0: of A^T) last looked up: info[0..7] =
+ * { 1 in use / -1 declined (the dense tiles hold too few of the entries) / 0 none considered yet,
+ *   entries multiplied out of LDS, active tiles, units (workgroups), row panels with several units,
+ *   entries left to the row-wise kernels, entries a tile needs, ranked columns }.  No counterpart in the
+ * reference, which hands the whole product to cusparseSpMM (sparse-extension/sparse_coo_tensor.cu:215-226). */
+int cg_csr_panel_info(const cg_csr_t *h, int transpose, int64_t info[8]);
 /* Device pointers of the arrays the handle owns (transpose != 0: those of A^T). */
 int cg_csr_arrays(const cg_csr_t *h, int transpose, const int32_t **d_rowptr, const int32_t **d_colind,
                   const float **d_values);
@@ -302,6 +308,11 @@ int cg_prof_enable(int on);
  *   "spmm_hub_groups" XCD groups the hot columns are dealt to (1, 2, 4, 8)
  *   "spmm_hub_tiers"  tiers of hot columns (0: chosen from the column counts; groups * tiers <= 64)
  *   "spmm_hub_row"    rows with fewer entries keep all of them in the cold class (0: 64)
+ *   "spmm_panel"      panel plan (dense row-panel x column-block tiles multiplied out of LDS; even widths
+ *                     258..636): -1 never, 1 always, 0 when the tiles hold at least a quarter of the entries
+ *   "spmm_panel_emin" entries a 128 x 32 tile needs to be staged (0: 64)
+ *   "spmm_panel_cols" ranked columns that can be part of a tile (0: 65536)
+ *   "spmm_panel_unit" entries after which the tiles of a row panel go to another workgroup (0: 32768)
  *   "dense_mfma"      -1: dense products on the vector ALU tile kernel only
  *   "coo_cache_blocks" blocks cg_spmm_coo_cached keeps (0: 8; negative: none)
  * An unknown key returns CG_ERR_UNSUPPORTED. */

@@ -541,8 +541,11 @@ def test_spmm_hub_plan_is_declined_when_columns_are_not_skewed(cuda):
         got = A.spmm(Bd)
         assert torch.equal(got, A.spmm(Bd))
         assert key.numel() * f >= 3e9                                  # large enough for a plan to be considered
-        tiers = A.info()["plan_tiers"]
-        assert (tiers >= 1) if skewed else (tiers == -1), tiers
+        tiers, panel = A.info()["plan_tiers"], _panel_info(A)["state"]
+        if skewed:                                                     # one of the two plans takes the popular columns
+            assert panel == 1 or tiers >= 1, (panel, tiers)
+        else:                                                          # both were looked at and declined
+            assert panel == -1 and tiers == -1, (panel, tiers)
         keep = torch.isin(r, sample)
         ref_rows = torch.unique(r[keep])
         remap = torch.full((n,), -1, dtype=torch.long)
@@ -812,3 +815,88 @@ def test_spmm_from_two_host_threads_on_two_streams(cuda, tune):
             assert spmm_error(C, row, col, val, n, n, B) <= REL_TOL
         assert all(torch.equal(results[k][0], C) for C in results[k][2::2])      # cached form: bit-identical repeats
         assert all(torch.equal(results[k][1], C) for C in results[k][3::2])      # handle form likewise
+
+
+def _panel_info(A, transpose=False):
+    import ctypes
+    from cagnet_amd._lib import check, lib
+    buf = (ctypes.c_int64 * 8)()
+    check(lib.cg_csr_panel_info(A._handle, int(transpose), buf), "cg_csr_panel_info")
+    return dict(state=buf[0], covered=buf[1], tiles=buf[2], units=buf[3], split=buf[4], rest=buf[5], emin=buf[6], cols=buf[7])
+
+
+@pytest.mark.parametrize("f", [258, 300, 384, 602, 636])
+@pytest.mark.parametrize("emin,unit", [(4, 300), (24, 100000)])
+def test_spmm_panel_plan_matches_oracle(cuda, tune, f, emin, unit):
+    """Wide products with the panel plan forced on: dense (row panel, column block) tiles are multiplied
+    out of LDS into partial rows, the other entries by the row-wise kernels, which add those rows in.
+    Small units split the heavy panels over several workgroups (their partial blocks are then summed)."""
+    from cagnet_amd import ops
+    row, col, val, n = small_graph(12, 120000, seed=7 * f + emin)
+    B = torch.randn(n, f, generator=torch.Generator().manual_seed(f))
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n, transpose=True)
+    tune("spmm_panel", 1)
+    tune("spmm_panel_emin", emin)
+    tune("spmm_panel_cols", 1024)
+    tune("spmm_panel_unit", unit)
+    got = A.spmm(B.to(cuda))
+    info = _panel_info(A)
+    assert info["state"] == 1 and info["covered"] > 0 and info["covered"] + info["rest"] == row.numel()
+    assert info["tiles"] > 0 and info["units"] >= 1
+    if unit < 1000:
+        assert info["split"] > 0
+    assert spmm_error(got, row, col, val, n, n, B) <= REL_TOL
+    assert torch.equal(got, A.spmm(B.to(cuda)))                      # fixed summation order
+    C0 = torch.randn(n, f, generator=torch.Generator().manual_seed(f + 1))
+    C = C0.to(cuda).clone()
+    A.spmm(B.to(cuda), out=C, beta=1.0)
+    assert spmm_error(C, row, col, val, n, n, B, C0) <= REL_TOL
+    gotT = A.spmm(B.to(cuda), transpose=True)                        # the graph is symmetric: same product
+    assert _panel_info(A, transpose=True)["state"] == 1
+    assert spmm_error(gotT, row, col, val, n, n, B) <= REL_TOL
+    tune("spmm_panel", -1)
+    plain = A.spmm(B.to(cuda))
+    assert spmm_error(plain, row, col, val, n, n, B) <= REL_TOL
+
+
+def test_spmm_panel_plan_rectangular_strided_and_declined(cuda, tune):
+    """A non-symmetric rectangular matrix, B and C as column slices of wider matrices, rows without any
+    entry; and a matrix without dense tiles, on which the automatic choice declines the plan."""
+    from cagnet_amd import ops
+    n, m, f = 700, 1500, 302
+    rng = np.random.default_rng(5)
+    # skewed pattern: popular columns and heavy rows, plus empty rows at the end
+    r = (rng.pareto(1.2, 90000) * 20).astype(np.int64) % (n - 50)
+    c = (rng.pareto(1.2, 90000) * 30).astype(np.int64) % m
+    key = np.unique(r * m + c)
+    row, col = torch.from_numpy(key // m), torch.from_numpy(key % m)
+    val = torch.from_numpy(rng.standard_normal(key.size).astype(np.float32))
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, m, transpose=True)
+    tune("spmm_panel", 1)
+    tune("spmm_panel_emin", 6)
+    tune("spmm_panel_cols", 512)
+    big = torch.randn(m, f + 10, generator=torch.Generator().manual_seed(1)).to(cuda)
+    B = big[:, 4:4 + f]                                              # ld f + 10, base 16 bytes into a row
+    Cbig = torch.zeros(n, f + 6, device=cuda)
+    C = Cbig[:, 2:2 + f]
+    A.spmm(B, out=C)
+    assert _panel_info(A)["state"] == 1
+    assert spmm_error(C, row, col, val, n, m, B.cpu()) <= REL_TOL
+    assert float(Cbig[:, :2].abs().max()) == 0.0 and float(Cbig[:, 2 + f:].abs().max()) == 0.0
+    G = torch.randn(n, f, device=cuda)
+    got = A.spmm(G, transpose=True)
+    assert _panel_info(A, transpose=True)["state"] == 1
+    assert spmm_error(got, col, row, val, m, n, G.cpu()) <= REL_TOL
+    # uniform pattern: no tile reaches the threshold
+    tune("spmm_panel", 0)
+    tune("spmm_panel_emin", 0)
+    tune("spmm_panel_cols", 0)
+    ur, uc, uv = random_coo(3000, 3000, 60000, 3)
+    U = ops.CsrMatrix(_i32(ur, cuda), _i32(uc, cuda), uv.to(cuda), 3000, 3000)
+    Bu = torch.randn(3000, 300, device=cuda)
+    got = U.spmm(Bu)
+    assert _panel_info(U)["state"] in (0, -1)                       # not considered (small product) or declined
+    assert spmm_error(got, ur, uc, uv, 3000, 3000, Bu.cpu()) <= REL_TOL
+    tune("spmm_panel", 1)
+    got = U.spmm(Bu)                                                 # forced: still correct, whatever the coverage
+    assert spmm_error(got, ur, uc, uv, 3000, 3000, Bu.cpu()) <= REL_TOL
