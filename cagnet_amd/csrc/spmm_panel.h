@@ -136,7 +136,28 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
       for (int s = 0; s < kPanelSlots; ++s) {
         const int c = __builtin_popcountll(__ballot(lane < cnt && myslot == (uint32_t)s));
         const int end = i + c;
-        for (; i < end; ++i) {
+        for (; i + 1 < end; i += 2) {  // two rows of B in flight
+          const uint32_t x0 = __builtin_amdgcn_readlane(r.x, i), x1 = __builtin_amdgcn_readlane(r.x, i + 1);
+          const float v0 = __uint_as_float(__builtin_amdgcn_readlane(r.y, i));
+          const float v1 = __uint_as_float(__builtin_amdgcn_readlane(r.y, i + 1));
+          const char *src0 = lbase + (x0 & 0xffu) * rs, *src1 = lbase + (x1 & 0xffu) * rs;
+          float2 b0[CHUNKS], b1[CHUNKS];
+#pragma unroll
+          for (int ch = 0; ch < CHUNKS; ++ch) b0[ch] = *reinterpret_cast<const float2 *>(src0 + ch * 512);
+#pragma unroll
+          for (int ch = 0; ch < CHUNKS; ++ch) b1[ch] = *reinterpret_cast<const float2 *>(src1 + ch * 512);
+#pragma unroll
+          for (int ch = 0; ch < CHUNKS; ++ch) {
+            acc[s][ch].x = fmaf(v0, b0[ch].x, acc[s][ch].x);
+            acc[s][ch].y = fmaf(v0, b0[ch].y, acc[s][ch].y);
+          }
+#pragma unroll
+          for (int ch = 0; ch < CHUNKS; ++ch) {
+            acc[s][ch].x = fmaf(v1, b1[ch].x, acc[s][ch].x);
+            acc[s][ch].y = fmaf(v1, b1[ch].y, acc[s][ch].y);
+          }
+        }
+        if (i < end) {
           const uint32_t x = __builtin_amdgcn_readlane(r.x, i);
           const float v = __uint_as_float(__builtin_amdgcn_readlane(r.y, i));
           const char *src = lbase + (x & 0xffu) * rs;
@@ -148,6 +169,7 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
             acc[s][ch].x = fmaf(v, b[ch].x, acc[s][ch].x);
             acc[s][ch].y = fmaf(v, b[ch].y, acc[s][ch].y);
           }
+          ++i;
         }
       }
     };

@@ -9,8 +9,8 @@ constexpr int64_t kPanelMaxTiles = (int64_t)1 << 26;  // (panel, column block) p
 constexpr double kPanelMinCoverage = 0.25;            // share of the entries the active tiles must hold
 constexpr int32_t kPanelDefaultEmin = 64;             // entries a 128 x 32 tile needs to be staged: twice the
                                                       // 32 gathers its staging costs
-constexpr int32_t kPanelDefaultCols = 65536;          // ranked columns that can be part of a tile
-constexpr int32_t kPanelDefaultUnit = 32768;          // entries after which a panel's tiles start a new unit
+constexpr int32_t kPanelDefaultCols = 131072;         // ranked columns that can be part of a tile
+constexpr int32_t kPanelDefaultUnit = 65536;          // entries after which a panel's tiles start a new unit
 
 struct DevTemps {  // device temporaries of a plan build, freed when the build ends
   std::vector<void *> p;
