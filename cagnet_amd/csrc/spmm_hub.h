@@ -96,6 +96,7 @@ struct CsrSide {
   HubPlan hub[kHubPlans];
   uint64_t hub_used[kHubPlans] = {0, 0};
   uint64_t hub_clock = 0;
+  bool is_rest = false;  // this side is the rest matrix of a panel plan: its dense part is gone already
   PanelPlan panel;  // plan of the wide products that multiply the dense part out of LDS (spmm_panel.h)
   void release() {
     panel.release();
@@ -285,7 +286,9 @@ static int build_hub(CsrSide &s, HubPlan &h, int32_t hot, int32_t hot_single, in
       CG_HIP(hipStreamSynchronize(stream));
       // Measured over R-MAT graphs of 16 to 492 entries per row and blocks of them: with 45 % or more
       // of the entries in the first tier the plan gains 20 to 37 %, with 25 to 29 % it gains 1 to 4 %.
-      if (may_decline && (double)sums[0] < kHubMinHotFraction * (double)nnz) {
+      // (the rest matrix of a panel plan has lost its dense tiles to that plan: what its popular columns still
+      // hold pays from a smaller share on: Reddit shape, rest of 22.8 M entries, 7.6 -> 7.0 ms with a plan)
+      if (may_decline && (double)sums[0] < (s.is_rest ? kHubMinHotFractionRest : kHubMinHotFraction) * (double)nnz) {
         h.declined = true;
         h.groups = groups;
         h.seg = seg;

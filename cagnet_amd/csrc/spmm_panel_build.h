@@ -152,6 +152,7 @@ static int build_panel(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot_req,
   pp.rest = new (std::nothrow) CsrSide();
   if (!pp.rest) CG_FAIL(CG_ERR_ALLOC, "panel plan: host allocation failed");
   CsrSide &rest = *pp.rest;
+  rest.is_rest = true;
   rest.rows = n;
   rest.cols = m;
   rest.nnz = nrest;

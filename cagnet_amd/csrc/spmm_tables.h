@@ -23,6 +23,7 @@ constexpr int kMaxHubClasses = 64;  // column classes of a hub plan (XCD groups 
 constexpr int kHubAutoTiers = 6;    // most tiers the automatic choice takes
 constexpr double kHubTierEntriesPerPair = 2.4;  // entries per (class, row) pair below which a tier no longer pays
 constexpr double kHubMinHotFraction = 0.35;     // share of the entries the first tier must hold for a plan to pay
+constexpr double kHubMinHotFractionRest = 0.12; // the same for the rest matrix of a panel plan
 constexpr int kMaxChunks = 10;  // full-wave teams cover up to 64 * kMaxChunks * VEC columns per launch
 
 // Widest vector the operands allow.
