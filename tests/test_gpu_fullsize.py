@@ -267,3 +267,143 @@ def test_reddit_shape_grid_row_of_blocks(cuda):
         a, hb = val[s:e].double(), H[col[s:e]].double()
         err = ((z[i - b[r]].double() - a @ hb).abs() / (a.abs() @ hb.abs()).clamp_min(1e-30)).max()
         assert float(err) <= REL_TOL, f"row {i}: {float(err)}"
+
+
+# ------------------------------------------------------------------------------------------------
+# whole epochs at full size: forward, loss and backward of the 2-layer model through the library,
+# against torch in fp64 on the device, computed from the COO arrays in the order A (H W) so that
+# no fp64 product is wider than the hidden or class count
+# ------------------------------------------------------------------------------------------------
+def _spmm64(rows_out, tgt, src, val, M, chunk=1 << 23):
+    """out[tgt[k]] += val[k] * M[src[k]] in fp64, entries taken in chunks."""
+    out = torch.zeros(rows_out, M.shape[1], dtype=torch.float64, device=M.device)
+    for lo in range(0, val.numel(), chunk):
+        out.index_add_(0, tgt[lo:lo + chunk], val[lo:lo + chunk].double()[:, None] * M[src[lo:lo + chunk]])
+    return out
+
+
+def _matmul64(X, W, chunk=1 << 20):
+    return torch.cat([X[lo:lo + chunk].double() @ W for lo in range(0, X.shape[0], chunk)])
+
+
+def _xt_g64(X, G, chunk=1 << 20):
+    out = torch.zeros(X.shape[1], G.shape[1], dtype=torch.float64, device=X.device)
+    for lo in range(0, X.shape[0], chunk):
+        out += X[lo:lo + chunk].double().t() @ G[lo:lo + chunk]
+    return out
+
+
+def _close_rel_max(got, ref64, what, tol=2e-4):
+    """End-to-end quantities chain several products: relative to the largest entry of the reference
+    (the per-product 1e-5 bound against the row-sum magnitude is checked product by product above)."""
+    err = float((got.double() - ref64).abs().max()) / max(float(ref64.abs().max()), 1e-30)
+    assert err <= tol, f"{what}: {err}"
+
+
+def _reference_epoch(stages_fwd, stages_bwd, X, W1, W2, y, mask, rows):
+    """fp64 forward + loss + backward.  stages_*: lists of (tgt, src, val, H or None): the layer sums
+    sum_k A_k (H_k W); H None stands for the rank's own operand.  GCNFunc.backward multiplies the
+    gradient by the same blocks as forward (gcn_distr.py:326); stages_bwd carries the peers' gradients."""
+    W1d, W2d = W1.double(), W2.double()
+
+    def layer_sum(stages, own, Wd, which):
+        z = torch.zeros(rows, Wd.shape[1] if Wd is not None else own.shape[1], dtype=torch.float64, device=X.device)
+        for tgt, src, val, peers in stages:
+            op = own if peers is None else peers[which]
+            opw = _matmul64(op, Wd) if Wd is not None else op.double()
+            z += _spmm64(rows, tgt, src, val, opw)
+        return z
+
+    z1 = layer_sum(stages_fwd, X, W1d, 0)
+    h = z1.clamp_min(0.0)
+    z2 = layer_sum(stages_fwd, h, W2d, 1)
+    logp = torch.log_softmax(z2, dim=1)
+    cnt = int(mask.sum())
+    loss = -(logp[torch.arange(rows, device=X.device), y] * mask.double()).sum() / cnt
+    dz2 = torch.exp(logp)
+    dz2[torch.arange(rows, device=X.device), y] -= 1.0
+    dz2 *= (mask.double() / cnt)[:, None]
+    ag2 = layer_sum(stages_bwd, dz2, None, 3)
+    dw2 = h.t() @ ag2
+    dz1 = (ag2 @ W2d.t()) * (z1 > 0).double()
+    ag1 = layer_sum(stages_bwd, dz1, None, 2)
+    dw1 = _xt_g64(X, ag1)
+    return dict(loss=float(loss), hidden=h, outputs=logp, dw1=dw1, dw2=dw2, ag1=ag1, w1=W1d)
+
+
+def _check_epoch(ref, x, w1, w2, h, out, loss, sample_seed):
+    assert abs(float(loss) - ref["loss"]) <= 1e-4, (float(loss), ref["loss"])
+    _close_rel_max(w2.grad, ref["dw2"], "dW2")
+    _close_rel_max(w1.grad, ref["dw1"], "dW1")
+    rows = torch.randint(0, x.shape[0], (256,), generator=torch.Generator().manual_seed(sample_seed)).to(x.device)
+    _close_rel_max(h[rows], ref["hidden"][rows], "sampled rows of the hidden layer")
+    _close_rel_max(out[rows], ref["outputs"][rows], "sampled rows of the outputs")
+    _close_rel_max(x.grad[rows], ref["ag1"][rows] @ ref["w1"].t(), "sampled rows of dX")
+
+
+@pytest.mark.parametrize("spec", [REDDIT, AMAZON], ids=["reddit", "amazon"])
+def test_full_size_epoch_matches_fp64(cuda, spec):
+    """Configurations 3 and 5: one forward + loss + backward of `train`'s model (gcn_distr.py:341-358)
+    at the size the benchmark times, with the library's defaults (plans, fusion), against fp64."""
+    from cagnet_amd import gcn, ops
+    import torch.nn.functional as F
+    if spec is AMAZON and torch.cuda.get_device_properties(cuda).total_memory < 200 * (1 << 30):
+        pytest.skip("needs about 150 GB of device memory")
+    p = synth.make_problem(n=spec["n"], target_nnz=spec["target_nnz"], features=spec["f"], hidden=spec["hidden"],
+                           classes=spec["classes"], mask_fraction=0.66 if spec is REDDIT else 1.0, seed=0, device=cuda)
+    n = p.n
+    blk = ops.CsrMatrix(p.row.int(), p.col.int(), p.val, n, n, is_sorted=True, transpose=True)
+    x = p.x.requires_grad_(True)
+    w1 = p.w1.clone().requires_grad_(True)
+    w2 = p.w2.clone().requires_grad_(True)
+    h = gcn.GCNFunc.apply(x, w1, n, [blk], 0, 1, None, F.relu)
+    z = gcn.GCNFunc.apply(h, w2, n, [blk], 0, 1, None, None)
+    out, loss = gcn.LogSoftmaxNLLLoss.apply(z, p.y, p.train_mask)
+    loss.backward()
+    torch.cuda.synchronize()
+    del blk
+    # backward multiplies by A^T: row and column indices change places
+    fwd = [(p.row, p.col, p.val, None)]
+    bwd = [(p.col, p.row, p.val, None)]
+    ref = _reference_epoch(fwd, bwd, p.x.detach(), p.w1, p.w2, p.y, p.train_mask, n)
+    _check_epoch(ref, x, w1, w2, h.detach(), out.detach(), loss.detach(), 31)
+
+
+def test_reddit_shape_grid_row_epoch_matches_fp64(cuda):
+    """Configuration 4: forward and backward of both layers for the last process row of the 4 x 4 grid,
+    four resident stages per product (gcn_distr_2d.py:333-417 without the broadcasts), against fp64."""
+    from cagnet_amd import gcn, ops
+    import torch.nn.functional as F
+    spec = REDDIT
+    q, r = 4, 3
+    p = synth.make_problem(n=spec["n"], target_nnz=spec["target_nnz"], features=spec["f"], hidden=spec["hidden"],
+                           classes=spec["classes"], mask_fraction=0.66, seed=0, device=cuda)
+    b = synth.block_bounds_2d(p.n, q)
+    rows = b[r + 1] - b[r]
+    r32, c32 = p.row.int(), p.col.int()
+    gen = torch.Generator(device=cuda).manual_seed(37)
+    blocks, coo = [], []
+    for k in range(q):
+        br, bc, bv = ops.coo_block(r32, c32, p.val, b[r], b[r + 1], b[k], b[k + 1])
+        blocks.append(ops.CsrMatrix(br, bc, bv, rows, b[k + 1] - b[k]))
+        coo.append((br.long(), bc.long(), bv))
+    del r32, c32
+
+    def peers(width):
+        return [None if k == r else torch.randn(b[k + 1] - b[k], width, device=cuda, generator=gen) for k in range(q)]
+
+    p1f, p1b, p2f, p2b = peers(spec["f"]), peers(spec["hidden"]), peers(spec["hidden"]), peers(spec["classes"])
+    x = p.x[b[r]:b[r + 1]].clone().requires_grad_(True)
+    y, mask = p.y[b[r]:b[r + 1]], p.train_mask[b[r]:b[r + 1]]
+    w1 = p.w1.clone().requires_grad_(True)
+    w2 = p.w2.clone().requires_grad_(True)
+    h = gcn.GCNFunc.apply(x, w1, rows, blocks, r, q, gcn.ResidentBlocks(p1f, p1b), F.relu)
+    out = gcn.GCNFunc.apply(h, w2, rows, blocks, r, q, gcn.ResidentBlocks(p2f, p2b), F.log_softmax)
+    loss = gcn.masked_nll_loss(out, y, mask)
+    loss.backward()
+    torch.cuda.synchronize()
+    del blocks
+    # per stage: (target rows, source rows, values, (layer-1 fwd, layer-2 fwd, layer-1 bwd, layer-2 bwd) operands)
+    stages = [(coo[k][0], coo[k][1], coo[k][2], None if k == r else (p1f[k], p2f[k], p1b[k], p2b[k])) for k in range(q)]
+    ref = _reference_epoch(stages, stages, x.detach(), p.w1, p.w2, y, mask, rows)
+    _check_epoch(ref, x, w1, w2, h.detach(), out.detach(), loss.detach(), 41)
