@@ -2,18 +2,28 @@
 """Benchmark of the per-rank GCN compute path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload reddit|rmat20|amazon|tiny]
+                    [--no-extra] [--no-cpu-baseline] [--cpu-budget SECONDS] [--optimizer adam|sgd] [--print-losses]
 
-A step is one epoch of the 2-layer GCN (forward, loss, backward, Adam step: `train`,
+A step is one epoch of the 2-layer GCN (forward, loss, backward, optimizer step: `train`,
 gcn_distr.py:341-366) over a seeded synthetic graph that is resident in HBM before the timed
 region starts.  The default workload is the Reddit-shaped configuration the headline metric is
 quoted on: 232,965 vertices, ~114.6 M stored entries, 602 features, hidden 16, 41 classes.
 
 One JSON line is printed:
-  value      SpMM GFLOP/s (2*nnz*f / kernel time) of the dominant launch, the f = 602 forward
-             SpMM, measured with HIP events on the launch stream inside the timed epochs
+  value        SpMM GFLOP/s (2*nnz*f / kernel time) of the dominant launch, the f = 602 forward
+               SpMM, measured with HIP events on the launch stream inside the timed epochs
   ms_per_step  epoch wall time
-  roofline   algorithmic bytes of that launch / its duration, against 8 TB/s
-  cpu_baseline  torch.sparse.mm on the host cores over a bounded row sample of the same product
+  roofline     algorithmic bytes of that launch / its duration, against 8 TB/s; `traffic` is the HBM-side
+               byte count of the same launch from the rocprofv3 counter runs recorded in
+               profiles/spmm_traffic.txt (a profile-run figure, not measured by this run; null when that
+               record was taken with other kernels than the ones this run launched)
+  cpu_baseline torch.sparse.mm of the same product, and one epoch of the CPU restatement, on the host cores
+  configs      (default workload only, unless --no-extra) the other benchmark configurations, each with its
+               algorithmic bytes and roofline fraction: R-MAT scale 20 products at four widths, one rank's
+               share of the 4 x 4 grid, and the Amazon-shaped epoch
+
+`--workload tiny --optimizer sgd --steps 100 --warmup 0 --print-losses` is the plumbing run of the
+single-process harness (the role of gcn.py:104-126): it prints the loss of every epoch to stderr.
 """
 from __future__ import annotations
 
@@ -30,6 +40,7 @@ if str(ROOT) not in sys.path:
     sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+FP32_PEAK_TFLOPS = 157.3
 
 WORKLOADS = {
     # name: graph spec, features, hidden, classes, mask fraction
@@ -44,11 +55,8 @@ WORKLOADS = {
                  desc="R-MAT scale 12 plumbing configuration"),
 }
 
-# HBM bytes per launch of the dominant product (all of its kernels together) from rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE runs, reads scaled by 2.0 and writes by 1.0 as calibrated on a 1 GiB copy
-# kernel: profiles/spmm_f602_reddit_counters.txt (89.3 GB read + 6.0 GB written) and
-# profiles/spmm_amazon_counters.txt (291.6 GB read + 17.6 GB written, f = 300).
-MEASURED_TRAFFIC_BYTES = {"reddit": 95.3e9, "amazon": 309.2e9}
+SPMM_KERNELS = ("spmm_panel", "spmm_hub_hot", "spmm_rowseg", "spmm_reduce", "spmm_hub_reduce")
+TRAFFIC_FILE = ROOT / "profiles" / "spmm_traffic.txt"
 
 
 def spmm_alg_bytes(nnz: int, n: int, m: int, f: int, reads_c: bool) -> int:
@@ -57,50 +65,338 @@ def spmm_alg_bytes(nnz: int, n: int, m: int, f: int, reads_c: bool) -> int:
     return 8 * nnz + 4 * (n + 1) + 4 * m * f + 4 * n * f * (2 if reads_c else 1)
 
 
+def load_traffic() -> dict:
+    """profiles/spmm_traffic.txt: `workload f kernels read_bytes write_bytes` per line (kernels joined by +),
+    HBM-side bytes of one product from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, already scaled."""
+    out = {}
+    if not TRAFFIC_FILE.exists():
+        return out
+    for line in TRAFFIC_FILE.read_text().splitlines():
+        line = line.split("#", 1)[0].split()
+        if len(line) == 5:
+            out[(line[0], int(line[1]))] = dict(kernels=frozenset(line[2].split("+")), read=float(line[3]),
+                                               write=float(line[4]))
+    return out
+
+
+def traffic_of(table: dict, workload: str, f: int, launched: set):
+    """Bytes of the recorded profile run when it launched the same kernels as this run, else None."""
+    rec = table.get((workload, f))
+    if rec is None or rec["kernels"] != frozenset(launched):
+        return None
+    return rec["read"] + rec["write"]
+
+
 def prof_read(lib, name: str):
     ms, cnt = ctypes.c_double(0.0), ctypes.c_int64(0)
     lib.cg_prof_read(name.encode(), ctypes.byref(ms), ctypes.byref(cnt))
     return ms.value, cnt.value
 
 
-def cpu_baseline(prob, f: int, budget_s: float = 25.0):
+def median_ms(fn, reps: int) -> float:
+    import torch
+
+    fn()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        torch.cuda.synchronize()
+        times.append(e0.elapsed_time(e1))
+    times.sort()
+    return times[len(times) // 2]
+
+
+def roofline_fields(alg_bytes: int, flops: float, ms: float, traffic=None) -> dict:
+    achieved = alg_bytes / (ms * 1e-3) / 1e9
+    return {"ms": round(ms, 4), "gflops": round(flops / ms / 1e6, 1), "algorithmic_bytes": int(alg_bytes),
+            "achieved_gbs": round(achieved, 1), "frac": round(achieved / HBM_PEAK_GBS, 5),
+            "time_lower_bound_ms": round(max(alg_bytes / 8e12, flops / (FP32_PEAK_TFLOPS * 1e12)) * 1e3, 4),
+            "traffic": traffic}
+
+
+def cpu_baseline(prob_cpu: dict, f: int, budget_s: float):
     """The oracle's SpMM (torch.sparse.mm on a coalesced COO tensor: the reference's tensor type,
-    gcn_distr.py:493-512, and the torch.sparse line it keeps beside spmm_gpu, gcn_distr_3d.py:478)
-    timed on the host cores over every 8th row of A times the full dense operand."""
+    gcn_distr.py:493-512, and the torch.sparse line it keeps beside spmm_gpu, gcn_distr_3d.py:478) over the
+    whole product, and one epoch of the CPU restatement of `train` (gcn_distr.py:341-366), on the host cores."""
     import torch
     from oracle import gcn_oracle as orc
 
-    stride = 8 if prob.nnz > 4_000_000 else 1
-    keep = (prob.row % stride) == 0
-    row = (prob.row[keep] // stride).cpu()
-    col = prob.col[keep].cpu()
-    val = prob.val[keep].cpu()
-    n_s = (prob.n + stride - 1) // stride
-    B = prob.x[:, :f].cpu().contiguous()
-    A = orc.coo_tensor(row, col, val, n_s, prob.n, torch.float32)
-    nnz_s = int(val.numel())
+    n = prob_cpu["n"]
+    A = orc.coo_tensor(prob_cpu["row"], prob_cpu["col"], prob_cpu["val"], n, n, torch.float32)
+    B = prob_cpu["x"]
+    nnz = int(prob_cpu["val"].numel())
+    t0 = time.perf_counter()
+    torch.sparse.mm(A, B)
+    t_warm = time.perf_counter() - t0
+    reps = max(0, min(3, int((budget_s * 0.6 - t_warm) / max(t_warm, 1e-9))))
     times = []
-    t_begin = time.perf_counter()
-    for rep in range(4):
+    for _ in range(reps):
         t0 = time.perf_counter()
         torch.sparse.mm(A, B)
-        dt = time.perf_counter() - t0
-        if rep > 0:
-            times.append(dt)
-        if time.perf_counter() - t_begin > budget_s and times:
-            break
+        times.append(time.perf_counter() - t0)
+    sample = (f"the whole product torch.sparse.mm(COO fp32 {n} x {n}, {nnz} nnz) times the {n} x {f} dense operand; "
+              f"median of {len(times)} after 1 warm-up")
+    if not times:  # the warm-up alone used the budget: it is the measurement
+        times = [t_warm]
+        sample = sample.replace("median of 0 after 1 warm-up", "a single run, no warm-up (budget)")
     times.sort()
     t = times[len(times) // 2]
-    return {
-        "value": round(2.0 * nnz_s * f / t / 1e9, 3),
+    out = {
+        "value": round(2.0 * nnz * f / t / 1e9, 3),
         "unit": "GFLOP/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"torch.sparse.mm(COO fp32) of every {stride}th row of A ({n_s} x {prob.n}, {nnz_s} nnz) times the "
-                  f"full {prob.n} x {f} dense operand; median of {len(times)} after 1 warm-up; host has "
-                  f"{os.cpu_count()} logical CPUs",
+        "sample": sample + f"; host has {os.cpu_count()} logical CPUs, torch uses {torch.get_num_threads()} threads",
         "seconds_per_rep": round(t, 4),
     }
+    # one epoch of the restatement (Adam, as in the timed GPU epochs), with a warm-up epoch when the budget allows
+    spent = t_warm + sum(times)
+    est_epoch = 1.6 * t  # the f-wide product dominates; the other three products and the dense passes add about half
+    if spent + est_epoch <= budget_s * 1.5:
+        epochs = 2 if spent + 2 * est_epoch <= budget_s * 1.5 else 1
+        ep_times = []
+        for _ in range(epochs):
+            t0 = time.perf_counter()
+            orc.train_epochs(prob_cpu["x"], prob_cpu["w1"], prob_cpu["w2"], [A], prob_cpu["y"], prob_cpu["mask"], epochs=1,
+                             optimizer="adam")
+            ep_times.append(time.perf_counter() - t0)
+        out["epoch_ms"] = round(ep_times[-1] * 1e3, 1)
+        out["epoch_sample"] = ("one epoch (forward, loss, backward, Adam step) of the CPU restatement of train, "
+                               + ("after one warm-up epoch" if epochs == 2 else "no warm-up (budget)"))
+    else:
+        out["epoch_ms"] = None
+        out["epoch_sample"] = "skipped: the CPU budget was used up by the product"
+    return out
+
+
+def read_kernels(lib, f_in: int, hidden: int, classes: int) -> dict:
+    kernels = {}
+    widths = sorted({f_in, hidden, classes, (classes + 3) // 4 * 4, (classes + 15) // 16 * 16})
+    for f in widths:
+        for kname in SPMM_KERNELS:
+            ms, cnt = prof_read(lib, f"{kname}/f={f}")
+            if cnt:
+                kernels[f"{kname}/f={f}"] = {"launches": cnt, "avg_ms": ms / cnt}
+    for kname in ("dense_xw", "dense_gwt", "dense_xtg"):
+        for k in (f_in, hidden):
+            ms, cnt = prof_read(lib, f"{kname}/f={k}")
+            if cnt:
+                kernels[f"{kname}/k={k}"] = {"launches": cnt, "avg_ms": ms / cnt}
+    for kname in ("relu_fwd", "relu_bwd"):
+        ms, cnt = prof_read(lib, kname)
+        if cnt:
+            kernels[kname] = {"launches": cnt, "avg_ms": ms / cnt}
+    for kname in ("log_softmax_fwd", "log_softmax_bwd", "nll_fwd", "nll_bwd", "log_softmax_nll_bwd"):
+        ms, cnt = prof_read(lib, f"{kname}/f={classes}")
+        if cnt:
+            kernels[f"{kname}/c={classes}"] = {"launches": cnt, "avg_ms": ms / cnt}
+    return kernels
+
+
+def run_epochs(prob, spec, blk, steps: int, warmup: int, optimizer: str, keep_losses: bool):
+    """Timed epochs of `train` with the reference's operator sequence (one SpMM, then one dense product per
+    layer, gcn_distr.py:271-275), so that the dominant kernel is exactly the f = f_in SpMM."""
+    import torch
+
+    from cagnet_amd import _lib, gcn
+
+    n, f_in, hidden, classes = prob.n, spec["features"], spec["hidden"], spec["classes"]
+
+    class Data:
+        y = prob.y
+        train_mask = prob.train_mask
+
+    x = prob.x.requires_grad_(True)  # the reference asks for the input gradient too (gcn_distr.py:736)
+    w1 = prob.w1.clone().requires_grad_(True)
+    w2 = prob.w2.clone().requires_grad_(True)
+    opt = torch.optim.Adam([w1, w2], lr=0.01) if optimizer == "adam" else torch.optim.SGD([w1, w2], lr=0.01)
+    losses = []
+    state = {"keep": keep_losses}
+
+    def step():
+        gcn.train(x, w1, w2, n, [blk], opt, Data, 0, 1, None)
+        x.grad = None
+        if state["keep"]:
+            losses.append(float(gcn.train.last_loss))
+
+    gcn.fused_forward = False
+    gcn.fused_loss = False
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.lib.cg_prof_enable(1)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    _lib.lib.cg_prof_enable(0)
+    state["keep"] = False
+    kernels = read_kernels(_lib.lib, f_in, hidden, classes)
+    rec = {"epoch_ms": elapsed / steps * 1e3, "final_loss": float(gcn.train.last_loss), "kernels": kernels, "losses": losses}
+
+    def timed_variant(count):
+        for _ in range(2):
+            step()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(count):
+            step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / count * 1e3
+
+    # library default: the layer product Z = act((A H) W) is fused (no n x f intermediate) where rows are short
+    # enough for it to pay, and the last log_softmax and the loss share one backward kernel
+    count = min(steps, 10)
+    gcn.fused_forward = True
+    gcn.fused_loss = True
+    rec["epoch_ms_default_fusion_policy"] = timed_variant(count)
+    # opt-in product order A (H W): same model, SpMM at the output width; reported beside the headline
+    gcn.spmm_first = False
+    rec["epoch_ms_opt_in_reordered_A_HW"] = timed_variant(count)
+    gcn.spmm_first = True
+    rec["model"] = (x, w1, w2, Data)
+    return rec
+
+
+def dominant_product(kernels: dict, f_in: int):
+    parts = {k: v["avg_ms"] for k, v in kernels.items() if k.startswith("spmm") and k.endswith(f"/f={f_in}")}
+    return parts, (sum(parts.values()) if parts else float("nan"))
+
+
+def extra_rmat20(dev, reps: int) -> dict:
+    """Configuration 2: R-MAT scale 20, A H and A^T G at f in {16, 64, 128, 602}, and the build times."""
+    import torch
+
+    from cagnet_amd import ops, synth
+
+    row, col, n = synth.rmat_graph(20, 16_777_216, 1, dev)
+    val = synth.gcn_normalize(row, col, n)
+    nnz = int(val.numel())
+    r32, c32 = row.int(), col.int()
+    del row, col
+
+    def build(**kw):
+        best, a = float("inf"), None
+        for _ in range(3):
+            del a
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            a = ops.CsrMatrix(**kw)
+            torch.cuda.synchronize()
+            best = min(best, (time.perf_counter() - t0) * 1e3)
+        return a, best
+
+    build(row=r32, col=c32, val=val, n=n, m=n)  # grows the scratch buffers
+    _, t_sorted = build(row=r32, col=c32, val=val, n=n, m=n)
+    A, t_with_t = build(row=r32, col=c32, val=val, n=n, m=n, transpose=True)
+    perm = torch.randperm(nnz, device=dev, generator=torch.Generator(device=dev).manual_seed(3))
+    rp, cp, vp = r32[perm], c32[perm], val[perm]
+    del perm
+    _, t_unsorted = build(row=rp, col=cp, val=vp, n=n, m=n, is_sorted=False)
+    del rp, cp, vp
+    products = []
+    for f in (16, 64, 128, 602):
+        B = torch.randn(n, f, device=dev)
+        C = torch.empty(n, f, device=dev)
+        alg = spmm_alg_bytes(nnz, n, n, f, reads_c=False)
+        for name, tr in (("A@H", False), ("A^T@G", True)):
+            ms = median_ms(lambda: A.spmm(B, out=C, beta=0.0, transpose=tr), reps)
+            products.append(dict(product=name, f=f, **roofline_fields(alg, 2.0 * nnz * f, ms)))
+        del B, C
+    return {"workload": "R-MAT scale 20 (1,048,576 vertices, 16,777,216 directed edges), symmetrised, self-loops, "
+                        "GCN-normalised; median of %d" % reps,
+            "n": n, "nnz": nnz, "bound": "hbm",
+            "build_ms": {"coo2csr_sorted": round(t_sorted, 3), "coo2csr_plus_transpose": round(t_with_t, 3),
+                         "coo2csr_unsorted_radix": round(t_unsorted, 3)},
+            "products": products}
+
+
+def extra_grid_row(prob, spec, dev, reps: int) -> dict:
+    """Configuration 4: the last process row of the 4 x 4 grid on the Reddit-shaped graph: four resident
+    stages per product; the stage loop at f = 602 and forward + backward of both layers."""
+    import torch
+    import torch.nn.functional as F
+
+    from cagnet_amd import gcn, ops, synth
+
+    q, r = 4, 3
+    feats, hidden, classes = spec["features"], spec["hidden"], spec["classes"]
+    b = synth.block_bounds_2d(prob.n, q)
+    rows = b[r + 1] - b[r]
+    r32, c32 = prob.row.int(), prob.col.int()
+    blocks, nnzs = [], []
+    for k in range(q):
+        rr, cc, vv = ops.coo_block(r32, c32, prob.val, b[r], b[r + 1], b[k], b[k + 1])
+        blocks.append(ops.CsrMatrix(rr, cc, vv, rows, b[k + 1] - b[k]))
+        nnzs.append(int(vv.numel()))
+    del r32, c32
+    gen = torch.Generator(device=dev).manual_seed(11)
+
+    def peers(width):
+        return [None if k == r else torch.randn(b[k + 1] - b[k], width, device=dev, generator=gen) for k in range(q)]
+
+    g1 = gcn.ResidentBlocks(peers(feats), peers(hidden))
+    g2 = gcn.ResidentBlocks(peers(hidden), peers(classes))
+    x = prob.x.detach()[b[r]:b[r + 1]].clone().requires_grad_(True)
+    w1 = prob.w1.clone().requires_grad_(True)
+    w2 = prob.w2.clone().requires_grad_(True)
+    y, mask = prob.y[b[r]:b[r + 1]], prob.train_mask[b[r]:b[r + 1]]
+
+    def step():
+        h = gcn.GCNFunc.apply(x, w1, rows, blocks, r, q, g1, F.relu)
+        out = gcn.GCNFunc.apply(h, w2, rows, blocks, r, q, g2, F.log_softmax)
+        loss = gcn.masked_nll_loss(out, y, mask)
+        loss.backward()
+        x.grad = w1.grad = w2.grad = None
+
+    ms_epoch = median_ms(step, reps)
+    H = [x.detach() if k == r else g1.forward[k] for k in range(q)]
+    z = torch.empty(rows, feats, device=dev)
+
+    def stages():
+        for k in range(q):
+            blocks[k].spmm(H[k], out=z, beta=0.0 if k == 0 else 1.0)
+
+    ms_stage = median_ms(stages, reps)
+    alg = sum(spmm_alg_bytes(nz, rows, b[k + 1] - b[k], feats, reads_c=k > 0) for k, nz in enumerate(nnzs))
+    return {"workload": "last process row of the 4 x 4 grid on the Reddit-shaped graph, four stages resident in HBM; "
+                        "median of %d" % reps,
+            "rows": rows, "block_cols": [b[k + 1] - b[k] for k in range(q)], "block_nnz": nnzs, "bound": "hbm",
+            "stage_loop_f%d" % feats: roofline_fields(alg, 2.0 * sum(nnzs) * feats, ms_stage),
+            "fwd_bwd_both_layers_ms": round(ms_epoch, 4)}
+
+
+def extra_amazon(dev, traffic_table: dict, steps: int) -> dict:
+    """Configuration 5: the Amazon-shaped epoch and its f = 300 SpMM."""
+    import torch
+
+    from cagnet_amd import ops, synth
+
+    spec = WORKLOADS["amazon"]
+    prob = synth.make_problem(n=spec["n"], target_nnz=spec["target_nnz"], features=spec["features"], hidden=spec["hidden"],
+                              classes=spec["classes"], mask_fraction=spec["mask"], seed=0, device=dev)
+    blk = ops.CsrMatrix(prob.row.int(), prob.col.int(), prob.val, prob.n, prob.n, is_sorted=True, transpose=True)
+    rec = run_epochs(prob, spec, blk, steps, 2, "adam", False)
+    f_in = spec["features"]
+    parts, dom_ms = dominant_product(rec["kernels"], f_in)
+    alg = spmm_alg_bytes(prob.nnz, prob.n, prob.n, f_in, reads_c=False)
+    launched = {k.split("/")[0] for k in parts}
+    out = {"workload": spec["desc"] + "; Adam, input gradient on; %d timed epochs" % steps, "n": prob.n, "nnz": prob.nnz,
+           "bound": "hbm", "epoch_ms": round(rec["epoch_ms"], 3),
+           "epoch_ms_default_fusion_policy": round(rec["epoch_ms_default_fusion_policy"], 3),
+           "final_loss": rec["final_loss"],
+           "spmm_f%d" % f_in: dict(kernels="+".join(sorted(launched)),
+                                   **roofline_fields(alg, 2.0 * prob.nnz * f_in, dom_ms,
+                                                     traffic_of(traffic_table, "amazon", f_in, launched))),
+           "kernels": {k: {"launches": v["launches"], "avg_ms": round(v["avg_ms"], 5)} for k, v in rec["kernels"].items()}}
+    del rec, blk, prob
+    torch.cuda.empty_cache()
+    return out
 
 
 def main() -> int:
@@ -109,7 +405,11 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="reddit", choices=sorted(WORKLOADS))
+    ap.add_argument("--optimizer", default="adam", choices=("adam", "sgd"))
+    ap.add_argument("--print-losses", action="store_true", help="print the loss of every timed epoch to stderr")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-budget", type=float, default=90.0, help="seconds of host time the CPU baseline may take")
+    ap.add_argument("--no-extra", action="store_true", help="skip the sub-records of the other configurations")
     ap.add_argument("--hip-graph", action="store_true",
                     help="also time the epoch captured into a HIP graph and replayed (always done for --workload tiny)")
     ap.add_argument("--no-dropin", action="store_true",
@@ -127,7 +427,7 @@ def main() -> int:
 
     if not cg_build.LIB_PATH.exists():
         cg_build.build_library()
-    from cagnet_amd import _lib, gcn, ops, synth
+    from cagnet_amd import gcn, ops, synth
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; cagnet_amd has no CPU path", file=sys.stderr)
@@ -135,6 +435,7 @@ def main() -> int:
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     spec = WORKLOADS[args.workload]
+    traffic_table = load_traffic()
 
     t0 = time.perf_counter()
     prob = synth.make_problem(scale=spec.get("scale"), n_edges=spec.get("n_edges"), n=spec.get("n"),
@@ -151,64 +452,12 @@ def main() -> int:
     t_build = time.perf_counter() - t0
     del row32, col32
 
-    class Data:
-        y = prob.y
-        train_mask = prob.train_mask
-
-    x = prob.x.requires_grad_(True)  # the reference asks for the input gradient too (gcn_distr.py:736)
-    w1 = prob.w1.clone().requires_grad_(True)
-    w2 = prob.w2.clone().requires_grad_(True)
-    opt = torch.optim.Adam([w1, w2], lr=0.01)
-
-    def step():
-        gcn.train(x, w1, w2, n, [blk], opt, Data, 0, 1, None)
-        x.grad = None
-
-    # The timed region runs the reference's operator sequence, one SpMM then one dense product per
-    # layer (gcn_distr.py:271-275), so that the headline kernel is exactly the f = f_in SpMM; the
-    # library's default, which folds the W product into that SpMM, is timed separately below.
-    gcn.fused_forward = False
-    gcn.fused_loss = False
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    _lib.lib.cg_prof_enable(1)
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    _lib.lib.cg_prof_enable(0)
-    ms_per_step = elapsed / args.steps * 1e3
-    loss = float(gcn.train.last_loss)
-
-    def timed_variant():
-        for _ in range(2):
-            step()
-        torch.cuda.synchronize()
-        t = time.perf_counter()
-        for _ in range(args.steps):
-            step()
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t) / args.steps * 1e3
-
-    # library default: the layer product Z = act((A H) W) is fused (no n x f intermediate) where rows are
-    # short enough for it to pay (the Amazon shape; on the Reddit shape this equals the headline)
-    gcn.fused_forward = True
-    gcn.fused_loss = True      # ... and the last log_softmax and the loss share one backward kernel
-    fused_ms = timed_variant()
-
-    # opt-in product order A (H W): same model, SpMM at the output width; reported beside the headline
-    gcn.spmm_first = False
-    for _ in range(2):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    reordered_ms = (time.perf_counter() - t0) / args.steps * 1e3
-    gcn.spmm_first = True
+    rec = run_epochs(prob, spec, blk, args.steps, args.warmup, args.optimizer, args.print_losses)
+    for i, l in enumerate(rec["losses"]):
+        print(f"Epoch: {i + 1:03d} loss {l:.6f}", file=sys.stderr)
+    x, _, _, Data = rec["model"]
+    ms_per_step = rec["epoch_ms"]
+    kernels = rec["kernels"]
 
     # the same epoch (library defaults) recorded once into a HIP graph and replayed: for graphs of a few
     # thousand vertices the eager epoch is bound by launches and host work
@@ -220,10 +469,10 @@ def main() -> int:
         graphed.step()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(min(args.steps, 20)):
             graphed.step()
         torch.cuda.synchronize()
-        graph_ms = (time.perf_counter() - t0) / args.steps * 1e3
+        graph_ms = (time.perf_counter() - t0) / min(args.steps, 20) * 1e3
         del graphed
         x.grad = None
 
@@ -247,41 +496,21 @@ def main() -> int:
     ops.coo_cache_clear()
     del c_acc
 
-    kernels = {}
-    widths = sorted({f_in, hidden, classes, (classes + 3) // 4 * 4})  # backward carries 41 classes padded to 44
-    for f in widths:
-        for kname in ("spmm_panel", "spmm_rowseg", "spmm_reduce", "spmm_hub_hot", "spmm_hub_reduce"):
-            ms, cnt = prof_read(_lib.lib, f"{kname}/f={f}")
-            if cnt:
-                kernels[f"{kname}/f={f}"] = {"launches": cnt, "avg_ms": ms / cnt}
-    for kname, ks in (("dense_xw", (f_in, hidden)), ("dense_gwt", (f_in, hidden)), ("dense_xtg", (f_in, hidden))):
-        for k in ks:
-            ms, cnt = prof_read(_lib.lib, f"{kname}/f={k}")
-            if cnt:
-                kernels[f"{kname}/k={k}"] = {"launches": cnt, "avg_ms": ms / cnt}
-
-    for kname in ("relu_fwd", "relu_bwd"):
-        ms, cnt = prof_read(_lib.lib, kname)
-        if cnt:
-            kernels[kname] = {"launches": cnt, "avg_ms": ms / cnt}
-    for kname in ("log_softmax_fwd", "log_softmax_bwd", "nll_fwd", "nll_bwd", "log_softmax_nll_bwd"):
-        ms, cnt = prof_read(_lib.lib, f"{kname}/f={classes}")
-        if cnt:
-            kernels[f"{kname}/c={classes}"] = {"launches": cnt, "avg_ms": ms / cnt}
-
-    # the f = f_in product is one logical launch made of up to four kernels (cold class, its split-row
-    # fold, hot classes, partial-row fold); its duration is the sum of their average durations
-    dom_parts = {k: v["avg_ms"] for k, v in kernels.items() if k.startswith("spmm") and k.endswith(f"/f={f_in}")}
-    dom_ms = sum(dom_parts.values()) if dom_parts else float("nan")
+    # the f = f_in product is one logical launch made of several kernels (panel part, hot classes, cold class
+    # and fold, split-row sums); its duration is the sum of their average durations
+    dom_parts, dom_ms = dominant_product(kernels, f_in)
+    launched = {k.split("/")[0] for k in dom_parts}
     flops = 2.0 * nnz * f_in
     gflops = flops / (dom_ms * 1e-3) / 1e9
     alg_bytes = spmm_alg_bytes(nnz, n, n, f_in, reads_c=False)
     achieved = alg_bytes / (dom_ms * 1e-3) / 1e9
     gather_bytes = 8 * nnz + 4 * (n + 1) + 4 * nnz * f_in + 4 * n * f_in
-    spmm_total_ms = sum(v["avg_ms"] * v["launches"] for k, v in kernels.items() if k.startswith("spmm")) / args.steps
-    dense_total_ms = sum(v["avg_ms"] * v["launches"] for k, v in kernels.items() if k.startswith("dense")) / args.steps
+    traffic = traffic_of(traffic_table, args.workload, f_in, launched)
+    steps = args.steps
+    spmm_total_ms = sum(v["avg_ms"] * v["launches"] for k, v in kernels.items() if k.startswith("spmm")) / steps
+    dense_total_ms = sum(v["avg_ms"] * v["launches"] for k, v in kernels.items() if k.startswith("dense")) / steps
     ew_total_ms = sum(v["avg_ms"] * v["launches"] for k, v in kernels.items()
-                      if not k.startswith(("dense", "spmm"))) / args.steps
+                      if not k.startswith(("dense", "spmm"))) / steps
 
     out = {
         "metric": "SpMM GFLOP/s (2*nnz*f) of the f=%d forward SpMM inside the 2-layer GCN epoch" % f_in,
@@ -297,20 +526,20 @@ def main() -> int:
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": spec["desc"], "name": args.workload, "n": n, "nnz": nnz, "features": f_in,
-                   "hidden": hidden, "classes": classes, "optimizer": "adam lr 0.01", "input_grad": True,
+                   "hidden": hidden, "classes": classes, "optimizer": f"{args.optimizer} lr 0.01", "input_grad": True,
                    "seeds": prob.seeds},
         "epoch_ms": round(ms_per_step, 4),
         "scomp_ms_per_epoch": round(spmm_total_ms, 4),
         "dcomp_ms_per_epoch": round(dense_total_ms, 4),
         "activation_and_loss_ms_per_epoch": round(ew_total_ms, 4),
-        "final_loss": loss,
-        "epoch_ms_default_fusion_policy": round(fused_ms, 4),
-        "epoch_ms_opt_in_reordered_A_HW": round(reordered_ms, 4),
+        "final_loss": rec["final_loss"],
+        "epoch_ms_default_fusion_policy": round(rec["epoch_ms_default_fusion_policy"], 4),
+        "epoch_ms_opt_in_reordered_A_HW": round(rec["epoch_ms_opt_in_reordered_A_HW"], 4),
         "epoch_ms_hip_graph": None if graph_ms is None else round(graph_ms, 4),
         "dropin_spmm_gpu_ms_per_call": dropin_ms,
         "spmm_gbs_algorithmic": round(achieved, 2),
         "spmm_gbs_gather_model": round(gather_bytes / (dom_ms * 1e-3) / 1e9, 2),
-        "spmm_time_lower_bound_ms": round(max(alg_bytes / 8e12, flops / 157.3e12) * 1e3, 4),
+        "spmm_time_lower_bound_ms": round(max(alg_bytes / 8e12, flops / (FP32_PEAK_TFLOPS * 1e12)) * 1e3, 4),
         "kernels": {k: {"launches": v["launches"], "avg_ms": round(v["avg_ms"], 5)} for k, v in kernels.items()},
         "setup_s": {"generate": round(t_gen, 2), "csr_and_transpose_build": round(t_build, 3)},
         "roofline": {
@@ -320,19 +549,35 @@ def main() -> int:
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 5),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "traffic": traffic,
+            "traffic_source": ("HBM-side bytes of this product from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs recorded "
+                               "in profiles/spmm_traffic.txt (a profile-run figure, not measured by this run)"
+                               if traffic is not None else
+                               "no profile run of these kernels is recorded in profiles/spmm_traffic.txt"),
             "algorithmic_bytes": alg_bytes,
             "avg_launch_ms": round(dom_ms, 5),
-            # the same launch priced on the HBM-side bytes rocprofv3 counted for it (profiles/), not a substitute
-            # for `achieved`: how close the kernel runs to the memory system given the traffic it causes
-            "traffic_gbs": (round(MEASURED_TRAFFIC_BYTES[args.workload] / (dom_ms * 1e-3) / 1e9, 1)
-                            if args.workload in MEASURED_TRAFFIC_BYTES else None),
-            "traffic_frac_of_peak": (round(MEASURED_TRAFFIC_BYTES[args.workload] / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
-                                     if args.workload in MEASURED_TRAFFIC_BYTES else None),
+            # the same launch priced on the recorded HBM-side bytes, not a substitute for `achieved`: how
+            # close the kernels run to the memory system given the traffic they cause
+            "traffic_gbs": None if traffic is None else round(traffic / (dom_ms * 1e-3) / 1e9, 1),
+            "traffic_frac_of_peak": None if traffic is None else round(traffic / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         },
     }
+
+    extras = not args.no_extra and args.workload == "reddit"
+    if extras:
+        out["configs"] = {"cfg4_grid_row": extra_grid_row(prob, spec, dev, 5)}
+    prob_cpu = None
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(prob, f_in)
+        prob_cpu = dict(n=n, row=prob.row.cpu(), col=prob.col.cpu(), val=prob.val.cpu(), x=prob.x.detach().cpu().contiguous(),
+                        y=prob.y.cpu(), mask=prob.train_mask.cpu(), w1=prob.w1.cpu(), w2=prob.w2.cpu())
+    del rec, x, Data, blk, prob
+    torch.cuda.empty_cache()
+    if extras:
+        out["configs"]["cfg2_rmat20"] = extra_rmat20(dev, 5)
+        torch.cuda.empty_cache()
+        out["configs"]["cfg5_amazon"] = extra_amazon(dev, traffic_table, 5)
+    if prob_cpu is not None:
+        out["cpu_baseline"] = cpu_baseline(prob_cpu, f_in, args.cpu_budget)
     print(json.dumps(out))
     return 0
 
