@@ -111,10 +111,10 @@ struct CsrSide {
 };
 
 inline void PanelPlan::release() {
-  void *owned[] = {unit_tile, unit_order, tile_kb, tile_wptr, ent, qcol, dslot, split};
+  void *owned[] = {unit_tile, unit_order, hdr, ent, dslot, split};
   for (void *p : owned)
     if (p) (void)hipFree(p);
-  unit_tile = unit_order = tile_kb = tile_wptr = qcol = dslot = split = nullptr;
+  unit_tile = unit_order = hdr = dslot = split = nullptr;
   ent = nullptr;
   if (rest) {
     rest->release();

@@ -37,10 +37,8 @@ struct PanelPlan {
   int32_t ntiles = 0, nunits = 0, nsplit = 0;
   int32_t *unit_tile = nullptr;    // [nunits + 1] tiles of a unit (units never span panels)
   int32_t *unit_order = nullptr;   // [nunits] launch order: heaviest unit first
-  int32_t *tile_kb = nullptr;      // [ntiles] column block of a tile
-  int32_t *tile_wptr = nullptr;    // [ntiles * 16 + 1] records of (tile, wave)
+  int32_t *hdr = nullptr;          // [ntiles * 16 * 4] per (tile, wave): two rows of B to stage, record range
   uint2 *ent = nullptr;            // [covered] {column in block | slot << 8, value bits}, by (tile, wave, slot)
-  int32_t *qcol = nullptr;         // [hot_cols] column (row of B) of every ranked hot column
   int32_t *dslot = nullptr;        // [rows] partial row of a row of A: unit * 128 + position, or -1
   int32_t *split = nullptr;        // [2 * nsplit] (first unit, units) of panels that have several units
   CsrSide *rest = nullptr;         // entries outside active tiles, same rows and columns
@@ -60,11 +58,13 @@ __device__ __forceinline__ void panel_copy4(uint32_t lds_addr, const float *src)
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_addr), "v"(src) : "memory");
 }
 
+// hdr[(tile * 16 + wave) * 4 ..]: the two rows of B the wave stages for the tile and the range of its records.
+// It is read two tiles ahead and the records one tile ahead, so that no load of a tile depends on another
+// load of the same tile: the copies of the next tile go out as soon as the barrier has been passed.
 template <int CHUNKS>
 __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
-    const int32_t *__restrict__ unit_tile, const int32_t *__restrict__ unit_order, const int32_t *__restrict__ tile_kb,
-    const int32_t *__restrict__ tile_wptr, const uint2 *__restrict__ ent, const int32_t *__restrict__ qcol,
-    const float *__restrict__ B, int64_t ldb, float *__restrict__ P, int32_t f) {
+    const int32_t *__restrict__ unit_tile, const int32_t *__restrict__ unit_order, const int32_t *__restrict__ hdr,
+    const uint2 *__restrict__ ent, const float *__restrict__ B, int64_t ldb, float *__restrict__ P, int32_t f) {
   extern __shared__ __align__(16) char panel_lds[];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -74,6 +74,7 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
   const int rs = (f * 4 + 15) & ~15;  // bytes of a staged row: 16-byte aligned for the direct copies
   const int bufsz = kPanelCols * rs;
   constexpr int RPW = kPanelCols / kPanelWaves;  // rows of B a wave stages per tile
+  static_assert(RPW == 2, "the header holds two staged rows per wave");
   float2 acc[kPanelSlots][CHUNKS];
 #pragma unroll
   for (int s = 0; s < kPanelSlots; ++s)
@@ -82,50 +83,64 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
 
   const int nq = f >> 2;     // whole 16-byte pieces of a row of B
   const int tail0 = nq * 4;  // first float of the 4-byte pieces behind them
-  auto stage_row = [&](int t, int r, int buf) {
-    const int kb = tile_kb[t];
-    const int row = wave + r * kPanelWaves;
-    const int q = qcol[kb * kPanelCols + row];
-    const float *src = B + (int64_t)q * ldb;
-    const uint32_t dst = (uint32_t)(uintptr_t)(panel_lds + buf * bufsz + row * rs);
-    for (int p0 = 0; p0 < nq; p0 += kWave) {
-      const int p = p0 + lane;
-      if (p < nq) panel_copy16(dst + p0 * 16, src + 4 * p);
-    }
-    for (int c0 = tail0; c0 < f; c0 += kWave) {
-      const int c = c0 + lane;
-      if (c < f) panel_copy4(dst + c0 * 4, src + c);
+  // A wave stages two rows of B per tile, in pieces of one copy instruction each: per row nx4 of 64 x 16
+  // bytes and, for widths that are not a multiple of 4, one of 4-byte pieces (at most 8 pieces for the
+  // widths this kernel is built for).  One copy instruction keeps the CU's vector memory path busy for 16
+  // cycles, and a wave that issues its copies back to back sits behind those of the 15 other waves: the
+  // pieces of the next tile are therefore issued one at a time, between the slot runs of this tile.
+  const int nx4 = (nq + kWave - 1) / kWave;
+  const int ppr = nx4 + (f > tail0 ? 1 : 0);
+  const int npieces = RPW * ppr;
+  auto stage_piece = [&](int pc, const float *srca, const float *srcb, int buf) {
+    const bool second = pc >= ppr;
+    const int j = second ? pc - ppr : pc;
+    const float *src = second ? srcb : srca;
+    const uint32_t dst = (uint32_t)(uintptr_t)(panel_lds + buf * bufsz + (wave + (second ? kPanelWaves : 0)) * rs);
+    if (j < nx4) {
+      const int p = j * kWave + lane;
+      if (p < nq) panel_copy16(dst + j * (kWave * 16), src + 4 * p);
+    } else {
+      const int c = tail0 + lane;
+      if (c < f) panel_copy4(dst + tail0 * 4, src + c);
     }
   };
-  // records of a (tile, wave), first 64 of them: one per lane, loaded a tile ahead
-  auto rec_load = [&](int t, uint2 &r, int &b0, int &b1) {
-    b0 = tile_wptr[t * kPanelWaves + wave];
-    b1 = tile_wptr[t * kPanelWaves + wave + 1];
-    int idx = b0 + lane;
-    idx = idx < b1 ? idx : (b1 > b0 ? b1 - 1 : 0);  // unconditional, clamped
-    r = ent[idx];
+  // lanes 0..3 of a wave fetch the four words of its header (a vector load: its wait is the one at the
+  // end of the tile, with the copies, not the LDS counter)
+  auto hdr_load = [&](int t) { return hdr[((int64_t)t * kPanelWaves + wave) * 4 + (lane & 3)]; };
+  // records of a (tile, wave), 64 of them from `first`: one per lane, clamped to the range
+  auto rec_load = [&](int first, int b0, int b1) {
+    int idx = first + lane;
+    idx = idx < b1 ? idx : (b1 > b0 ? b1 - 1 : 0);
+    return ent[idx];
   };
   uint2 rec = make_uint2(0u, 0u);
-  int e0 = 0, e1 = 0;
+  int e0 = 0, e1 = 0, hn = 0;
   if (t1 > t0) {
-#pragma unroll
-    for (int r = 0; r < RPW; ++r) stage_row(t0, r, 0);
-    rec_load(t0, rec, e0, e1);
+    const int h0 = hdr_load(t0);
+    hn = hdr_load(t0 + 1 < t1 ? t0 + 1 : t0);
+    const float *srca = B + (int64_t)__builtin_amdgcn_readlane(h0, 0) * ldb;
+    const float *srcb = B + (int64_t)__builtin_amdgcn_readlane(h0, 1) * ldb;
+    for (int pc = 0; pc < npieces; ++pc) stage_piece(pc, srca, srcb, 0);
+    e0 = __builtin_amdgcn_readlane(h0, 2);
+    e1 = __builtin_amdgcn_readlane(h0, 3);
+    rec = rec_load(e0, e0, e1);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   for (int t = t0; t < t1; ++t) {
     const int buf = (t - t0) & 1;
-    const int tn = t + 1 < t1 ? t + 1 : t;  // the last tile stages itself again: no branch around the copies
     const char *lbase = panel_lds + buf * bufsz + lane * 8;
-    // The records of this tile arrived before the last barrier.  Touching them here puts the compiler's
-    // wait for them ahead of the copies it cannot see, so that nothing below waits for those.
-    asm volatile("" ::"v"(rec.x), "v"(rec.y));
-    uint2 recn;
-    int e0n, e1n;
-    rec_load(tn, recn, e0n, e1n);
-#pragma unroll
-    for (int r = 0; r < RPW; ++r) stage_row(tn, r, buf ^ 1);
+    // The records of this tile and the header of the next arrived before the last barrier.  Touching them
+    // here puts the compiler's wait for them ahead of the copies it cannot see, so that nothing below
+    // waits for those.
+    asm volatile("" ::"v"(rec.x), "v"(rec.y), "v"(hn));
+    // the next tile (the last tile names itself and is staged once more)
+    const int q0 = __builtin_amdgcn_readlane(hn, 0), q1 = __builtin_amdgcn_readlane(hn, 1);
+    const int e0n = __builtin_amdgcn_readlane(hn, 2), e1n = __builtin_amdgcn_readlane(hn, 3);
+    const int hn2 = hdr_load(t + 2 < t1 ? t + 2 : t1 - 1);
+    const uint2 recn = rec_load(e0n, e0n, e1n);
+    const float *srca = B + (int64_t)q0 * ldb, *srcb = B + (int64_t)q1 * ldb;
+    int piece = 0;
 
     // records are sorted by slot: the lanes' ballots give the length of every slot's run, and a run
     // adds into that slot's registers (static register indices)
@@ -134,6 +149,10 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
       int i = 0;
 #pragma unroll
       for (int s = 0; s < kPanelSlots; ++s) {
+        if (piece < npieces) {
+          stage_piece(piece, srca, srcb, buf ^ 1);
+          ++piece;
+        }
         const int c = __builtin_popcountll(__ballot(lane < cnt && myslot == (uint32_t)s));
         const int end = i + c;
         for (; i + 1 < end; i += 2) {  // two rows of B in flight
@@ -173,20 +192,20 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
         }
       }
     };
-    {
-      const int cnt = e1 - e0;
-      process(rec, cnt > kWave ? kWave : cnt);
+    // 64 records at a time; a dense tile's further records are fetched while the batch before them is multiplied
+    uint2 cur = rec;
+    for (int base = e0; base < e1; base += kWave) {
+      const int left = e1 - base;
+      uint2 nxt = cur;
+      if (left > kWave) nxt = rec_load(base + kWave, e0, e1);
+      process(cur, left > kWave ? kWave : left);
+      cur = nxt;
     }
-    for (int base = e0 + kWave; base < e1; base += kWave) {  // further records of a dense tile, fetched on demand
-      int idx = base + lane;
-      idx = idx < e1 ? idx : e1 - 1;
-      const uint2 r2 = ent[idx];
-      const int cnt = e1 - base;
-      process(r2, cnt > kWave ? kWave : cnt);
-    }
+    for (; piece < npieces; ++piece) stage_piece(piece, srca, srcb, buf ^ 1);  // a wave without records in this tile
     rec = recn;
     e0 = e0n;
     e1 = e1n;
+    hn = hn2;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   }
@@ -336,6 +355,19 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_entry_finish_kernel(
     rest_col[k - covered] = colind[p];
     rest_val[k - covered] = val[p];
   }
+}
+
+// hdr[(t * 16 + w) * 4 ..] = {row of B of column w of the tile's block, the same of column w + 16, first record, end}
+__global__ __launch_bounds__(kSpmmThreads) void panel_hdr_kernel(const int32_t *__restrict__ tile_kb,
+                                                                  const int32_t *__restrict__ tile_wptr,
+                                                                  const int32_t *__restrict__ qcol, int64_t ntiles,
+                                                                  int4 *__restrict__ hdr) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k >= ntiles * kPanelWaves) return;
+  const int64_t t = k / kPanelWaves;
+  const int w = (int)(k % kPanelWaves);
+  const int64_t c = (int64_t)tile_kb[t] * kPanelCols + w;
+  hdr[k] = make_int4(qcol[c], qcol[c + kPanelWaves], tile_wptr[k], tile_wptr[k + 1]);
 }
 
 __global__ __launch_bounds__(kSpmmThreads) void panel_dslot_kernel(const int32_t *__restrict__ row_rank, int32_t n,

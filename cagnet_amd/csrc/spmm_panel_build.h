@@ -82,7 +82,8 @@ static int build_panel(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot_req,
   int32_t *row_rank = nullptr, *col_rank = nullptr;
   CG_TRY(tmp.alloc((void **)&row_rank, (size_t)n * 4));
   CG_TRY(tmp.alloc((void **)&col_rank, (size_t)m * 4));
-  CG_TRY(dev_alloc((void **)&pp.qcol, (size_t)hot * 4));
+  int32_t *qcol = nullptr;  // row of B of every ranked hot column
+  CG_TRY(tmp.alloc((void **)&qcol, (size_t)hot * 4));
   {
     DevTemps t2;
     SortBuffers buf;
@@ -113,7 +114,7 @@ static int build_panel(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot_req,
     CG_TRY(radix_sort_pairs(buf, m, bits_for((int32_t)maxcount + 1), 0, &set, stream));
     panel_invert_kernel<<<gm, kSpmmThreads, 0, stream>>>(buf.payload[set], m, col_rank);
     CG_LAUNCH_CHECK();
-    CG_HIP(hipMemcpyAsync(pp.qcol, buf.payload[set], (size_t)hot * 4, hipMemcpyDeviceToDevice, stream));
+    CG_HIP(hipMemcpyAsync(qcol, buf.payload[set], (size_t)hot * 4, hipMemcpyDeviceToDevice, stream));
     CG_HIP(hipStreamSynchronize(stream));
   }
 
@@ -142,10 +143,10 @@ static int build_panel(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot_req,
   if (ntiles * kPanelWaves + 1 > 0x7fffffffLL) return decline();
 
   // 3. tables of the active tiles
-  int32_t *tile_panel = nullptr;
-  CG_TRY(dev_alloc((void **)&pp.tile_kb, (size_t)ntiles * 4));
+  int32_t *tile_panel = nullptr, *tile_kb = nullptr, *tile_wptr = nullptr;
+  CG_TRY(tmp.alloc((void **)&tile_kb, (size_t)ntiles * 4));
   CG_TRY(tmp.alloc((void **)&tile_panel, (size_t)ntiles * 4));
-  panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, tindex, tiles, (uint32_t)emin, nkb, pp.tile_kb, tile_panel);
+  panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, tindex, tiles, (uint32_t)emin, nkb, tile_kb, tile_panel);
   CG_LAUNCH_CHECK();
 
   // 4. one stable sort puts the covered entries first, by (tile, wave, slot), and leaves the others
@@ -162,7 +163,8 @@ static int build_panel(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot_req,
   CG_TRY(dev_alloc((void **)&rest.colind, (size_t)nrest * 4));
   CG_TRY(dev_alloc((void **)&rest.val, (size_t)nrest * 4));
   CG_TRY(dev_alloc((void **)&pp.ent, (size_t)covered * 8));
-  CG_TRY(dev_alloc((void **)&pp.tile_wptr, (size_t)(ntiles * kPanelWaves + 1) * 4));
+  CG_TRY(tmp.alloc((void **)&tile_wptr, (size_t)(ntiles * kPanelWaves + 1) * 4));
+  CG_TRY(dev_alloc((void **)&pp.hdr, (size_t)ntiles * kPanelWaves * 16));
   {
     DevTemps t2;
     SortBuffers buf;
@@ -179,7 +181,10 @@ static int build_panel(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot_req,
     panel_entry_finish_kernel<<<ge, kSpmmThreads, 0, stream>>>(buf.key_b[set], buf.payload[set], nnz, covered, erow, s.colind,
                                                                s.val, col_rank, pp.ent, rest_row, rest.colind, rest.val);
     CG_LAUNCH_CHECK();
-    CG_TRY(launch_rowptr(buf.key_a[set], covered, sentinel, pp.tile_wptr, stream));
+    CG_TRY(launch_rowptr(buf.key_a[set], covered, sentinel, tile_wptr, stream));
+    panel_hdr_kernel<<<(unsigned)ceil_div64(ntiles * kPanelWaves, kSpmmThreads), kSpmmThreads, 0, stream>>>(
+        tile_kb, tile_wptr, qcol, ntiles, (int4 *)pp.hdr);
+    CG_LAUNCH_CHECK();
     CG_TRY(launch_rowptr(rest_row, nrest, n, rest.rowptr, stream));
     CG_HIP(hipStreamSynchronize(stream));
   }
@@ -191,7 +196,7 @@ static int build_panel(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot_req,
     // entries of active tile k = difference of the scanned kept[] at its all-tile index; read them compacted
     // through the (tile, wave) table instead: tile_wptr[16 k] is the first record of tile k
     std::vector<int32_t> h_wptr((size_t)ntiles * kPanelWaves + 1);
-    CG_HIP(hipMemcpyAsync(h_wptr.data(), pp.tile_wptr, h_wptr.size() * 4, hipMemcpyDeviceToHost, stream));
+    CG_HIP(hipMemcpyAsync(h_wptr.data(), tile_wptr, h_wptr.size() * 4, hipMemcpyDeviceToHost, stream));
     CG_HIP(hipMemcpyAsync(h_panel.data(), tile_panel, (size_t)ntiles * 4, hipMemcpyDeviceToHost, stream));
     CG_HIP(hipStreamSynchronize(stream));
     for (int64_t k = 0; k <= ntiles; ++k) h_base[(size_t)k] = h_wptr[(size_t)k * kPanelWaves];
@@ -275,8 +280,8 @@ static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_
       CG_HIP(hipFuncSetAttribute((const void *)spmm_panel_kernel<CH>, hipFuncAttributeMaxDynamicSharedMemorySize,     \
                                  (int)lds));                                                                          \
     }                                                                                                                 \
-    spmm_panel_kernel<CH><<<(unsigned)pp.nunits, kPanelThreads, lds, stream>>>(pp.unit_tile, pp.unit_order, pp.tile_kb, \
-                                                                               pp.tile_wptr, pp.ent, pp.qcol, B, ldb, P, f); \
+    spmm_panel_kernel<CH><<<(unsigned)pp.nunits, kPanelThreads, lds, stream>>>(pp.unit_tile, pp.unit_order, pp.hdr, pp.ent, B, \
+                                                                               ldb, P, f);                                 \
   } break;
     switch (chunks) {
       CG_PANEL(3)
