@@ -438,9 +438,15 @@ def main() -> int:
     traffic_table = load_traffic()
 
     t0 = time.perf_counter()
+    # the plumbing configuration is drawn with torch's CPU generator, like the golden losses it is checked
+    # against (a device generator gives another instance for the same seed); the large shapes are drawn on the GPU
+    gen_dev = "cpu" if args.workload == "tiny" else dev
     prob = synth.make_problem(scale=spec.get("scale"), n_edges=spec.get("n_edges"), n=spec.get("n"),
                               target_nnz=spec.get("target_nnz"), features=spec["features"], hidden=spec["hidden"],
-                              classes=spec["classes"], mask_fraction=spec["mask"], seed=args.seed, device=dev)
+                              classes=spec["classes"], mask_fraction=spec["mask"], seed=args.seed, device=gen_dev)
+    if gen_dev == "cpu":
+        for name in ("row", "col", "val", "x", "y", "train_mask", "w1", "w2"):
+            setattr(prob, name, getattr(prob, name).to(dev))
     torch.cuda.synchronize()
     t_gen = time.perf_counter() - t0
     n, nnz, f_in, hidden, classes = prob.n, prob.nnz, spec["features"], spec["hidden"], spec["classes"]

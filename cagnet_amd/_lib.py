@@ -20,7 +20,7 @@ CG_ERR_UNSUPPORTED = 8
 STATUS_NAMES = {
     0: "CG_OK", 1: "CG_ERR_NULL", 2: "CG_ERR_SIZE", 3: "CG_ERR_OVERFLOW", 4: "CG_ERR_UNSORTED",
     5: "CG_ERR_INDEX", 6: "CG_ERR_HIP", 7: "CG_ERR_ALLOC", 8: "CG_ERR_UNSUPPORTED",
-    9: "CG_ERR_NO_TRANSPOSE", 10: "CG_ERR_ALIAS",
+    9: "CG_ERR_NO_TRANSPOSE", 10: "CG_ERR_ALIAS", 11: "CG_ERR_CAPTURE",
 }
 
 
@@ -51,6 +51,8 @@ _SIGNATURES = {
     "cg_coo_cache_info": [POINTER(c_int64)],
     "cg_csr_create": [POINTER(c_void_p), P, P, P, c_int64, c_int32, c_int32, c_uint32, P],
     "cg_csr_destroy": [P],
+    "cg_csr_unpin": [P, POINTER(c_int64)],
+    "cg_scratch_release": [P, POINTER(c_int64)],
     "cg_csr_spmm": [P, c_int, P, c_int64, P, c_int64, c_int32, c_float, P],
     "cg_csr_spmm_xw": [P, c_int, P, c_int64, P, c_int64, c_float, P, c_int64, P, c_int64, c_int32, c_int32, c_int, P],
     "cg_csr_info": [P, POINTER(c_int64)],

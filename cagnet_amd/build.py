@@ -46,9 +46,18 @@ def sources() -> list[Path]:
     return sorted(CSRC_DIR.glob("*.hip"))
 
 
-def _compile_one(src: Path) -> Path:
-    obj = OBJ_DIR / (src.stem + ".o")
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", str(src), "-o", str(obj)]
+# Host-side AddressSanitizer + UndefinedBehaviorSanitizer build (the device code is compiled as usual): every
+# -fsanitize= sits directly behind -Xarch_host so that it reaches the host pass only.
+SAN_LIB_PATH = LIB_DIR / "libcagnet_amd_hostsan.so"
+SAN_OBJ_DIR = LIB_DIR / "obj_hostsan"
+HOST_SANITIZE_FLAGS = ["-g", "-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined",
+                       "-Xarch_host", "-fno-sanitize-recover=undefined", "-Xarch_host", "-fno-omit-frame-pointer"]
+
+
+def _compile_one(src: Path, sanitize: bool = False) -> Path:
+    obj = (SAN_OBJ_DIR if sanitize else OBJ_DIR) / (src.stem + ".o")
+    flags = [f for f in HIPCC_FLAGS if f != "-O3"] + ["-O1"] + HOST_SANITIZE_FLAGS if sanitize else HIPCC_FLAGS
+    cmd = [_hipcc(), *flags, "-c", str(src), "-o", str(obj)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src.name}:\n{proc.stdout}\n{proc.stderr}")
@@ -79,5 +88,45 @@ def build_library(jobs: int | None = None, verbose: bool = True) -> Path:
     return LIB_PATH
 
 
+def build_host_sanitized(jobs: int | None = None) -> Path:
+    """The same sources with the host code instrumented by ASan and UBSan, as
+    lib/libcagnet_amd_hostsan.so.  It is only ever linked into a sanitized test driver
+    (tests/abi_host_driver.cpp); the product never loads it."""
+    SAN_OBJ_DIR.mkdir(parents=True, exist_ok=True)
+    srcs = sources()
+    jobs = jobs or min(len(srcs), int(os.environ.get("MAX_JOBS", "8")))
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        objs = list(pool.map(lambda src: _compile_one(src, True), srcs))
+    cmd = [_hipcc(), "-shared", "-fPIC", f"--offload-arch={ARCH}", "-Xarch_host", "-fsanitize=address", "-Xarch_host",
+           "-fsanitize=undefined", "-o", str(SAN_LIB_PATH), *map(str, objs)]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"sanitized link failed:\n{proc.stdout}\n{proc.stderr}")
+    return SAN_LIB_PATH
+
+
+SAN_DRIVER_SRC = PKG_DIR.parent / "tests" / "abi_host_driver.cpp"
+SAN_DRIVER_PATH = LIB_DIR / "abi_host_driver"
+
+
+def build_host_driver() -> Path:
+    """tests/abi_host_driver.cpp compiled with ASan + UBSan and linked against the sanitized library (built
+    first).  The program carries the sanitizer runtime itself, so it runs without any preloading."""
+    lib = build_host_sanitized()
+    rocm = Path(os.environ.get("ROCM_PATH", "/opt/rocm"))
+    clang = rocm / "llvm" / "bin" / "clang++"
+    cmd = [str(clang), "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
+           "-fno-omit-frame-pointer", "-D__HIP_PLATFORM_AMD__", f"-I{rocm / 'include'}", f"-I{PKG_DIR.parent / 'include'}",
+           str(SAN_DRIVER_SRC), "-o", str(SAN_DRIVER_PATH), str(lib), f"-L{rocm / 'lib'}", "-lamdhip64",
+           f"-Wl,-rpath,{LIB_DIR}", f"-Wl,-rpath,{rocm / 'lib'}"]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"sanitized driver build failed:\n{proc.stdout}\n{proc.stderr}")
+    return SAN_DRIVER_PATH
+
+
 if __name__ == "__main__":
-    build_library()
+    if "--host-sanitize" in sys.argv[1:]:
+        print(build_host_driver())
+    else:
+        build_library()

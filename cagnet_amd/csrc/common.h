@@ -40,6 +40,26 @@ int hip_fail(hipError_t e, const char *what, const char *file, int line);
 enum ScratchSlot { kSlotA = 0, kSlotB = 1, kSlotC = 2, kSlotD = 3, kSlotE = 4, kNumSlots = 5 };
 int scratch_get(hipStream_t stream, int slot, size_t bytes, void **out);
 
+// Frees every scratch buffer of (current device, stream), parked ones included, after the stream has drained.
+int scratch_release(hipStream_t stream, int64_t *released_bytes);
+
+// ---- memory that a captured graph may still name -------------------------------------------------
+// A HIP graph captured from calls of this library keeps the raw addresses of the scratch buffers and
+// of the handle's tables those calls used.  A buffer or table that was used under capture is therefore
+// never freed by later calls: when it has to be replaced (scratch growth, plan eviction, schedule
+// recycling, a changed tuning value) the old memory is parked and only the owner's release frees it.
+bool stream_capturing(hipStream_t stream);
+// Free `p`, or park it when the calling thread is inside a product on a pinned handle (ParkScope).
+void table_free(void *p);
+struct ParkScope {  // tables released inside the scope go to `sink` instead of hipFree (sink == nullptr: no change)
+  void *prev;
+  bool set;
+  explicit ParkScope(void *sink_vector);
+  ~ParkScope();
+};
+// CG_ERR_CAPTURE unless `stream` is not being captured: for steps that allocate, synchronise or read back.
+int refuse_under_capture(hipStream_t stream, const char *what);
+
 // ---- optional kernel timing with HIP events on the launch stream (runtime.hip) -------------------
 bool prof_on();
 void prof_begin(const char *name, int tag, hipStream_t stream);  // tag < 0: no "/f=" suffix

@@ -248,7 +248,7 @@ __global__ __launch_bounds__(kEwThreads) void nll_bwd_vec_kernel(const float *__
   for (int64_t r0 = w.first; r0 < n; r0 += w.step) {
     const int64_t row = r0 + w.sub;
     const int64_t rc = row < n ? row : n - 1;
-    const bool on = total > 0 && (!mask || mask[rc]);
+    const bool on = total > 0 && (!mask || mask[rc]) && y[rc] >= 0 && y[rc] < c;
     const float wgt = on ? unit : 0.f;
     const int32_t hit = (int32_t)(y[rc] - col);  // 0..3 when the label falls into this lane's piece
     float4 v;
@@ -293,9 +293,11 @@ __global__ __launch_bounds__(kEwThreads) void nll_partial_kernel(const float *__
   float v = 0.f;
   int cnt = 0;
   if (i < n && (!mask || mask[i])) {
-    cnt = 1;
     const int64_t label = y[i];
-    if (label >= 0 && label < c) v = -logp[i * ld + label];
+    if (label >= 0 && label < c) {  // other labels are ignored, as F.nll_loss ignores ignore_index rows
+      cnt = 1;
+      v = -logp[i * ld + label];
+    }
   }
 #pragma unroll
   for (int off = kWave / 2; off > 0; off >>= 1) {
@@ -324,15 +326,16 @@ __global__ __launch_bounds__(kEwThreads) void nll_partial_kernel(const float *__
 // The same partial sums from the per-row contributions a fused forward pass left behind: same rows
 // per workgroup and the same order of additions as nll_partial_kernel, so the loss is the same float.
 __global__ __launch_bounds__(kEwThreads) void nll_rows_partial_kernel(const float *__restrict__ rowloss,
+                                                                      const int64_t *__restrict__ y,
                                                                       const uint8_t *__restrict__ mask, int64_t n,
-                                                                      float *__restrict__ psum,
+                                                                      int32_t c, float *__restrict__ psum,
                                                                       int64_t *__restrict__ pcnt) {
   __shared__ float ssum[kEwThreads / kWave];
   __shared__ int scnt[kEwThreads / kWave];
   const int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x;
   float v = 0.f;
   int cnt = 0;
-  if (i < n && (!mask || mask[i])) {
+  if (i < n && (!mask || mask[i]) && y[i] >= 0 && y[i] < c) {
     cnt = 1;
     v = rowloss[i];
   }
@@ -398,9 +401,9 @@ __global__ __launch_bounds__(kEwThreads) void nll_bwd_kernel(const float *__rest
   const int j = threadIdx.x % kTeam;
   if (row >= n) return;
   const int64_t total = *count;
-  const bool on = total > 0 && (!mask || mask[row]);
-  const float w = on ? (gscale ? *gscale : 1.f) / (float)total : 0.f;
   const int64_t label = y[row];
+  const bool on = total > 0 && (!mask || mask[row]) && label >= 0 && label < c;
+  const float w = on ? (gscale ? *gscale : 1.f) / (float)total : 0.f;
   float *d = dst + row * ldd;
   for (int32_t k = j; k < c; k += kTeam) {
     const float onehot = (k == label) ? 1.f : 0.f;
@@ -610,7 +613,7 @@ int cg_log_softmax_nll_fwd(const float *d_z, int64_t ldz, const int64_t *d_y, co
   }
   ProfScope prof("nll_fwd", c, s);
   if (parts > 0) {
-    nll_rows_partial_kernel<<<(unsigned)parts, kEwThreads, 0, s>>>(rowloss, d_mask, n, psum, pcnt);
+    nll_rows_partial_kernel<<<(unsigned)parts, kEwThreads, 0, s>>>(rowloss, d_y, d_mask, n, c, psum, pcnt);
     CG_LAUNCH_CHECK();
   }
   nll_final_kernel<<<1, kEwThreads, 0, s>>>(psum, pcnt, parts, d_loss, d_count);

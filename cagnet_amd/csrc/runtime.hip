@@ -26,24 +26,69 @@ int hip_fail(hipError_t e, const char *what, const char *file, int line) {
 struct ScratchBuf {
   void *ptr = nullptr;
   size_t bytes = 0;
+  bool pinned = false;  // handed out while its stream was being captured: a graph may name it
 };
 
 static std::mutex g_scratch_mu;
 static std::map<std::tuple<int, hipStream_t, int>, ScratchBuf> g_scratch;
+static std::map<std::pair<int, hipStream_t>, std::vector<ScratchBuf>> g_scratch_parked;
 
-// Grow-only.  Growing frees the old buffer after the stream has drained, so work already
-// enqueued on `stream` that still reads it stays valid.
+bool stream_capturing(hipStream_t stream) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &st) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return st == hipStreamCaptureStatusActive;
+}
+
+int refuse_under_capture(hipStream_t stream, const char *what) {
+  if (stream_capturing(stream))
+    CG_FAIL(CG_ERR_CAPTURE, "%s cannot run while its stream is being captured: run the same call once before the capture",
+            what);
+  return CG_OK;
+}
+
+static thread_local std::vector<void *> *g_park_sink = nullptr;
+
+void table_free(void *p) {
+  if (!p) return;
+  if (g_park_sink)
+    g_park_sink->push_back(p);
+  else
+    (void)hipFree(p);
+}
+
+ParkScope::ParkScope(void *sink_vector) : prev(g_park_sink), set(sink_vector != nullptr) {
+  if (set) g_park_sink = static_cast<std::vector<void *> *>(sink_vector);
+}
+ParkScope::~ParkScope() {
+  if (set) g_park_sink = static_cast<std::vector<void *> *>(prev);
+}
+
+// Grow-only.  Growing frees the old buffer after the stream has drained, so work already enqueued on
+// `stream` that still reads it stays valid; a buffer that was handed out under capture is parked
+// instead (a graph replays with its address) until scratch_release.
 int scratch_get(hipStream_t stream, int slot, size_t bytes, void **out) {
   int dev = 0;
   CG_HIP(hipGetDevice(&dev));
+  const bool capturing = stream_capturing(stream);
   std::lock_guard<std::mutex> lock(g_scratch_mu);
   ScratchBuf &b = g_scratch[std::make_tuple(dev, stream, slot)];
   if (bytes > b.bytes) {
+    if (capturing)
+      CG_FAIL(CG_ERR_CAPTURE,
+              "scratch slot %d would grow from %zu to %zu bytes while its stream is being captured: run the same call "
+              "once before the capture",
+              slot, b.bytes, bytes);
     if (b.ptr) {
-      CG_HIP(hipStreamSynchronize(stream));
-      CG_HIP(hipFree(b.ptr));
-      b.ptr = nullptr;
-      b.bytes = 0;
+      if (b.pinned) {
+        g_scratch_parked[std::make_pair(dev, stream)].push_back(b);
+      } else {
+        CG_HIP(hipStreamSynchronize(stream));
+        CG_HIP(hipFree(b.ptr));
+      }
+      b = ScratchBuf();
     }
     size_t want = bytes + bytes / 4;  // headroom so slowly growing requests do not reallocate each time
     want = (want + 255) & ~(size_t)255;
@@ -56,7 +101,34 @@ int scratch_get(hipStream_t stream, int slot, size_t bytes, void **out) {
     }
     b.bytes = want;
   }
+  if (capturing) b.pinned = true;
   *out = b.ptr;
+  return CG_OK;
+}
+
+int scratch_release(hipStream_t stream, int64_t *released_bytes) {
+  int dev = 0;
+  CG_HIP(hipGetDevice(&dev));
+  CG_TRY(refuse_under_capture(stream, "cg_scratch_release"));
+  CG_HIP(hipStreamSynchronize(stream));
+  int64_t total = 0;
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  for (int slot = 0; slot < kNumSlots; ++slot) {
+    auto it = g_scratch.find(std::make_tuple(dev, stream, slot));
+    if (it == g_scratch.end()) continue;
+    if (it->second.ptr) (void)hipFree(it->second.ptr);
+    total += (int64_t)it->second.bytes;
+    g_scratch.erase(it);
+  }
+  auto pit = g_scratch_parked.find(std::make_pair(dev, stream));
+  if (pit != g_scratch_parked.end()) {
+    for (ScratchBuf &b : pit->second) {
+      if (b.ptr) (void)hipFree(b.ptr);
+      total += (int64_t)b.bytes;
+    }
+    g_scratch_parked.erase(pit);
+  }
+  if (released_bytes) *released_bytes = total;
   return CG_OK;
 }
 
@@ -139,6 +211,10 @@ int cg_prof_read(const char *name, double *total_ms, int64_t *launches) {
 
 int cg_abi_version(void) { return CG_ABI_VERSION; }
 
+int cg_scratch_release(cg_stream_t stream, int64_t *released_bytes) {
+  return cg::scratch_release((hipStream_t)stream, released_bytes);
+}
+
 const char *cg_status_string(int status) {
   switch (status) {
     case CG_OK: return "ok";
@@ -152,6 +228,7 @@ const char *cg_status_string(int status) {
     case CG_ERR_UNSUPPORTED: return "unsupported arguments";
     case CG_ERR_NO_TRANSPOSE: return "handle has no transpose";
     case CG_ERR_ALIAS: return "output aliases an input";
+    case CG_ERR_CAPTURE: return "not possible while the stream is being captured";
     default: return "unknown status";
   }
 }

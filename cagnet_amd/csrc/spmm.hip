@@ -62,6 +62,7 @@ static int spmm_plain(const int32_t *rowptr, const int32_t *colind, const float 
   StreamTab &tab = cache.tab_of(sc);
   const int32_t S = window_entries();
   if (tab.S != S) {
+    CG_TRY(refuse_under_capture(stream, "building the window table of a schedule"));
     const int64_t first[2] = {0, sc->ntasks};
     Alloc owned;
     CG_TRY(build_stream(*sc, rowptr, rows, false, 1, first, S, nnz, tab, owned, false, stream));
@@ -208,7 +209,7 @@ static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream, 
   for (int i = 0; i < CsrSide::kHubPlans; ++i)
     if (s.hub[i].valid && s.hub[i].req_hot == (int32_t)hot && s.hub[i].req_single == (int32_t)hot_single &&
         s.hub[i].req_tiers == tiers && s.hub[i].groups == groups && s.hub[i].seg == seg &&
-        s.hub[i].min_degree == min_degree && (may_decline || !s.hub[i].declined))
+        s.hub[i].min_degree == min_degree && (may_decline || !s.hub[i].declined || s.hub[i].failed))
       slot = i;
   if (slot < 0) {
     slot = 0;
@@ -219,8 +220,26 @@ static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream, 
       }
       if (s.hub_used[i] < s.hub_used[slot]) slot = i;
     }
-    CG_TRY(build_hub(s, s.hub[slot], (int32_t)hot, (int32_t)hot_single, groups, tiers, seg, min_degree, may_decline,
-                     stream));
+    const int st = build_hub(s, s.hub[slot], (int32_t)hot, (int32_t)hot_single, groups, tiers, seg, min_degree,
+                             may_decline, stream);
+    if (st == CG_ERR_ALLOC || st == CG_ERR_OVERFLOW) {
+      // No memory for the plan (its build needs about 6 x 4 nnz bytes of temporaries and a second copy of
+      // the entries) or a matrix its virtual rows cannot index: the product goes through the plain
+      // schedule, and the refusal is remembered so that later calls do not try again.
+      HubPlan &hp = s.hub[slot];
+      hp.release();
+      hp.req_hot = (int32_t)hot;
+      hp.req_single = (int32_t)hot_single;
+      hp.req_tiers = tiers;
+      hp.groups = groups;
+      hp.seg = seg;
+      hp.min_degree = min_degree;
+      hp.declined = true;
+      hp.failed = true;
+      hp.valid = true;
+    } else if (st != CG_OK) {
+      return st;
+    }
   }
   s.hub_used[slot] = ++s.hub_clock;
   HubPlan &h = s.hub[slot];
@@ -237,6 +256,7 @@ static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream, 
     CG_TRY(scratch_get(stream, kSlotC, (size_t)hot_tasks * f * sizeof(float), &p));
     const int32_t S = window_entries();
     if (h.hot_tab.S != S || h.hot_tab.groups != nclass) {
+      CG_TRY(refuse_under_capture(stream, "building the window table of a hub plan"));
       Alloc owned;
       CG_TRY(build_stream(h.hot_sched, h.vrowptr, nclass * n, true, nclass, h.tstart, S, s.nnz, h.hot_tab, owned, false,
                           stream));
@@ -334,8 +354,20 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
     if (unit <= 0) unit = kPanelDefaultUnit;
     const bool may_decline = g_tune_panel.load(std::memory_order_relaxed) == 0;
     PanelPlan &pp = s.panel;
-    if (!pp.valid || pp.emin != emin || pp.hot_cols != cols || pp.unit_entries != unit || (pp.declined && !may_decline))
-      CG_TRY(build_panel(s, pp, emin, cols, unit, may_decline, stream));
+    if (!pp.valid || pp.emin != emin || pp.hot_cols != cols || pp.unit_entries != unit ||
+        (pp.declined && !may_decline && !pp.failed))
+    {
+      const int st = build_panel(s, pp, emin, cols, unit, may_decline, stream);
+      if (st == CG_ERR_ALLOC || st == CG_ERR_OVERFLOW) {  // no memory for the plan: remembered as declined
+        pp.release();
+        pp.emin = emin;
+        pp.hot_cols = cols;
+        pp.unit_entries = unit;
+        pp.declined = pp.failed = pp.valid = true;
+      } else if (st != CG_OK) {
+        return st;
+      }
+    }
     if (!pp.declined) {
       float *P = nullptr;
       CG_TRY(launch_panel(pp, B, ldb, f, &P, stream));
@@ -358,6 +390,17 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
     CG_TRY(spmm_plain(s.rowptr, s.colind, s.val, s.rows, s.nnz, s.sched, vec, dr, f, stream));
   }
   return CG_OK;
+}
+
+// Entry of every product on a handle's side.  A product issued while its stream is being captured pins
+// the side: from then on tables of the side that have to go (an evicted hub plan, a recycled schedule,
+// a panel plan rebuilt for other tuning values) are parked on the side instead of freed, because the
+// captured graph replays with their addresses.  cg_csr_unpin or the handle's destruction frees them.
+static int spmm_entry(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t ldc, int32_t f, float beta,
+                      hipStream_t stream, const DenseOps *epi = nullptr) {
+  if (stream_capturing(stream)) s.pinned = true;
+  ParkScope park(s.pinned ? &s.parked : nullptr);
+  return spmm_side(s, B, ldb, C, ldc, f, beta, stream, epi);
 }
 
 // One-shot product from row-sorted COO: rowptr, schedule and window tables are rebuilt in a
@@ -572,6 +615,7 @@ struct CooCacheEntry {
   int32_t n = 0, m = 0;
   int device = 0;
   uint64_t tick = 0;
+  int64_t bytes = 0;  // estimate of the device memory the block holds (CSR copy and up to two plan copies of the entries)
   std::shared_ptr<cg_csr> h;
   std::mutex use;  // one product at a time per block: a handle's schedule caches are not re-entrant
 };
@@ -586,6 +630,10 @@ static int64_t g_coo_cache_hits = 0, g_coo_cache_misses = 0, g_coo_cache_evictio
 static int coo_cache_capacity() {
   const int v = g_tune_coo_cache.load(std::memory_order_relaxed);
   return v == 0 ? 8 : (v < 0 ? 0 : v);
+}
+static int64_t coo_cache_byte_cap() {  // kept blocks may hold this much device memory together (the newest one always stays)
+  const int v = g_tune_coo_cache_mib.load(std::memory_order_relaxed);
+  return (int64_t)(v <= 0 ? 32768 : v) << 20;
 }
 
 static int coo_digest(const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz,
@@ -639,6 +687,7 @@ int cg_spmm_coo_cached(const int32_t *d_row, const int32_t *d_col, const float *
     CG_FAIL(CG_ERR_OVERFLOW, "cg_spmm_coo_cached: nnz=%lld n=%d m=%d exceed int32", (long long)nnz, n, m);
   if (!d_row || !d_col || !d_val) CG_FAIL(CG_ERR_NULL, "cg_spmm_coo_cached: null sparse operand");
   CG_TRY(check_dense("cg_spmm_coo_cached", d_B, ldb, d_C, ldc, f, m, n));
+  CG_TRY(refuse_under_capture(stream, "cg_spmm_coo_cached (it reads the digest of the block back)"));
   int device = 0;
   CG_HIP(hipGetDevice(&device));
   unsigned long long dg[2] = {0, 0};
@@ -674,6 +723,7 @@ int cg_spmm_coo_cached(const int32_t *d_row, const int32_t *d_col, const float *
     entry->n = n;
     entry->m = m;
     entry->device = device;
+    entry->bytes = 3 * (nnz * 8) + 4 * ((int64_t)n + 1) * 4;
     entry->h = h;
     std::vector<std::shared_ptr<CooCacheEntry>> evicted;  // released after the lock is dropped
     {
@@ -681,7 +731,13 @@ int cg_spmm_coo_cached(const int32_t *d_row, const int32_t *d_col, const float *
       ++g_coo_cache_misses;
       entry->tick = ++g_coo_cache_tick;
       g_coo_cache.push_back(entry);
-      while ((int)g_coo_cache.size() > capacity) {
+      const int64_t byte_cap = coo_cache_byte_cap();
+      auto held = [&]() {
+        int64_t total = 0;
+        for (auto &e : g_coo_cache) total += e->bytes;
+        return total;
+      };
+      while ((int)g_coo_cache.size() > capacity || (g_coo_cache.size() > 1 && held() > byte_cap)) {
         size_t oldest = 0;
         for (size_t i = 1; i < g_coo_cache.size(); ++i)
           if (g_coo_cache[i]->tick < g_coo_cache[oldest]->tick) oldest = i;
@@ -692,7 +748,7 @@ int cg_spmm_coo_cached(const int32_t *d_row, const int32_t *d_col, const float *
     }
   }
   std::lock_guard<std::mutex> use(entry->use);
-  return spmm_side(entry->h->fwd, d_B, ldb, d_C, ldc, f, beta, stream);
+  return spmm_entry(entry->h->fwd, d_B, ldb, d_C, ldc, f, beta, stream);
 }
 
 int cg_coo_cache_clear(void) {
@@ -746,6 +802,18 @@ int cg_csr_destroy(cg_csr_t *h) {
   return CG_OK;
 }
 
+int cg_csr_unpin(cg_csr_t *h, int64_t *released) {
+  if (!h) CG_FAIL(CG_ERR_NULL, "cg_csr_unpin: handle is NULL");
+  (void)hipDeviceSynchronize();
+  int64_t count = 0;
+  for (cg::CsrSide *s : {&h->fwd, &h->tr}) {
+    count += s->unpin();
+    if (s->panel.rest) count += s->panel.rest->unpin();
+  }
+  if (released) *released = count;
+  return CG_OK;
+}
+
 int cg_csr_spmm(cg_csr_t *h, int transpose, const float *d_B, int64_t ldb, float *d_C, int64_t ldc, int32_t f,
                 float beta, cg_stream_t stream) {
   using namespace cg;
@@ -753,7 +821,7 @@ int cg_csr_spmm(cg_csr_t *h, int transpose, const float *d_B, int64_t ldb, float
   if (transpose && !h->has_t) CG_FAIL(CG_ERR_NO_TRANSPOSE, "cg_csr_spmm: handle was built without CG_CSR_TRANSPOSE");
   CsrSide &s = transpose ? h->tr : h->fwd;
   CG_TRY(check_dense("cg_csr_spmm", d_B, ldb, d_C, ldc, f, s.cols, s.rows));
-  return spmm_side(s, d_B, ldb, d_C, ldc, f, beta, (hipStream_t)stream);
+  return spmm_entry(s, d_B, ldb, d_C, ldc, f, beta, (hipStream_t)stream);
 }
 
 int cg_csr_spmm_xw(cg_csr_t *h, int transpose, const float *d_B, int64_t ldb, const float *d_C, int64_t ldc, float beta,
@@ -777,7 +845,7 @@ int cg_csr_spmm_xw(cg_csr_t *h, int transpose, const float *d_B, int64_t ldb, co
   epi.epi_fo = fo;
   epi.epi_relu = relu ? 1 : 0;
   // C is never written on this path
-  return spmm_side(s, d_B, ldb, beta != 0.f ? const_cast<float *>(d_C) : nullptr, ldc, f, beta, (hipStream_t)stream, &epi);
+  return spmm_entry(s, d_B, ldb, beta != 0.f ? const_cast<float *>(d_C) : nullptr, ldc, f, beta, (hipStream_t)stream, &epi);
 }
 
 int cg_tune_set(const char *key, int value) {
@@ -796,6 +864,8 @@ int cg_tune_set(const char *key, int value) {
   else if (!strcmp(key, "spmm_panel_unit")) cg::g_tune_panel_unit.store(value);
   else if (!strcmp(key, "dense_mfma")) cg::g_tune_dense_mfma.store(value);
   else if (!strcmp(key, "coo_cache_blocks")) cg::g_tune_coo_cache.store(value);
+  else if (!strcmp(key, "coo_cache_mib")) cg::g_tune_coo_cache_mib.store(value);
+  else if (!strcmp(key, "test_alloc_fail")) cg::g_test_alloc_fail.store(value);
   else CG_FAIL(CG_ERR_UNSUPPORTED, "cg_tune_set: unknown key %s", key);
   return CG_OK;
 }

@@ -29,6 +29,7 @@ struct SchedCache {
         *out = &sched[i];
         return CG_OK;
       }
+    CG_TRY(refuse_under_capture(stream, "building a schedule"));
     if (count == kMax) {  // recycle the oldest
       CG_HIP(hipStreamSynchronize(stream));
       sched[0].release();
@@ -58,6 +59,7 @@ struct HubPlan {
   int32_t hot = 0, groups = 0, tiers = 0, seg = 0, min_degree = 0;
   int32_t req_hot = 0, req_tiers = 0, req_single = 0;  // what was asked for (tiers 0: chosen from the column counts)
   bool declined = false;  // the column counts said a plan does not pay: the plain schedule is used
+  bool failed = false;    // declined because the build ran out of memory or of int32 range
   int32_t classes() const { return groups * tiers; }
   int32_t *vrowptr = nullptr, *colind = nullptr;
   float *val = nullptr;
@@ -71,15 +73,16 @@ struct HubPlan {
     hot_sched.release();
     hot_tab.release();
     cold_sched.release();
-    if (vrowptr) (void)hipFree(vrowptr);
-    if (colind) (void)hipFree(colind);
-    if (val) (void)hipFree(val);
-    if (row_hot) (void)hipFree(row_hot);
+    table_free(vrowptr);
+    table_free(colind);
+    table_free(val);
+    table_free(row_hot);
     vrowptr = colind = nullptr;
     val = nullptr;
     row_hot = nullptr;
     valid = false;
     declined = false;
+    failed = false;
   }
 };
 
@@ -98,13 +101,24 @@ struct CsrSide {
   uint64_t hub_clock = 0;
   bool is_rest = false;  // this side is the rest matrix of a panel plan: its dense part is gone already
   PanelPlan panel;  // plan of the wide products that multiply the dense part out of LDS (spmm_panel.h)
+  bool pinned = false;          // a product on this side was captured into a graph (spmm_entry)
+  std::vector<void *> parked;   // tables replaced since then: a captured graph may still read them
+  int64_t unpin() {  // the caller has made sure that no captured graph will replay any more
+    const int64_t count = (int64_t)parked.size();
+    for (void *p : parked) (void)hipFree(p);
+    parked.clear();
+    pinned = false;
+    return count;
+  }
   void release() {
+    for (void *p : parked) table_free(p);  // inside another side's product these move to that side's list
+    parked.clear();
     panel.release();
     sched.release();
     for (int i = 0; i < kHubPlans; ++i) hub[i].release();
-    if (rowptr) (void)hipFree(rowptr);
-    if (colind) (void)hipFree(colind);
-    if (val) (void)hipFree(val);
+    table_free(rowptr);
+    table_free(colind);
+    table_free(val);
     rowptr = colind = nullptr;
     val = nullptr;
   }
@@ -113,7 +127,7 @@ struct CsrSide {
 inline void PanelPlan::release() {
   void *owned[] = {unit_tile, unit_order, hdr, ent, dslot, split};
   for (void *p : owned)
-    if (p) (void)hipFree(p);
+    table_free(p);
   unit_tile = unit_order = hdr = dslot = split = nullptr;
   ent = nullptr;
   if (rest) {
@@ -121,7 +135,7 @@ inline void PanelPlan::release() {
     delete rest;
     rest = nullptr;
   }
-  valid = declined = false;
+  valid = declined = failed = false;
   covered = 0;
   ntiles = nunits = nsplit = 0;
 }
@@ -235,6 +249,7 @@ __global__ __launch_bounds__(kSpmmThreads) void csr_rows_kernel(const int32_t *_
 // kHubMinHotFraction of the entries.
 static int build_hub(CsrSide &s, HubPlan &h, int32_t hot, int32_t hot_single, int32_t groups, int32_t tiers,
                      int32_t seg, int32_t min_degree, bool may_decline, hipStream_t stream) {
+  CG_TRY(refuse_under_capture(stream, "building a hub plan"));
   CG_HIP(hipStreamSynchronize(stream));
   h.release();
   h.req_hot = hot;

@@ -31,7 +31,7 @@ static std::atomic<int> g_tune_panel{0}, g_tune_panel_emin{0}, g_tune_panel_cols
 struct CsrSide;
 
 struct PanelPlan {
-  bool valid = false, declined = false;
+  bool valid = false, declined = false, failed = false;  // failed: declined because the build ran out of memory
   int32_t emin = 0, hot_cols = 0, unit_entries = 0;  // what the plan was built with
   int64_t covered = 0;      // entries the panel kernel multiplies
   int32_t ntiles = 0, nunits = 0, nsplit = 0;

@@ -50,6 +50,7 @@ static int alloc_sort_buffers(DevTemps &tmp, SortBuffers &buf, int64_t count) {
 // may_decline: leave the plan empty (pp.declined) when the active tiles hold too few of the entries.
 static int build_panel(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot_req, int32_t unit_entries, bool may_decline,
                        hipStream_t stream) {
+  CG_TRY(refuse_under_capture(stream, "building a panel plan"));
   CG_HIP(hipStreamSynchronize(stream));
   pp.release();
   pp.emin = emin;

@@ -10,6 +10,8 @@ namespace cg {
 // Tuning knobs (cg_tune_set): 0 = built-in choice.
 static std::atomic<int> g_tune_seg{0}, g_tune_vec{0}, g_tune_win{0};
 static std::atomic<int> g_tune_hub{0}, g_tune_hub_kb{0}, g_tune_hub_groups{0}, g_tune_hub_tiers{0}, g_tune_hub_row{0};
+static std::atomic<int> g_test_alloc_fail{0};  // test hook: k > 0 makes the k-th table allocation from now fail once
+static std::atomic<int> g_tune_coo_cache_mib{0};  // MiB the kept blocks may hold together: 0 = 32768
 static std::atomic<int> g_tune_coo_cache{0};  // blocks cg_spmm_coo_cached keeps: 0 = 8, negative = none
 
 // ---------------------------------------------------------------------------------------------
@@ -79,6 +81,10 @@ static int check_dense(const char *who, const float *B, int64_t ldb, float *C, i
 // (the one-shot entry point, which builds its tables anew on every call)
 // ---------------------------------------------------------------------------------------------
 static int dev_alloc(void **p, size_t bytes) {
+  if (g_test_alloc_fail.load(std::memory_order_relaxed) > 0 && g_test_alloc_fail.fetch_sub(1) == 1) {
+    *p = nullptr;
+    CG_FAIL(CG_ERR_ALLOC, "hipMalloc of %zu bytes failed: injected by the test_alloc_fail tuning key", bytes);
+  }
   hipError_t e = hipMalloc(p, bytes ? bytes : 4);
   if (e != hipSuccess) {
     (void)hipGetLastError();
@@ -199,10 +205,10 @@ struct Sched {
   uint32_t *d_counts = nullptr;  // {ntasks, nslots, nmulti} on the device (asynchronous builds only)
   void release() {
     if (owned) {
-      if (task_row) (void)hipFree(task_row);
-      if (tbase) (void)hipFree(tbase);
-      if (pbase) (void)hipFree(pbase);
-      if (multi_rows) (void)hipFree(multi_rows);
+      table_free(task_row);
+      table_free(tbase);
+      table_free(pbase);
+      table_free(multi_rows);
     }
     task_row = tbase = pbase = multi_rows = nullptr;
     d_counts = nullptr;
@@ -306,9 +312,9 @@ struct StreamTab {
   int64_t win_first[kMaxHubClasses + 2] = {0};
   void release() {
     if (owned) {
-      if (task_start) (void)hipFree(task_start);
-      if (task_dst) (void)hipFree(task_dst);
-      if (wstart) (void)hipFree(wstart);
+      table_free(task_start);
+      table_free(task_dst);
+      table_free(wstart);
     }
     task_start = task_dst = wstart = nullptr;
     d_nwin = nullptr;

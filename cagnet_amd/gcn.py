@@ -320,7 +320,13 @@ class GraphedTrain:
     and optimizer state advance) and then records one more epoch without executing it; `step()`
     replays it.  Every tensor the epoch reads (`inputs`, the weights, `data.y`, `data.train_mask`)
     is read from the same memory on every replay: update them in place.  Optimizers that keep
-    scalars on the host must be built for capture (`torch.optim.Adam(..., capturable=True)`)."""
+    scalars on the host must be built for capture (`torch.optim.Adam(..., capturable=True)`).
+
+    The graph replays with the addresses of the library's scratch buffers of its stream and of the
+    tables of the matrices it multiplies with; the library keeps both alive for as long as the matrices
+    live (later eager calls that need other tables or more scratch get new memory).  `close()` drops
+    the graph and hands that memory back: the private stream's scratch at once, the matrices' parked
+    tables through `unpin()`."""
 
     def __init__(self, inputs, weight1, weight2, adj_matrix, am_partitions, optimizer, data, rank=0, size=1,
                  group=None, warmup: int = 3):
@@ -341,10 +347,30 @@ class GraphedTrain:
             self.outputs = train(*args)
             self.loss = train.last_loss
         self.epochs_run = warmup
+        self._matrices = [m for m in am_partitions if hasattr(m, "unpin")]
+
+    def close(self) -> None:
+        """Drop the captured graph and free what the library kept alive for it.  Idempotent."""
+        if getattr(self, "graph", None) is None:
+            return
+        self.graph = None
+        torch.cuda.synchronize(self.stream.device)
+        ops.scratch_release(self.stream)
+        for m in self._matrices:
+            m.unpin()
+        self._matrices = []
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:  # interpreter shutdown: the driver reclaims the memory
+            pass
 
     def step(self) -> torch.Tensor:
         """One more epoch.  Returns the epoch's outputs (the same tensor every time; `self.loss`
         likewise holds the epoch's loss after the replay has run)."""
+        if self.graph is None:
+            raise RuntimeError("GraphedTrain.step() after close()")
         self.graph.replay()
         self.epochs_run += 1
         return self.outputs

@@ -26,6 +26,16 @@ def _stream() -> c_void_p:
     return c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
+def scratch_release(stream: "torch.cuda.Stream | None" = None) -> int:
+    """Free the library's scratch buffers of `stream` (default: the current stream), including
+    buffers kept alive because a captured HIP graph used them (cg_scratch_release).  Synchronises
+    the stream.  Returns the number of bytes freed."""
+    released = ctypes.c_int64(0)
+    handle = c_void_p(stream.cuda_stream) if stream is not None else _stream()
+    check(lib.cg_scratch_release(handle, ctypes.byref(released)), "cg_scratch_release")
+    return int(released.value)
+
+
 def _ptr(t: Optional[torch.Tensor]) -> c_void_p:
     return c_void_p(t.data_ptr()) if t is not None and t.numel() > 0 else c_void_p(0)
 
@@ -308,6 +318,14 @@ class CsrMatrix:
     @property
     def shape(self) -> Tuple[int, int]:
         return (self.n, self.m)
+
+    def unpin(self) -> int:
+        """Free the tables this matrix has kept alive for HIP graphs captured over its products
+        (cg_csr_unpin): call it only when none of those graphs will be replayed again.  Returns the
+        number of device allocations freed."""
+        released = ctypes.c_int64(0)
+        check(lib.cg_csr_unpin(self._handle, ctypes.byref(released)), "cg_csr_unpin")
+        return int(released.value)
 
     def info(self) -> dict:
         buf = (c_int64 * 8)()

@@ -17,7 +17,18 @@ Differences a caller can observe, all deliberate:
 `cache_blocks`: the reference's callers pass the same block at every stage of every epoch, as
 fresh `.int()` temporaries.  When True, spmm_gpu recognises a block by a digest of its arrays and
 reuses the CSR, schedules and plans built when it first saw it (cg_spmm_coo_cached); when False
-every call rebuilds them on the device (cg_spmm_coo).
+every call rebuilds them on the device (cg_spmm_coo).  Kept blocks hold device memory (about three
+copies of a block's entries each, at most 8 blocks or 32 GiB, least recently used dropped first;
+`ops.coo_cache_clear()` hands it back).  A caller whose values change on every call should set it to
+False: every call would otherwise build a handle and a plan for a block that is never seen again.
+
+Precondition, as in the reference (cusparseXcoo2csr needs sorted rows, sparse_coo_tensor.cu:137-142):
+rows ascending, 0 <= row < n, 0 <= col < m.  What happens when it does not hold depends on the path:
+  * wide products over dense blocks (f >= 64, at least 8 entries per row, nnz * f >= 3e9) with
+    `cache_blocks`: checked when a block is first seen; CagnetError (CG_ERR_UNSORTED, CG_ERR_INDEX);
+  * every other product: not checked.  Indices are clamped, so nothing outside the operands is
+    touched, but C is then as meaningless as in the reference.  Set `validate_inputs = True` to
+    check every call first (one more pass over the indices and one stream synchronisation per call).
 """
 from __future__ import annotations
 
@@ -27,9 +38,10 @@ import torch
 
 from . import ops
 
-__all__ = ["spmm_gpu", "sparse_coo_tensor_gpu", "coo2csr", "cache_blocks"]
+__all__ = ["spmm_gpu", "sparse_coo_tensor_gpu", "coo2csr", "cache_blocks", "validate_inputs"]
 
 cache_blocks = True
+validate_inputs = False
 
 
 def spmm_gpu(A_rowindices: torch.Tensor, A_colindices: torch.Tensor, A_values: torch.Tensor, n: int, m: int,
@@ -37,6 +49,8 @@ def spmm_gpu(A_rowindices: torch.Tensor, A_colindices: torch.Tensor, A_values: t
     """C += A @ B.  A is n x m, given as row-sorted COO with int32 indices and fp32 values
     (the callers pass `.indices()[k].int()` of a coalesced tensor, gcn_distr.py:238-240);
     B is m x f and C is n x f, both fp32.  Returns None, like the reference."""
+    if validate_inputs:
+        ops.coo_check(A_rowindices, A_colindices, int(n), int(m), require_sorted=True)
     if C.dim() == 2 and C.numel() > 0 and C.stride(1) != 1:
         # a transposed view, e.g. a C that an earlier reference-style call left column-major
         tmp = C.contiguous()
@@ -55,8 +69,18 @@ def sparse_coo_tensor_gpu(indices: torch.Tensor, values: torch.Tensor, size: Seq
     return torch.sparse_coo_tensor(indices, values, tuple(size), check_invariants=False)
 
 
-def coo2csr(A_rowindices: torch.Tensor, A_colindices: torch.Tensor, A_values: torch.Tensor, n: int, m: int):
+def coo2csr(A_rowindices: torch.Tensor, A_colindices: torch.Tensor, A_values: torch.Tensor, n: int, m: int,
+            transpose: bool = False):
     """(rowptr[n+1], colind[nnz], values[nnz]) in (row, col) order, from COO in any order.
     The reference performs only the row compression, on sorted input, inside spmm_gpu
-    (cusparseXcoo2csr, sparse_coo_tensor.cu:137-142)."""
-    return ops.coo2csr(A_rowindices, A_colindices, A_values, int(n), int(m))
+    (cusparseXcoo2csr, sparse_coo_tensor.cu:137-142).
+
+    transpose=True appends the CSR of A^T, which the backward products A^T G read
+    (gcn_distr.py:306, :326 pass `adj_matrix.t()` blocks): the result is then
+    (rowptr, colind, values, colptr[m+1], rowind[nnz], values_t[nnz], perm[nnz]) with
+    values_t[k] == values[perm[k]], entry k of A^T being entry perm[k] of A."""
+    rowptr, colind, values = ops.coo2csr(A_rowindices, A_colindices, A_values, int(n), int(m))
+    if not transpose:
+        return rowptr, colind, values
+    colptr, rowind, values_t, perm = ops.csr_transpose(rowptr, colind, values, int(n), int(m), return_perm=True)
+    return rowptr, colind, values, colptr, rowind, values_t, perm

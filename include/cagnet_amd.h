@@ -20,7 +20,21 @@
  *     two calls with the same arguments give bit-identical results.
  *   - Library scratch memory is kept per (device, stream); calls that share a
  *     stream are ordered by it.  Calls on different streams use different
- *     scratch and may overlap.
+ *     scratch and may overlap.  A cg_csr_t handle is used by one host thread
+ *     at a time (its schedule and plan caches are not re-entrant).
+ *   - Stream capture (hipStreamBeginCapture): cg_csr_spmm, cg_csr_spmm_xw,
+ *     cg_spmm_coo, the dense and the elementwise entry points may be captured
+ *     once the same call has run eagerly on that stream (the first call of a
+ *     shape builds tables and grows scratch, which a capture cannot hold; such
+ *     a step returns CG_ERR_CAPTURE and leaves the capture usable for nothing).
+ *     A captured graph keeps the addresses of the scratch buffers and handle
+ *     tables its calls used.  The library therefore never frees those while
+ *     the handle lives: a scratch buffer handed out under capture, and every
+ *     table of a handle that ran a product under capture, is parked instead of
+ *     freed when a later call has to replace it (growth, plan eviction, new
+ *     tuning values).  cg_csr_unpin / cg_csr_destroy and cg_scratch_release
+ *     free parked memory; call them only when no graph that used the handle or
+ *     the stream will be replayed again.
  */
 #ifndef CAGNET_AMD_H
 #define CAGNET_AMD_H
@@ -47,7 +61,8 @@ enum cg_status {
   CG_ERR_ALLOC = 7,        /* device or host allocation failed */
   CG_ERR_UNSUPPORTED = 8,  /* argument combination not implemented */
   CG_ERR_NO_TRANSPOSE = 9, /* transpose product asked of a handle built without CG_CSR_TRANSPOSE */
-  CG_ERR_ALIAS = 10        /* output aliases an input where that is not allowed */
+  CG_ERR_ALIAS = 10,       /* output aliases an input where that is not allowed */
+  CG_ERR_CAPTURE = 11      /* the call would allocate, build tables or read back while its stream is being captured */
 };
 
 /* flags of cg_csr_create */
@@ -58,6 +73,11 @@ enum cg_status {
 int cg_abi_version(void);
 const char *cg_status_string(int status);
 const char *cg_last_error(void);
+/* Frees the library's scratch buffers of (current device, stream), including buffers parked because a
+ * captured graph used them (see Conventions), after synchronising the stream; the next call on the
+ * stream allocates afresh.  *released_bytes is nullable.  CG_ERR_CAPTURE while the stream is capturing.
+ * No counterpart in the reference (torch's caching allocator owns cuSPARSE's workspace there). */
+int cg_scratch_release(cg_stream_t stream, int64_t *released_bytes);
 
 /* ------------------------------------------------------------------------------------------
  * coo2csr.  Replaces the cusparseXcoo2csr step that the reference runs inside every spmm_gpu
@@ -125,7 +145,14 @@ int cg_spmm_coo(const int32_t *d_row, const int32_t *d_col, const float *d_val, 
  * (CG_ERR_INDEX, CG_ERR_UNSORTED).  Two different blocks with equal digests (probability about
  * 2^-128 per pair) would be taken for one another.  The least recently used block is dropped
  * beyond cg_tune_set("coo_cache_blocks", k) blocks (default 8; negative: keep none and behave as
- * cg_spmm_coo).  Thread safe; products on one block are serialised. */
+ * cg_spmm_coo) or beyond "coo_cache_mib" MiB of kept device memory (default 32 GiB).
+ * Input that is not row-sorted or out of range is therefore reported on this path only; the products
+ * passed on to cg_spmm_coo have that entry point's precondition (see there) and report nothing.
+ * A caller whose values change on every call pays the digest, the handle and the plan build (about
+ * 40 ms at 114.6 M entries) each time and should call cg_spmm_coo instead.
+ * May be called from several host threads at once, also on different streams (the table of blocks is
+ * locked, products on one block are serialised); cannot be captured into a HIP graph (CG_ERR_CAPTURE:
+ * it reads the digest back). */
 int cg_spmm_coo_cached(const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz, int32_t n,
                        int32_t m, const float *d_B, int64_t ldb, float *d_C, int64_t ldc, int32_t f, float beta,
                        cg_stream_t stream);
@@ -143,6 +170,11 @@ int cg_coo_cache_info(int64_t info[4]);
 int cg_csr_create(cg_csr_t **out, const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz,
                   int32_t n, int32_t m, uint32_t flags, cg_stream_t stream);
 int cg_csr_destroy(cg_csr_t *h);
+/* Frees the tables parked on a handle since one of its products was captured into a HIP graph (see
+ * Conventions) and lets later replacements free at once again.  Synchronises the device.  *released
+ * (nullable) receives the number of device allocations freed.  Only for callers that have dropped every
+ * graph captured over this handle.  No counterpart in the reference, which captures no graphs. */
+int cg_csr_unpin(cg_csr_t *h, int64_t *released);
 
 /* C[rows,f] = beta*C + op(A) * B, op(A) = A (transpose == 0: rows = n, B is m x f) or A^T
  * (transpose != 0: rows = m, B is n x f).  The first call for a given width class builds its
@@ -204,8 +236,11 @@ int cg_dense_xtg(const float *d_X, int64_t ldx, const float *d_G, int64_t ldg, f
  *                         train ends in exactly this pair, gcn_distr.py:344 and :356); the loss is
  *                         the same float nll_loss_fwd returns for the log-probabilities written
  * y is int64 (torch labels); mask is one byte per row (torch.bool / uint8), NULL = all rows.
- * A label outside [0, c) contributes nothing (torch would raise).  d_count receives |mask| as
- * int64 (device).  Both reductions run in a fixed order.
+ * In these formulas "mask" means the rows that are in the mask AND carry a label in [0, c): a row with any
+ * other label (torch's ignore_index = -100 among them) adds nothing to the sum, does not count in |mask|
+ * and gets a zero gradient, which is what F.nll_loss does with ignore_index rows (for other labels outside
+ * the range torch raises; here they are ignored the same way).  d_count receives |mask| as int64
+ * (device).  Both reductions run in a fixed order.
  */
 int cg_relu_fwd(const float *d_z, float *d_h, int64_t count, cg_stream_t stream);
 int cg_relu_bwd(const float *d_g, const float *d_h, float *d_dz, int64_t count, cg_stream_t stream);
@@ -311,10 +346,15 @@ int cg_prof_enable(int on);
  *   "spmm_panel"      panel plan (dense row-panel x column-block tiles multiplied out of LDS; even widths
  *                     258..636): -1 never, 1 always, 0 when the tiles hold at least half of the entries
  *   "spmm_panel_emin" entries a 128 x 32 tile needs to be staged (0: 64)
- *   "spmm_panel_cols" ranked columns that can be part of a tile (0: 65536)
- *   "spmm_panel_unit" entries after which the tiles of a row panel go to another workgroup (0: 32768)
+ *   "spmm_panel_cols" ranked columns that can be part of a tile (0: 131072)
+ *   "spmm_panel_unit" entries after which the tiles of a row panel go to another workgroup (0: 65536)
  *   "dense_mfma"      -1: dense products on the vector ALU tile kernel only
  *   "coo_cache_blocks" blocks cg_spmm_coo_cached keeps (0: 8; negative: none)
+ *   "coo_cache_mib"   device memory those blocks may hold together, in MiB (0: 32768); a block counts as three
+ *                     copies of its entries (the CSR and up to two plans); the newest block always stays
+ *   "test_alloc_fail" test hook: k > 0 makes the k-th device allocation for handle tables from now on fail
+ *                     once with CG_ERR_ALLOC (a plan whose build fails that way is given up for good and the
+ *                     product runs on the plain schedule)
  * An unknown key returns CG_ERR_UNSUPPORTED. */
 int cg_tune_set(const char *key, int value);
 int cg_prof_read(const char *name, double *total_ms, int64_t *launches);

@@ -56,6 +56,17 @@ def training_case(name: str) -> None:
                         w2_after=w2.numpy())
 
 
+def harness_case(name: str) -> None:
+    """Losses of the single-process harness run `bench.py --workload tiny --optimizer sgd --steps 100
+    --warmup 0 --seed 0 --print-losses` (scale 12, 32,768 edges, 128 features, hidden 16, 8 classes,
+    SGD 0.01), from the fp64 oracle."""
+    p = synth.make_problem(scale=12, n_edges=32768, features=128, hidden=16, classes=8, mask_fraction=1.0, seed=0)
+    A64 = orc.coo_tensor(p.row, p.col, p.val, p.n, p.n, torch.float64)
+    losses, _, _ = orc.train_epochs(p.x, p.w1, p.w2, [A64], p.y, p.train_mask, epochs=100, lr=0.01,
+                                    optimizer="sgd", dtype=torch.float64)
+    np.savez_compressed(OUT / f"{name}.npz", n=p.n, nnz=p.row.numel(), sgd_losses_f64=np.array(losses))
+
+
 def prep_case(name: str) -> None:
     """Raw pattern -> self-loops -> normalised values -> one block of a 3 x 3 partition -> blob."""
     rng = np.random.default_rng(41)
@@ -78,7 +89,8 @@ if __name__ == "__main__":
     cases = {"graph_s6_f5": lambda: graph_case("graph_s6_f5", 6, 400, 5, 31),
              "graph_s8_f41": lambda: graph_case("graph_s8_f41", 8, 2500, 41, 32),
              "train_s7": lambda: training_case("train_s7"),
-             "prep_n97": lambda: prep_case("prep_n97")}
+             "prep_n97": lambda: prep_case("prep_n97"),
+             "harness_tiny_sgd": lambda: harness_case("harness_tiny_sgd")}
     for key, make in cases.items():
         if not only or key in only:
             make()

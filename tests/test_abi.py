@@ -131,3 +131,30 @@ def test_python_surface_rejects_cpu_tensors_and_wrong_types():
     assert shim.spmm_gpu is spmm_gpu
     from cagnet_amd import sparse_coo_tensor_cpp as mod
     assert mod.cache_blocks is True      # blocks seen before are recognised by default
+
+
+def _host_driver():
+    """The ASan + UBSan build of the library's host code and its driver (tests/abi_host_driver.cpp); built here
+    only when nothing is there yet."""
+    from cagnet_amd import build
+    if not build.SAN_DRIVER_PATH.exists() or not build.SAN_LIB_PATH.exists():
+        build.build_host_driver()
+    return build.SAN_DRIVER_PATH
+
+
+def run_host_driver(*args):
+    import os
+    import subprocess
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1")
+    proc = subprocess.run([str(_host_driver()), *args], capture_output=True, text=True, timeout=600, env=env)
+    report = proc.stdout[-3000:] + proc.stderr[-6000:]
+    assert proc.returncode == 0, report
+    assert "AddressSanitizer" not in proc.stderr and "runtime error:" not in proc.stderr, report
+    assert "abi_host_driver: ok" in proc.stdout
+
+
+def test_host_code_under_address_and_ub_sanitizers():
+    """Argument checks, status strings, tuning keys, blob header parsing and the recorder of the library,
+    compiled with -fsanitize=address,undefined on the host side, driven by a sanitized C++ program: no GPU is
+    needed for these paths.  (Leak checking is off: the HIP runtime keeps its own allocations until exit.)"""
+    run_host_driver()

@@ -118,11 +118,33 @@ def test_nll_loss_forward_backward(cuda, n, c, frac):
     loss1, count1 = ops.nll_loss_fwd(out, y.to(cuda), m)
     assert torch.equal(logp2, out) and int(count2) == int(count1) == expect_count
     assert float(loss2) == float(loss1)
+    # labels outside [0, c): ignored like F.nll_loss's ignore_index rows (not in the sum, not in the count,
+    # zero gradient); torch's default ignore_index is -100
+    y_ign = y.clone()
+    y_ign[::7] = -100
+    l2 = ops.log_softmax_nll_fwd(z.to(cuda), y_ign.to(cuda), m)
+    l1 = ops.nll_loss_fwd(out, y_ign.to(cuda), m)
+    assert float(l2[1]) == float(l1[0]) and int(l2[2]) == int(l1[1])
+    counted = (y_ign >= 0) if mask is None else (mask & (y_ign >= 0))
+    assert int(l1[1]) == int(counted.sum())
+    dz_ign = ops.log_softmax_nll_bwd(out, y_ign.to(cuda), m, l1[1], gs.to(cuda))
+    d_ign = ops.nll_loss_bwd(y_ign.to(cuda), m, l1[1], gs.to(cuda), n, c)
+    assert float((dz_ign - ops.log_softmax_bwd(d_ign, out)).abs().max()) <= 1e-6
+    if int(counted.sum()) > 0:
+        zr = z.double().requires_grad_(True)
+        ref = F.nll_loss(F.log_softmax(zr, dim=1)[sel], y_ign[sel])
+        assert abs(float(l1[0]) - float(ref)) <= 1e-5 * max(1.0, abs(float(ref)))
+        (ref * 0.5).backward()
+        assert float((dz_ign.cpu().double() - zr.grad).abs().max()) <= 1e-6
+        assert torch.count_nonzero(dz_ign[~counted.to(cuda)]) == 0
+    else:
+        assert float(l1[0]) == 0.0 and torch.count_nonzero(dz_ign) == 0
     y_bad = y.clone()
-    y_bad[0] = c + 3                           # a label outside [0, c) contributes nothing but is counted
+    y_bad[0] = c + 3                           # other labels outside the range are ignored the same way (torch raises)
     l2 = ops.log_softmax_nll_fwd(z.to(cuda), y_bad.to(cuda), m)
     l1 = ops.nll_loss_fwd(out, y_bad.to(cuda), m)
     assert float(l2[1]) == float(l1[0]) and int(l2[2]) == int(l1[1])
+    assert int(l1[1]) == expect_count - (1 if (mask is None or bool(mask[0])) else 0)
 
 
 def test_rowwise_kernels_on_views(cuda):

@@ -354,3 +354,27 @@ def test_adam_epochs_with_reference_init_match_oracle(cuda, classes, features, s
     assert losses[-1] < losses[0]
     _close(w1, w1_64, "w1 after 60 Adam epochs", 1e-3)
     _close(w2, w2_64, "w2 after 60 Adam epochs", 1e-3)
+
+
+def test_single_process_harness_prints_golden_losses(cuda):
+    """The runnable plumbing harness (the role of the reference's gcn.py:104-126):
+    `bench.py --workload tiny --optimizer sgd --steps 100 --warmup 0 --print-losses` prints one loss per
+    epoch; they must match the fp64 oracle's losses for the same configuration, committed under
+    tests/golden/ (written by tests/golden/make_golden.py), to 1e-4."""
+    import re
+    import subprocess
+    import sys
+    from pathlib import Path
+    import numpy as np
+    root = Path(__file__).resolve().parents[1]
+    proc = subprocess.run([sys.executable, str(root / "bench.py"), "--workload", "tiny", "--optimizer", "sgd",
+                           "--steps", "100", "--warmup", "0", "--seed", "0", "--print-losses", "--no-cpu-baseline",
+                           "--no-extra"], capture_output=True, text=True, timeout=600, cwd=str(root))
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    losses = [float(m.group(1)) for m in re.finditer(r"^Epoch: \d+ loss ([0-9.eE+-]+)$", proc.stderr, re.M)]
+    golden = np.load(root / "tests" / "golden" / "harness_tiny_sgd.npz")
+    want = golden["sgd_losses_f64"]
+    assert len(losses) == len(want) == 100
+    assert float(np.abs(np.array(losses) - want).max()) <= 1e-4
+    rec = __import__("json").loads(proc.stdout.strip().splitlines()[-1])
+    assert rec["config"]["workload"].startswith("R-MAT scale 12") and rec["steps"] == 100

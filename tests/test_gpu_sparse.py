@@ -900,3 +900,129 @@ def test_spmm_panel_plan_rectangular_strided_and_declined(cuda, tune):
     tune("spmm_panel", 1)
     got = U.spmm(Bu)                                                 # forced: still correct, whatever the coverage
     assert spmm_error(got, ur, uc, uv, 3000, 3000, Bu.cpu()) <= REL_TOL
+
+
+def test_captured_graph_outlives_plan_eviction_and_scratch_growth(cuda, tune):
+    """A HIP graph captured over a product keeps the addresses of the handle's tables and of the
+    stream's scratch.  Later eager products at other widths evict hub plans (two are kept per side),
+    recycle schedules and grow the scratch; the tables and buffers the graph names must be parked, not
+    freed: the replay stays bit-identical, unpin() and scratch_release() report what was kept."""
+    from cagnet_amd import ops
+    from cagnet_amd._lib import CagnetError
+    row, col, val, n = small_graph(11, 60000, seed=77)
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n)
+    tune("spmm_hub", 1)
+    tune("spmm_hub_kb", 64)
+    f = 256
+    B = torch.randn(n, f, generator=torch.Generator().manual_seed(1)).to(cuda)
+    C = torch.empty(n, f, device=cuda)
+    s = torch.cuda.Stream(device=cuda)
+    s.wait_stream(torch.cuda.current_stream(cuda))
+    with torch.cuda.stream(s):
+        A.spmm(B, out=C)                      # builds the plan and grows the scratch: not possible under capture
+    s.synchronize()
+    expect = C.clone()
+    assert spmm_error(expect, row, col, val, n, n, B.cpu()) <= REL_TOL
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        A.spmm(B, out=C)
+        # a width that has never run would have to build tables: refused, with nothing enqueued
+        with pytest.raises(CagnetError, match="CG_ERR_CAPTURE"):
+            A.spmm(torch.empty(n, 272, device=cuda), out=torch.empty(n, 272, device=cuda))
+    C.zero_()
+    g.replay()
+    s.synchronize()
+    assert torch.equal(C, expect)
+    with torch.cuda.stream(s):
+        for f2 in (288, 320, 384, 636):       # other plans, other schedules, more scratch, on the graph's stream
+            B2 = torch.randn(n, f2, generator=torch.Generator().manual_seed(f2)).to(cuda)
+            assert spmm_error(A.spmm(B2), row, col, val, n, n, B2.cpu()) <= REL_TOL
+        tune("spmm_win", 128)                 # other window tables for the schedule the graph uses
+        assert torch.equal(A.spmm(B), expect) or spmm_error(A.spmm(B), row, col, val, n, n, B.cpu()) <= REL_TOL
+    s.synchronize()
+    for _ in range(2):
+        C.zero_()
+        g.replay()
+        s.synchronize()
+        assert torch.equal(C, expect)
+    del g
+    assert A.unpin() > 0                      # tables were parked for the graph
+    assert ops.scratch_release(s) > 0
+    with torch.cuda.stream(s):
+        assert spmm_error(A.spmm(B), row, col, val, n, n, B.cpu()) <= REL_TOL   # and everything still works
+    s.synchronize()
+
+
+def test_plan_build_that_runs_out_of_memory_falls_back_for_good(cuda, tune):
+    """An allocation failure while a hub or panel plan is built must not fail the product: it runs on the
+    plain schedule, and the plan is not tried again on later calls."""
+    from cagnet_amd import ops
+    from cagnet_amd._lib import CagnetError
+    row, col, val, n = small_graph(11, 60000, seed=78)
+    f = 300
+    B = torch.randn(n, f, generator=torch.Generator().manual_seed(2)).to(cuda)
+    for knob in ("spmm_hub", "spmm_panel"):
+        A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n)
+        tune("spmm_hub", -1)
+        tune("spmm_panel", -1)
+        plain = A.spmm(B)
+        tune(knob, 1)
+        tune("test_alloc_fail", 2)            # the second table allocation of the build fails
+        got = A.spmm(B)
+        assert torch.equal(got, plain)
+        if knob == "spmm_hub":
+            assert A.info()["plan_tiers"] == -1
+        else:
+            assert _panel_info(A)["state"] == -1
+        tune("test_alloc_fail", 1)            # would hit the first allocation of a second attempt
+        assert torch.equal(A.spmm(B), plain)
+        with pytest.raises(CagnetError, match="CG_ERR_ALLOC"):   # still armed: the product allocated nothing
+            ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n)
+        tune("test_alloc_fail", 0)
+        tune(knob, 0)
+
+
+def test_dropin_coo2csr_with_transpose_outputs_and_validate_flag(cuda):
+    """The drop-in module's coo2csr: three arrays by default, seven with transpose=True (the CSR of A^T
+    and the permutation that links the two value arrays), bit-exact against the oracle.  validate_inputs
+    makes spmm_gpu report unsorted rows on the path that otherwise checks nothing."""
+    import cagnet_amd.sparse_coo_tensor_cpp as mod
+    n, m = 300, 700
+    row, col, val = random_coo(n, m, 5000, seed=5, sort=False)
+    out = mod.coo2csr(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, m)
+    assert len(out) == 3
+    rp, ci, vv, cp, ri, vt, perm = mod.coo2csr(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, m, transpose=True)
+    erp, eci, evv, _ = orc.coo2csr(row.numpy(), col.numpy(), val.numpy(), n, m)
+    ecp, eri, evt, eperm = orc.csr_transpose(erp, eci, evv, n, m)
+    for got, want in ((rp, erp), (ci, eci), (vv, evv), (cp, ecp), (ri, eri), (vt, evt), (perm, eperm)):
+        assert np.array_equal(got.cpu().numpy(), want)
+    assert torch.equal(vt, vv[perm.long()])
+    assert all(torch.equal(a, b) for a, b in zip(out, (rp, ci, vv)))
+
+    bad_r = torch.tensor([5, 3, 7], dtype=torch.int32, device=cuda)   # rows descend
+    cols = torch.tensor([1, 2, 3], dtype=torch.int32, device=cuda)
+    B, C = torch.ones(10, 4, device=cuda), torch.zeros(10, 4, device=cuda)
+    mod.spmm_gpu(bad_r, cols, torch.ones(3, device=cuda), 10, 10, B, C)   # unchecked on the narrow path, like the reference
+    mod.validate_inputs = True
+    try:
+        with pytest.raises(ops_error()):
+            mod.spmm_gpu(bad_r, cols, torch.ones(3, device=cuda), 10, 10, B, C)
+        good_r = torch.tensor([3, 5, 7], dtype=torch.int32, device=cuda)
+        C.zero_()
+        mod.spmm_gpu(good_r, cols, torch.ones(3, device=cuda), 10, 10, B, C)
+        assert float(C.sum()) == 12.0
+    finally:
+        mod.validate_inputs = False
+
+
+def ops_error():
+    from cagnet_amd._lib import CagnetError
+    return CagnetError
+
+
+def test_host_code_under_sanitizers_with_real_products(cuda):
+    """The same sanitized build doing real work on the GPU: handle creation, hub and panel plans at seven
+    widths (plan eviction, schedule recycling), a plan build that runs out of memory, the block cache with
+    evictions, unpin and scratch release; the driver checks every product against a host loop."""
+    from tests.test_abi import run_host_driver
+    run_host_driver("gpu")
