@@ -346,23 +346,12 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
   // Panel plan: the entries of dense (row panel, column block) tiles are multiplied out of LDS into
   // partial rows; the row-wise kernels then run over the other entries and add those rows in.
   if (!epi && allow_panel && f <= cap && want_panel(s, f)) {
-    int32_t emin = g_tune_panel_emin.load(std::memory_order_relaxed);
-    if (emin <= 0) emin = kPanelDefaultEmin;
-    int32_t cols = g_tune_panel_cols.load(std::memory_order_relaxed);
-    if (cols <= 0) cols = kPanelDefaultCols;
-    int32_t unit = g_tune_panel_unit.load(std::memory_order_relaxed);
-    if (unit <= 0) unit = kPanelDefaultUnit;
+    const PanelParams par = panel_params();
     const bool may_decline = g_tune_panel.load(std::memory_order_relaxed) == 0;
     PanelPlan &pp = s.panel;
-    if (!pp.valid || pp.emin != emin || pp.hot_cols != cols || pp.unit_entries != unit ||
-        (pp.declined && !may_decline && !pp.failed))
-    {
-      const int st = build_panel(s, pp, emin, cols, unit, may_decline, stream);
+    if (!pp.valid || !par.same(pp) || (pp.declined && !may_decline && !pp.failed)) {
+      const int st = build_panel(s, pp, par, may_decline, stream);
       if (st == CG_ERR_ALLOC || st == CG_ERR_OVERFLOW) {  // no memory for the plan: remembered as declined
-        pp.release();
-        pp.emin = emin;
-        pp.hot_cols = cols;
-        pp.unit_entries = unit;
         pp.declined = pp.failed = pp.valid = true;
       } else if (st != CG_OK) {
         return st;
@@ -862,6 +851,8 @@ int cg_tune_set(const char *key, int value) {
   else if (!strcmp(key, "spmm_panel_emin")) cg::g_tune_panel_emin.store(value);
   else if (!strcmp(key, "spmm_panel_cols")) cg::g_tune_panel_cols.store(value);
   else if (!strcmp(key, "spmm_panel_unit")) cg::g_tune_panel_unit.store(value);
+  else if (!strcmp(key, "spmm_panel_dmin")) cg::g_tune_panel_dmin.store(value);
+  else if (!strcmp(key, "spmm_panel_dwg")) cg::g_tune_panel_dwg.store(value);
   else if (!strcmp(key, "dense_mfma")) cg::g_tune_dense_mfma.store(value);
   else if (!strcmp(key, "coo_cache_blocks")) cg::g_tune_coo_cache.store(value);
   else if (!strcmp(key, "coo_cache_mib")) cg::g_tune_coo_cache_mib.store(value);
@@ -893,7 +884,7 @@ int cg_csr_info(const cg_csr_t *h, int64_t info[8]) {
   return CG_OK;
 }
 
-int cg_csr_panel_info(const cg_csr_t *h, int transpose, int64_t info[8]) {
+int cg_csr_panel_info(const cg_csr_t *h, int transpose, int64_t info[12]) {
   if (!h || !info) CG_FAIL(CG_ERR_NULL, "cg_csr_panel_info: null pointer");
   if (transpose && !h->has_t) CG_FAIL(CG_ERR_NO_TRANSPOSE, "cg_csr_panel_info: handle was built without CG_CSR_TRANSPOSE");
   const cg::PanelPlan &pp = (transpose ? h->tr : h->fwd).panel;
@@ -906,6 +897,10 @@ int cg_csr_panel_info(const cg_csr_t *h, int transpose, int64_t info[8]) {
   info[5] = used && pp.rest ? pp.rest->nnz : 0;
   info[6] = pp.valid ? pp.emin : 0;
   info[7] = pp.valid ? pp.hot_cols : 0;
+  info[8] = used ? pp.dcovered : 0;
+  info[9] = used ? pp.ndtiles : 0;
+  info[10] = used ? pp.ndunits : 0;
+  info[11] = pp.valid ? pp.dmin : 0;
   return CG_OK;
 }
 

@@ -125,19 +125,20 @@ struct CsrSide {
 };
 
 inline void PanelPlan::release() {
-  void *owned[] = {unit_tile, unit_order, hdr, ent, dslot, split};
+  void *owned[] = {unit_tile, unit_order, unit_block, dwg_unit, dunit_tile, dunit_block, dhdr, dA, hdr, ent, dslot, split};
   for (void *p : owned)
     table_free(p);
-  unit_tile = unit_order = hdr = dslot = split = nullptr;
+  unit_tile = unit_order = unit_block = dwg_unit = dunit_tile = dunit_block = dhdr = hdr = dslot = split = nullptr;
   ent = nullptr;
+  dA = nullptr;
   if (rest) {
     rest->release();
     delete rest;
     rest = nullptr;
   }
   valid = declined = failed = false;
-  covered = 0;
-  ntiles = nunits = nsplit = 0;
+  covered = dcovered = 0;
+  ntiles = nunits = nsplit = ndtiles = ndunits = ndwg = nblocks = 0;
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -10,8 +10,13 @@
 // panel; wave w holds the accumulators of the 8 rows {w, w + 16, ...} of the panel in registers for the
 // whole unit and writes them out once as partial rows.  Entries of tiles that are not active stay in a
 // second CSR matrix (the "rest") that the row-wise kernels multiply; their finished rows add the
-// partial rows in.  Replaces nothing in the reference beyond cusparseSpMM itself
-// (sparse-extension/sparse_coo_tensor.cu:215-226); sums are in a fixed order, no atomics on floats.
+// partial rows in.  Tiles that are at least a quarter full ("dense" tiles) are stored as full 128 x 32
+// blocks instead and multiplied on the fp32 matrix cores (v_mfma_f32_16x16x4_f32: exact fp32 products,
+// fp32 accumulation) by a second kernel, in units of their own; the zeros of such a block are multiplied
+// too, so a row of B that holds an infinity or a NaN reaches every row of the block (the row-wise
+// kernels and cusparseSpMM would only touch the rows that reference it).  Replaces nothing in the
+// reference beyond cusparseSpMM itself (sparse-extension/sparse_coo_tensor.cu:215-226); sums are in a
+// fixed order, no atomics on floats.
 #pragma once
 #include "spmm_tables.h"
 #include <algorithm>
@@ -26,21 +31,36 @@ constexpr int kPanelCols = 32;    // columns of a block = rows of B staged per t
 constexpr int kPanelThreads = kPanelWaves * kWave;
 constexpr int32_t kPanelMinF = 258, kPanelMaxF = 636;  // widths the kernel is instantiated for (even)
 
+constexpr int kDenseWaves = 8;    // waves of a workgroup of the dense-tile kernel; wave w owns rows 16 w .. 16 w + 15
+constexpr int kDenseThreads = kDenseWaves * kWave;
+constexpr int kDenseTileFloats = kPanelRows * kPanelCols;
+
 static std::atomic<int> g_tune_panel{0}, g_tune_panel_emin{0}, g_tune_panel_cols{0}, g_tune_panel_unit{0};
+static std::atomic<int> g_tune_panel_dmin{0}, g_tune_panel_dwg{0};
 
 struct CsrSide;
 
 struct PanelPlan {
   bool valid = false, declined = false, failed = false;  // failed: declined because the build ran out of memory
-  int32_t emin = 0, hot_cols = 0, unit_entries = 0;  // what the plan was built with
+  int32_t emin = 0, hot_cols = 0, unit_entries = 0, dmin = 0, dwg = 0;  // what the plan was built with
   int64_t covered = 0;      // entries the panel kernel multiplies
+  int64_t dcovered = 0;     // entries in dense tiles (the matrix-core kernel)
   int32_t ntiles = 0, nunits = 0, nsplit = 0;
+  int32_t ndtiles = 0, ndunits = 0;
+  int32_t nblocks = 0;             // blocks of 128 partial rows, one per unit of either kind
   int32_t *unit_tile = nullptr;    // [nunits + 1] tiles of a unit (units never span panels)
   int32_t *unit_order = nullptr;   // [nunits] launch order: heaviest unit first
+  int32_t *unit_block = nullptr;   // [nunits] block of partial rows a unit writes
+  int32_t ndwg = 0;                // workgroups of the dense-tile kernel: equal shares of the list of dense tiles
+  int32_t *dwg_unit = nullptr;     // [ndwg + 1] units of a workgroup (runs of tiles of one panel inside its share)
+  int32_t *dunit_tile = nullptr;   // [ndunits + 1] dense tiles of a unit
+  int32_t *dunit_block = nullptr;  // [ndunits] block of partial rows a unit writes
+  int32_t *dhdr = nullptr;         // [ndtiles * 32] row of B of every column of a dense tile
+  float *dA = nullptr;             // [ndtiles * 4096] dense tiles in the operand layout of the matrix instruction
   int32_t *hdr = nullptr;          // [ntiles * 16 * 4] per (tile, wave): two rows of B to stage, record range
   uint2 *ent = nullptr;            // [covered] {column in block | slot << 8, value bits}, by (tile, wave, slot)
-  int32_t *dslot = nullptr;        // [rows] partial row of a row of A: unit * 128 + position, or -1
-  int32_t *split = nullptr;        // [2 * nsplit] (first unit, units) of panels that have several units
+  int32_t *dslot = nullptr;        // [rows] partial row of a row of A: block * 128 + position, or -1
+  int32_t *split = nullptr;        // [2 * nsplit] (first block, blocks) of panels that have several units
   CsrSide *rest = nullptr;         // entries outside active tiles, same rows and columns
   void release();
 };
@@ -57,14 +77,22 @@ __device__ __forceinline__ void panel_copy16(uint32_t lds_addr, const float *src
 __device__ __forceinline__ void panel_copy4(uint32_t lds_addr, const float *src) {
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_addr), "v"(src) : "memory");
 }
+// The same with the source as a wave-uniform base and a 32-bit byte offset per lane (no 64-bit address per lane).
+__device__ __forceinline__ void panel_copy16_at(uint32_t lds_addr, const float *base, uint32_t byte_off) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(byte_off), "s"(base) : "memory");
+}
+__device__ __forceinline__ void panel_copy4_at(uint32_t lds_addr, const float *base, uint32_t byte_off) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(byte_off), "s"(base) : "memory");
+}
 
 // hdr[(tile * 16 + wave) * 4 ..]: the two rows of B the wave stages for the tile and the range of its records.
 // It is read two tiles ahead and the records one tile ahead, so that no load of a tile depends on another
 // load of the same tile: the copies of the next tile go out as soon as the barrier has been passed.
 template <int CHUNKS>
 __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
-    const int32_t *__restrict__ unit_tile, const int32_t *__restrict__ unit_order, const int32_t *__restrict__ hdr,
-    const uint2 *__restrict__ ent, const float *__restrict__ B, int64_t ldb, float *__restrict__ P, int32_t f) {
+    const int32_t *__restrict__ unit_tile, const int32_t *__restrict__ unit_order, const int32_t *__restrict__ unit_block,
+    const int32_t *__restrict__ hdr, const uint2 *__restrict__ ent, const float *__restrict__ B, int64_t ldb,
+    float *__restrict__ P, int32_t f) {
   extern __shared__ __align__(16) char panel_lds[];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -209,14 +237,191 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   }
-  // P[unit][slot * 16 + wave][:]: position in the block = rank of the row inside its panel
+  // P[block][slot * 16 + wave][:]: position in the block = rank of the row inside its panel
+  const int block = unit_block[unit];
 #pragma unroll
   for (int s = 0; s < kPanelSlots; ++s) {
-    float *prow = P + ((int64_t)unit * kPanelRows + s * kPanelWaves + wave) * f;
+    float *prow = P + ((int64_t)block * kPanelRows + s * kPanelWaves + wave) * f;
 #pragma unroll
     for (int ch = 0; ch < CHUNKS; ++ch) {
       const int p = lane + kWave * ch;
       if (p < npair) *reinterpret_cast<float2 *>(prow + 2 * p) = acc[s][ch];
+    }
+  }
+}
+
+// -------------------------------------------------------------------------------------------------
+// dense tiles on the fp32 matrix cores
+// -------------------------------------------------------------------------------------------------
+// A dense tile is a full 128 x 32 block of A.  Wave w of 8 owns rows 16 w .. 16 w + 15 of the panel and all
+// columns of the result: per tile 8 reduction steps of 4 columns of A (= 4 staged rows of B), each one
+// v_mfma_f32_16x16x4_f32 per 16 result columns.  Register layout of the instruction (lane l):
+//   A (16 x 4): lane holds A[l % 16][l / 16]      B (4 x 16): lane holds B[l / 16][l % 16]
+//   D (16 x 16) in 4 registers: register v holds D[4 (l / 16) + v][l % 16]
+// The 16 columns of one instruction are taken 4 apart: lane (q, c) = (l / 16, l % 16) reads the 16 bytes
+// B[4 ks + q][64 g + 4 c .. + 3] from LDS and feeds its four floats to four instructions, so that the lane ends
+// up with four consecutive result columns per group g of 64 columns.
+// dA[((tile * 8 + wave) * 2 + ks / 4) * 256 + lane * 4 + ks % 4] = A[16 wave + lane % 16][4 ks + lane / 16].
+//
+// All dense tiles cost the same, so every workgroup takes an equal share of the list of dense tiles (in
+// (panel, column block) order) and walks it in one pipeline.  A unit is a run of tiles of one panel inside one
+// share; after a unit's last tile the accumulators go out as that unit's block of partial rows.
+//
+// The loop over the tiles of a unit has no branch in it: the accumulators of the matrix instructions are
+// live across it, and a loop body of many basic blocks makes the register allocator move them from register
+// to register between the instructions (and spill).  The copies of the next tile are therefore predicated
+// inside their asm statement (exec is narrowed to the lanes that have a piece and put back).
+typedef float panel_f4 __attribute__((ext_vector_type(4)));
+
+// Lanes with byte_off < limit copy 16 (4) bytes from base + byte_off to LDS at lds_addr + lane * 16 (4).
+__device__ __forceinline__ void panel_copy16_if(uint32_t lds_addr, const float *base, uint32_t byte_off, uint32_t limit) {
+  uint64_t saved;
+  asm volatile(
+      "s_mov_b64 %0, exec\n\t"
+      "v_cmp_gt_u32 vcc, %4, %2\n\t"
+      "s_and_b64 exec, exec, vcc\n\t"
+      "s_mov_b32 m0, %1\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %2, %3\n\t"
+      "s_mov_b64 exec, %0"
+      : "=&s"(saved)
+      : "s"(lds_addr), "v"(byte_off), "s"(base), "s"(limit)
+      : "vcc", "scc", "memory");  // s_and writes scc
+}
+__device__ __forceinline__ void panel_copy4_if(uint32_t lds_addr, const float *base, uint32_t byte_off, uint32_t limit) {
+  uint64_t saved;
+  asm volatile(
+      "s_mov_b64 %0, exec\n\t"
+      "v_cmp_gt_u32 vcc, %4, %2\n\t"
+      "s_and_b64 exec, exec, vcc\n\t"
+      "s_mov_b32 m0, %1\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dword %2, %3\n\t"
+      "s_mov_b64 exec, %0"
+      : "=&s"(saved)
+      : "s"(lds_addr), "v"(byte_off), "s"(base), "s"(limit)
+      : "vcc", "scc", "memory");  // s_and writes scc
+}
+
+template <int NG>  // groups of 64 result columns: ceil(f / 64)
+__global__ __launch_bounds__(kDenseThreads) void spmm_panel_dense_kernel(
+    const int32_t *__restrict__ wg_unit, const int32_t *__restrict__ unit_tile, const int32_t *__restrict__ unit_block,
+    const int32_t *__restrict__ dhdr, const float *__restrict__ dA, const float *__restrict__ B, int64_t ldb,
+    float *__restrict__ P, int32_t f) {
+  extern __shared__ __align__(16) char panel_lds[];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int c16 = lane & 15, q = lane >> 4;
+  const int u0 = wg_unit[blockIdx.x], u1 = wg_unit[blockIdx.x + 1];
+  if (u0 >= u1) return;
+  const int t_first = unit_tile[u0], t_end = unit_tile[u1];  // the units of a workgroup are consecutive, and so are their tiles
+  const int rs = (f * 4 + 15) & ~15;  // bytes of a staged row
+  const int bufsz = kPanelCols * rs;
+  constexpr int RPW = kPanelCols / kDenseWaves;  // rows of B a wave stages per tile
+  static_assert(RPW == 4, "a wave reads the four rows it stages from lanes 0..3 of its header");
+  // A row is staged in NX4 pieces of 64 x 16 bytes and one of up to 3 x 4 bytes behind the last whole 16 bytes
+  // (widths that are not a multiple of 4); which lanes of a piece have something to copy depends on f.
+  constexpr int NX4 = (NG + 3) / 4, PPR = NX4 + 1, NPIECES = RPW * PPR;
+  static_assert(NPIECES <= 4 * NG, "one copy per two groups of a tile's 8 NG group steps must cover all pieces");
+  const uint32_t lim16 = (uint32_t)(f >> 2) * 16u, lim4 = (uint32_t)f * 4u;
+  const uint32_t tail_off = lim16 + (uint32_t)lane * 4u;  // byte offset of the lane's 4-byte piece
+  auto stage_piece = [&](int pc, const float *const (&src4)[RPW], int buf) {  // pc is a constant after unrolling
+    const int r = pc / PPR, j = pc % PPR;
+    const uint32_t dst = (uint32_t)(uintptr_t)(panel_lds + buf * bufsz + (wave + r * kDenseWaves) * rs);
+    if (j < NX4)
+      panel_copy16_if(dst + j * (kWave * 16), src4[r], (uint32_t)(j * kWave + lane) * 16u, lim16);
+    else
+      panel_copy4_if(dst + lim16, src4[r], tail_off, lim4);
+  };
+  auto hdr_load = [&](int t) { return dhdr[(int64_t)t * kPanelCols + wave + kDenseWaves * (lane & 3)]; };
+  auto a_load = [&](int t, float4 (&a)[2]) {
+    const float4 *src = reinterpret_cast<const float4 *>(dA) + ((int64_t)t * kDenseWaves + wave) * 2 * kWave + lane;
+    a[0] = src[0];
+    a[1] = src[kWave];
+  };
+  // byte offset of the lane's piece of group g inside a staged buffer at reduction step 0: off_main + 256 g,
+  // except that the last group's pieces beyond the row end are clamped to the row's last piece (their result
+  // columns are never stored)
+  const int off_main = q * rs + 16 * c16;
+  int last_col = (NG - 1) * 64 + 4 * c16;
+  last_col = last_col < rs / 4 - 4 ? last_col : rs / 4 - 4;
+  const int off_last = q * rs + last_col * 4;
+  auto b_read = [&](const char *lb, int ks, int g) {
+    return *reinterpret_cast<const float4 *>(lb + ks * 4 * rs + (g < NG - 1 ? off_main + g * 256 : off_last));
+  };
+
+  float4 a_cur[2];
+  int hn;
+  {
+    const int h0 = hdr_load(t_first);
+    hn = hdr_load(t_first + 1 < t_end ? t_first + 1 : t_first);
+    const float *src4[RPW];
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) src4[r] = B + (int64_t)__builtin_amdgcn_readlane(h0, r) * ldb;
+#pragma unroll
+    for (int pc = 0; pc < NPIECES; ++pc) stage_piece(pc, src4, 0);
+    a_load(t_first, a_cur);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  int buf = 0;
+  for (int u = u0; u < u1; ++u) {
+    panel_f4 acc[NG][4];
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[g][j] = (panel_f4){0.f, 0.f, 0.f, 0.f};
+    const int ut1 = unit_tile[u + 1];
+    for (int t = unit_tile[u]; t < ut1; ++t) {
+      // the operands of this tile and the header of the next arrived before the last barrier: naming them here
+      // puts the compiler's wait for them ahead of the copies it cannot see
+      asm volatile("" ::"v"(a_cur[0].x), "v"(a_cur[1].x), "v"(hn));
+      const float *src4[RPW];  // the next tile (the last tile of the share names itself and is staged once more)
+#pragma unroll
+      for (int r = 0; r < RPW; ++r) src4[r] = B + (int64_t)__builtin_amdgcn_readlane(hn, r) * ldb;
+      int hn2 = 0;
+      float4 a_nxt[2];
+      const float a8[8] = {a_cur[0].x, a_cur[0].y, a_cur[0].z, a_cur[0].w, a_cur[1].x, a_cur[1].y, a_cur[1].z, a_cur[1].w};
+      const char *lb = panel_lds + buf * bufsz;
+      float4 b[NG];
+#pragma unroll
+      for (int g = 0; g < NG; ++g) b[g] = b_read(lb, 0, g);
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        if (ks == 6) {  // operands of the next tile and the header of the one after it: late, when most of a8 is dead
+          hn2 = hdr_load(t + 2 < t_end ? t + 2 : t_end - 1);
+          a_load(t + 1 < t_end ? t + 1 : t, a_nxt);
+        }
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+          acc[g][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a8[ks], b[g].x, acc[g][0], 0, 0, 0);
+          acc[g][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a8[ks], b[g].y, acc[g][1], 0, 0, 0);
+          acc[g][2] = __builtin_amdgcn_mfma_f32_16x16x4f32(a8[ks], b[g].z, acc[g][2], 0, 0, 0);
+          acc[g][3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a8[ks], b[g].w, acc[g][3], 0, 0, 0);
+          // the piece of the next reduction step replaces the one just used, NG - 1 groups ahead of its use
+          if (ks + 1 < 8) b[g] = b_read(lb, ks + 1, g);
+          // the next tile's copies, spread over this tile's steps
+          if ((ks * NG + g) % 2 == 0 && (ks * NG + g) / 2 < NPIECES) stage_piece((ks * NG + g) / 2, src4, buf ^ 1);
+        }
+      }
+      a_cur[0] = a_nxt[0];
+      a_cur[1] = a_nxt[1];
+      hn = hn2;
+      buf ^= 1;
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+    }
+    // register v of acc[g][j] is row 16 w + 4 q + v, column 64 g + 4 c + j of the unit's block
+    const int block = unit_block[u];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      float *prow = P + ((int64_t)block * kPanelRows + wave * 16 + 4 * q + v) * f;
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const int col = g * 64 + 4 * c16;
+        if (col + 1 < f) *reinterpret_cast<float2 *>(prow + col) = make_float2(acc[g][0][v], acc[g][1][v]);
+        if (col + 3 < f) *reinterpret_cast<float2 *>(prow + col + 2) = make_float2(acc[g][2][v], acc[g][3][v]);
+      }
     }
   }
 }
@@ -294,45 +499,70 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_tile_count_kernel(
   if (t >= 0) atomicAdd(&tcount[t], 1u);
 }
 
-// flag[t] = 1 and kept[t] = tcount[t] for tiles with at least emin entries, else 0 (both arrays are then scanned)
-__global__ __launch_bounds__(kSpmmThreads) void panel_tile_select_kernel(const uint32_t *__restrict__ tcount, int64_t tiles,
-                                                                         uint32_t emin, uint32_t *__restrict__ flag,
-                                                                         uint32_t *__restrict__ kept) {
-  const int64_t t = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
-  if (t > tiles) return;
-  const bool on = t < tiles && tcount[t] >= emin;  // entry `tiles` is the slot the scans leave their totals in
-  flag[t] = on ? 1u : 0u;
-  kept[t] = on ? tcount[t] : 0u;
+// Tiles with emin .. dmin - 1 entries are staged ("active"), tiles with at least dmin entries are dense
+// (dmin == 0: none).  flag[t] = 1 and kept[t] = tcount[t] for active tiles, dflag / dkept the same for
+// dense ones, else 0 (the four arrays are then scanned).
+__device__ __forceinline__ int panel_tile_kind(uint32_t count, uint32_t emin, uint32_t dmin) {
+  if (dmin > 0 && count >= dmin) return 2;
+  return count >= emin ? 1 : 0;
 }
 
-// compact tables of the active tiles
+__global__ __launch_bounds__(kSpmmThreads) void panel_tile_select_kernel(const uint32_t *__restrict__ tcount, int64_t tiles,
+                                                                         uint32_t emin, uint32_t dmin,
+                                                                         uint32_t *__restrict__ flag, uint32_t *__restrict__ kept,
+                                                                         uint32_t *__restrict__ dflag,
+                                                                         uint32_t *__restrict__ dkept) {
+  const int64_t t = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (t > tiles) return;
+  const int kind = t < tiles ? panel_tile_kind(tcount[t], emin, dmin) : 0;  // entry `tiles` is the slot the scans leave their totals in
+  flag[t] = kind == 1 ? 1u : 0u;
+  kept[t] = kind == 1 ? tcount[t] : 0u;
+  dflag[t] = kind == 2 ? 1u : 0u;
+  dkept[t] = kind == 2 ? tcount[t] : 0u;
+}
+
+// compact tables of the tiles of one kind (1: active, 2: dense)
 __global__ __launch_bounds__(kSpmmThreads) void panel_tile_tables_kernel(const uint32_t *__restrict__ tcount,
                                                                          const uint32_t *__restrict__ tindex, int64_t tiles,
-                                                                         uint32_t emin, int32_t nkb,
+                                                                         uint32_t emin, uint32_t dmin, int kind, int32_t nkb,
                                                                          int32_t *__restrict__ tile_kb,
                                                                          int32_t *__restrict__ tile_panel) {
   const int64_t t = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
-  if (t >= tiles || tcount[t] < emin) return;
+  if (t >= tiles || panel_tile_kind(tcount[t], emin, dmin) != kind) return;
   tile_kb[tindex[t]] = (int32_t)(t % nkb);
   tile_panel[tindex[t]] = (int32_t)(t / nkb);
 }
 
-// sort keys: covered entries get (active tile * 16 + wave) as major and the slot as minor key, all others the
-// sentinel `ntiles * 16`, which a stable sort leaves behind the covered ones in their (row, col) order
+// sort keys: entries of active tiles get (active tile * 16 + wave) as major and the slot as minor key, entries of
+// no tile the sentinel `ntiles * 16`, which a stable sort leaves behind the first ones in their (row, col)
+// order, and entries of dense tiles sentinel + 1: those are written into their place of the dense tile right
+// here and take no further part.  Two entries of one (row, column) pair would land in the same place: the
+// exchange finds the second one (unless one of them is +0, which changes nothing) and raises *collision,
+// after which the caller builds the plan again without dense tiles.
 __global__ __launch_bounds__(kSpmmThreads) void panel_entry_key_kernel(
-    const int32_t *__restrict__ erow, const int32_t *__restrict__ colind, int64_t nnz, const int32_t *__restrict__ row_rank,
-    const int32_t *__restrict__ col_rank, int32_t prows, int32_t hot, int32_t nkb, const uint32_t *__restrict__ tcount,
-    const uint32_t *__restrict__ tindex, uint32_t emin, int32_t sentinel, int32_t *__restrict__ key,
-    int32_t *__restrict__ slot, int32_t *__restrict__ pos) {
+    const int32_t *__restrict__ erow, const int32_t *__restrict__ colind, const float *__restrict__ val, int64_t nnz,
+    const int32_t *__restrict__ row_rank, const int32_t *__restrict__ col_rank, int32_t prows, int32_t hot, int32_t nkb,
+    const uint32_t *__restrict__ tcount, const uint32_t *__restrict__ tindex, const uint32_t *__restrict__ dindex,
+    uint32_t emin, uint32_t dmin, int32_t sentinel, int32_t *__restrict__ key, int32_t *__restrict__ slot,
+    int32_t *__restrict__ pos, uint32_t *__restrict__ dA_bits, uint32_t *__restrict__ collision) {
   const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (k >= nnz) return;
   const int32_t rr = row_rank[erow[k]];
-  const int64_t t = panel_tile_of(rr, col_rank[colind[k]], prows, hot, nkb);
+  const int32_t cr = col_rank[colind[k]];
+  const int64_t t = panel_tile_of(rr, cr, prows, hot, nkb);
   int32_t ky = sentinel, sl = 0;
-  if (t >= 0 && tcount[t] >= emin) {
+  const int kind = t >= 0 ? panel_tile_kind(tcount[t], emin, dmin) : 0;
+  if (kind == 1) {
     const int32_t p = rr % kPanelRows;
     ky = (int32_t)tindex[t] * kPanelWaves + p % kPanelWaves;
     sl = p / kPanelWaves;
+  } else if (kind == 2) {
+    const int32_t p = rr % kPanelRows, c = cr % kPanelCols;
+    const int32_t w = p / 16, ks = c / 4, lane = (c % 4) * 16 + p % 16;
+    const int64_t at = (((int64_t)dindex[t] * kDenseWaves + w) * 2 + ks / 4) * 256 + lane * 4 + ks % 4;
+    const uint32_t old = atomicExch(&dA_bits[at], __float_as_uint(val[k]));  // integer exchange of the value's bits
+    if (old != 0u) atomicOr(collision, 1u);
+    ky = sentinel + 1;
   }
   key[k] = ky;
   slot[k] = sl;
@@ -341,12 +571,12 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_entry_key_kernel(
 
 // after the sort: records of the covered entries, and the arrays of the rest
 __global__ __launch_bounds__(kSpmmThreads) void panel_entry_finish_kernel(
-    const int32_t *__restrict__ slot_sorted, const int32_t *__restrict__ pos, int64_t nnz, int64_t covered,
+    const int32_t *__restrict__ slot_sorted, const int32_t *__restrict__ pos, int64_t count, int64_t covered,
     const int32_t *__restrict__ erow, const int32_t *__restrict__ colind, const float *__restrict__ val,
     const int32_t *__restrict__ col_rank, uint2 *__restrict__ ent, int32_t *__restrict__ rest_row,
     int32_t *__restrict__ rest_col, float *__restrict__ rest_val) {
   const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
-  if (k >= nnz) return;
+  if (k >= count) return;  // count = entries of active tiles + rest; the entries of dense tiles lie behind them
   const int32_t p = pos[k];
   if (k < covered) {
     ent[k] = make_uint2((uint32_t)(col_rank[colind[p]] % kPanelCols) | ((uint32_t)slot_sorted[k] << 8), __float_as_uint(val[p]));
@@ -368,6 +598,15 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_hdr_kernel(const int32_t *
   const int w = (int)(k % kPanelWaves);
   const int64_t c = (int64_t)tile_kb[t] * kPanelCols + w;
   hdr[k] = make_int4(qcol[c], qcol[c + kPanelWaves], tile_wptr[k], tile_wptr[k + 1]);
+}
+
+// dhdr[t * 32 + j] = row of B of column j of dense tile t's block
+__global__ __launch_bounds__(kSpmmThreads) void panel_dense_hdr_kernel(const int32_t *__restrict__ dtile_kb,
+                                                                        const int32_t *__restrict__ qcol, int64_t ndtiles,
+                                                                        int32_t *__restrict__ dhdr) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k >= ndtiles * kPanelCols) return;
+  dhdr[k] = qcol[(int64_t)dtile_kb[k / kPanelCols] * kPanelCols + k % kPanelCols];
 }
 
 __global__ __launch_bounds__(kSpmmThreads) void panel_dslot_kernel(const int32_t *__restrict__ row_rank, int32_t n,

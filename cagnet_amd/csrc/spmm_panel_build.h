@@ -47,22 +47,19 @@ static int alloc_sort_buffers(DevTemps &tmp, SortBuffers &buf, int64_t count) {
   return CG_OK;
 }
 
-// may_decline: leave the plan empty (pp.declined) when the active tiles hold too few of the entries.
-static int build_panel(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot_req, int32_t unit_entries, bool may_decline,
-                       hipStream_t stream) {
-  CG_TRY(refuse_under_capture(stream, "building a panel plan"));
-  CG_HIP(hipStreamSynchronize(stream));
-  pp.release();
-  pp.emin = emin;
-  pp.hot_cols = hot_req;
-  pp.unit_entries = unit_entries;
+constexpr int32_t kPanelDefaultDmin = 2048;            // entries from which a 128 x 32 tile is stored whole and multiplied
+                                                       // on the matrix cores (half full); negative tuning value: never
+
+// may_decline: leave the plan empty (pp.declined) when the tiles hold too few of the entries.
+// *collision: two entries of one (row, column) pair fell into a dense tile; the plan is unusable.
+// dwg: workgroups of the dense-tile kernel (each takes an equal share of the dense tiles).
+static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot_req, int32_t unit_entries, int32_t dmin,
+                            int32_t dwg, bool may_decline, bool *collision, hipStream_t stream) {
+  *collision = false;
   const int64_t nnz = s.nnz;
   const int32_t n = s.rows, m = s.cols;
   auto decline = [&]() {
     pp.release();
-    pp.emin = emin;
-    pp.hot_cols = hot_req;
-    pp.unit_entries = unit_entries;
     pp.declined = true;
     pp.valid = true;
     return CG_OK;
@@ -119,40 +116,62 @@ static int build_panel(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot_req,
     CG_HIP(hipStreamSynchronize(stream));
   }
 
-  // 2. entries per tile; active tiles = those with at least emin entries
+  // 2. entries per tile; active tiles = those with emin .. dmin - 1 entries, dense tiles = those with more
   int32_t *erow = nullptr;
-  uint32_t *tcount = nullptr, *tindex = nullptr, *kept = nullptr, *d_tot = nullptr;
+  uint32_t *tcount = nullptr, *tindex = nullptr, *kept = nullptr, *dindex = nullptr, *dkept = nullptr, *d_tot = nullptr;
   CG_TRY(tmp.alloc((void **)&erow, (size_t)nnz * 4));
   CG_TRY(tmp.alloc((void **)&tcount, (size_t)(tiles + 1) * 4));
   CG_TRY(tmp.alloc((void **)&tindex, (size_t)(tiles + 1) * 4));
   CG_TRY(tmp.alloc((void **)&kept, (size_t)(tiles + 1) * 4));
-  CG_TRY(tmp.alloc((void **)&d_tot, 2 * 4));
+  CG_TRY(tmp.alloc((void **)&dindex, (size_t)(tiles + 1) * 4));
+  CG_TRY(tmp.alloc((void **)&dkept, (size_t)(tiles + 1) * 4));
+  CG_TRY(tmp.alloc((void **)&d_tot, 5 * 4));
   panel_expand_rows_kernel<<<(unsigned)ceil_div64((int64_t)n * kWave, kSpmmThreads), kSpmmThreads, 0, stream>>>(s.rowptr, n, erow);
   CG_LAUNCH_CHECK();
   CG_TRY(fill_u32(tcount, tiles + 1, 0u, stream));
+  CG_TRY(fill_u32(d_tot, 5, 0u, stream));
   panel_tile_count_kernel<<<ge, kSpmmThreads, 0, stream>>>(erow, s.colind, nnz, row_rank, col_rank, prows, hot, nkb, tcount);
   CG_LAUNCH_CHECK();
-  panel_tile_select_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, tiles, (uint32_t)emin, tindex, kept);
+  panel_tile_select_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, tiles, (uint32_t)emin, (uint32_t)dmin, tindex, kept, dindex,
+                                                           dkept);
   CG_LAUNCH_CHECK();
   CG_TRY(exclusive_scan_u32(tindex, tindex, tiles + 1, d_tot + 0, stream));
   CG_TRY(exclusive_scan_u32(kept, kept, tiles + 1, d_tot + 1, stream));
-  uint32_t tot[2] = {0, 0};
-  CG_HIP(hipMemcpyAsync(tot, d_tot, sizeof(tot), hipMemcpyDeviceToHost, stream));
+  CG_TRY(exclusive_scan_u32(dindex, dindex, tiles + 1, d_tot + 2, stream));
+  CG_TRY(exclusive_scan_u32(dkept, dkept, tiles + 1, d_tot + 3, stream));
+  uint32_t tot[5] = {0, 0, 0, 0, 0};
+  CG_HIP(hipMemcpyAsync(tot, d_tot, 4 * 4, hipMemcpyDeviceToHost, stream));
   CG_HIP(hipStreamSynchronize(stream));
-  const int64_t ntiles = tot[0], covered = tot[1];
-  if (ntiles == 0 || covered == 0 || (may_decline && (double)covered < kPanelMinCoverage * (double)nnz)) return decline();
-  if (ntiles * kPanelWaves + 1 > 0x7fffffffLL) return decline();
+  const int64_t ntiles = tot[0], covered = tot[1], ndtiles = tot[2], dcovered = tot[3];
+  if (ntiles + ndtiles == 0 || covered + dcovered == 0 ||
+      (may_decline && (double)(covered + dcovered) < kPanelMinCoverage * (double)nnz))
+    return decline();
+  if (ntiles * kPanelWaves + 2 > 0x7fffffffLL || ndtiles * kDenseTileFloats > 0x7fffffffLL * 4) return decline();
 
-  // 3. tables of the active tiles
-  int32_t *tile_panel = nullptr, *tile_kb = nullptr, *tile_wptr = nullptr;
-  CG_TRY(tmp.alloc((void **)&tile_kb, (size_t)ntiles * 4));
-  CG_TRY(tmp.alloc((void **)&tile_panel, (size_t)ntiles * 4));
-  panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, tindex, tiles, (uint32_t)emin, nkb, tile_kb, tile_panel);
+  // 3. tables of the active and of the dense tiles
+  int32_t *tile_panel = nullptr, *tile_kb = nullptr, *tile_wptr = nullptr, *dtile_panel = nullptr, *dtile_kb = nullptr;
+  CG_TRY(tmp.alloc((void **)&tile_kb, (size_t)(ntiles + 1) * 4));
+  CG_TRY(tmp.alloc((void **)&tile_panel, (size_t)(ntiles + 1) * 4));
+  CG_TRY(tmp.alloc((void **)&dtile_kb, (size_t)(ndtiles + 1) * 4));
+  CG_TRY(tmp.alloc((void **)&dtile_panel, (size_t)(ndtiles + 1) * 4));
+  panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, tindex, tiles, (uint32_t)emin, (uint32_t)dmin, 1, nkb, tile_kb,
+                                                           tile_panel);
   CG_LAUNCH_CHECK();
+  if (ndtiles > 0) {
+    panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, dindex, tiles, (uint32_t)emin, (uint32_t)dmin, 2, nkb,
+                                                             dtile_kb, dtile_panel);
+    CG_LAUNCH_CHECK();
+    CG_TRY(dev_alloc((void **)&pp.dA, (size_t)ndtiles * kDenseTileFloats * 4));
+    CG_TRY(dev_alloc((void **)&pp.dhdr, (size_t)ndtiles * kPanelCols * 4));
+    CG_HIP(hipMemsetAsync(pp.dA, 0, (size_t)ndtiles * kDenseTileFloats * 4, stream));
+    panel_dense_hdr_kernel<<<(unsigned)ceil_div64(ndtiles * kPanelCols, kSpmmThreads), kSpmmThreads, 0, stream>>>(
+        dtile_kb, qcol, ndtiles, pp.dhdr);
+    CG_LAUNCH_CHECK();
+  }
 
-  // 4. one stable sort puts the covered entries first, by (tile, wave, slot), and leaves the others
-  //    behind them in (row, col) order: those are the rest matrix
-  const int64_t nrest = nnz - covered;
+  // 4. one stable sort puts the entries of active tiles first, by (tile, wave, slot), leaves those of no tile
+  //    behind them in (row, col) order (the rest matrix) and those of dense tiles, already stored, last
+  const int64_t nrest = nnz - covered - dcovered;
   pp.rest = new (std::nothrow) CsrSide();
   if (!pp.rest) CG_FAIL(CG_ERR_ALLOC, "panel plan: host allocation failed");
   CsrSide &rest = *pp.rest;
@@ -173,73 +192,115 @@ static int build_panel(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot_req,
     CG_TRY(alloc_sort_buffers(t2, buf, nnz));
     CG_TRY(t2.alloc((void **)&rest_row, (size_t)(nrest > 0 ? nrest : 1) * 4));
     const int32_t sentinel = (int32_t)(ntiles * kPanelWaves);
-    panel_entry_key_kernel<<<ge, kSpmmThreads, 0, stream>>>(erow, s.colind, nnz, row_rank, col_rank, prows, hot, nkb, tcount,
-                                                            tindex, (uint32_t)emin, sentinel, buf.key_a[0], buf.key_b[0],
-                                                            buf.payload[0]);
+    panel_entry_key_kernel<<<ge, kSpmmThreads, 0, stream>>>(erow, s.colind, s.val, nnz, row_rank, col_rank, prows, hot, nkb, tcount,
+                                                            tindex, dindex, (uint32_t)emin, (uint32_t)dmin, sentinel,
+                                                            buf.key_a[0], buf.key_b[0], buf.payload[0], (uint32_t *)pp.dA,
+                                                            d_tot + 4);
     CG_LAUNCH_CHECK();
     int set = 0;
-    CG_TRY(radix_sort_pairs(buf, nnz, bits_for(sentinel + 1), bits_for(kPanelSlots), &set, stream));
-    panel_entry_finish_kernel<<<ge, kSpmmThreads, 0, stream>>>(buf.key_b[set], buf.payload[set], nnz, covered, erow, s.colind,
-                                                               s.val, col_rank, pp.ent, rest_row, rest.colind, rest.val);
-    CG_LAUNCH_CHECK();
+    CG_TRY(radix_sort_pairs(buf, nnz, bits_for(sentinel + 2), bits_for(kPanelSlots), &set, stream));
+    if (covered + nrest > 0) {
+      panel_entry_finish_kernel<<<(unsigned)ceil_div64(covered + nrest, kSpmmThreads), kSpmmThreads, 0, stream>>>(
+          buf.key_b[set], buf.payload[set], covered + nrest, covered, erow, s.colind, s.val, col_rank, pp.ent, rest_row,
+          rest.colind, rest.val);
+      CG_LAUNCH_CHECK();
+    }
     CG_TRY(launch_rowptr(buf.key_a[set], covered, sentinel, tile_wptr, stream));
-    panel_hdr_kernel<<<(unsigned)ceil_div64(ntiles * kPanelWaves, kSpmmThreads), kSpmmThreads, 0, stream>>>(
-        tile_kb, tile_wptr, qcol, ntiles, (int4 *)pp.hdr);
-    CG_LAUNCH_CHECK();
+    if (ntiles > 0) {
+      panel_hdr_kernel<<<(unsigned)ceil_div64(ntiles * kPanelWaves, kSpmmThreads), kSpmmThreads, 0, stream>>>(
+          tile_kb, tile_wptr, qcol, ntiles, (int4 *)pp.hdr);
+      CG_LAUNCH_CHECK();
+    }
     CG_TRY(launch_rowptr(rest_row, nrest, n, rest.rowptr, stream));
+    CG_HIP(hipMemcpyAsync(tot + 4, d_tot + 4, 4, hipMemcpyDeviceToHost, stream));
     CG_HIP(hipStreamSynchronize(stream));
+  }
+  if (tot[4] != 0) {
+    *collision = true;
+    return CG_OK;
   }
   CG_TRY(side_max_degree(rest, stream));
 
-  // 5. units: runs of tiles of one panel with about unit_entries entries, heaviest first at launch
-  std::vector<int32_t> h_panel((size_t)ntiles), h_base((size_t)ntiles + 1);
+  // 5. units: runs of tiles of one panel and one kind, with about unit_entries entries (active tiles) or inside one
+  //    workgroup's share (dense tiles); each unit writes one block of 128 partial rows, the blocks of a panel are
+  //    consecutive
+  std::vector<int32_t> h_panel((size_t)ntiles), h_base((size_t)ntiles + 1, 0), h_dpanel((size_t)ndtiles);
   {
-    // entries of active tile k = difference of the scanned kept[] at its all-tile index; read them compacted
-    // through the (tile, wave) table instead: tile_wptr[16 k] is the first record of tile k
+    // entries of active tile k: tile_wptr[16 k] is its first record
     std::vector<int32_t> h_wptr((size_t)ntiles * kPanelWaves + 1);
     CG_HIP(hipMemcpyAsync(h_wptr.data(), tile_wptr, h_wptr.size() * 4, hipMemcpyDeviceToHost, stream));
-    CG_HIP(hipMemcpyAsync(h_panel.data(), tile_panel, (size_t)ntiles * 4, hipMemcpyDeviceToHost, stream));
+    if (ntiles > 0) CG_HIP(hipMemcpyAsync(h_panel.data(), tile_panel, (size_t)ntiles * 4, hipMemcpyDeviceToHost, stream));
+    if (ndtiles > 0) CG_HIP(hipMemcpyAsync(h_dpanel.data(), dtile_panel, (size_t)ndtiles * 4, hipMemcpyDeviceToHost, stream));
     CG_HIP(hipStreamSynchronize(stream));
     for (int64_t k = 0; k <= ntiles; ++k) h_base[(size_t)k] = h_wptr[(size_t)k * kPanelWaves];
   }
-  std::vector<int32_t> unit_tile, split, panel_unit((size_t)npanels, -1);
-  std::vector<int64_t> unit_size;
-  unit_tile.push_back(0);
-  int64_t in_unit = 0;
-  for (int64_t k = 0; k < ntiles; ++k) {
-    const int64_t e = (int64_t)h_base[(size_t)k + 1] - h_base[(size_t)k];
-    const bool new_panel = k > 0 && h_panel[(size_t)k] != h_panel[(size_t)k - 1];
-    if (k > unit_tile.back() && (new_panel || in_unit + e > unit_entries)) {
-      unit_size.push_back(in_unit);
-      unit_tile.push_back((int32_t)k);
-      in_unit = 0;
+  struct Unit {
+    int32_t panel, t0, t1;
+    int64_t weight;
+  };
+  std::vector<Unit> su, du;  // units of active tiles, of dense tiles; both in panel order
+  for (int64_t k = 0; k < ntiles;) {
+    int64_t j = k, in_unit = 0;
+    while (j < ntiles && h_panel[(size_t)j] == h_panel[(size_t)k]) {
+      const int64_t e = (int64_t)h_base[(size_t)j + 1] - h_base[(size_t)j];
+      if (j > k && in_unit + e > unit_entries) break;
+      in_unit += e;
+      ++j;
     }
-    in_unit += e;
+    su.push_back(Unit{h_panel[(size_t)k], (int32_t)k, (int32_t)j, in_unit});
+    k = j;
   }
-  unit_size.push_back(in_unit);
-  unit_tile.push_back((int32_t)ntiles);
-  const int32_t nunits = (int32_t)unit_size.size();
-  for (int32_t u = 0; u < nunits;) {  // units of one panel are consecutive
-    const int32_t panel = h_panel[(size_t)unit_tile[(size_t)u]];
-    int32_t v = u + 1;
-    while (v < nunits && h_panel[(size_t)unit_tile[(size_t)v]] == panel) ++v;
-    panel_unit[(size_t)panel] = u;
-    if (v - u > 1) {
-      split.push_back(u);
-      split.push_back(v - u);
+  const int32_t ndwg = (int32_t)(ndtiles < dwg ? ndtiles : dwg);
+  std::vector<int32_t> dwg_unit((size_t)ndwg + 1, 0);
+  for (int64_t k = 0, w = 0; k < ndtiles;) {
+    while ((int64_t)ndtiles * (w + 1) / ndwg <= k) dwg_unit[(size_t)++w] = (int32_t)du.size();  // share that holds tile k
+    const int64_t share_end = (int64_t)ndtiles * (w + 1) / ndwg;
+    int64_t j = k;
+    while (j < ndtiles && h_dpanel[(size_t)j] == h_dpanel[(size_t)k] && j < share_end) ++j;
+    du.push_back(Unit{h_dpanel[(size_t)k], (int32_t)k, (int32_t)j, j - k});
+    k = j;
+  }
+  if (ndwg > 0) dwg_unit[(size_t)ndwg] = (int32_t)du.size();
+  const int32_t nunits = (int32_t)su.size(), ndunits = (int32_t)du.size();
+  std::vector<int32_t> unit_tile((size_t)nunits + 1, 0), unit_block((size_t)nunits), dunit_tile((size_t)ndunits + 1, 0),
+      dunit_block((size_t)ndunits), split, panel_unit((size_t)npanels, -1);
+  int32_t nblocks = 0;
+  for (size_t a = 0, b = 0; a < su.size() || b < du.size();) {  // merge by panel: dense units first, then the others
+    const int32_t pa = a < su.size() ? su[a].panel : 0x7fffffff, pb = b < du.size() ? du[b].panel : 0x7fffffff;
+    const int32_t panel = pa < pb ? pa : pb;
+    const int32_t first = nblocks;
+    for (; b < du.size() && du[b].panel == panel; ++b) dunit_block[b] = nblocks++;
+    for (; a < su.size() && su[a].panel == panel; ++a) unit_block[a] = nblocks++;
+    panel_unit[(size_t)panel] = first;
+    if (nblocks - first > 1) {
+      split.push_back(first);
+      split.push_back(nblocks - first);
     }
-    u = v;
   }
+  for (int32_t u = 0; u < nunits; ++u) unit_tile[(size_t)u + 1] = su[(size_t)u].t1;
+  for (int32_t u = 0; u < ndunits; ++u) dunit_tile[(size_t)u + 1] = du[(size_t)u].t1;
   std::vector<int32_t> order((size_t)nunits);
   for (int32_t u = 0; u < nunits; ++u) order[(size_t)u] = u;
-  std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return unit_size[(size_t)a] > unit_size[(size_t)b]; });
+  std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return su[(size_t)a].weight > su[(size_t)b].weight; });
   int32_t *d_panel_unit = nullptr;
   CG_TRY(tmp.alloc((void **)&d_panel_unit, (size_t)npanels * 4));
   CG_TRY(dev_alloc((void **)&pp.unit_tile, (size_t)(nunits + 1) * 4));
   CG_TRY(dev_alloc((void **)&pp.unit_order, (size_t)nunits * 4));
+  CG_TRY(dev_alloc((void **)&pp.unit_block, (size_t)nunits * 4));
   CG_TRY(dev_alloc((void **)&pp.dslot, (size_t)n * 4));
   CG_HIP(hipMemcpyAsync(pp.unit_tile, unit_tile.data(), (size_t)(nunits + 1) * 4, hipMemcpyHostToDevice, stream));
-  CG_HIP(hipMemcpyAsync(pp.unit_order, order.data(), (size_t)nunits * 4, hipMemcpyHostToDevice, stream));
+  if (nunits > 0) {
+    CG_HIP(hipMemcpyAsync(pp.unit_order, order.data(), (size_t)nunits * 4, hipMemcpyHostToDevice, stream));
+    CG_HIP(hipMemcpyAsync(pp.unit_block, unit_block.data(), (size_t)nunits * 4, hipMemcpyHostToDevice, stream));
+  }
+  if (ndunits > 0) {
+    CG_TRY(dev_alloc((void **)&pp.dwg_unit, (size_t)(ndwg + 1) * 4));
+    CG_TRY(dev_alloc((void **)&pp.dunit_tile, (size_t)(ndunits + 1) * 4));
+    CG_TRY(dev_alloc((void **)&pp.dunit_block, (size_t)ndunits * 4));
+    CG_HIP(hipMemcpyAsync(pp.dwg_unit, dwg_unit.data(), (size_t)(ndwg + 1) * 4, hipMemcpyHostToDevice, stream));
+    CG_HIP(hipMemcpyAsync(pp.dunit_tile, dunit_tile.data(), (size_t)(ndunits + 1) * 4, hipMemcpyHostToDevice, stream));
+    CG_HIP(hipMemcpyAsync(pp.dunit_block, dunit_block.data(), (size_t)ndunits * 4, hipMemcpyHostToDevice, stream));
+  }
   CG_HIP(hipMemcpyAsync(d_panel_unit, panel_unit.data(), (size_t)npanels * 4, hipMemcpyHostToDevice, stream));
   if (!split.empty()) {
     CG_TRY(dev_alloc((void **)&pp.split, split.size() * 4));
@@ -249,50 +310,139 @@ static int build_panel(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot_req,
   CG_LAUNCH_CHECK();
   CG_HIP(hipStreamSynchronize(stream));
   pp.covered = covered;
+  pp.dcovered = dcovered;
   pp.ntiles = (int32_t)ntiles;
+  pp.ndtiles = (int32_t)ndtiles;
   pp.nunits = nunits;
+  pp.ndunits = ndunits;
+  pp.ndwg = ndwg;
+  pp.nblocks = nblocks;
   pp.nsplit = (int32_t)(split.size() / 2);
-  pp.hot_cols = hot_req;
   pp.valid = true;
   return CG_OK;
 }
 
-// The panel part of C = A B: partial rows of every row that has entries in active tiles, in *P
+struct PanelParams {
+  int32_t emin, cols, unit, dmin, dwg;
+  bool same(const PanelPlan &pp) const {
+    return pp.emin == emin && pp.hot_cols == cols && pp.unit_entries == unit && pp.dmin == dmin && pp.dwg == dwg;
+  }
+  void stamp(PanelPlan &pp) const {
+    pp.emin = emin;
+    pp.hot_cols = cols;
+    pp.unit_entries = unit;
+    pp.dmin = dmin;
+    pp.dwg = dwg;
+  }
+};
+
+static PanelParams panel_params() {
+  PanelParams p;
+  p.emin = g_tune_panel_emin.load(std::memory_order_relaxed);
+  if (p.emin <= 0) p.emin = kPanelDefaultEmin;
+  p.cols = g_tune_panel_cols.load(std::memory_order_relaxed);
+  if (p.cols <= 0) p.cols = kPanelDefaultCols;
+  p.unit = g_tune_panel_unit.load(std::memory_order_relaxed);
+  if (p.unit <= 0) p.unit = kPanelDefaultUnit;
+  p.dmin = g_tune_panel_dmin.load(std::memory_order_relaxed);
+  p.dmin = p.dmin < 0 ? 0 : (p.dmin == 0 ? kPanelDefaultDmin : p.dmin);  // 0 from here on: no dense tiles
+  if (p.dmin > 0 && p.dmin < p.emin) p.dmin = p.emin;
+  p.dwg = g_tune_panel_dwg.load(std::memory_order_relaxed);
+  if (p.dwg <= 0) {  // four workgroups per compute unit, one after the other (a workgroup's staging buffers fill a unit's LDS)
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        cus < 1) {
+      (void)hipGetLastError();
+      cus = 256;
+    }
+    p.dwg = 4 * cus;
+  }
+  return p;
+}
+
+// Builds the plan for the given values; the plan carries them whatever the outcome (in use, declined).
+static int build_panel(CsrSide &s, PanelPlan &pp, const PanelParams &par, bool may_decline, hipStream_t stream) {
+  CG_TRY(refuse_under_capture(stream, "building a panel plan"));
+  CG_HIP(hipStreamSynchronize(stream));
+  pp.release();
+  bool collision = false;
+  int st = build_panel_once(s, pp, par.emin, par.cols, par.unit, par.dmin, par.dwg, may_decline, &collision, stream);
+  if (st == CG_OK && collision) {  // the matrix stores a (row, column) pair twice: every tile goes the record way
+    pp.release();
+    st = build_panel_once(s, pp, par.emin, par.cols, par.unit, 0, par.dwg, may_decline, &collision, stream);
+  }
+  if (st != CG_OK) pp.release();
+  par.stamp(pp);
+  return st;
+}
+
+// One bit per device and kernel: the dynamic LDS limit of the kernel has been raised there.
+template <typename K>
+static int panel_lds_attr(K kernel, std::atomic<uint64_t> &done, int dev, size_t lds_max, size_t lds_now) {
+  if (dev < 64 && !(done.load() >> dev & 1)) {
+    CG_HIP(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_max));
+    done.fetch_or((uint64_t)1 << dev);
+  } else if (dev >= 64) {
+    CG_HIP(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_now));
+  }
+  return CG_OK;
+}
+
+// The panel part of C = A B: partial rows of every row that has entries in active or dense tiles, in *P
 // (row r: P + dslot[r] * f).  P is stream scratch and stays valid until the next panel product on `stream`.
 static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_t f, float **P_out, hipStream_t stream) {
   const int chunks = (f / 2 + kWave - 1) / kWave;
+  const int groups = (f + 63) / 64;
   const size_t rs = ((size_t)f * 4 + 15) & ~(size_t)15;
   const size_t lds = 2 * (size_t)kPanelCols * rs;
+  const size_t lds_max = 2 * (size_t)kPanelCols * ((kPanelMaxF * 4 + 15) & ~15);
   void *p = nullptr;
-  CG_TRY(scratch_get(stream, kSlotE, (size_t)pp.nunits * kPanelRows * f * sizeof(float), &p));
+  CG_TRY(scratch_get(stream, kSlotE, (size_t)pp.nblocks * kPanelRows * f * sizeof(float), &p));
   float *P = (float *)p;
   int dev = 0;
   CG_HIP(hipGetDevice(&dev));
+  if (pp.ndunits > 0) {
+    ProfScope prof("spmm_panel_dense", f, stream);
+#define CG_PANEL_DENSE(NG)                                                                                              \
+  case NG: {                                                                                                            \
+    static std::atomic<uint64_t> attr_set{0};                                                                           \
+    CG_TRY(panel_lds_attr(spmm_panel_dense_kernel<NG>, attr_set, dev, lds_max, lds));                                   \
+    spmm_panel_dense_kernel<NG><<<(unsigned)pp.ndwg, kDenseThreads, lds, stream>>>(                                     \
+        pp.dwg_unit, pp.dunit_tile, pp.dunit_block, pp.dhdr, pp.dA, B, ldb, P, f);                                      \
+  } break;
+    switch (groups) {
+      CG_PANEL_DENSE(5)
+      CG_PANEL_DENSE(6)
+      CG_PANEL_DENSE(7)
+      CG_PANEL_DENSE(8)
+      CG_PANEL_DENSE(9)
+      CG_PANEL_DENSE(10)
+      default:
+        CG_FAIL(CG_ERR_UNSUPPORTED, "panel product: no dense-tile kernel for f=%d", f);
+    }
+#undef CG_PANEL_DENSE
+    CG_LAUNCH_CHECK();
+  }
   {
     ProfScope prof("spmm_panel", f, stream);
-#define CG_PANEL(CH)                                                                                                  \
-  case CH: {                                                                                                          \
-    static std::atomic<uint64_t> attr_set{0}; /* one bit per device: the LDS size of this kernel has been raised */   \
-    if (dev < 64 && !(attr_set.load() >> dev & 1)) {                                                                  \
-      CG_HIP(hipFuncSetAttribute((const void *)spmm_panel_kernel<CH>, hipFuncAttributeMaxDynamicSharedMemorySize,     \
-                                 (int)(2 * (size_t)kPanelCols * ((kPanelMaxF * 4 + 15) & ~15))));                     \
-      attr_set.fetch_or((uint64_t)1 << dev);                                                                          \
-    } else if (dev >= 64) {                                                                                           \
-      CG_HIP(hipFuncSetAttribute((const void *)spmm_panel_kernel<CH>, hipFuncAttributeMaxDynamicSharedMemorySize,     \
-                                 (int)lds));                                                                          \
-    }                                                                                                                 \
-    spmm_panel_kernel<CH><<<(unsigned)pp.nunits, kPanelThreads, lds, stream>>>(pp.unit_tile, pp.unit_order, pp.hdr, pp.ent, B, \
-                                                                               ldb, P, f);                                 \
+#define CG_PANEL(CH)                                                                                                   \
+  case CH: {                                                                                                           \
+    static std::atomic<uint64_t> attr_set{0};                                                                          \
+    CG_TRY(panel_lds_attr(spmm_panel_kernel<CH>, attr_set, dev, lds_max, lds));                                        \
+    spmm_panel_kernel<CH><<<(unsigned)pp.nunits, kPanelThreads, lds, stream>>>(pp.unit_tile, pp.unit_order, pp.unit_block, \
+                                                                               pp.hdr, pp.ent, B, ldb, P, f);          \
   } break;
-    switch (chunks) {
-      CG_PANEL(3)
-      CG_PANEL(4)
-      CG_PANEL(5)
-      default:
-        CG_FAIL(CG_ERR_UNSUPPORTED, "panel product: no kernel for f=%d", f);
+    if (pp.nunits > 0) {
+      switch (chunks) {
+        CG_PANEL(3)
+        CG_PANEL(4)
+        CG_PANEL(5)
+        default:
+          CG_FAIL(CG_ERR_UNSUPPORTED, "panel product: no kernel for f=%d", f);
+      }
+      CG_LAUNCH_CHECK();
     }
 #undef CG_PANEL
-    CG_LAUNCH_CHECK();
     if (pp.nsplit > 0) {
       const dim3 grid((unsigned)ceil_div64((int64_t)kPanelRows * f, kSpmmThreads), (unsigned)pp.nsplit);
       panel_reduce_kernel<<<grid, kSpmmThreads, 0, stream>>>(pp.split, P, f);

@@ -199,12 +199,14 @@ int cg_csr_spmm_xw(cg_csr_t *h, int transpose, const float *d_B, int64_t ldb, co
  *                column-popularity plan last looked up by a wide product of A, of A^T:
  *                tiers in use, -1 when the column counts declined it, 0 when none was considered } */
 int cg_csr_info(const cg_csr_t *h, int64_t info[8]);
-/* Panel plan a wide product of A (transpose != 0: of A^T) last looked up: info[0..7] =
- * { 1 in use / -1 declined (the dense tiles hold too few of the entries) / 0 none considered yet,
- *   entries multiplied out of LDS, active tiles, units (workgroups), row panels with several units,
- *   entries left to the row-wise kernels, entries a tile needs, ranked columns }.  No counterpart in the
+/* Panel plan a wide product of A (transpose != 0: of A^T) last looked up: info[0..11] =
+ * { 1 in use / -1 declined (the tiles hold too few of the entries) / 0 none considered yet,
+ *   entries multiplied out of LDS by the vector ALUs, their (active) tiles, their units (workgroups),
+ *   row panels with several units of either kind, entries left to the row-wise kernels, entries a tile
+ *   needs, ranked columns, entries in dense tiles (multiplied on the fp32 matrix cores), dense tiles, their
+ *   units, entries from which a tile is dense (0: no dense tiles were allowed) }.  No counterpart in the
  * reference, which hands the whole product to cusparseSpMM (sparse-extension/sparse_coo_tensor.cu:215-226). */
-int cg_csr_panel_info(const cg_csr_t *h, int transpose, int64_t info[8]);
+int cg_csr_panel_info(const cg_csr_t *h, int transpose, int64_t info[12]);
 /* Device pointers of the arrays the handle owns (transpose != 0: those of A^T). */
 int cg_csr_arrays(const cg_csr_t *h, int transpose, const int32_t **d_rowptr, const int32_t **d_colind,
                   const float **d_values);
@@ -348,6 +350,10 @@ int cg_prof_enable(int on);
  *   "spmm_panel_emin" entries a 128 x 32 tile needs to be staged (0: 64)
  *   "spmm_panel_cols" ranked columns that can be part of a tile (0: 131072)
  *   "spmm_panel_unit" entries after which the tiles of a row panel go to another workgroup (0: 65536)
+ *   "spmm_panel_dmin" entries from which a 128 x 32 tile is stored whole and multiplied on the fp32 matrix
+ *                     cores (0: 2048, half full; negative: never).  Such a tile multiplies its zeros too:
+ *                     a row of B with an infinity or a NaN then reaches all 128 rows of the tile
+ *   "spmm_panel_dwg"  workgroups that share the dense tiles equally (0: four per compute unit)
  *   "dense_mfma"      -1: dense products on the vector ALU tile kernel only
  *   "coo_cache_blocks" blocks cg_spmm_coo_cached keeps (0: 8; negative: none)
  *   "coo_cache_mib"   device memory those blocks may hold together, in MiB (0: 32768); a block counts as three

@@ -41,7 +41,7 @@ static void host_only() {
   EXPECT(cg_spmm_coo_cached(nullptr, nullptr, nullptr, -1, 4, 4, fone, 4, (float *)32, 4, 4, 1.f, nullptr) == CG_ERR_SIZE);
   EXPECT(cg_spmm_coo_cached(ione, ione, fone, 5, 4, 4, fone, 3, (float *)32, 4, 4, 1.f, nullptr) == CG_ERR_SIZE);
   EXPECT(cg_coo_cache_info(nullptr) == CG_ERR_NULL);
-  int64_t info[8] = {0};
+  int64_t info[12] = {0};
   EXPECT(cg_coo_cache_info(info) == CG_OK);
   EXPECT(cg_coo_cache_clear() == CG_OK);
   cg_csr_t *h = nullptr;
@@ -174,7 +174,7 @@ static void with_gpu() {
   const int widths[] = {16, 41, 258, 300, 384, 602, 636};
   cg_csr_t *h = nullptr;
   EXPECT(cg_csr_create(&h, d_row, d_col, d_val, nnz, n, m, CG_CSR_SORTED | CG_CSR_TRANSPOSE | CG_CSR_VALIDATE, stream) == CG_OK);
-  int64_t info[8] = {0};
+  int64_t info[12] = {0};
   EXPECT(cg_csr_info(h, info) == CG_OK && info[0] == n && info[1] == m && info[2] == nnz);
   for (int pass = 0; pass < 3; ++pass) {
     // pass 0: built-in choices; 1: hub plans forced (7 widths through 2 plan slots and 4 schedule slots);

@@ -3,7 +3,7 @@ import numpy as np
 import pytest
 import torch
 
-from tests.util import REL_TOL, random_coo, small_graph, spmm_error
+from tests.util import REL_TOL, gemm_error, random_coo, small_graph, spmm_error
 from oracle import gcn_oracle as orc
 
 pytestmark = pytest.mark.gpu
@@ -820,9 +820,10 @@ def test_spmm_from_two_host_threads_on_two_streams(cuda, tune):
 def _panel_info(A, transpose=False):
     import ctypes
     from cagnet_amd._lib import check, lib
-    buf = (ctypes.c_int64 * 8)()
+    buf = (ctypes.c_int64 * 12)()
     check(lib.cg_csr_panel_info(A._handle, int(transpose), buf), "cg_csr_panel_info")
-    return dict(state=buf[0], covered=buf[1], tiles=buf[2], units=buf[3], split=buf[4], rest=buf[5], emin=buf[6], cols=buf[7])
+    return dict(state=buf[0], covered=buf[1], tiles=buf[2], units=buf[3], split=buf[4], rest=buf[5], emin=buf[6], cols=buf[7],
+                dense_covered=buf[8], dense_tiles=buf[9], dense_units=buf[10], dmin=buf[11])
 
 
 @pytest.mark.parametrize("f", [258, 300, 384, 602, 636])
@@ -841,7 +842,8 @@ def test_spmm_panel_plan_matches_oracle(cuda, tune, f, emin, unit):
     tune("spmm_panel_unit", unit)
     got = A.spmm(B.to(cuda))
     info = _panel_info(A)
-    assert info["state"] == 1 and info["covered"] > 0 and info["covered"] + info["rest"] == row.numel()
+    assert info["state"] == 1 and info["covered"] > 0
+    assert info["covered"] + info["dense_covered"] + info["rest"] == row.numel()
     assert info["tiles"] > 0 and info["units"] >= 1
     if unit < 1000:
         assert info["split"] > 0
@@ -857,6 +859,86 @@ def test_spmm_panel_plan_matches_oracle(cuda, tune, f, emin, unit):
     tune("spmm_panel", -1)
     plain = A.spmm(B.to(cuda))
     assert spmm_error(plain, row, col, val, n, n, B) <= REL_TOL
+
+
+@pytest.mark.parametrize("f", [258, 320, 384, 448, 512, 576, 602, 636])
+@pytest.mark.parametrize("dmin,dwg", [(40, 3), (200, 0)])
+def test_spmm_panel_dense_tiles_on_matrix_cores(cuda, tune, f, dmin, dwg):
+    """The panel plan with its dense tiles forced on: (row panel, column block) tiles with at least dmin entries are
+    stored whole and multiplied by v_mfma_f32_16x16x4_f32 (exact fp32 products); dwg workgroups (0: one per compute
+    unit) share them equally, and the blocks of partial rows their units write are summed with those of the other
+    units of the panel; every result width class
+    (5..10 groups of 64 columns).  Same 1e-5 bound against the fp64 oracle, bit-identical repeats."""
+    from cagnet_amd import ops
+    row, col, val, n = small_graph(12, 160000, seed=11 * f + dmin)
+    B = torch.randn(n, f, generator=torch.Generator().manual_seed(f))
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n, transpose=True)
+    tune("spmm_panel", 1)
+    tune("spmm_panel_emin", 8)
+    tune("spmm_panel_cols", 2048)
+    tune("spmm_panel_dmin", dmin)
+    tune("spmm_panel_dwg", dwg)
+    got = A.spmm(B.to(cuda))
+    info = _panel_info(A)
+    assert info["state"] == 1 and info["dmin"] == dmin
+    assert info["dense_tiles"] > 0 and info["dense_covered"] >= dmin * info["dense_tiles"]
+    assert info["dense_units"] >= (min(dwg, info["dense_tiles"]) if dwg else 1)
+    assert info["covered"] + info["dense_covered"] + info["rest"] == row.numel()
+    assert spmm_error(got, row, col, val, n, n, B) <= REL_TOL
+    assert torch.equal(got, A.spmm(B.to(cuda)))                      # fixed summation order
+    C0 = torch.randn(n, f, generator=torch.Generator().manual_seed(f + 1))
+    C = C0.to(cuda).clone()
+    A.spmm(B.to(cuda), out=C, beta=1.0)
+    assert spmm_error(C, row, col, val, n, n, B, C0) <= REL_TOL
+    gotT = A.spmm(B.to(cuda), transpose=True)
+    assert _panel_info(A, transpose=True)["dense_tiles"] > 0
+    assert spmm_error(gotT, row, col, val, n, n, B) <= REL_TOL
+    tune("spmm_panel_dmin", -1)                                      # the same plan without dense tiles
+    rec = A.spmm(B.to(cuda))
+    assert _panel_info(A)["dense_tiles"] == 0 and _panel_info(A)["dmin"] == 0
+    assert spmm_error(rec, row, col, val, n, n, B) <= REL_TOL
+
+
+def test_spmm_panel_all_tiles_dense_and_duplicate_entries(cuda, tune):
+    """A small full matrix: every tile is dense and no unit of the record kind is left (also with a row count that is
+    not a multiple of the panel height and B as a strided slice).  Then a matrix that stores some (row, column) pairs
+    twice: two entries cannot share a place of a dense tile, so the plan falls back to records for every tile and the
+    product still adds both."""
+    from cagnet_amd import ops
+    n, m, f = 300, 200, 602
+    g = torch.Generator().manual_seed(3)
+    dense = torch.randn(n, m, generator=g)
+    row, col = torch.nonzero(torch.ones(n, m), as_tuple=True)
+    val = dense[row, col].contiguous()
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, m, transpose=True)
+    tune("spmm_panel", 1)
+    tune("spmm_panel_dmin", 512)
+    big = torch.randn(m, f + 8, generator=g).to(cuda)
+    B = big[:, 2:2 + f]
+    got = A.spmm(B)
+    info = _panel_info(A)
+    assert info["state"] == 1 and info["dense_tiles"] > 0 and info["dense_covered"] > 0
+    assert spmm_error(got, row, col, val, n, m, B.cpu()) <= REL_TOL
+    assert gemm_error(got, dense, B.cpu()) <= REL_TOL
+    G = torch.randn(n, f, generator=g).to(cuda)
+    gotT = A.spmm(G, transpose=True)
+    assert spmm_error(gotT, col, row, val, m, n, G.cpu()) <= REL_TOL
+    # duplicates: rows stay sorted, some pairs appear twice
+    rng = np.random.default_rng(9)
+    r = np.sort(rng.integers(0, 256, 40000))
+    c = rng.integers(0, 64, 40000)
+    order = np.lexsort((c, r))
+    r, c = torch.from_numpy(r[order]), torch.from_numpy(c[order])
+    v = torch.from_numpy(rng.standard_normal(40000).astype(np.float32))
+    try:
+        D = ops.CsrMatrix(_i32(r, cuda), _i32(c, cuda), v.to(cuda), 256, 64)
+    except Exception:
+        pytest.skip("handles refuse duplicate (row, column) pairs")
+    Bd = torch.randn(64, 300, generator=g).to(cuda)
+    got = D.spmm(Bd)
+    info = _panel_info(D)
+    assert info["state"] == 1 and info["dense_tiles"] == 0 and info["covered"] > 0
+    assert spmm_error(got, r, c, v, 256, 64, Bd.cpu()) <= REL_TOL
 
 
 def test_spmm_panel_plan_rectangular_strided_and_declined(cuda, tune):
