@@ -137,7 +137,7 @@ inline void PanelPlan::release() {
     rest = nullptr;
   }
   valid = declined = failed = false;
-  covered = dcovered = 0;
+  covered = dcovered = nrec = 0;
   ntiles = nunits = nsplit = ndtiles = ndunits = ndwg = nblocks = 0;
 }
 

@@ -58,7 +58,9 @@ struct PanelPlan {
   int32_t *dhdr = nullptr;         // [ndtiles * 32] row of B of every column of a dense tile
   float *dA = nullptr;             // [ndtiles * 4096] dense tiles in the operand layout of the matrix instruction
   int32_t *hdr = nullptr;          // [ntiles * 16 * 4] per (tile, wave): two rows of B to stage, record range
-  uint2 *ent = nullptr;            // [covered] {column in block | slot << 8, value bits}, by (tile, wave, slot)
+  int64_t nrec = 0;                // records: the covered entries and the zeros that pad odd runs
+  uint2 *ent = nullptr;            // [nrec] {column in block | slot << 8, value bits}, by (tile, wave, slot); every
+                                   // (tile, wave, slot) run has an even number of records
   int32_t *dslot = nullptr;        // [rows] partial row of a row of A: block * 128 + position, or -1
   int32_t *split = nullptr;        // [2 * nsplit] (first block, blocks) of panels that have several units
   CsrSide *rest = nullptr;         // entries outside active tiles, same rows and columns
@@ -85,9 +87,43 @@ __device__ __forceinline__ void panel_copy4_at(uint32_t lds_addr, const float *b
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(byte_off), "s"(base) : "memory");
 }
 
+// Lanes with byte_off < limit copy 16 (4) bytes from base + byte_off to LDS at lds_addr + lane * 16 (4).
+__device__ __forceinline__ void panel_copy16_if(uint32_t lds_addr, const float *base, uint32_t byte_off, uint32_t limit) {
+  uint64_t saved;
+  asm volatile(
+      "s_mov_b64 %0, exec\n\t"
+      "v_cmp_gt_u32 vcc, %4, %2\n\t"
+      "s_and_b64 exec, exec, vcc\n\t"
+      "s_mov_b32 m0, %1\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %2, %3\n\t"
+      "s_mov_b64 exec, %0"
+      : "=&s"(saved)
+      : "s"(lds_addr), "v"(byte_off), "s"(base), "s"(limit)
+      : "vcc", "scc", "memory");  // s_and writes scc
+}
+__device__ __forceinline__ void panel_copy4_if(uint32_t lds_addr, const float *base, uint32_t byte_off, uint32_t limit) {
+  uint64_t saved;
+  asm volatile(
+      "s_mov_b64 %0, exec\n\t"
+      "v_cmp_gt_u32 vcc, %4, %2\n\t"
+      "s_and_b64 exec, exec, vcc\n\t"
+      "s_mov_b32 m0, %1\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dword %2, %3\n\t"
+      "s_mov_b64 exec, %0"
+      : "=&s"(saved)
+      : "s"(lds_addr), "v"(byte_off), "s"(base), "s"(limit)
+      : "vcc", "scc", "memory");  // s_and writes scc
+}
+
 // hdr[(tile * 16 + wave) * 4 ..]: the two rows of B the wave stages for the tile and the range of its records.
 // It is read two tiles ahead and the records one tile ahead, so that no load of a tile depends on another
 // load of the same tile: the copies of the next tile go out as soon as the barrier has been passed.
+//
+// A wave walks its records of a tile two at a time and has the row of B of the record behind the current one on
+// its way from LDS while the current one is multiplied: a record costs 2408 bytes of LDS reads (f = 602)
+// whose latency four waves per SIMD do not hide by themselves.
 template <int CHUNKS>
 __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
     const int32_t *__restrict__ unit_tile, const int32_t *__restrict__ unit_order, const int32_t *__restrict__ unit_block,
@@ -109,28 +145,26 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
 #pragma unroll
     for (int ch = 0; ch < CHUNKS; ++ch) acc[s][ch] = make_float2(0.f, 0.f);
 
-  const int nq = f >> 2;     // whole 16-byte pieces of a row of B
-  const int tail0 = nq * 4;  // first float of the 4-byte pieces behind them
   // A wave stages two rows of B per tile, in pieces of one copy instruction each: per row nx4 of 64 x 16
-  // bytes and, for widths that are not a multiple of 4, one of 4-byte pieces (at most 8 pieces for the
-  // widths this kernel is built for).  One copy instruction keeps the CU's vector memory path busy for 16
-  // cycles, and a wave that issues its copies back to back sits behind those of the 15 other waves: the
-  // pieces of the next tile are therefore issued one at a time, between the slot runs of this tile.
+  // bytes and, for widths that are not a multiple of 4, one of 4-byte pieces.  One copy instruction keeps the
+  // CU's vector memory path busy for 16 cycles, and a wave that issues its copies back to back sits behind
+  // those of the 15 other waves: the pieces of the next tile are therefore issued one at a time, between the
+  // records of this tile.
+  const int nq = f >> 2;
+  const uint32_t lim16 = (uint32_t)nq * 16u, lim4 = (uint32_t)f * 4u;
   const int nx4 = (nq + kWave - 1) / kWave;
-  const int ppr = nx4 + (f > tail0 ? 1 : 0);
+  const int ppr = nx4 + (f > nq * 4 ? 1 : 0);
   const int npieces = RPW * ppr;
+  const uint32_t tail_off = lim16 + (uint32_t)lane * 4u;
   auto stage_piece = [&](int pc, const float *srca, const float *srcb, int buf) {
     const bool second = pc >= ppr;
     const int j = second ? pc - ppr : pc;
     const float *src = second ? srcb : srca;
     const uint32_t dst = (uint32_t)(uintptr_t)(panel_lds + buf * bufsz + (wave + (second ? kPanelWaves : 0)) * rs);
-    if (j < nx4) {
-      const int p = j * kWave + lane;
-      if (p < nq) panel_copy16(dst + j * (kWave * 16), src + 4 * p);
-    } else {
-      const int c = tail0 + lane;
-      if (c < f) panel_copy4(dst + tail0 * 4, src + c);
-    }
+    if (j < nx4)
+      panel_copy16_if(dst + j * (kWave * 16), src, (uint32_t)(j * kWave + lane) * 16u, lim16);
+    else
+      panel_copy4_if(dst + lim16, src, tail_off, lim4);
   };
   // lanes 0..3 of a wave fetch the four words of its header (a vector load: its wait is the one at the
   // end of the tile, with the copies, not the LDS counter)
@@ -170,10 +204,20 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
     const float *srca = B + (int64_t)q0 * ldb, *srcb = B + (int64_t)q1 * ldb;
     int piece = 0;
 
-    // records are sorted by slot: the lanes' ballots give the length of every slot's run, and a run
-    // adds into that slot's registers (static register indices)
+    // cnt >= 2 records in the lanes of r, sorted by slot, every slot's run of even length (the plan pads odd
+    // runs with a record of value 0): the lanes' ballots give the length of every slot's run, and a run adds
+    // into that slot's registers (static register indices), two records per step.  While a record is
+    // multiplied the row of B of the record behind it (whatever its slot) is on its way from LDS into the
+    // other of two sets of registers.
     auto process = [&](const uint2 r, int cnt) {
+      float2 ba[CHUNKS], bb[CHUNKS];
       const uint32_t myslot = (r.x >> 8) & 0x7u;
+      auto row_read = [&](int idx, float2 (&b)[CHUNKS]) {
+        const char *src = lbase + (__builtin_amdgcn_readlane(r.x, idx) & 0xffu) * rs;
+#pragma unroll
+        for (int ch = 0; ch < CHUNKS; ++ch) b[ch] = *reinterpret_cast<const float2 *>(src + ch * 512);
+      };
+      row_read(0, ba);
       int i = 0;
 #pragma unroll
       for (int s = 0; s < kPanelSlots; ++s) {
@@ -181,42 +225,24 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
           stage_piece(piece, srca, srcb, buf ^ 1);
           ++piece;
         }
-        const int c = __builtin_popcountll(__ballot(lane < cnt && myslot == (uint32_t)s));
-        const int end = i + c;
-        for (; i + 1 < end; i += 2) {  // two rows of B in flight
-          const uint32_t x0 = __builtin_amdgcn_readlane(r.x, i), x1 = __builtin_amdgcn_readlane(r.x, i + 1);
+        const int end = i + __builtin_popcountll(__ballot(lane < cnt && myslot == (uint32_t)s));
+        for (; i < end; i += 2) {
           const float v0 = __uint_as_float(__builtin_amdgcn_readlane(r.y, i));
           const float v1 = __uint_as_float(__builtin_amdgcn_readlane(r.y, i + 1));
-          const char *src0 = lbase + (x0 & 0xffu) * rs, *src1 = lbase + (x1 & 0xffu) * rs;
-          float2 b0[CHUNKS], b1[CHUNKS];
-#pragma unroll
-          for (int ch = 0; ch < CHUNKS; ++ch) b0[ch] = *reinterpret_cast<const float2 *>(src0 + ch * 512);
-#pragma unroll
-          for (int ch = 0; ch < CHUNKS; ++ch) b1[ch] = *reinterpret_cast<const float2 *>(src1 + ch * 512);
+          row_read(i + 1, bb);
+          __builtin_amdgcn_sched_barrier(0);  // the reads stay ahead of the multiplies they overlap with
 #pragma unroll
           for (int ch = 0; ch < CHUNKS; ++ch) {
-            acc[s][ch].x = fmaf(v0, b0[ch].x, acc[s][ch].x);
-            acc[s][ch].y = fmaf(v0, b0[ch].y, acc[s][ch].y);
+            acc[s][ch].x = fmaf(v0, ba[ch].x, acc[s][ch].x);
+            acc[s][ch].y = fmaf(v0, ba[ch].y, acc[s][ch].y);
           }
+          row_read(i + 2 < cnt ? i + 2 : i + 1, ba);  // the last pair reads its second row again
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int ch = 0; ch < CHUNKS; ++ch) {
-            acc[s][ch].x = fmaf(v1, b1[ch].x, acc[s][ch].x);
-            acc[s][ch].y = fmaf(v1, b1[ch].y, acc[s][ch].y);
+            acc[s][ch].x = fmaf(v1, bb[ch].x, acc[s][ch].x);
+            acc[s][ch].y = fmaf(v1, bb[ch].y, acc[s][ch].y);
           }
-        }
-        if (i < end) {
-          const uint32_t x = __builtin_amdgcn_readlane(r.x, i);
-          const float v = __uint_as_float(__builtin_amdgcn_readlane(r.y, i));
-          const char *src = lbase + (x & 0xffu) * rs;
-          float2 b[CHUNKS];
-#pragma unroll
-          for (int ch = 0; ch < CHUNKS; ++ch) b[ch] = *reinterpret_cast<const float2 *>(src + ch * 512);
-#pragma unroll
-          for (int ch = 0; ch < CHUNKS; ++ch) {
-            acc[s][ch].x = fmaf(v, b[ch].x, acc[s][ch].x);
-            acc[s][ch].y = fmaf(v, b[ch].y, acc[s][ch].y);
-          }
-          ++i;
         }
       }
     };
@@ -229,7 +255,7 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
       process(cur, left > kWave ? kWave : left);
       cur = nxt;
     }
-    for (; piece < npieces; ++piece) stage_piece(piece, srca, srcb, buf ^ 1);  // a wave without records in this tile
+    for (; piece < npieces; ++piece) stage_piece(piece, srca, srcb, buf ^ 1);  // a wave with few records in this tile
     rec = recn;
     e0 = e0n;
     e1 = e1n;
@@ -272,36 +298,6 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
 // to register between the instructions (and spill).  The copies of the next tile are therefore predicated
 // inside their asm statement (exec is narrowed to the lanes that have a piece and put back).
 typedef float panel_f4 __attribute__((ext_vector_type(4)));
-
-// Lanes with byte_off < limit copy 16 (4) bytes from base + byte_off to LDS at lds_addr + lane * 16 (4).
-__device__ __forceinline__ void panel_copy16_if(uint32_t lds_addr, const float *base, uint32_t byte_off, uint32_t limit) {
-  uint64_t saved;
-  asm volatile(
-      "s_mov_b64 %0, exec\n\t"
-      "v_cmp_gt_u32 vcc, %4, %2\n\t"
-      "s_and_b64 exec, exec, vcc\n\t"
-      "s_mov_b32 m0, %1\n\t"
-      "s_nop 0\n\t"
-      "global_load_lds_dwordx4 %2, %3\n\t"
-      "s_mov_b64 exec, %0"
-      : "=&s"(saved)
-      : "s"(lds_addr), "v"(byte_off), "s"(base), "s"(limit)
-      : "vcc", "scc", "memory");  // s_and writes scc
-}
-__device__ __forceinline__ void panel_copy4_if(uint32_t lds_addr, const float *base, uint32_t byte_off, uint32_t limit) {
-  uint64_t saved;
-  asm volatile(
-      "s_mov_b64 %0, exec\n\t"
-      "v_cmp_gt_u32 vcc, %4, %2\n\t"
-      "s_and_b64 exec, exec, vcc\n\t"
-      "s_mov_b32 m0, %1\n\t"
-      "s_nop 0\n\t"
-      "global_load_lds_dword %2, %3\n\t"
-      "s_mov_b64 exec, %0"
-      : "=&s"(saved)
-      : "s"(lds_addr), "v"(byte_off), "s"(base), "s"(limit)
-      : "vcc", "scc", "memory");  // s_and writes scc
-}
 
 template <int NG>  // groups of 64 result columns: ceil(f / 64)
 __global__ __launch_bounds__(kDenseThreads) void spmm_panel_dense_kernel(
@@ -585,6 +581,60 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_entry_finish_kernel(
     rest_col[k - covered] = colind[p];
     rest_val[k - covered] = val[p];
   }
+}
+
+// Runs of records = maximal stretches of equal (key, slot) in the sorted order.  The product kernel takes the
+// records of a run two at a time, so a run of odd length gets one more record behind its last one: the same
+// column and slot with the value +0 (which adds nothing as long as that row of B is finite).
+__global__ __launch_bounds__(kSpmmThreads) void panel_run_start_kernel(const int32_t *__restrict__ key,
+                                                                        const int32_t *__restrict__ slot, int64_t count,
+                                                                        uint32_t *__restrict__ start) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k > count) return;
+  start[k] = k < count && (k == 0 || key[k] != key[k - 1] || slot[k] != slot[k - 1]) ? 1u : 0u;  // entry `count`: slot of the scan's total
+}
+
+// run_first[run] = first record of the run; runs_before[k] is the exclusive scan of start[]
+__global__ __launch_bounds__(kSpmmThreads) void panel_run_first_kernel(const uint32_t *__restrict__ start,
+                                                                        const uint32_t *__restrict__ runs_before,
+                                                                        int64_t count, uint32_t *__restrict__ run_first) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k < count && start[k]) run_first[runs_before[k]] = (uint32_t)k;
+}
+
+// pad[k] = 1 when record k is the last of a run of odd length (entry `count` is the slot of the scan's total)
+__global__ __launch_bounds__(kSpmmThreads) void panel_run_pad_kernel(const uint32_t *__restrict__ start,
+                                                                      const uint32_t *__restrict__ runs_before,
+                                                                      const uint32_t *__restrict__ run_first, int64_t count,
+                                                                      uint32_t *__restrict__ pad) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k > count) return;
+  uint32_t p = 0;
+  if (k < count && (k + 1 == count || start[k + 1])) {
+    const uint32_t run = runs_before[k] + start[k] - 1u;  // runs_before counts the starts ahead of k
+    p = ((uint32_t)k - run_first[run] + 1u) & 1u;
+  }
+  pad[k] = p;
+}
+
+// shift[k] = exclusive scan of pad[]: record k moves to k + shift[k], its padding record (if any) behind it
+__global__ __launch_bounds__(kSpmmThreads) void panel_pad_write_kernel(const uint2 *__restrict__ in,
+                                                                        const uint32_t *__restrict__ pad,
+                                                                        const uint32_t *__restrict__ shift, int64_t count,
+                                                                        uint2 *__restrict__ out) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k >= count) return;
+  const uint2 r = in[k];
+  const int64_t at = k + shift[k];
+  out[at] = r;
+  if (pad[k]) out[at + 1] = make_uint2(r.x, 0u);
+}
+
+// wptr[j] += shift[wptr[j]] (shift[count] = all padding records)
+__global__ __launch_bounds__(kSpmmThreads) void panel_pad_wptr_kernel(int32_t *__restrict__ wptr, int64_t entries,
+                                                                       const uint32_t *__restrict__ shift) {
+  const int64_t j = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (j < entries) wptr[j] += (int32_t)shift[wptr[j]];
 }
 
 // hdr[(t * 16 + w) * 4 ..] = {row of B of column w of the tile's block, the same of column w + 16, first record, end}

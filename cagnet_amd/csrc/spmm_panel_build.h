@@ -47,8 +47,8 @@ static int alloc_sort_buffers(DevTemps &tmp, SortBuffers &buf, int64_t count) {
   return CG_OK;
 }
 
-constexpr int32_t kPanelDefaultDmin = 2048;            // entries from which a 128 x 32 tile is stored whole and multiplied
-                                                       // on the matrix cores (half full); negative tuning value: never
+constexpr int32_t kPanelDefaultDmin = 1024;            // entries from which a 128 x 32 tile is stored whole and multiplied
+                                                       // on the matrix cores (a quarter full); negative tuning value: never
 
 // may_decline: leave the plan empty (pp.declined) when the tiles hold too few of the entries.
 // *collision: two entries of one (row, column) pair fell into a dense tile; the plan is unusable.
@@ -182,7 +182,6 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   CG_TRY(dev_alloc((void **)&rest.rowptr, (size_t)(n + 1) * 4));
   CG_TRY(dev_alloc((void **)&rest.colind, (size_t)nrest * 4));
   CG_TRY(dev_alloc((void **)&rest.val, (size_t)nrest * 4));
-  CG_TRY(dev_alloc((void **)&pp.ent, (size_t)covered * 8));
   CG_TRY(tmp.alloc((void **)&tile_wptr, (size_t)(ntiles * kPanelWaves + 1) * 4));
   CG_TRY(dev_alloc((void **)&pp.hdr, (size_t)ntiles * kPanelWaves * 16));
   {
@@ -199,13 +198,46 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     CG_LAUNCH_CHECK();
     int set = 0;
     CG_TRY(radix_sort_pairs(buf, nnz, bits_for(sentinel + 2), bits_for(kPanelSlots), &set, stream));
+    uint2 *ent_raw = nullptr;  // the records before padding
+    CG_TRY(t2.alloc((void **)&ent_raw, (size_t)(covered > 0 ? covered : 1) * 8));
     if (covered + nrest > 0) {
       panel_entry_finish_kernel<<<(unsigned)ceil_div64(covered + nrest, kSpmmThreads), kSpmmThreads, 0, stream>>>(
-          buf.key_b[set], buf.payload[set], covered + nrest, covered, erow, s.colind, s.val, col_rank, pp.ent, rest_row,
+          buf.key_b[set], buf.payload[set], covered + nrest, covered, erow, s.colind, s.val, col_rank, ent_raw, rest_row,
           rest.colind, rest.val);
       CG_LAUNCH_CHECK();
     }
     CG_TRY(launch_rowptr(buf.key_a[set], covered, sentinel, tile_wptr, stream));
+    // runs of odd length get a padding record
+    {
+      uint32_t *start = nullptr, *runs_before = nullptr, *run_first = nullptr, *padf = nullptr, *shift = nullptr;
+      CG_TRY(t2.alloc((void **)&start, (size_t)(covered + 1) * 4));
+      CG_TRY(t2.alloc((void **)&runs_before, (size_t)(covered + 1) * 4));
+      CG_TRY(t2.alloc((void **)&run_first, (size_t)(covered + 1) * 4));
+      CG_TRY(t2.alloc((void **)&padf, (size_t)(covered + 1) * 4));
+      CG_TRY(t2.alloc((void **)&shift, (size_t)(covered + 1) * 4));
+      const unsigned gc = (unsigned)ceil_div64(covered + 1, kSpmmThreads);
+      panel_run_start_kernel<<<gc, kSpmmThreads, 0, stream>>>(buf.key_a[set], buf.key_b[set], covered, start);
+      CG_LAUNCH_CHECK();
+      CG_TRY(exclusive_scan_u32(start, runs_before, covered + 1, nullptr, stream));
+      panel_run_first_kernel<<<gc, kSpmmThreads, 0, stream>>>(start, runs_before, covered, run_first);
+      CG_LAUNCH_CHECK();
+      panel_run_pad_kernel<<<gc, kSpmmThreads, 0, stream>>>(start, runs_before, run_first, covered, padf);
+      CG_LAUNCH_CHECK();
+      CG_TRY(exclusive_scan_u32(padf, shift, covered + 1, d_tot + 0, stream));
+      uint32_t npad = 0;
+      CG_HIP(hipMemcpyAsync(&npad, d_tot + 0, 4, hipMemcpyDeviceToHost, stream));
+      CG_HIP(hipStreamSynchronize(stream));
+      if (covered + (int64_t)npad > 0x7fffffffLL) CG_FAIL(CG_ERR_OVERFLOW, "panel plan: records exceed the int32 range");
+      pp.nrec = covered + npad;
+      CG_TRY(dev_alloc((void **)&pp.ent, (size_t)pp.nrec * 8));
+      if (covered > 0) {
+        panel_pad_write_kernel<<<gc, kSpmmThreads, 0, stream>>>(ent_raw, padf, shift, covered, pp.ent);
+        CG_LAUNCH_CHECK();
+      }
+      panel_pad_wptr_kernel<<<(unsigned)ceil_div64(ntiles * kPanelWaves + 1, kSpmmThreads), kSpmmThreads, 0, stream>>>(
+          tile_wptr, ntiles * kPanelWaves + 1, shift);
+      CG_LAUNCH_CHECK();
+    }
     if (ntiles > 0) {
       panel_hdr_kernel<<<(unsigned)ceil_div64(ntiles * kPanelWaves, kSpmmThreads), kSpmmThreads, 0, stream>>>(
           tile_kb, tile_wptr, qcol, ntiles, (int4 *)pp.hdr);
@@ -394,7 +426,7 @@ static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_
   const int chunks = (f / 2 + kWave - 1) / kWave;
   const int groups = (f + 63) / 64;
   const size_t rs = ((size_t)f * 4 + 15) & ~(size_t)15;
-  const size_t lds = 2 * (size_t)kPanelCols * rs;
+  const size_t lds = 2 * (size_t)kPanelCols * rs;  // two tiles of staged rows
   const size_t lds_max = 2 * (size_t)kPanelCols * ((kPanelMaxF * 4 + 15) & ~15);
   void *p = nullptr;
   CG_TRY(scratch_get(stream, kSlotE, (size_t)pp.nblocks * kPanelRows * f * sizeof(float), &p));

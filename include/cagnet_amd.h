@@ -328,7 +328,8 @@ int cg_coo_block(const int32_t *d_row, const int32_t *d_col, const float *d_val,
  * of classes of a row-wise kernel.  Names: "spmm_rowseg" (the main kernel of a
  * product, or the cold class of a hub plan), "spmm_hub_hot" (all hot tiers of a hub plan as one
  * record), "spmm_reduce" (rows split into segments), "spmm_hub_reduce" (partial rows of a hub plan
- * with narrow teams), "dense_xw", "dense_gwt", "dense_xtg" (partial products and their sum),
+ * with narrow teams), "spmm_panel" (staged tiles of a panel plan and the sum of a panel's blocks of
+ * partial rows), "spmm_panel_dense" (its dense tiles on the matrix cores), "dense_xw", "dense_gwt", "dense_xtg" (partial products and their sum),
  * "relu_fwd", "relu_bwd" (no suffix), "log_softmax_fwd", "log_softmax_bwd", "nll_fwd", "nll_bwd",
  * "log_softmax_nll_bwd".
  * Recording is off by default and costs nothing then.
@@ -351,7 +352,7 @@ int cg_prof_enable(int on);
  *   "spmm_panel_cols" ranked columns that can be part of a tile (0: 131072)
  *   "spmm_panel_unit" entries after which the tiles of a row panel go to another workgroup (0: 65536)
  *   "spmm_panel_dmin" entries from which a 128 x 32 tile is stored whole and multiplied on the fp32 matrix
- *                     cores (0: 2048, half full; negative: never).  Such a tile multiplies its zeros too:
+ *                     cores (0: 1024, a quarter full; negative: never).  Such a tile multiplies its zeros too:
  *                     a row of B with an infinity or a NaN then reaches all 128 rows of the tile
  *   "spmm_panel_dwg"  workgroups that share the dense tiles equally (0: four per compute unit)
  *   "dense_mfma"      -1: dense products on the vector ALU tile kernel only
