@@ -268,7 +268,21 @@ def dominant_product(kernels: dict, f_in: int):
     return parts, (sum(parts.values()) if parts else float("nan"))
 
 
-def extra_rmat20(dev, reps: int) -> dict:
+def launched_spmm_kernels(fn, f: int) -> set:
+    """Profiling names of the SpMM kernels one call of fn launches at width f."""
+    import torch
+
+    from cagnet_amd import _lib
+
+    torch.cuda.synchronize()
+    _lib.lib.cg_prof_enable(1)
+    fn()
+    torch.cuda.synchronize()
+    _lib.lib.cg_prof_enable(0)
+    return {k for k in SPMM_KERNELS if prof_read(_lib.lib, f"{k}/f={f}")[1]}
+
+
+def extra_rmat20(dev, reps: int, traffic_table: dict) -> dict:
     """Configuration 2: R-MAT scale 20, A H and A^T G at f in {16, 64, 128, 602}, and the build times."""
     import torch
 
@@ -306,7 +320,9 @@ def extra_rmat20(dev, reps: int) -> dict:
         alg = spmm_alg_bytes(nnz, n, n, f, reads_c=False)
         for name, tr in (("A@H", False), ("A^T@G", True)):
             ms = median_ms(lambda: A.spmm(B, out=C, beta=0.0, transpose=tr), reps)
-            products.append(dict(product=name, f=f, **roofline_fields(alg, 2.0 * nnz * f, ms)))
+            launched = launched_spmm_kernels(lambda: A.spmm(B, out=C, beta=0.0, transpose=tr), f)
+            products.append(dict(product=name, f=f, kernels="+".join(sorted(launched)),
+                                 **roofline_fields(alg, 2.0 * nnz * f, ms, traffic_of(traffic_table, "rmat20", f, launched))))
         del B, C
     return {"workload": "R-MAT scale 20 (1,048,576 vertices, 16,777,216 directed edges), symmetrised, self-loops, "
                         "GCN-normalised; median of %d" % reps,
@@ -579,7 +595,7 @@ def main() -> int:
     del rec, x, Data, blk, prob
     torch.cuda.empty_cache()
     if extras:
-        out["configs"]["cfg2_rmat20"] = extra_rmat20(dev, 5)
+        out["configs"]["cfg2_rmat20"] = extra_rmat20(dev, 5, traffic_table)
         torch.cuda.empty_cache()
         out["configs"]["cfg5_amazon"] = extra_amazon(dev, traffic_table, 5)
     if prob_cpu is not None:
