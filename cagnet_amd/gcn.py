@@ -43,6 +43,39 @@ fused_forward = True
 fused_forward_max_row_entries = 64
 
 
+# A wide dense operand whose rows are not a whole number of 128-byte lines long (602 floats = 2408 bytes) is read by the
+# SpMM kernels through rows that start at every alignment and span 20 lines instead of 19: measured at the Reddit shape,
+# the f = 602 product takes 12.3 ms on X as it is, 12.2 ms with the rows 604 floats apart and 11.9 ms with 608 or 640
+# (0.25 ms to make the copy).  The features are the same tensor in every epoch, so the copy is kept for as long as the
+# tensor is unchanged.  Tensors beyond 2 GiB are left alone (the copy would double them).
+aligned_operands = True
+_ALIGNED_MIN_COLS = 64
+_ALIGNED_MAX_BYTES = 2 << 30
+_aligned_cache: List[tuple] = []   # (weakref to the tensor, its version, the copy's column slice); newest last, at most 2
+
+
+def _aligned_rows(t: torch.Tensor) -> torch.Tensor:
+    """t, or a copy of t with the rows a multiple of 128 bytes apart when that pays (see `aligned_operands`)."""
+    import weakref
+
+    if (not aligned_operands or t.dim() != 2 or t.dtype != torch.float32 or not t.is_cuda or t.shape[1] < _ALIGNED_MIN_COLS
+            or t.stride(1) != 1 or t.stride(0) % 32 == 0 or t.shape[0] == 0 or t.numel() * 4 > _ALIGNED_MAX_BYTES):
+        return t
+    if torch.cuda.is_current_stream_capturing():
+        return t  # a captured graph must keep reading the caller's tensor, whose contents may change between replays
+    for ref, version, copy in _aligned_cache:
+        if ref() is t and version == t._version:
+            return copy
+    _aligned_cache[:] = [e for e in _aligned_cache if e[0]() is not None and e[0]() is not t][-1:]
+    ld = (t.shape[1] + 31) // 32 * 32
+    with torch.no_grad():
+        wide = torch.empty(t.shape[0], ld, dtype=t.dtype, device=t.device)
+        wide[:, :t.shape[1]].copy_(t)
+    copy = wide[:, :t.shape[1]]
+    _aligned_cache.append((weakref.ref(t), t._version, copy))
+    return copy
+
+
 class ResidentBlocks:
     """Stands where the reference passes a process group: the dense blocks that its broadcasts
     would deliver (gcn_distr.py:230), already resident in HBM.  `forward[i]` is the H block and
@@ -78,7 +111,7 @@ def broad_func(node_count: int, am_partitions: Sequence[CsrMatrix], inputs: torc
         raise ValueError(f"{len(am_partitions)} sparse blocks for size {size}")
     z_loc = None
     for i in range(size):
-        h_i = _stage_operand(i, rank, inputs, group)
+        h_i = _aligned_rows(_stage_operand(i, rank, inputs, group))
         blk = am_partitions[i]
         if z_loc is None:
             z_loc = blk.spmm(h_i, transpose=transpose) if out is None else blk.spmm(h_i, out=out, beta=0.0,
@@ -176,7 +209,7 @@ class GCNFunc(torch.autograd.Function):
             if fused_forward and short_rows and weight.shape[1] <= 64 and inputs.shape[1] >= 128:
                 # stages 0 .. size-2 accumulate as usual, the last one also applies W (and ReLU)
                 z = broad_func(node_count, am_partitions[:-1], inputs, rank, size - 1, peers_fwd) if size > 1 else None
-                h_last = _stage_operand(size - 1, rank, inputs, peers_fwd)
+                h_last = _aligned_rows(_stage_operand(size - 1, rank, inputs, peers_fwd))
                 out = am_partitions[size - 1].spmm_xw(h_last, weight, relu=(kind == "relu"), acc=z)
                 if out is None and z is not None:      # no fused form for this width: finish the stage loop
                     am_partitions[size - 1].spmm(h_last, out=z, beta=1.0)

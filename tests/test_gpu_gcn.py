@@ -378,3 +378,32 @@ def test_single_process_harness_prints_golden_losses(cuda):
     assert float(np.abs(np.array(losses) - want).max()) <= 1e-4
     rec = __import__("json").loads(proc.stdout.strip().splitlines()[-1])
     assert rec["config"]["workload"].startswith("R-MAT scale 12") and rec["steps"] == 100
+
+
+def test_row_aligned_copy_of_a_wide_operand(cuda):
+    """The stage loop multiplies a wide operand whose rows are not a multiple of 128 bytes long (602 floats) through a
+    copy with rows 608 floats apart: same bits as on the tensor itself, the copy is reused while the tensor is
+    unchanged and made again after an in-place change; widths that are aligned already are used as they are."""
+    from cagnet_amd import gcn, ops
+    from tests.util import small_graph
+    row, col, val, n = small_graph(10, 20000, seed=5)
+    A = ops.CsrMatrix(row.int().to(cuda), col.int().to(cuda), val.to(cuda), n, n)
+    x = torch.randn(n, 602, device=cuda)
+    c1 = gcn._aligned_rows(x)
+    assert c1.data_ptr() != x.data_ptr() and c1.stride(0) == 608 and torch.equal(c1, x)
+    assert gcn._aligned_rows(x) is c1                                 # cached
+    direct = A.spmm(x)
+    assert torch.equal(gcn.broad_func(n, [A], x, 0, 1), direct)       # goes through the copy: same bits
+    x.mul_(2.0)                                                       # in-place change: the copy is stale
+    c2 = gcn._aligned_rows(x)
+    assert c2 is not c1 and torch.equal(c2, x)
+    assert torch.equal(gcn.broad_func(n, [A], x, 0, 1), A.spmm(x))
+    y = torch.randn(n, 640, device=cuda)
+    assert gcn._aligned_rows(y) is y
+    z = torch.randn(n, 41, device=cuda)
+    assert gcn._aligned_rows(z) is z                                  # narrow: not worth a copy
+    gcn.aligned_operands = False
+    try:
+        assert gcn._aligned_rows(x) is x
+    finally:
+        gcn.aligned_operands = True
