@@ -77,6 +77,9 @@ def _out_rowmajor(t: torch.Tensor, name: str) -> int:
     rows, cols = t.shape
     if (cols > 1 and t.stride(1) != 1) or (rows > 1 and t.stride(0) < cols):
         raise ValueError(f"{name}: output must be row-major with unit column stride (strides {t.stride()})")
+    # the library is about to write into t behind torch's back: say so, for everything that goes by a tensor's
+    # version (autograd's saved tensors, the copies aligned_rows keeps)
+    torch.autograd.graph.increment_version(t)
     return max(t.stride(0) if rows > 1 else cols, cols, 1)
 
 
@@ -551,3 +554,36 @@ def log_softmax_nll_bwd(logp: torch.Tensor, y: torch.Tensor, mask: Optional[torc
                                      c_void_p(gs.data_ptr()) if gs is not None else c_void_p(0), _ptr(dz), max(c, 1),
                                      n, c, _stream()), "cg_log_softmax_nll_bwd")
     return dz
+
+
+# A wide dense operand whose rows are not a whole number of 128-byte lines long (602 floats = 2408 bytes) is read by the
+# SpMM kernels through rows that start at every alignment and span 20 lines instead of 19: measured at the Reddit shape,
+# the f = 602 product takes 12.3 ms on X as it is, 12.2 ms with the rows 604 floats apart and 11.9 ms with 608 or 640
+# (0.25 ms to make the copy).  The features are the same tensor in every epoch, so the copy is kept for as long as the
+# tensor is unchanged.  Tensors beyond 2 GiB are left alone (the copy would double them).
+aligned_operands = True
+_ALIGNED_MIN_COLS = 64
+_ALIGNED_MAX_BYTES = 2 << 30
+_aligned_cache: list = []   # (weakref to the tensor, its version, the copy's column slice); newest last, at most 2
+
+
+def aligned_rows(t: torch.Tensor) -> torch.Tensor:
+    """t, or a copy of t with the rows a multiple of 128 bytes apart when that pays (see `aligned_operands`)."""
+    import weakref
+
+    if (not aligned_operands or t.dim() != 2 or t.dtype != torch.float32 or not t.is_cuda or t.shape[1] < _ALIGNED_MIN_COLS
+            or t.stride(1) != 1 or t.stride(0) % 32 == 0 or t.shape[0] == 0 or t.numel() * 4 > _ALIGNED_MAX_BYTES):
+        return t
+    if torch.cuda.is_current_stream_capturing():
+        return t  # a captured graph must keep reading the caller's tensor, whose contents may change between replays
+    for ref, version, copy in _aligned_cache:
+        if ref() is t and version == t._version:
+            return copy
+    _aligned_cache[:] = [e for e in _aligned_cache if e[0]() is not None and e[0]() is not t][-1:]
+    ld = (t.shape[1] + 31) // 32 * 32
+    with torch.no_grad():
+        wide = torch.empty(t.shape[0], ld, dtype=t.dtype, device=t.device)
+        wide[:, :t.shape[1]].copy_(t)
+    copy = wide[:, :t.shape[1]]
+    _aligned_cache.append((weakref.ref(t), t._version, copy))
+    return copy

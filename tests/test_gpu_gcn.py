@@ -398,12 +398,15 @@ def test_row_aligned_copy_of_a_wide_operand(cuda):
     c2 = gcn._aligned_rows(x)
     assert c2 is not c1 and torch.equal(c2, x)
     assert torch.equal(gcn.broad_func(n, [A], x, 0, 1), A.spmm(x))
+    A.spmm(torch.randn(n, 602, device=cuda), out=x)                   # written by the library: counts as a change
+    c3 = gcn._aligned_rows(x)
+    assert c3 is not c2 and torch.equal(c3, x)
     y = torch.randn(n, 640, device=cuda)
     assert gcn._aligned_rows(y) is y
     z = torch.randn(n, 41, device=cuda)
     assert gcn._aligned_rows(z) is z                                  # narrow: not worth a copy
-    gcn.aligned_operands = False
+    ops.aligned_operands = False
     try:
         assert gcn._aligned_rows(x) is x
     finally:
-        gcn.aligned_operands = True
+        ops.aligned_operands = True
