@@ -398,6 +398,7 @@ __global__ __launch_bounds__(kDenseThreads) void spmm_panel_dense_kernel(
           if (ks + 1 < 8) b[g] = b_read(lb, ks + 1, g);
           // the next tile's copies, spread over this tile's steps
           if ((ks * NG + g) % 2 == 0 && (ks * NG + g) / 2 < NPIECES) stage_piece((ks * NG + g) / 2, src4, buf ^ 1);
+          __builtin_amdgcn_sched_barrier(0);  // keeps the read where it is: NG - 1 groups of instructions ahead of its use
         }
       }
       a_cur[0] = a_nxt[0];
