@@ -424,7 +424,7 @@ def main() -> int:
     ap.add_argument("--optimizer", default="adam", choices=("adam", "sgd"))
     ap.add_argument("--print-losses", action="store_true", help="print the loss of every timed epoch to stderr")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-budget", type=float, default=90.0, help="seconds of host time the CPU baseline may take")
+    ap.add_argument("--cpu-budget", type=float, default=180.0, help="seconds of host time the CPU baseline may take")
     ap.add_argument("--no-extra", action="store_true", help="skip the sub-records of the other configurations")
     ap.add_argument("--hip-graph", action="store_true",
                     help="also time the epoch captured into a HIP graph and replayed (always done for --workload tiny)")

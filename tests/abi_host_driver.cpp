@@ -176,13 +176,15 @@ static void with_gpu() {
   EXPECT(cg_csr_create(&h, d_row, d_col, d_val, nnz, n, m, CG_CSR_SORTED | CG_CSR_TRANSPOSE | CG_CSR_VALIDATE, stream) == CG_OK);
   int64_t info[12] = {0};
   EXPECT(cg_csr_info(h, info) == CG_OK && info[0] == n && info[1] == m && info[2] == nnz);
-  for (int pass = 0; pass < 3; ++pass) {
+  for (int pass = 0; pass < 4; ++pass) {
     // pass 0: built-in choices; 1: hub plans forced (7 widths through 2 plan slots and 4 schedule slots);
-    // 2: panel plans forced as well, with small tiles
+    // 2: panel plans forced as well, with small tiles; 3: with dense tiles from 48 entries on, three workgroups
     EXPECT(cg_tune_set("spmm_hub", pass >= 1 ? 1 : 0) == CG_OK);
     EXPECT(cg_tune_set("spmm_hub_kb", pass >= 1 ? 64 : 0) == CG_OK);
-    EXPECT(cg_tune_set("spmm_panel", pass == 2 ? 1 : 0) == CG_OK);
-    EXPECT(cg_tune_set("spmm_panel_emin", pass == 2 ? 8 : 0) == CG_OK);
+    EXPECT(cg_tune_set("spmm_panel", pass >= 2 ? 1 : 0) == CG_OK);
+    EXPECT(cg_tune_set("spmm_panel_emin", pass >= 2 ? 8 : 0) == CG_OK);
+    EXPECT(cg_tune_set("spmm_panel_dmin", pass == 3 ? 48 : 0) == CG_OK);
+    EXPECT(cg_tune_set("spmm_panel_dwg", pass == 3 ? 3 : 0) == CG_OK);
     for (int f : widths) {
       Lcg g{(uint64_t)f * 31 + pass};
       std::vector<float> B((size_t)m * f), C((size_t)n * f, 0.f);
@@ -197,6 +199,7 @@ static void with_gpu() {
         ++g_fail;
       }
       EXPECT(cg_csr_panel_info(h, 0, info) == CG_OK);
+      if (pass == 3 && f >= 258) EXPECT(info[0] == 1 && info[9] > 0 && info[1] + info[8] + info[5] == nnz);
       HIP_OK(hipFree(d_B));
       HIP_OK(hipFree(d_C));
     }
@@ -247,7 +250,8 @@ static void with_gpu() {
     HIP_OK(hipFree(d_B));
     HIP_OK(hipFree(d_C));
   }
-  for (const char *k : {"spmm_hub", "spmm_hub_kb", "spmm_panel", "spmm_panel_emin"}) EXPECT(cg_tune_set(k, 0) == CG_OK);
+  for (const char *k : {"spmm_hub", "spmm_hub_kb", "spmm_panel", "spmm_panel_emin", "spmm_panel_dmin", "spmm_panel_dwg"})
+    EXPECT(cg_tune_set(k, 0) == CG_OK);
   int64_t released = -1;
   EXPECT(cg_csr_unpin(h, &released) == CG_OK && released == 0);  // nothing was captured: nothing was parked
   EXPECT(cg_csr_destroy(h) == CG_OK);
