@@ -90,6 +90,76 @@ def test_spmm_schedules_random(cuda, knobs_restored, seed):
     ops.coo_cache_clear()
 
 
+PANEL_KNOBS = [b"spmm_panel", b"spmm_panel_emin", b"spmm_panel_cols", b"spmm_panel_unit", b"spmm_panel_dmin", b"spmm_panel_dwg"]
+
+
+@pytest.mark.parametrize("seed", [31, 32])
+def test_spmm_panel_plan_random(cuda, knobs_restored, seed):
+    """The panel plan forced on over random patterns (skewed and uniform, with full rows and columns, rectangular),
+    every even width class it is built for, both sides, accumulate forms, padded leading dimensions, and random plan
+    knobs: entries a tile needs, ranked columns, unit size, dense-tile threshold (off, low, high) and the number of
+    workgroups that share the dense tiles.  Every entry is in exactly one of the three parts of the plan."""
+    import ctypes
+    from cagnet_amd import ops
+    from cagnet_amd._lib import check
+    lib = knobs_restored
+    rng = random.Random(seed)
+    try:
+        for case in range(150):
+            n = rng.choice([1, 64, 127, 128, 129, 300, 1000, 2500])
+            m = rng.choice([31, 32, 33, 64, 500, 1000, 3001])
+            g = torch.Generator().manual_seed(rng.randrange(1 << 30))
+            if rng.random() < 0.6:       # skewed: popular columns and heavy rows
+                pr = torch.rand(n, 1, generator=g) ** 3
+                pc = torch.rand(1, m, generator=g) ** 3
+                mask = torch.rand(n, m, generator=g) < (pr * pc * rng.choice([0.5, 2.0, 8.0])).clamp(max=1.0)
+            else:
+                mask = torch.rand(n, m, generator=g) < rng.choice([0.01, 0.1, 0.6, 1.0])
+            if rng.random() < 0.5 and n > 2:
+                mask[rng.randrange(n)] = True
+                mask[:, rng.randrange(m)] = True
+            dense = torch.where(mask, torch.randn(n, m, generator=g), torch.zeros(()))
+            idx = mask.nonzero()
+            if idx.shape[0] == 0:
+                continue
+            row, col, val = idx[:, 0].int().to(cuda), idx[:, 1].int().to(cuda), dense[mask].to(cuda)
+            f = rng.choice([258, 260, 300, 320, 322, 384, 448, 450, 512, 576, 602, 636])
+            values = [1, rng.choice([1, 4, 16, 64]), rng.choice([0, 32, 64, 1024]), rng.choice([0, 50, 2000]),
+                      rng.choice([-1, 0, 8, 40, 200, 3000]), rng.choice([0, 1, 5, 300])]
+            for key, v in zip(PANEL_KNOBS, values):
+                assert lib.cg_tune_set(key, v) == 0
+            tr = rng.random() < 0.4
+            beta = rng.choice([0.0, 1.0, -0.5])
+            extra_b, extra_c = rng.choice([0, 0, 2, 6]), rng.choice([0, 0, 2, 4])
+            what = f"seed {seed} case {case}: n={n} m={m} nnz={val.numel()} f={f} tr={tr} beta={beta} ld+{extra_b}/{extra_c} knobs={values}"
+            gen = torch.Generator(device=cuda).manual_seed(case)
+            B = _strided(n if tr else m, f, extra_b, gen, cuda)
+            C0 = torch.randn(m if tr else n, f, device=cuda, generator=gen)
+            A = ops.CsrMatrix(row, col, val, n, m, is_sorted=True, transpose=tr)
+            outs = []
+            for _ in range(2):
+                C = torch.empty(C0.shape[0], f + extra_c, device=cuda)[:, :f].copy_(C0)
+                A.spmm(B, out=C, beta=beta, transpose=tr)
+                outs.append(C)
+            info = (ctypes.c_int64 * 12)()
+            check(lib.cg_csr_panel_info(A._handle, int(tr), info), "cg_csr_panel_info")
+            assert info[0] in (1, -1), what                       # in use, or no tile reached the threshold
+            if info[0] == 1:
+                assert info[1] + info[8] + info[5] == val.numel(), what
+                if values[4] < 0:
+                    assert info[9] == 0, what
+            A64 = dense.double().to(cuda)
+            A64 = A64.t() if tr else A64
+            ref = beta * C0.double() + A64 @ B.double()
+            mag = abs(beta) * C0.double().abs() + A64.abs() @ B.double().abs()
+            assert _rel(outs[0], ref, mag) <= REL_TOL, what
+            assert torch.equal(outs[0], outs[1]), what
+            del A
+    finally:
+        for key in PANEL_KNOBS:
+            lib.cg_tune_set(key, 0)
+
+
 @pytest.mark.parametrize("seed", [21, 22])
 def test_dense_and_rowwise_random(cuda, knobs_restored, seed):
     """The three dense products (both kernel families) on strided operands and outputs, and the
