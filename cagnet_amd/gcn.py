@@ -48,6 +48,15 @@ fused_forward_max_row_entries = 64
 _aligned_rows = ops.aligned_rows
 
 
+# Backward of a layer that widens (16 -> 41 classes).  The reference multiplies A by the output-width gradient first,
+# AG = A G, and takes dH = AG W^T and dW = H^T AG from it (gcn_distr.py:326-337).  With this flag such a layer keeps
+# Z = A H from its forward pass and computes dW = Z^T G and dH = A^T (G W^T) instead: the same mathematics (for the
+# symmetric A the reference assumes, or with the block's stored transpose), with the SpMM at the input width (16)
+# instead of the output width (41, carried as 44); different rounding.  Single-block products only: with several
+# stages the per-rank partial sums of dW would differ from the reference's before their all-reduce.
+narrow_backward = True
+
+
 class ResidentBlocks:
     """Stands where the reference passes a process group: the dense blocks that its broadcasts
     would deliver (gcn_distr.py:230), already resident in HBM.  `forward[i]` is the H block and
@@ -174,6 +183,7 @@ class GCNFunc(torch.autograd.Function):
         kind = _kind(func) if activations else "none"
         node_count = adj_matrix if isinstance(adj_matrix, int) else adj_matrix.size(0)
         peers_fwd = group.forward if isinstance(group, ResidentBlocks) else None
+        z_kept = None
         if spmm_first or size != 1 or weight.shape[1] >= inputs.shape[1]:  # reordering only pays when the layer narrows
             out = None
             last = am_partitions[size - 1]
@@ -189,6 +199,8 @@ class GCNFunc(torch.autograd.Function):
             if out is None:
                 z = broad_func(node_count, am_partitions, inputs, rank, size, peers_fwd)
                 out = ops.dense_xw(z, weight, relu=(kind == "relu"))
+                if narrow_backward and size == 1 and _padded_width(weight.shape[1]) > inputs.shape[1]:
+                    z_kept = z
                 del z
         else:
             out = broad_func(node_count, am_partitions, ops.dense_xw(inputs, weight), rank, size, peers_fwd)
@@ -197,6 +209,7 @@ class GCNFunc(torch.autograd.Function):
         if kind == "log_softmax":
             out = ops.log_softmax_fwd(out)
         ctx.save_for_backward(inputs, weight, out)
+        ctx.z_kept = z_kept
         ctx.am_partitions = am_partitions
         ctx.rank, ctx.size, ctx.group, ctx.kind, ctx.node_count = rank, size, group, kind, node_count
         return out
@@ -212,6 +225,14 @@ class GCNFunc(torch.autograd.Function):
         peers_bwd = ctx.group.backward if isinstance(ctx.group, ResidentBlocks) else None
         blocks = ctx.am_partitions
         use_t = ctx.size == 1 and blocks[0].has_transpose
+        if ctx.z_kept is not None:  # the layer widens: SpMM at the input width (see narrow_backward)
+            grad_weight = ops.dense_xtg(ctx.z_kept, grad_output) if ctx.needs_input_grad[1] else None
+            grad_input = None
+            if ctx.needs_input_grad[0]:
+                dz = ops.dense_gwt(grad_output, weight)
+                grad_input = broad_func(ctx.node_count, blocks, dz, ctx.rank, ctx.size, peers_bwd, transpose=use_t)
+            ctx.z_kept = None
+            return grad_input, grad_weight, None, None, None, None, None, None
         width = grad_output.shape[1]
         padded = _padded_width(width)
         ag_out = None

@@ -30,14 +30,17 @@ def _close(got, ref64, what, tol=2e-4):
     assert err <= tol, f"{what}: {err}"
 
 
+@pytest.mark.parametrize("narrow", [True, False])
 @pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("transpose", [False, True])
-def test_forward_backward_matches_oracle(cuda, monkeypatch, transpose, fused):
+def test_forward_backward_matches_oracle(cuda, monkeypatch, transpose, fused, narrow):
     """Both forms of the layer product: SpMM with the W product folded in (rows are short here, so
-    the default takes it) and the reference's two separate kernels."""
+    the default takes it) and the reference's two separate kernels; and both orders of the backward
+    pass of the layer that widens (the reference's A G first, or dW = (A H)^T G and dH = A^T (G W^T))."""
     from cagnet_amd import gcn
     monkeypatch.setattr(gcn, "fused_forward", fused)
-    p = synth.make_problem(scale=11, n_edges=16384, features=128, hidden=16, classes=8, mask_fraction=0.66, seed=3)
+    monkeypatch.setattr(gcn, "narrow_backward", narrow)
+    p = synth.make_problem(scale=11, n_edges=16384, features=128, hidden=16, classes=24, mask_fraction=0.66, seed=3)
     assert p.row.numel() <= gcn.fused_forward_max_row_entries * p.n
     A = orc.coo_tensor(p.row, p.col, p.val, p.n, p.n, torch.float64)
     ref = orc.forward_backward(p.x, p.w1, p.w2, [A], p.y, p.train_mask, dtype=torch.float64)
@@ -322,12 +325,17 @@ def test_activations_off_is_the_plain_linear_model(cuda, monkeypatch):
     _close(x.grad, xr.grad, "dx")
 
 
+@pytest.mark.parametrize("narrow", [False, True])
 @pytest.mark.parametrize("classes,features,scale,edges", [(8, 128, 12, 32768), (41, 64, 11, 16384)])
-def test_adam_epochs_with_reference_init_match_oracle(cuda, classes, features, scale, edges):
+def test_adam_epochs_with_reference_init_match_oracle(cuda, monkeypatch, classes, features, scale, edges, narrow):
     """The reference's own set-up of a run (gcn_distr.py:550-562): torch.manual_seed(0), weights
     torch.rand(features, 16) and torch.rand(16, classes), Adam lr 0.01.  60 epochs of `train`: the loss of
     every epoch within 1e-4 of the fp32 CPU oracle and of its fp64 twin, and the weights after them."""
     from cagnet_amd import gcn
+    # narrow = False is the reference's order of the backward products; True the library's default, which takes the
+    # backward SpMM of the layer that widens (41 classes) at its input width: other rounding, which 60 Adam steps
+    # (each normalises the gradient) amplify a little more in the weights
+    monkeypatch.setattr(gcn, "narrow_backward", narrow)
     p = synth.make_problem(scale=scale, n_edges=edges, features=features, hidden=16, classes=classes,
                            mask_fraction=0.66, seed=0)
     torch.manual_seed(0)
@@ -352,8 +360,8 @@ def test_adam_epochs_with_reference_init_match_oracle(cuda, classes, features, s
     assert max(abs(a - b) for a, b in zip(losses, ref64)) <= LOSS_TOL
     assert max(abs(a - b) for a, b in zip(losses, ref32)) <= LOSS_TOL
     assert losses[-1] < losses[0]
-    _close(w1, w1_64, "w1 after 60 Adam epochs", 1e-3)
-    _close(w2, w2_64, "w2 after 60 Adam epochs", 1e-3)
+    _close(w1, w1_64, "w1 after 60 Adam epochs", 2e-3 if narrow else 1e-3)
+    _close(w2, w2_64, "w2 after 60 Adam epochs", 2e-3 if narrow else 1e-3)
 
 
 def test_single_process_harness_prints_golden_losses(cuda):
