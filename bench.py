@@ -55,7 +55,7 @@ WORKLOADS = {
                  desc="R-MAT scale 12 plumbing configuration"),
 }
 
-SPMM_KERNELS = ("spmm_panel_dense", "spmm_panel", "spmm_hub_hot", "spmm_rowseg", "spmm_reduce", "spmm_hub_reduce")
+SPMM_KERNELS = ("spmm_panel_dense", "spmm_panel", "spmm_panel_add", "spmm_hub_hot", "spmm_rowseg", "spmm_reduce", "spmm_hub_reduce")
 TRAFFIC_FILE = ROOT / "profiles" / "spmm_traffic.txt"
 
 

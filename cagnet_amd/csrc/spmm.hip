@@ -7,6 +7,7 @@
 // (sparse-extension/sparse_coo_tensor.cu:136-231): B and C stay row-major, nothing is transposed,
 // and the CSR, its transpose, the schedules and the hub plan live in a handle.
 #include "spmm_panel_build.h"
+#include "spmm_panel_narrow.h"
 #include <stdlib.h>
 #include <string.h>
 #include <atomic>
@@ -364,6 +365,27 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
       fd.fold_D = P;
       fd.fold_dslot = pp.dslot;
       return spmm_side(*pp.rest, B, ldb, C, ldc, f, beta, stream, nullptr, &fd, false);
+    }
+  }
+  // Narrow products: the dense tiles of a panel plan of their own on the matrix cores, the other entries by the
+  // row-wise kernels, then the partial rows are added in (a pass over an n x f array, which is small here).
+  if (!epi && !fold && allow_panel && want_panel_narrow(s, f)) {
+    const PanelParams par = panel_narrow_params();
+    const bool may_decline = g_tune_panel_narrow.load(std::memory_order_relaxed) == 0;
+    PanelPlan &pp = s.panel_narrow;
+    if (!pp.valid || !par.same(pp) || (pp.declined && !may_decline && !pp.failed)) {
+      const int st = build_panel(s, pp, par, may_decline, stream, kPanelNarrowMinCoverage);
+      if (st == CG_ERR_ALLOC || st == CG_ERR_OVERFLOW) {
+        pp.declined = pp.failed = pp.valid = true;
+      } else if (st != CG_OK) {
+        return st;
+      }
+    }
+    if (!pp.declined && pp.ndtiles > 0) {
+      float *P = nullptr;
+      CG_TRY(launch_panel_narrow(pp, B, ldb, f, &P, stream));
+      CG_TRY(spmm_side(*pp.rest, B, ldb, C, ldc, f, beta, stream, nullptr, nullptr, false));
+      return launch_panel_add_rows(pp, P, C, ldc, s.rows, f, stream);
     }
   }
   if (f <= range_cap(vec == 4 ? 4 : 1) && want_hub(s, f)) {
@@ -798,6 +820,7 @@ int cg_csr_unpin(cg_csr_t *h, int64_t *released) {
   for (cg::CsrSide *s : {&h->fwd, &h->tr}) {
     count += s->unpin();
     if (s->panel.rest) count += s->panel.rest->unpin();
+    if (s->panel_narrow.rest) count += s->panel_narrow.rest->unpin();
   }
   if (released) *released = count;
   return CG_OK;
@@ -853,6 +876,8 @@ int cg_tune_set(const char *key, int value) {
   else if (!strcmp(key, "spmm_panel_unit")) cg::g_tune_panel_unit.store(value);
   else if (!strcmp(key, "spmm_panel_dmin")) cg::g_tune_panel_dmin.store(value);
   else if (!strcmp(key, "spmm_panel_dwg")) cg::g_tune_panel_dwg.store(value);
+  else if (!strcmp(key, "spmm_panel_narrow")) cg::g_tune_panel_narrow.store(value);
+  else if (!strcmp(key, "spmm_panel_narrow_dmin")) cg::g_tune_panel_narrow_dmin.store(value);
   else if (!strcmp(key, "dense_mfma")) cg::g_tune_dense_mfma.store(value);
   else if (!strcmp(key, "coo_cache_blocks")) cg::g_tune_coo_cache.store(value);
   else if (!strcmp(key, "coo_cache_mib")) cg::g_tune_coo_cache_mib.store(value);
@@ -886,8 +911,9 @@ int cg_csr_info(const cg_csr_t *h, int64_t info[8]) {
 
 int cg_csr_panel_info(const cg_csr_t *h, int transpose, int64_t info[12]) {
   if (!h || !info) CG_FAIL(CG_ERR_NULL, "cg_csr_panel_info: null pointer");
-  if (transpose && !h->has_t) CG_FAIL(CG_ERR_NO_TRANSPOSE, "cg_csr_panel_info: handle was built without CG_CSR_TRANSPOSE");
-  const cg::PanelPlan &pp = (transpose ? h->tr : h->fwd).panel;
+  if ((transpose & 1) && !h->has_t) CG_FAIL(CG_ERR_NO_TRANSPOSE, "cg_csr_panel_info: handle was built without CG_CSR_TRANSPOSE");
+  const cg::CsrSide &side = (transpose & 1) ? h->tr : h->fwd;
+  const cg::PanelPlan &pp = (transpose & 2) ? side.panel_narrow : side.panel;
   const bool used = pp.valid && !pp.declined;
   info[0] = !pp.valid ? 0 : (pp.declined ? -1 : 1);
   info[1] = used ? pp.covered : 0;

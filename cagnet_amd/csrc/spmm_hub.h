@@ -101,6 +101,7 @@ struct CsrSide {
   uint64_t hub_clock = 0;
   bool is_rest = false;  // this side is the rest matrix of a panel plan: its dense part is gone already
   PanelPlan panel;  // plan of the wide products that multiply the dense part out of LDS (spmm_panel.h)
+  PanelPlan panel_narrow;  // plan of the narrow products: dense tiles only (spmm_panel_narrow.h)
   bool pinned = false;          // a product on this side was captured into a graph (spmm_entry)
   std::vector<void *> parked;   // tables replaced since then: a captured graph may still read them
   int64_t unpin() {  // the caller has made sure that no captured graph will replay any more
@@ -114,6 +115,7 @@ struct CsrSide {
     for (void *p : parked) table_free(p);  // inside another side's product these move to that side's list
     parked.clear();
     panel.release();
+    panel_narrow.release();
     sched.release();
     for (int i = 0; i < kHubPlans; ++i) hub[i].release();
     table_free(rowptr);

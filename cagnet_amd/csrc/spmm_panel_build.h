@@ -54,7 +54,7 @@ constexpr int32_t kPanelDefaultDmin = 1024;            // entries from which a 1
 // *collision: two entries of one (row, column) pair fell into a dense tile; the plan is unusable.
 // dwg: workgroups of the dense-tile kernel (each takes an equal share of the dense tiles).
 static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot_req, int32_t unit_entries, int32_t dmin,
-                            int32_t dwg, bool may_decline, bool *collision, hipStream_t stream) {
+                            int32_t dwg, bool may_decline, double min_coverage, bool *collision, hipStream_t stream) {
   *collision = false;
   const int64_t nnz = s.nnz;
   const int32_t n = s.rows, m = s.cols;
@@ -144,7 +144,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   CG_HIP(hipStreamSynchronize(stream));
   const int64_t ntiles = tot[0], covered = tot[1], ndtiles = tot[2], dcovered = tot[3];
   if (ntiles + ndtiles == 0 || covered + dcovered == 0 ||
-      (may_decline && (double)(covered + dcovered) < kPanelMinCoverage * (double)nnz))
+      (may_decline && (double)(covered + dcovered) < min_coverage * (double)nnz))
     return decline();
   if (ntiles * kPanelWaves + 2 > 0x7fffffffLL || ndtiles * kDenseTileFloats > 0x7fffffffLL * 4) return decline();
 
@@ -393,15 +393,17 @@ static PanelParams panel_params() {
 }
 
 // Builds the plan for the given values; the plan carries them whatever the outcome (in use, declined).
-static int build_panel(CsrSide &s, PanelPlan &pp, const PanelParams &par, bool may_decline, hipStream_t stream) {
+static int build_panel(CsrSide &s, PanelPlan &pp, const PanelParams &par, bool may_decline, hipStream_t stream,
+                       double min_coverage = kPanelMinCoverage) {
   CG_TRY(refuse_under_capture(stream, "building a panel plan"));
   CG_HIP(hipStreamSynchronize(stream));
   pp.release();
   bool collision = false;
-  int st = build_panel_once(s, pp, par.emin, par.cols, par.unit, par.dmin, par.dwg, may_decline, &collision, stream);
+  int st = build_panel_once(s, pp, par.emin, par.cols, par.unit, par.dmin, par.dwg, may_decline, min_coverage, &collision,
+                            stream);
   if (st == CG_OK && collision) {  // the matrix stores a (row, column) pair twice: every tile goes the record way
     pp.release();
-    st = build_panel_once(s, pp, par.emin, par.cols, par.unit, 0, par.dwg, may_decline, &collision, stream);
+    st = build_panel_once(s, pp, par.emin, par.cols, par.unit, 0, par.dwg, may_decline, min_coverage, &collision, stream);
   }
   if (st != CG_OK) pp.release();
   par.stamp(pp);

@@ -199,7 +199,8 @@ int cg_csr_spmm_xw(cg_csr_t *h, int transpose, const float *d_B, int64_t ldb, co
  *                column-popularity plan last looked up by a wide product of A, of A^T:
  *                tiers in use, -1 when the column counts declined it, 0 when none was considered } */
 int cg_csr_info(const cg_csr_t *h, int64_t info[8]);
-/* Panel plan a wide product of A (transpose != 0: of A^T) last looked up: info[0..11] =
+/* Panel plan a wide product of A (bit 0 of `transpose` set: of A^T) last looked up; with bit 1 of `transpose` set the
+ * plan of the narrow products (f <= 64), which has dense tiles only: info[0..11] =
  * { 1 in use / -1 declined (the tiles hold too few of the entries) / 0 none considered yet,
  *   entries multiplied out of LDS by the vector ALUs, their (active) tiles, their units (workgroups),
  *   row panels with several units of either kind, entries left to the row-wise kernels, entries a tile
@@ -329,7 +330,8 @@ int cg_coo_block(const int32_t *d_row, const int32_t *d_col, const float *d_val,
  * product, or the cold class of a hub plan), "spmm_hub_hot" (all hot tiers of a hub plan as one
  * record), "spmm_reduce" (rows split into segments), "spmm_hub_reduce" (partial rows of a hub plan
  * with narrow teams), "spmm_panel" (staged tiles of a panel plan and the sum of a panel's blocks of
- * partial rows), "spmm_panel_dense" (its dense tiles on the matrix cores), "dense_xw", "dense_gwt", "dense_xtg" (partial products and their sum),
+ * partial rows), "spmm_panel_dense" (its dense tiles on the matrix cores), "spmm_panel_add" (partial rows added to a narrow
+ * product), "dense_xw", "dense_gwt", "dense_xtg" (partial products and their sum),
  * "relu_fwd", "relu_bwd" (no suffix), "log_softmax_fwd", "log_softmax_bwd", "nll_fwd", "nll_bwd",
  * "log_softmax_nll_bwd".
  * Recording is off by default and costs nothing then.
@@ -355,6 +357,11 @@ int cg_prof_enable(int on);
  *                     cores (0: 1024, a quarter full; negative: never).  Such a tile multiplies its zeros too:
  *                     a row of B with an infinity or a NaN then reaches all 128 rows of the tile
  *   "spmm_panel_dwg"  workgroups that share the dense tiles equally (0: four per compute unit)
+ *   "spmm_panel_narrow" the same plan with dense tiles only for narrow products (f <= 64; the other entries go to the
+ *                     row-wise kernels and the partial rows are added in afterwards): -1 never, 1 always, 0 when rows
+ *                     hold at least 64 entries on average, the product has at least 1e9 multiply-adds and the dense
+ *                     tiles hold at least a quarter of the entries
+ *   "spmm_panel_narrow_dmin" entries from which a tile is dense for narrow products (0: 512)
  *   "dense_mfma"      -1: dense products on the vector ALU tile kernel only
  *   "coo_cache_blocks" blocks cg_spmm_coo_cached keeps (0: 8; negative: none)
  *   "coo_cache_mib"   device memory those blocks may hold together, in MiB (0: 32768); a block counts as three

@@ -90,15 +90,17 @@ def test_spmm_schedules_random(cuda, knobs_restored, seed):
     ops.coo_cache_clear()
 
 
-PANEL_KNOBS = [b"spmm_panel", b"spmm_panel_emin", b"spmm_panel_cols", b"spmm_panel_unit", b"spmm_panel_dmin", b"spmm_panel_dwg"]
+PANEL_KNOBS = [b"spmm_panel", b"spmm_panel_emin", b"spmm_panel_cols", b"spmm_panel_unit", b"spmm_panel_dmin", b"spmm_panel_dwg",
+               b"spmm_panel_narrow", b"spmm_panel_narrow_dmin"]
 
 
 @pytest.mark.parametrize("seed", [31, 32])
 def test_spmm_panel_plan_random(cuda, knobs_restored, seed):
     """The panel plan forced on over random patterns (skewed and uniform, with full rows and columns, rectangular),
-    every even width class it is built for, both sides, accumulate forms, padded leading dimensions, and random plan
-    knobs: entries a tile needs, ranked columns, unit size, dense-tile threshold (off, low, high) and the number of
-    workgroups that share the dense tiles.  Every entry is in exactly one of the three parts of the plan."""
+    every even width class it is built for and the narrow widths (dense tiles only), both sides, accumulate forms,
+    padded leading dimensions, and random plan knobs: entries a tile needs, ranked columns, unit size, dense-tile
+    threshold (off, low, high) and the number of workgroups that share the dense tiles.  Every entry is in exactly one
+    of the parts of the plan."""
     import ctypes
     from cagnet_amd import ops
     from cagnet_amd._lib import check
@@ -123,9 +125,10 @@ def test_spmm_panel_plan_random(cuda, knobs_restored, seed):
             if idx.shape[0] == 0:
                 continue
             row, col, val = idx[:, 0].int().to(cuda), idx[:, 1].int().to(cuda), dense[mask].to(cuda)
-            f = rng.choice([258, 260, 300, 320, 322, 384, 448, 450, 512, 576, 602, 636])
+            f = rng.choice([258, 260, 300, 320, 322, 384, 448, 450, 512, 576, 602, 636, 1, 3, 16, 17, 41, 44, 63, 64])
+            narrow = f <= 64
             values = [1, rng.choice([1, 4, 16, 64]), rng.choice([0, 32, 64, 1024]), rng.choice([0, 50, 2000]),
-                      rng.choice([-1, 0, 8, 40, 200, 3000]), rng.choice([0, 1, 5, 300])]
+                      rng.choice([-1, 0, 8, 40, 200, 3000]), rng.choice([0, 1, 5, 300]), 1, rng.choice([0, 4, 30, 500])]
             for key, v in zip(PANEL_KNOBS, values):
                 assert lib.cg_tune_set(key, v) == 0
             tr = rng.random() < 0.4
@@ -142,11 +145,13 @@ def test_spmm_panel_plan_random(cuda, knobs_restored, seed):
                 A.spmm(B, out=C, beta=beta, transpose=tr)
                 outs.append(C)
             info = (ctypes.c_int64 * 12)()
-            check(lib.cg_csr_panel_info(A._handle, int(tr), info), "cg_csr_panel_info")
+            check(lib.cg_csr_panel_info(A._handle, int(tr) | (2 if narrow else 0), info), "cg_csr_panel_info")
             assert info[0] in (1, -1), what                       # in use, or no tile reached the threshold
             if info[0] == 1:
                 assert info[1] + info[8] + info[5] == val.numel(), what
-                if values[4] < 0:
+                if narrow:
+                    assert info[1] == 0 and info[2] == 0, what    # no staged tiles
+                elif values[4] < 0:
                     assert info[9] == 0, what
             A64 = dense.double().to(cuda)
             A64 = A64.t() if tr else A64

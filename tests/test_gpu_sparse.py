@@ -821,7 +821,7 @@ def _panel_info(A, transpose=False):
     import ctypes
     from cagnet_amd._lib import check, lib
     buf = (ctypes.c_int64 * 12)()
-    check(lib.cg_csr_panel_info(A._handle, int(transpose), buf), "cg_csr_panel_info")
+    check(lib.cg_csr_panel_info(A._handle, int(transpose), buf), "cg_csr_panel_info")   # bit 1: plan of the narrow products
     return dict(state=buf[0], covered=buf[1], tiles=buf[2], units=buf[3], split=buf[4], rest=buf[5], emin=buf[6], cols=buf[7],
                 dense_covered=buf[8], dense_tiles=buf[9], dense_units=buf[10], dmin=buf[11])
 
@@ -897,6 +897,44 @@ def test_spmm_panel_dense_tiles_on_matrix_cores(cuda, tune, f, dmin, dwg):
     rec = A.spmm(B.to(cuda))
     assert _panel_info(A)["dense_tiles"] == 0 and _panel_info(A)["dmin"] == 0
     assert spmm_error(rec, row, col, val, n, n, B) <= REL_TOL
+
+
+@pytest.mark.parametrize("f", [1, 8, 16, 24, 41, 44, 48, 64])
+@pytest.mark.parametrize("dmin,dwg", [(40, 3), (300, 0)])
+def test_spmm_narrow_products_with_dense_tiles(cuda, tune, f, dmin, dwg):
+    """Narrow products (f <= 64) with their panel plan forced on: tiles with at least dmin entries are multiplied on
+    the fp32 matrix cores, the other entries by the row-wise kernels, and the partial rows are added to the result
+    afterwards.  Same 1e-5 bound against the fp64 oracle, bit-identical repeats, accumulate form, A^T, strided
+    operands; every entry is in the dense tiles or in the rest."""
+    from cagnet_amd import ops
+    row, col, val, n = small_graph(12, 160000, seed=13 * f + dmin)
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n, transpose=True)
+    tune("spmm_panel_narrow", 1)
+    tune("spmm_panel_narrow_dmin", dmin)
+    tune("spmm_panel_cols", 2048)
+    tune("spmm_panel_dwg", dwg)
+    g = torch.Generator().manual_seed(f)
+    big = torch.randn(n, f + 3, generator=g).to(cuda)
+    B = big[:, 1:1 + f]
+    got = A.spmm(B)
+    info = _panel_info(A, transpose=2)
+    assert info["state"] == 1 and info["dense_tiles"] > 0 and info["tiles"] == 0 and info["covered"] == 0
+    assert info["dense_covered"] + info["rest"] == row.numel() and info["dmin"] == dmin
+    assert spmm_error(got, row, col, val, n, n, B.cpu()) <= REL_TOL
+    assert torch.equal(got, A.spmm(B))
+    C0 = torch.randn(n, f, generator=g)
+    Cbig = torch.zeros(n, f + 5, device=cuda)
+    C = Cbig[:, 2:2 + f]
+    C.copy_(C0)
+    A.spmm(B, out=C, beta=1.0)
+    assert spmm_error(C, row, col, val, n, n, B.cpu(), C0) <= REL_TOL
+    assert float(Cbig[:, :2].abs().max()) == 0.0 and float(Cbig[:, 2 + f:].abs().max()) == 0.0
+    gotT = A.spmm(B, transpose=True)
+    assert _panel_info(A, transpose=3)["dense_tiles"] > 0
+    assert spmm_error(gotT, row, col, val, n, n, B.cpu()) <= REL_TOL
+    tune("spmm_panel_narrow", -1)
+    plain = A.spmm(B)
+    assert spmm_error(plain, row, col, val, n, n, B.cpu()) <= REL_TOL
 
 
 def test_spmm_panel_all_tiles_dense_and_duplicate_entries(cuda, tune):
