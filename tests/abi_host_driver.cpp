@@ -185,6 +185,8 @@ static void with_gpu() {
     EXPECT(cg_tune_set("spmm_panel_emin", pass >= 2 ? 8 : 0) == CG_OK);
     EXPECT(cg_tune_set("spmm_panel_dmin", pass == 3 ? 48 : 0) == CG_OK);
     EXPECT(cg_tune_set("spmm_panel_dwg", pass == 3 ? 3 : 0) == CG_OK);
+    EXPECT(cg_tune_set("spmm_panel_narrow", pass == 3 ? 1 : 0) == CG_OK);  // the narrow widths take dense tiles too
+    EXPECT(cg_tune_set("spmm_panel_narrow_dmin", pass == 3 ? 48 : 0) == CG_OK);
     for (int f : widths) {
       Lcg g{(uint64_t)f * 31 + pass};
       std::vector<float> B((size_t)m * f), C((size_t)n * f, 0.f);
@@ -200,6 +202,10 @@ static void with_gpu() {
       }
       EXPECT(cg_csr_panel_info(h, 0, info) == CG_OK);
       if (pass == 3 && f >= 258) EXPECT(info[0] == 1 && info[9] > 0 && info[1] + info[8] + info[5] == nnz);
+      if (pass == 3 && f <= 64) {
+        EXPECT(cg_csr_panel_info(h, 2, info) == CG_OK);
+        EXPECT(info[0] == 1 && info[9] > 0 && info[1] == 0 && info[8] + info[5] == nnz);
+      }
       HIP_OK(hipFree(d_B));
       HIP_OK(hipFree(d_C));
     }
@@ -250,7 +256,8 @@ static void with_gpu() {
     HIP_OK(hipFree(d_B));
     HIP_OK(hipFree(d_C));
   }
-  for (const char *k : {"spmm_hub", "spmm_hub_kb", "spmm_panel", "spmm_panel_emin", "spmm_panel_dmin", "spmm_panel_dwg"})
+  for (const char *k : {"spmm_hub", "spmm_hub_kb", "spmm_panel", "spmm_panel_emin", "spmm_panel_dmin", "spmm_panel_dwg",
+                        "spmm_panel_narrow", "spmm_panel_narrow_dmin"})
     EXPECT(cg_tune_set(k, 0) == CG_OK);
   int64_t released = -1;
   EXPECT(cg_csr_unpin(h, &released) == CG_OK && released == 0);  // nothing was captured: nothing was parked
