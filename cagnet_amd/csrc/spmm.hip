@@ -734,7 +734,7 @@ int cg_spmm_coo_cached(const int32_t *d_row, const int32_t *d_col, const float *
     entry->n = n;
     entry->m = m;
     entry->device = device;
-    entry->bytes = 3 * (nnz * 8) + 4 * ((int64_t)n + 1) * 4;
+    entry->bytes = 4 * (nnz * 8) + 4 * ((int64_t)n + 1) * 4;  // the CSR, a panel plan (tiles, records, rest) and the rest's hub plans
     entry->h = h;
     std::vector<std::shared_ptr<CooCacheEntry>> evicted;  // released after the lock is dropped
     {

@@ -338,6 +338,16 @@ class CsrMatrix:
                 # column-popularity plan the last wide product looked up: tiers, -1 declined, 0 none
                 "plan_tiers": buf[6], "plan_tiers_transpose": buf[7]}
 
+    def panel_info(self, transpose: bool = False, narrow: bool = False) -> dict:
+        """Panel plan the last wide (narrow=True: narrow, f <= 64) product of A (transpose=True: of A^T) looked up:
+        state 1 in use / -1 declined / 0 none considered; entries multiplied out of LDS, in dense tiles on the matrix
+        cores, left to the row-wise kernels; tile and unit counts; the thresholds the plan was built with."""
+        buf = (c_int64 * 12)()
+        check(lib.cg_csr_panel_info(self._handle, int(transpose) | (2 if narrow else 0), buf), "cg_csr_panel_info")
+        return {"state": buf[0], "staged_entries": buf[1], "staged_tiles": buf[2], "staged_units": buf[3],
+                "split_panels": buf[4], "rest_entries": buf[5], "tile_min_entries": buf[6], "ranked_columns": buf[7],
+                "dense_entries": buf[8], "dense_tiles": buf[9], "dense_units": buf[10], "dense_min_entries": buf[11]}
+
     def arrays(self, transpose: bool = False):
         """(rowptr, colind, values) of A, or of A^T, as tensors that alias the handle's memory."""
         p = [c_void_p(0), c_void_p(0), c_void_p(0)]

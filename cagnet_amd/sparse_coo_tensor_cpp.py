@@ -17,7 +17,7 @@ Differences a caller can observe, all deliberate:
 `cache_blocks`: the reference's callers pass the same block at every stage of every epoch, as
 fresh `.int()` temporaries.  When True, spmm_gpu recognises a block by a digest of its arrays and
 reuses the CSR, schedules and plans built when it first saw it (cg_spmm_coo_cached); when False
-every call rebuilds them on the device (cg_spmm_coo).  Kept blocks hold device memory (about three
+every call rebuilds them on the device (cg_spmm_coo).  Kept blocks hold device memory (about four
 copies of a block's entries each, at most 8 blocks or 32 GiB, least recently used dropped first;
 `ops.coo_cache_clear()` hands it back).  A caller whose values change on every call should set it to
 False: every call would otherwise build a handle and a plan for a block that is never seen again.

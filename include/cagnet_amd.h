@@ -364,8 +364,8 @@ int cg_prof_enable(int on);
  *   "spmm_panel_narrow_dmin" entries from which a tile is dense for narrow products (0: 512)
  *   "dense_mfma"      -1: dense products on the vector ALU tile kernel only
  *   "coo_cache_blocks" blocks cg_spmm_coo_cached keeps (0: 8; negative: none)
- *   "coo_cache_mib"   device memory those blocks may hold together, in MiB (0: 32768); a block counts as three
- *                     copies of its entries (the CSR and up to two plans); the newest block always stays
+ *   "coo_cache_mib"   device memory those blocks may hold together, in MiB (0: 32768); a block counts as four
+ *                     copies of its entries (the CSR and its plans); the newest block always stays
  *   "test_alloc_fail" test hook: k > 0 makes the k-th device allocation for handle tables from now on fail
  *                     once with CG_ERR_ALLOC (a plan whose build fails that way is given up for good and the
  *                     product runs on the plain schedule)

@@ -920,6 +920,8 @@ def test_spmm_narrow_products_with_dense_tiles(cuda, tune, f, dmin, dwg):
     info = _panel_info(A, transpose=2)
     assert info["state"] == 1 and info["dense_tiles"] > 0 and info["tiles"] == 0 and info["covered"] == 0
     assert info["dense_covered"] + info["rest"] == row.numel() and info["dmin"] == dmin
+    pi = A.panel_info(narrow=True)
+    assert pi["state"] == 1 and pi["dense_entries"] == info["dense_covered"] and pi["rest_entries"] == info["rest"]
     assert spmm_error(got, row, col, val, n, n, B.cpu()) <= REL_TOL
     assert torch.equal(got, A.spmm(B))
     C0 = torch.randn(n, f, generator=g)
