@@ -2,8 +2,10 @@
 //
 // A row-wise SpMM gathers one row of B per stored entry (2408 bytes at f = 602); on a matrix with a
 // few hundred entries per row nearly all of that traffic is re-reading rows of B that other rows of A
-// also use.  Here rows and columns are ranked by their entry counts, rows are taken in panels of 128
-// consecutive ranks and columns in blocks of 32 consecutive ranks.  A (panel, block) tile that holds
+// also use.  Here rows are ranked by their entry counts and taken in panels of 128 consecutive ranks;
+// inside a panel the columns are ranked by the entries they have in these 128 rows and taken in blocks
+// of 32 consecutive ranks (every panel has its own blocks: a column with two entries in the panel sits
+// among its likes, wherever it stands in the matrix as a whole).  A (panel, block) tile that holds
 // enough entries is "active": its 32 rows of B are copied into LDS once (global -> LDS directly, no
 // registers in between) and all of the tile's entries read them from there, at LDS bandwidth instead
 // of through the vector memory path.  A workgroup of 16 waves owns a unit = a run of active tiles of one
@@ -487,22 +489,116 @@ __device__ __forceinline__ int64_t panel_tile_of(int32_t rrank, int32_t crank, i
   return (int64_t)(rrank / kPanelRows) * nkb + crank / kPanelCols;
 }
 
-__global__ __launch_bounds__(kSpmmThreads) void panel_tile_count_kernel(
-    const int32_t *__restrict__ erow, const int32_t *__restrict__ colind, int64_t nnz, const int32_t *__restrict__ row_rank,
-    const int32_t *__restrict__ col_rank, int32_t prows, int32_t hot, int32_t nkb, uint32_t *__restrict__ tcount) {
-  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
-  if (k >= nnz) return;
-  const int64_t t = panel_tile_of(row_rank[erow[k]], col_rank[colind[k]], prows, hot, nkb);
-  if (t >= 0) atomicAdd(&tcount[t], 1u);
-}
-
 // Tiles with emin .. dmin - 1 entries are staged ("active"), tiles with at least dmin entries are dense
-// (dmin == 0: none).  flag[t] = 1 and kept[t] = tcount[t] for active tiles, dflag / dkept the same for
-// dense ones, else 0 (the four arrays are then scanned).
+// (dmin == 0: none).
 __device__ __forceinline__ int panel_tile_kind(uint32_t count, uint32_t emin, uint32_t dmin) {
   if (dmin > 0 && count >= dmin) return 2;
   return count >= emin ? 1 : 0;
 }
+
+__global__ __launch_bounds__(kSpmmThreads) void panel_tile_count_kernel(
+    const int32_t *__restrict__ erow, const int32_t *__restrict__ ecr, int64_t nnz, const int32_t *__restrict__ row_rank,
+    int32_t prows, int32_t hot, int32_t nkb, uint32_t *__restrict__ tcount) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k >= nnz) return;
+  const int64_t t = panel_tile_of(row_rank[erow[k]], ecr[k], prows, hot, nkb);
+  if (t >= 0) atomicAdd(&tcount[t], 1u);
+}
+
+// Column ranks inside the panels.  The entries are sorted by (panel, column); a run of equal keys is a
+// (panel, column) pair, and the pairs of a panel are ranked by descending length (ties: by column).
+// Entries of rows behind the ranked panels get the panel number `npanels`, which sorts them last.
+__global__ __launch_bounds__(kSpmmThreads) void panel_pair_key_kernel(const int32_t *__restrict__ erow,
+                                                                      const int32_t *__restrict__ colind, int64_t nnz,
+                                                                      const int32_t *__restrict__ row_rank, int32_t prows,
+                                                                      int32_t npanels, int32_t *__restrict__ kpanel,
+                                                                      int32_t *__restrict__ kcol, int32_t *__restrict__ pos) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k >= nnz) return;
+  const int32_t rr = row_rank[erow[k]];
+  kpanel[k] = rr < prows ? rr / kPanelRows : npanels;
+  kcol[k] = colind[k];
+  pos[k] = (int32_t)k;
+}
+
+// sort keys of the pairs: (panel, 255 - min(entries, 255)), payload the pair's number; pair_col[pair] = its column.
+// pair_first[npairs] = number of entries.
+__global__ __launch_bounds__(kSpmmThreads) void panel_pair_count_key_kernel(
+    const uint32_t *__restrict__ pair_first, int64_t npairs, const int32_t *__restrict__ kpanel_sorted,
+    const int32_t *__restrict__ kcol_sorted, int32_t *__restrict__ pk_panel, int32_t *__restrict__ pk_count,
+    int32_t *__restrict__ pk_pair, int32_t *__restrict__ pair_col) {
+  const int64_t p = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (p >= npairs) return;
+  const uint32_t first = pair_first[p], count = pair_first[p + 1] - first;
+  pk_panel[p] = kpanel_sorted[first];
+  pk_count[p] = 255 - (int32_t)(count < 255u ? count : 255u);
+  pk_pair[p] = (int32_t)p;
+  pair_col[p] = kcol_sorted[first];
+}
+
+// pair_lr[pair] = rank of the pair's column inside its panel, `hot` for ranks from `hot` on and for the rows
+// behind the panels (hot = the ranks that can be part of a tile)
+__global__ __launch_bounds__(kSpmmThreads) void panel_pair_rank_kernel(const int32_t *__restrict__ spanel,
+                                                                       const int32_t *__restrict__ spair, int64_t npairs,
+                                                                       const int32_t *__restrict__ pstart, int32_t npanels,
+                                                                       int32_t hot, int32_t *__restrict__ pair_lr) {
+  const int64_t j = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (j >= npairs) return;
+  const int32_t panel = spanel[j];
+  int64_t lr = hot;
+  if (panel < npanels) {
+    lr = j - pstart[panel];
+    if (lr > hot) lr = hot;
+  }
+  pair_lr[spair[j]] = (int32_t)lr;
+}
+
+// ecr[entry] = rank of the entry's column inside the entry's panel (start / runs_before: the run starts of the
+// sorted entries and their exclusive scan; pos_sorted: the entry at a sorted position)
+__global__ __launch_bounds__(kSpmmThreads) void panel_entry_rank_kernel(const uint32_t *__restrict__ start,
+                                                                        const uint32_t *__restrict__ runs_before,
+                                                                        const int32_t *__restrict__ pos_sorted, int64_t nnz,
+                                                                        const int32_t *__restrict__ pair_lr,
+                                                                        int32_t *__restrict__ ecr) {
+  const int64_t i = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (i >= nnz) return;
+  ecr[pos_sorted[i]] = pair_lr[runs_before[i] + start[i] - 1u];
+}
+
+// The column of every place of the active and of the dense tiles, from the ranked pairs: place c of an active
+// tile is staged by wave c % 16 as its row c / 16 (hdr[(tile * 16 + wave) * 4 + c / 16]), place c of a dense
+// tile is dhdr[tile * 32 + c].  Both arrays hold -1 beforehand; a panel's last block can have fewer than 32
+// columns, and its empty places are then given the block's first column (panel_hdr_kernel,
+// panel_dense_hdr_fill_kernel): no entry refers to them, a dense tile holds zeros there.
+__global__ __launch_bounds__(kSpmmThreads) void panel_pair_hdr_kernel(
+    const int32_t *__restrict__ spanel, const int32_t *__restrict__ spair, int64_t npairs, const int32_t *__restrict__ pstart,
+    int32_t npanels, int32_t hot, int32_t nkb, const int32_t *__restrict__ pair_col, const uint32_t *__restrict__ tcount,
+    const uint32_t *__restrict__ tindex, const uint32_t *__restrict__ dindex, uint32_t emin, uint32_t dmin,
+    int32_t *__restrict__ hdr, int32_t *__restrict__ dhdr) {
+  const int64_t j = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (j >= npairs) return;
+  const int32_t panel = spanel[j];
+  if (panel >= npanels) return;
+  const int64_t lr = j - pstart[panel];
+  if (lr >= hot) return;
+  const int64_t t = (int64_t)panel * nkb + lr / kPanelCols;
+  const int c = (int)(lr % kPanelCols);
+  const int kind = panel_tile_kind(tcount[t], emin, dmin);
+  const int32_t col = pair_col[spair[j]];
+  if (kind == 1)
+    hdr[((int64_t)tindex[t] * kPanelWaves + c % kPanelWaves) * 4 + c / kPanelWaves] = col;
+  else if (kind == 2)
+    dhdr[(int64_t)dindex[t] * kPanelCols + c] = col;
+}
+
+__global__ __launch_bounds__(kSpmmThreads) void panel_dense_hdr_fill_kernel(int32_t *__restrict__ dhdr, int64_t ndtiles) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k >= ndtiles * kPanelCols || k % kPanelCols == 0) return;  // place 0 of a tile is always taken
+  if (dhdr[k] < 0) dhdr[k] = dhdr[k / kPanelCols * kPanelCols];
+}
+
+// flag[t] = 1 and kept[t] = tcount[t] for active tiles, dflag / dkept the same for dense ones, else 0 (the four
+// arrays are then scanned).
 
 __global__ __launch_bounds__(kSpmmThreads) void panel_tile_select_kernel(const uint32_t *__restrict__ tcount, int64_t tiles,
                                                                          uint32_t emin, uint32_t dmin,
@@ -518,15 +614,13 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_tile_select_kernel(const u
   dkept[t] = kind == 2 ? tcount[t] : 0u;
 }
 
-// compact tables of the tiles of one kind (1: active, 2: dense)
+// panel of every tile of one kind (1: active, 2: dense), in the compacted numbering
 __global__ __launch_bounds__(kSpmmThreads) void panel_tile_tables_kernel(const uint32_t *__restrict__ tcount,
                                                                          const uint32_t *__restrict__ tindex, int64_t tiles,
                                                                          uint32_t emin, uint32_t dmin, int kind, int32_t nkb,
-                                                                         int32_t *__restrict__ tile_kb,
                                                                          int32_t *__restrict__ tile_panel) {
   const int64_t t = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (t >= tiles || panel_tile_kind(tcount[t], emin, dmin) != kind) return;
-  tile_kb[tindex[t]] = (int32_t)(t % nkb);
   tile_panel[tindex[t]] = (int32_t)(t / nkb);
 }
 
@@ -537,15 +631,15 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_tile_tables_kernel(const u
 // exchange finds the second one (unless one of them is +0, which changes nothing) and raises *collision,
 // after which the caller builds the plan again without dense tiles.
 __global__ __launch_bounds__(kSpmmThreads) void panel_entry_key_kernel(
-    const int32_t *__restrict__ erow, const int32_t *__restrict__ colind, const float *__restrict__ val, int64_t nnz,
-    const int32_t *__restrict__ row_rank, const int32_t *__restrict__ col_rank, int32_t prows, int32_t hot, int32_t nkb,
+    const int32_t *__restrict__ erow, const int32_t *__restrict__ ecr, const float *__restrict__ val, int64_t nnz,
+    const int32_t *__restrict__ row_rank, int32_t prows, int32_t hot, int32_t nkb,
     const uint32_t *__restrict__ tcount, const uint32_t *__restrict__ tindex, const uint32_t *__restrict__ dindex,
     uint32_t emin, uint32_t dmin, int32_t sentinel, int32_t *__restrict__ key, int32_t *__restrict__ slot,
     int32_t *__restrict__ pos, uint32_t *__restrict__ dA_bits, uint32_t *__restrict__ collision) {
   const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (k >= nnz) return;
   const int32_t rr = row_rank[erow[k]];
-  const int32_t cr = col_rank[colind[k]];
+  const int32_t cr = ecr[k];
   const int64_t t = panel_tile_of(rr, cr, prows, hot, nkb);
   int32_t ky = sentinel, sl = 0;
   const int kind = t >= 0 ? panel_tile_kind(tcount[t], emin, dmin) : 0;
@@ -570,13 +664,13 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_entry_key_kernel(
 __global__ __launch_bounds__(kSpmmThreads) void panel_entry_finish_kernel(
     const int32_t *__restrict__ slot_sorted, const int32_t *__restrict__ pos, int64_t count, int64_t covered,
     const int32_t *__restrict__ erow, const int32_t *__restrict__ colind, const float *__restrict__ val,
-    const int32_t *__restrict__ col_rank, uint2 *__restrict__ ent, int32_t *__restrict__ rest_row,
+    const int32_t *__restrict__ ecr, uint2 *__restrict__ ent, int32_t *__restrict__ rest_row,
     int32_t *__restrict__ rest_col, float *__restrict__ rest_val) {
   const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (k >= count) return;  // count = entries of active tiles + rest; the entries of dense tiles lie behind them
   const int32_t p = pos[k];
   if (k < covered) {
-    ent[k] = make_uint2((uint32_t)(col_rank[colind[p]] % kPanelCols) | ((uint32_t)slot_sorted[k] << 8), __float_as_uint(val[p]));
+    ent[k] = make_uint2((uint32_t)(ecr[p] % kPanelCols) | ((uint32_t)slot_sorted[k] << 8), __float_as_uint(val[p]));
   } else {
     rest_row[k - covered] = erow[p];
     rest_col[k - covered] = colind[p];
@@ -638,26 +732,18 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_pad_wptr_kernel(int32_t *_
   if (j < entries) wptr[j] += (int32_t)shift[wptr[j]];
 }
 
-// hdr[(t * 16 + w) * 4 ..] = {row of B of column w of the tile's block, the same of column w + 16, first record, end}
-__global__ __launch_bounds__(kSpmmThreads) void panel_hdr_kernel(const int32_t *__restrict__ tile_kb,
-                                                                  const int32_t *__restrict__ tile_wptr,
-                                                                  const int32_t *__restrict__ qcol, int64_t ntiles,
-                                                                  int4 *__restrict__ hdr) {
+// hdr[(t * 16 + w) * 4 ..] = {row of B of place w of the tile, the same of place w + 16, first record, end}: the rows
+// are there already (panel_pair_hdr_kernel) except for empty places, which get the row of the tile's place 0
+__global__ __launch_bounds__(kSpmmThreads) void panel_hdr_kernel(const int32_t *__restrict__ tile_wptr, int64_t ntiles,
+                                                                  int32_t *__restrict__ hdr) {
   const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (k >= ntiles * kPanelWaves) return;
   const int64_t t = k / kPanelWaves;
-  const int w = (int)(k % kPanelWaves);
-  const int64_t c = (int64_t)tile_kb[t] * kPanelCols + w;
-  hdr[k] = make_int4(qcol[c], qcol[c + kPanelWaves], tile_wptr[k], tile_wptr[k + 1]);
-}
-
-// dhdr[t * 32 + j] = row of B of column j of dense tile t's block
-__global__ __launch_bounds__(kSpmmThreads) void panel_dense_hdr_kernel(const int32_t *__restrict__ dtile_kb,
-                                                                        const int32_t *__restrict__ qcol, int64_t ndtiles,
-                                                                        int32_t *__restrict__ dhdr) {
-  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
-  if (k >= ndtiles * kPanelCols) return;
-  dhdr[k] = qcol[(int64_t)dtile_kb[k / kPanelCols] * kPanelCols + k % kPanelCols];
+  const int32_t first = hdr[t * kPanelWaves * 4];  // place 0 of a tile is always taken, and nobody writes it here
+  if (hdr[k * 4 + 1] < 0) hdr[k * 4 + 1] = first;
+  if (k % kPanelWaves != 0 && hdr[k * 4] < 0) hdr[k * 4] = first;
+  hdr[k * 4 + 2] = tile_wptr[k];
+  hdr[k * 4 + 3] = tile_wptr[k + 1];
 }
 
 __global__ __launch_bounds__(kSpmmThreads) void panel_dslot_kernel(const int32_t *__restrict__ row_rank, int32_t n,

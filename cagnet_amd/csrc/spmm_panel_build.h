@@ -72,16 +72,13 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   if (npanels < 1) return decline();
   const int32_t prows = (int32_t)(npanels * kPanelRows < n ? npanels * kPanelRows : n);
   const int64_t tiles = npanels * nkb;
-  const unsigned gn = (unsigned)ceil_div64(n, kSpmmThreads), gm = (unsigned)ceil_div64(m, kSpmmThreads);
+  const unsigned gn = (unsigned)ceil_div64(n, kSpmmThreads);
   const unsigned ge = (unsigned)ceil_div64(nnz, kSpmmThreads), gt = (unsigned)ceil_div64(tiles + 1, kSpmmThreads);
   DevTemps tmp;
 
-  // 1. rows ranked by descending degree, columns by descending entry count (ties: by index)
-  int32_t *row_rank = nullptr, *col_rank = nullptr;
+  // 1. rows ranked by descending degree (ties: by index)
+  int32_t *row_rank = nullptr;
   CG_TRY(tmp.alloc((void **)&row_rank, (size_t)n * 4));
-  CG_TRY(tmp.alloc((void **)&col_rank, (size_t)m * 4));
-  int32_t *qcol = nullptr;  // row of B of every ranked hot column
-  CG_TRY(tmp.alloc((void **)&qcol, (size_t)hot * 4));
   {
     DevTemps t2;
     SortBuffers buf;
@@ -95,42 +92,81 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     CG_LAUNCH_CHECK();
     CG_HIP(hipStreamSynchronize(stream));
   }
+
+  // 1b. columns ranked inside every panel by the entries they have there: the entries sorted by (panel, column),
+  //     the runs of that order (= pairs) sorted by (panel, descending length).  ecr[entry] = rank of its column
+  //     in its panel; the sorted pairs stay for the tile headers.
+  int32_t *erow = nullptr, *ecr = nullptr, *pstart = nullptr, *pair_col = nullptr, *spanel = nullptr, *spair = nullptr;
+  int64_t npairs = 0;
+  CG_TRY(tmp.alloc((void **)&erow, (size_t)nnz * 4));
+  CG_TRY(tmp.alloc((void **)&ecr, (size_t)nnz * 4));
+  CG_TRY(tmp.alloc((void **)&pstart, (size_t)(npanels + 2) * 4));
+  panel_expand_rows_kernel<<<(unsigned)ceil_div64((int64_t)n * kWave, kSpmmThreads), kSpmmThreads, 0, stream>>>(s.rowptr, n, erow);
+  CG_LAUNCH_CHECK();
   {
     DevTemps t2;
     SortBuffers buf;
-    uint32_t *count = nullptr;
-    CG_TRY(t2.alloc((void **)&count, (size_t)m * 4));
-    CG_TRY(alloc_sort_buffers(t2, buf, m));
-    CG_TRY(fill_u32(count, m, 0u, stream));
-    panel_col_count_kernel<<<ge, kSpmmThreads, 0, stream>>>(s.colind, nnz, count);
+    uint32_t *start = nullptr, *runs_before = nullptr, *pair_first = nullptr, *d_np = nullptr;
+    int32_t *pair_lr = nullptr;
+    CG_TRY(alloc_sort_buffers(t2, buf, nnz));
+    CG_TRY(t2.alloc((void **)&start, (size_t)(nnz + 1) * 4));
+    CG_TRY(t2.alloc((void **)&runs_before, (size_t)(nnz + 1) * 4));
+    CG_TRY(t2.alloc((void **)&d_np, 4));
+    panel_pair_key_kernel<<<ge, kSpmmThreads, 0, stream>>>(erow, s.colind, nnz, row_rank, prows, (int32_t)npanels, buf.key_a[0],
+                                                           buf.key_b[0], buf.payload[0]);
     CG_LAUNCH_CHECK();
-    const uint32_t maxcount = (uint32_t)(nnz < 0x7ffffffeLL ? nnz : 0x7ffffffeLL);
-    panel_count_key_kernel<<<gm, kSpmmThreads, 0, stream>>>(count, m, maxcount, buf.key_a[0], buf.payload[0]);
-    CG_LAUNCH_CHECK();
-    CG_TRY(fill_u32((uint32_t *)buf.key_b[0], m, 0u, stream));
     int set = 0;
-    CG_TRY(radix_sort_pairs(buf, m, bits_for((int32_t)maxcount + 1), 0, &set, stream));
-    panel_invert_kernel<<<gm, kSpmmThreads, 0, stream>>>(buf.payload[set], m, col_rank);
+    CG_TRY(radix_sort_pairs(buf, nnz, bits_for((int32_t)npanels + 1), bits_for(m), &set, stream));
+    const unsigned ge1 = (unsigned)ceil_div64(nnz + 1, kSpmmThreads);
+    panel_run_start_kernel<<<ge1, kSpmmThreads, 0, stream>>>(buf.key_a[set], buf.key_b[set], nnz, start);
     CG_LAUNCH_CHECK();
-    CG_HIP(hipMemcpyAsync(qcol, buf.payload[set], (size_t)hot * 4, hipMemcpyDeviceToDevice, stream));
+    CG_TRY(exclusive_scan_u32(start, runs_before, nnz + 1, d_np, stream));
+    uint32_t h_np = 0;
+    CG_HIP(hipMemcpyAsync(&h_np, d_np, 4, hipMemcpyDeviceToHost, stream));
+    CG_HIP(hipStreamSynchronize(stream));
+    npairs = h_np;
+    CG_TRY(t2.alloc((void **)&pair_first, (size_t)(npairs + 1) * 4));
+    CG_TRY(t2.alloc((void **)&pair_lr, (size_t)npairs * 4));
+    CG_TRY(tmp.alloc((void **)&pair_col, (size_t)npairs * 4));
+    CG_TRY(tmp.alloc((void **)&spanel, (size_t)npairs * 4));
+    CG_TRY(tmp.alloc((void **)&spair, (size_t)npairs * 4));
+    panel_run_first_kernel<<<ge1, kSpmmThreads, 0, stream>>>(start, runs_before, nnz, pair_first);
+    CG_LAUNCH_CHECK();
+    CG_TRY(fill_u32(pair_first + npairs, 1, (uint32_t)nnz, stream));
+    {
+      DevTemps t3;
+      SortBuffers pb;
+      CG_TRY(alloc_sort_buffers(t3, pb, npairs));
+      const unsigned gp = (unsigned)ceil_div64(npairs, kSpmmThreads);
+      panel_pair_count_key_kernel<<<gp, kSpmmThreads, 0, stream>>>(pair_first, npairs, buf.key_a[set], buf.key_b[set], pb.key_a[0],
+                                                                   pb.key_b[0], pb.payload[0], pair_col);
+      CG_LAUNCH_CHECK();
+      int pset = 0;
+      CG_TRY(radix_sort_pairs(pb, npairs, bits_for((int32_t)npanels + 1), 8, &pset, stream));
+      CG_TRY(launch_rowptr(pb.key_a[pset], npairs, (int32_t)npanels + 1, pstart, stream));
+      panel_pair_rank_kernel<<<gp, kSpmmThreads, 0, stream>>>(pb.key_a[pset], pb.payload[pset], npairs, pstart, (int32_t)npanels,
+                                                              hot, pair_lr);
+      CG_LAUNCH_CHECK();
+      CG_HIP(hipMemcpyAsync(spanel, pb.key_a[pset], (size_t)npairs * 4, hipMemcpyDeviceToDevice, stream));
+      CG_HIP(hipMemcpyAsync(spair, pb.payload[pset], (size_t)npairs * 4, hipMemcpyDeviceToDevice, stream));
+      CG_HIP(hipStreamSynchronize(stream));
+    }
+    panel_entry_rank_kernel<<<ge, kSpmmThreads, 0, stream>>>(start, runs_before, buf.payload[set], nnz, pair_lr, ecr);
+    CG_LAUNCH_CHECK();
     CG_HIP(hipStreamSynchronize(stream));
   }
 
   // 2. entries per tile; active tiles = those with emin .. dmin - 1 entries, dense tiles = those with more
-  int32_t *erow = nullptr;
   uint32_t *tcount = nullptr, *tindex = nullptr, *kept = nullptr, *dindex = nullptr, *dkept = nullptr, *d_tot = nullptr;
-  CG_TRY(tmp.alloc((void **)&erow, (size_t)nnz * 4));
   CG_TRY(tmp.alloc((void **)&tcount, (size_t)(tiles + 1) * 4));
   CG_TRY(tmp.alloc((void **)&tindex, (size_t)(tiles + 1) * 4));
   CG_TRY(tmp.alloc((void **)&kept, (size_t)(tiles + 1) * 4));
   CG_TRY(tmp.alloc((void **)&dindex, (size_t)(tiles + 1) * 4));
   CG_TRY(tmp.alloc((void **)&dkept, (size_t)(tiles + 1) * 4));
   CG_TRY(tmp.alloc((void **)&d_tot, 5 * 4));
-  panel_expand_rows_kernel<<<(unsigned)ceil_div64((int64_t)n * kWave, kSpmmThreads), kSpmmThreads, 0, stream>>>(s.rowptr, n, erow);
-  CG_LAUNCH_CHECK();
   CG_TRY(fill_u32(tcount, tiles + 1, 0u, stream));
   CG_TRY(fill_u32(d_tot, 5, 0u, stream));
-  panel_tile_count_kernel<<<ge, kSpmmThreads, 0, stream>>>(erow, s.colind, nnz, row_rank, col_rank, prows, hot, nkb, tcount);
+  panel_tile_count_kernel<<<ge, kSpmmThreads, 0, stream>>>(erow, ecr, nnz, row_rank, prows, hot, nkb, tcount);
   CG_LAUNCH_CHECK();
   panel_tile_select_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, tiles, (uint32_t)emin, (uint32_t)dmin, tindex, kept, dindex,
                                                            dkept);
@@ -148,24 +184,30 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     return decline();
   if (ntiles * kPanelWaves + 2 > 0x7fffffffLL || ndtiles * kDenseTileFloats > 0x7fffffffLL * 4) return decline();
 
-  // 3. tables of the active and of the dense tiles
-  int32_t *tile_panel = nullptr, *tile_kb = nullptr, *tile_wptr = nullptr, *dtile_panel = nullptr, *dtile_kb = nullptr;
-  CG_TRY(tmp.alloc((void **)&tile_kb, (size_t)(ntiles + 1) * 4));
+  // 3. tables of the active and of the dense tiles; the columns of their places
+  int32_t *tile_panel = nullptr, *tile_wptr = nullptr, *dtile_panel = nullptr;
   CG_TRY(tmp.alloc((void **)&tile_panel, (size_t)(ntiles + 1) * 4));
-  CG_TRY(tmp.alloc((void **)&dtile_kb, (size_t)(ndtiles + 1) * 4));
   CG_TRY(tmp.alloc((void **)&dtile_panel, (size_t)(ndtiles + 1) * 4));
-  panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, tindex, tiles, (uint32_t)emin, (uint32_t)dmin, 1, nkb, tile_kb,
-                                                           tile_panel);
+  panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, tindex, tiles, (uint32_t)emin, (uint32_t)dmin, 1, nkb, tile_panel);
   CG_LAUNCH_CHECK();
+  CG_TRY(dev_alloc((void **)&pp.hdr, (size_t)(ntiles > 0 ? ntiles : 1) * kPanelWaves * 16));
+  CG_TRY(fill_u32((uint32_t *)pp.hdr, ntiles * kPanelWaves * 4, 0xffffffffu, stream));
   if (ndtiles > 0) {
     panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, dindex, tiles, (uint32_t)emin, (uint32_t)dmin, 2, nkb,
-                                                             dtile_kb, dtile_panel);
+                                                             dtile_panel);
     CG_LAUNCH_CHECK();
     CG_TRY(dev_alloc((void **)&pp.dA, (size_t)ndtiles * kDenseTileFloats * 4));
     CG_TRY(dev_alloc((void **)&pp.dhdr, (size_t)ndtiles * kPanelCols * 4));
     CG_HIP(hipMemsetAsync(pp.dA, 0, (size_t)ndtiles * kDenseTileFloats * 4, stream));
-    panel_dense_hdr_kernel<<<(unsigned)ceil_div64(ndtiles * kPanelCols, kSpmmThreads), kSpmmThreads, 0, stream>>>(
-        dtile_kb, qcol, ndtiles, pp.dhdr);
+    CG_TRY(fill_u32((uint32_t *)pp.dhdr, ndtiles * kPanelCols, 0xffffffffu, stream));
+  }
+  panel_pair_hdr_kernel<<<(unsigned)ceil_div64(npairs, kSpmmThreads), kSpmmThreads, 0, stream>>>(
+      spanel, spair, npairs, pstart, (int32_t)npanels, hot, nkb, pair_col, tcount, tindex, dindex, (uint32_t)emin, (uint32_t)dmin,
+      pp.hdr, pp.dhdr);
+  CG_LAUNCH_CHECK();
+  if (ndtiles > 0) {
+    panel_dense_hdr_fill_kernel<<<(unsigned)ceil_div64(ndtiles * kPanelCols, kSpmmThreads), kSpmmThreads, 0, stream>>>(pp.dhdr,
+                                                                                                                     ndtiles);
     CG_LAUNCH_CHECK();
   }
 
@@ -183,7 +225,6 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   CG_TRY(dev_alloc((void **)&rest.colind, (size_t)nrest * 4));
   CG_TRY(dev_alloc((void **)&rest.val, (size_t)nrest * 4));
   CG_TRY(tmp.alloc((void **)&tile_wptr, (size_t)(ntiles * kPanelWaves + 1) * 4));
-  CG_TRY(dev_alloc((void **)&pp.hdr, (size_t)ntiles * kPanelWaves * 16));
   {
     DevTemps t2;
     SortBuffers buf;
@@ -191,7 +232,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     CG_TRY(alloc_sort_buffers(t2, buf, nnz));
     CG_TRY(t2.alloc((void **)&rest_row, (size_t)(nrest > 0 ? nrest : 1) * 4));
     const int32_t sentinel = (int32_t)(ntiles * kPanelWaves);
-    panel_entry_key_kernel<<<ge, kSpmmThreads, 0, stream>>>(erow, s.colind, s.val, nnz, row_rank, col_rank, prows, hot, nkb, tcount,
+    panel_entry_key_kernel<<<ge, kSpmmThreads, 0, stream>>>(erow, ecr, s.val, nnz, row_rank, prows, hot, nkb, tcount,
                                                             tindex, dindex, (uint32_t)emin, (uint32_t)dmin, sentinel,
                                                             buf.key_a[0], buf.key_b[0], buf.payload[0], (uint32_t *)pp.dA,
                                                             d_tot + 4);
@@ -202,7 +243,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     CG_TRY(t2.alloc((void **)&ent_raw, (size_t)(covered > 0 ? covered : 1) * 8));
     if (covered + nrest > 0) {
       panel_entry_finish_kernel<<<(unsigned)ceil_div64(covered + nrest, kSpmmThreads), kSpmmThreads, 0, stream>>>(
-          buf.key_b[set], buf.payload[set], covered + nrest, covered, erow, s.colind, s.val, col_rank, ent_raw, rest_row,
+          buf.key_b[set], buf.payload[set], covered + nrest, covered, erow, s.colind, s.val, ecr, ent_raw, rest_row,
           rest.colind, rest.val);
       CG_LAUNCH_CHECK();
     }
@@ -239,8 +280,8 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
       CG_LAUNCH_CHECK();
     }
     if (ntiles > 0) {
-      panel_hdr_kernel<<<(unsigned)ceil_div64(ntiles * kPanelWaves, kSpmmThreads), kSpmmThreads, 0, stream>>>(
-          tile_kb, tile_wptr, qcol, ntiles, (int4 *)pp.hdr);
+      panel_hdr_kernel<<<(unsigned)ceil_div64(ntiles * kPanelWaves, kSpmmThreads), kSpmmThreads, 0, stream>>>(tile_wptr, ntiles,
+                                                                                                              pp.hdr);
       CG_LAUNCH_CHECK();
     }
     CG_TRY(launch_rowptr(rest_row, nrest, n, rest.rowptr, stream));
