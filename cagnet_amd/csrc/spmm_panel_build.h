@@ -6,12 +6,13 @@
 namespace cg {
 
 constexpr int64_t kPanelMaxTiles = (int64_t)1 << 26;  // (panel, column block) pairs whose entries are counted
-constexpr double kPanelMinCoverage = 0.5;             // share of the entries the active tiles must hold: measured
-                                                      // 0.80 (232,965 vertices, 492 entries per row) 17.1 -> 12.6 ms,
-                                                      // 0.42 (R-MAT scale 20, 31 per row) 8.0 -> 9.0 ms at f = 602
+constexpr double kPanelMinCoverage = 0.5;             // share of the entries the tiles must hold: measured at f = 602
+                                                      // 0.88 (232,965 vertices, 492 entries per row) 17.1 -> 11.1 ms,
+                                                      // just over 0.5 (R-MAT scale 20, 31 per row) 8.1 -> 8.05 ms; with
+                                                      // 0.42 (the same matrix, columns ranked over the whole matrix) 8.0 -> 9.0
 constexpr int32_t kPanelDefaultEmin = 64;             // entries a 128 x 32 tile needs to be staged: twice the
                                                       // 32 gathers its staging costs
-constexpr int32_t kPanelDefaultCols = 131072;         // ranked columns that can be part of a tile
+constexpr int32_t kPanelDefaultCols = 131072;         // column ranks of a panel that can be part of a tile
 constexpr int32_t kPanelDefaultUnit = 65536;          // entries after which a panel's tiles start a new unit
 
 struct DevTemps {  // device temporaries of a plan build, freed when the build ends

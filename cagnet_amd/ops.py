@@ -345,7 +345,7 @@ class CsrMatrix:
         buf = (c_int64 * 12)()
         check(lib.cg_csr_panel_info(self._handle, int(transpose) | (2 if narrow else 0), buf), "cg_csr_panel_info")
         return {"state": buf[0], "staged_entries": buf[1], "staged_tiles": buf[2], "staged_units": buf[3],
-                "split_panels": buf[4], "rest_entries": buf[5], "tile_min_entries": buf[6], "ranked_columns": buf[7],
+                "split_panels": buf[4], "rest_entries": buf[5], "tile_min_entries": buf[6], "column_ranks": buf[7],
                 "dense_entries": buf[8], "dense_tiles": buf[9], "dense_units": buf[10], "dense_min_entries": buf[11]}
 
     def arrays(self, transpose: bool = False):

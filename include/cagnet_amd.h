@@ -204,7 +204,7 @@ int cg_csr_info(const cg_csr_t *h, int64_t info[8]);
  * { 1 in use / -1 declined (the tiles hold too few of the entries) / 0 none considered yet,
  *   entries multiplied out of LDS by the vector ALUs, their (active) tiles, their units (workgroups),
  *   row panels with several units of either kind, entries left to the row-wise kernels, entries a tile
- *   needs, ranked columns, entries in dense tiles (multiplied on the fp32 matrix cores), dense tiles, their
+ *   needs, column ranks per panel, entries in dense tiles (multiplied on the fp32 matrix cores), dense tiles, their
  *   units, entries from which a tile is dense (0: no dense tiles were allowed) }.  No counterpart in the
  * reference, which hands the whole product to cusparseSpMM (sparse-extension/sparse_coo_tensor.cu:215-226). */
 int cg_csr_panel_info(const cg_csr_t *h, int transpose, int64_t info[12]);
@@ -351,7 +351,7 @@ int cg_prof_enable(int on);
  *   "spmm_panel"      panel plan (dense row-panel x column-block tiles multiplied out of LDS; even widths
  *                     258..636): -1 never, 1 always, 0 when the tiles hold at least half of the entries
  *   "spmm_panel_emin" entries a 128 x 32 tile needs to be staged (0: 64)
- *   "spmm_panel_cols" ranked columns that can be part of a tile (0: 131072)
+ *   "spmm_panel_cols" column ranks inside a row panel that can be part of a tile (0: 131072)
  *   "spmm_panel_unit" entries after which the tiles of a row panel go to another workgroup (0: 65536)
  *   "spmm_panel_dmin" entries from which a 128 x 32 tile is stored whole and multiplied on the fp32 matrix
  *                     cores (0: 1024, a quarter full; negative: never).  Such a tile multiplies its zeros too:
