@@ -335,7 +335,7 @@ def extra_rmat20(dev, reps: int, traffic_table: dict) -> dict:
             "products": products}
 
 
-def extra_grid_row(prob, spec, dev, reps: int) -> dict:
+def extra_grid_row(prob, spec, dev, reps: int, traffic_table: dict) -> dict:
     """Configuration 4: the last process row of the 4 x 4 grid on the Reddit-shaped graph: four resident
     stages per product; the stage loop at f = 602 and forward + backward of both layers."""
     import torch
@@ -382,11 +382,12 @@ def extra_grid_row(prob, spec, dev, reps: int) -> dict:
             blocks[k].spmm(H[k], out=z, beta=0.0 if k == 0 else 1.0)
 
     ms_stage = median_ms(stages, reps)
+    traffic = traffic_of(traffic_table, "grid_row", feats, launched_spmm_kernels(stages, feats))
     alg = sum(spmm_alg_bytes(nz, rows, b[k + 1] - b[k], feats, reads_c=k > 0) for k, nz in enumerate(nnzs))
     return {"workload": "last process row of the 4 x 4 grid on the Reddit-shaped graph, four stages resident in HBM; "
                         "median of %d" % reps,
             "rows": rows, "block_cols": [b[k + 1] - b[k] for k in range(q)], "block_nnz": nnzs, "bound": "hbm",
-            "stage_loop_f%d" % feats: roofline_fields(alg, 2.0 * sum(nnzs) * feats, ms_stage),
+            "stage_loop_f%d" % feats: roofline_fields(alg, 2.0 * sum(nnzs) * feats, ms_stage, traffic),
             "fwd_bwd_both_layers_ms": round(ms_epoch, 4)}
 
 
@@ -590,7 +591,7 @@ def main() -> int:
 
     extras = not args.no_extra and args.workload == "reddit"
     if extras:
-        out["configs"] = {"cfg4_grid_row": extra_grid_row(prob, spec, dev, 5)}
+        out["configs"] = {"cfg4_grid_row": extra_grid_row(prob, spec, dev, 5, traffic_table)}
     prob_cpu = None
     if not args.no_cpu_baseline:
         prob_cpu = dict(n=n, row=prob.row.cpu(), col=prob.col.cpu(), val=prob.val.cpu(), x=prob.x.detach().cpu().contiguous(),

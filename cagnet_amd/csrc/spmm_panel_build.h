@@ -36,7 +36,10 @@ static bool want_panel(const CsrSide &s, int32_t f) {
   const int t = g_tune_panel.load(std::memory_order_relaxed);
   if (t < 0 || !panel_width_ok(f) || s.rows == 0 || s.nnz == 0) return false;
   if (t > 0) return true;
-  return s.nnz / s.rows >= 8 && (double)s.nnz * f >= 3e9;
+  // Below about 1e10 multiply-adds the plan's fixed costs (a block of partial rows per unit, a pipeline of lightly
+  // filled tiles, few units per compute unit) outweigh what it saves: blocks of a 4 x 4 grid over 232,965 vertices at
+  // f = 602, plan against row-wise kernels: 5.4 M entries 1.84 / 1.28 ms, 12.5 M 2.06 / 2.06 ms, 29.4 M 2.56 / 4.31 ms.
+  return s.nnz / s.rows >= 8 && (double)s.nnz * f >= 1e10;
 }
 
 static int alloc_sort_buffers(DevTemps &tmp, SortBuffers &buf, int64_t count) {

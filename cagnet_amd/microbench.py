@@ -166,7 +166,7 @@ def run_grid2d(args) -> None:
         loss.backward()
         x.grad = w1.grad = w2.grad = None
 
-    ms = _time(step, args.reps)
+    ms = float("nan") if args.stages_only else _time(step, args.reps)
     # the four accumulate-SpMMs of one stage loop at the input width
     H = [x.detach() if k == r else g1.forward[k] for k in range(q)]
     z = torch.empty(rows, feats, device=dev)
@@ -180,7 +180,8 @@ def run_grid2d(args) -> None:
     alg = sum(8 * nz + 4 * (rows + 1) + 4 * (b[k + 1] - b[k]) * feats + 4 * rows * feats * (1 if k == 0 else 2)
               for k, nz in enumerate(nnzs))
     print(json.dumps({"what": "grid2d rank share", "grid": f"{q}x{q}", "process_row": r, "rows": rows, "block_nnz": nnzs,
-                      "fwd_bwd_both_layers_ms": round(ms, 3), "stage_loop_f602_ms": round(ms_stage, 3),
+                      "fwd_bwd_both_layers_ms": None if args.stages_only else round(ms, 3),
+                      "stage_loop_f602_ms": round(ms_stage, 3), "stage_loops_run": args.reps + 1,
                       "stage_loop_gflops": round(flops / ms_stage / 1e6, 1),
                       "stage_loop_algorithmic_gbs": round(alg / ms_stage / 1e6, 1)}), flush=True)
 
@@ -232,6 +233,8 @@ def main() -> int:
     g.add_argument("--grid", type=int, default=4)
     g.add_argument("--row", type=int, default=1)
     g.add_argument("--reps", type=int, default=5)
+    g.add_argument("--stages-only", action="store_true",
+                   help="run the stage loop only (reps + 1 times): what a counter run of the stage loop profiles")
     pr = sub.add_parser("prep")
     pr.add_argument("--graph", default="reddit", choices=sorted(GRAPHS))
     pr.add_argument("--reps", type=int, default=3)

@@ -544,8 +544,8 @@ def test_spmm_hub_plan_is_declined_when_columns_are_not_skewed(cuda):
         tiers, panel = A.info()["plan_tiers"], _panel_info(A)["state"]
         if skewed:                                                     # one of the two plans takes the popular columns
             assert panel == 1 or tiers >= 1, (panel, tiers)
-        else:                                                          # both were looked at and declined
-            assert panel == -1 and tiers == -1, (panel, tiers)
+        else:                                                          # the hub plan was looked at and declined; the panel
+            assert panel in (0, -1) and tiers == -1, (panel, tiers)    # plan likewise, or not considered at this size
         keep = torch.isin(r, sample)
         ref_rows = torch.unique(r[keep])
         remap = torch.full((n,), -1, dtype=torch.long)
