@@ -68,7 +68,8 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     pp.valid = true;
     return CG_OK;
   };
-  const int32_t hot = (hot_req < m ? hot_req : m) / kPanelCols * kPanelCols;
+  // column ranks of a panel that can be part of a tile: whole blocks; a panel's last block may be partly empty
+  const int32_t hot = (int32_t)(ceil_div64(hot_req < m ? hot_req : m, kPanelCols) * kPanelCols);
   if (hot < kPanelCols || n < 1 || nnz < 1) return decline();
   const int32_t nkb = hot / kPanelCols;
   int64_t npanels = ceil_div64(n, kPanelRows);

@@ -981,6 +981,46 @@ def test_spmm_panel_all_tiles_dense_and_duplicate_entries(cuda, tune):
     assert spmm_error(got, r, c, v, 256, 64, Bd.cpu()) <= REL_TOL
 
 
+def test_spmm_panel_last_block_with_empty_places_and_columns_ranked_per_panel(cuda, tune):
+    """Columns are ranked inside every panel, so a panel's last block can have fewer than 32 columns: 40 columns give
+    one full block and one of 8, as a dense tile (1024 entries) and, with dense tiles off, as a staged one (the empty
+    places name a column of the tile).  Second matrix: two panels whose busy columns interleave (the even columns
+    0..62 in the first 128 rows, the odd columns 1..63 in the next 128, one stray entry per row elsewhere): each panel
+    gets one full tile of its own 32 busy columns, where blocks of one ranking for the whole matrix would have given
+    each panel two half-filled ones, and only the stray entries stay in the rest matrix."""
+    from cagnet_amd import ops
+    n, m, f = 128, 40, 300
+    g = torch.Generator().manual_seed(12)
+    dense = torch.randn(n, m, generator=g)
+    row, col = torch.nonzero(torch.ones(n, m), as_tuple=True)
+    val = dense[row, col].contiguous()
+    B = torch.randn(m, f, generator=g)
+    Bd = B.to(cuda)
+    tune("spmm_panel", 1)
+    for dmin, kind in ((0, "dense_tiles"), (-1, "tiles")):
+        tune("spmm_panel_dmin", dmin)
+        A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, m)
+        got = A.spmm(Bd)
+        info = _panel_info(A)
+        assert info["state"] == 1 and info[kind] == 2 and info["rest"] == 0, info
+        assert gemm_error(got, dense, B) <= REL_TOL
+    tune("spmm_panel_dmin", -1)
+    n, m = 256, 2000
+    rng = np.random.default_rng(21)
+    r = np.repeat(np.arange(n), 32)
+    c = 2 * np.tile(np.arange(32), n) + np.where(r < 128, 0, 1)
+    stray_c = 100 + rng.permutation(800)[:n]                            # one more entry per row, all in different columns
+    key = np.unique(np.concatenate([r * m + c, np.arange(n) * m + stray_c]))
+    row, col = torch.from_numpy(key // m), torch.from_numpy(key % m)
+    val = torch.from_numpy(rng.standard_normal(key.size).astype(np.float32))
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, m)
+    Bd = torch.randn(m, f, generator=g).to(cuda)
+    got = A.spmm(Bd)
+    info = _panel_info(A)
+    assert info["state"] == 1 and info["tiles"] == 2 and info["covered"] == n * 32 and info["rest"] == n, info
+    assert spmm_error(got, row, col, val, n, m, Bd.cpu()) <= REL_TOL
+
+
 def test_spmm_panel_plan_rectangular_strided_and_declined(cuda, tune):
     """A non-symmetric rectangular matrix, B and C as column slices of wider matrices, rows without any
     entry; and a matrix without dense tiles, on which the automatic choice declines the plan."""
