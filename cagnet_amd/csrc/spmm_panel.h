@@ -496,15 +496,6 @@ __device__ __forceinline__ int panel_tile_kind(uint32_t count, uint32_t emin, ui
   return count >= emin ? 1 : 0;
 }
 
-__global__ __launch_bounds__(kSpmmThreads) void panel_tile_count_kernel(
-    const int32_t *__restrict__ erow, const int32_t *__restrict__ ecr, int64_t nnz, const int32_t *__restrict__ row_rank,
-    int32_t prows, int32_t hot, int32_t nkb, uint32_t *__restrict__ tcount) {
-  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
-  if (k >= nnz) return;
-  const int64_t t = panel_tile_of(row_rank[erow[k]], ecr[k], prows, hot, nkb);
-  if (t >= 0) atomicAdd(&tcount[t], 1u);
-}
-
 // Column ranks inside the panels.  The entries are sorted by (panel, column); a run of equal keys is a
 // (panel, column) pair, and the pairs of a panel are ranked by descending length (ties: by column).
 // Entries of rows behind the ranked panels get the panel number `npanels`, which sorts them last.
@@ -537,20 +528,27 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_pair_count_key_kernel(
 }
 
 // pair_lr[pair] = rank of the pair's column inside its panel, `hot` for ranks from `hot` on and for the rows
-// behind the panels (hot = the ranks that can be part of a tile)
+// behind the panels (hot = the ranks that can be part of a tile); the pair's entries are counted into its tile
+// (integer counts: order independent)
 __global__ __launch_bounds__(kSpmmThreads) void panel_pair_rank_kernel(const int32_t *__restrict__ spanel,
                                                                        const int32_t *__restrict__ spair, int64_t npairs,
                                                                        const int32_t *__restrict__ pstart, int32_t npanels,
-                                                                       int32_t hot, int32_t *__restrict__ pair_lr) {
+                                                                       int32_t hot, int32_t nkb,
+                                                                       const uint32_t *__restrict__ pair_first,
+                                                                       int32_t *__restrict__ pair_lr,
+                                                                       uint32_t *__restrict__ tcount) {
   const int64_t j = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (j >= npairs) return;
-  const int32_t panel = spanel[j];
+  const int32_t panel = spanel[j], pair = spair[j];
   int64_t lr = hot;
   if (panel < npanels) {
     lr = j - pstart[panel];
-    if (lr > hot) lr = hot;
+    if (lr >= hot)
+      lr = hot;
+    else
+      atomicAdd(&tcount[(int64_t)panel * nkb + lr / kPanelCols], pair_first[pair + 1] - pair_first[pair]);
   }
-  pair_lr[spair[j]] = (int32_t)lr;
+  pair_lr[pair] = (int32_t)lr;
 }
 
 // ecr[entry] = rank of the entry's column inside the entry's panel (start / runs_before: the run starts of the

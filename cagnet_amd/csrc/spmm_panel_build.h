@@ -102,7 +102,10 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   //     the runs of that order (= pairs) sorted by (panel, descending length).  ecr[entry] = rank of its column
   //     in its panel; the sorted pairs stay for the tile headers.
   int32_t *erow = nullptr, *ecr = nullptr, *pstart = nullptr, *pair_col = nullptr, *spanel = nullptr, *spair = nullptr;
+  uint32_t *tcount = nullptr;  // entries per (panel, block) tile
   int64_t npairs = 0;
+  CG_TRY(tmp.alloc((void **)&tcount, (size_t)(tiles + 1) * 4));
+  CG_TRY(fill_u32(tcount, tiles + 1, 0u, stream));
   CG_TRY(tmp.alloc((void **)&erow, (size_t)nnz * 4));
   CG_TRY(tmp.alloc((void **)&ecr, (size_t)nnz * 4));
   CG_TRY(tmp.alloc((void **)&pstart, (size_t)(npanels + 2) * 4));
@@ -150,7 +153,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
       CG_TRY(radix_sort_pairs(pb, npairs, bits_for((int32_t)npanels + 1), 8, &pset, stream));
       CG_TRY(launch_rowptr(pb.key_a[pset], npairs, (int32_t)npanels + 1, pstart, stream));
       panel_pair_rank_kernel<<<gp, kSpmmThreads, 0, stream>>>(pb.key_a[pset], pb.payload[pset], npairs, pstart, (int32_t)npanels,
-                                                              hot, pair_lr);
+                                                              hot, nkb, pair_first, pair_lr, tcount);
       CG_LAUNCH_CHECK();
       CG_HIP(hipMemcpyAsync(spanel, pb.key_a[pset], (size_t)npairs * 4, hipMemcpyDeviceToDevice, stream));
       CG_HIP(hipMemcpyAsync(spair, pb.payload[pset], (size_t)npairs * 4, hipMemcpyDeviceToDevice, stream));
@@ -161,18 +164,14 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     CG_HIP(hipStreamSynchronize(stream));
   }
 
-  // 2. entries per tile; active tiles = those with emin .. dmin - 1 entries, dense tiles = those with more
-  uint32_t *tcount = nullptr, *tindex = nullptr, *kept = nullptr, *dindex = nullptr, *dkept = nullptr, *d_tot = nullptr;
-  CG_TRY(tmp.alloc((void **)&tcount, (size_t)(tiles + 1) * 4));
+  // 2. active tiles = those with emin .. dmin - 1 entries, dense tiles = those with more
+  uint32_t *tindex = nullptr, *kept = nullptr, *dindex = nullptr, *dkept = nullptr, *d_tot = nullptr;
   CG_TRY(tmp.alloc((void **)&tindex, (size_t)(tiles + 1) * 4));
   CG_TRY(tmp.alloc((void **)&kept, (size_t)(tiles + 1) * 4));
   CG_TRY(tmp.alloc((void **)&dindex, (size_t)(tiles + 1) * 4));
   CG_TRY(tmp.alloc((void **)&dkept, (size_t)(tiles + 1) * 4));
   CG_TRY(tmp.alloc((void **)&d_tot, 5 * 4));
-  CG_TRY(fill_u32(tcount, tiles + 1, 0u, stream));
   CG_TRY(fill_u32(d_tot, 5, 0u, stream));
-  panel_tile_count_kernel<<<ge, kSpmmThreads, 0, stream>>>(erow, ecr, nnz, row_rank, prows, hot, nkb, tcount);
-  CG_LAUNCH_CHECK();
   panel_tile_select_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, tiles, (uint32_t)emin, (uint32_t)dmin, tindex, kept, dindex,
                                                            dkept);
   CG_LAUNCH_CHECK();
