@@ -15,8 +15,8 @@ namespace cg {
 
 constexpr int32_t kPanelNarrowMaxF = 64;
 constexpr int32_t kPanelNarrowDmin = 512;        // entries from which a tile is stored whole for narrow products: measured at
-                                                 // 232,965 vertices, 492 entries per row: f = 16 0.86 -> 0.71 ms, f = 44 1.82 -> 1.54,
-                                                 // f = 64 1.83 -> 1.40; 384 the same within 1 %, 256 and 1024 slower
+                                                 // 232,965 vertices, 492 entries per row: f = 16 0.88 -> 0.70 ms, f = 44 1.83 -> 1.53,
+                                                 // f = 64 1.84 -> 1.42; 384 .. 448 the same within 2.5 %, 192, 256 and 768 slower
 constexpr double kPanelNarrowMinCoverage = 0.25;  // share of the entries the dense tiles must hold
 
 static std::atomic<int> g_tune_panel_narrow{0}, g_tune_panel_narrow_dmin{0};
