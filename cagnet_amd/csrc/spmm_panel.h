@@ -38,7 +38,7 @@ constexpr int kDenseThreads = kDenseWaves * kWave;
 constexpr int kDenseTileFloats = kPanelRows * kPanelCols;
 
 static std::atomic<int> g_tune_panel{0}, g_tune_panel_emin{0}, g_tune_panel_cols{0}, g_tune_panel_unit{0};
-static std::atomic<int> g_tune_panel_dmin{0}, g_tune_panel_dwg{0};
+static std::atomic<int> g_tune_panel_dmin{0}, g_tune_panel_dwg{0}, g_tune_panel_share{0};
 
 struct CsrSide;
 
@@ -514,17 +514,22 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_pair_key_kernel(const int3
 
 // sort keys of the pairs: (panel, 255 - min(entries, 255)), payload the pair's number; pair_col[pair] = its column.
 // pair_first[npairs] = number of entries.
+// With col_rank (the columns' ranks by entry count over the whole matrix) the minor key is that rank for the pairs
+// with at least cmin entries and m + rank for the others: a panel's blocks then hold the columns that are worth
+// staging in the same order in every panel, so that workgroups on different panels walk the rows of B alike.
 __global__ __launch_bounds__(kSpmmThreads) void panel_pair_count_key_kernel(
     const uint32_t *__restrict__ pair_first, int64_t npairs, const int32_t *__restrict__ kpanel_sorted,
-    const int32_t *__restrict__ kcol_sorted, int32_t *__restrict__ pk_panel, int32_t *__restrict__ pk_count,
-    int32_t *__restrict__ pk_pair, int32_t *__restrict__ pair_col) {
+    const int32_t *__restrict__ kcol_sorted, const int32_t *__restrict__ col_rank, uint32_t cmin, int32_t m,
+    int32_t *__restrict__ pk_panel, int32_t *__restrict__ pk_count, int32_t *__restrict__ pk_pair,
+    int32_t *__restrict__ pair_col) {
   const int64_t p = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (p >= npairs) return;
   const uint32_t first = pair_first[p], count = pair_first[p + 1] - first;
+  const int32_t col = kcol_sorted[first];
   pk_panel[p] = kpanel_sorted[first];
-  pk_count[p] = 255 - (int32_t)(count < 255u ? count : 255u);
+  pk_count[p] = col_rank ? col_rank[col] + (count >= cmin ? 0 : m) : 255 - (int32_t)(count < 255u ? count : 255u);
   pk_pair[p] = (int32_t)p;
-  pair_col[p] = kcol_sorted[first];
+  pair_col[p] = col;
 }
 
 // pair_lr[pair] = rank of the pair's column inside its panel, `hot` for ranks from `hot` on and for the rows
@@ -612,14 +617,16 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_tile_select_kernel(const u
   dkept[t] = kind == 2 ? tcount[t] : 0u;
 }
 
-// panel of every tile of one kind (1: active, 2: dense), in the compacted numbering
+// panel (and block number inside it) of every tile of one kind (1: active, 2: dense), in the compacted numbering
 __global__ __launch_bounds__(kSpmmThreads) void panel_tile_tables_kernel(const uint32_t *__restrict__ tcount,
                                                                          const uint32_t *__restrict__ tindex, int64_t tiles,
                                                                          uint32_t emin, uint32_t dmin, int kind, int32_t nkb,
-                                                                         int32_t *__restrict__ tile_panel) {
+                                                                         int32_t *__restrict__ tile_panel,
+                                                                         int32_t *__restrict__ tile_kb) {
   const int64_t t = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (t >= tiles || panel_tile_kind(tcount[t], emin, dmin) != kind) return;
   tile_panel[tindex[t]] = (int32_t)(t / nkb);
+  if (tile_kb) tile_kb[tindex[t]] = (int32_t)(t % nkb);
 }
 
 // sort keys: entries of active tiles get (active tile * 16 + wave) as major and the slot as minor key, entries of

@@ -98,6 +98,32 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     CG_HIP(hipStreamSynchronize(stream));
   }
 
+  // 1a. columns ranked by their entries in the whole matrix (ties: by index): the order of a panel's columns that are
+  //     worth staging
+  const bool share = g_tune_panel_share.load(std::memory_order_relaxed) >= 0 && m < (1 << 30);
+  int32_t *col_rank = nullptr;
+  if (share) {
+    DevTemps t2;
+    SortBuffers buf;
+    uint32_t *count = nullptr;
+    CG_TRY(tmp.alloc((void **)&col_rank, (size_t)m * 4));
+    CG_TRY(t2.alloc((void **)&count, (size_t)m * 4));
+    CG_TRY(alloc_sort_buffers(t2, buf, m));
+    CG_TRY(fill_u32(count, m, 0u, stream));
+    panel_col_count_kernel<<<ge, kSpmmThreads, 0, stream>>>(s.colind, nnz, count);
+    CG_LAUNCH_CHECK();
+    const uint32_t maxcount = (uint32_t)(nnz < 0x7ffffffeLL ? nnz : 0x7ffffffeLL);
+    const unsigned gm = (unsigned)ceil_div64(m, kSpmmThreads);
+    panel_count_key_kernel<<<gm, kSpmmThreads, 0, stream>>>(count, m, maxcount, buf.key_a[0], buf.payload[0]);
+    CG_LAUNCH_CHECK();
+    CG_TRY(fill_u32((uint32_t *)buf.key_b[0], m, 0u, stream));
+    int set = 0;
+    CG_TRY(radix_sort_pairs(buf, m, bits_for((int32_t)maxcount + 1), 0, &set, stream));
+    panel_invert_kernel<<<gm, kSpmmThreads, 0, stream>>>(buf.payload[set], m, col_rank);
+    CG_LAUNCH_CHECK();
+    CG_HIP(hipStreamSynchronize(stream));
+  }
+
   // 1b. columns ranked inside every panel by the entries they have there: the entries sorted by (panel, column),
   //     the runs of that order (= pairs) sorted by (panel, descending length).  ecr[entry] = rank of its column
   //     in its panel; the sorted pairs stay for the tile headers.
@@ -146,11 +172,12 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
       SortBuffers pb;
       CG_TRY(alloc_sort_buffers(t3, pb, npairs));
       const unsigned gp = (unsigned)ceil_div64(npairs, kSpmmThreads);
-      panel_pair_count_key_kernel<<<gp, kSpmmThreads, 0, stream>>>(pair_first, npairs, buf.key_a[set], buf.key_b[set], pb.key_a[0],
-                                                                   pb.key_b[0], pb.payload[0], pair_col);
+      const uint32_t cmin = (uint32_t)((emin + kPanelCols - 1) / kPanelCols);  // a block of such columns reaches emin
+      panel_pair_count_key_kernel<<<gp, kSpmmThreads, 0, stream>>>(pair_first, npairs, buf.key_a[set], buf.key_b[set], col_rank, cmin,
+                                                                   m, pb.key_a[0], pb.key_b[0], pb.payload[0], pair_col);
       CG_LAUNCH_CHECK();
       int pset = 0;
-      CG_TRY(radix_sort_pairs(pb, npairs, bits_for((int32_t)npanels + 1), 8, &pset, stream));
+      CG_TRY(radix_sort_pairs(pb, npairs, bits_for((int32_t)npanels + 1), share ? bits_for(2 * m) : 8, &pset, stream));
       CG_TRY(launch_rowptr(pb.key_a[pset], npairs, (int32_t)npanels + 1, pstart, stream));
       panel_pair_rank_kernel<<<gp, kSpmmThreads, 0, stream>>>(pb.key_a[pset], pb.payload[pset], npairs, pstart, (int32_t)npanels,
                                                               hot, nkb, pair_first, pair_lr, tcount);
@@ -189,16 +216,18 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   if (ntiles * kPanelWaves + 2 > 0x7fffffffLL || ndtiles * kDenseTileFloats > 0x7fffffffLL * 4) return decline();
 
   // 3. tables of the active and of the dense tiles; the columns of their places
-  int32_t *tile_panel = nullptr, *tile_wptr = nullptr, *dtile_panel = nullptr;
+  int32_t *tile_panel = nullptr, *tile_kb = nullptr, *tile_wptr = nullptr, *dtile_panel = nullptr;
   CG_TRY(tmp.alloc((void **)&tile_panel, (size_t)(ntiles + 1) * 4));
+  CG_TRY(tmp.alloc((void **)&tile_kb, (size_t)(ntiles + 1) * 4));
   CG_TRY(tmp.alloc((void **)&dtile_panel, (size_t)(ndtiles + 1) * 4));
-  panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, tindex, tiles, (uint32_t)emin, (uint32_t)dmin, 1, nkb, tile_panel);
+  panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, tindex, tiles, (uint32_t)emin, (uint32_t)dmin, 1, nkb, tile_panel,
+                                                           tile_kb);
   CG_LAUNCH_CHECK();
   CG_TRY(dev_alloc((void **)&pp.hdr, (size_t)(ntiles > 0 ? ntiles : 1) * kPanelWaves * 16));
   CG_TRY(fill_u32((uint32_t *)pp.hdr, ntiles * kPanelWaves * 4, 0xffffffffu, stream));
   if (ndtiles > 0) {
     panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, dindex, tiles, (uint32_t)emin, (uint32_t)dmin, 2, nkb,
-                                                             dtile_panel);
+                                                             dtile_panel, nullptr);
     CG_LAUNCH_CHECK();
     CG_TRY(dev_alloc((void **)&pp.dA, (size_t)ndtiles * kDenseTileFloats * 4));
     CG_TRY(dev_alloc((void **)&pp.dhdr, (size_t)ndtiles * kPanelCols * 4));
@@ -301,12 +330,13 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   // 5. units: runs of tiles of one panel and one kind, with about unit_entries entries (active tiles) or inside one
   //    workgroup's share (dense tiles); each unit writes one block of 128 partial rows, the blocks of a panel are
   //    consecutive
-  std::vector<int32_t> h_panel((size_t)ntiles), h_base((size_t)ntiles + 1, 0), h_dpanel((size_t)ndtiles);
+  std::vector<int32_t> h_panel((size_t)ntiles), h_kb((size_t)ntiles), h_base((size_t)ntiles + 1, 0), h_dpanel((size_t)ndtiles);
   {
     // entries of active tile k: tile_wptr[16 k] is its first record
     std::vector<int32_t> h_wptr((size_t)ntiles * kPanelWaves + 1);
     CG_HIP(hipMemcpyAsync(h_wptr.data(), tile_wptr, h_wptr.size() * 4, hipMemcpyDeviceToHost, stream));
     if (ntiles > 0) CG_HIP(hipMemcpyAsync(h_panel.data(), tile_panel, (size_t)ntiles * 4, hipMemcpyDeviceToHost, stream));
+    if (ntiles > 0) CG_HIP(hipMemcpyAsync(h_kb.data(), tile_kb, (size_t)ntiles * 4, hipMemcpyDeviceToHost, stream));
     if (ndtiles > 0) CG_HIP(hipMemcpyAsync(h_dpanel.data(), dtile_panel, (size_t)ndtiles * 4, hipMemcpyDeviceToHost, stream));
     CG_HIP(hipStreamSynchronize(stream));
     for (int64_t k = 0; k <= ntiles; ++k) h_base[(size_t)k] = h_wptr[(size_t)k * kPanelWaves];
@@ -316,11 +346,17 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     int64_t weight;
   };
   std::vector<Unit> su, du;  // units of active tiles, of dense tiles; both in panel order
+  constexpr int32_t kUnitGrid = 32;  // with shared column order a unit starts where a panel's block number passes a multiple
+  constexpr int32_t kXcds = 8;       // XCDs of the device: workgroup i of a launch runs on XCD i % 8
   for (int64_t k = 0; k < ntiles;) {
     int64_t j = k, in_unit = 0;
     while (j < ntiles && h_panel[(size_t)j] == h_panel[(size_t)k]) {
       const int64_t e = (int64_t)h_base[(size_t)j + 1] - h_base[(size_t)j];
-      if (j > k && in_unit + e > unit_entries) break;
+      if (share) {
+        if (j > k && in_unit >= unit_entries / 2 && h_kb[(size_t)j] / kUnitGrid != h_kb[(size_t)j - 1] / kUnitGrid) break;
+      } else if (j > k && in_unit + e > unit_entries) {
+        break;
+      }
       in_unit += e;
       ++j;
     }
@@ -358,7 +394,42 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   for (int32_t u = 0; u < ndunits; ++u) dunit_tile[(size_t)u + 1] = du[(size_t)u].t1;
   std::vector<int32_t> order((size_t)nunits);
   for (int32_t u = 0; u < nunits; ++u) order[(size_t)u] = u;
-  std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return su[(size_t)a].weight > su[(size_t)b].weight; });
+  if (!share) {
+    std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return su[(size_t)a].weight > su[(size_t)b].weight; });
+  } else {
+    // Units that start at the same block number in neighbouring panels walk nearly the same rows of B: groups of as
+    // many of them as an XCD has compute units are launched on one XCD together (workgroup i runs on XCD i % 8), heaviest
+    // group first, so that one copy from memory serves the whole group out of that XCD's L2.
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        cus < kXcds) {
+      (void)hipGetLastError();
+      cus = 256;
+    }
+    const int32_t gsize = cus / kXcds;
+    std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) {
+      const int32_t ka = h_kb[(size_t)su[(size_t)a].t0] / kUnitGrid, kb = h_kb[(size_t)su[(size_t)b].t0] / kUnitGrid;
+      return ka != kb ? ka < kb : su[(size_t)a].panel < su[(size_t)b].panel;
+    });
+    const int32_t ngroups = (nunits + gsize - 1) / gsize;
+    std::vector<int64_t> gweight((size_t)ngroups, 0);
+    for (int32_t i = 0; i < nunits; ++i) gweight[(size_t)(i / gsize)] += su[(size_t)order[(size_t)i]].weight;
+    std::vector<int32_t> gorder((size_t)ngroups);
+    for (int32_t g = 0; g < ngroups; ++g) gorder[(size_t)g] = g;
+    std::stable_sort(gorder.begin(), gorder.end(), [&](int32_t a, int32_t b) { return gweight[(size_t)a] > gweight[(size_t)b]; });
+    // launch position of member j of the g-th heaviest group: round g / 8, XCD g % 8
+    std::vector<int32_t> placed((size_t)((ngroups + kXcds - 1) / kXcds) * kXcds * gsize, -1);
+    for (int32_t g = 0; g < ngroups; ++g)
+      for (int32_t j = 0; j < gsize; ++j) {
+        const int32_t i = gorder[(size_t)g] * gsize + j;
+        if (i < nunits) placed[(size_t)(g / kXcds) * kXcds * gsize + (size_t)j * kXcds + (size_t)(g % kXcds)] = order[(size_t)i];
+      }
+    int32_t at = 0;
+    std::vector<int32_t> compact((size_t)nunits);
+    for (int32_t v : placed)
+      if (v >= 0) compact[(size_t)at++] = v;
+    order.swap(compact);
+  }
   int32_t *d_panel_unit = nullptr;
   CG_TRY(tmp.alloc((void **)&d_panel_unit, (size_t)npanels * 4));
   CG_TRY(dev_alloc((void **)&pp.unit_tile, (size_t)(nunits + 1) * 4));
