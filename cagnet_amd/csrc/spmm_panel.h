@@ -45,6 +45,7 @@ struct CsrSide;
 struct PanelPlan {
   bool valid = false, declined = false, failed = false;  // failed: declined because the build ran out of memory
   int32_t emin = 0, hot_cols = 0, unit_entries = 0, dmin = 0, dwg = 0;  // what the plan was built with
+  bool share = true;
   int64_t covered = 0;      // entries the panel kernel multiplies
   int64_t dcovered = 0;     // entries in dense tiles (the matrix-core kernel)
   int32_t ntiles = 0, nunits = 0, nsplit = 0;

@@ -58,7 +58,8 @@ constexpr int32_t kPanelDefaultDmin = 1024;            // entries from which a 1
 // *collision: two entries of one (row, column) pair fell into a dense tile; the plan is unusable.
 // dwg: workgroups of the dense-tile kernel (each takes an equal share of the dense tiles).
 static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot_req, int32_t unit_entries, int32_t dmin,
-                            int32_t dwg, bool may_decline, double min_coverage, bool *collision, hipStream_t stream) {
+                            int32_t dwg, bool share_order, bool may_decline, double min_coverage, bool *collision,
+                            hipStream_t stream) {
   *collision = false;
   const int64_t nnz = s.nnz;
   const int32_t n = s.rows, m = s.cols;
@@ -100,7 +101,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
 
   // 1a. columns ranked by their entries in the whole matrix (ties: by index): the order of a panel's columns that are
   //     worth staging
-  const bool share = g_tune_panel_share.load(std::memory_order_relaxed) >= 0 && m < (1 << 30);
+  const bool share = share_order && m < (1 << 30);
   int32_t *col_rank = nullptr;
   if (share) {
     DevTemps t2;
@@ -472,8 +473,10 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
 
 struct PanelParams {
   int32_t emin, cols, unit, dmin, dwg;
+  bool share;  // staged columns in the whole matrix's order, units launched in XCD groups
   bool same(const PanelPlan &pp) const {
-    return pp.emin == emin && pp.hot_cols == cols && pp.unit_entries == unit && pp.dmin == dmin && pp.dwg == dwg;
+    return pp.emin == emin && pp.hot_cols == cols && pp.unit_entries == unit && pp.dmin == dmin && pp.dwg == dwg &&
+           pp.share == share;
   }
   void stamp(PanelPlan &pp) const {
     pp.emin = emin;
@@ -481,6 +484,7 @@ struct PanelParams {
     pp.unit_entries = unit;
     pp.dmin = dmin;
     pp.dwg = dwg;
+    pp.share = share;
   }
 };
 
@@ -505,6 +509,7 @@ static PanelParams panel_params() {
     }
     p.dwg = 4 * cus;
   }
+  p.share = g_tune_panel_share.load(std::memory_order_relaxed) >= 0;
   return p;
 }
 
@@ -515,11 +520,11 @@ static int build_panel(CsrSide &s, PanelPlan &pp, const PanelParams &par, bool m
   CG_HIP(hipStreamSynchronize(stream));
   pp.release();
   bool collision = false;
-  int st = build_panel_once(s, pp, par.emin, par.cols, par.unit, par.dmin, par.dwg, may_decline, min_coverage, &collision,
+  int st = build_panel_once(s, pp, par.emin, par.cols, par.unit, par.dmin, par.dwg, par.share, may_decline, min_coverage, &collision,
                             stream);
   if (st == CG_OK && collision) {  // the matrix stores a (row, column) pair twice: every tile goes the record way
     pp.release();
-    st = build_panel_once(s, pp, par.emin, par.cols, par.unit, 0, par.dwg, may_decline, min_coverage, &collision, stream);
+    st = build_panel_once(s, pp, par.emin, par.cols, par.unit, 0, par.dwg, par.share, may_decline, min_coverage, &collision, stream);
   }
   if (st != CG_OK) pp.release();
   par.stamp(pp);

@@ -91,7 +91,7 @@ def test_spmm_schedules_random(cuda, knobs_restored, seed):
 
 
 PANEL_KNOBS = [b"spmm_panel", b"spmm_panel_emin", b"spmm_panel_cols", b"spmm_panel_unit", b"spmm_panel_dmin", b"spmm_panel_dwg",
-               b"spmm_panel_narrow", b"spmm_panel_narrow_dmin"]
+               b"spmm_panel_narrow", b"spmm_panel_narrow_dmin", b"spmm_panel_share"]
 
 
 @pytest.mark.parametrize("seed", [31, 32])
@@ -99,8 +99,8 @@ def test_spmm_panel_plan_random(cuda, knobs_restored, seed):
     """The panel plan forced on over random patterns (skewed and uniform, with full rows and columns, rectangular),
     every even width class it is built for and the narrow widths (dense tiles only), both sides, accumulate forms,
     padded leading dimensions, and random plan knobs: entries a tile needs, ranked columns, unit size, dense-tile
-    threshold (off, low, high) and the number of workgroups that share the dense tiles.  Every entry is in exactly one
-    of the parts of the plan."""
+    threshold (off, low, high), the number of workgroups that share the dense tiles and the order of a panel's
+    columns (the whole matrix's, or the panel's own).  Every entry is in exactly one of the parts of the plan."""
     import ctypes
     from cagnet_amd import ops
     from cagnet_amd._lib import check
@@ -128,7 +128,8 @@ def test_spmm_panel_plan_random(cuda, knobs_restored, seed):
             f = rng.choice([258, 260, 300, 320, 322, 384, 448, 450, 512, 576, 602, 636, 1, 3, 16, 17, 41, 44, 63, 64])
             narrow = f <= 64
             values = [1, rng.choice([1, 4, 16, 64]), rng.choice([0, 32, 64, 1024]), rng.choice([0, 50, 2000]),
-                      rng.choice([-1, 0, 8, 40, 200, 3000]), rng.choice([0, 1, 5, 300]), 1, rng.choice([0, 4, 30, 500])]
+                      rng.choice([-1, 0, 8, 40, 200, 3000]), rng.choice([0, 1, 5, 300]), 1, rng.choice([0, 4, 30, 500]),
+                      rng.choice([0, 0, -1])]
             for key, v in zip(PANEL_KNOBS, values):
                 assert lib.cg_tune_set(key, v) == 0
             tr = rng.random() < 0.4
