@@ -6,10 +6,10 @@
 namespace cg {
 
 constexpr int64_t kPanelMaxTiles = (int64_t)1 << 26;  // (panel, column block) pairs whose entries are counted
-constexpr double kPanelMinCoverage = 0.5;             // share of the entries the tiles must hold: measured at f = 602
+constexpr double kPanelMinCoverage = 0.6;             // share of the entries the tiles must hold: measured at f = 602
                                                       // 0.88 (232,965 vertices, 492 entries per row) 17.1 -> 11.1 ms,
-                                                      // just over 0.5 (R-MAT scale 20, 31 per row) 8.1 -> 8.05 ms; with
-                                                      // 0.42 (the same matrix, columns ranked over the whole matrix) 8.0 -> 9.0
+                                                      // 0.54 (R-MAT scale 20, 31 per row) 7.76 -> 8.25 ms (7.96 with
+                                                      // spmm_panel_share = -1), although the traffic falls from 56.9 to 46.8 GB
 constexpr int32_t kPanelDefaultEmin = 64;             // entries a 128 x 32 tile needs to be staged: twice the
                                                       // 32 gathers its staging costs
 constexpr int32_t kPanelDefaultCols = 131072;         // column ranks of a panel that can be part of a tile

@@ -350,7 +350,7 @@ int cg_prof_enable(int on);
  *   "spmm_hub_row"    rows with fewer entries keep all of them in the cold class (0: 64)
  *   "spmm_panel"      panel plan (dense row-panel x column-block tiles multiplied out of LDS; even widths
  *                     258..636): -1 never, 1 always, 0 when the product has at least 1e10 multiply-adds, rows hold at
- *                     least 8 entries on average and the tiles hold at least half of the entries
+ *                     least 8 entries on average and the tiles hold at least 60 % of the entries
  *   "spmm_panel_emin" entries a 128 x 32 tile needs to be staged (0: 64)
  *   "spmm_panel_cols" column ranks inside a row panel that can be part of a tile (0: 131072)
  *   "spmm_panel_unit" entries after which the tiles of a row panel go to another workgroup (0: 65536)
