@@ -148,24 +148,26 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
 #pragma unroll
     for (int ch = 0; ch < CHUNKS; ++ch) acc[s][ch] = make_float2(0.f, 0.f);
 
-  // A wave stages two rows of B per tile, in pieces of one copy instruction each: per row nx4 of 64 x 16
-  // bytes and, for widths that are not a multiple of 4, one of 4-byte pieces.  One copy instruction keeps the
-  // CU's vector memory path busy for 16 cycles, and a wave that issues its copies back to back sits behind
-  // those of the 15 other waves: the pieces of the next tile are therefore issued one at a time, between the
-  // records of this tile.
+  // A wave stages two rows of B per tile, in pieces of one copy instruction each: per row NX4 of 64 x 16
+  // bytes and one of 4-byte words (for widths that are not a multiple of 4; lanes without a piece are switched
+  // off inside the copy).  One copy instruction keeps the CU's vector memory path busy for 16 cycles, and a
+  // wave that issues its copies back to back sits behind those of the 15 other waves: the pieces of the next
+  // tile are therefore issued one at a time, piece s ahead of the records of slot s.  Which piece that is
+  // (row, position, kind) is known when the slot loop is unrolled, so that no address arithmetic is left.
+  constexpr int NX4 = CHUNKS == 5 ? 3 : 2;  // 16-byte pieces of a row at the widest f of the class (636 / 512 / 384)
+  constexpr int PPR = NX4 + 1, NPIECES = RPW * PPR;
+  static_assert(NPIECES <= kPanelSlots, "one piece per slot");
   const int nq = f >> 2;
   const uint32_t lim16 = (uint32_t)nq * 16u, lim4 = (uint32_t)f * 4u;
-  const int nx4 = (nq + kWave - 1) / kWave;
-  const int ppr = nx4 + (f > nq * 4 ? 1 : 0);
-  const int npieces = RPW * ppr;
-  const uint32_t tail_off = lim16 + (uint32_t)lane * 4u;
-  auto stage_piece = [&](int pc, const float *srca, const float *srcb, int buf) {
-    const bool second = pc >= ppr;
-    const int j = second ? pc - ppr : pc;
-    const float *src = second ? srcb : srca;
-    const uint32_t dst = (uint32_t)(uintptr_t)(panel_lds + buf * bufsz + (wave + (second ? kPanelWaves : 0)) * rs);
-    if (j < nx4)
-      panel_copy16_if(dst + j * (kWave * 16), src, (uint32_t)(j * kWave + lane) * 16u, lim16);
+  const uint32_t lane16 = (uint32_t)lane * 16u, tail_off = lim16 + (uint32_t)lane * 4u;
+  const uint32_t lds_wave = (uint32_t)(uintptr_t)panel_lds + (uint32_t)(wave * rs);  // the wave's first row in buffer 0
+  const uint32_t lds_row1 = (uint32_t)(kPanelWaves * rs);                             // its second row behind it
+  auto stage_piece = [&](int pc, const float *srca, const float *srcb, uint32_t dst0) {  // pc: a constant after unrolling
+    const int r = pc / PPR, j = pc % PPR;
+    const uint32_t dst = dst0 + (r ? lds_row1 : 0u);
+    const float *src = r ? srcb : srca;
+    if (j < NX4)
+      panel_copy16_if(dst + j * (kWave * 16), src, lane16 + (uint32_t)(j * kWave * 16), lim16);
     else
       panel_copy4_if(dst + lim16, src, tail_off, lim4);
   };
@@ -185,7 +187,8 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
     hn = hdr_load(t0 + 1 < t1 ? t0 + 1 : t0);
     const float *srca = B + (int64_t)__builtin_amdgcn_readlane(h0, 0) * ldb;
     const float *srcb = B + (int64_t)__builtin_amdgcn_readlane(h0, 1) * ldb;
-    for (int pc = 0; pc < npieces; ++pc) stage_piece(pc, srca, srcb, 0);
+#pragma unroll
+    for (int pc = 0; pc < NPIECES; ++pc) stage_piece(pc, srca, srcb, lds_wave);
     e0 = __builtin_amdgcn_readlane(h0, 2);
     e1 = __builtin_amdgcn_readlane(h0, 3);
     rec = rec_load(e0, e0, e1);
@@ -205,18 +208,19 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
     const int hn2 = hdr_load(t + 2 < t1 ? t + 2 : t1 - 1);
     const uint2 recn = rec_load(e0n, e0n, e1n);
     const float *srca = B + (int64_t)q0 * ldb, *srcb = B + (int64_t)q1 * ldb;
-    int piece = 0;
+    const uint32_t dst0 = lds_wave + (uint32_t)((buf ^ 1) * bufsz);
 
     // cnt >= 2 records in the lanes of r, sorted by slot, every slot's run of even length (the plan pads odd
     // runs with a record of value 0): the lanes' ballots give the length of every slot's run, and a run adds
     // into that slot's registers (static register indices), two records per step.  While a record is
     // multiplied the row of B of the record behind it (whatever its slot) is on its way from LDS into the
     // other of two sets of registers.
-    auto process = [&](const uint2 r, int cnt) {
+    auto process = [&](const uint2 r, int cnt, bool stage) {
       float2 ba[CHUNKS], bb[CHUNKS];
       const uint32_t myslot = (r.x >> 8) & 0x7u;
+      const uint32_t row_off = (r.x & 0xffu) * (uint32_t)rs;  // of every record of the batch at once
       auto row_read = [&](int idx, float2 (&b)[CHUNKS]) {
-        const char *src = lbase + (__builtin_amdgcn_readlane(r.x, idx) & 0xffu) * rs;
+        const char *src = lbase + __builtin_amdgcn_readlane(row_off, idx);
 #pragma unroll
         for (int ch = 0; ch < CHUNKS; ++ch) b[ch] = *reinterpret_cast<const float2 *>(src + ch * 512);
       };
@@ -224,10 +228,7 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
       int i = 0;
 #pragma unroll
       for (int s = 0; s < kPanelSlots; ++s) {
-        if (piece < npieces) {
-          stage_piece(piece, srca, srcb, buf ^ 1);
-          ++piece;
-        }
+        if (s < NPIECES && stage) stage_piece(s, srca, srcb, dst0);
         const int end = i + __builtin_popcountll(__ballot(lane < cnt && myslot == (uint32_t)s));
         for (; i < end; i += 2) {
           const float v0 = __uint_as_float(__builtin_amdgcn_readlane(r.y, i));
@@ -239,7 +240,7 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
             acc[s][ch].x = fmaf(v0, ba[ch].x, acc[s][ch].x);
             acc[s][ch].y = fmaf(v0, ba[ch].y, acc[s][ch].y);
           }
-          row_read(i + 2 < cnt ? i + 2 : i + 1, ba);  // the last pair reads its second row again
+          row_read((i + 2) & (kWave - 1), ba);  // behind the last record: a lane that holds a copy of it (rec_load)
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int ch = 0; ch < CHUNKS; ++ch) {
@@ -255,10 +256,13 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
       const int left = e1 - base;
       uint2 nxt = cur;
       if (left > kWave) nxt = rec_load(base + kWave, e0, e1);
-      process(cur, left > kWave ? kWave : left);
+      process(cur, left > kWave ? kWave : left, base == e0);
       cur = nxt;
     }
-    for (; piece < npieces; ++piece) stage_piece(piece, srca, srcb, buf ^ 1);  // a wave with few records in this tile
+    if (e0 >= e1) {  // a wave without records in this tile
+#pragma unroll
+      for (int pc = 0; pc < NPIECES; ++pc) stage_piece(pc, srca, srcb, dst0);
+    }
     rec = recn;
     e0 = e0n;
     e1 = e1n;
