@@ -166,7 +166,9 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
     const int r = pc / PPR, j = pc % PPR;
     const uint32_t dst = dst0 + (r ? lds_row1 : 0u);
     const float *src = r ? srcb : srca;
-    if (j < NX4)
+    if (j < NX4 - 1)  // every width of the class fills these pieces: no lane to switch off
+      panel_copy16_at(dst + j * (kWave * 16), src, lane16 + (uint32_t)(j * kWave * 16));
+    else if (j < NX4)
       panel_copy16_if(dst + j * (kWave * 16), src, lane16 + (uint32_t)(j * kWave * 16), lim16);
     else
       panel_copy4_if(dst + lim16, src, tail_off, lim4);
