@@ -162,6 +162,7 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
   const uint32_t lane16 = (uint32_t)lane * 16u, tail_off = lim16 + (uint32_t)lane * 4u;
   const uint32_t lds_wave = (uint32_t)(uintptr_t)panel_lds + (uint32_t)(wave * rs);  // the wave's first row in buffer 0
   const uint32_t lds_row1 = (uint32_t)(kPanelWaves * rs);                             // its second row behind it
+  const uint32_t ldb32 = (uint32_t)ldb;                                               // ldb < 2^31 (launch_panel refuses larger ones)
   auto stage_piece = [&](int pc, const float *srca, const float *srcb, uint32_t dst0) {  // pc: a constant after unrolling
     const int r = pc / PPR, j = pc % PPR;
     const uint32_t dst = dst0 + (r ? lds_row1 : 0u);
@@ -209,7 +210,7 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
     const int e0n = __builtin_amdgcn_readlane(hn, 2), e1n = __builtin_amdgcn_readlane(hn, 3);
     const int hn2 = hdr_load(t + 2 < t1 ? t + 2 : t1 - 1);
     const uint2 recn = rec_load(e0n, e0n, e1n);
-    const float *srca = B + (int64_t)q0 * ldb, *srcb = B + (int64_t)q1 * ldb;
+    const float *srca = B + (uint64_t)(uint32_t)q0 * ldb32, *srcb = B + (uint64_t)(uint32_t)q1 * ldb32;  // unsigned 32 x 32 -> 64
     const uint32_t dst0 = lds_wave + (uint32_t)((buf ^ 1) * bufsz);
 
     // cnt >= 2 records in the lanes of r, sorted by slot, every slot's run of even length (the plan pads odd

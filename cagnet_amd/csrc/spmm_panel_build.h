@@ -546,6 +546,7 @@ static int panel_lds_attr(K kernel, std::atomic<uint64_t> &done, int dev, size_t
 // The panel part of C = A B: partial rows of every row that has entries in active or dense tiles, in *P
 // (row r: P + dslot[r] * f).  P is stream scratch and stays valid until the next panel product on `stream`.
 static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_t f, float **P_out, hipStream_t stream) {
+  if (ldb > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "panel product: leading dimension %lld >= 2^31", (long long)ldb);
   const int chunks = (f / 2 + kWave - 1) / kWave;
   const int groups = (f + 63) / 64;
   const size_t rs = ((size_t)f * 4 + 15) & ~(size_t)15;
