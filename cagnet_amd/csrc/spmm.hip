@@ -361,6 +361,7 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
     if (!pp.declined) {
       float *P = nullptr;
       CG_TRY(launch_panel(pp, B, ldb, f, &P, stream));
+      if (pp.rest->nnz == 0 && !fold) return launch_panel_finish(pp, P, C, ldc, s.rows, f, beta, stream);
       DenseOps fd{};
       fd.fold_D = P;
       fd.fold_dslot = pp.dslot;
@@ -374,7 +375,7 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
     const bool may_decline = g_tune_panel_narrow.load(std::memory_order_relaxed) == 0;
     PanelPlan &pp = s.panel_narrow;
     if (!pp.valid || !par.same(pp) || (pp.declined && !may_decline && !pp.failed)) {
-      const int st = build_panel(s, pp, par, may_decline, stream, kPanelNarrowMinCoverage);
+      const int st = build_panel(s, pp, par, may_decline, stream, kPanelNarrowMinCoverage, 0.0);
       if (st == CG_ERR_ALLOC || st == CG_ERR_OVERFLOW) {
         pp.declined = pp.failed = pp.valid = true;
       } else if (st != CG_OK) {

@@ -454,6 +454,42 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_reduce_kernel(const int32_
   p[0] = s;
 }
 
+// C[r, :] = beta C[r, :] + P[dslot[r], :] for a plan whose tiles hold every entry (the rest matrix is empty);
+// f is even, a thread takes two columns; beta == 0 does not read C.
+__global__ __launch_bounds__(kSpmmThreads) void panel_finish_kernel(float *__restrict__ C, int64_t ldc,
+                                                                     const float *__restrict__ P,
+                                                                     const int32_t *__restrict__ dslot, int32_t rows,
+                                                                     int32_t f, float beta) {
+  const int32_t half = f >> 1;
+  const int64_t idx = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  const int64_t r = idx / half;
+  if (r >= rows) return;
+  const int32_t c = (int32_t)(idx - r * half) * 2;
+  const int32_t d = dslot[r];
+  float2 v = d >= 0 ? *reinterpret_cast<const float2 *>(P + (int64_t)d * f + c) : make_float2(0.f, 0.f);
+  float *out = C + r * ldc + c;
+  if (beta != 0.f) {
+    v.x += beta * out[0];
+    v.y += beta * out[1];
+  }
+  out[0] = v.x;
+  out[1] = v.y;
+}
+
+// Entries in (panel, column) pairs that hold at least two entries (sorted pair order; one 64-bit integer add per wave)
+__global__ __launch_bounds__(kSpmmThreads) void panel_pair_reuse_kernel(const uint32_t *__restrict__ pair_first, int64_t npairs,
+                                                                        unsigned long long *__restrict__ reuse) {
+  const int64_t p = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  uint32_t v = 0;
+  if (p < npairs) {
+    const uint32_t len = pair_first[p + 1] - pair_first[p];
+    v = len >= 2u ? len : 0u;
+  }
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  if ((threadIdx.x & (kWave - 1)) == 0 && v) atomicAdd(reuse, (unsigned long long)v);
+}
+
 // -------------------------------------------------------------------------------------------------
 // plan construction kernels
 // -------------------------------------------------------------------------------------------------
@@ -490,11 +526,25 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_invert_kernel(const int32_
   if (k < count) rank_of[ranked[k]] = (int32_t)k;
 }
 
-// tile of an entry: (row rank / 128) * nkb + column rank / 32 when both ranks are inside the ranked
-// area (the first prows row ranks, the first hot column ranks), else -1
-__device__ __forceinline__ int64_t panel_tile_of(int32_t rrank, int32_t crank, int32_t prows, int32_t hot, int32_t nkb) {
-  if (rrank >= prows || crank >= hot) return -1;
-  return (int64_t)(rrank / kPanelRows) * nkb + crank / kPanelCols;
+// Tiles are numbered panel by panel: panel p has tbase[p + 1] - tbase[p] of them, one per 32 column ranks it uses
+// (at most `hot` ranks).  Tile of an entry from its row rank and its column's rank in the row's panel, -1 for a
+// column rank from `hot` on.
+__device__ __forceinline__ int64_t panel_tile_of(int32_t rrank, int32_t crank, int32_t hot, const int32_t *__restrict__ tbase) {
+  if (crank >= hot) return -1;
+  return (int64_t)tbase[rrank / kPanelRows] + crank / kPanelCols;
+}
+
+// blocks[p] = tiles of panel p = ceil(min(column ranks of the panel, hot) / 32); blocks[npanels] = 0 (slot of the scan's total)
+__global__ __launch_bounds__(kSpmmThreads) void panel_tile_base_kernel(const int32_t *__restrict__ pstart, int32_t npanels,
+                                                                       int32_t hot, uint32_t *__restrict__ blocks) {
+  const int64_t p = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (p > npanels) return;
+  uint32_t b = 0;
+  if (p < npanels) {
+    const int32_t ranks = pstart[p + 1] - pstart[p];
+    b = (uint32_t)(((ranks < hot ? ranks : hot) + kPanelCols - 1) / kPanelCols);
+  }
+  blocks[p] = b;
 }
 
 // Tiles with emin .. dmin - 1 entries are staged ("active"), tiles with at least dmin entries are dense
@@ -546,7 +596,7 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_pair_count_key_kernel(
 __global__ __launch_bounds__(kSpmmThreads) void panel_pair_rank_kernel(const int32_t *__restrict__ spanel,
                                                                        const int32_t *__restrict__ spair, int64_t npairs,
                                                                        const int32_t *__restrict__ pstart, int32_t npanels,
-                                                                       int32_t hot, int32_t nkb,
+                                                                       int32_t hot, const int32_t *__restrict__ tbase,
                                                                        const uint32_t *__restrict__ pair_first,
                                                                        int32_t *__restrict__ pair_lr,
                                                                        uint32_t *__restrict__ tcount) {
@@ -559,7 +609,7 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_pair_rank_kernel(const int
     if (lr >= hot)
       lr = hot;
     else
-      atomicAdd(&tcount[(int64_t)panel * nkb + lr / kPanelCols], pair_first[pair + 1] - pair_first[pair]);
+      atomicAdd(&tcount[(int64_t)tbase[panel] + lr / kPanelCols], pair_first[pair + 1] - pair_first[pair]);
   }
   pair_lr[pair] = (int32_t)lr;
 }
@@ -583,7 +633,8 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_entry_rank_kernel(const ui
 // panel_dense_hdr_fill_kernel): no entry refers to them, a dense tile holds zeros there.
 __global__ __launch_bounds__(kSpmmThreads) void panel_pair_hdr_kernel(
     const int32_t *__restrict__ spanel, const int32_t *__restrict__ spair, int64_t npairs, const int32_t *__restrict__ pstart,
-    int32_t npanels, int32_t hot, int32_t nkb, const int32_t *__restrict__ pair_col, const uint32_t *__restrict__ tcount,
+    int32_t npanels, int32_t hot, const int32_t *__restrict__ tbase, const int32_t *__restrict__ pair_col,
+    const uint32_t *__restrict__ tcount,
     const uint32_t *__restrict__ tindex, const uint32_t *__restrict__ dindex, uint32_t emin, uint32_t dmin,
     int32_t *__restrict__ hdr, int32_t *__restrict__ dhdr) {
   const int64_t j = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
@@ -592,7 +643,7 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_pair_hdr_kernel(
   if (panel >= npanels) return;
   const int64_t lr = j - pstart[panel];
   if (lr >= hot) return;
-  const int64_t t = (int64_t)panel * nkb + lr / kPanelCols;
+  const int64_t t = (int64_t)tbase[panel] + lr / kPanelCols;
   const int c = (int)(lr % kPanelCols);
   const int kind = panel_tile_kind(tcount[t], emin, dmin);
   const int32_t col = pair_col[spair[j]];
@@ -628,13 +679,22 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_tile_select_kernel(const u
 // panel (and block number inside it) of every tile of one kind (1: active, 2: dense), in the compacted numbering
 __global__ __launch_bounds__(kSpmmThreads) void panel_tile_tables_kernel(const uint32_t *__restrict__ tcount,
                                                                          const uint32_t *__restrict__ tindex, int64_t tiles,
-                                                                         uint32_t emin, uint32_t dmin, int kind, int32_t nkb,
+                                                                         uint32_t emin, uint32_t dmin, int kind,
+                                                                         const int32_t *__restrict__ tbase, int32_t npanels,
                                                                          int32_t *__restrict__ tile_panel,
                                                                          int32_t *__restrict__ tile_kb) {
   const int64_t t = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (t >= tiles || panel_tile_kind(tcount[t], emin, dmin) != kind) return;
-  tile_panel[tindex[t]] = (int32_t)(t / nkb);
-  if (tile_kb) tile_kb[tindex[t]] = (int32_t)(t % nkb);
+  int32_t lo = 0, hi = npanels;  // the panel with tbase[panel] <= t < tbase[panel + 1]
+  while (hi - lo > 1) {
+    const int32_t mid = lo + (hi - lo) / 2;
+    if ((int64_t)tbase[mid] <= t)
+      lo = mid;
+    else
+      hi = mid;
+  }
+  tile_panel[tindex[t]] = lo;
+  if (tile_kb) tile_kb[tindex[t]] = (int32_t)(t - tbase[lo]);
 }
 
 // sort keys: entries of active tiles get (active tile * 16 + wave) as major and the slot as minor key, entries of
@@ -645,7 +705,7 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_tile_tables_kernel(const u
 // after which the caller builds the plan again without dense tiles.
 __global__ __launch_bounds__(kSpmmThreads) void panel_entry_key_kernel(
     const int32_t *__restrict__ erow, const int32_t *__restrict__ ecr, const float *__restrict__ val, int64_t nnz,
-    const int32_t *__restrict__ row_rank, int32_t prows, int32_t hot, int32_t nkb,
+    const int32_t *__restrict__ row_rank, int32_t hot, const int32_t *__restrict__ tbase,
     const uint32_t *__restrict__ tcount, const uint32_t *__restrict__ tindex, const uint32_t *__restrict__ dindex,
     uint32_t emin, uint32_t dmin, int32_t sentinel, int32_t *__restrict__ key, int32_t *__restrict__ slot,
     int32_t *__restrict__ pos, uint32_t *__restrict__ dA_bits, uint32_t *__restrict__ collision) {
@@ -653,7 +713,7 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_entry_key_kernel(
   if (k >= nnz) return;
   const int32_t rr = row_rank[erow[k]];
   const int32_t cr = ecr[k];
-  const int64_t t = panel_tile_of(rr, cr, prows, hot, nkb);
+  const int64_t t = panel_tile_of(rr, cr, hot, tbase);
   int32_t ky = sentinel, sl = 0;
   const int kind = t >= 0 ? panel_tile_kind(tcount[t], emin, dmin) : 0;
   if (kind == 1) {

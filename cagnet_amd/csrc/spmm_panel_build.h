@@ -5,14 +5,15 @@
 
 namespace cg {
 
-constexpr int64_t kPanelMaxTiles = (int64_t)1 << 26;  // (panel, column block) pairs whose entries are counted
-constexpr double kPanelMinCoverage = 0.6;             // share of the entries the tiles must hold: measured at f = 602
-                                                      // 0.88 (232,965 vertices, 492 entries per row) 17.1 -> 11.1 ms,
-                                                      // 0.54 (R-MAT scale 20, 31 per row) 7.76 -> 8.25 ms (7.96 with
-                                                      // spmm_panel_share = -1), although the traffic falls from 56.9 to 46.8 GB
-constexpr int32_t kPanelDefaultEmin = 64;             // entries a 128 x 32 tile needs to be staged: twice the
-                                                      // 32 gathers its staging costs
-constexpr int32_t kPanelDefaultCols = 131072;         // column ranks of a panel that can be part of a tile
+constexpr double kPanelMinReuse = 0.5;                // share of the entries that must sit in (panel, column) pairs of at
+                                                      // least two, i.e. use a staged row of B more than once: measured at
+                                                      // f = 602: 0.88 (232,965 vertices, 492 entries per row) 17.1 -> 8.9 ms,
+                                                      // 0.54 (R-MAT scale 20, 31 per row) 7.80 -> 7.69 ms, 0.27 (14,249,639
+                                                      // vertices, 16 per row, f = 300) 42.8 -> 45.5 ms
+constexpr int32_t kPanelDefaultEmin = 1;              // entries a 128 x 32 tile needs to be staged: every tile is (a tile of
+                                                      // columns with one entry each costs what the row-wise kernels' gathers
+                                                      // cost, and nothing is left for them to do): 64 -> 1 10.2 -> 8.9 ms
+constexpr int32_t kPanelDefaultCols = 1 << 30;        // column ranks of a panel that can be part of a tile: all of them
 constexpr int32_t kPanelDefaultUnit = 65536;          // entries after which a panel's tiles start a new unit
 
 struct DevTemps {  // device temporaries of a plan build, freed when the build ends
@@ -36,10 +37,11 @@ static bool want_panel(const CsrSide &s, int32_t f) {
   const int t = g_tune_panel.load(std::memory_order_relaxed);
   if (t < 0 || !panel_width_ok(f) || s.rows == 0 || s.nnz == 0) return false;
   if (t > 0) return true;
-  // Below about 1e10 multiply-adds the plan's fixed costs (a block of partial rows per unit, a pipeline of lightly
-  // filled tiles, few units per compute unit) outweigh what it saves: blocks of a 4 x 4 grid over 232,965 vertices at
-  // f = 602, plan against row-wise kernels: 5.4 M entries 1.84 / 1.28 ms, 12.5 M 2.06 / 2.06 ms, 29.4 M 2.56 / 4.31 ms.
-  return s.nnz / s.rows >= 8 && (double)s.nnz * f >= 1e10;
+  // Below about 5e9 multiply-adds the plan's fixed costs (a block of partial rows per unit, few units per compute
+  // unit) outweigh what it saves: blocks of a 4 x 4 grid over 232,965 vertices at f = 602, plan against row-wise
+  // kernels: 0.6 M entries 0.69 / 0.30 ms, 1.7 M 0.74 / 0.58, 5.4 M 1.02 / 1.29 and 1.39 / 1.17, 12.5 M 1.52 / 2.03,
+  // 29.4 M 2.38 / 4.33 ms.
+  return s.nnz / s.rows >= 8 && (double)s.nnz * f >= 5e9;
 }
 
 static int alloc_sort_buffers(DevTemps &tmp, SortBuffers &buf, int64_t count) {
@@ -51,15 +53,16 @@ static int alloc_sort_buffers(DevTemps &tmp, SortBuffers &buf, int64_t count) {
   return CG_OK;
 }
 
-constexpr int32_t kPanelDefaultDmin = 1024;            // entries from which a 128 x 32 tile is stored whole and multiplied
-                                                       // on the matrix cores (a quarter full); negative tuning value: never
+constexpr int32_t kPanelDefaultDmin = 768;             // entries from which a 128 x 32 tile is stored whole and multiplied
+                                                       // on the matrix cores (3/16 full; 640 / 768 / 896 / 1024: 8.93 / 8.82 /
+                                                       // 9.43 / 8.92 ms at 232,965 vertices, f = 602); negative tuning value: never
 
 // may_decline: leave the plan empty (pp.declined) when the tiles hold too few of the entries.
 // *collision: two entries of one (row, column) pair fell into a dense tile; the plan is unusable.
 // dwg: workgroups of the dense-tile kernel (each takes an equal share of the dense tiles).
 static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot_req, int32_t unit_entries, int32_t dmin,
-                            int32_t dwg, bool share_order, bool may_decline, double min_coverage, bool *collision,
-                            hipStream_t stream) {
+                            int32_t dwg, bool share_order, bool may_decline, double min_coverage, double min_reuse,
+                            bool *collision, hipStream_t stream) {
   *collision = false;
   const int64_t nnz = s.nnz;
   const int32_t n = s.rows, m = s.cols;
@@ -72,14 +75,11 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   // column ranks of a panel that can be part of a tile: whole blocks; a panel's last block may be partly empty
   const int32_t hot = (int32_t)(ceil_div64(hot_req < m ? hot_req : m, kPanelCols) * kPanelCols);
   if (hot < kPanelCols || n < 1 || nnz < 1) return decline();
-  const int32_t nkb = hot / kPanelCols;
-  int64_t npanels = ceil_div64(n, kPanelRows);
-  if (npanels > kPanelMaxTiles / nkb) npanels = kPanelMaxTiles / nkb;  // rows are ranked: the panels left out are the sparsest
-  if (npanels < 1) return decline();
-  const int32_t prows = (int32_t)(npanels * kPanelRows < n ? npanels * kPanelRows : n);
-  const int64_t tiles = npanels * nkb;
+  const int64_t npanels = ceil_div64(n, kPanelRows);
+  const int32_t prows = n;  // every row is in a panel
+  int64_t tiles = 0;        // all (panel, block) tiles, numbered panel by panel (tbase)
   const unsigned gn = (unsigned)ceil_div64(n, kSpmmThreads);
-  const unsigned ge = (unsigned)ceil_div64(nnz, kSpmmThreads), gt = (unsigned)ceil_div64(tiles + 1, kSpmmThreads);
+  const unsigned ge = (unsigned)ceil_div64(nnz, kSpmmThreads);
   DevTemps tmp;
 
   // 1. rows ranked by descending degree (ties: by index)
@@ -130,9 +130,9 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   //     in its panel; the sorted pairs stay for the tile headers.
   int32_t *erow = nullptr, *ecr = nullptr, *pstart = nullptr, *pair_col = nullptr, *spanel = nullptr, *spair = nullptr;
   uint32_t *tcount = nullptr;  // entries per (panel, block) tile
+  int32_t *tbase = nullptr;    // [npanels + 1] first tile of a panel
   int64_t npairs = 0;
-  CG_TRY(tmp.alloc((void **)&tcount, (size_t)(tiles + 1) * 4));
-  CG_TRY(fill_u32(tcount, tiles + 1, 0u, stream));
+  CG_TRY(tmp.alloc((void **)&tbase, (size_t)(npanels + 1) * 4));
   CG_TRY(tmp.alloc((void **)&erow, (size_t)nnz * 4));
   CG_TRY(tmp.alloc((void **)&ecr, (size_t)nnz * 4));
   CG_TRY(tmp.alloc((void **)&pstart, (size_t)(npanels + 2) * 4));
@@ -168,6 +168,18 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     panel_run_first_kernel<<<ge1, kSpmmThreads, 0, stream>>>(start, runs_before, nnz, pair_first);
     CG_LAUNCH_CHECK();
     CG_TRY(fill_u32(pair_first + npairs, 1, (uint32_t)nnz, stream));
+    if (may_decline && min_reuse > 0.0) {
+      // A staged row of B pays where it is used more than once: the share of the entries that sit in (panel, column)
+      // pairs of at least two decides about the plan before the rest of it is built.
+      unsigned long long *d_reuse = nullptr, h_reuse = 0;
+      CG_TRY(t2.alloc((void **)&d_reuse, 8));
+      CG_HIP(hipMemsetAsync(d_reuse, 0, 8, stream));
+      panel_pair_reuse_kernel<<<(unsigned)ceil_div64(npairs, kSpmmThreads), kSpmmThreads, 0, stream>>>(pair_first, npairs, d_reuse);
+      CG_LAUNCH_CHECK();
+      CG_HIP(hipMemcpyAsync(&h_reuse, d_reuse, 8, hipMemcpyDeviceToHost, stream));
+      CG_HIP(hipStreamSynchronize(stream));
+      if ((double)h_reuse < min_reuse * (double)nnz) return decline();
+    }
     {
       DevTemps t3;
       SortBuffers pb;
@@ -180,8 +192,21 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
       int pset = 0;
       CG_TRY(radix_sort_pairs(pb, npairs, bits_for((int32_t)npanels + 1), share ? bits_for(2 * m) : 8, &pset, stream));
       CG_TRY(launch_rowptr(pb.key_a[pset], npairs, (int32_t)npanels + 1, pstart, stream));
+      {
+        uint32_t *d_tiles = nullptr, h_tiles = 0;
+        CG_TRY(t3.alloc((void **)&d_tiles, 4));
+        panel_tile_base_kernel<<<(unsigned)ceil_div64(npanels + 1, kSpmmThreads), kSpmmThreads, 0, stream>>>(
+            pstart, (int32_t)npanels, hot, (uint32_t *)tbase);
+        CG_LAUNCH_CHECK();
+        CG_TRY(exclusive_scan_u32((uint32_t *)tbase, (uint32_t *)tbase, npanels + 1, d_tiles, stream));
+        CG_HIP(hipMemcpyAsync(&h_tiles, d_tiles, 4, hipMemcpyDeviceToHost, stream));
+        CG_HIP(hipStreamSynchronize(stream));
+        tiles = h_tiles;
+      }
+      CG_TRY(tmp.alloc((void **)&tcount, (size_t)(tiles + 1) * 4));
+      CG_TRY(fill_u32(tcount, tiles + 1, 0u, stream));
       panel_pair_rank_kernel<<<gp, kSpmmThreads, 0, stream>>>(pb.key_a[pset], pb.payload[pset], npairs, pstart, (int32_t)npanels,
-                                                              hot, nkb, pair_first, pair_lr, tcount);
+                                                              hot, tbase, pair_first, pair_lr, tcount);
       CG_LAUNCH_CHECK();
       CG_HIP(hipMemcpyAsync(spanel, pb.key_a[pset], (size_t)npairs * 4, hipMemcpyDeviceToDevice, stream));
       CG_HIP(hipMemcpyAsync(spair, pb.payload[pset], (size_t)npairs * 4, hipMemcpyDeviceToDevice, stream));
@@ -193,6 +218,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   }
 
   // 2. active tiles = those with emin .. dmin - 1 entries, dense tiles = those with more
+  const unsigned gt = (unsigned)ceil_div64(tiles + 1, kSpmmThreads);
   uint32_t *tindex = nullptr, *kept = nullptr, *dindex = nullptr, *dkept = nullptr, *d_tot = nullptr;
   CG_TRY(tmp.alloc((void **)&tindex, (size_t)(tiles + 1) * 4));
   CG_TRY(tmp.alloc((void **)&kept, (size_t)(tiles + 1) * 4));
@@ -221,14 +247,14 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   CG_TRY(tmp.alloc((void **)&tile_panel, (size_t)(ntiles + 1) * 4));
   CG_TRY(tmp.alloc((void **)&tile_kb, (size_t)(ntiles + 1) * 4));
   CG_TRY(tmp.alloc((void **)&dtile_panel, (size_t)(ndtiles + 1) * 4));
-  panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, tindex, tiles, (uint32_t)emin, (uint32_t)dmin, 1, nkb, tile_panel,
-                                                           tile_kb);
+  panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, tindex, tiles, (uint32_t)emin, (uint32_t)dmin, 1, tbase,
+                                                           (int32_t)npanels, tile_panel, tile_kb);
   CG_LAUNCH_CHECK();
   CG_TRY(dev_alloc((void **)&pp.hdr, (size_t)(ntiles > 0 ? ntiles : 1) * kPanelWaves * 16));
   CG_TRY(fill_u32((uint32_t *)pp.hdr, ntiles * kPanelWaves * 4, 0xffffffffu, stream));
   if (ndtiles > 0) {
-    panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, dindex, tiles, (uint32_t)emin, (uint32_t)dmin, 2, nkb,
-                                                             dtile_panel, nullptr);
+    panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, dindex, tiles, (uint32_t)emin, (uint32_t)dmin, 2, tbase,
+                                                             (int32_t)npanels, dtile_panel, nullptr);
     CG_LAUNCH_CHECK();
     CG_TRY(dev_alloc((void **)&pp.dA, (size_t)ndtiles * kDenseTileFloats * 4));
     CG_TRY(dev_alloc((void **)&pp.dhdr, (size_t)ndtiles * kPanelCols * 4));
@@ -236,7 +262,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     CG_TRY(fill_u32((uint32_t *)pp.dhdr, ndtiles * kPanelCols, 0xffffffffu, stream));
   }
   panel_pair_hdr_kernel<<<(unsigned)ceil_div64(npairs, kSpmmThreads), kSpmmThreads, 0, stream>>>(
-      spanel, spair, npairs, pstart, (int32_t)npanels, hot, nkb, pair_col, tcount, tindex, dindex, (uint32_t)emin, (uint32_t)dmin,
+      spanel, spair, npairs, pstart, (int32_t)npanels, hot, tbase, pair_col, tcount, tindex, dindex, (uint32_t)emin, (uint32_t)dmin,
       pp.hdr, pp.dhdr);
   CG_LAUNCH_CHECK();
   if (ndtiles > 0) {
@@ -266,7 +292,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     CG_TRY(alloc_sort_buffers(t2, buf, nnz));
     CG_TRY(t2.alloc((void **)&rest_row, (size_t)(nrest > 0 ? nrest : 1) * 4));
     const int32_t sentinel = (int32_t)(ntiles * kPanelWaves);
-    panel_entry_key_kernel<<<ge, kSpmmThreads, 0, stream>>>(erow, ecr, s.val, nnz, row_rank, prows, hot, nkb, tcount,
+    panel_entry_key_kernel<<<ge, kSpmmThreads, 0, stream>>>(erow, ecr, s.val, nnz, row_rank, hot, tbase, tcount,
                                                             tindex, dindex, (uint32_t)emin, (uint32_t)dmin, sentinel,
                                                             buf.key_a[0], buf.key_b[0], buf.payload[0], (uint32_t *)pp.dA,
                                                             d_tot + 4);
@@ -515,16 +541,18 @@ static PanelParams panel_params() {
 
 // Builds the plan for the given values; the plan carries them whatever the outcome (in use, declined).
 static int build_panel(CsrSide &s, PanelPlan &pp, const PanelParams &par, bool may_decline, hipStream_t stream,
-                       double min_coverage = kPanelMinCoverage) {
+                       double min_coverage = 0.0, double min_reuse = kPanelMinReuse) {
   CG_TRY(refuse_under_capture(stream, "building a panel plan"));
   CG_HIP(hipStreamSynchronize(stream));
   pp.release();
   bool collision = false;
-  int st = build_panel_once(s, pp, par.emin, par.cols, par.unit, par.dmin, par.dwg, par.share, may_decline, min_coverage, &collision,
+  int st = build_panel_once(s, pp, par.emin, par.cols, par.unit, par.dmin, par.dwg, par.share, may_decline, min_coverage, min_reuse,
+                            &collision,
                             stream);
   if (st == CG_OK && collision) {  // the matrix stores a (row, column) pair twice: every tile goes the record way
     pp.release();
-    st = build_panel_once(s, pp, par.emin, par.cols, par.unit, 0, par.dwg, par.share, may_decline, min_coverage, &collision, stream);
+    st = build_panel_once(s, pp, par.emin, par.cols, par.unit, 0, par.dwg, par.share, may_decline, min_coverage, min_reuse, &collision,
+                          stream);
   }
   if (st != CG_OK) pp.release();
   par.stamp(pp);
@@ -606,6 +634,16 @@ static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_
     }
   }
   *P_out = P;
+  return CG_OK;
+}
+
+// C = beta C + the partial rows, for a plan without a rest matrix to multiply
+static int launch_panel_finish(const PanelPlan &pp, const float *P, float *C, int64_t ldc, int32_t rows, int32_t f, float beta,
+                               hipStream_t stream) {
+  ProfScope prof("spmm_panel_add", f, stream);
+  panel_finish_kernel<<<(unsigned)ceil_div64((int64_t)rows * (f / 2), kSpmmThreads), kSpmmThreads, 0, stream>>>(C, ldc, P, pp.dslot,
+                                                                                                                rows, f, beta);
+  CG_LAUNCH_CHECK();
   return CG_OK;
 }
 
