@@ -1,24 +1,25 @@
-// Panel plan of the wide CSR SpMM: the dense part of a power-law matrix is multiplied out of LDS.
+// Panel plan of the wide CSR SpMM: a matrix whose rows share columns is multiplied out of LDS, tile by tile.
 //
 // A row-wise SpMM gathers one row of B per stored entry (2408 bytes at f = 602); on a matrix with a
 // few hundred entries per row nearly all of that traffic is re-reading rows of B that other rows of A
 // also use.  Here rows are ranked by their entry counts and taken in panels of 128 consecutive ranks;
-// inside a panel the columns are ranked by the entries they have in these 128 rows and taken in blocks
-// of 32 consecutive ranks (every panel has its own blocks: a column with two entries in the panel sits
-// among its likes, wherever it stands in the matrix as a whole).  A (panel, block) tile that holds
-// enough entries is "active": its 32 rows of B are copied into LDS once (global -> LDS directly, no
+// inside a panel the columns the panel uses are ranked (those with several entries in these 128 rows
+// first, each group in the order of the columns' entry counts over the whole matrix) and taken in blocks
+// of 32 consecutive ranks: every panel has its own blocks, and all panels walk the columns in the same
+// order.  A (panel, block) tile has its 32 rows of B copied into LDS once (global -> LDS directly, no
 // registers in between) and all of the tile's entries read them from there, at LDS bandwidth instead
-// of through the vector memory path.  A workgroup of 16 waves owns a unit = a run of active tiles of one
+// of through the vector memory path.  A workgroup of 16 waves owns a unit = a run of tiles of one
 // panel; wave w holds the accumulators of the 8 rows {w, w + 16, ...} of the panel in registers for the
-// whole unit and writes them out once as partial rows.  Entries of tiles that are not active stay in a
-// second CSR matrix (the "rest") that the row-wise kernels multiply; their finished rows add the
-// partial rows in.  Tiles that are at least a quarter full ("dense" tiles) are stored as full 128 x 32
-// blocks instead and multiplied on the fp32 matrix cores (v_mfma_f32_16x16x4_f32: exact fp32 products,
-// fp32 accumulation) by a second kernel, in units of their own; the zeros of such a block are multiplied
-// too, so a row of B that holds an infinity or a NaN reaches every row of the block (the row-wise
-// kernels and cusparseSpMM would only touch the rows that reference it).  Replaces nothing in the
-// reference beyond cusparseSpMM itself (sparse-extension/sparse_coo_tensor.cu:215-226); sums are in a
-// fixed order, no atomics on floats.
+// whole unit and writes them out once as partial rows.  Tiles with many entries ("dense" tiles) are
+// stored as full 128 x 32 blocks instead and multiplied on the fp32 matrix cores
+// (v_mfma_f32_16x16x4_f32: exact fp32 products, fp32 accumulation) by a second kernel, in units of
+// their own; the zeros of such a block are multiplied too, so a row of B that holds an infinity or a
+// NaN reaches every row of the block (the row-wise kernels and cusparseSpMM would only touch the rows
+// that reference it).  By default every tile is multiplied by one of the two kernels and a last pass
+// writes C = beta C + the partial rows; tiles that a threshold leaves out keep their entries in a
+// second CSR matrix (the "rest") that the row-wise kernels multiply, and their finished rows add the
+// partial rows in.  Replaces nothing in the reference beyond cusparseSpMM itself
+// (sparse-extension/sparse_coo_tensor.cu:215-226); sums are in a fixed order, no atomics on floats.
 #pragma once
 #include "spmm_tables.h"
 #include <algorithm>
@@ -476,18 +477,25 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_finish_kernel(float *__res
   out[1] = v.y;
 }
 
-// Entries in (panel, column) pairs that hold at least two entries (sorted pair order; one 64-bit integer add per wave)
+// Entries in (panel, column) pairs that hold at least two entries: every thread walks a stretch of the pairs, a
+// workgroup adds its threads' sums in LDS and makes one 64-bit integer add
 __global__ __launch_bounds__(kSpmmThreads) void panel_pair_reuse_kernel(const uint32_t *__restrict__ pair_first, int64_t npairs,
                                                                         unsigned long long *__restrict__ reuse) {
-  const int64_t p = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
-  uint32_t v = 0;
-  if (p < npairs) {
+  __shared__ unsigned long long part[kSpmmThreads / kWave];
+  unsigned long long v = 0;
+  for (int64_t p = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x; p < npairs; p += (int64_t)gridDim.x * kSpmmThreads) {
     const uint32_t len = pair_first[p + 1] - pair_first[p];
-    v = len >= 2u ? len : 0u;
+    v += len >= 2u ? len : 0u;
   }
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
-  if ((threadIdx.x & (kWave - 1)) == 0 && v) atomicAdd(reuse, (unsigned long long)v);
+  if ((threadIdx.x & (kWave - 1)) == 0) part[threadIdx.x / kWave] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned long long t = 0;
+    for (int w = 0; w < kSpmmThreads / kWave; ++w) t += part[w];
+    if (t) atomicAdd(reuse, t);
+  }
 }
 
 // -------------------------------------------------------------------------------------------------

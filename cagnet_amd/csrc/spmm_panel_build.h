@@ -174,7 +174,8 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
       unsigned long long *d_reuse = nullptr, h_reuse = 0;
       CG_TRY(t2.alloc((void **)&d_reuse, 8));
       CG_HIP(hipMemsetAsync(d_reuse, 0, 8, stream));
-      panel_pair_reuse_kernel<<<(unsigned)ceil_div64(npairs, kSpmmThreads), kSpmmThreads, 0, stream>>>(pair_first, npairs, d_reuse);
+      const int64_t want = ceil_div64(npairs, kSpmmThreads);
+      panel_pair_reuse_kernel<<<(unsigned)(want < 2048 ? want : 2048), kSpmmThreads, 0, stream>>>(pair_first, npairs, d_reuse);
       CG_LAUNCH_CHECK();
       CG_HIP(hipMemcpyAsync(&h_reuse, d_reuse, 8, hipMemcpyDeviceToHost, stream));
       CG_HIP(hipStreamSynchronize(stream));

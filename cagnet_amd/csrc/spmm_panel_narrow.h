@@ -1,4 +1,4 @@
-// Narrow products (f <= 64) of a matrix with a dense corner: the dense tiles of a panel plan on the fp32
+// Narrow products (f <= 64) of a matrix with well-filled tiles: the dense tiles of a panel plan on the fp32
 // matrix cores, everything else by the row-wise kernels.
 //
 // A row-wise product at f = 16 gathers a 64-byte row of B per entry and is bound by the rate at which L2

@@ -349,13 +349,15 @@ int cg_prof_enable(int on);
  *   "spmm_hub_tiers"  tiers of hot columns (0: chosen from the column counts; groups * tiers <= 64)
  *   "spmm_hub_row"    rows with fewer entries keep all of them in the cold class (0: 64)
  *   "spmm_panel"      panel plan (dense row-panel x column-block tiles multiplied out of LDS; even widths
- *                     258..636): -1 never, 1 always, 0 when the product has at least 1e10 multiply-adds, rows hold at
- *                     least 8 entries on average and the tiles hold at least 60 % of the entries
- *   "spmm_panel_emin" entries a 128 x 32 tile needs to be staged (0: 64)
- *   "spmm_panel_cols" column ranks inside a row panel that can be part of a tile (0: 131072)
+ *                     258..636): -1 never, 1 always, 0 when the product has at least 5e9 multiply-adds, rows hold at
+ *                     least 8 entries on average and at least half of the entries share their column with another
+ *                     entry of the same panel of 128 rows
+ *   "spmm_panel_emin" entries a 128 x 32 tile needs to be staged (0: 1, every tile; tiles below it leave their
+ *                     entries to the row-wise kernels)
+ *   "spmm_panel_cols" column ranks inside a row panel that can be part of a tile (0: all)
  *   "spmm_panel_unit" entries after which the tiles of a row panel go to another workgroup (0: 65536)
  *   "spmm_panel_dmin" entries from which a 128 x 32 tile is stored whole and multiplied on the fp32 matrix
- *                     cores (0: 1024, a quarter full; negative: never).  Such a tile multiplies its zeros too:
+ *                     cores (0: 768; negative: never).  Such a tile multiplies its zeros too:
  *                     a row of B with an infinity or a NaN then reaches all 128 rows of the tile
  *   "spmm_panel_dwg"  workgroups that share the dense tiles equally (0: four per compute unit)
  *   "spmm_panel_share" 0: the columns a row panel stages keep the order of their entry counts in the whole matrix, and
