@@ -360,8 +360,9 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
     }
     if (!pp.declined) {
       float *P = nullptr;
-      CG_TRY(launch_panel(pp, B, ldb, f, &P, stream));
-      if (pp.rest->nnz == 0 && !fold) return launch_panel_finish(pp, P, C, ldc, s.rows, f, beta, stream);
+      const bool direct = pp.rest->nnz == 0 && !fold;  // nothing for the row-wise kernels: one pass sums the blocks into C
+      CG_TRY(launch_panel(pp, B, ldb, f, &P, stream, !direct));
+      if (direct) return launch_panel_finish(pp, P, C, ldc, s.rows, f, beta, stream);
       DenseOps fd{};
       fd.fold_D = P;
       fd.fold_dslot = pp.dslot;

@@ -127,10 +127,10 @@ struct CsrSide {
 };
 
 inline void PanelPlan::release() {
-  void *owned[] = {unit_tile, unit_order, unit_block, dwg_unit, dunit_tile, dunit_block, dhdr, dA, hdr, ent, dslot, split};
+  void *owned[] = {unit_tile, unit_order, unit_block, dwg_unit, dunit_tile, dunit_block, dhdr, dA, hdr, ent, dslot, split, bcount};
   for (void *p : owned)
     table_free(p);
-  unit_tile = unit_order = unit_block = dwg_unit = dunit_tile = dunit_block = dhdr = hdr = dslot = split = nullptr;
+  unit_tile = unit_order = unit_block = dwg_unit = dunit_tile = dunit_block = dhdr = hdr = dslot = split = bcount = nullptr;
   ent = nullptr;
   dA = nullptr;
   if (rest) {

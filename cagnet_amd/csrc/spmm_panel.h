@@ -67,6 +67,7 @@ struct PanelPlan {
                                    // (tile, wave, slot) run has an even number of records
   int32_t *dslot = nullptr;        // [rows] partial row of a row of A: block * 128 + position, or -1
   int32_t *split = nullptr;        // [2 * nsplit] (first block, blocks) of panels that have several units
+  int32_t *bcount = nullptr;       // [nblocks] blocks of the panel whose first block this is (0 for its other blocks)
   CsrSide *rest = nullptr;         // entries outside active tiles, same rows and columns
   void release();
 };
@@ -455,11 +456,13 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_reduce_kernel(const int32_
   p[0] = s;
 }
 
-// C[r, :] = beta C[r, :] + P[dslot[r], :] for a plan whose tiles hold every entry (the rest matrix is empty);
-// f is even, a thread takes two columns; beta == 0 does not read C.
+// C[r, :] = beta C[r, :] + the row's partial rows, one per block of its panel and added in block order, for a plan
+// whose tiles hold every entry (the rest matrix is empty); f is even, a thread takes two columns; beta == 0 does
+// not read C.
 __global__ __launch_bounds__(kSpmmThreads) void panel_finish_kernel(float *__restrict__ C, int64_t ldc,
                                                                      const float *__restrict__ P,
-                                                                     const int32_t *__restrict__ dslot, int32_t rows,
+                                                                     const int32_t *__restrict__ dslot,
+                                                                     const int32_t *__restrict__ bcount, int32_t rows,
                                                                      int32_t f, float beta) {
   const int32_t half = f >> 1;
   const int64_t idx = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
@@ -467,7 +470,17 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_finish_kernel(float *__res
   if (r >= rows) return;
   const int32_t c = (int32_t)(idx - r * half) * 2;
   const int32_t d = dslot[r];
-  float2 v = d >= 0 ? *reinterpret_cast<const float2 *>(P + (int64_t)d * f + c) : make_float2(0.f, 0.f);
+  float2 v = make_float2(0.f, 0.f);
+  if (d >= 0) {
+    const int32_t blocks = bcount[d / kPanelRows];
+    const float *p = P + (int64_t)d * f + c;
+    v = *reinterpret_cast<const float2 *>(p);
+    for (int32_t k = 1; k < blocks; ++k) {
+      const float2 w = *reinterpret_cast<const float2 *>(p + (int64_t)k * kPanelRows * f);
+      v.x += w.x;
+      v.y += w.y;
+    }
+  }
   float *out = C + r * ldc + c;
   if (beta != 0.f) {
     v.x += beta * out[0];

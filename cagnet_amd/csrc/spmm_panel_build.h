@@ -404,7 +404,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   if (ndwg > 0) dwg_unit[(size_t)ndwg] = (int32_t)du.size();
   const int32_t nunits = (int32_t)su.size(), ndunits = (int32_t)du.size();
   std::vector<int32_t> unit_tile((size_t)nunits + 1, 0), unit_block((size_t)nunits), dunit_tile((size_t)ndunits + 1, 0),
-      dunit_block((size_t)ndunits), split, panel_unit((size_t)npanels, -1);
+      dunit_block((size_t)ndunits), split, panel_unit((size_t)npanels, -1), bcount;
   int32_t nblocks = 0;
   for (size_t a = 0, b = 0; a < su.size() || b < du.size();) {  // merge by panel: dense units first, then the others
     const int32_t pa = a < su.size() ? su[a].panel : 0x7fffffff, pb = b < du.size() ? du[b].panel : 0x7fffffff;
@@ -413,6 +413,8 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     for (; b < du.size() && du[b].panel == panel; ++b) dunit_block[b] = nblocks++;
     for (; a < su.size() && su[a].panel == panel; ++a) unit_block[a] = nblocks++;
     panel_unit[(size_t)panel] = first;
+    bcount.resize((size_t)nblocks, 0);
+    bcount[(size_t)first] = nblocks - first;
     if (nblocks - first > 1) {
       split.push_back(first);
       split.push_back(nblocks - first);
@@ -478,6 +480,10 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     CG_HIP(hipMemcpyAsync(pp.dunit_block, dunit_block.data(), (size_t)ndunits * 4, hipMemcpyHostToDevice, stream));
   }
   CG_HIP(hipMemcpyAsync(d_panel_unit, panel_unit.data(), (size_t)npanels * 4, hipMemcpyHostToDevice, stream));
+  if (nblocks > 0) {
+    CG_TRY(dev_alloc((void **)&pp.bcount, (size_t)nblocks * 4));
+    CG_HIP(hipMemcpyAsync(pp.bcount, bcount.data(), (size_t)nblocks * 4, hipMemcpyHostToDevice, stream));
+  }
   if (!split.empty()) {
     CG_TRY(dev_alloc((void **)&pp.split, split.size() * 4));
     CG_HIP(hipMemcpyAsync(pp.split, split.data(), split.size() * 4, hipMemcpyHostToDevice, stream));
@@ -574,7 +580,9 @@ static int panel_lds_attr(K kernel, std::atomic<uint64_t> &done, int dev, size_t
 
 // The panel part of C = A B: partial rows of every row that has entries in active or dense tiles, in *P
 // (row r: P + dslot[r] * f).  P is stream scratch and stays valid until the next panel product on `stream`.
-static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_t f, float **P_out, hipStream_t stream) {
+// sum_blocks: add the blocks of a panel into its first one (false: the caller's pass over the partial rows does that)
+static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_t f, float **P_out, hipStream_t stream,
+                        bool sum_blocks = true) {
   if (ldb > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "panel product: leading dimension %lld >= 2^31", (long long)ldb);
   const int chunks = (f / 2 + kWave - 1) / kWave;
   const int groups = (f + 63) / 64;
@@ -628,7 +636,7 @@ static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_
       CG_LAUNCH_CHECK();
     }
 #undef CG_PANEL
-    if (pp.nsplit > 0) {
+    if (sum_blocks && pp.nsplit > 0) {
       const dim3 grid((unsigned)ceil_div64((int64_t)kPanelRows * f, kSpmmThreads), (unsigned)pp.nsplit);
       panel_reduce_kernel<<<grid, kSpmmThreads, 0, stream>>>(pp.split, P, f);
       CG_LAUNCH_CHECK();
@@ -638,12 +646,12 @@ static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_
   return CG_OK;
 }
 
-// C = beta C + the partial rows, for a plan without a rest matrix to multiply
+// C = beta C + the partial rows (every block of a row's panel), for a plan without a rest matrix to multiply
 static int launch_panel_finish(const PanelPlan &pp, const float *P, float *C, int64_t ldc, int32_t rows, int32_t f, float beta,
                                hipStream_t stream) {
   ProfScope prof("spmm_panel_add", f, stream);
-  panel_finish_kernel<<<(unsigned)ceil_div64((int64_t)rows * (f / 2), kSpmmThreads), kSpmmThreads, 0, stream>>>(C, ldc, P, pp.dslot,
-                                                                                                                rows, f, beta);
+  panel_finish_kernel<<<(unsigned)ceil_div64((int64_t)rows * (f / 2), kSpmmThreads), kSpmmThreads, 0, stream>>>(
+      C, ldc, P, pp.dslot, pp.bcount, rows, f, beta);
   CG_LAUNCH_CHECK();
   return CG_OK;
 }
