@@ -524,10 +524,15 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_degree_key_kernel(const in
   }
 }
 
-__global__ __launch_bounds__(kSpmmThreads) void panel_col_count_kernel(const int32_t *__restrict__ colind, int64_t nnz,
+// count[column] = its entries in the whole matrix, added up pair by pair (a pair = the entries of one column in one
+// panel, a run of the entries sorted by (panel, column): one atomic per pair instead of one per entry)
+__global__ __launch_bounds__(kSpmmThreads) void panel_col_count_kernel(const uint32_t *__restrict__ pair_first, int64_t npairs,
+                                                                       const int32_t *__restrict__ kcol_sorted,
                                                                        uint32_t *__restrict__ count) {
-  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
-  if (k < nnz) atomicAdd(&count[colind[k]], 1u);  // integer count: order independent
+  const int64_t p = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (p >= npairs) return;
+  const uint32_t first = pair_first[p];
+  atomicAdd(&count[kcol_sorted[first]], pair_first[p + 1] - first);  // integer count: order independent
 }
 
 __global__ __launch_bounds__(kSpmmThreads) void panel_count_key_kernel(const uint32_t *__restrict__ count, int32_t m,
@@ -817,6 +822,13 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_pad_write_kernel(const uin
   const int64_t at = k + shift[k];
   out[at] = r;
   if (pad[k]) out[at + 1] = make_uint2(r.x, 0u);
+}
+
+// first[k] = wptr[16 k]: the first record of tile k (k = tiles: all records)
+__global__ __launch_bounds__(kSpmmThreads) void panel_tile_first_kernel(const int32_t *__restrict__ wptr, int64_t count,
+                                                                        int32_t *__restrict__ first) {
+  const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (k < count) first[k] = wptr[k * kPanelWaves];
 }
 
 // wptr[j] += shift[wptr[j]] (shift[count] = all padding records)

@@ -99,31 +99,8 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     CG_HIP(hipStreamSynchronize(stream));
   }
 
-  // 1a. columns ranked by their entries in the whole matrix (ties: by index): the order of a panel's columns that are
-  //     worth staging
   const bool share = share_order && m < (1 << 30);
-  int32_t *col_rank = nullptr;
-  if (share) {
-    DevTemps t2;
-    SortBuffers buf;
-    uint32_t *count = nullptr;
-    CG_TRY(tmp.alloc((void **)&col_rank, (size_t)m * 4));
-    CG_TRY(t2.alloc((void **)&count, (size_t)m * 4));
-    CG_TRY(alloc_sort_buffers(t2, buf, m));
-    CG_TRY(fill_u32(count, m, 0u, stream));
-    panel_col_count_kernel<<<ge, kSpmmThreads, 0, stream>>>(s.colind, nnz, count);
-    CG_LAUNCH_CHECK();
-    const uint32_t maxcount = (uint32_t)(nnz < 0x7ffffffeLL ? nnz : 0x7ffffffeLL);
-    const unsigned gm = (unsigned)ceil_div64(m, kSpmmThreads);
-    panel_count_key_kernel<<<gm, kSpmmThreads, 0, stream>>>(count, m, maxcount, buf.key_a[0], buf.payload[0]);
-    CG_LAUNCH_CHECK();
-    CG_TRY(fill_u32((uint32_t *)buf.key_b[0], m, 0u, stream));
-    int set = 0;
-    CG_TRY(radix_sort_pairs(buf, m, bits_for((int32_t)maxcount + 1), 0, &set, stream));
-    panel_invert_kernel<<<gm, kSpmmThreads, 0, stream>>>(buf.payload[set], m, col_rank);
-    CG_LAUNCH_CHECK();
-    CG_HIP(hipStreamSynchronize(stream));
-  }
+  int32_t *col_rank = nullptr;  // columns ranked by their entries in the whole matrix (step 1a, inside 1b)
 
   // 1b. columns ranked inside every panel by the entries they have there: the entries sorted by (panel, column),
   //     the runs of that order (= pairs) sorted by (panel, descending length).  ecr[entry] = rank of its column
@@ -181,11 +158,36 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
       CG_HIP(hipStreamSynchronize(stream));
       if ((double)h_reuse < min_reuse * (double)nnz) return decline();
     }
+    const unsigned gp = (unsigned)ceil_div64(npairs, kSpmmThreads);
+    // 1a. columns ranked by their entries in the whole matrix (ties: by index): the order of a panel's columns that
+    //     are worth staging
+    if (share) {
+      DevTemps t3;
+      SortBuffers cb;
+      uint32_t *count = nullptr;
+      CG_TRY(tmp.alloc((void **)&col_rank, (size_t)m * 4));
+      CG_TRY(t3.alloc((void **)&count, (size_t)m * 4));
+      CG_TRY(alloc_sort_buffers(t3, cb, m));
+      CG_TRY(fill_u32(count, m, 0u, stream));
+      if (npairs > 0) {
+        panel_col_count_kernel<<<gp, kSpmmThreads, 0, stream>>>(pair_first, npairs, buf.key_b[set], count);
+        CG_LAUNCH_CHECK();
+      }
+      const uint32_t maxcount = (uint32_t)(nnz < 0x7ffffffeLL ? nnz : 0x7ffffffeLL);
+      const unsigned gm = (unsigned)ceil_div64(m, kSpmmThreads);
+      panel_count_key_kernel<<<gm, kSpmmThreads, 0, stream>>>(count, m, maxcount, cb.key_a[0], cb.payload[0]);
+      CG_LAUNCH_CHECK();
+      CG_TRY(fill_u32((uint32_t *)cb.key_b[0], m, 0u, stream));
+      int cset = 0;
+      CG_TRY(radix_sort_pairs(cb, m, bits_for((int32_t)maxcount + 1), 0, &cset, stream));
+      panel_invert_kernel<<<gm, kSpmmThreads, 0, stream>>>(cb.payload[cset], m, col_rank);
+      CG_LAUNCH_CHECK();
+      CG_HIP(hipStreamSynchronize(stream));
+    }
     {
       DevTemps t3;
       SortBuffers pb;
       CG_TRY(alloc_sort_buffers(t3, pb, npairs));
-      const unsigned gp = (unsigned)ceil_div64(npairs, kSpmmThreads);
       const uint32_t cmin = (uint32_t)((emin + kPanelCols - 1) / kPanelCols);  // a block of such columns reaches emin
       panel_pair_count_key_kernel<<<gp, kSpmmThreads, 0, stream>>>(pair_first, npairs, buf.key_a[set], buf.key_b[set], col_rank, cmin,
                                                                    m, pb.key_a[0], pb.key_b[0], pb.payload[0], pair_col);
@@ -360,14 +362,16 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   //    consecutive
   std::vector<int32_t> h_panel((size_t)ntiles), h_kb((size_t)ntiles), h_base((size_t)ntiles + 1, 0), h_dpanel((size_t)ndtiles);
   {
-    // entries of active tile k: tile_wptr[16 k] is its first record
-    std::vector<int32_t> h_wptr((size_t)ntiles * kPanelWaves + 1);
-    CG_HIP(hipMemcpyAsync(h_wptr.data(), tile_wptr, h_wptr.size() * 4, hipMemcpyDeviceToHost, stream));
+    // entries of active tile k: tile_wptr[16 k] is its first record (picked out on the device: a sixteenth to copy)
+    int32_t *d_base = nullptr;
+    CG_TRY(tmp.alloc((void **)&d_base, (size_t)(ntiles + 1) * 4));
+    panel_tile_first_kernel<<<(unsigned)ceil_div64(ntiles + 1, kSpmmThreads), kSpmmThreads, 0, stream>>>(tile_wptr, ntiles + 1, d_base);
+    CG_LAUNCH_CHECK();
+    CG_HIP(hipMemcpyAsync(h_base.data(), d_base, (size_t)(ntiles + 1) * 4, hipMemcpyDeviceToHost, stream));
     if (ntiles > 0) CG_HIP(hipMemcpyAsync(h_panel.data(), tile_panel, (size_t)ntiles * 4, hipMemcpyDeviceToHost, stream));
     if (ntiles > 0) CG_HIP(hipMemcpyAsync(h_kb.data(), tile_kb, (size_t)ntiles * 4, hipMemcpyDeviceToHost, stream));
     if (ndtiles > 0) CG_HIP(hipMemcpyAsync(h_dpanel.data(), dtile_panel, (size_t)ndtiles * 4, hipMemcpyDeviceToHost, stream));
     CG_HIP(hipStreamSynchronize(stream));
-    for (int64_t k = 0; k <= ntiles; ++k) h_base[(size_t)k] = h_wptr[(size_t)k * kPanelWaves];
   }
   struct Unit {
     int32_t panel, t0, t1;
