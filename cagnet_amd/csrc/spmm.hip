@@ -361,8 +361,11 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
     if (!pp.declined) {
       float *P = nullptr;
       const bool direct = pp.rest->nnz == 0 && !fold;  // nothing for the row-wise kernels: one pass sums the blocks into C
-      CG_TRY(launch_panel(pp, B, ldb, f, &P, stream, !direct));
-      if (direct) return launch_panel_finish(pp, P, C, ldc, s.rows, f, beta, stream);
+      if (direct) {  // units that are their panel's only block write their rows of C, the pass over the others skips them
+        CG_TRY(launch_panel(pp, B, ldb, f, &P, stream, false, C, ldc, s.rows, beta));
+        return launch_panel_finish(pp, P, C, ldc, s.rows, f, beta, stream, true);
+      }
+      CG_TRY(launch_panel(pp, B, ldb, f, &P, stream, true));
       DenseOps fd{};
       fd.fold_D = P;
       fd.fold_dslot = pp.dslot;

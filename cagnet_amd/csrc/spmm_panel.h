@@ -67,7 +67,10 @@ struct PanelPlan {
                                    // (tile, wave, slot) run has an even number of records
   int32_t *dslot = nullptr;        // [rows] partial row of a row of A: block * 128 + position, or -1
   int32_t *split = nullptr;        // [2 * nsplit] (first block, blocks) of panels that have several units
-  int32_t *bcount = nullptr;       // [nblocks] blocks of the panel whose first block this is (0 for its other blocks)
+  int32_t *bcount = nullptr;       // [nblocks] blocks of the panel whose first block this is (0 for its other blocks);
+                                   // -1: one block, of a staged unit, which can write its rows of C itself
+  int32_t *unit_row0 = nullptr;    // [nunits] rank of the first row of the unit's panel if the unit is its only block, else -1
+  int32_t *rank_row = nullptr;     // [rows] the row of every rank (rows by descending length)
   CsrSide *rest = nullptr;         // entries outside active tiles, same rows and columns
   void release();
 };
@@ -133,7 +136,8 @@ template <int CHUNKS>
 __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
     const int32_t *__restrict__ unit_tile, const int32_t *__restrict__ unit_order, const int32_t *__restrict__ unit_block,
     const int32_t *__restrict__ hdr, const uint2 *__restrict__ ent, const float *__restrict__ B, int64_t ldb,
-    float *__restrict__ P, int32_t f) {
+    float *__restrict__ P, int32_t f, const int32_t *__restrict__ unit_row0, const int32_t *__restrict__ rank_row,
+    float *__restrict__ C, int64_t ldc, int32_t rows, float beta) {
   extern __shared__ __align__(16) char panel_lds[];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -274,6 +278,31 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
     hn = hn2;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+  }
+  // The only block of its panel (C given): C[row, :] = beta C[row, :] + the sums, nothing left to add up.
+  const int row0 = C ? unit_row0[unit] : -1;
+  if (row0 >= 0) {
+#pragma unroll
+    for (int s = 0; s < kPanelSlots; ++s) {
+      const int rank = row0 + s * kPanelWaves + wave;  // position in the panel = rank of the row inside it
+      if (rank < rows) {
+        float *crow = C + (int64_t)rank_row[rank] * ldc;
+#pragma unroll
+        for (int ch = 0; ch < CHUNKS; ++ch) {
+          const int p = lane + kWave * ch;
+          if (p < npair) {
+            float2 v = acc[s][ch];
+            if (beta != 0.f) {
+              v.x += beta * crow[2 * p];
+              v.y += beta * crow[2 * p + 1];
+            }
+            crow[2 * p] = v.x;
+            crow[2 * p + 1] = v.y;
+          }
+        }
+      }
+    }
+    return;
   }
   // P[block][slot * 16 + wave][:]: position in the block = rank of the row inside its panel
   const int block = unit_block[unit];
@@ -458,12 +487,12 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_reduce_kernel(const int32_
 
 // C[r, :] = beta C[r, :] + the row's partial rows, one per block of its panel and added in block order, for a plan
 // whose tiles hold every entry (the rest matrix is empty); f is even, a thread takes two columns; beta == 0 does
-// not read C.
+// not read C.  direct_written: the rows of a panel with a single staged block (bcount -1) are in C already.
 __global__ __launch_bounds__(kSpmmThreads) void panel_finish_kernel(float *__restrict__ C, int64_t ldc,
                                                                      const float *__restrict__ P,
                                                                      const int32_t *__restrict__ dslot,
                                                                      const int32_t *__restrict__ bcount, int32_t rows,
-                                                                     int32_t f, float beta) {
+                                                                     int32_t f, float beta, int direct_written) {
   const int32_t half = f >> 1;
   const int64_t idx = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   const int64_t r = idx / half;
@@ -472,7 +501,11 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_finish_kernel(float *__res
   const int32_t d = dslot[r];
   float2 v = make_float2(0.f, 0.f);
   if (d >= 0) {
-    const int32_t blocks = bcount[d / kPanelRows];
+    int32_t blocks = bcount[d / kPanelRows];
+    if (blocks < 0) {
+      if (direct_written) return;
+      blocks = 1;
+    }
     const float *p = P + (int64_t)d * f + c;
     v = *reinterpret_cast<const float2 *>(p);
     for (int32_t k = 1; k < blocks; ++k) {

@@ -96,6 +96,8 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     CG_TRY(radix_sort_pairs(buf, n, bits_for(s.max_degree + 1), 0, &set, stream));
     panel_invert_kernel<<<gn, kSpmmThreads, 0, stream>>>(buf.payload[set], n, row_rank);
     CG_LAUNCH_CHECK();
+    CG_TRY(dev_alloc((void **)&pp.rank_row, (size_t)n * 4));
+    CG_HIP(hipMemcpyAsync(pp.rank_row, buf.payload[set], (size_t)n * 4, hipMemcpyDeviceToDevice, stream));
     CG_HIP(hipStreamSynchronize(stream));
   }
 
@@ -382,9 +384,15 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   constexpr int32_t kXcds = 8;       // XCDs of the device: workgroup i of a launch runs on XCD i % 8
   for (int64_t k = 0; k < ntiles;) {
     int64_t j = k, in_unit = 0;
+    // a panel of up to one and a half units' records stays whole: its unit is then its only block and writes C itself
+    int64_t pend = k;
+    while (pend < ntiles && h_panel[(size_t)pend] == h_panel[(size_t)k]) ++pend;
+    const bool whole = (k == 0 || h_panel[(size_t)k - 1] != h_panel[(size_t)k]) &&
+                       (int64_t)h_base[(size_t)pend] - h_base[(size_t)k] <= (int64_t)unit_entries + unit_entries / 2;
     while (j < ntiles && h_panel[(size_t)j] == h_panel[(size_t)k]) {
       const int64_t e = (int64_t)h_base[(size_t)j + 1] - h_base[(size_t)j];
-      if (share) {
+      if (whole) {
+      } else if (share) {
         if (j > k && in_unit >= unit_entries / 2 && h_kb[(size_t)j] / kUnitGrid != h_kb[(size_t)j - 1] / kUnitGrid) break;
       } else if (j > k && in_unit + e > unit_entries) {
         break;
@@ -408,7 +416,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   if (ndwg > 0) dwg_unit[(size_t)ndwg] = (int32_t)du.size();
   const int32_t nunits = (int32_t)su.size(), ndunits = (int32_t)du.size();
   std::vector<int32_t> unit_tile((size_t)nunits + 1, 0), unit_block((size_t)nunits), dunit_tile((size_t)ndunits + 1, 0),
-      dunit_block((size_t)ndunits), split, panel_unit((size_t)npanels, -1), bcount;
+      dunit_block((size_t)ndunits), split, panel_unit((size_t)npanels, -1), bcount, unit_row0((size_t)nunits, -1);
   int32_t nblocks = 0;
   for (size_t a = 0, b = 0; a < su.size() || b < du.size();) {  // merge by panel: dense units first, then the others
     const int32_t pa = a < su.size() ? su[a].panel : 0x7fffffff, pb = b < du.size() ? du[b].panel : 0x7fffffff;
@@ -419,6 +427,10 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     panel_unit[(size_t)panel] = first;
     bcount.resize((size_t)nblocks, 0);
     bcount[(size_t)first] = nblocks - first;
+    if (nblocks - first == 1 && a > 0 && su[a - 1].panel == panel) {  // one block, and a staged unit's: it can write C itself
+      bcount[(size_t)first] = -1;
+      unit_row0[a - 1] = panel * kPanelRows;
+    }
     if (nblocks - first > 1) {
       split.push_back(first);
       split.push_back(nblocks - first);
@@ -499,11 +511,13 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   CG_TRY(dev_alloc((void **)&pp.unit_tile, (size_t)(nunits + 1) * 4));
   CG_TRY(dev_alloc((void **)&pp.unit_order, (size_t)nunits * 4));
   CG_TRY(dev_alloc((void **)&pp.unit_block, (size_t)nunits * 4));
+  CG_TRY(dev_alloc((void **)&pp.unit_row0, (size_t)(nunits > 0 ? nunits : 1) * 4));
   CG_TRY(dev_alloc((void **)&pp.dslot, (size_t)n * 4));
   CG_HIP(hipMemcpyAsync(pp.unit_tile, unit_tile.data(), (size_t)(nunits + 1) * 4, hipMemcpyHostToDevice, stream));
   if (nunits > 0) {
     CG_HIP(hipMemcpyAsync(pp.unit_order, order.data(), (size_t)nunits * 4, hipMemcpyHostToDevice, stream));
     CG_HIP(hipMemcpyAsync(pp.unit_block, unit_block.data(), (size_t)nunits * 4, hipMemcpyHostToDevice, stream));
+    CG_HIP(hipMemcpyAsync(pp.unit_row0, unit_row0.data(), (size_t)nunits * 4, hipMemcpyHostToDevice, stream));
   }
   if (ndunits > 0) {
     CG_TRY(dev_alloc((void **)&pp.dwg_unit, (size_t)(ndwg + 1) * 4));
@@ -615,8 +629,10 @@ static int panel_lds_attr(K kernel, std::atomic<uint64_t> &done, int dev, size_t
 // The panel part of C = A B: partial rows of every row that has entries in active or dense tiles, in *P
 // (row r: P + dslot[r] * f).  P is stream scratch and stays valid until the next panel product on `stream`.
 // sum_blocks: add the blocks of a panel into its first one (false: the caller's pass over the partial rows does that)
+// C_direct (with ldc, rows, beta): staged units that are their panel's only block write C = beta C + their rows
+// themselves; launch_panel_finish(direct_written = true) then leaves those rows alone.
 static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_t f, float **P_out, hipStream_t stream,
-                        bool sum_blocks = true) {
+                        bool sum_blocks = true, float *C_direct = nullptr, int64_t ldc = 0, int32_t rows = 0, float beta = 0.f) {
   if (ldb > 0x7fffffffLL) CG_FAIL(CG_ERR_SIZE, "panel product: leading dimension %lld >= 2^31", (long long)ldb);
   const int chunks = (f / 2 + kWave - 1) / kWave;
   const int groups = (f + 63) / 64;
@@ -657,7 +673,8 @@ static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_
     static std::atomic<uint64_t> attr_set{0};                                                                          \
     CG_TRY(panel_lds_attr(spmm_panel_kernel<CH>, attr_set, dev, lds_max, lds));                                        \
     spmm_panel_kernel<CH><<<(unsigned)pp.nunits, kPanelThreads, lds, stream>>>(pp.unit_tile, pp.unit_order, pp.unit_block, \
-                                                                               pp.hdr, pp.ent, B, ldb, P, f);          \
+                                                                               pp.hdr, pp.ent, B, ldb, P, f, pp.unit_row0, \
+                                                                               pp.rank_row, C_direct, ldc, rows, beta); \
   } break;
     if (pp.nunits > 0) {
       switch (chunks) {
@@ -682,10 +699,10 @@ static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_
 
 // C = beta C + the partial rows (every block of a row's panel), for a plan without a rest matrix to multiply
 static int launch_panel_finish(const PanelPlan &pp, const float *P, float *C, int64_t ldc, int32_t rows, int32_t f, float beta,
-                               hipStream_t stream) {
+                               hipStream_t stream, bool direct_written) {
   ProfScope prof("spmm_panel_add", f, stream);
   panel_finish_kernel<<<(unsigned)ceil_div64((int64_t)rows * (f / 2), kSpmmThreads), kSpmmThreads, 0, stream>>>(
-      C, ldc, P, pp.dslot, pp.bcount, rows, f, beta);
+      C, ldc, P, pp.dslot, pp.bcount, rows, f, beta, direct_written ? 1 : 0);
   CG_LAUNCH_CHECK();
   return CG_OK;
 }

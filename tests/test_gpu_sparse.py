@@ -1022,6 +1022,44 @@ def test_spmm_panel_last_block_with_empty_places_and_columns_ranked_per_panel(cu
     assert spmm_error(got, row, col, val, n, m, Bd.cpu()) <= REL_TOL
 
 
+def test_spmm_panel_single_block_panels_write_c_themselves(cuda, tune):
+    """A panel whose tiles are one staged unit has a single block of partial rows: that unit writes its rows of C
+    (in the order of the rows' ranks) and the pass over the partial rows leaves them alone.  Five panels (one of 60
+    rows, rows without entries among them), one heavy enough for several units; C is a column slice of a wider
+    matrix and is read only where beta asks for it: full of NaN for beta = 0, then beta = -0.5 on known values,
+    and what lies beside the slice stays as it was."""
+    from cagnet_amd import ops
+    n, m, f = 572, 2400, 262                                            # 75 column blocks: units are cut every 32
+    rng = np.random.default_rng(33)
+    deg = np.where(np.arange(n) < 128, 300, rng.integers(0, 12, n))    # first panel: 38,400 entries, the others light
+    r = np.repeat(np.arange(n), deg)
+    c = np.concatenate([rng.choice(m, d, replace=False) for d in deg])
+    perm = rng.permutation(n)                                           # ranks are not the row numbers
+    key = np.unique(perm[r] * m + c)
+    row, col = torch.from_numpy(key // m), torch.from_numpy(key % m)
+    val = torch.from_numpy(rng.standard_normal(key.size).astype(np.float32))
+    tune("spmm_panel", 1)
+    tune("spmm_panel_unit", 8192)                                       # the heavy panel is cut into several units
+    tune("spmm_panel_dmin", -1)                                         # ... of staged tiles
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, m)
+    B = torch.randn(m, f, generator=torch.Generator().manual_seed(3)).to(cuda)
+    Cbig = torch.full((n, f + 5), float("nan"), device=cuda)
+    C = Cbig[:, 3:3 + f]
+    A.spmm(B, out=C, beta=0.0)
+    info = _panel_info(A)
+    assert info["state"] == 1 and info["rest"] == 0 and info["units"] >= 6, info
+    assert torch.isnan(Cbig[:, :3]).all() and torch.isnan(Cbig[:, 3 + f:]).all() and not torch.isnan(C).any()
+    assert spmm_error(C, row, col, val, n, m, B.cpu()) <= REL_TOL
+    C0 = torch.randn(n, f, generator=torch.Generator().manual_seed(4))
+    Cbig.zero_()
+    C.copy_(C0)
+    A.spmm(B, out=C, beta=-0.5)
+    ref = -0.5 * C0.double() + torch.sparse_coo_tensor(torch.stack([row, col]), val.double(), (n, m)) @ B.cpu().double()
+    mag = 0.5 * C0.double().abs() + torch.sparse_coo_tensor(torch.stack([row, col]), val.double().abs(), (n, m)) @ B.cpu().double().abs()
+    assert ((C.cpu().double() - ref).abs() / mag.clamp_min(1e-30)).max().item() <= REL_TOL
+    assert (Cbig[:, :3] == 0).all() and (Cbig[:, 3 + f:] == 0).all()
+
+
 def test_spmm_panel_plan_rectangular_strided_and_declined(cuda, tune):
     """A non-symmetric rectangular matrix, B and C as column slices of wider matrices, rows without any
     entry; and a matrix without dense tiles, on which the automatic choice declines the plan."""
