@@ -127,10 +127,10 @@ struct CsrSide {
 };
 
 inline void PanelPlan::release() {
-  void *owned[] = {unit_tile, unit_order, unit_block, dwg_unit, dunit_tile, dunit_block, dhdr, dA, hdr, ent, dslot, split, bcount, unit_row0, rank_row};
+  void *owned[] = {unit_tile, unit_order, unit_qstart, unit_block, dwg_unit, dunit_tile, dunit_block, dhdr, dA, hdr, ent, dslot, split, bcount, unit_row0, rank_row};
   for (void *p : owned)
     table_free(p);
-  unit_tile = unit_order = unit_block = dwg_unit = dunit_tile = dunit_block = dhdr = hdr = dslot = split = bcount = unit_row0 = rank_row = nullptr;
+  unit_tile = unit_order = unit_qstart = unit_block = dwg_unit = dunit_tile = dunit_block = dhdr = hdr = dslot = split = bcount = unit_row0 = rank_row = nullptr;
   ent = nullptr;
   dA = nullptr;
   if (rest) {

@@ -53,7 +53,8 @@ struct PanelPlan {
   int32_t ndtiles = 0, ndunits = 0;
   int32_t nblocks = 0;             // blocks of 128 partial rows, one per unit of either kind
   int32_t *unit_tile = nullptr;    // [nunits + 1] tiles of a unit (units never span panels)
-  int32_t *unit_order = nullptr;   // [nunits] launch order: heaviest unit first
+  int32_t *unit_order = nullptr;   // [nunits] the units in eight queues, one per XCD, each in launch order
+  int32_t *unit_qstart = nullptr;  // [9] where the queues start in unit_order
   int32_t *unit_block = nullptr;   // [nunits] block of partial rows a unit writes
   int32_t ndwg = 0;                // workgroups of the dense-tile kernel: equal shares of the list of dense tiles
   int32_t *dwg_unit = nullptr;     // [ndwg + 1] units of a workgroup (runs of tiles of one panel inside its share)
@@ -132,16 +133,43 @@ __device__ __forceinline__ void panel_copy4_if(uint32_t lds_addr, const float *b
 // A wave walks its records of a tile two at a time and has the row of B of the record behind the current one on
 // its way from LDS while the current one is multiplied: a record costs 2408 bytes of LDS reads (f = 602)
 // whose latency four waves per SIMD do not hide by themselves.
+// A workgroup takes the next unit from the queue of the XCD it runs on (the plan fills the queues so that the
+// workgroups of an XCD walk the same rows of B at the same time, and evenly by its estimate of the units' costs) and,
+// once that queue is empty, from the next XCD's that is not: what an XCD is short of by the estimate's error the
+// others make up.  Returns -1 when every queue is empty.  qhead: eight counters, zero at launch.
+__device__ __forceinline__ int panel_take_unit(const int32_t *__restrict__ unit_queue, const int32_t *__restrict__ qstart,
+                                               int32_t *__restrict__ qhead) {
+  __shared__ int taken;
+  if (threadIdx.x == 0) {
+    const int xcd = (int)__builtin_amdgcn_s_getreg((3 << 11) | 20) & 7;  // hardware register XCC_ID, bits 0..3
+    int unit = -1;
+    for (int k = 0; k < 8 && unit < 0; ++k) {
+      const int q = (xcd + k) & 7;
+      const int first = qstart[q], count = qstart[q + 1] - first;
+      if (count <= 0) continue;
+      const int pos = atomicAdd(&qhead[q], 1);
+      if (pos < count) unit = unit_queue[first + pos];
+    }
+    taken = unit;
+  }
+  __syncthreads();
+  return __builtin_amdgcn_readfirstlane(taken);
+}
+
 template <int CHUNKS>
 __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
-    const int32_t *__restrict__ unit_tile, const int32_t *__restrict__ unit_order, const int32_t *__restrict__ unit_block,
+    const int32_t *__restrict__ unit_tile, const int32_t *__restrict__ unit_order, const int32_t *__restrict__ unit_qstart,
+    int32_t *__restrict__ qhead, const int32_t *__restrict__ unit_block,
     const int32_t *__restrict__ hdr, const uint2 *__restrict__ ent, const float *__restrict__ B, int64_t ldb,
     float *__restrict__ P, int32_t f, const int32_t *__restrict__ unit_row0, const int32_t *__restrict__ rank_row,
     float *__restrict__ C, int64_t ldc, int32_t rows, float beta) {
   extern __shared__ __align__(16) char panel_lds[];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int unit = unit_order[blockIdx.x];
+  // One workgroup per compute unit, each taking units until the queues are empty (no workgroup waits for another).
+  for (;;) {
+  const int unit = panel_take_unit(unit_order, unit_qstart, qhead);
+  if (unit < 0) return;
   const int t0 = unit_tile[unit], t1 = unit_tile[unit + 1];
   const int npair = f >> 1;
   const int rs = (f * 4 + 15) & ~15;  // bytes of a staged row: 16-byte aligned for the direct copies
@@ -302,7 +330,7 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
         }
       }
     }
-    return;
+    continue;
   }
   // P[block][slot * 16 + wave][:]: position in the block = rank of the row inside its panel
   const int block = unit_block[unit];
@@ -315,6 +343,7 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
       if (p < npair) *reinterpret_cast<float2 *>(prow + 2 * p) = acc[s][ch];
     }
   }
+  }  // the next unit
 }
 
 // -------------------------------------------------------------------------------------------------

@@ -53,6 +53,7 @@ static int alloc_sort_buffers(DevTemps &tmp, SortBuffers &buf, int64_t count) {
   return CG_OK;
 }
 
+constexpr int32_t kXcdQueues = 8;                       // queues of units, one per XCD (spmm_panel_kernel)
 constexpr int32_t kPanelDefaultDmin = 768;             // entries from which a 128 x 32 tile is stored whole and multiplied
                                                        // on the matrix cores (3/16 full; 640 / 768 / 896 / 1024: 8.93 / 8.82 /
                                                        // 9.43 / 8.92 ms at 232,965 vertices, f = 602); negative tuning value: never
@@ -448,14 +449,17 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     const double T = (double)(su[(size_t)u].t1 - su[(size_t)u].t0), R = (double)su[(size_t)u].weight;
     return T > 0.0 ? 1.50 * T + 0.0034 * R + 8.7e-6 * R * R / T : 0.0;
   };
+  // The units go into eight queues, one per XCD; a workgroup takes the next unit of the queue of the XCD it runs on
+  // (spmm_panel_kernel: panel_take_unit).
+  std::vector<int32_t> queue[kXcds];
   if (!share) {
     std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return cost(a) > cost(b); });
+    for (int32_t i = 0; i < nunits; ++i) queue[i % kXcds].push_back(order[(size_t)i]);
   } else {
     // Units that start at the same block number in neighbouring panels walk nearly the same rows of B: groups of as
-    // many of them as an XCD has compute units are launched on one XCD together (workgroup i runs on XCD i % 8), so
-    // that one copy from memory serves the whole group out of that XCD's L2.  The groups go out in rounds of one per
-    // XCD, costliest groups first, and within a round the costliest group goes to the XCD that has been given the
-    // least so far: every XCD works through its own queue, and what one is short of no other can take over.
+    // many of them as an XCD has compute units sit in one queue one behind the other, so that they run on that XCD
+    // together and one copy from memory serves the whole group out of its L2.  The groups are dealt out in rounds
+    // of one per queue, and within a round the costliest group goes to the queue that has been given the least so far.
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
         cus < kXcds) {
@@ -467,14 +471,11 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
       const int32_t ka = h_kb[(size_t)su[(size_t)a].t0] / kUnitGrid, kb = h_kb[(size_t)su[(size_t)b].t0] / kUnitGrid;
       return ka != kb ? ka < kb : su[(size_t)a].panel < su[(size_t)b].panel;
     });
-    // the units behind the last full group go first, one after the other (their places would otherwise be holes
-    // that shift every later workgroup to another XCD)
+    // the units behind the last full group go first, one to a queue in turn
     const int32_t ngroups = nunits / gsize, loose = nunits - ngroups * gsize;
-    std::vector<int32_t> placed;
-    placed.reserve((size_t)nunits);
-    for (int32_t i = 0; i < loose; ++i) placed.push_back(order[(size_t)(ngroups * gsize + i)]);
+    for (int32_t i = 0; i < loose; ++i) queue[i % kXcds].push_back(order[(size_t)(ngroups * gsize + i)]);
     // a group's place in the order goes by its costliest member (a group that straddles two block numbers holds light
-    // and heavy units, and a heavy unit that starts late is what the launch ends on), an XCD's load by the sums
+    // and heavy units, and a heavy unit that starts late is what the launch ends on), a queue's load by the sums
     std::vector<double> gcost((size_t)ngroups, 0.0), gmax((size_t)ngroups, 0.0);
     for (int32_t i = 0; i < ngroups * gsize; ++i) {
       const double c = cost(order[(size_t)i]);
@@ -489,27 +490,27 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     double given[kXcds] = {0, 0, 0, 0, 0, 0, 0, 0};
     for (int32_t r0 = 0; r0 < ngroups; r0 += kXcds) {
       const int32_t in_round = ngroups - r0 < kXcds ? ngroups - r0 : kXcds;
-      int32_t lane_of[kXcds], by_load[kXcds];  // lane_of[x]: the group (place in gorder) that XCD lane x gets, or -1
-      for (int32_t x = 0; x < kXcds; ++x) {
-        lane_of[x] = -1;
-        by_load[x] = x;
-      }
+      int32_t by_load[kXcds];
+      for (int32_t x = 0; x < kXcds; ++x) by_load[x] = x;
       std::stable_sort(by_load, by_load + kXcds, [&](int32_t a, int32_t b) { return given[a] < given[b]; });
       for (int32_t k = 0; k < in_round; ++k) {
-        lane_of[by_load[k]] = r0 + k;
-        given[by_load[k]] += gcost[(size_t)gorder[(size_t)(r0 + k)]];
+        const int32_t g = gorder[(size_t)(r0 + k)];
+        given[by_load[k]] += gcost[(size_t)g];
+        for (int32_t j = 0; j < gsize; ++j) queue[by_load[k]].push_back(order[(size_t)(g * gsize + j)]);
       }
-      // lane x of a round = launch positions loose + 8 r0 gsize + x, + 8, ...; a last round of fewer groups leaves lanes out
-      for (int32_t j = 0; j < gsize; ++j)
-        for (int32_t x = 0; x < kXcds; ++x)
-          if (lane_of[x] >= 0) placed.push_back(order[(size_t)(gorder[(size_t)lane_of[x]] * gsize + j)]);
     }
-    order.swap(placed);
+  }
+  int32_t qstart[kXcds + 1] = {0};
+  for (int32_t x = 0, at = 0; x < kXcds; ++x) {
+    for (int32_t u : queue[x]) order[(size_t)at++] = u;
+    qstart[x + 1] = at;
   }
   int32_t *d_panel_unit = nullptr;
   CG_TRY(tmp.alloc((void **)&d_panel_unit, (size_t)npanels * 4));
   CG_TRY(dev_alloc((void **)&pp.unit_tile, (size_t)(nunits + 1) * 4));
-  CG_TRY(dev_alloc((void **)&pp.unit_order, (size_t)nunits * 4));
+  CG_TRY(dev_alloc((void **)&pp.unit_order, (size_t)(nunits > 0 ? nunits : 1) * 4));
+  CG_TRY(dev_alloc((void **)&pp.unit_qstart, sizeof(qstart)));
+  CG_HIP(hipMemcpyAsync(pp.unit_qstart, qstart, sizeof(qstart), hipMemcpyHostToDevice, stream));
   CG_TRY(dev_alloc((void **)&pp.unit_block, (size_t)nunits * 4));
   CG_TRY(dev_alloc((void **)&pp.unit_row0, (size_t)(nunits > 0 ? nunits : 1) * 4));
   CG_TRY(dev_alloc((void **)&pp.dslot, (size_t)n * 4));
@@ -640,10 +641,14 @@ static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_
   const size_t lds = 2 * (size_t)kPanelCols * rs;  // two tiles of staged rows
   const size_t lds_max = 2 * (size_t)kPanelCols * ((kPanelMaxF * 4 + 15) & ~15);
   void *p = nullptr;
-  CG_TRY(scratch_get(stream, kSlotE, (size_t)pp.nblocks * kPanelRows * f * sizeof(float), &p));
+  const size_t p_bytes = ((size_t)pp.nblocks * kPanelRows * f * sizeof(float) + 15) & ~(size_t)15;
+  CG_TRY(scratch_get(stream, kSlotE, p_bytes + kXcdQueues * sizeof(int32_t), &p));
   float *P = (float *)p;
-  int dev = 0;
+  int32_t *qhead = (int32_t *)((char *)p + p_bytes);  // the queues' counters of this launch (panel_take_unit)
+  int dev = 0, cus = 0;
   CG_HIP(hipGetDevice(&dev));
+  CG_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));  // a workgroup of the staged-tile kernel fills a compute unit's LDS
+  if (cus < 1) cus = 256;
   if (pp.ndunits > 0) {
     ProfScope prof("spmm_panel_dense", f, stream);
 #define CG_PANEL_DENSE(NG)                                                                                              \
@@ -672,11 +677,12 @@ static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_
   case CH: {                                                                                                           \
     static std::atomic<uint64_t> attr_set{0};                                                                          \
     CG_TRY(panel_lds_attr(spmm_panel_kernel<CH>, attr_set, dev, lds_max, lds));                                        \
-    spmm_panel_kernel<CH><<<(unsigned)pp.nunits, kPanelThreads, lds, stream>>>(pp.unit_tile, pp.unit_order, pp.unit_block, \
+    spmm_panel_kernel<CH><<<(unsigned)(pp.nunits < cus ? pp.nunits : cus), kPanelThreads, lds, stream>>>(pp.unit_tile, pp.unit_order, pp.unit_qstart, qhead, pp.unit_block, \
                                                                                pp.hdr, pp.ent, B, ldb, P, f, pp.unit_row0, \
                                                                                pp.rank_row, C_direct, ldc, rows, beta); \
   } break;
     if (pp.nunits > 0) {
+      CG_TRY(fill_u32((uint32_t *)qhead, kXcdQueues, 0u, stream));
       switch (chunks) {
         CG_PANEL(3)
         CG_PANEL(4)
