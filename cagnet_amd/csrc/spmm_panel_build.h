@@ -382,7 +382,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   };
   std::vector<Unit> su, du;  // units of active tiles, of dense tiles; both in panel order
   constexpr int32_t kUnitGrid = 32;  // with shared column order a unit starts where a panel's block number passes a multiple
-  constexpr int32_t kXcds = 8;       // XCDs of the device: workgroup i of a launch runs on XCD i % 8
+  constexpr int32_t kXcds = kXcdQueues;  // XCDs of the device
   for (int64_t k = 0; k < ntiles;) {
     int64_t j = k, in_unit = 0;
     // a panel of up to one and a half units' records stays whole: its unit is then its only block and writes C itself

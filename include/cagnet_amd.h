@@ -361,9 +361,9 @@ int cg_prof_enable(int on);
  *                     a row of B with an infinity or a NaN then reaches all 128 rows of the tile
  *   "spmm_panel_dwg"  workgroups that share the dense tiles equally (0: four per compute unit)
  *   "spmm_panel_share" 0: the columns a row panel stages keep the order of their entry counts in the whole matrix, and
- *                     workgroups whose panels start at the same place of that order are launched on one XCD together
+ *                     units whose panels start at the same place of that order are queued for one XCD together
  *                     (one copy from memory then serves them all out of that XCD's L2); -1: every panel orders its
- *                     columns by their entries in the panel, heaviest workgroups first
+ *                     columns by their entries in the panel, costliest units first
  *   "spmm_panel_narrow" the same plan with dense tiles only for narrow products (f <= 64; the other entries go to the
  *                     row-wise kernels and the partial rows are added in afterwards): -1 never, 1 always, 0 when rows
  *                     hold at least 64 entries on average, the product has at least 1e9 multiply-adds and the dense
