@@ -363,7 +363,7 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
       const bool direct = pp.rest->nnz == 0 && !fold;  // nothing for the row-wise kernels: one pass sums the blocks into C
       if (direct) {  // units that are their panel's only block write their rows of C, the pass over the others skips them
         CG_TRY(launch_panel(pp, B, ldb, f, &P, stream, false, C, ldc, s.rows, beta));
-        return launch_panel_finish(pp, P, C, ldc, s.rows, f, beta, stream, true);
+        return launch_panel_finish(pp, P, C, ldc, f, beta, stream);
       }
       CG_TRY(launch_panel(pp, B, ldb, f, &P, stream, true));
       DenseOps fd{};

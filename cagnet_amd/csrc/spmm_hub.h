@@ -127,10 +127,11 @@ struct CsrSide {
 };
 
 inline void PanelPlan::release() {
-  void *owned[] = {unit_tile, unit_order, unit_qstart, unit_block, dwg_unit, dunit_tile, dunit_block, dhdr, dA, hdr, ent, dslot, split, bcount, unit_row0, rank_row};
+  void *owned[] = {unit_tile, unit_order, unit_qstart, unit_block, dwg_unit, dunit_tile, dunit_block, dhdr, dA, hdr, ent, dslot, split, bcount, unit_row0, rank_row, finish_rows};
   for (void *p : owned)
     table_free(p);
-  unit_tile = unit_order = unit_qstart = unit_block = dwg_unit = dunit_tile = dunit_block = dhdr = hdr = dslot = split = bcount = unit_row0 = rank_row = nullptr;
+  unit_tile = unit_order = unit_qstart = unit_block = dwg_unit = dunit_tile = dunit_block = dhdr = hdr = dslot = split = bcount = unit_row0 = rank_row = finish_rows = nullptr;
+  nfinish = 0;
   ent = nullptr;
   dA = nullptr;
   if (rest) {

@@ -72,6 +72,9 @@ struct PanelPlan {
                                    // -1: one block, of a staged unit, which can write its rows of C itself
   int32_t *unit_row0 = nullptr;    // [nunits] rank of the first row of the unit's panel if the unit is its only block, else -1
   int32_t *rank_row = nullptr;     // [rows] the row of every rank (rows by descending length)
+  int32_t *finish_rows = nullptr;  // [nfinish] the rows that the pass over the partial rows writes: all but those of panels
+                                   // whose only block is a staged unit's
+  int32_t nfinish = 0;
   CsrSide *rest = nullptr;         // entries outside active tiles, same rows and columns
   void release();
 };
@@ -516,25 +519,23 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_reduce_kernel(const int32_
 
 // C[r, :] = beta C[r, :] + the row's partial rows, one per block of its panel and added in block order, for a plan
 // whose tiles hold every entry (the rest matrix is empty); f is even, a thread takes two columns; beta == 0 does
-// not read C.  direct_written: the rows of a panel with a single staged block (bcount -1) are in C already.
+// not read C.  list: the rows to write (the rows of a panel whose only block is a staged unit's are in C already).
 __global__ __launch_bounds__(kSpmmThreads) void panel_finish_kernel(float *__restrict__ C, int64_t ldc,
                                                                      const float *__restrict__ P,
                                                                      const int32_t *__restrict__ dslot,
-                                                                     const int32_t *__restrict__ bcount, int32_t rows,
-                                                                     int32_t f, float beta, int direct_written) {
+                                                                     const int32_t *__restrict__ bcount,
+                                                                     const int32_t *__restrict__ list, int32_t count,
+                                                                     int32_t f, float beta) {
   const int32_t half = f >> 1;
   const int64_t idx = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
-  const int64_t r = idx / half;
-  if (r >= rows) return;
-  const int32_t c = (int32_t)(idx - r * half) * 2;
+  const int64_t i = idx / half;
+  if (i >= count) return;
+  const int64_t r = list[i];
+  const int32_t c = (int32_t)(idx - i * half) * 2;
   const int32_t d = dslot[r];
   float2 v = make_float2(0.f, 0.f);
   if (d >= 0) {
-    int32_t blocks = bcount[d / kPanelRows];
-    if (blocks < 0) {
-      if (direct_written) return;
-      blocks = 1;
-    }
+    const int32_t blocks = bcount[d / kPanelRows];
     const float *p = P + (int64_t)d * f + c;
     v = *reinterpret_cast<const float2 *>(p);
     for (int32_t k = 1; k < blocks; ++k) {
@@ -884,6 +885,28 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_pad_write_kernel(const uin
   const int64_t at = k + shift[k];
   out[at] = r;
   if (pad[k]) out[at + 1] = make_uint2(r.x, 0u);
+}
+
+// flag[r] = 1 for the rows the pass over the partial rows writes: rows without a partial row (C = beta C) and rows
+// of panels with several blocks or a dense one
+__global__ __launch_bounds__(kSpmmThreads) void panel_finish_flag_kernel(const int32_t *__restrict__ dslot,
+                                                                         const int32_t *__restrict__ bcount, int32_t rows,
+                                                                         uint32_t *__restrict__ flag) {
+  const int64_t r = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (r > rows) return;
+  uint32_t fl = 0;
+  if (r < rows) {
+    const int32_t d = dslot[r];
+    fl = d < 0 || bcount[d / kPanelRows] >= 0 ? 1u : 0u;
+  }
+  flag[r] = fl;  // flag[rows] = 0: the place of the scan's total
+}
+
+__global__ __launch_bounds__(kSpmmThreads) void panel_finish_list_kernel(const uint32_t *__restrict__ flag,
+                                                                         const uint32_t *__restrict__ pos, int32_t rows,
+                                                                         int32_t *__restrict__ list) {
+  const int64_t r = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  if (r < rows && flag[r]) list[pos[r]] = (int32_t)r;
 }
 
 // first[k] = wptr[16 k]: the first record of tile k (k = tiles: all records)

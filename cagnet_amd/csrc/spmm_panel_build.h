@@ -539,6 +539,22 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   }
   panel_dslot_kernel<<<gn, kSpmmThreads, 0, stream>>>(row_rank, n, d_panel_unit, (int32_t)npanels, pp.dslot);
   CG_LAUNCH_CHECK();
+  {  // the rows the pass over the partial rows writes
+    uint32_t *flag = nullptr, *pos = nullptr, *d_count = nullptr, h_count = 0;
+    CG_TRY(tmp.alloc((void **)&flag, (size_t)(n + 1) * 4));
+    CG_TRY(tmp.alloc((void **)&pos, (size_t)(n + 1) * 4));
+    CG_TRY(tmp.alloc((void **)&d_count, 4));
+    const unsigned gn1 = (unsigned)ceil_div64((int64_t)n + 1, kSpmmThreads);
+    panel_finish_flag_kernel<<<gn1, kSpmmThreads, 0, stream>>>(pp.dslot, pp.bcount, n, flag);
+    CG_LAUNCH_CHECK();
+    CG_TRY(exclusive_scan_u32(flag, pos, (int64_t)n + 1, d_count, stream));
+    CG_HIP(hipMemcpyAsync(&h_count, d_count, 4, hipMemcpyDeviceToHost, stream));
+    CG_HIP(hipStreamSynchronize(stream));
+    CG_TRY(dev_alloc((void **)&pp.finish_rows, (size_t)(h_count > 0 ? h_count : 1) * 4));
+    panel_finish_list_kernel<<<gn1, kSpmmThreads, 0, stream>>>(flag, pos, n, pp.finish_rows);
+    CG_LAUNCH_CHECK();
+    pp.nfinish = (int32_t)h_count;
+  }
   CG_HIP(hipStreamSynchronize(stream));
   pp.covered = covered;
   pp.dcovered = dcovered;
@@ -704,11 +720,12 @@ static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_
 }
 
 // C = beta C + the partial rows (every block of a row's panel), for a plan without a rest matrix to multiply
-static int launch_panel_finish(const PanelPlan &pp, const float *P, float *C, int64_t ldc, int32_t rows, int32_t f, float beta,
-                               hipStream_t stream, bool direct_written) {
+static int launch_panel_finish(const PanelPlan &pp, const float *P, float *C, int64_t ldc, int32_t f, float beta,
+                               hipStream_t stream) {
   ProfScope prof("spmm_panel_add", f, stream);
-  panel_finish_kernel<<<(unsigned)ceil_div64((int64_t)rows * (f / 2), kSpmmThreads), kSpmmThreads, 0, stream>>>(
-      C, ldc, P, pp.dslot, pp.bcount, rows, f, beta, direct_written ? 1 : 0);
+  if (pp.nfinish == 0) return CG_OK;
+  panel_finish_kernel<<<(unsigned)ceil_div64((int64_t)pp.nfinish * (f / 2), kSpmmThreads), kSpmmThreads, 0, stream>>>(
+      C, ldc, P, pp.dslot, pp.bcount, pp.finish_rows, pp.nfinish, f, beta);
   CG_LAUNCH_CHECK();
   return CG_OK;
 }
