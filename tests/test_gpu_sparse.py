@@ -1154,6 +1154,40 @@ def test_captured_graph_outlives_plan_eviction_and_scratch_growth(cuda, tune):
     s.synchronize()
 
 
+def test_captured_panel_product_replays(cuda, tune):
+    """A product with the panel plan, captured into a HIP graph: the staged-tile kernel takes its units from queues
+    whose counters a small kernel of the same capture zeroes, so every replay — with eager products of the same
+    handle on the same stream in between — gives the eager result bit for bit, also with beta != 0."""
+    from cagnet_amd import ops
+    row, col, val, n = small_graph(12, 120000, seed=41)
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n)
+    tune("spmm_panel", 1)
+    tune("spmm_panel_unit", 4096)             # many units per queue
+    f = 300
+    B = torch.randn(n, f, generator=torch.Generator().manual_seed(1)).to(cuda)
+    C0 = torch.randn(n, f, generator=torch.Generator().manual_seed(2)).to(cuda)
+    C = C0.clone()
+    s = torch.cuda.Stream(device=cuda)
+    s.wait_stream(torch.cuda.current_stream(cuda))
+    with torch.cuda.stream(s):
+        A.spmm(B, out=C, beta=0.5)            # builds the plan: not possible under capture
+    s.synchronize()
+    assert _panel_info(A)["state"] == 1 and _panel_info(A)["units"] > 16
+    expect = C.clone()
+    g = torch.cuda.CUDAGraph()
+    C.copy_(C0)
+    with torch.cuda.graph(g, stream=s):
+        A.spmm(B, out=C, beta=0.5)
+    for k in range(3):
+        C.copy_(C0)
+        g.replay()
+        s.synchronize()
+        assert torch.equal(C, expect), k
+        with torch.cuda.stream(s):
+            assert spmm_error(A.spmm(B), row, col, val, n, n, B.cpu()) <= REL_TOL
+        s.synchronize()
+
+
 def test_plan_build_that_runs_out_of_memory_falls_back_for_good(cuda, tune):
     """An allocation failure while a hub or panel plan is built must not fail the product: it runs on the
     plain schedule, and the plan is not tried again on later calls."""
