@@ -15,10 +15,13 @@
 // (v_mfma_f32_16x16x4_f32: exact fp32 products, fp32 accumulation) by a second kernel, in units of
 // their own; the zeros of such a block are multiplied too, so a row of B that holds an infinity or a
 // NaN reaches every row of the block (the row-wise kernels and cusparseSpMM would only touch the rows
-// that reference it).  By default every tile is multiplied by one of the two kernels and a last pass
-// writes C = beta C + the partial rows; tiles that a threshold leaves out keep their entries in a
-// second CSR matrix (the "rest") that the row-wise kernels multiply, and their finished rows add the
-// partial rows in.  Replaces nothing in the reference beyond cusparseSpMM itself
+// that reference it).  By default every tile is multiplied by one of the two kernels; a unit that is
+// the only one of its panel writes C = beta C + its rows itself, and a last pass writes the other rows
+// as C = beta C + the sum of their panel's partial rows.  Tiles that a threshold leaves out keep their
+// entries in a second CSR matrix (the "rest") that the row-wise kernels multiply, and their finished
+// rows add the partial rows in.  The staged-tile kernel runs one workgroup per compute unit; the units
+// wait in one queue per XCD (neighbouring panels' units, which walk the same rows of B, one behind the
+// other, so that they share that XCD's L2) and a workgroup takes units until all queues are empty.  Replaces nothing in the reference beyond cusparseSpMM itself
 // (sparse-extension/sparse_coo_tensor.cu:215-226); sums are in a fixed order, no atomics on floats.
 #pragma once
 #include "spmm_tables.h"
