@@ -37,11 +37,11 @@ static bool want_panel(const CsrSide &s, int32_t f) {
   const int t = g_tune_panel.load(std::memory_order_relaxed);
   if (t < 0 || !panel_width_ok(f) || s.rows == 0 || s.nnz == 0) return false;
   if (t > 0) return true;
-  // Below about 5e9 multiply-adds the plan's fixed costs (a block of partial rows per unit, few units per compute
+  // Below about 8e8 multiply-adds the plan's fixed costs (a block of partial rows per unit, few units per compute
   // unit) outweigh what it saves: blocks of a 4 x 4 grid over 232,965 vertices at f = 602, plan against row-wise
-  // kernels: 0.6 M entries 0.69 / 0.30 ms, 1.7 M 0.74 / 0.58, 5.4 M 1.02 / 1.29 and 1.39 / 1.17, 12.5 M 1.52 / 2.03,
-  // 29.4 M 2.38 / 4.33 ms.
-  return s.nnz / s.rows >= 8 && (double)s.nnz * f >= 5e9;
+  // kernels: 0.6 M entries 0.29 / 0.30 ms, 1.6 M 0.41 / 0.54, 1.7 M 0.48 / 0.58, 5.4 M 0.87 / 1.17 and 0.87 / 1.29,
+  // 12.5 M 1.28 / 2.02, 29.4 M 2.07 / 4.31 ms.
+  return s.nnz / s.rows >= 8 && (double)s.nnz * f >= 8e8;
 }
 
 static int alloc_sort_buffers(DevTemps &tmp, SortBuffers &buf, int64_t count) {
@@ -383,22 +383,51 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   std::vector<Unit> su, du;  // units of active tiles, of dense tiles; both in panel order
   constexpr int32_t kUnitGrid = 32;  // with shared column order a unit starts where a panel's block number passes a multiple
   constexpr int32_t kXcds = kXcdQueues;  // XCDs of the device
+  // What a run of tiles costs, in microseconds: a tile with e records 1.50 + 0.0034 e + 8.7e-6 e^2 (fitted to the
+  // durations of the 3744 units of the matrix with 232,965 vertices and 492 entries per row at f = 602: 3.4 % off
+  // in the median; a tile costs its copies and its barrier whatever it holds, and the waves' records run the more
+  // unevenly the more of them a tile has).  Only ratios matter.  A unit is also cut when it has an eighth of a
+  // compute unit's share of the whole cost (at least 100 us), so that a small matrix still gets balanced work.
+  auto tile_cost = [&](int64_t t) {
+    const double e = (double)(h_base[(size_t)t + 1] - h_base[(size_t)t]);
+    return 1.50 + 0.0034 * e + 8.7e-6 * e * e;
+  };
+  double cost_cap = 100.0;
+  {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        cus < 1) {
+      (void)hipGetLastError();
+      cus = 256;
+    }
+    double total = 0.0;
+    for (int64_t t = 0; t < ntiles; ++t) total += tile_cost(t);
+    if (total / (8.0 * cus) > cost_cap) cost_cap = total / (8.0 * cus);
+  }
   for (int64_t k = 0; k < ntiles;) {
     int64_t j = k, in_unit = 0;
-    // a panel of up to one and a half units' records stays whole: its unit is then its only block and writes C itself
-    int64_t pend = k;
-    while (pend < ntiles && h_panel[(size_t)pend] == h_panel[(size_t)k]) ++pend;
-    const bool whole = (k == 0 || h_panel[(size_t)k - 1] != h_panel[(size_t)k]) &&
-                       (int64_t)h_base[(size_t)pend] - h_base[(size_t)k] <= (int64_t)unit_entries + unit_entries / 2;
+    double unit_cost = 0.0;
+    // a panel of up to one and a half units' records and cost stays whole: its unit is then its only block and
+    // writes C itself
+    bool whole = k == 0 || h_panel[(size_t)k - 1] != h_panel[(size_t)k];
+    if (whole) {
+      int64_t pend = k;
+      double pcost = 0.0;
+      for (; pend < ntiles && h_panel[(size_t)pend] == h_panel[(size_t)k]; ++pend) pcost += tile_cost(pend);
+      whole = (int64_t)h_base[(size_t)pend] - h_base[(size_t)k] <= (int64_t)unit_entries + unit_entries / 2 && pcost <= 1.5 * cost_cap;
+    }
     while (j < ntiles && h_panel[(size_t)j] == h_panel[(size_t)k]) {
       const int64_t e = (int64_t)h_base[(size_t)j + 1] - h_base[(size_t)j];
       if (whole) {
       } else if (share) {
-        if (j > k && in_unit >= unit_entries / 2 && h_kb[(size_t)j] / kUnitGrid != h_kb[(size_t)j - 1] / kUnitGrid) break;
-      } else if (j > k && in_unit + e > unit_entries) {
+        if (j > k && (in_unit >= unit_entries / 2 || unit_cost >= cost_cap) &&
+            h_kb[(size_t)j] / kUnitGrid != h_kb[(size_t)j - 1] / kUnitGrid)
+          break;
+      } else if (j > k && (in_unit + e > unit_entries || unit_cost >= cost_cap)) {
         break;
       }
       in_unit += e;
+      unit_cost += tile_cost(j);
       ++j;
     }
     su.push_back(Unit{h_panel[(size_t)k], (int32_t)k, (int32_t)j, in_unit});
@@ -441,10 +470,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   for (int32_t u = 0; u < ndunits; ++u) dunit_tile[(size_t)u + 1] = du[(size_t)u].t1;
   std::vector<int32_t> order((size_t)nunits);
   for (int32_t u = 0; u < nunits; ++u) order[(size_t)u] = u;
-  // What a unit costs, in microseconds, from its tiles T and its records R: T (1.50 + 0.0034 R/T + 8.7e-6 (R/T)^2) fits
-  // the durations of the 3744 units of the matrix with 232,965 vertices and 492 entries per row at f = 602 to 3.4 % in
-  // the median (a tile costs its copies and its barrier whatever it holds, and the waves' records run the more
-  // unevenly the more of them a tile has).  Only ratios matter: the launch order goes by it.
+  // the launch order goes by the units' costs (a unit's tiles taken as alike)
   auto cost = [&](int32_t u) {
     const double T = (double)(su[(size_t)u].t1 - su[(size_t)u].t0), R = (double)su[(size_t)u].weight;
     return T > 0.0 ? 1.50 * T + 0.0034 * R + 8.7e-6 * R * R / T : 0.0;

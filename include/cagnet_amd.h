@@ -349,7 +349,7 @@ int cg_prof_enable(int on);
  *   "spmm_hub_tiers"  tiers of hot columns (0: chosen from the column counts; groups * tiers <= 64)
  *   "spmm_hub_row"    rows with fewer entries keep all of them in the cold class (0: 64)
  *   "spmm_panel"      panel plan (dense row-panel x column-block tiles multiplied out of LDS; even widths
- *                     258..636): -1 never, 1 always, 0 when the product has at least 5e9 multiply-adds, rows hold at
+ *                     258..636): -1 never, 1 always, 0 when the product has at least 8e8 multiply-adds, rows hold at
  *                     least 8 entries on average and at least half of the entries share their column with another
  *                     entry of the same panel of 128 rows
  *   "spmm_panel_emin" entries a 128 x 32 tile needs to be staged (0: 1, every tile; tiles below it leave their
