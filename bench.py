@@ -202,7 +202,7 @@ def run_epochs(prob, spec, blk, steps: int, warmup: int, optimizer: str, keep_lo
     layer, gcn_distr.py:271-275), so that the dominant kernel is exactly the f = f_in SpMM."""
     import torch
 
-    from cagnet_amd import _lib, gcn
+    from cagnet_amd import _lib, gcn, ops
 
     n, f_in, hidden, classes = prob.n, spec["features"], spec["hidden"], spec["classes"]
 
@@ -211,6 +211,15 @@ def run_epochs(prob, spec, blk, steps: int, warmup: int, optimizer: str, keep_lo
         train_mask = prob.train_mask
 
     x = prob.x.requires_grad_(True)  # the reference asks for the input gradient too (gcn_distr.py:736)
+    # The features are the same tensor in every epoch (as the reference's are): registered, so that the stage loop
+    # reads them through a copy with line-aligned rows that is made once, in warm-up, outside the timed epochs.
+    ops.keep_aligned(x)
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    copied = ops.aligned_rows(x) is not x
+    ev1.record()
+    torch.cuda.synchronize()
+    aligned_copy_ms = ev0.elapsed_time(ev1) if copied else None
     w1 = prob.w1.clone().requires_grad_(True)
     w2 = prob.w2.clone().requires_grad_(True)
     opt = torch.optim.Adam([w1, w2], lr=0.01) if optimizer == "adam" else torch.optim.SGD([w1, w2], lr=0.01)
@@ -238,7 +247,8 @@ def run_epochs(prob, spec, blk, steps: int, warmup: int, optimizer: str, keep_lo
     _lib.lib.cg_prof_enable(0)
     state["keep"] = False
     kernels = read_kernels(_lib.lib, f_in, hidden, classes)
-    rec = {"epoch_ms": elapsed / steps * 1e3, "final_loss": float(gcn.train.last_loss), "kernels": kernels, "losses": losses}
+    rec = {"epoch_ms": elapsed / steps * 1e3, "final_loss": float(gcn.train.last_loss), "kernels": kernels, "losses": losses,
+           "aligned_copy_ms": aligned_copy_ms}
 
     def timed_variant(count):
         for _ in range(2):
@@ -553,7 +563,11 @@ def main() -> int:
         "data": "synthetic",
         "config": {"workload": spec["desc"], "name": args.workload, "n": n, "nnz": nnz, "features": f_in,
                    "hidden": hidden, "classes": classes, "optimizer": f"{args.optimizer} lr 0.01", "input_grad": True,
-                   "seeds": prob.seeds},
+                   "seeds": prob.seeds,
+                   # X is constant over the epochs and is multiplied through a copy with rows 128-byte aligned, made
+                   # once before the timed region (null: the rows were aligned already, no copy)
+                   "x_row_aligned_copy": rec["aligned_copy_ms"] is not None,
+                   "x_row_aligned_copy_one_off_ms": None if rec["aligned_copy_ms"] is None else round(rec["aligned_copy_ms"], 3)},
         "epoch_ms": round(ms_per_step, 4),
         "scomp_ms_per_epoch": round(spmm_total_ms, 4),
         "dcomp_ms_per_epoch": round(dense_total_ms, 4),

@@ -76,9 +76,6 @@ _SIGNATURES = {
     "cg_add_self_loops": [P, P, c_int64, c_int32, P, P, c_int64, POINTER(c_int64), P],
     "cg_gcn_normalize": [P, P, c_int64, c_int32, P, P, P],
     "cg_coo_block": [P, P, P, c_int64, c_int32, c_int32, c_int32, c_int32, P, P, P, c_int64, POINTER(c_int64), P],
-    "cg_probe_lds_read": [c_int32, c_int32, POINTER(ctypes.c_double)],
-    "cg_probe_stream": [c_int64, c_int32, POINTER(ctypes.c_double)],
-    "cg_probe_mfma_dense": [c_int32, c_int32, POINTER(ctypes.c_double), POINTER(ctypes.c_double)],
     "cg_prof_enable": [c_int],
     "cg_tune_set": [c_char_p, c_int],
     "cg_prof_read": [c_char_p, POINTER(ctypes.c_double), POINTER(c_int64)],

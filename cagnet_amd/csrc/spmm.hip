@@ -344,6 +344,27 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
     d.epi_fo = epi->epi_fo;
     d.epi_relu = epi->epi_relu;
   }
+  // Tile plan: every entry is multiplied out of LDS by spmm_tile_kernel, in panels whose height goes by the width.
+  if (!epi && !fold && allow_panel && want_tile(s, f) &&
+      tile_operands_ok(tile_params(tile_geometry(f)).prows, tile_params(tile_geometry(f)).tcols, B, ldb, f, s.cols)) {
+    const int geom = tile_geometry(f);
+    const PanelParams par = tile_params(geom);
+    const bool may_decline = g_tune_tile.load(std::memory_order_relaxed) == 0;
+    PanelPlan &pp = s.tile[geom];
+    if (!pp.valid || !par.same(pp) || (pp.declined && !may_decline && !pp.failed)) {
+      const int st = build_panel(s, pp, par, may_decline, stream);
+      if (st == CG_ERR_ALLOC || st == CG_ERR_OVERFLOW) {  // no memory for the plan: remembered as declined
+        pp.declined = pp.failed = pp.valid = true;
+      } else if (st != CG_OK) {
+        return st;
+      }
+    }
+    if (!pp.declined && pp.rest->nnz == 0) {
+      float *P = nullptr;
+      CG_TRY(launch_panel(pp, B, ldb, f, &P, stream, false, C, ldc, s.rows, beta));
+      return launch_panel_finish(pp, P, C, ldc, f, beta, stream);
+    }
+  }
   // Panel plan: the entries of dense (row panel, column block) tiles are multiplied out of LDS into
   // partial rows; the row-wise kernels then run over the other entries and add those rows in.
   if (!epi && allow_panel && f <= cap && want_panel(s, f)) {
@@ -826,6 +847,8 @@ int cg_csr_unpin(cg_csr_t *h, int64_t *released) {
     count += s->unpin();
     if (s->panel.rest) count += s->panel.rest->unpin();
     if (s->panel_narrow.rest) count += s->panel_narrow.rest->unpin();
+    for (int i = 0; i < cg::CsrSide::kTilePlans; ++i)
+      if (s->tile[i].rest) count += s->tile[i].rest->unpin();
   }
   if (released) *released = count;
   return CG_OK;
@@ -882,6 +905,7 @@ int cg_tune_set(const char *key, int value) {
   else if (!strcmp(key, "spmm_panel_dmin")) cg::g_tune_panel_dmin.store(value);
   else if (!strcmp(key, "spmm_panel_dwg")) cg::g_tune_panel_dwg.store(value);
   else if (!strcmp(key, "spmm_panel_share")) cg::g_tune_panel_share.store(value);
+  else if (!strcmp(key, "spmm_tile")) cg::g_tune_tile.store(value);
   else if (!strcmp(key, "spmm_panel_narrow")) cg::g_tune_panel_narrow.store(value);
   else if (!strcmp(key, "spmm_panel_narrow_dmin")) cg::g_tune_panel_narrow_dmin.store(value);
   else if (!strcmp(key, "dense_mfma")) cg::g_tune_dense_mfma.store(value);
@@ -919,7 +943,9 @@ int cg_csr_panel_info(const cg_csr_t *h, int transpose, int64_t info[12]) {
   if (!h || !info) CG_FAIL(CG_ERR_NULL, "cg_csr_panel_info: null pointer");
   if ((transpose & 1) && !h->has_t) CG_FAIL(CG_ERR_NO_TRANSPOSE, "cg_csr_panel_info: handle was built without CG_CSR_TRANSPOSE");
   const cg::CsrSide &side = (transpose & 1) ? h->tr : h->fwd;
-  const cg::PanelPlan &pp = (transpose & 2) ? side.panel_narrow : side.panel;
+  // bits 2..3: 0 the plan of the wide products, 1 .. 3 the tile plans with panels of 256, 512, 1024 rows
+  const int which = (transpose >> 2) & 3;
+  const cg::PanelPlan &pp = which ? side.tile[which - 1] : (transpose & 2) ? side.panel_narrow : side.panel;
   const bool used = pp.valid && !pp.declined;
   info[0] = !pp.valid ? 0 : (pp.declined ? -1 : 1);
   info[1] = used ? pp.covered : 0;

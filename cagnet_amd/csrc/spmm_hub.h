@@ -102,6 +102,8 @@ struct CsrSide {
   bool is_rest = false;  // this side is the rest matrix of a panel plan: its dense part is gone already
   PanelPlan panel;  // plan of the wide products that multiply the dense part out of LDS (spmm_panel.h)
   PanelPlan panel_narrow;  // plan of the narrow products: dense tiles only (spmm_panel_narrow.h)
+  static constexpr int kTilePlans = 3;
+  PanelPlan tile[kTilePlans];  // plans of spmm_tile_kernel: panels of 256, 512 and 1024 rows (spmm_tile.h)
   bool pinned = false;          // a product on this side was captured into a graph (spmm_entry)
   std::vector<void *> parked;   // tables replaced since then: a captured graph may still read them
   int64_t unpin() {  // the caller has made sure that no captured graph will replay any more
@@ -116,6 +118,7 @@ struct CsrSide {
     parked.clear();
     panel.release();
     panel_narrow.release();
+    for (int i = 0; i < kTilePlans; ++i) tile[i].release();
     sched.release();
     for (int i = 0; i < kHubPlans; ++i) hub[i].release();
     table_free(rowptr);

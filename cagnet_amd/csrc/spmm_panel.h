@@ -42,7 +42,7 @@ constexpr int kDenseThreads = kDenseWaves * kWave;
 constexpr int kDenseTileFloats = kPanelRows * kPanelCols;
 
 static std::atomic<int> g_tune_panel{0}, g_tune_panel_emin{0}, g_tune_panel_cols{0}, g_tune_panel_unit{0};
-static std::atomic<int> g_tune_panel_dmin{0}, g_tune_panel_dwg{0}, g_tune_panel_share{0};
+static std::atomic<int> g_tune_panel_dmin{0}, g_tune_panel_dwg{0}, g_tune_panel_share{0}, g_tune_tile{0};
 
 struct CsrSide;
 
@@ -50,9 +50,13 @@ struct PanelPlan {
   bool valid = false, declined = false, failed = false;  // failed: declined because the build ran out of memory
   int32_t emin = 0, hot_cols = 0, unit_entries = 0, dmin = 0, dwg = 0;  // what the plan was built with
   bool share = true;
+  int32_t prows = 128, tcols = 32;  // rows of a panel (a multiple of 16) and columns of a tile (a multiple of 16, at most
+                                    // 256); the matrix-core kernels and spmm_panel_kernel need 128 x 32
+  bool padded = true;               // odd (tile, wave, slot) runs of records are padded (spmm_panel_kernel needs that)
   int64_t covered = 0;      // entries the panel kernel multiplies
   int64_t dcovered = 0;     // entries in dense tiles (the matrix-core kernel)
   int32_t ntiles = 0, nunits = 0, nsplit = 0;
+  int32_t bcols = 0;               // columns of the matrix = rows of B
   int32_t ndtiles = 0, ndunits = 0;
   int32_t nblocks = 0;             // blocks of 128 partial rows, one per unit of either kind
   int32_t *unit_tile = nullptr;    // [nunits + 1] tiles of a unit (units never span panels)
@@ -85,21 +89,22 @@ struct PanelPlan {
 // -------------------------------------------------------------------------------------------------
 // the product kernel
 // -------------------------------------------------------------------------------------------------
-// One 16-byte (or 4-byte) piece per lane from global memory straight into LDS at lds_addr + lane * size.
+// One 16-byte (or 4-byte) piece per lane from global memory straight into LDS at lds_addr + lane * size (the
+// instruction takes the LDS address from m0, one wait state after the move that sets it).
 // The compiler does not see these loads: it would otherwise wait for them before every LDS read (it
 // cannot tell the two LDS buffers apart); the kernel waits for them itself before the barrier.
 __device__ __forceinline__ void panel_copy16(uint32_t lds_addr, const float *src) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(src) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(src) : "m0", "memory");
 }
 __device__ __forceinline__ void panel_copy4(uint32_t lds_addr, const float *src) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_addr), "v"(src) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_addr), "v"(src) : "m0", "memory");
 }
 // The same with the source as a wave-uniform base and a 32-bit byte offset per lane (no 64-bit address per lane).
 __device__ __forceinline__ void panel_copy16_at(uint32_t lds_addr, const float *base, uint32_t byte_off) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(byte_off), "s"(base) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(byte_off), "s"(base) : "m0", "memory");
 }
 __device__ __forceinline__ void panel_copy4_at(uint32_t lds_addr, const float *base, uint32_t byte_off) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(byte_off), "s"(base) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(byte_off), "s"(base) : "m0", "memory");
 }
 
 // Lanes with byte_off < limit copy 16 (4) bytes from base + byte_off to LDS at lds_addr + lane * 16 (4).
@@ -115,7 +120,7 @@ __device__ __forceinline__ void panel_copy16_if(uint32_t lds_addr, const float *
       "s_mov_b64 exec, %0"
       : "=&s"(saved)
       : "s"(lds_addr), "v"(byte_off), "s"(base), "s"(limit)
-      : "vcc", "scc", "memory");  // s_and writes scc
+      : "vcc", "scc", "m0", "memory");  // s_and writes scc
 }
 __device__ __forceinline__ void panel_copy4_if(uint32_t lds_addr, const float *base, uint32_t byte_off, uint32_t limit) {
   uint64_t saved;
@@ -129,7 +134,7 @@ __device__ __forceinline__ void panel_copy4_if(uint32_t lds_addr, const float *b
       "s_mov_b64 exec, %0"
       : "=&s"(saved)
       : "s"(lds_addr), "v"(byte_off), "s"(base), "s"(limit)
-      : "vcc", "scc", "memory");  // s_and writes scc
+      : "vcc", "scc", "m0", "memory");  // s_and writes scc
 }
 
 // hdr[(tile * 16 + wave) * 4 ..]: the two rows of B the wave stages for the tile and the range of its records.
@@ -501,9 +506,9 @@ __global__ __launch_bounds__(kDenseThreads) void spmm_panel_dense_kernel(
 
 // Panels with several units: the blocks of the later units are added to the first one's, in unit order.
 __global__ __launch_bounds__(kSpmmThreads) void panel_reduce_kernel(const int32_t *__restrict__ split, float *__restrict__ P,
-                                                                    int32_t f) {
+                                                                    int32_t f, int32_t prows) {
   const int32_t first = split[2 * blockIdx.y], count = split[2 * blockIdx.y + 1];
-  const int64_t block = (int64_t)kPanelRows * f;
+  const int64_t block = (int64_t)prows * f;
   const int64_t idx = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (idx >= block) return;
   float *p = P + (int64_t)first * block + idx;
@@ -528,7 +533,7 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_finish_kernel(float *__res
                                                                      const int32_t *__restrict__ dslot,
                                                                      const int32_t *__restrict__ bcount,
                                                                      const int32_t *__restrict__ list, int32_t count,
-                                                                     int32_t f, float beta) {
+                                                                     int32_t f, float beta, int32_t prows) {
   const int32_t half = f >> 1;
   const int64_t idx = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   const int64_t i = idx / half;
@@ -538,11 +543,11 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_finish_kernel(float *__res
   const int32_t d = dslot[r];
   float2 v = make_float2(0.f, 0.f);
   if (d >= 0) {
-    const int32_t blocks = bcount[d / kPanelRows];
+    const int32_t blocks = bcount[d / prows];
     const float *p = P + (int64_t)d * f + c;
     v = *reinterpret_cast<const float2 *>(p);
     for (int32_t k = 1; k < blocks; ++k) {
-      const float2 w = *reinterpret_cast<const float2 *>(p + (int64_t)k * kPanelRows * f);
+      const float2 w = *reinterpret_cast<const float2 *>(p + (int64_t)k * prows * f);
       v.x += w.x;
       v.y += w.y;
     }
@@ -554,6 +559,31 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_finish_kernel(float *__res
   }
   out[0] = v.x;
   out[1] = v.y;
+}
+
+// The same for an odd f: a thread takes one column.
+__global__ __launch_bounds__(kSpmmThreads) void panel_finish1_kernel(float *__restrict__ C, int64_t ldc,
+                                                                      const float *__restrict__ P,
+                                                                      const int32_t *__restrict__ dslot,
+                                                                      const int32_t *__restrict__ bcount,
+                                                                      const int32_t *__restrict__ list, int32_t count,
+                                                                      int32_t f, float beta, int32_t prows) {
+  const int64_t idx = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
+  const int64_t i = idx / f;
+  if (i >= count) return;
+  const int64_t r = list[i];
+  const int32_t c = (int32_t)(idx - i * f);
+  const int32_t d = dslot[r];
+  float v = 0.f;
+  if (d >= 0) {
+    const int32_t blocks = bcount[d / prows];
+    const float *p = P + (int64_t)d * f + c;
+    v = p[0];
+    for (int32_t k = 1; k < blocks; ++k) v += p[(int64_t)k * prows * f];
+  }
+  float *out = C + r * ldc + c;
+  if (beta != 0.f) v += beta * out[0];
+  out[0] = v;
 }
 
 // Entries in (panel, column) pairs that hold at least two entries: every thread walks a stretch of the pairs, a
@@ -621,20 +651,21 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_invert_kernel(const int32_
 // Tiles are numbered panel by panel: panel p has tbase[p + 1] - tbase[p] of them, one per 32 column ranks it uses
 // (at most `hot` ranks).  Tile of an entry from its row rank and its column's rank in the row's panel, -1 for a
 // column rank from `hot` on.
-__device__ __forceinline__ int64_t panel_tile_of(int32_t rrank, int32_t crank, int32_t hot, const int32_t *__restrict__ tbase) {
+__device__ __forceinline__ int64_t panel_tile_of(int32_t rrank, int32_t crank, int32_t hot, const int32_t *__restrict__ tbase,
+                                                 int32_t prows, int32_t tcols) {
   if (crank >= hot) return -1;
-  return (int64_t)tbase[rrank / kPanelRows] + crank / kPanelCols;
+  return (int64_t)tbase[rrank / prows] + crank / tcols;
 }
 
 // blocks[p] = tiles of panel p = ceil(min(column ranks of the panel, hot) / 32); blocks[npanels] = 0 (slot of the scan's total)
 __global__ __launch_bounds__(kSpmmThreads) void panel_tile_base_kernel(const int32_t *__restrict__ pstart, int32_t npanels,
-                                                                       int32_t hot, uint32_t *__restrict__ blocks) {
+                                                                       int32_t hot, int32_t tcols, uint32_t *__restrict__ blocks) {
   const int64_t p = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (p > npanels) return;
   uint32_t b = 0;
   if (p < npanels) {
     const int32_t ranks = pstart[p + 1] - pstart[p];
-    b = (uint32_t)(((ranks < hot ? ranks : hot) + kPanelCols - 1) / kPanelCols);
+    b = (uint32_t)(((ranks < hot ? ranks : hot) + tcols - 1) / tcols);
   }
   blocks[p] = b;
 }
@@ -651,13 +682,13 @@ __device__ __forceinline__ int panel_tile_kind(uint32_t count, uint32_t emin, ui
 // Entries of rows behind the ranked panels get the panel number `npanels`, which sorts them last.
 __global__ __launch_bounds__(kSpmmThreads) void panel_pair_key_kernel(const int32_t *__restrict__ erow,
                                                                       const int32_t *__restrict__ colind, int64_t nnz,
-                                                                      const int32_t *__restrict__ row_rank, int32_t prows,
-                                                                      int32_t npanels, int32_t *__restrict__ kpanel,
+                                                                      const int32_t *__restrict__ row_rank, int32_t ranked_rows,
+                                                                      int32_t npanels, int32_t prows, int32_t *__restrict__ kpanel,
                                                                       int32_t *__restrict__ kcol, int32_t *__restrict__ pos) {
   const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (k >= nnz) return;
   const int32_t rr = row_rank[erow[k]];
-  kpanel[k] = rr < prows ? rr / kPanelRows : npanels;
+  kpanel[k] = rr < ranked_rows ? rr / prows : npanels;
   kcol[k] = colind[k];
   pos[k] = (int32_t)k;
 }
@@ -688,7 +719,7 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_pair_count_key_kernel(
 __global__ __launch_bounds__(kSpmmThreads) void panel_pair_rank_kernel(const int32_t *__restrict__ spanel,
                                                                        const int32_t *__restrict__ spair, int64_t npairs,
                                                                        const int32_t *__restrict__ pstart, int32_t npanels,
-                                                                       int32_t hot, const int32_t *__restrict__ tbase,
+                                                                       int32_t hot, int32_t tcols, const int32_t *__restrict__ tbase,
                                                                        const uint32_t *__restrict__ pair_first,
                                                                        int32_t *__restrict__ pair_lr,
                                                                        uint32_t *__restrict__ tcount) {
@@ -701,7 +732,7 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_pair_rank_kernel(const int
     if (lr >= hot)
       lr = hot;
     else
-      atomicAdd(&tcount[(int64_t)tbase[panel] + lr / kPanelCols], pair_first[pair + 1] - pair_first[pair]);
+      atomicAdd(&tcount[(int64_t)tbase[panel] + lr / tcols], pair_first[pair + 1] - pair_first[pair]);
   }
   pair_lr[pair] = (int32_t)lr;
 }
@@ -720,14 +751,14 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_entry_rank_kernel(const ui
 
 // The column of every place of the active and of the dense tiles, from the ranked pairs: place c of an active
 // tile is staged by wave c % 16 as its row c / 16 (hdr[(tile * 16 + wave) * 4 + c / 16]), place c of a dense
-// tile is dhdr[tile * 32 + c].  Both arrays hold -1 beforehand; a panel's last block can have fewer than 32
+// tile is dhdr[tile * 32 + c] (a header of an active tile has tcols / 16 + 2 ints: 4 for tiles of 32 columns).  Both arrays hold -1 beforehand; a panel's last block can have fewer than 32
 // columns, and its empty places are then given the block's first column (panel_hdr_kernel,
 // panel_dense_hdr_fill_kernel): no entry refers to them, a dense tile holds zeros there.
 __global__ __launch_bounds__(kSpmmThreads) void panel_pair_hdr_kernel(
     const int32_t *__restrict__ spanel, const int32_t *__restrict__ spair, int64_t npairs, const int32_t *__restrict__ pstart,
     int32_t npanels, int32_t hot, const int32_t *__restrict__ tbase, const int32_t *__restrict__ pair_col,
     const uint32_t *__restrict__ tcount,
-    const uint32_t *__restrict__ tindex, const uint32_t *__restrict__ dindex, uint32_t emin, uint32_t dmin,
+    const uint32_t *__restrict__ tindex, const uint32_t *__restrict__ dindex, uint32_t emin, uint32_t dmin, int32_t tcols,
     int32_t *__restrict__ hdr, int32_t *__restrict__ dhdr) {
   const int64_t j = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (j >= npairs) return;
@@ -735,12 +766,13 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_pair_hdr_kernel(
   if (panel >= npanels) return;
   const int64_t lr = j - pstart[panel];
   if (lr >= hot) return;
-  const int64_t t = (int64_t)tbase[panel] + lr / kPanelCols;
-  const int c = (int)(lr % kPanelCols);
+  const int64_t t = (int64_t)tbase[panel] + lr / tcols;
+  const int c = (int)(lr % tcols);
   const int kind = panel_tile_kind(tcount[t], emin, dmin);
   const int32_t col = pair_col[spair[j]];
+  const int hs = tcols / kPanelWaves + 2;  // ints of a (tile, wave) header: its rows of B, then its record range
   if (kind == 1)
-    hdr[((int64_t)tindex[t] * kPanelWaves + c % kPanelWaves) * 4 + c / kPanelWaves] = col;
+    hdr[((int64_t)tindex[t] * kPanelWaves + c % kPanelWaves) * hs + c / kPanelWaves] = col;
   else if (kind == 2)
     dhdr[(int64_t)dindex[t] * kPanelCols + c] = col;
 }
@@ -799,17 +831,17 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_entry_key_kernel(
     const int32_t *__restrict__ erow, const int32_t *__restrict__ ecr, const float *__restrict__ val, int64_t nnz,
     const int32_t *__restrict__ row_rank, int32_t hot, const int32_t *__restrict__ tbase,
     const uint32_t *__restrict__ tcount, const uint32_t *__restrict__ tindex, const uint32_t *__restrict__ dindex,
-    uint32_t emin, uint32_t dmin, int32_t sentinel, int32_t *__restrict__ key, int32_t *__restrict__ slot,
-    int32_t *__restrict__ pos, uint32_t *__restrict__ dA_bits, uint32_t *__restrict__ collision) {
+    uint32_t emin, uint32_t dmin, int32_t sentinel, int32_t prows, int32_t tcols, int32_t *__restrict__ key,
+    int32_t *__restrict__ slot, int32_t *__restrict__ pos, uint32_t *__restrict__ dA_bits, uint32_t *__restrict__ collision) {
   const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (k >= nnz) return;
   const int32_t rr = row_rank[erow[k]];
   const int32_t cr = ecr[k];
-  const int64_t t = panel_tile_of(rr, cr, hot, tbase);
+  const int64_t t = panel_tile_of(rr, cr, hot, tbase, prows, tcols);
   int32_t ky = sentinel, sl = 0;
   const int kind = t >= 0 ? panel_tile_kind(tcount[t], emin, dmin) : 0;
   if (kind == 1) {
-    const int32_t p = rr % kPanelRows;
+    const int32_t p = rr % prows;
     ky = (int32_t)tindex[t] * kPanelWaves + p % kPanelWaves;
     sl = p / kPanelWaves;
   } else if (kind == 2) {
@@ -829,13 +861,13 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_entry_key_kernel(
 __global__ __launch_bounds__(kSpmmThreads) void panel_entry_finish_kernel(
     const int32_t *__restrict__ slot_sorted, const int32_t *__restrict__ pos, int64_t count, int64_t covered,
     const int32_t *__restrict__ erow, const int32_t *__restrict__ colind, const float *__restrict__ val,
-    const int32_t *__restrict__ ecr, uint2 *__restrict__ ent, int32_t *__restrict__ rest_row,
+    const int32_t *__restrict__ ecr, int32_t tcols, uint2 *__restrict__ ent, int32_t *__restrict__ rest_row,
     int32_t *__restrict__ rest_col, float *__restrict__ rest_val) {
   const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (k >= count) return;  // count = entries of active tiles + rest; the entries of dense tiles lie behind them
   const int32_t p = pos[k];
   if (k < covered) {
-    ent[k] = make_uint2((uint32_t)(ecr[p] % kPanelCols) | ((uint32_t)slot_sorted[k] << 8), __float_as_uint(val[p]));
+    ent[k] = make_uint2((uint32_t)(ecr[p] % tcols) | ((uint32_t)slot_sorted[k] << 8), __float_as_uint(val[p]));
   } else {
     rest_row[k - covered] = erow[p];
     rest_col[k - covered] = colind[p];
@@ -894,13 +926,13 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_pad_write_kernel(const uin
 // of panels with several blocks or a dense one
 __global__ __launch_bounds__(kSpmmThreads) void panel_finish_flag_kernel(const int32_t *__restrict__ dslot,
                                                                          const int32_t *__restrict__ bcount, int32_t rows,
-                                                                         uint32_t *__restrict__ flag) {
+                                                                         int32_t prows, uint32_t *__restrict__ flag) {
   const int64_t r = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (r > rows) return;
   uint32_t fl = 0;
   if (r < rows) {
     const int32_t d = dslot[r];
-    fl = d < 0 || bcount[d / kPanelRows] >= 0 ? 1u : 0u;
+    fl = d < 0 || bcount[d / prows] >= 0 ? 1u : 0u;
   }
   flag[r] = fl;  // flag[rows] = 0: the place of the scan's total
 }
@@ -926,29 +958,30 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_pad_wptr_kernel(int32_t *_
   if (j < entries) wptr[j] += (int32_t)shift[wptr[j]];
 }
 
-// hdr[(t * 16 + w) * 4 ..] = {row of B of place w of the tile, the same of place w + 16, first record, end}: the rows
-// are there already (panel_pair_hdr_kernel) except for empty places, which get the row of the tile's place 0
+// hdr[(t * 16 + w) * hs ..] = {rows of B of places w, w + 16, ... of the tile, first record, end}, hs = tcols / 16 + 2:
+// the rows are there already (panel_pair_hdr_kernel) except for empty places, which get the row of the tile's place 0
 __global__ __launch_bounds__(kSpmmThreads) void panel_hdr_kernel(const int32_t *__restrict__ tile_wptr, int64_t ntiles,
-                                                                  int32_t *__restrict__ hdr) {
+                                                                  int32_t tcols, int32_t *__restrict__ hdr) {
   const int64_t k = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (k >= ntiles * kPanelWaves) return;
+  const int tcw = tcols / kPanelWaves, hs = tcw + 2;
   const int64_t t = k / kPanelWaves;
-  const int32_t first = hdr[t * kPanelWaves * 4];  // place 0 of a tile is always taken, and nobody writes it here
-  if (hdr[k * 4 + 1] < 0) hdr[k * 4 + 1] = first;
-  if (k % kPanelWaves != 0 && hdr[k * 4] < 0) hdr[k * 4] = first;
-  hdr[k * 4 + 2] = tile_wptr[k];
-  hdr[k * 4 + 3] = tile_wptr[k + 1];
+  const int32_t first = hdr[t * kPanelWaves * hs];  // place 0 of a tile is always taken, and nobody writes it here
+  for (int j = 0; j < tcw; ++j)
+    if ((j > 0 || k % kPanelWaves != 0) && hdr[k * hs + j] < 0) hdr[k * hs + j] = first;
+  hdr[k * hs + tcw] = tile_wptr[k];
+  hdr[k * hs + tcw + 1] = tile_wptr[k + 1];
 }
 
 __global__ __launch_bounds__(kSpmmThreads) void panel_dslot_kernel(const int32_t *__restrict__ row_rank, int32_t n,
                                                                    const int32_t *__restrict__ panel_unit, int32_t npanels,
-                                                                   int32_t *__restrict__ dslot) {
+                                                                   int32_t prows, int32_t *__restrict__ dslot) {
   const int64_t r = (int64_t)blockIdx.x * kSpmmThreads + threadIdx.x;
   if (r >= n) return;
   const int32_t rr = row_rank[r];
-  const int32_t panel = rr / kPanelRows;
+  const int32_t panel = rr / prows;
   const int32_t u = panel < npanels ? panel_unit[panel] : -1;
-  dslot[r] = u < 0 ? -1 : u * kPanelRows + rr % kPanelRows;
+  dslot[r] = u < 0 ? -1 : u * prows + rr % prows;
 }
 
 __global__ __launch_bounds__(kSpmmThreads) void panel_expand_rows_kernel(const int32_t *__restrict__ rowptr, int32_t n,

@@ -2,6 +2,7 @@
 // device, and the launch of a product's panel part.  Included by spmm.hip after spmm_hub.h.
 #pragma once
 #include "spmm_hub.h"
+#include "spmm_tile.h"
 
 namespace cg {
 
@@ -44,6 +45,17 @@ static bool want_panel(const CsrSide &s, int32_t f) {
   return s.nnz / s.rows >= 8 && (double)s.nnz * f >= 8e8;
 }
 
+// Tile plans (spmm_tile_kernel): the panel height goes by the width of the product.
+//   geometry 0: panels of 256 rows, tiles of 64 columns: widths above 128, in slices of up to 316 columns
+//   geometry 1: 512 x 128: widths 65 .. 128          geometry 2: 1024 x 256: widths up to 64
+static int tile_geometry(int32_t f) { return f <= 64 ? 2 : f <= 128 ? 1 : 0; }
+static bool want_tile(const CsrSide &s, int32_t f) {
+  const int t = g_tune_tile.load(std::memory_order_relaxed);
+  if (t < 0 || s.rows == 0 || s.nnz == 0 || s.is_rest || f < 1) return false;
+  if (t > 0) return true;
+  return false;
+}
+
 static int alloc_sort_buffers(DevTemps &tmp, SortBuffers &buf, int64_t count) {
   for (int i = 0; i < 2; ++i) {
     CG_TRY(tmp.alloc((void **)&buf.key_a[i], (size_t)count * 4));
@@ -63,8 +75,13 @@ constexpr int32_t kPanelDefaultDmin = 768;             // entries from which a 1
 // dwg: workgroups of the dense-tile kernel (each takes an equal share of the dense tiles).
 static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot_req, int32_t unit_entries, int32_t dmin,
                             int32_t dwg, bool share_order, bool may_decline, double min_coverage, double min_reuse,
-                            bool *collision, hipStream_t stream) {
+                            bool *collision, hipStream_t stream, int32_t PR = kPanelRows, int32_t TC = kPanelCols,
+                            bool padded = true) {
   *collision = false;
+  if (PR % kPanelWaves != 0 || TC % kPanelWaves != 0 || TC > 256 || PR / kPanelWaves > 128)
+    CG_FAIL(CG_ERR_UNSUPPORTED, "panel plan: panels of %d rows and tiles of %d columns are not supported", PR, TC);
+  if (PR != kPanelRows || TC != kPanelCols) dmin = 0;  // the matrix-core kernels take 128 x 32 tiles only
+  const int32_t HS = TC / kPanelWaves + 2;            // ints of a (tile, wave) header
   const int64_t nnz = s.nnz;
   const int32_t n = s.rows, m = s.cols;
   auto decline = [&]() {
@@ -74,9 +91,9 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     return CG_OK;
   };
   // column ranks of a panel that can be part of a tile: whole blocks; a panel's last block may be partly empty
-  const int32_t hot = (int32_t)(ceil_div64(hot_req < m ? hot_req : m, kPanelCols) * kPanelCols);
-  if (hot < kPanelCols || n < 1 || nnz < 1) return decline();
-  const int64_t npanels = ceil_div64(n, kPanelRows);
+  const int32_t hot = (int32_t)(ceil_div64(hot_req < m ? hot_req : m, TC) * TC);
+  if (hot < TC || n < 1 || nnz < 1) return decline();
+  const int64_t npanels = ceil_div64(n, PR);
   const int32_t prows = n;  // every row is in a panel
   int64_t tiles = 0;        // all (panel, block) tiles, numbered panel by panel (tbase)
   const unsigned gn = (unsigned)ceil_div64(n, kSpmmThreads);
@@ -127,7 +144,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     CG_TRY(t2.alloc((void **)&start, (size_t)(nnz + 1) * 4));
     CG_TRY(t2.alloc((void **)&runs_before, (size_t)(nnz + 1) * 4));
     CG_TRY(t2.alloc((void **)&d_np, 4));
-    panel_pair_key_kernel<<<ge, kSpmmThreads, 0, stream>>>(erow, s.colind, nnz, row_rank, prows, (int32_t)npanels, buf.key_a[0],
+    panel_pair_key_kernel<<<ge, kSpmmThreads, 0, stream>>>(erow, s.colind, nnz, row_rank, prows, (int32_t)npanels, PR, buf.key_a[0],
                                                            buf.key_b[0], buf.payload[0]);
     CG_LAUNCH_CHECK();
     int set = 0;
@@ -191,7 +208,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
       DevTemps t3;
       SortBuffers pb;
       CG_TRY(alloc_sort_buffers(t3, pb, npairs));
-      const uint32_t cmin = (uint32_t)((emin + kPanelCols - 1) / kPanelCols);  // a block of such columns reaches emin
+      const uint32_t cmin = (uint32_t)((emin + TC - 1) / TC);  // a block of such columns reaches emin
       panel_pair_count_key_kernel<<<gp, kSpmmThreads, 0, stream>>>(pair_first, npairs, buf.key_a[set], buf.key_b[set], col_rank, cmin,
                                                                    m, pb.key_a[0], pb.key_b[0], pb.payload[0], pair_col);
       CG_LAUNCH_CHECK();
@@ -202,7 +219,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
         uint32_t *d_tiles = nullptr, h_tiles = 0;
         CG_TRY(t3.alloc((void **)&d_tiles, 4));
         panel_tile_base_kernel<<<(unsigned)ceil_div64(npanels + 1, kSpmmThreads), kSpmmThreads, 0, stream>>>(
-            pstart, (int32_t)npanels, hot, (uint32_t *)tbase);
+            pstart, (int32_t)npanels, hot, TC, (uint32_t *)tbase);
         CG_LAUNCH_CHECK();
         CG_TRY(exclusive_scan_u32((uint32_t *)tbase, (uint32_t *)tbase, npanels + 1, d_tiles, stream));
         CG_HIP(hipMemcpyAsync(&h_tiles, d_tiles, 4, hipMemcpyDeviceToHost, stream));
@@ -212,7 +229,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
       CG_TRY(tmp.alloc((void **)&tcount, (size_t)(tiles + 1) * 4));
       CG_TRY(fill_u32(tcount, tiles + 1, 0u, stream));
       panel_pair_rank_kernel<<<gp, kSpmmThreads, 0, stream>>>(pb.key_a[pset], pb.payload[pset], npairs, pstart, (int32_t)npanels,
-                                                              hot, tbase, pair_first, pair_lr, tcount);
+                                                              hot, TC, tbase, pair_first, pair_lr, tcount);
       CG_LAUNCH_CHECK();
       CG_HIP(hipMemcpyAsync(spanel, pb.key_a[pset], (size_t)npairs * 4, hipMemcpyDeviceToDevice, stream));
       CG_HIP(hipMemcpyAsync(spair, pb.payload[pset], (size_t)npairs * 4, hipMemcpyDeviceToDevice, stream));
@@ -246,7 +263,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   if (ntiles + ndtiles == 0 || covered + dcovered == 0 ||
       (may_decline && (double)(covered + dcovered) < min_coverage * (double)nnz))
     return decline();
-  if (ntiles * kPanelWaves + 2 > 0x7fffffffLL || ndtiles * kDenseTileFloats > 0x7fffffffLL * 4) return decline();
+  if (ntiles * kPanelWaves * HS + 2 > 0x7fffffffLL || ndtiles * kDenseTileFloats > 0x7fffffffLL * 4) return decline();
 
   // 3. tables of the active and of the dense tiles; the columns of their places
   int32_t *tile_panel = nullptr, *tile_kb = nullptr, *tile_wptr = nullptr, *dtile_panel = nullptr;
@@ -256,8 +273,8 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, tindex, tiles, (uint32_t)emin, (uint32_t)dmin, 1, tbase,
                                                            (int32_t)npanels, tile_panel, tile_kb);
   CG_LAUNCH_CHECK();
-  CG_TRY(dev_alloc((void **)&pp.hdr, (size_t)(ntiles > 0 ? ntiles : 1) * kPanelWaves * 16));
-  CG_TRY(fill_u32((uint32_t *)pp.hdr, ntiles * kPanelWaves * 4, 0xffffffffu, stream));
+  CG_TRY(dev_alloc((void **)&pp.hdr, (size_t)(ntiles > 0 ? ntiles : 1) * kPanelWaves * HS * 4));
+  CG_TRY(fill_u32((uint32_t *)pp.hdr, ntiles * kPanelWaves * HS, 0xffffffffu, stream));
   if (ndtiles > 0) {
     panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, dindex, tiles, (uint32_t)emin, (uint32_t)dmin, 2, tbase,
                                                              (int32_t)npanels, dtile_panel, nullptr);
@@ -269,7 +286,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   }
   panel_pair_hdr_kernel<<<(unsigned)ceil_div64(npairs, kSpmmThreads), kSpmmThreads, 0, stream>>>(
       spanel, spair, npairs, pstart, (int32_t)npanels, hot, tbase, pair_col, tcount, tindex, dindex, (uint32_t)emin, (uint32_t)dmin,
-      pp.hdr, pp.dhdr);
+      TC, pp.hdr, pp.dhdr);
   CG_LAUNCH_CHECK();
   if (ndtiles > 0) {
     panel_dense_hdr_fill_kernel<<<(unsigned)ceil_div64(ndtiles * kPanelCols, kSpmmThreads), kSpmmThreads, 0, stream>>>(pp.dhdr,
@@ -299,23 +316,28 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     CG_TRY(t2.alloc((void **)&rest_row, (size_t)(nrest > 0 ? nrest : 1) * 4));
     const int32_t sentinel = (int32_t)(ntiles * kPanelWaves);
     panel_entry_key_kernel<<<ge, kSpmmThreads, 0, stream>>>(erow, ecr, s.val, nnz, row_rank, hot, tbase, tcount,
-                                                            tindex, dindex, (uint32_t)emin, (uint32_t)dmin, sentinel,
+                                                            tindex, dindex, (uint32_t)emin, (uint32_t)dmin, sentinel, PR, TC,
                                                             buf.key_a[0], buf.key_b[0], buf.payload[0], (uint32_t *)pp.dA,
                                                             d_tot + 4);
     CG_LAUNCH_CHECK();
     int set = 0;
-    CG_TRY(radix_sort_pairs(buf, nnz, bits_for(sentinel + 2), bits_for(kPanelSlots), &set, stream));
+    CG_TRY(radix_sort_pairs(buf, nnz, bits_for(sentinel + 2), bits_for(PR / kPanelWaves), &set, stream));
     uint2 *ent_raw = nullptr;  // the records before padding
     CG_TRY(t2.alloc((void **)&ent_raw, (size_t)(covered > 0 ? covered : 1) * 8));
     if (covered + nrest > 0) {
       panel_entry_finish_kernel<<<(unsigned)ceil_div64(covered + nrest, kSpmmThreads), kSpmmThreads, 0, stream>>>(
-          buf.key_b[set], buf.payload[set], covered + nrest, covered, erow, s.colind, s.val, ecr, ent_raw, rest_row,
+          buf.key_b[set], buf.payload[set], covered + nrest, covered, erow, s.colind, s.val, ecr, TC, ent_raw, rest_row,
           rest.colind, rest.val);
       CG_LAUNCH_CHECK();
     }
     CG_TRY(launch_rowptr(buf.key_a[set], covered, sentinel, tile_wptr, stream));
-    // runs of odd length get a padding record
-    {
+    // runs of odd length get a padding record (spmm_panel_kernel takes the records of a run two at a time)
+    if (!padded) {
+      if (covered > 0x7fffffffLL) CG_FAIL(CG_ERR_OVERFLOW, "panel plan: records exceed the int32 range");
+      pp.nrec = covered;
+      CG_TRY(dev_alloc((void **)&pp.ent, (size_t)(covered > 0 ? covered : 1) * 8));
+      if (covered > 0) CG_HIP(hipMemcpyAsync(pp.ent, ent_raw, (size_t)covered * 8, hipMemcpyDeviceToDevice, stream));
+    } else {
       uint32_t *start = nullptr, *runs_before = nullptr, *run_first = nullptr, *padf = nullptr, *shift = nullptr;
       CG_TRY(t2.alloc((void **)&start, (size_t)(covered + 1) * 4));
       CG_TRY(t2.alloc((void **)&runs_before, (size_t)(covered + 1) * 4));
@@ -347,7 +369,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     }
     if (ntiles > 0) {
       panel_hdr_kernel<<<(unsigned)ceil_div64(ntiles * kPanelWaves, kSpmmThreads), kSpmmThreads, 0, stream>>>(tile_wptr, ntiles,
-                                                                                                              pp.hdr);
+                                                                                                              TC, pp.hdr);
       CG_LAUNCH_CHECK();
     }
     CG_TRY(launch_rowptr(rest_row, nrest, n, rest.rowptr, stream));
@@ -459,7 +481,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     bcount[(size_t)first] = nblocks - first;
     if (nblocks - first == 1 && a > 0 && su[a - 1].panel == panel) {  // one block, and a staged unit's: it can write C itself
       bcount[(size_t)first] = -1;
-      unit_row0[a - 1] = panel * kPanelRows;
+      unit_row0[a - 1] = panel * PR;
     }
     if (nblocks - first > 1) {
       split.push_back(first);
@@ -563,7 +585,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     CG_TRY(dev_alloc((void **)&pp.split, split.size() * 4));
     CG_HIP(hipMemcpyAsync(pp.split, split.data(), split.size() * 4, hipMemcpyHostToDevice, stream));
   }
-  panel_dslot_kernel<<<gn, kSpmmThreads, 0, stream>>>(row_rank, n, d_panel_unit, (int32_t)npanels, pp.dslot);
+  panel_dslot_kernel<<<gn, kSpmmThreads, 0, stream>>>(row_rank, n, d_panel_unit, (int32_t)npanels, PR, pp.dslot);
   CG_LAUNCH_CHECK();
   {  // the rows the pass over the partial rows writes
     uint32_t *flag = nullptr, *pos = nullptr, *d_count = nullptr, h_count = 0;
@@ -571,7 +593,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     CG_TRY(tmp.alloc((void **)&pos, (size_t)(n + 1) * 4));
     CG_TRY(tmp.alloc((void **)&d_count, 4));
     const unsigned gn1 = (unsigned)ceil_div64((int64_t)n + 1, kSpmmThreads);
-    panel_finish_flag_kernel<<<gn1, kSpmmThreads, 0, stream>>>(pp.dslot, pp.bcount, n, flag);
+    panel_finish_flag_kernel<<<gn1, kSpmmThreads, 0, stream>>>(pp.dslot, pp.bcount, n, PR, flag);
     CG_LAUNCH_CHECK();
     CG_TRY(exclusive_scan_u32(flag, pos, (int64_t)n + 1, d_count, stream));
     CG_HIP(hipMemcpyAsync(&h_count, d_count, 4, hipMemcpyDeviceToHost, stream));
@@ -583,6 +605,10 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   }
   CG_HIP(hipStreamSynchronize(stream));
   pp.covered = covered;
+  pp.bcols = m;
+  pp.prows = PR;
+  pp.tcols = TC;
+  pp.padded = padded;
   pp.dcovered = dcovered;
   pp.ntiles = (int32_t)ntiles;
   pp.ndtiles = (int32_t)ndtiles;
@@ -598,9 +624,11 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
 struct PanelParams {
   int32_t emin, cols, unit, dmin, dwg;
   bool share;  // staged columns in the whole matrix's order, units launched in XCD groups
+  int32_t prows = kPanelRows, tcols = kPanelCols;  // rows of a panel, columns of a tile
+  bool padded = true;
   bool same(const PanelPlan &pp) const {
     return pp.emin == emin && pp.hot_cols == cols && pp.unit_entries == unit && pp.dmin == dmin && pp.dwg == dwg &&
-           pp.share == share;
+           pp.share == share && pp.prows == prows && pp.tcols == tcols && pp.padded == padded;
   }
   void stamp(PanelPlan &pp) const {
     pp.emin = emin;
@@ -609,6 +637,9 @@ struct PanelParams {
     pp.dmin = dmin;
     pp.dwg = dwg;
     pp.share = share;
+    pp.prows = prows;
+    pp.tcols = tcols;
+    pp.padded = padded;
   }
 };
 
@@ -637,6 +668,18 @@ static PanelParams panel_params() {
   return p;
 }
 
+static PanelParams tile_params(int geom) {
+  PanelParams p = panel_params();
+  p.prows = geom == 0 ? 256 : geom == 1 ? 512 : 1024;
+  p.tcols = geom == 0 ? 64 : geom == 1 ? 128 : 256;
+  p.padded = false;
+  p.emin = 1;                 // every tile is staged: nothing is left for the row-wise kernels
+  p.cols = kPanelDefaultCols;
+  p.dmin = 0;                 // no tiles for the matrix cores
+  if (g_tune_panel_unit.load(std::memory_order_relaxed) <= 0) p.unit = kPanelDefaultUnit * (p.prows / kPanelRows);
+  return p;
+}
+
 // Builds the plan for the given values; the plan carries them whatever the outcome (in use, declined).
 static int build_panel(CsrSide &s, PanelPlan &pp, const PanelParams &par, bool may_decline, hipStream_t stream,
                        double min_coverage = 0.0, double min_reuse = kPanelMinReuse) {
@@ -645,12 +688,11 @@ static int build_panel(CsrSide &s, PanelPlan &pp, const PanelParams &par, bool m
   pp.release();
   bool collision = false;
   int st = build_panel_once(s, pp, par.emin, par.cols, par.unit, par.dmin, par.dwg, par.share, may_decline, min_coverage, min_reuse,
-                            &collision,
-                            stream);
+                            &collision, stream, par.prows, par.tcols, par.padded);
   if (st == CG_OK && collision) {  // the matrix stores a (row, column) pair twice: every tile goes the record way
     pp.release();
     st = build_panel_once(s, pp, par.emin, par.cols, par.unit, 0, par.dwg, par.share, may_decline, min_coverage, min_reuse, &collision,
-                          stream);
+                          stream, par.prows, par.tcols, par.padded);
   }
   if (st != CG_OK) pp.release();
   par.stamp(pp);
@@ -669,6 +711,103 @@ static int panel_lds_attr(K kernel, std::atomic<uint64_t> &done, int dev, size_t
   return CG_OK;
 }
 
+// Slices of a product of width f on a plan with panels of `prows` rows: a wave owns prows / 16 rows and has 80
+// accumulator registers, so a row of a slice takes at most 80 / (prows / 16) registers (see spmm_tile.h for the
+// widths the register layouts cover), and two tiles of the slice's rows of B must fit the LDS.
+struct TileShape {
+  int32_t nr = 0, nsl = 0, fsw = 0;  // registers per row, slices, columns of a slice (a multiple of 4)
+};
+static bool tile_shape(int32_t prows, int32_t tcols, int32_t f, TileShape &sh) {
+  const int32_t R = prows / kPanelWaves;
+  int32_t cap = R <= 8 ? 636 : R <= 16 ? 316 : R <= 32 ? 128 : R <= 64 ? 64 : 0;
+  const int32_t lds_cap = (int32_t)((160 * 1024 - 64) / (2 * (size_t)tcols) / 16 * 4);  // columns two tiles leave room for
+  if (lds_cap < cap) cap = lds_cap;
+  if (cap < 4 || f < 1) return false;
+  sh.nsl = (f + cap - 1) / cap;
+  sh.fsw = ((f + sh.nsl - 1) / sh.nsl + 3) & ~3;
+  if (sh.fsw > cap) sh.fsw = cap & ~3;
+  sh.nsl = (f + sh.fsw - 1) / sh.fsw;
+  if (R <= 8)
+    sh.nr = sh.fsw > 512 ? 10 : 8;
+  else if (R <= 16)
+    sh.nr = sh.fsw > 256 ? 5 : 4;
+  else
+    sh.nr = R <= 32 ? 2 : 1;
+  return true;
+}
+
+// Can spmm_tile_kernel read this B?  Its copies move 16 bytes per lane straight into LDS, from addresses that must
+// be multiples of 8 (measured: rows 4 bytes off give wrong data); narrow slices address B by 32-bit offsets and copy
+// whole 16-byte pieces only.
+static bool tile_operands_ok(int32_t prows, int32_t tcols, const float *B, int64_t ldb, int32_t f, int32_t m) {
+  TileShape sh;
+  if (!tile_shape(prows, tcols, f, sh)) return false;
+  if (((uintptr_t)B & 7u) != 0 || (ldb & 1) != 0 || ldb > 0x7fffffffLL) return false;
+  if (sh.nr < 4) {
+    if (f % 4 != 0) return false;
+    if ((int64_t)m * ldb * 4 >= (int64_t)1 << 32) return false;
+    if (((uintptr_t)B & 15u) != 0 || (ldb & 3) != 0) return false;  // every piece of a narrow row on a 16-byte boundary
+  }
+  return true;
+}
+
+// The staged tiles of a plan through spmm_tile_kernel (any width; panels of 128, 256, 512 or 1024 rows).
+static int launch_tile(const PanelPlan &pp, const float *B, int64_t ldb, int32_t f, float *P, int32_t *qhead, float *C_direct,
+                       int64_t ldc, int32_t rows, float beta, int dev, int cus, hipStream_t stream) {
+  TileShape sh;
+  if (!tile_shape(pp.prows, pp.tcols, f, sh)) CG_FAIL(CG_ERR_UNSUPPORTED, "tile product: no kernel for f=%d", f);
+  TileArgs ta{};
+  ta.unit_tile = pp.unit_tile;
+  ta.unit_order = pp.unit_order;
+  ta.unit_qstart = pp.unit_qstart;
+  ta.qhead = qhead;
+  ta.unit_block = pp.unit_block;
+  ta.hdr = pp.hdr;
+  ta.ent = pp.ent;
+  ta.B = B;
+  ta.ldb = ldb;
+  ta.P = P;
+  ta.f = f;
+  ta.fsw = sh.fsw;
+  ta.nsl = sh.nsl;
+  ta.m = pp.bcols;
+  ta.unit_row0 = pp.unit_row0;
+  ta.rank_row = pp.rank_row;
+  ta.C = C_direct;
+  ta.ldc = ldc;
+  ta.rows = rows;
+  ta.beta = beta;
+  ta.dbg = g_tune_tile.load(std::memory_order_relaxed) > 0 ? (g_tune_tile.load(std::memory_order_relaxed) & ~1) : 0;
+  // two tiles of staged rows (narrow slices: a wave's staging area is a whole number of 1 KiB pieces) and some room
+  // behind them: the lanes of a row read beyond the slice's last column
+  const size_t tlds_max = 160 * 1024 - 64;
+  const size_t rs = (size_t)sh.fsw * 4;
+  const size_t area = sh.nr >= 4 ? (size_t)(pp.tcols / kPanelWaves) * rs
+                                 : (size_t)ceil_div64((int64_t)(pp.tcols / kPanelWaves) * (sh.fsw / 4), kWave) * (kWave * 16);
+  size_t tlds = 2 * (size_t)kPanelWaves * area + 256;
+  if (tlds > tlds_max) tlds = tlds_max;
+  if (2 * (size_t)kPanelWaves * area > tlds_max) CG_FAIL(CG_ERR_UNSUPPORTED, "tile product: f=%d does not fit the LDS", f);
+  const int64_t items = (int64_t)pp.nunits * sh.nsl;
+  const unsigned grid = (unsigned)(items < cus ? items : cus);
+#define CG_TILE(NR, R, TCW)                                                                        \
+  {                                                                                                \
+    static std::atomic<uint64_t> attr_set{0};                                                      \
+    CG_TRY(panel_lds_attr(spmm_tile_kernel<NR, R, TCW>, attr_set, dev, tlds_max, tlds));           \
+    spmm_tile_kernel<NR, R, TCW><<<grid, kPanelThreads, tlds, stream>>>(ta);                       \
+  }
+  const int32_t R = pp.prows / kPanelWaves, TCW = pp.tcols / kPanelWaves;
+  if (R == 8 && TCW == 2 && sh.nr == 10) CG_TILE(10, 8, 2)
+  else if (R == 8 && TCW == 2 && sh.nr == 8) CG_TILE(8, 8, 2)
+  else if (R == 16 && TCW == 4 && sh.nr == 5) CG_TILE(5, 16, 4)
+  else if (R == 16 && TCW == 4 && sh.nr == 4) CG_TILE(4, 16, 4)
+  else if (R == 32 && TCW == 8 && sh.nr == 2) CG_TILE(2, 32, 8)
+  else if (R == 64 && TCW == 16 && sh.nr == 1) CG_TILE(1, 64, 16)
+  else CG_FAIL(CG_ERR_UNSUPPORTED, "tile product: no kernel for panels of %d rows and tiles of %d columns", pp.prows, pp.tcols);
+#undef CG_TILE
+  CG_LAUNCH_CHECK();
+  return CG_OK;
+}
+
 // The panel part of C = A B: partial rows of every row that has entries in active or dense tiles, in *P
 // (row r: P + dslot[r] * f).  P is stream scratch and stays valid until the next panel product on `stream`.
 // sum_blocks: add the blocks of a panel into its first one (false: the caller's pass over the partial rows does that)
@@ -683,7 +822,7 @@ static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_
   const size_t lds = 2 * (size_t)kPanelCols * rs;  // two tiles of staged rows
   const size_t lds_max = 2 * (size_t)kPanelCols * ((kPanelMaxF * 4 + 15) & ~15);
   void *p = nullptr;
-  const size_t p_bytes = ((size_t)pp.nblocks * kPanelRows * f * sizeof(float) + 15) & ~(size_t)15;
+  const size_t p_bytes = ((size_t)pp.nblocks * pp.prows * f * sizeof(float) + 15) & ~(size_t)15;
   CG_TRY(scratch_get(stream, kSlotE, p_bytes + kXcdQueues * sizeof(int32_t), &p));
   float *P = (float *)p;
   int32_t *qhead = (int32_t *)((char *)p + p_bytes);  // the queues' counters of this launch (panel_take_unit)
@@ -723,7 +862,12 @@ static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_
                                                                                pp.hdr, pp.ent, B, ldb, P, f, pp.unit_row0, \
                                                                                pp.rank_row, C_direct, ldc, rows, beta); \
   } break;
-    if (pp.nunits > 0) {
+    const bool legacy = pp.padded && pp.prows == kPanelRows && pp.tcols == kPanelCols && panel_width_ok(f) &&
+                        g_tune_tile.load(std::memory_order_relaxed) <= 0;
+    if (pp.nunits > 0 && !legacy) {
+      CG_TRY(fill_u32((uint32_t *)qhead, kXcdQueues, 0u, stream));
+      CG_TRY(launch_tile(pp, B, ldb, f, P, qhead, C_direct, ldc, rows, beta, dev, cus, stream));
+    } else if (pp.nunits > 0) {
       CG_TRY(fill_u32((uint32_t *)qhead, kXcdQueues, 0u, stream));
       switch (chunks) {
         CG_PANEL(3)
@@ -736,8 +880,8 @@ static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_
     }
 #undef CG_PANEL
     if (sum_blocks && pp.nsplit > 0) {
-      const dim3 grid((unsigned)ceil_div64((int64_t)kPanelRows * f, kSpmmThreads), (unsigned)pp.nsplit);
-      panel_reduce_kernel<<<grid, kSpmmThreads, 0, stream>>>(pp.split, P, f);
+      const dim3 grid((unsigned)ceil_div64((int64_t)pp.prows * f, kSpmmThreads), (unsigned)pp.nsplit);
+      panel_reduce_kernel<<<grid, kSpmmThreads, 0, stream>>>(pp.split, P, f, pp.prows);
       CG_LAUNCH_CHECK();
     }
   }
@@ -750,8 +894,12 @@ static int launch_panel_finish(const PanelPlan &pp, const float *P, float *C, in
                                hipStream_t stream) {
   ProfScope prof("spmm_panel_add", f, stream);
   if (pp.nfinish == 0) return CG_OK;
-  panel_finish_kernel<<<(unsigned)ceil_div64((int64_t)pp.nfinish * (f / 2), kSpmmThreads), kSpmmThreads, 0, stream>>>(
-      C, ldc, P, pp.dslot, pp.bcount, pp.finish_rows, pp.nfinish, f, beta);
+  if (f % 2 == 0)
+    panel_finish_kernel<<<(unsigned)ceil_div64((int64_t)pp.nfinish * (f / 2), kSpmmThreads), kSpmmThreads, 0, stream>>>(
+        C, ldc, P, pp.dslot, pp.bcount, pp.finish_rows, pp.nfinish, f, beta, pp.prows);
+  else
+    panel_finish1_kernel<<<(unsigned)ceil_div64((int64_t)pp.nfinish * f, kSpmmThreads), kSpmmThreads, 0, stream>>>(
+        C, ldc, P, pp.dslot, pp.bcount, pp.finish_rows, pp.nfinish, f, beta, pp.prows);
   CG_LAUNCH_CHECK();
   return CG_OK;
 }

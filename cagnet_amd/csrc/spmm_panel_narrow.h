@@ -164,7 +164,7 @@ static int launch_panel_narrow(const PanelPlan &pp, const float *B, int64_t ldb,
     CG_LAUNCH_CHECK();
     if (pp.nsplit > 0) {
       const dim3 grid((unsigned)ceil_div64((int64_t)kPanelRows * f, kSpmmThreads), (unsigned)pp.nsplit);
-      panel_reduce_kernel<<<grid, kSpmmThreads, 0, stream>>>(pp.split, P, f);
+      panel_reduce_kernel<<<grid, kSpmmThreads, 0, stream>>>(pp.split, P, f, kPanelRows);
       CG_LAUNCH_CHECK();
     }
   }

@@ -1,0 +1,431 @@
+// Staged tiles of a panel plan, multiplied with the accumulators addressed through the register index.
+//
+// A workgroup of 16 waves owns a unit (a run of tiles of one panel) and one column slice of the dense
+// operands; wave w keeps R rows of the panel (w, w + 16, ...) times the slice in NR registers per row,
+// NR * R <= 80 of them, for the whole unit.  A tile's rows of B (16 * TCW of them, TCW per wave) go
+// global -> LDS directly, double buffered; the tile's entries are records {column in tile | row slot << 8,
+// value} in (tile, wave) order.  A record is multiplied as
+//     s_set_gpr_idx_on  slot * NR        ; destination and addend registers are taken relative to it
+//     v_fma_f32 v[48 + k], value, b[k], v[48 + k]        k = 0 .. NR - 1
+// so one piece of code serves every row slot: the records of a wave need no order, no padding and no
+// run lengths, and the number of rows a wave owns is a template parameter instead of an unrolled loop.
+// The accumulators are the physical registers v48 .. v127: every asm statement that touches them names
+// them as operands tied to those registers, and nothing else in the kernel refers to them, so the
+// register allocator leaves them where they are.
+//
+// Narrow slices make tall panels: a panel of 16 R rows needs 64 R NR accumulator floats per lane column,
+// so that NR = 5 (a slice of up to 320 columns) allows 256 rows and NR = 1 (64 columns) 1024, and the
+// number of (panel, column) pairs - rows of B that have to be copied - falls with the panel height.  A
+// product wider than a slice runs one workgroup per (unit, slice).
+//
+// Replaces nothing in the reference beyond cusparseSpMM itself
+// (sparse-extension/sparse_coo_tensor.cu:215-226); sums are in a fixed order, no atomics on floats.
+#pragma once
+#include "spmm_panel.h"
+
+namespace cg {
+
+typedef float tile_f32x32 __attribute__((ext_vector_type(32)));
+typedef float tile_f32x16 __attribute__((ext_vector_type(16)));
+
+struct TileAcc {  // v[48:79], v[80:111], v[112:127]
+  tile_f32x32 a0, a1;
+  tile_f32x16 a2;
+};
+#define CG_TILE_ACC(acc) "+{v[48:79]}"((acc).a0), "+{v[80:111]}"((acc).a1), "+{v[112:127]}"((acc).a2)
+
+// Layout of a slice row over the lanes, by NR (lane l, register k -> column of the slice):
+//   1: float   at 4 l                                  col = l
+//   2: float2  at 8 l                                  col = 2 l + k
+//   4: float4  at 16 l                                 col = 4 l + k
+//   5: float4  at 16 l, float at 1024 + 4 l            col = 4 l + k | 256 + l
+//   6: float4  at 16 l, float2 at 1024 + 8 l           col = 4 l + k | 256 + 2 l + (k - 4)
+//   8: float4  at 16 l, float4 at 1024 + 16 l          col = 4 l + k | 256 + 4 l + (k - 4)
+//  10: two float4 as for 8, float2 at 2048 + 8 l       ... | 512 + 2 l + (k - 8)
+template <int NR>
+__device__ __forceinline__ constexpr int tile_max_width() {
+  return NR == 1 ? 64 : NR == 2 ? 128 : NR == 4 ? 256 : NR == 5 ? 320 : NR == 6 ? 384 : NR == 8 ? 512 : 640;
+}
+template <int NR>
+__device__ __forceinline__ int tile_col(int k, int lane) {
+  if (NR == 1) return lane;
+  if (NR == 2) return 2 * lane + k;
+  if (k < 4) return 4 * lane + k;
+  if (NR == 5) return 256 + lane;
+  if (NR == 6) return 256 + 2 * lane + (k - 4);
+  if (k < 8) return 256 + 4 * lane + (k - 4);
+  return 512 + 2 * lane + (k - 8);
+}
+
+template <int NR>
+__device__ __forceinline__ void tile_row_read(const char *src, int lane, float (&b)[NR]) {
+  if constexpr (NR == 1) {
+    b[0] = *reinterpret_cast<const float *>(src + lane * 4);
+  } else if constexpr (NR == 2) {
+    const float2 v = *reinterpret_cast<const float2 *>(src + lane * 8);
+    b[0] = v.x;
+    b[1] = v.y;
+  } else {
+    const float4 v = *reinterpret_cast<const float4 *>(src + lane * 16);
+    b[0] = v.x;
+    b[1] = v.y;
+    b[2] = v.z;
+    b[3] = v.w;
+    if constexpr (NR == 5) {
+      b[4] = *reinterpret_cast<const float *>(src + 1024 + lane * 4);
+    } else if constexpr (NR == 6) {
+      const float2 w = *reinterpret_cast<const float2 *>(src + 1024 + lane * 8);
+      b[4] = w.x;
+      b[5] = w.y;
+    } else if constexpr (NR >= 8) {
+      const float4 w = *reinterpret_cast<const float4 *>(src + 1024 + lane * 16);
+      b[4] = w.x;
+      b[5] = w.y;
+      b[6] = w.z;
+      b[7] = w.w;
+      if constexpr (NR == 10) {
+        const float2 u = *reinterpret_cast<const float2 *>(src + 2048 + lane * 8);
+        b[8] = u.x;
+        b[9] = u.y;
+      }
+    }
+  }
+}
+
+// acc[idx + k] += v * b[k], k < NR (idx = row slot * NR, wave-uniform)
+#define CG_TILE_FMA(k, op) "v_fma_f32 v" #k ", %4, %" #op ", v" #k "\n\t"
+template <int NR>
+__device__ __forceinline__ void tile_fma(TileAcc &acc, uint32_t idx, float v, const float (&b)[NR]) {
+  if constexpr (NR == 1) {
+    asm volatile("s_set_gpr_idx_on %3, 0xc\n\t" CG_TILE_FMA(48, 5) "s_set_gpr_idx_off"
+                 : CG_TILE_ACC(acc)
+                 : "s"(idx), "s"(v), "v"(b[0])
+                 : "m0");
+  } else if constexpr (NR == 2) {
+    asm volatile("s_set_gpr_idx_on %3, 0xc\n\t" CG_TILE_FMA(48, 5) CG_TILE_FMA(49, 6) "s_set_gpr_idx_off"
+                 : CG_TILE_ACC(acc)
+                 : "s"(idx), "s"(v), "v"(b[0]), "v"(b[1])
+                 : "m0");
+  } else if constexpr (NR == 4) {
+    asm volatile("s_set_gpr_idx_on %3, 0xc\n\t" CG_TILE_FMA(48, 5) CG_TILE_FMA(49, 6) CG_TILE_FMA(50, 7)
+                     CG_TILE_FMA(51, 8) "s_set_gpr_idx_off"
+                 : CG_TILE_ACC(acc)
+                 : "s"(idx), "s"(v), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3])
+                 : "m0");
+  } else if constexpr (NR == 5) {
+    asm volatile("s_set_gpr_idx_on %3, 0xc\n\t" CG_TILE_FMA(48, 5) CG_TILE_FMA(49, 6) CG_TILE_FMA(50, 7)
+                     CG_TILE_FMA(51, 8) CG_TILE_FMA(52, 9) "s_set_gpr_idx_off"
+                 : CG_TILE_ACC(acc)
+                 : "s"(idx), "s"(v), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]), "v"(b[4])
+                 : "m0");
+  } else if constexpr (NR == 6) {
+    asm volatile("s_set_gpr_idx_on %3, 0xc\n\t" CG_TILE_FMA(48, 5) CG_TILE_FMA(49, 6) CG_TILE_FMA(50, 7)
+                     CG_TILE_FMA(51, 8) CG_TILE_FMA(52, 9) CG_TILE_FMA(53, 10) "s_set_gpr_idx_off"
+                 : CG_TILE_ACC(acc)
+                 : "s"(idx), "s"(v), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]), "v"(b[4]), "v"(b[5])
+                 : "m0");
+  } else if constexpr (NR == 8) {
+    asm volatile("s_set_gpr_idx_on %3, 0xc\n\t" CG_TILE_FMA(48, 5) CG_TILE_FMA(49, 6) CG_TILE_FMA(50, 7)
+                     CG_TILE_FMA(51, 8) CG_TILE_FMA(52, 9) CG_TILE_FMA(53, 10) CG_TILE_FMA(54, 11)
+                         CG_TILE_FMA(55, 12) "s_set_gpr_idx_off"
+                 : CG_TILE_ACC(acc)
+                 : "s"(idx), "s"(v), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]), "v"(b[4]), "v"(b[5]), "v"(b[6]),
+                   "v"(b[7])
+                 : "m0");
+  } else {
+    static_assert(NR == 10, "register layouts exist for 1, 2, 4, 5, 6, 8 and 10 registers per row");
+    asm volatile("s_set_gpr_idx_on %3, 0xc\n\t" CG_TILE_FMA(48, 5) CG_TILE_FMA(49, 6) CG_TILE_FMA(50, 7)
+                     CG_TILE_FMA(51, 8) CG_TILE_FMA(52, 9) CG_TILE_FMA(53, 10) CG_TILE_FMA(54, 11)
+                         CG_TILE_FMA(55, 12) CG_TILE_FMA(56, 13) CG_TILE_FMA(57, 14) "s_set_gpr_idx_off"
+                 : CG_TILE_ACC(acc)
+                 : "s"(idx), "s"(v), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]), "v"(b[4]), "v"(b[5]), "v"(b[6]),
+                   "v"(b[7]), "v"(b[8]), "v"(b[9])
+                 : "m0");
+  }
+}
+#undef CG_TILE_FMA
+
+// All 80 accumulators = 0, by moves of their own: a zero vector assigned in C++ is a loop-invariant value of 32
+// registers that the register allocator keeps alive (and spills) across the kernel's loop over units.
+#define CG_TILE_Z4(a, b, c, d) "v_mov_b32 v" #a ", 0\n\tv_mov_b32 v" #b ", 0\n\tv_mov_b32 v" #c ", 0\n\tv_mov_b32 v" #d ", 0\n\t"
+__device__ __forceinline__ void tile_acc_zero(TileAcc &acc) {
+  asm volatile(CG_TILE_Z4(48, 49, 50, 51) CG_TILE_Z4(52, 53, 54, 55) CG_TILE_Z4(56, 57, 58, 59) CG_TILE_Z4(60, 61, 62, 63)
+                   CG_TILE_Z4(64, 65, 66, 67) CG_TILE_Z4(68, 69, 70, 71) CG_TILE_Z4(72, 73, 74, 75) CG_TILE_Z4(76, 77, 78, 79)
+                       CG_TILE_Z4(80, 81, 82, 83) CG_TILE_Z4(84, 85, 86, 87) CG_TILE_Z4(88, 89, 90, 91) CG_TILE_Z4(92, 93, 94, 95)
+                           CG_TILE_Z4(96, 97, 98, 99) CG_TILE_Z4(100, 101, 102, 103) CG_TILE_Z4(104, 105, 106, 107)
+                               CG_TILE_Z4(108, 109, 110, 111) CG_TILE_Z4(112, 113, 114, 115) CG_TILE_Z4(116, 117, 118, 119)
+                                   CG_TILE_Z4(120, 121, 122, 123) CG_TILE_Z4(124, 125, 126, 127)
+               : "={v[48:79]}"(acc.a0), "={v[80:111]}"(acc.a1), "={v[112:127]}"(acc.a2));
+}
+#undef CG_TILE_Z4
+
+// accumulator e (a constant after unrolling) of the 80
+__device__ __forceinline__ float tile_acc_get(const TileAcc &acc, int e) {
+  return e < 32 ? acc.a0[e] : e < 64 ? acc.a1[e - 32] : acc.a2[e - 64];
+}
+
+struct TileArgs {
+  const int32_t *unit_tile, *unit_order, *unit_qstart;
+  int32_t *qhead;
+  const int32_t *unit_block, *hdr;
+  const uint2 *ent;
+  const float *B;
+  int64_t ldb;
+  float *P;
+  int32_t f;        // columns of the product
+  int32_t fsw;      // columns of a slice (a multiple of 4); slice s covers [s fsw, min(f, (s + 1) fsw))
+  int32_t nsl;      // slices
+  int32_t m;        // rows of B
+  const int32_t *unit_row0, *rank_row;
+  float *C;         // nullable: units that are their panel's only block write C = beta C + their rows themselves
+  int64_t ldc;
+  int32_t rows;
+  float beta;
+  int32_t dbg;      // timing experiments: 2 no multiplies, 4 no copies, 8 no records
+};
+
+// The next (unit, slice) of the queue of the XCD the workgroup runs on, or of the next queue that is not empty:
+// unit * nsl + slice, -1 when all queues are empty.  qhead: eight counters, zero at launch.
+__device__ __forceinline__ int tile_take_item(const int32_t *__restrict__ unit_queue, const int32_t *__restrict__ qstart,
+                                              int32_t *__restrict__ qhead, int nsl) {
+  __shared__ int taken;
+  if (threadIdx.x == 0) {
+    const int xcd = (int)__builtin_amdgcn_s_getreg((3 << 11) | 20) & 7;  // hardware register XCC_ID, bits 0..3
+    int item = -1;
+    for (int k = 0; k < 8 && item < 0; ++k) {
+      const int q = (xcd + k) & 7;
+      const int first = qstart[q], count = (qstart[q + 1] - first) * nsl;
+      if (count <= 0) continue;
+      const int pos = atomicAdd(&qhead[q], 1);
+      if (pos < count) item = unit_queue[first + pos / nsl] * nsl + pos % nsl;
+    }
+    taken = item;
+  }
+  __syncthreads();
+  const int item = __builtin_amdgcn_readfirstlane(taken);
+  __syncthreads();  // `taken` is free for the next round
+  return item;
+}
+
+// NR registers per row, R rows per wave (the panel has 16 R rows), TCW rows of B per wave and tile (the tile has
+// 16 TCW columns).  hdr[(tile * 16 + wave) * (TCW + 2) ..]: the TCW rows of B the wave stages, then the range of
+// the wave's records.  Place c of a tile is staged by wave c % 16 as its row c / 16 and sits in row c / 16 of
+// that wave's staging area of the tile's buffer.
+template <int NR, int R, int TCW>
+__global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs a) {
+  static_assert(NR * R <= 80, "80 accumulator registers");
+  extern __shared__ __align__(16) char panel_lds[];
+  constexpr int HS = TCW + 2;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int32_t *__restrict__ hdr = a.hdr;
+  const uint2 *__restrict__ ent = a.ent;
+  for (;;) {
+    const int item = tile_take_item(a.unit_order, a.unit_qstart, a.qhead, a.nsl);
+    if (item < 0) return;
+    const int unit = item / a.nsl, slice = item - unit * a.nsl;
+    const int col0 = slice * a.fsw;
+    const int fs = a.f - col0 < a.fsw ? a.f - col0 : a.fsw;  // columns of this slice
+    const float *__restrict__ Bs = a.B + col0;
+    const int t0 = a.unit_tile[unit], t1 = a.unit_tile[unit + 1];
+    const int c16 = (a.fsw + 3) >> 2;                 // 16-byte pieces of a staged row (every slice alike)
+    const int rs = c16 * 16;                          // bytes of a staged row
+    const uint32_t lim = (uint32_t)fs * 4u;              // bytes of a slice row
+    // The last piece of a row may reach up to 12 bytes beyond the slice: into the next slice or the next row of B,
+    // which is harmless (those columns of the accumulators are never stored) except behind the last row of B in
+    // the last slice, where the bytes may not exist: that one piece is copied float by float instead.
+    const bool tail = (fs & 3) != 0 && slice == a.nsl - 1;
+    const uint32_t clast = (uint32_t)fs >> 2;
+    TileAcc acc;
+    tile_acc_zero(acc);
+
+    // Copies of a tile's rows of B.  Slices of at least 256 columns (NR >= 4): row by row, a row in pieces of
+    // 64 x 16 bytes from a wave-uniform base address (scalar arithmetic only; the lanes beyond the row's end are
+    // switched off inside the copy).  The state below names the next piece; a tile has TCW * ppr of them.
+    const int ppr = (c16 + kWave - 1) / kWave;  // pieces of a row
+    const int npieces = NR >= 4 ? TCW * ppr : (TCW * c16 + kWave - 1) / kWave;
+    const int bufsz = kPanelWaves * (NR >= 4 ? TCW * rs : npieces * (kWave * 16));  // bytes of a tile's buffer
+    const uint32_t lane16 = (uint32_t)lane * 16u;
+    const uint32_t ldb32 = (uint32_t)a.ldb;  // the launch refuses leading dimensions of 2^31 and more
+    int st_r = 0, st_j = 0;
+    const float *st_base = Bs;
+    uint32_t st_lim = 0;
+    auto stage_row = [&](int hrows, int r) {
+      const int ridx = __builtin_amdgcn_readlane(hrows, r);
+      st_base = Bs + (uint64_t)(uint32_t)ridx * ldb32;
+      st_lim = tail && ridx == a.m - 1 ? (lim & ~15u) : lim;
+    };
+    auto stage_begin = [&](int hrows) {
+      st_r = 0;
+      st_j = 0;
+      stage_row(hrows, 0);
+    };
+    auto stage_next = [&](int hrows, uint32_t dst_wave) {
+      const uint32_t off = lane16 + (uint32_t)st_j * (kWave * 16u);
+      if (!(a.dbg & 4)) panel_copy16_if(dst_wave + (uint32_t)(st_r * rs) + (uint32_t)st_j * (kWave * 16u), st_base, off, st_lim);
+      if (++st_j == ppr) {
+        st_j = 0;
+        if (++st_r < TCW) stage_row(hrows, st_r);
+      }
+    };
+    // Narrower slices (NR < 4): a copy instruction covers several rows of B, so every lane has an offset of its own
+    // (32 bits from the slice's base: the launch makes sure that B fits).  A wave's staging area is a whole number
+    // of pieces; piece q = pc * 64 + lane of it is row q / c16, position q % c16.  Nothing is switched off: the
+    // lanes behind the wave's last row, and the positions behind a row's end, copy a valid piece once more into
+    // places nobody reads.  (The launch hands narrow products to this kernel only when f is a multiple of 4, so that
+    // every row of B ends with a whole piece.)
+    constexpr int NPN = NR >= 4 ? 1 : 4;  // pieces of a tile at most: 16 rows of 256 bytes, 8 of 512
+    int nsel[NPN];
+    uint32_t noff[NPN];
+    if constexpr (NR < 4) {
+      const uint32_t cmax = (lim - 1u) >> 4;  // the last piece that starts inside a row
+#pragma unroll
+      for (int pc = 0; pc < NPN; ++pc) {
+        const uint32_t q = (uint32_t)(pc * kWave + lane);
+        uint32_t row = q / (uint32_t)c16;
+        uint32_t c = q - row * (uint32_t)c16;
+        row = row < (uint32_t)TCW ? row : (uint32_t)TCW - 1u;
+        c = c < cmax ? c : cmax;
+        nsel[pc] = (int)(row << 2);
+        noff[pc] = c * 16u;
+      }
+    }
+    const uint32_t ldb_bytes = ldb32 * 4u;
+    auto stage_narrow = [&](int hrows, uint32_t dst_wave) {
+#pragma unroll
+      for (int pc = 0; pc < NPN; ++pc) {
+        if (pc < npieces) {
+          const uint32_t ridx = (uint32_t)__builtin_amdgcn_ds_bpermute(nsel[pc], hrows);
+          panel_copy16_at(dst_wave + (uint32_t)pc * (kWave * 16u), Bs, ridx * ldb_bytes + noff[pc]);
+        }
+      }
+    };
+    auto stage_tail = [&](int hrows, char *dst_wave) {  // the piece left out above
+      if (!tail) return;
+      const unsigned long long last = __ballot(lane < TCW && hrows == a.m - 1);
+      if (last == 0ull) return;
+      const int j = __builtin_ctzll(last);
+      if (lane < (fs & 3))
+        *reinterpret_cast<float *>(dst_wave + j * rs + clast * 16u + lane * 4) =
+            Bs[(int64_t)(a.m - 1) * a.ldb + clast * 4u + lane];
+    };
+    auto hdr_load = [&](int t) { return hdr[((int64_t)t * kPanelWaves + wave) * HS + (lane < HS ? lane : HS - 1)]; };
+    auto rec_load = [&](int first, int b0, int b1) {
+      int idx = first + lane;
+      idx = idx < b1 ? idx : (b1 > b0 ? b1 - 1 : 0);
+      return ent[idx];
+    };
+    const int area = NR >= 4 ? TCW * rs : npieces * (kWave * 16);  // bytes of a wave's staging area in a buffer
+    char *const wave_area = panel_lds + wave * area;
+    const uint32_t wave_area32 = (uint32_t)(uintptr_t)wave_area;
+
+    uint2 rec = make_uint2(0u, 0u);
+    int e0 = 0, e1 = 0, hn = 0;
+    if (t1 > t0) {
+      const int h0 = hdr_load(t0);
+      hn = hdr_load(t0 + 1 < t1 ? t0 + 1 : t0);
+      if constexpr (NR >= 4) {
+        stage_begin(h0);
+        for (int pc = 0; pc < npieces; ++pc) stage_next(h0, wave_area32);
+      } else {
+        stage_narrow(h0, wave_area32);
+      }
+      if constexpr (NR >= 4) stage_tail(h0, wave_area);
+      e0 = __builtin_amdgcn_readlane(h0, TCW);
+      e1 = __builtin_amdgcn_readlane(h0, TCW + 1);
+      rec = rec_load(e0, e0, e1);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    for (int t = t0; t < t1; ++t) {
+      const int buf = (t - t0) & 1;
+      const char *lbase = panel_lds + buf * bufsz;
+      // The records of this tile and the header of the next arrived before the last barrier.  Touching them
+      // here puts the compiler's wait for them ahead of the copies it cannot see.
+      asm volatile("" ::"v"(rec.x), "v"(rec.y), "v"(hn));
+      const int e0n = __builtin_amdgcn_readlane(hn, TCW), e1n = __builtin_amdgcn_readlane(hn, TCW + 1);
+      const int hn2 = hdr_load(t + 2 < t1 ? t + 2 : t1 - 1);
+      const uint2 recn = rec_load(e0n, e0n, e1n);
+      const uint32_t dst32 = wave_area32 + (uint32_t)((buf ^ 1) * bufsz);
+      int pc = 0;  // the next tile's copies go out one at a time between the records (the last tile stages itself once more)
+      if constexpr (NR >= 4) {
+        stage_begin(hn);
+      } else {
+        stage_narrow(hn, dst32);
+        pc = npieces;
+      }
+
+      auto process = [&](const uint2 r, int cnt) {
+        const uint32_t c = r.x & 0xffu;
+        const uint32_t packed = ((c & 15u) * (uint32_t)area + (c >> 4) * (uint32_t)rs) | (((r.x >> 8) * (uint32_t)NR) << 20);
+        float ba[NR], bb[NR];
+        uint32_t s0 = __builtin_amdgcn_readlane(packed, 0);
+        tile_row_read<NR>(lbase + (s0 & 0xfffffu), lane, ba);
+        int i = 0;
+        for (; i + 1 < cnt; i += 2) {
+          const uint32_t s1 = __builtin_amdgcn_readlane(packed, i + 1);
+          const float v0 = __uint_as_float(__builtin_amdgcn_readlane(r.y, i));
+          const float v1 = __uint_as_float(__builtin_amdgcn_readlane(r.y, i + 1));
+          tile_row_read<NR>(lbase + (s1 & 0xfffffu), lane, bb);
+          __builtin_amdgcn_sched_barrier(0);  // the reads stay ahead of the multiplies they overlap with
+          if (!(a.dbg & 2)) tile_fma<NR>(acc, s0 >> 20, v0, ba);
+          s0 = __builtin_amdgcn_readlane(packed, (i + 2) & (kWave - 1));  // behind the last record: some lane's valid record
+          tile_row_read<NR>(lbase + (s0 & 0xfffffu), lane, ba);
+          __builtin_amdgcn_sched_barrier(0);
+          if (!(a.dbg & 2)) tile_fma<NR>(acc, s1 >> 20, v1, bb);
+          if (NR >= 4 && pc < npieces) {
+            stage_next(hn, dst32);
+            ++pc;
+          }
+        }
+        if (i < cnt) tile_fma<NR>(acc, s0 >> 20, __uint_as_float(__builtin_amdgcn_readlane(r.y, i)), ba);
+      };
+      uint2 cur = rec;
+      for (int base = e0; base < ((a.dbg & 8) ? e0 : e1); base += kWave) {
+        const int left = e1 - base;
+        uint2 nxt = cur;
+        if (left > kWave) nxt = rec_load(base + kWave, e0, e1);
+        process(cur, left > kWave ? kWave : left);
+        cur = nxt;
+      }
+      if constexpr (NR >= 4)
+        for (; pc < npieces; ++pc) stage_next(hn, dst32);
+      if constexpr (NR >= 4) stage_tail(hn, wave_area + (buf ^ 1) * bufsz);
+      rec = recn;
+      e0 = e0n;
+      e1 = e1n;
+      hn = hn2;
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+    }
+
+    // C[row, slice] = beta C[row, slice] + the sums (the unit is the only block of its panel), or the unit's block
+    // of partial rows: P[block][slot * 16 + wave][:], position in the block = rank of the row inside its panel.
+    const int row0 = a.C ? a.unit_row0[unit] : -1;
+    const int block = a.unit_block[unit];
+#pragma unroll
+    for (int s = 0; s < R; ++s) {
+      float *out;
+      float beta = 0.f;
+      if (row0 >= 0) {
+        const int rank = row0 + s * kPanelWaves + wave;
+        if (rank >= a.rows) continue;
+        out = a.C + (int64_t)a.rank_row[rank] * a.ldc + col0;
+        beta = a.beta;
+      } else {
+        out = a.P + ((int64_t)block * (kPanelWaves * R) + s * kPanelWaves + wave) * a.f + col0;
+      }
+#pragma unroll
+      for (int k = 0; k < NR; ++k) {
+        const int col = tile_col<NR>(k, lane);
+        if (col < fs) {
+          float v = tile_acc_get(acc, s * NR + k);
+          if (beta != 0.f) v += beta * out[col];
+          out[col] = v;
+        }
+      }
+    }
+  }  // the next (unit, slice)
+}
+
+}  // namespace cg

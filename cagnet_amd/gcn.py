@@ -43,8 +43,9 @@ fused_forward = True
 fused_forward_max_row_entries = 64
 
 
-# The stage loop reads wide operands whose rows are not a whole number of 128-byte lines long through a kept copy
-# with line-aligned rows (ops.aligned_rows; ops.aligned_operands = False turns that off).
+# The stage loop reads a wide operand that the caller registered with ops.keep_aligned (the input features, say)
+# through a kept copy with line-aligned rows when its own rows are not a whole number of 128-byte lines long
+# (ops.aligned_rows; ops.aligned_operands = False turns that off).
 _aligned_rows = ops.aligned_rows
 
 
@@ -199,7 +200,10 @@ class GCNFunc(torch.autograd.Function):
             if out is None:
                 z = broad_func(node_count, am_partitions, inputs, rank, size, peers_fwd)
                 out = ops.dense_xw(z, weight, relu=(kind == "relu"))
-                if narrow_backward and size == 1 and _padded_width(weight.shape[1]) > inputs.shape[1]:
+                # dW = (A H)^T G is H^T (A^T G): the same as the reference's H^T (A G) only where backward multiplies
+                # with A^T as well, i.e. the block stores its transpose (or the caller has declared A symmetric)
+                if (narrow_backward and size == 1 and _padded_width(weight.shape[1]) > inputs.shape[1]
+                        and (last.has_transpose or getattr(last, "symmetric", False))):
                     z_kept = z
                 del z
         else:
@@ -351,8 +355,9 @@ class GraphedTrain:
     The graph replays with the addresses of the library's scratch buffers of its stream and of the
     tables of the matrices it multiplies with; the library keeps both alive for as long as the matrices
     live (later eager calls that need other tables or more scratch get new memory).  `close()` drops
-    the graph and hands that memory back: the private stream's scratch at once, the matrices' parked
-    tables through `unpin()`."""
+    the graph and hands that memory back: the private stream's scratch at once, a matrix's parked
+    tables when the last graph captured over it is closed (the matrices count their graphs: `graph_retain`,
+    `graph_release`)."""
 
     def __init__(self, inputs, weight1, weight2, adj_matrix, am_partitions, optimizer, data, rank=0, size=1,
                  group=None, warmup: int = 3):
@@ -373,7 +378,9 @@ class GraphedTrain:
             self.outputs = train(*args)
             self.loss = train.last_loss
         self.epochs_run = warmup
-        self._matrices = [m for m in am_partitions if hasattr(m, "unpin")]
+        self._matrices = [m for m in am_partitions if hasattr(m, "graph_release")]
+        for m in self._matrices:
+            m.graph_retain()
 
     def close(self) -> None:
         """Drop the captured graph and free what the library kept alive for it.  Idempotent."""
@@ -383,7 +390,7 @@ class GraphedTrain:
         torch.cuda.synchronize(self.stream.device)
         ops.scratch_release(self.stream)
         for m in self._matrices:
-            m.unpin()
+            m.graph_release()  # frees the parked tables only when no other live graph was captured over the matrix
         self._matrices = []
 
     def __del__(self):

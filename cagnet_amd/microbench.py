@@ -3,7 +3,6 @@
     python -m cagnet_amd.microbench spmm   [--graph rmat20|reddit|amazon] [--widths 16,64,128,602]
     python -m cagnet_amd.microbench grid2d [--grid 4] [--row 1]
     python -m cagnet_amd.microbench prep   [--graph reddit]
-    python -m cagnet_amd.microbench probes
 
 `spmm`   builds the CSR (sorted input, unsorted input, transpose) and times A @ H and A^T @ G at
          each width: GFLOP/s = 2 nnz f / t, algorithmic GB/s = (8 nnz + 4 (n+1) + 4 m f + 4 n f) / t.
@@ -12,9 +11,6 @@
          dense block, accumulated over q stages; forward and backward of both layers.
 `prep`   times the device-side input preparation on the graph's pattern: self-loop insertion,
          D^-1/2 A D^-1/2 values, and the 16 block extractions of a 4 x 4 partition.
-`probes` measures machine ceilings with the library's probe kernels: LDS read bandwidth per access width
-         (B/clk/CU at the published 2.4 GHz), streaming read / copy bandwidth over working-set sizes, and a
-         dense fp32 matrix-core product in the tile shape a dense hub block of a wide SpMM would take.
 One JSON object per line.  Timing: HIP events on the current stream, median of `--reps`.
 """
 from __future__ import annotations
@@ -60,33 +56,6 @@ def _time(fn, reps: int) -> float:
         times.append(e0.elapsed_time(e1))
     times.sort()
     return times[len(times) // 2]
-
-
-def run_probes(args) -> None:
-    import ctypes
-
-    from ._lib import check, lib
-
-    cus = torch.cuda.get_device_properties(0).multi_processor_count
-    clock_hz = 2.4e9  # published peak engine clock of the MI355X
-    for width in (4, 8, 16):
-        for threads in (256, 1024):
-            tbs = ctypes.c_double(0)
-            check(lib.cg_probe_lds_read(width, threads, ctypes.byref(tbs)), "cg_probe_lds_read")
-            print(json.dumps({"what": "lds read", "instruction": f"ds_read_b{8 * width}", "threads_per_workgroup": threads,
-                              "tb_per_s": round(tbs.value, 2),
-                              "bytes_per_clk_per_cu": round(tbs.value * 1e12 / clock_hz / cus, 1), "cus": cus}), flush=True)
-    for mib in (16, 64, 128, 200, 512, 1024, 4096):
-        for copy in (0, 1):
-            tbs = ctypes.c_double(0)
-            check(lib.cg_probe_stream(mib << 20, copy, ctypes.byref(tbs)), "cg_probe_stream")
-            print(json.dumps({"what": "stream copy" if copy else "stream read", "mib": mib, "tb_per_s": round(tbs.value, 2)}),
-                  flush=True)
-    for k in (4000, 8000, 16000):
-        ms, tf = ctypes.c_double(0), ctypes.c_double(0)
-        check(lib.cg_probe_mfma_dense(k, 602, ctypes.byref(ms), ctypes.byref(tf)), "cg_probe_mfma_dense")
-        print(json.dumps({"what": "dense fp32 mfma product", "k": k, "f": 602, "ms": round(ms.value, 3),
-                          "dense_tflops": round(tf.value, 1), "pct_of_157.3": round(tf.value / 1.573, 1)}), flush=True)
 
 
 def run_spmm(args) -> None:
@@ -238,14 +207,11 @@ def main() -> int:
     pr = sub.add_parser("prep")
     pr.add_argument("--graph", default="reddit", choices=sorted(GRAPHS))
     pr.add_argument("--reps", type=int, default=3)
-    sub.add_parser("probes")
     args = ap.parse_args()
     if not torch.cuda.is_available():
         print("microbench: no GPU visible; cagnet_amd has no CPU path", file=sys.stderr)
         return 2
-    if args.cmd == "probes":
-        run_probes(args)
-    elif args.cmd == "spmm":
+    if args.cmd == "spmm":
         run_spmm(args)
     elif args.cmd == "prep":
         run_prep(args)

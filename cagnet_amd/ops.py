@@ -322,6 +322,20 @@ class CsrMatrix:
     def shape(self) -> Tuple[int, int]:
         return (self.n, self.m)
 
+    def graph_retain(self) -> None:
+        """A captured graph that multiplies with this matrix now exists (`gcn.GraphedTrain` calls this)."""
+        self._graph_refs = getattr(self, "_graph_refs", 0) + 1
+
+    def graph_release(self) -> int:
+        """One of the graphs counted by `graph_retain` is gone.  The tables the library parked for captured
+        graphs are freed (`unpin`) only when the last one is: a graph that is still alive replays with their
+        addresses.  Returns the number of device allocations freed."""
+        refs = getattr(self, "_graph_refs", 0)
+        if refs <= 0:
+            return 0
+        self._graph_refs = refs - 1
+        return self.unpin() if self._graph_refs == 0 else 0
+
     def unpin(self) -> int:
         """Free the tables this matrix has kept alive for HIP graphs captured over its products
         (cg_csr_unpin): call it only when none of those graphs will be replayed again.  Returns the
@@ -567,33 +581,62 @@ def log_softmax_nll_bwd(logp: torch.Tensor, y: torch.Tensor, mask: Optional[torc
 
 
 # A wide dense operand whose rows are not a whole number of 128-byte lines long (602 floats = 2408 bytes) is read by the
-# SpMM kernels through rows that start at every alignment and span 20 lines instead of 19: measured at the Reddit shape,
-# the f = 602 product takes 12.3 ms on X as it is, 12.2 ms with the rows 604 floats apart and 11.9 ms with 608 or 640
-# (0.25 ms to make the copy).  The features are the same tensor in every epoch, so the copy is kept for as long as the
-# tensor is unchanged.  Tensors beyond 2 GiB are left alone (the copy would double them).
+# SpMM kernels through rows that start at every alignment and span 20 lines instead of 19: measured on a graph of
+# 232,965 vertices with 492 entries per row, the f = 602 product takes 12.3 ms on X as it is, 12.2 ms with the rows 604
+# floats apart and 11.9 ms with 608 or 640 (0.25 ms to make the copy).  A feature matrix is the same tensor in every epoch,
+# so a caller can register it (`keep_aligned`): the stage loop and the drop-in `spmm_gpu` then read it through a kept copy
+# with line-aligned rows.  Only registered tensors are ever copied.  The copy is remade when the tensor's version counter
+# has moved; writes that do not move it (`x.data.copy_()`, DLPack or custom-kernel writers, direct calls of the C ABI)
+# leave the copy stale: call `keep_aligned(x)` again or `aligned_cache_clear()` after such a write.  Tensors beyond 2 GiB
+# are left alone (the copy would double them).
 aligned_operands = True
 _ALIGNED_MIN_COLS = 64
 _ALIGNED_MAX_BYTES = 2 << 30
-_aligned_cache: list = []   # (weakref to the tensor, its version, the copy's column slice); newest last, at most 2
+_aligned_cache: dict = {}   # id(tensor) -> [weakref, key, copy or None, event or None, stream the copy was made on]
+
+
+def _aligned_key(t: torch.Tensor):
+    return (t.data_ptr(), tuple(t.shape), tuple(t.stride()), t._version)
+
+
+def _aligned_wanted(t: torch.Tensor) -> bool:
+    return (aligned_operands and t.dim() == 2 and t.dtype == torch.float32 and t.is_cuda and t.shape[1] >= _ALIGNED_MIN_COLS
+            and t.stride(1) == 1 and t.stride(0) % 32 != 0 and t.shape[0] > 0 and t.numel() * 4 <= _ALIGNED_MAX_BYTES)
+
+
+def keep_aligned(t: torch.Tensor) -> torch.Tensor:
+    """Register `t` (a dense operand that stays the same over many products, e.g. the input features) for a kept
+    copy with line-aligned rows; registering again drops a copy made earlier.  Returns `t`."""
+    import weakref
+
+    _aligned_cache[id(t)] = [weakref.ref(t), None, None, None, None]
+    for k in [k for k, e in _aligned_cache.items() if e[0]() is None]:
+        del _aligned_cache[k]
+    return t
+
+
+def aligned_cache_clear() -> None:
+    """Forget every registration and free the kept copies."""
+    _aligned_cache.clear()
 
 
 def aligned_rows(t: torch.Tensor) -> torch.Tensor:
-    """t, or a copy of t with the rows a multiple of 128 bytes apart when that pays (see `aligned_operands`)."""
-    import weakref
-
-    if (not aligned_operands or t.dim() != 2 or t.dtype != torch.float32 or not t.is_cuda or t.shape[1] < _ALIGNED_MIN_COLS
-            or t.stride(1) != 1 or t.stride(0) % 32 == 0 or t.shape[0] == 0 or t.numel() * 4 > _ALIGNED_MAX_BYTES):
+    """`t`, or the kept copy of a registered `t` with the rows a multiple of 128 bytes apart (see `keep_aligned`)."""
+    entry = _aligned_cache.get(id(t))
+    if entry is None or entry[0]() is not t or not _aligned_wanted(t):
         return t
-    if torch.cuda.is_current_stream_capturing():
-        return t  # a captured graph must keep reading the caller's tensor, whose contents may change between replays
-    for ref, version, copy in _aligned_cache:
-        if ref() is t and version == t._version:
-            return copy
-    _aligned_cache[:] = [e for e in _aligned_cache if e[0]() is not None and e[0]() is not t][-1:]
-    ld = (t.shape[1] + 31) // 32 * 32
-    with torch.no_grad():
-        wide = torch.empty(t.shape[0], ld, dtype=t.dtype, device=t.device)
-        wide[:, :t.shape[1]].copy_(t)
-    copy = wide[:, :t.shape[1]]
-    _aligned_cache.append((weakref.ref(t), t._version, copy))
-    return copy
+    key = _aligned_key(t)
+    stream = torch.cuda.current_stream(t.device)
+    if entry[1] != key or entry[2] is None:
+        if torch.cuda.is_current_stream_capturing():
+            return t  # no copy yet: the graph reads the caller's tensor
+        ld = (t.shape[1] + 31) // 32 * 32
+        with torch.no_grad():
+            wide = torch.empty(t.shape[0], ld, dtype=t.dtype, device=t.device)
+            wide[:, :t.shape[1]].copy_(t)
+        event = torch.cuda.Event()
+        event.record(stream)
+        entry[1:] = [key, wide[:, :t.shape[1]], event, stream]
+    elif entry[4] != stream and not torch.cuda.is_current_stream_capturing():
+        stream.wait_event(entry[3])  # the copy was made on another stream
+    return entry[2]

@@ -51,7 +51,7 @@ def spmm_gpu(A_rowindices: torch.Tensor, A_colindices: torch.Tensor, A_values: t
     B is m x f and C is n x f, both fp32.  Returns None, like the reference."""
     if validate_inputs:
         ops.coo_check(A_rowindices, A_colindices, int(n), int(m), require_sorted=True)
-    B = ops.aligned_rows(B)   # wide B with unaligned rows: read through a kept copy with line-aligned rows
+    B = ops.aligned_rows(B)   # a B registered with ops.keep_aligned: read through its kept copy with line-aligned rows
     if C.dim() == 2 and C.numel() > 0 and C.stride(1) != 1:
         # a transposed view, e.g. a C that an earlier reference-style call left column-major
         tmp = C.contiguous()

@@ -380,20 +380,6 @@ int cg_prof_enable(int on);
 int cg_tune_set(const char *key, int value);
 int cg_prof_read(const char *name, double *total_ms, int64_t *launches);
 
-/* ------------------------------------------------------------------------------------------
- * Machine probes (no counterpart in the reference): the ceilings the kernels are judged against,
- * measured on the device the library runs on.  Each allocates what it needs, runs on the null stream,
- * synchronises and frees.  `python -m cagnet_amd.microbench probes` prints them.
- *   cg_probe_lds_read    conflict-free ds_read_b32 / b64 / b128 (bytes_per_lane 4 / 8 / 16) by every lane,
- *                        eight reads in flight per wave: aggregate TB/s over all CUs
- *   cg_probe_stream      grid-stride float4 read (copy == 0) or copy (bytes counted twice) of `bytes`
- *                        of device memory: TB/s
- *   cg_probe_mfma_dense  P[k x f] = D[k x k] * (k rows picked from a 232,965 x f matrix) on
- *                        v_mfma_f32_16x16x4_f32, D as pre-swizzled 64 x 16 tiles, the rows of B staged in LDS:
- *                        the form a dense hub block of a wide SpMM would take.  ms and dense TFLOP/s. */
-int cg_probe_lds_read(int32_t bytes_per_lane, int32_t threads_per_workgroup, double *tb_per_s);
-int cg_probe_stream(int64_t bytes, int32_t copy, double *tb_per_s);
-int cg_probe_mfma_dense(int32_t k, int32_t f, double *ms, double *tflops);
 
 #ifdef __cplusplus
 }

@@ -61,6 +61,39 @@ def test_forward_backward_matches_oracle(cuda, monkeypatch, transpose, fused, na
     _close(x.grad, ref["dx"], "dx")
 
 
+@pytest.mark.parametrize("transpose", [False, True])
+def test_backward_on_a_non_symmetric_block(cuda, monkeypatch, transpose):
+    """A block that is not symmetric.  Without a stored transpose the backward pass multiplies with the block
+    itself, as the reference does (gcn_distr.py:326): dW = H^T (A G), dH = (A G) W^T, also with the library's default
+    backward order switched on (which would give H^T (A^T G) and must therefore stand back).  With a stored transpose
+    both gradients use A^T, in either order."""
+    from cagnet_amd import gcn, ops
+    from tests.util import random_coo
+    n = 700
+    row, col, val = random_coo(n, n, 9000, seed=11)
+    torch.manual_seed(4)
+    x = torch.randn(n, 24)
+    w1 = torch.randn(24, 16) * 0.3
+    w2 = torch.randn(16, 41) * 0.3   # the layer widens: where the default backward order applies
+    y = torch.randint(0, 41, (n,))
+    mask = torch.rand(n) < 0.7
+    A = orc.coo_tensor(row, col, val, n, n, torch.float64)
+    At = orc.coo_tensor(col, row, val, n, n, torch.float64)
+    ref = orc.forward_backward(x, w1, w2, [A], y, mask, blocks_bwd=[At] if transpose else None, dtype=torch.float64)
+    blk = ops.CsrMatrix(row.int().to(cuda), col.int().to(cuda), val.to(cuda), n, n, transpose=transpose)
+    for narrow in (True, False):
+        monkeypatch.setattr(gcn, "narrow_backward", narrow)
+        xg = x.to(cuda).requires_grad_(True)
+        g1 = w1.to(cuda).requires_grad_(True)
+        g2 = w2.to(cuda).requires_grad_(True)
+        h = gcn.GCNFunc.apply(xg, g1, n, [blk], 0, 1, None, F.relu)
+        out = gcn.GCNFunc.apply(h, g2, n, [blk], 0, 1, None, F.log_softmax)
+        gcn.masked_nll_loss(out, y.to(cuda), mask.to(cuda)).backward()
+        _close(g2.grad, ref["dw2"], f"dw2 (narrow_backward={narrow})")
+        _close(g1.grad, ref["dw1"], f"dw1 (narrow_backward={narrow})")
+        _close(xg.grad, ref["dx"], f"dx (narrow_backward={narrow})")
+
+
 @pytest.mark.parametrize("fused_loss", [True, False])
 def test_training_losses_match_oracle(cuda, monkeypatch, fused_loss):
     """100 epochs of SGD lr 0.01 on the R-MAT scale-12 plumbing configuration: per-epoch loss
@@ -343,8 +376,8 @@ def test_adam_epochs_with_reference_init_match_oracle(cuda, monkeypatch, classes
     w2_0 = torch.rand(16, classes)
     A = orc.coo_tensor(p.row, p.col, p.val, p.n, p.n, torch.float32)
     epochs = 60
-    ref32, _, _ = orc.train_epochs(p.x, w1_0, w2_0, [A], p.y, p.train_mask, epochs=epochs, optimizer="adam",
-                                   dtype=torch.float32)
+    ref32, w1_32, w2_32 = orc.train_epochs(p.x, w1_0, w2_0, [A], p.y, p.train_mask, epochs=epochs, optimizer="adam",
+                                           dtype=torch.float32)
     ref64, w1_64, w2_64 = orc.train_epochs(p.x, w1_0, w2_0, [A], p.y, p.train_mask, epochs=epochs, optimizer="adam",
                                            dtype=torch.float64)
     blk = _block(p, cuda, transpose=True)
@@ -353,15 +386,44 @@ def test_adam_epochs_with_reference_init_match_oracle(cuda, monkeypatch, classes
     w2 = w2_0.to(cuda).requires_grad_(True)
     opt = torch.optim.Adam([w1, w2], lr=0.01)
     data = _Data(p.y.to(cuda), p.train_mask.to(cuda))
+    A64 = orc.coo_tensor(p.row, p.col, p.val, p.n, p.n, torch.float64)
     losses = []
-    for _ in range(epochs):
+    for epoch in range(epochs):
+        if epoch % 10 == 0:
+            # the gradients at the library's own weights against the fp64 oracle at the same weights: this is what
+            # each step contributes, free of what the steps before it did to the trajectory
+            at = orc.forward_backward(p.x, w1.detach().cpu(), w2.detach().cpu(), [A64], p.y, p.train_mask,
+                                      dtype=torch.float64, x_requires_grad=False)
+            a = w1.detach().clone().requires_grad_(True)
+            b = w2.detach().clone().requires_grad_(True)
+            h = gcn.GCNFunc.apply(x, a, p.n, [blk], 0, 1, None, F.relu)
+            out = gcn.GCNFunc.apply(h, b, p.n, [blk], 0, 1, None, F.log_softmax)
+            gcn.masked_nll_loss(out, data.y, data.train_mask).backward()
+            _close(a.grad, at["dw1"], f"dw1 at the weights of epoch {epoch}", 2e-5)
+            _close(b.grad, at["dw2"], f"dw2 at the weights of epoch {epoch}", 2e-5)
         gcn.train(x, w1, w2, p.n, [blk], opt, data, 0, 1, None)
         losses.append(float(gcn.train.last_loss))
     assert max(abs(a - b) for a, b in zip(losses, ref64)) <= LOSS_TOL
     assert max(abs(a - b) for a, b in zip(losses, ref32)) <= LOSS_TOL
     assert losses[-1] < losses[0]
-    _close(w1, w1_64, "w1 after 60 Adam epochs", 2e-3 if narrow else 1e-3)
-    _close(w2, w2_64, "w2 after 60 Adam epochs", 2e-3 if narrow else 1e-3)
+
+    def drift(got, ref64):
+        return float((got.detach().cpu().double() - ref64).abs().max()) / max(float(ref64.abs().max()), 1e-30)
+
+    # Weights after the 60 steps.  With the reference's order of the backward products the library stays within a few
+    # 1e-6 of the fp64 trajectory (the fp32 oracle: 4e-7), and the bound is tied to the fp32 oracle's own distance.
+    # With the library's default order the gradients are as close at every epoch (checked above at equal weights:
+    # 3e-6), but on the 41-class case the trajectory itself leaves the fp64 one around epoch 20, in one column of W1
+    # (one hidden unit), and ends 1.1e-3 away: Adam divides every gradient entry by its running magnitude, so a
+    # column with small gradients turns a rounding-sized difference into steps of the size of the learning rate.
+    # Hence the wider absolute bound there, next to the per-epoch gradient check that a real defect would fail.
+    for name, got, w32, w64 in (("w1", w1, w1_32, w1_64), ("w2", w2, w2_32, w2_64)):
+        own, oracle32 = drift(got, w64), drift(w32, w64)
+        print(f"{name}: library {own:.3e} from fp64, fp32 oracle {oracle32:.3e} (narrow_backward={narrow})")
+        if narrow:
+            assert own <= 2e-3, f"{name} after 60 Adam epochs: {own} from fp64"
+        else:
+            assert own <= max(30.0 * oracle32, 2e-5), f"{name} after 60 Adam epochs: {own} from fp64, the fp32 oracle {oracle32}"
 
 
 def test_single_process_harness_prints_golden_losses(cuda):
@@ -389,32 +451,50 @@ def test_single_process_harness_prints_golden_losses(cuda):
 
 
 def test_row_aligned_copy_of_a_wide_operand(cuda):
-    """The stage loop multiplies a wide operand whose rows are not a multiple of 128 bytes long (602 floats) through a
-    copy with rows 608 floats apart: same bits as on the tensor itself, the copy is reused while the tensor is
-    unchanged and made again after an in-place change; widths that are aligned already are used as they are."""
+    """A wide operand registered with ops.keep_aligned, whose rows are not a multiple of 128 bytes long (602 floats),
+    is multiplied by the stage loop through a copy with rows 608 floats apart: same bits as on the tensor itself,
+    the copy is reused while the tensor is unchanged and made again after an in-place change; tensors that were not
+    registered, and widths that are aligned already, are used as they are."""
     from cagnet_amd import gcn, ops
     from tests.util import small_graph
     row, col, val, n = small_graph(10, 20000, seed=5)
     A = ops.CsrMatrix(row.int().to(cuda), col.int().to(cuda), val.to(cuda), n, n)
     x = torch.randn(n, 602, device=cuda)
-    c1 = gcn._aligned_rows(x)
-    assert c1.data_ptr() != x.data_ptr() and c1.stride(0) == 608 and torch.equal(c1, x)
-    assert gcn._aligned_rows(x) is c1                                 # cached
-    direct = A.spmm(x)
-    assert torch.equal(gcn.broad_func(n, [A], x, 0, 1), direct)       # goes through the copy: same bits
-    x.mul_(2.0)                                                       # in-place change: the copy is stale
-    c2 = gcn._aligned_rows(x)
-    assert c2 is not c1 and torch.equal(c2, x)
-    assert torch.equal(gcn.broad_func(n, [A], x, 0, 1), A.spmm(x))
-    A.spmm(torch.randn(n, 602, device=cuda), out=x)                   # written by the library: counts as a change
-    c3 = gcn._aligned_rows(x)
-    assert c3 is not c2 and torch.equal(c3, x)
-    y = torch.randn(n, 640, device=cuda)
-    assert gcn._aligned_rows(y) is y
-    z = torch.randn(n, 41, device=cuda)
-    assert gcn._aligned_rows(z) is z                                  # narrow: not worth a copy
-    ops.aligned_operands = False
+    ops.aligned_cache_clear()
     try:
+        assert gcn._aligned_rows(x) is x                                  # not registered: never copied
+        ops.keep_aligned(x)
+        c1 = gcn._aligned_rows(x)
+        assert c1.data_ptr() != x.data_ptr() and c1.stride(0) == 608 and torch.equal(c1, x)
+        assert gcn._aligned_rows(x) is c1                                 # cached
+        direct = A.spmm(x)
+        assert torch.equal(gcn.broad_func(n, [A], x, 0, 1), direct)       # goes through the copy: same bits
+        x.mul_(2.0)                                                       # in-place change: the copy is stale
+        c2 = gcn._aligned_rows(x)
+        assert c2 is not c1 and torch.equal(c2, x)
+        assert torch.equal(gcn.broad_func(n, [A], x, 0, 1), A.spmm(x))
+        A.spmm(torch.randn(n, 602, device=cuda), out=x)                   # written by the library: counts as a change
+        c3 = gcn._aligned_rows(x)
+        assert c3 is not c2 and torch.equal(c3, x)
+        x.data.mul_(0.5)                                                  # a write that moves no version counter ...
+        assert gcn._aligned_rows(x) is c3 and not torch.equal(c3, x)      # ... leaves the copy stale, as documented,
+        ops.keep_aligned(x)                                               # until the tensor is registered again
+        assert torch.equal(gcn._aligned_rows(x), x)
+        side = torch.cuda.Stream(device=cuda)                             # a copy made on one stream, used on another
+        side.wait_stream(torch.cuda.current_stream(cuda))
+        with torch.cuda.stream(side):
+            assert torch.equal(gcn.broad_func(n, [A], x, 0, 1), A.spmm(x))
+        torch.cuda.current_stream(cuda).wait_stream(side)
+        y = ops.keep_aligned(torch.randn(n, 640, device=cuda))
+        assert gcn._aligned_rows(y) is y
+        z = ops.keep_aligned(torch.randn(n, 41, device=cuda))
+        assert gcn._aligned_rows(z) is z                                  # narrow: not worth a copy
+        ops.aligned_operands = False
+        try:
+            assert gcn._aligned_rows(x) is x
+        finally:
+            ops.aligned_operands = True
+        ops.aligned_cache_clear()
         assert gcn._aligned_rows(x) is x
     finally:
-        ops.aligned_operands = True
+        ops.aligned_cache_clear()
