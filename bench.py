@@ -391,13 +391,23 @@ def extra_grid_row(prob, spec, dev, reps: int, traffic_table: dict) -> dict:
         for k in range(q):
             blocks[k].spmm(H[k], out=z, beta=0.0 if k == 0 else 1.0)
 
-    ms_stage = median_ms(stages, reps)
-    traffic = traffic_of(traffic_table, "grid_row", feats, launched_spmm_kernels(stages, feats))
-    alg = sum(spmm_alg_bytes(nz, rows, b[k + 1] - b[k], feats, reads_c=k > 0) for k, nz in enumerate(nnzs))
+    ms_per_stage = median_ms(stages, reps)
+
+    # the library's stage loop: all four stages as one product of the blocks side by side with the stacked operands
+    # (gcn.fuse_stages; the rank's own block is copied into its slot of the stacked buffer inside the timed call)
+    def fused():
+        gcn.broad_func(rows, blocks, x.detach(), r, q, g1.forward, out=z)
+
+    ms_stage = median_ms(fused, reps)
+    traffic = traffic_of(traffic_table, "grid_row", feats, launched_spmm_kernels(fused, feats))
+    alg_per_stage = sum(spmm_alg_bytes(nz, rows, b[k + 1] - b[k], feats, reads_c=k > 0) for k, nz in enumerate(nnzs))
+    alg = spmm_alg_bytes(sum(nnzs), rows, prob.n, feats, reads_c=False)
     return {"workload": "last process row of the 4 x 4 grid on the Reddit-shaped graph, four stages resident in HBM; "
                         "median of %d" % reps,
             "rows": rows, "block_cols": [b[k + 1] - b[k] for k in range(q)], "block_nnz": nnzs, "bound": "hbm",
             "stage_loop_f%d" % feats: roofline_fields(alg, 2.0 * sum(nnzs) * feats, ms_stage, traffic),
+            "stage_loop_f%d_one_product_per_stage" % feats: roofline_fields(alg_per_stage, 2.0 * sum(nnzs) * feats,
+                                                                            ms_per_stage, None),
             "fwd_bwd_both_layers_ms": round(ms_epoch, 4)}
 
 

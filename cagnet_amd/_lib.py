@@ -52,6 +52,7 @@ _SIGNATURES = {
     "cg_csr_create": [POINTER(c_void_p), P, P, P, c_int64, c_int32, c_int32, c_uint32, P],
     "cg_csr_destroy": [P],
     "cg_csr_unpin": [P, POINTER(c_int64)],
+    "cg_csr_hstack": [POINTER(P), POINTER(P), c_int32, c_uint32, P],
     "cg_scratch_release": [P, POINTER(c_int64)],
     "cg_csr_spmm": [P, c_int, P, c_int64, P, c_int64, c_int32, c_float, P],
     "cg_csr_spmm_xw": [P, c_int, P, c_int64, P, c_int64, c_float, P, c_int64, P, c_int64, c_int32, c_int32, c_int, P],

@@ -191,6 +191,50 @@ __global__ __launch_bounds__(kPrepThreads) void block_compact_kernel(
   }
 }
 
+// ---- blocks side by side ------------------------------------------------------------------------
+// [A_0 | A_1 | ...]: the blocks of one block row of a partitioned matrix as one matrix, so that the stage loop
+// sum_k A_k H_k (gcn_distr.py:221-244, gcn_distr_2d.py:333-417) becomes one product with the stacked H_k.
+constexpr int kStackMax = 16;  // blocks of one call
+struct StackArgs {
+  const int32_t *rowptr[kStackMax];
+  const int32_t *colind[kStackMax];
+  const float *val[kStackMax];
+  int32_t coloff[kStackMax];
+  int32_t count;
+};
+
+// counts[i] = entries of row i over all blocks (counts[n] = 0: the place of the scan's total)
+__global__ __launch_bounds__(kPrepThreads) void stack_count_kernel(const StackArgs a, int32_t n, uint32_t *__restrict__ counts) {
+  const int64_t i = (int64_t)blockIdx.x * kPrepThreads + threadIdx.x;
+  if (i > n) return;
+  uint32_t c = 0;
+  if (i < n)
+    for (int k = 0; k < a.count; ++k) c += (uint32_t)(a.rowptr[k][i + 1] - a.rowptr[k][i]);
+  counts[i] = c;
+}
+
+// One wave per row: the row's entries of block 0, then of block 1, ... with the blocks' column offsets added;
+// the (row, column) order of the blocks is kept.
+__global__ __launch_bounds__(kPrepThreads) void stack_rows_kernel(const StackArgs a, int32_t n,
+                                                                  const uint32_t *__restrict__ rowptr_out,
+                                                                  int32_t *__restrict__ row_out, int32_t *__restrict__ col_out,
+                                                                  float *__restrict__ val_out) {
+  const int64_t i = ((int64_t)blockIdx.x * kPrepThreads + threadIdx.x) / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  if (i >= n) return;
+  int64_t at = rowptr_out[i];
+  for (int k = 0; k < a.count; ++k) {
+    const int32_t s = a.rowptr[k][i], e = a.rowptr[k][i + 1];
+    for (int32_t j = s + lane; j < e; j += kWave) {
+      const int64_t o = at + (j - s);
+      row_out[o] = (int32_t)i;
+      col_out[o] = a.colind[k][j] + a.coloff[k];
+      val_out[o] = a.val[k][j];
+    }
+    at += e - s;
+  }
+}
+
 static unsigned grid_for(int64_t count) { return (unsigned)ceil_div64(count > 0 ? count : 1, kPrepThreads); }
 
 }  // namespace cg
@@ -302,6 +346,62 @@ int cg_coo_block(const int32_t *d_row, const int32_t *d_col, const float *d_val,
   CG_LAUNCH_CHECK();
   CG_HIP(hipStreamSynchronize(stream));
   return CG_OK;
+}
+
+int cg_csr_hstack(cg_csr_t **out, cg_csr_t *const *blocks, int32_t count, uint32_t flags, cg_stream_t stream_) {
+  using namespace cg;
+  hipStream_t stream = (hipStream_t)stream_;
+  if (!out) CG_FAIL(CG_ERR_NULL, "cg_csr_hstack: out is NULL");
+  *out = nullptr;
+  if (!blocks) CG_FAIL(CG_ERR_NULL, "cg_csr_hstack: blocks is NULL");
+  if (count < 1 || count > kStackMax) CG_FAIL(CG_ERR_SIZE, "cg_csr_hstack: %d blocks (1 .. %d are supported)", count, kStackMax);
+  StackArgs a{};
+  a.count = count;
+  int64_t n = -1, m = 0, nnz = 0;
+  for (int k = 0; k < count; ++k) {
+    if (!blocks[k]) CG_FAIL(CG_ERR_NULL, "cg_csr_hstack: block %d is NULL", k);
+    int64_t info[8];
+    CG_TRY(cg_csr_info(blocks[k], info));
+    CG_TRY(cg_csr_arrays(blocks[k], 0, &a.rowptr[k], &a.colind[k], &a.val[k]));
+    if (n >= 0 && info[0] != n) CG_FAIL(CG_ERR_SIZE, "cg_csr_hstack: block %d has %lld rows, block 0 has %lld", k, (long long)info[0], (long long)n);
+    n = info[0];
+    a.coloff[k] = (int32_t)m;
+    m += info[1];
+    nnz += info[2];
+  }
+  if (m >= 0x7fffffffLL || nnz >= 0x7fffffffLL)
+    CG_FAIL(CG_ERR_OVERFLOW, "cg_csr_hstack: %lld columns and %lld entries are outside the int32 contract", (long long)m, (long long)nnz);
+  CG_TRY(refuse_under_capture(stream, "stacking blocks"));
+  uint32_t *counts = nullptr;
+  int32_t *d_row = nullptr, *d_col = nullptr;
+  float *d_val = nullptr;
+  int st = CG_OK;
+  do {
+    const size_t eb = (size_t)(nnz > 0 ? nnz : 1) * 4;
+    if (hipMalloc((void **)&counts, (size_t)(n + 1) * 4) != hipSuccess || hipMalloc((void **)&d_row, eb) != hipSuccess ||
+        hipMalloc((void **)&d_col, eb) != hipSuccess || hipMalloc((void **)&d_val, eb) != hipSuccess) {
+      (void)hipGetLastError();
+      set_error("cg_csr_hstack: device allocation failed");
+      st = CG_ERR_ALLOC;
+      break;
+    }
+    stack_count_kernel<<<grid_for(n + 1), kPrepThreads, 0, stream>>>(a, (int32_t)n, counts);
+    if (hipGetLastError() != hipSuccess) { st = CG_ERR_HIP; break; }
+    if ((st = exclusive_scan_u32(counts, counts, n + 1, nullptr, stream)) != CG_OK) break;
+    if (n > 0) {
+      stack_rows_kernel<<<grid_for(n * kWave), kPrepThreads, 0, stream>>>(a, (int32_t)n, counts, d_row, d_col, d_val);
+      if (hipGetLastError() != hipSuccess) { st = CG_ERR_HIP; break; }
+    }
+    st = cg_csr_create(out, d_row, d_col, d_val, nnz, (int32_t)n, (int32_t)m,
+                       CG_CSR_SORTED | (flags & CG_CSR_TRANSPOSE), stream);
+  } while (0);
+  if (st == CG_ERR_HIP) set_error("cg_csr_hstack: kernel launch failed");
+  (void)hipStreamSynchronize(stream);
+  if (counts) (void)hipFree(counts);
+  if (d_row) (void)hipFree(d_row);
+  if (d_col) (void)hipFree(d_col);
+  if (d_val) (void)hipFree(d_val);
+  return st;
 }
 
 }  // extern "C"

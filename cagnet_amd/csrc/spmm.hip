@@ -906,6 +906,7 @@ int cg_tune_set(const char *key, int value) {
   else if (!strcmp(key, "spmm_panel_dwg")) cg::g_tune_panel_dwg.store(value);
   else if (!strcmp(key, "spmm_panel_share")) cg::g_tune_panel_share.store(value);
   else if (!strcmp(key, "spmm_tile")) cg::g_tune_tile.store(value);
+  else if (!strcmp(key, "spmm_strict_nonfinite")) cg::g_tune_strict.store(value);
   else if (!strcmp(key, "spmm_panel_narrow")) cg::g_tune_panel_narrow.store(value);
   else if (!strcmp(key, "spmm_panel_narrow_dmin")) cg::g_tune_panel_narrow_dmin.store(value);
   else if (!strcmp(key, "dense_mfma")) cg::g_tune_dense_mfma.store(value);

@@ -42,7 +42,7 @@ constexpr int kDenseThreads = kDenseWaves * kWave;
 constexpr int kDenseTileFloats = kPanelRows * kPanelCols;
 
 static std::atomic<int> g_tune_panel{0}, g_tune_panel_emin{0}, g_tune_panel_cols{0}, g_tune_panel_unit{0};
-static std::atomic<int> g_tune_panel_dmin{0}, g_tune_panel_dwg{0}, g_tune_panel_share{0}, g_tune_tile{0};
+static std::atomic<int> g_tune_panel_dmin{0}, g_tune_panel_dwg{0}, g_tune_panel_share{0}, g_tune_tile{0}, g_tune_strict{0};
 
 struct CsrSide;
 

@@ -37,6 +37,7 @@ static bool panel_width_ok(int32_t f) { return f >= kPanelMinF && f <= kPanelMax
 static bool want_panel(const CsrSide &s, int32_t f) {
   const int t = g_tune_panel.load(std::memory_order_relaxed);
   if (t < 0 || !panel_width_ok(f) || s.rows == 0 || s.nnz == 0) return false;
+  if (g_tune_strict.load(std::memory_order_relaxed) > 0) return false;  // its dense tiles multiply zeros, its records are padded
   if (t > 0) return true;
   // Below about 8e8 multiply-adds the plan's fixed costs (a block of partial rows per unit, few units per compute
   // unit) outweigh what it saves: blocks of a 4 x 4 grid over 232,965 vertices at f = 602, plan against row-wise
@@ -403,16 +404,20 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     int64_t weight;
   };
   std::vector<Unit> su, du;  // units of active tiles, of dense tiles; both in panel order
-  constexpr int32_t kUnitGrid = 32;  // with shared column order a unit starts where a panel's block number passes a multiple
+  // with shared column order a unit starts where a panel's block number passes a multiple of this: every 1024 column ranks
+  const int32_t kUnitGrid = TC >= 1024 ? 1 : 1024 / TC;
   constexpr int32_t kXcds = kXcdQueues;  // XCDs of the device
   // What a run of tiles costs, in microseconds: a tile with e records 1.50 + 0.0034 e + 8.7e-6 e^2 (fitted to the
   // durations of the 3744 units of the matrix with 232,965 vertices and 492 entries per row at f = 602: 3.4 % off
   // in the median; a tile costs its copies and its barrier whatever it holds, and the waves' records run the more
   // unevenly the more of them a tile has).  Only ratios matter.  A unit is also cut when it has an eighth of a
   // compute unit's share of the whole cost (at least 100 us), so that a small matrix still gets balanced work.
+  // (Tiles of other shapes go to spmm_tile_kernel, whose waves take a record in about 60 cycles whatever the tile
+  // holds: a fixed part per tile and a linear one.)
+  const bool legacy_shape = PR == kPanelRows && TC == kPanelCols;
   auto tile_cost = [&](int64_t t) {
     const double e = (double)(h_base[(size_t)t + 1] - h_base[(size_t)t]);
-    return 1.50 + 0.0034 * e + 8.7e-6 * e * e;
+    return legacy_shape ? 1.50 + 0.0034 * e + 8.7e-6 * e * e : 1.50 + 0.0016 * e;
   };
   double cost_cap = 100.0;
   {
@@ -443,8 +448,8 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
       if (whole) {
       } else if (share) {
         if (j > k && (in_unit >= unit_entries / 2 || unit_cost >= cost_cap) &&
-            h_kb[(size_t)j] / kUnitGrid != h_kb[(size_t)j - 1] / kUnitGrid)
-          break;
+            (h_kb[(size_t)j] / kUnitGrid != h_kb[(size_t)j - 1] / kUnitGrid || in_unit >= 2 * (int64_t)unit_entries))
+          break;  // (a stretch of very full tiles is cut inside the grid as well)
       } else if (j > k && (in_unit + e > unit_entries || unit_cost >= cost_cap)) {
         break;
       }
@@ -495,6 +500,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   // the launch order goes by the units' costs (a unit's tiles taken as alike)
   auto cost = [&](int32_t u) {
     const double T = (double)(su[(size_t)u].t1 - su[(size_t)u].t0), R = (double)su[(size_t)u].weight;
+    if (!legacy_shape) return 1.50 * T + 0.0016 * R;
     return T > 0.0 ? 1.50 * T + 0.0034 * R + 8.7e-6 * R * R / T : 0.0;
   };
   // The units go into eight queues, one per XCD; a workgroup takes the next unit of the queue of the XCD it runs on
@@ -676,7 +682,7 @@ static PanelParams tile_params(int geom) {
   p.emin = 1;                 // every tile is staged: nothing is left for the row-wise kernels
   p.cols = kPanelDefaultCols;
   p.dmin = 0;                 // no tiles for the matrix cores
-  if (g_tune_panel_unit.load(std::memory_order_relaxed) <= 0) p.unit = kPanelDefaultUnit * (p.prows / kPanelRows);
+  // (units of kPanelDefaultUnit entries whatever the panel height: a unit is what one workgroup does in one go)
   return p;
 }
 
@@ -777,7 +783,6 @@ static int launch_tile(const PanelPlan &pp, const float *B, int64_t ldb, int32_t
   ta.ldc = ldc;
   ta.rows = rows;
   ta.beta = beta;
-  ta.dbg = g_tune_tile.load(std::memory_order_relaxed) > 0 ? (g_tune_tile.load(std::memory_order_relaxed) & ~1) : 0;
   // two tiles of staged rows (narrow slices: a wave's staging area is a whole number of 1 KiB pieces) and some room
   // behind them: the lanes of a row read beyond the slice's last column
   const size_t tlds_max = 160 * 1024 - 64;

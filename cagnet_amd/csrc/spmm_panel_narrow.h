@@ -128,6 +128,7 @@ __global__ __launch_bounds__(kSpmmThreads) void panel_add_rows_kernel(float *__r
 static bool want_panel_narrow(const CsrSide &s, int32_t f) {
   const int t = g_tune_panel_narrow.load(std::memory_order_relaxed);
   if (t < 0 || f < 1 || f > kPanelNarrowMaxF || s.rows == 0 || s.nnz == 0 || s.is_rest) return false;
+  if (g_tune_strict.load(std::memory_order_relaxed) > 0) return false;  // dense tiles multiply their zeros
   if (t > 0) return true;
   return s.nnz / s.rows >= 64 && (double)s.nnz * f >= 1e9;
 }

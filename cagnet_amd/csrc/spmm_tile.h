@@ -92,58 +92,184 @@ __device__ __forceinline__ void tile_row_read(const char *src, int lane, float (
   }
 }
 
-// acc[idx + k] += v * b[k], k < NR (idx = row slot * NR, wave-uniform)
-#define CG_TILE_FMA(k, op) "v_fma_f32 v" #k ", %4, %" #op ", v" #k "\n\t"
-template <int NR>
-__device__ __forceinline__ void tile_fma(TileAcc &acc, uint32_t idx, float v, const float (&b)[NR]) {
-  if constexpr (NR == 1) {
-    asm volatile("s_set_gpr_idx_on %3, 0xc\n\t" CG_TILE_FMA(48, 5) "s_set_gpr_idx_off"
-                 : CG_TILE_ACC(acc)
-                 : "s"(idx), "s"(v), "v"(b[0])
-                 : "m0");
-  } else if constexpr (NR == 2) {
-    asm volatile("s_set_gpr_idx_on %3, 0xc\n\t" CG_TILE_FMA(48, 5) CG_TILE_FMA(49, 6) "s_set_gpr_idx_off"
-                 : CG_TILE_ACC(acc)
-                 : "s"(idx), "s"(v), "v"(b[0]), "v"(b[1])
-                 : "m0");
-  } else if constexpr (NR == 4) {
-    asm volatile("s_set_gpr_idx_on %3, 0xc\n\t" CG_TILE_FMA(48, 5) CG_TILE_FMA(49, 6) CG_TILE_FMA(50, 7)
-                     CG_TILE_FMA(51, 8) "s_set_gpr_idx_off"
-                 : CG_TILE_ACC(acc)
-                 : "s"(idx), "s"(v), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3])
-                 : "m0");
-  } else if constexpr (NR == 5) {
-    asm volatile("s_set_gpr_idx_on %3, 0xc\n\t" CG_TILE_FMA(48, 5) CG_TILE_FMA(49, 6) CG_TILE_FMA(50, 7)
-                     CG_TILE_FMA(51, 8) CG_TILE_FMA(52, 9) "s_set_gpr_idx_off"
-                 : CG_TILE_ACC(acc)
-                 : "s"(idx), "s"(v), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]), "v"(b[4])
-                 : "m0");
-  } else if constexpr (NR == 6) {
-    asm volatile("s_set_gpr_idx_on %3, 0xc\n\t" CG_TILE_FMA(48, 5) CG_TILE_FMA(49, 6) CG_TILE_FMA(50, 7)
-                     CG_TILE_FMA(51, 8) CG_TILE_FMA(52, 9) CG_TILE_FMA(53, 10) "s_set_gpr_idx_off"
-                 : CG_TILE_ACC(acc)
-                 : "s"(idx), "s"(v), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]), "v"(b[4]), "v"(b[5])
-                 : "m0");
-  } else if constexpr (NR == 8) {
-    asm volatile("s_set_gpr_idx_on %3, 0xc\n\t" CG_TILE_FMA(48, 5) CG_TILE_FMA(49, 6) CG_TILE_FMA(50, 7)
-                     CG_TILE_FMA(51, 8) CG_TILE_FMA(52, 9) CG_TILE_FMA(53, 10) CG_TILE_FMA(54, 11)
-                         CG_TILE_FMA(55, 12) "s_set_gpr_idx_off"
-                 : CG_TILE_ACC(acc)
-                 : "s"(idx), "s"(v), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]), "v"(b[4]), "v"(b[5]), "v"(b[6]),
-                   "v"(b[7])
-                 : "m0");
-  } else {
-    static_assert(NR == 10, "register layouts exist for 1, 2, 4, 5, 6, 8 and 10 registers per row");
-    asm volatile("s_set_gpr_idx_on %3, 0xc\n\t" CG_TILE_FMA(48, 5) CG_TILE_FMA(49, 6) CG_TILE_FMA(50, 7)
-                     CG_TILE_FMA(51, 8) CG_TILE_FMA(52, 9) CG_TILE_FMA(53, 10) CG_TILE_FMA(54, 11)
-                         CG_TILE_FMA(55, 12) CG_TILE_FMA(56, 13) CG_TILE_FMA(57, 14) "s_set_gpr_idx_off"
-                 : CG_TILE_ACC(acc)
-                 : "s"(idx), "s"(v), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]), "v"(b[4]), "v"(b[5]), "v"(b[6]),
-                   "v"(b[7]), "v"(b[8]), "v"(b[9])
-                 : "m0");
-  }
+// K records in one stretch of index mode: the index register is set for the first record and moved for the others
+// (the low 8 bits of pk[k] are the record's first accumulator: row slot * NR); acc[idx_k + r] += v[k] * b[k][r].
+template <int NR, int K>
+__device__ __forceinline__ void tile_window(TileAcc &acc, const uint32_t (&pk)[K], const float (&v)[K], const float (&b)[K][NR]);
+template <>
+__device__ __forceinline__ void tile_window<1, 8>(TileAcc &acc, const uint32_t (&pk)[8], const float (&v)[8], const float (&b)[8][1]) {
+  asm volatile("s_set_gpr_idx_on %[p0], 0xc\n\ts_nop 0\n\tv_fma_f32 v48, %[v0], %[b0_0], v48\n\ts_set_gpr_idx_idx %[p1]\n\t"
+               "v_fma_f32 v48, %[v1], %[b1_0], v48\n\ts_set_gpr_idx_idx %[p2]\n\tv_fma_f32 v48, %[v2], %[b2_0], v48\n\t"
+               "s_set_gpr_idx_idx %[p3]\n\tv_fma_f32 v48, %[v3], %[b3_0], v48\n\ts_set_gpr_idx_idx %[p4]\n\t"
+               "v_fma_f32 v48, %[v4], %[b4_0], v48\n\ts_set_gpr_idx_idx %[p5]\n\tv_fma_f32 v48, %[v5], %[b5_0], v48\n\t"
+               "s_set_gpr_idx_idx %[p6]\n\tv_fma_f32 v48, %[v6], %[b6_0], v48\n\ts_set_gpr_idx_idx %[p7]\n\t"
+               "v_fma_f32 v48, %[v7], %[b7_0], v48\n\ts_set_gpr_idx_off"
+               : CG_TILE_ACC(acc)
+               : [p0] "s"(pk[0]), [v0] "s"(v[0]), [p1] "s"(pk[1]), [v1] "s"(v[1]), [p2] "s"(pk[2]), [v2] "s"(v[2]),
+                 [p3] "s"(pk[3]), [v3] "s"(v[3]), [p4] "s"(pk[4]), [v4] "s"(v[4]), [p5] "s"(pk[5]), [v5] "s"(v[5]),
+                 [p6] "s"(pk[6]), [v6] "s"(v[6]), [p7] "s"(pk[7]), [v7] "s"(v[7]), [b0_0] "v"(b[0][0]),
+                 [b1_0] "v"(b[1][0]), [b2_0] "v"(b[2][0]), [b3_0] "v"(b[3][0]), [b4_0] "v"(b[4][0]),
+                 [b5_0] "v"(b[5][0]), [b6_0] "v"(b[6][0]), [b7_0] "v"(b[7][0])
+               : "m0");
 }
-#undef CG_TILE_FMA
+template <>
+__device__ __forceinline__ void tile_window<2, 4>(TileAcc &acc, const uint32_t (&pk)[4], const float (&v)[4], const float (&b)[4][2]) {
+  asm volatile("s_set_gpr_idx_on %[p0], 0xc\n\ts_nop 0\n\tv_fma_f32 v48, %[v0], %[b0_0], v48\n\tv_fma_f32 v49, %[v0], %[b0_1], v49\n\t"
+               "s_set_gpr_idx_idx %[p1]\n\tv_fma_f32 v48, %[v1], %[b1_0], v48\n\tv_fma_f32 v49, %[v1], %[b1_1], v49\n\t"
+               "s_set_gpr_idx_idx %[p2]\n\tv_fma_f32 v48, %[v2], %[b2_0], v48\n\tv_fma_f32 v49, %[v2], %[b2_1], v49\n\t"
+               "s_set_gpr_idx_idx %[p3]\n\tv_fma_f32 v48, %[v3], %[b3_0], v48\n\tv_fma_f32 v49, %[v3], %[b3_1], v49\n\t"
+               "s_set_gpr_idx_off"
+               : CG_TILE_ACC(acc)
+               : [p0] "s"(pk[0]), [v0] "s"(v[0]), [p1] "s"(pk[1]), [v1] "s"(v[1]), [p2] "s"(pk[2]), [v2] "s"(v[2]),
+                 [p3] "s"(pk[3]), [v3] "s"(v[3]), [b0_0] "v"(b[0][0]), [b0_1] "v"(b[0][1]), [b1_0] "v"(b[1][0]),
+                 [b1_1] "v"(b[1][1]), [b2_0] "v"(b[2][0]), [b2_1] "v"(b[2][1]), [b3_0] "v"(b[3][0]),
+                 [b3_1] "v"(b[3][1])
+               : "m0");
+}
+template <>
+__device__ __forceinline__ void tile_window<4, 2>(TileAcc &acc, const uint32_t (&pk)[2], const float (&v)[2], const float (&b)[2][4]) {
+  asm volatile("s_set_gpr_idx_on %[p0], 0xc\n\ts_nop 0\n\tv_fma_f32 v48, %[v0], %[b0_0], v48\n\tv_fma_f32 v49, %[v0], %[b0_1], v49\n\t"
+               "v_fma_f32 v50, %[v0], %[b0_2], v50\n\tv_fma_f32 v51, %[v0], %[b0_3], v51\n\ts_set_gpr_idx_idx %[p1]\n\t"
+               "v_fma_f32 v48, %[v1], %[b1_0], v48\n\tv_fma_f32 v49, %[v1], %[b1_1], v49\n\tv_fma_f32 v50, %[v1], %[b1_2], v50\n\t"
+               "v_fma_f32 v51, %[v1], %[b1_3], v51\n\ts_set_gpr_idx_off"
+               : CG_TILE_ACC(acc)
+               : [p0] "s"(pk[0]), [v0] "s"(v[0]), [p1] "s"(pk[1]), [v1] "s"(v[1]), [b0_0] "v"(b[0][0]),
+                 [b0_1] "v"(b[0][1]), [b0_2] "v"(b[0][2]), [b0_3] "v"(b[0][3]), [b1_0] "v"(b[1][0]),
+                 [b1_1] "v"(b[1][1]), [b1_2] "v"(b[1][2]), [b1_3] "v"(b[1][3])
+               : "m0");
+}
+template <>
+__device__ __forceinline__ void tile_window<5, 2>(TileAcc &acc, const uint32_t (&pk)[2], const float (&v)[2], const float (&b)[2][5]) {
+  asm volatile("s_set_gpr_idx_on %[p0], 0xc\n\ts_nop 0\n\tv_fma_f32 v48, %[v0], %[b0_0], v48\n\tv_fma_f32 v49, %[v0], %[b0_1], v49\n\t"
+               "v_fma_f32 v50, %[v0], %[b0_2], v50\n\tv_fma_f32 v51, %[v0], %[b0_3], v51\n\tv_fma_f32 v52, %[v0], %[b0_4], v52\n\t"
+               "s_set_gpr_idx_idx %[p1]\n\tv_fma_f32 v48, %[v1], %[b1_0], v48\n\tv_fma_f32 v49, %[v1], %[b1_1], v49\n\t"
+               "v_fma_f32 v50, %[v1], %[b1_2], v50\n\tv_fma_f32 v51, %[v1], %[b1_3], v51\n\tv_fma_f32 v52, %[v1], %[b1_4], v52\n\t"
+               "s_set_gpr_idx_off"
+               : CG_TILE_ACC(acc)
+               : [p0] "s"(pk[0]), [v0] "s"(v[0]), [p1] "s"(pk[1]), [v1] "s"(v[1]), [b0_0] "v"(b[0][0]),
+                 [b0_1] "v"(b[0][1]), [b0_2] "v"(b[0][2]), [b0_3] "v"(b[0][3]), [b0_4] "v"(b[0][4]),
+                 [b1_0] "v"(b[1][0]), [b1_1] "v"(b[1][1]), [b1_2] "v"(b[1][2]), [b1_3] "v"(b[1][3]),
+                 [b1_4] "v"(b[1][4])
+               : "m0");
+}
+template <>
+__device__ __forceinline__ void tile_window<6, 2>(TileAcc &acc, const uint32_t (&pk)[2], const float (&v)[2], const float (&b)[2][6]) {
+  asm volatile("s_set_gpr_idx_on %[p0], 0xc\n\ts_nop 0\n\tv_fma_f32 v48, %[v0], %[b0_0], v48\n\tv_fma_f32 v49, %[v0], %[b0_1], v49\n\t"
+               "v_fma_f32 v50, %[v0], %[b0_2], v50\n\tv_fma_f32 v51, %[v0], %[b0_3], v51\n\tv_fma_f32 v52, %[v0], %[b0_4], v52\n\t"
+               "v_fma_f32 v53, %[v0], %[b0_5], v53\n\ts_set_gpr_idx_idx %[p1]\n\tv_fma_f32 v48, %[v1], %[b1_0], v48\n\t"
+               "v_fma_f32 v49, %[v1], %[b1_1], v49\n\tv_fma_f32 v50, %[v1], %[b1_2], v50\n\tv_fma_f32 v51, %[v1], %[b1_3], v51\n\t"
+               "v_fma_f32 v52, %[v1], %[b1_4], v52\n\tv_fma_f32 v53, %[v1], %[b1_5], v53\n\ts_set_gpr_idx_off"
+               : CG_TILE_ACC(acc)
+               : [p0] "s"(pk[0]), [v0] "s"(v[0]), [p1] "s"(pk[1]), [v1] "s"(v[1]), [b0_0] "v"(b[0][0]),
+                 [b0_1] "v"(b[0][1]), [b0_2] "v"(b[0][2]), [b0_3] "v"(b[0][3]), [b0_4] "v"(b[0][4]),
+                 [b0_5] "v"(b[0][5]), [b1_0] "v"(b[1][0]), [b1_1] "v"(b[1][1]), [b1_2] "v"(b[1][2]),
+                 [b1_3] "v"(b[1][3]), [b1_4] "v"(b[1][4]), [b1_5] "v"(b[1][5])
+               : "m0");
+}
+template <>
+__device__ __forceinline__ void tile_window<8, 2>(TileAcc &acc, const uint32_t (&pk)[2], const float (&v)[2], const float (&b)[2][8]) {
+  asm volatile("s_set_gpr_idx_on %[p0], 0xc\n\ts_nop 0\n\tv_fma_f32 v48, %[v0], %[b0_0], v48\n\tv_fma_f32 v49, %[v0], %[b0_1], v49\n\t"
+               "v_fma_f32 v50, %[v0], %[b0_2], v50\n\tv_fma_f32 v51, %[v0], %[b0_3], v51\n\tv_fma_f32 v52, %[v0], %[b0_4], v52\n\t"
+               "v_fma_f32 v53, %[v0], %[b0_5], v53\n\tv_fma_f32 v54, %[v0], %[b0_6], v54\n\tv_fma_f32 v55, %[v0], %[b0_7], v55\n\t"
+               "s_set_gpr_idx_idx %[p1]\n\tv_fma_f32 v48, %[v1], %[b1_0], v48\n\tv_fma_f32 v49, %[v1], %[b1_1], v49\n\t"
+               "v_fma_f32 v50, %[v1], %[b1_2], v50\n\tv_fma_f32 v51, %[v1], %[b1_3], v51\n\tv_fma_f32 v52, %[v1], %[b1_4], v52\n\t"
+               "v_fma_f32 v53, %[v1], %[b1_5], v53\n\tv_fma_f32 v54, %[v1], %[b1_6], v54\n\tv_fma_f32 v55, %[v1], %[b1_7], v55\n\t"
+               "s_set_gpr_idx_off"
+               : CG_TILE_ACC(acc)
+               : [p0] "s"(pk[0]), [v0] "s"(v[0]), [p1] "s"(pk[1]), [v1] "s"(v[1]), [b0_0] "v"(b[0][0]),
+                 [b0_1] "v"(b[0][1]), [b0_2] "v"(b[0][2]), [b0_3] "v"(b[0][3]), [b0_4] "v"(b[0][4]),
+                 [b0_5] "v"(b[0][5]), [b0_6] "v"(b[0][6]), [b0_7] "v"(b[0][7]), [b1_0] "v"(b[1][0]),
+                 [b1_1] "v"(b[1][1]), [b1_2] "v"(b[1][2]), [b1_3] "v"(b[1][3]), [b1_4] "v"(b[1][4]),
+                 [b1_5] "v"(b[1][5]), [b1_6] "v"(b[1][6]), [b1_7] "v"(b[1][7])
+               : "m0");
+}
+template <>
+__device__ __forceinline__ void tile_window<10, 2>(TileAcc &acc, const uint32_t (&pk)[2], const float (&v)[2], const float (&b)[2][10]) {
+  asm volatile("s_set_gpr_idx_on %[p0], 0xc\n\ts_nop 0\n\tv_fma_f32 v48, %[v0], %[b0_0], v48\n\tv_fma_f32 v49, %[v0], %[b0_1], v49\n\t"
+               "v_fma_f32 v50, %[v0], %[b0_2], v50\n\tv_fma_f32 v51, %[v0], %[b0_3], v51\n\tv_fma_f32 v52, %[v0], %[b0_4], v52\n\t"
+               "v_fma_f32 v53, %[v0], %[b0_5], v53\n\tv_fma_f32 v54, %[v0], %[b0_6], v54\n\tv_fma_f32 v55, %[v0], %[b0_7], v55\n\t"
+               "v_fma_f32 v56, %[v0], %[b0_8], v56\n\tv_fma_f32 v57, %[v0], %[b0_9], v57\n\ts_set_gpr_idx_idx %[p1]\n\t"
+               "v_fma_f32 v48, %[v1], %[b1_0], v48\n\tv_fma_f32 v49, %[v1], %[b1_1], v49\n\tv_fma_f32 v50, %[v1], %[b1_2], v50\n\t"
+               "v_fma_f32 v51, %[v1], %[b1_3], v51\n\tv_fma_f32 v52, %[v1], %[b1_4], v52\n\tv_fma_f32 v53, %[v1], %[b1_5], v53\n\t"
+               "v_fma_f32 v54, %[v1], %[b1_6], v54\n\tv_fma_f32 v55, %[v1], %[b1_7], v55\n\tv_fma_f32 v56, %[v1], %[b1_8], v56\n\t"
+               "v_fma_f32 v57, %[v1], %[b1_9], v57\n\ts_set_gpr_idx_off"
+               : CG_TILE_ACC(acc)
+               : [p0] "s"(pk[0]), [v0] "s"(v[0]), [p1] "s"(pk[1]), [v1] "s"(v[1]), [b0_0] "v"(b[0][0]),
+                 [b0_1] "v"(b[0][1]), [b0_2] "v"(b[0][2]), [b0_3] "v"(b[0][3]), [b0_4] "v"(b[0][4]),
+                 [b0_5] "v"(b[0][5]), [b0_6] "v"(b[0][6]), [b0_7] "v"(b[0][7]), [b0_8] "v"(b[0][8]),
+                 [b0_9] "v"(b[0][9]), [b1_0] "v"(b[1][0]), [b1_1] "v"(b[1][1]), [b1_2] "v"(b[1][2]),
+                 [b1_3] "v"(b[1][3]), [b1_4] "v"(b[1][4]), [b1_5] "v"(b[1][5]), [b1_6] "v"(b[1][6]),
+                 [b1_7] "v"(b[1][7]), [b1_8] "v"(b[1][8]), [b1_9] "v"(b[1][9])
+               : "m0");
+}
+template <>
+__device__ __forceinline__ void tile_window<1, 1>(TileAcc &acc, const uint32_t (&pk)[1], const float (&v)[1], const float (&b)[1][1]) {
+  asm volatile("s_set_gpr_idx_on %[p0], 0xc\n\ts_nop 0\n\tv_fma_f32 v48, %[v0], %[b0_0], v48\n\ts_set_gpr_idx_off"
+               : CG_TILE_ACC(acc)
+               : [p0] "s"(pk[0]), [v0] "s"(v[0]), [b0_0] "v"(b[0][0])
+               : "m0");
+}
+template <>
+__device__ __forceinline__ void tile_window<2, 1>(TileAcc &acc, const uint32_t (&pk)[1], const float (&v)[1], const float (&b)[1][2]) {
+  asm volatile("s_set_gpr_idx_on %[p0], 0xc\n\ts_nop 0\n\tv_fma_f32 v48, %[v0], %[b0_0], v48\n\tv_fma_f32 v49, %[v0], %[b0_1], v49\n\t"
+               "s_set_gpr_idx_off"
+               : CG_TILE_ACC(acc)
+               : [p0] "s"(pk[0]), [v0] "s"(v[0]), [b0_0] "v"(b[0][0]), [b0_1] "v"(b[0][1])
+               : "m0");
+}
+template <>
+__device__ __forceinline__ void tile_window<4, 1>(TileAcc &acc, const uint32_t (&pk)[1], const float (&v)[1], const float (&b)[1][4]) {
+  asm volatile("s_set_gpr_idx_on %[p0], 0xc\n\ts_nop 0\n\tv_fma_f32 v48, %[v0], %[b0_0], v48\n\tv_fma_f32 v49, %[v0], %[b0_1], v49\n\t"
+               "v_fma_f32 v50, %[v0], %[b0_2], v50\n\tv_fma_f32 v51, %[v0], %[b0_3], v51\n\ts_set_gpr_idx_off"
+               : CG_TILE_ACC(acc)
+               : [p0] "s"(pk[0]), [v0] "s"(v[0]), [b0_0] "v"(b[0][0]), [b0_1] "v"(b[0][1]), [b0_2] "v"(b[0][2]),
+                 [b0_3] "v"(b[0][3])
+               : "m0");
+}
+template <>
+__device__ __forceinline__ void tile_window<5, 1>(TileAcc &acc, const uint32_t (&pk)[1], const float (&v)[1], const float (&b)[1][5]) {
+  asm volatile("s_set_gpr_idx_on %[p0], 0xc\n\ts_nop 0\n\tv_fma_f32 v48, %[v0], %[b0_0], v48\n\tv_fma_f32 v49, %[v0], %[b0_1], v49\n\t"
+               "v_fma_f32 v50, %[v0], %[b0_2], v50\n\tv_fma_f32 v51, %[v0], %[b0_3], v51\n\tv_fma_f32 v52, %[v0], %[b0_4], v52\n\t"
+               "s_set_gpr_idx_off"
+               : CG_TILE_ACC(acc)
+               : [p0] "s"(pk[0]), [v0] "s"(v[0]), [b0_0] "v"(b[0][0]), [b0_1] "v"(b[0][1]), [b0_2] "v"(b[0][2]),
+                 [b0_3] "v"(b[0][3]), [b0_4] "v"(b[0][4])
+               : "m0");
+}
+template <>
+__device__ __forceinline__ void tile_window<6, 1>(TileAcc &acc, const uint32_t (&pk)[1], const float (&v)[1], const float (&b)[1][6]) {
+  asm volatile("s_set_gpr_idx_on %[p0], 0xc\n\ts_nop 0\n\tv_fma_f32 v48, %[v0], %[b0_0], v48\n\tv_fma_f32 v49, %[v0], %[b0_1], v49\n\t"
+               "v_fma_f32 v50, %[v0], %[b0_2], v50\n\tv_fma_f32 v51, %[v0], %[b0_3], v51\n\tv_fma_f32 v52, %[v0], %[b0_4], v52\n\t"
+               "v_fma_f32 v53, %[v0], %[b0_5], v53\n\ts_set_gpr_idx_off"
+               : CG_TILE_ACC(acc)
+               : [p0] "s"(pk[0]), [v0] "s"(v[0]), [b0_0] "v"(b[0][0]), [b0_1] "v"(b[0][1]), [b0_2] "v"(b[0][2]),
+                 [b0_3] "v"(b[0][3]), [b0_4] "v"(b[0][4]), [b0_5] "v"(b[0][5])
+               : "m0");
+}
+template <>
+__device__ __forceinline__ void tile_window<8, 1>(TileAcc &acc, const uint32_t (&pk)[1], const float (&v)[1], const float (&b)[1][8]) {
+  asm volatile("s_set_gpr_idx_on %[p0], 0xc\n\ts_nop 0\n\tv_fma_f32 v48, %[v0], %[b0_0], v48\n\tv_fma_f32 v49, %[v0], %[b0_1], v49\n\t"
+               "v_fma_f32 v50, %[v0], %[b0_2], v50\n\tv_fma_f32 v51, %[v0], %[b0_3], v51\n\tv_fma_f32 v52, %[v0], %[b0_4], v52\n\t"
+               "v_fma_f32 v53, %[v0], %[b0_5], v53\n\tv_fma_f32 v54, %[v0], %[b0_6], v54\n\tv_fma_f32 v55, %[v0], %[b0_7], v55\n\t"
+               "s_set_gpr_idx_off"
+               : CG_TILE_ACC(acc)
+               : [p0] "s"(pk[0]), [v0] "s"(v[0]), [b0_0] "v"(b[0][0]), [b0_1] "v"(b[0][1]), [b0_2] "v"(b[0][2]),
+                 [b0_3] "v"(b[0][3]), [b0_4] "v"(b[0][4]), [b0_5] "v"(b[0][5]), [b0_6] "v"(b[0][6]),
+                 [b0_7] "v"(b[0][7])
+               : "m0");
+}
+template <>
+__device__ __forceinline__ void tile_window<10, 1>(TileAcc &acc, const uint32_t (&pk)[1], const float (&v)[1], const float (&b)[1][10]) {
+  asm volatile("s_set_gpr_idx_on %[p0], 0xc\n\ts_nop 0\n\tv_fma_f32 v48, %[v0], %[b0_0], v48\n\tv_fma_f32 v49, %[v0], %[b0_1], v49\n\t"
+               "v_fma_f32 v50, %[v0], %[b0_2], v50\n\tv_fma_f32 v51, %[v0], %[b0_3], v51\n\tv_fma_f32 v52, %[v0], %[b0_4], v52\n\t"
+               "v_fma_f32 v53, %[v0], %[b0_5], v53\n\tv_fma_f32 v54, %[v0], %[b0_6], v54\n\tv_fma_f32 v55, %[v0], %[b0_7], v55\n\t"
+               "v_fma_f32 v56, %[v0], %[b0_8], v56\n\tv_fma_f32 v57, %[v0], %[b0_9], v57\n\ts_set_gpr_idx_off"
+               : CG_TILE_ACC(acc)
+               : [p0] "s"(pk[0]), [v0] "s"(v[0]), [b0_0] "v"(b[0][0]), [b0_1] "v"(b[0][1]), [b0_2] "v"(b[0][2]),
+                 [b0_3] "v"(b[0][3]), [b0_4] "v"(b[0][4]), [b0_5] "v"(b[0][5]), [b0_6] "v"(b[0][6]),
+                 [b0_7] "v"(b[0][7]), [b0_8] "v"(b[0][8]), [b0_9] "v"(b[0][9])
+               : "m0");
+}
 
 // All 80 accumulators = 0, by moves of their own: a zero vector assigned in C++ is a loop-invariant value of 32
 // registers that the register allocator keeps alive (and spills) across the kernel's loop over units.
@@ -181,7 +307,6 @@ struct TileArgs {
   int64_t ldc;
   int32_t rows;
   float beta;
-  int32_t dbg;      // timing experiments: 2 no multiplies, 4 no copies, 8 no records
 };
 
 // The next (unit, slice) of the queue of the XCD the workgroup runs on, or of the next queue that is not empty:
@@ -262,7 +387,7 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
     };
     auto stage_next = [&](int hrows, uint32_t dst_wave) {
       const uint32_t off = lane16 + (uint32_t)st_j * (kWave * 16u);
-      if (!(a.dbg & 4)) panel_copy16_if(dst_wave + (uint32_t)(st_r * rs) + (uint32_t)st_j * (kWave * 16u), st_base, off, st_lim);
+      panel_copy16_if(dst_wave + (uint32_t)(st_r * rs) + (uint32_t)st_j * (kWave * 16u), st_base, off, st_lim);
       if (++st_j == ppr) {
         st_j = 0;
         if (++st_r < TCW) stage_row(hrows, st_r);
@@ -355,33 +480,39 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
         pc = npieces;
       }
 
+      // cnt records in the lanes of r.  K records at a time: their rows of B are read from LDS, then one stretch of
+      // index mode multiplies them (while a wave waits for its reads the other waves of the SIMD multiply).
       auto process = [&](const uint2 r, int cnt) {
         const uint32_t c = r.x & 0xffu;
-        const uint32_t packed = ((c & 15u) * (uint32_t)area + (c >> 4) * (uint32_t)rs) | (((r.x >> 8) * (uint32_t)NR) << 20);
-        float ba[NR], bb[NR];
-        uint32_t s0 = __builtin_amdgcn_readlane(packed, 0);
-        tile_row_read<NR>(lbase + (s0 & 0xfffffu), lane, ba);
+        const uint32_t packed = (((c & 15u) * (uint32_t)area + (c >> 4) * (uint32_t)rs) << 8) | ((r.x >> 8) * (uint32_t)NR);
+        constexpr int K = NR == 1 ? 8 : NR == 2 ? 4 : 2;
         int i = 0;
-        for (; i + 1 < cnt; i += 2) {
-          const uint32_t s1 = __builtin_amdgcn_readlane(packed, i + 1);
-          const float v0 = __uint_as_float(__builtin_amdgcn_readlane(r.y, i));
-          const float v1 = __uint_as_float(__builtin_amdgcn_readlane(r.y, i + 1));
-          tile_row_read<NR>(lbase + (s1 & 0xfffffu), lane, bb);
-          __builtin_amdgcn_sched_barrier(0);  // the reads stay ahead of the multiplies they overlap with
-          if (!(a.dbg & 2)) tile_fma<NR>(acc, s0 >> 20, v0, ba);
-          s0 = __builtin_amdgcn_readlane(packed, (i + 2) & (kWave - 1));  // behind the last record: some lane's valid record
-          tile_row_read<NR>(lbase + (s0 & 0xfffffu), lane, ba);
-          __builtin_amdgcn_sched_barrier(0);
-          if (!(a.dbg & 2)) tile_fma<NR>(acc, s1 >> 20, v1, bb);
+        for (; i + K <= cnt; i += K) {
+          uint32_t pk[K];
+          float v[K], b[K][NR];
+#pragma unroll
+          for (int k = 0; k < K; ++k) {
+            pk[k] = __builtin_amdgcn_readlane(packed, i + k);
+            v[k] = __uint_as_float(__builtin_amdgcn_readlane(r.y, i + k));
+            tile_row_read<NR>(lbase + (pk[k] >> 8), lane, b[k]);
+          }
+          tile_window<NR, K>(acc, pk, v, b);
           if (NR >= 4 && pc < npieces) {
             stage_next(hn, dst32);
             ++pc;
           }
         }
-        if (i < cnt) tile_fma<NR>(acc, s0 >> 20, __uint_as_float(__builtin_amdgcn_readlane(r.y, i)), ba);
+        for (; i < cnt; ++i) {
+          uint32_t pk[1];
+          float v[1], b[1][NR];
+          pk[0] = __builtin_amdgcn_readlane(packed, i);
+          v[0] = __uint_as_float(__builtin_amdgcn_readlane(r.y, i));
+          tile_row_read<NR>(lbase + (pk[0] >> 8), lane, b[0]);
+          tile_window<NR, 1>(acc, pk, v, b);
+        }
       };
       uint2 cur = rec;
-      for (int base = e0; base < ((a.dbg & 8) ? e0 : e1); base += kWave) {
+      for (int base = e0; base < e1; base += kWave) {
         const int left = e1 - base;
         uint2 nxt = cur;
         if (left > kWave) nxt = rec_load(base + kWave, e0, e1);

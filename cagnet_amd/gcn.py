@@ -58,15 +58,75 @@ _aligned_rows = ops.aligned_rows
 narrow_backward = True
 
 
+# With every stage operand resident, the stage loop z = sum_k A_k H_k is one product of the blocks side by side,
+# [A_0 | A_1 | ...], with the H_k stacked (one plan over the whole block row, Z written once instead of read and
+# written again per stage); `fuse_stages = False` keeps the reference's one product per stage (gcn_distr.py:221-244).
+# Same sums, other order of the additions.  The stacked matrix is a second copy of the blocks' entries (built at
+# the first fused loop over a list of blocks and kept with it), and the stage operands are kept stacked in one
+# buffer per direction: the peers' blocks are copied into it once, the rank's own block before every product.
+fuse_stages = True
+
+
+class StackedPeers(list):
+    """The resident blocks of a stage loop (a list, None at the caller's own index), also kept stacked in one
+    buffer so that the loop can run as one product."""
+
+    def __init__(self, blocks: Sequence[Optional[torch.Tensor]]):
+        super().__init__(blocks)
+        self.buffer = None      # [sum of the blocks' rows, width], built on first use
+        self.offsets = None     # first row of every stage's block in it
+        self.filled_for = None  # rank whose peers have been copied in
+
+    def stacked(self, rank: int, own: torch.Tensor, rows: Sequence[int]) -> torch.Tensor:
+        """The buffer with the peers' blocks in place and `own` copied to the caller's slot."""
+        width = own.shape[1]
+        if self.buffer is None or self.buffer.shape[1] != width or self.filled_for != rank:
+            self.offsets = [sum(rows[:k]) for k in range(len(rows) + 1)]
+            ld = width if width % 32 == 0 or width < 64 else (width + 31) // 32 * 32  # wide rows on 128-byte boundaries
+            self.buffer = torch.empty(self.offsets[-1], ld, dtype=own.dtype, device=own.device)[:, :width]
+            for k, blk in enumerate(self):
+                if k != rank:
+                    if blk is None or blk.shape != (rows[k], width):
+                        raise ValueError(f"stage {k}: resident block is missing or has the wrong shape")
+                    self.buffer[self.offsets[k]:self.offsets[k + 1]].copy_(blk)
+            self.filled_for = rank
+        if own.shape[0] != rows[rank]:
+            raise ValueError(f"own block has {own.shape[0]} rows, the sparse block of stage {rank} has {rows[rank]} columns")
+        slot = self.buffer[self.offsets[rank]:self.offsets[rank + 1]]
+        if own.data_ptr() != slot.data_ptr():
+            with torch.no_grad():
+                slot.copy_(own)
+        return self.buffer
+
+
 class ResidentBlocks:
     """Stands where the reference passes a process group: the dense blocks that its broadcasts
     would deliver (gcn_distr.py:230), already resident in HBM.  `forward[i]` is the H block and
     `backward[i]` the gradient block of stage i; the entry of the calling rank itself is ignored
-    (its own tensor is used, as in the reference's `inputs.clone()` branch, gcn_distr.py:222-223)."""
+    (its own tensor is used, as in the reference's `inputs.clone()` branch, gcn_distr.py:222-223).
+    The blocks are taken as constant for the life of this object (they stand for received data)."""
 
     def __init__(self, forward: Sequence[Optional[torch.Tensor]], backward: Sequence[Optional[torch.Tensor]]):
-        self.forward = list(forward)
-        self.backward = list(backward)
+        self.forward = StackedPeers(forward)
+        self.backward = StackedPeers(backward)
+
+
+_stacks: dict = {}   # id of a list's first block -> (weak references to its blocks, transpose, the stacked matrix)
+
+
+def stacked_blocks(am_partitions: Sequence[CsrMatrix]) -> CsrMatrix:
+    """[A_0 | A_1 | ...] for a list of blocks, built once per list (ops.CsrMatrix.hstack)."""
+    import weakref
+
+    key = id(am_partitions[0])
+    hit = _stacks.get(key)
+    if hit is not None and len(hit[0]) == len(am_partitions) and all(r() is b for r, b in zip(hit[0], am_partitions)):
+        return hit[1]
+    for k in [k for k, v in _stacks.items() if any(r() is None for r in v[0])]:
+        del _stacks[k]
+    stacked = CsrMatrix.hstack(am_partitions)
+    _stacks[key] = ([weakref.ref(b) for b in am_partitions], stacked)
+    return stacked
 
 
 def _stage_operand(i: int, rank: int, own: torch.Tensor, peers: Optional[Sequence[Optional[torch.Tensor]]]):
@@ -91,6 +151,11 @@ def broad_func(node_count: int, am_partitions: Sequence[CsrMatrix], inputs: torc
     `out`, when given, receives the sum (it may be a column slice of a wider buffer)."""
     if len(am_partitions) != size:
         raise ValueError(f"{len(am_partitions)} sparse blocks for size {size}")
+    if (fuse_stages and 1 < size <= 16 and not transpose and isinstance(group, StackedPeers) and len(group) == size
+            and 0 <= rank < size):
+        stacked = stacked_blocks(am_partitions)
+        h_all = group.stacked(rank, inputs, [blk.m for blk in am_partitions])
+        return stacked.spmm(h_all) if out is None else stacked.spmm(h_all, out=out, beta=0.0)
     z_loc = None
     for i in range(size):
         h_i = _aligned_rows(_stage_operand(i, rank, inputs, group))

@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import ctypes
 from ctypes import c_int64, c_void_p
-from typing import Optional, Tuple
+from typing import Optional, Sequence, Tuple
 
 import torch
 
@@ -266,6 +266,28 @@ class CsrMatrix:
         a = a.coalesce()
         idx = a.indices()
         return cls(idx[0].int(), idx[1].int(), a.values().float(), a.shape[0], a.shape[1], is_sorted=True, **kw)
+
+    @classmethod
+    def hstack(cls, blocks: Sequence["CsrMatrix"], transpose: bool = False) -> "CsrMatrix":
+        """[A_0 | A_1 | ...]: the blocks of one block row side by side as one matrix (cg_csr_hstack).  One product
+        with the stacked dense blocks is the whole stage loop sum_k A_k H_k (gcn_distr.py:221-244).  The entries
+        are copied; `col_offsets[k]` is the first column of block k in the result."""
+        blocks = list(blocks)
+        if not blocks:
+            raise ValueError("hstack of no blocks")
+        self = cls.__new__(cls)
+        self._handle = None
+        self.device = blocks[0].device
+        arr = (c_void_p * len(blocks))(*[b._handle for b in blocks])
+        handle = c_void_p(0)
+        with torch.cuda.device(self.device):
+            check(lib.cg_csr_hstack(ctypes.byref(handle), arr, len(blocks), CG_CSR_TRANSPOSE if transpose else 0, _stream()),
+                  "cg_csr_hstack")
+        self._handle = handle
+        self.n, self.m, self.nnz = blocks[0].n, sum(b.m for b in blocks), sum(b.nnz for b in blocks)
+        self.has_transpose = bool(transpose)
+        self.col_offsets = [sum(b.m for b in blocks[:k]) for k in range(len(blocks) + 1)]
+        return self
 
     def __del__(self):
         h = getattr(self, "_handle", None)

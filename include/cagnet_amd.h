@@ -170,6 +170,14 @@ int cg_coo_cache_info(int64_t info[4]);
 int cg_csr_create(cg_csr_t **out, const int32_t *d_row, const int32_t *d_col, const float *d_val, int64_t nnz,
                   int32_t n, int32_t m, uint32_t flags, cg_stream_t stream);
 int cg_csr_destroy(cg_csr_t *h);
+/* [A_0 | A_1 | ... | A_{count-1}] as one handle: the blocks of one block row of a partitioned matrix (equal row
+ * counts; at most 16), side by side in the order given, block k's columns behind those of the blocks before it.
+ * One product of the new handle with the dense blocks H_k stacked in the same order (rows of H_0, then of H_1, ...)
+ * is the whole stage loop z = sum_k A_k H_k that the reference runs as one spmm_gpu call per stage
+ * (gcn_distr.py:221-244, gcn_distr_2d.py:333-417): Z is written once instead of once per stage.  The entries are
+ * copied (the blocks stay as they are and may be destroyed afterwards); CG_CSR_TRANSPOSE in `flags` also builds
+ * the transpose of the stacked matrix.  Synchronises `stream`. */
+int cg_csr_hstack(cg_csr_t **out, cg_csr_t *const *blocks, int32_t count, uint32_t flags, cg_stream_t stream);
 /* Frees the tables parked on a handle since one of its products was captured into a HIP graph (see
  * Conventions) and lets later replacements free at once again.  Synchronises the device.  *released
  * (nullable) receives the number of device allocations freed.  Only for callers that have dropped every

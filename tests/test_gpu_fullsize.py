@@ -267,6 +267,25 @@ def test_reddit_shape_grid_row_of_blocks(cuda):
         a, hb = val[s:e].double(), H[col[s:e]].double()
         err = ((z[i - b[r]].double() - a @ hb).abs() / (a.abs() @ hb.abs()).clamp_min(1e-30)).max()
         assert float(err) <= REL_TOL, f"row {i}: {float(err)}"
+    # the same stage loop as one product of the blocks side by side (gcn.broad_func with resident operands):
+    # against the per-stage sums, against the rows recomputed in fp64, and bit-identical when repeated
+    from cagnet_amd import gcn
+    blocks = []
+    for k in range(q):
+        br, bc, bv = ops.coo_block(r32, c32, val, b[r], b[r + 1], b[k], b[k + 1])
+        blocks.append(ops.CsrMatrix(br, bc, bv, rows, b[k + 1] - b[k]))
+        del br, bc, bv
+    peers = gcn.StackedPeers([None if k == r else H[b[k]:b[k + 1]] for k in range(q)])
+    own = H[b[r]:b[r + 1]].contiguous()
+    zf = gcn.broad_func(rows, blocks, own, r, q, peers)
+    assert gcn.stacked_blocks(blocks).nnz == total and gcn.stacked_blocks(blocks).m == n
+    assert float(((zf - z).abs() / mag.clamp_min(1e-30)).max()) <= 4 * REL_TOL
+    assert torch.equal(zf, gcn.broad_func(rows, blocks, own, r, q, peers))
+    for i in torch.randint(b[r], b[r + 1], (32,), generator=torch.Generator().manual_seed(31)).tolist():
+        s, e = int(rowptr[i]), int(rowptr[i + 1])
+        a, hb = val[s:e].double(), H[col[s:e]].double()
+        err = ((zf[i - b[r]].double() - a @ hb).abs() / (a.abs() @ hb.abs()).clamp_min(1e-30)).max()
+        assert float(err) <= REL_TOL, f"fused stage loop, row {i}: {float(err)}"
 
 
 # ------------------------------------------------------------------------------------------------

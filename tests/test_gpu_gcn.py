@@ -123,6 +123,50 @@ def test_training_losses_match_oracle(cuda, monkeypatch, fused_loss):
     _close(w2, w2_64, "w2 after 100 epochs", 1e-3)
 
 
+@pytest.mark.parametrize("width", [64, 602, 41])
+def test_fused_stage_loop_matches_oracle_stage_loop(cuda, monkeypatch, width):
+    """z = sum_k A(r,k) H_k as one product of the blocks side by side (CsrMatrix.hstack, gcn.fuse_stages) against the
+    oracle's stage loop (gcn_distr.py:221-244) and against the library's own per-stage loop; the stacked matrix has
+    the blocks' entries in (row, block, column) order; repeated calls give the same bits; a changed own block is
+    picked up (it is copied into its slot of the stacked operands on every call)."""
+    from cagnet_amd import gcn, ops
+    q, r = 4, 2
+    p = synth.make_problem(n=3001, target_nnz=90001, features=8, hidden=4, classes=3, mask_fraction=0.5, seed=9)
+    b = synth.block_bounds_2d(p.n, q)
+    rows = b[r + 1] - b[r]
+    blocks, cpu = [], []
+    for k in range(q):
+        rr, cc, vv = synth.coo_block(p.row, p.col, p.val, b[r], b[r + 1], b[k], b[k + 1])
+        blocks.append(ops.CsrMatrix(rr.int().to(cuda), cc.int().to(cuda), vv.to(cuda), rows, b[k + 1] - b[k]))
+        cpu.append(orc.coo_tensor(rr, cc, vv, rows, b[k + 1] - b[k], torch.float64))
+    S = ops.CsrMatrix.hstack(blocks)
+    assert (S.n, S.m, S.nnz) == (rows, p.n, sum(blk.nnz for blk in blocks)) and S.col_offsets == b
+    rowptr, colind, values = S.arrays()
+    wr, wc, wv = synth.coo_block(p.row, p.col, p.val, b[r], b[r + 1], 0, p.n)   # the same rows of the whole matrix
+    assert torch.equal(colind.cpu().long(), wc) and torch.equal(values.cpu(), wv)
+    assert torch.equal(rowptr.cpu().long(), torch.searchsorted(wr, torch.arange(rows + 1)))
+    gen = torch.Generator().manual_seed(3)
+    H = [torch.randn(b[k + 1] - b[k], width, generator=gen) for k in range(q)]
+    ref = orc.stage_loop(cpu, [h.double() for h in H], torch.float64)
+    mag = orc.stage_loop([c.abs() for c in cpu], [h.double().abs() for h in H], torch.float64)
+    peers = gcn.StackedPeers([None if k == r else H[k].to(cuda) for k in range(q)])
+    own = H[r].to(cuda)
+    fused = gcn.broad_func(rows, blocks, own, r, q, peers)
+    assert orc.max_rel_error(fused, ref, mag) <= REL_TOL
+    assert torch.equal(fused, gcn.broad_func(rows, blocks, own, r, q, peers))
+    monkeypatch.setattr(gcn, "fuse_stages", False)
+    loop = gcn.broad_func(rows, blocks, own, r, q, peers)
+    assert orc.max_rel_error(loop, ref, mag) <= REL_TOL
+    monkeypatch.setattr(gcn, "fuse_stages", True)
+    own2 = own * 2.0
+    H2 = [h.double() for h in H]
+    H2[r] = H2[r] * 2.0
+    assert orc.max_rel_error(gcn.broad_func(rows, blocks, own2, r, q, peers), orc.stage_loop(cpu, H2, torch.float64), 2 * mag) <= REL_TOL
+    out = torch.full((rows, width + 3), 7.0, device=cuda)                          # into a column slice of a wider buffer
+    gcn.broad_func(rows, blocks, own, r, q, peers, out=out[:, :width])
+    assert orc.max_rel_error(out[:, :width], ref, mag) <= REL_TOL and bool((out[:, width:] == 7.0).all())
+
+
 def test_one_rank_share_of_2d_grid(cuda):
     """One rank's share of the 4x4 2D algorithm (gcn_distr_2d.py:333-417) with the broadcast
     operands resident: z = sum_k A(r,k) H_k over 4 stages, both layers, forward and backward."""

@@ -817,11 +817,11 @@ def test_spmm_from_two_host_threads_on_two_streams(cuda, tune):
         assert all(torch.equal(results[k][1], C) for C in results[k][3::2])      # handle form likewise
 
 
-def _panel_info(A, transpose=False):
+def _panel_info(A, transpose=False, narrow=False):
     import ctypes
     from cagnet_amd._lib import check, lib
     buf = (ctypes.c_int64 * 12)()
-    check(lib.cg_csr_panel_info(A._handle, int(transpose), buf), "cg_csr_panel_info")   # bit 1: plan of the narrow products
+    check(lib.cg_csr_panel_info(A._handle, int(transpose) | (2 if narrow else 0), buf), "cg_csr_panel_info")   # bit 1: plan of the narrow products
     return dict(state=buf[0], covered=buf[1], tiles=buf[2], units=buf[3], split=buf[4], rest=buf[5], emin=buf[6], cols=buf[7],
                 dense_covered=buf[8], dense_tiles=buf[9], dense_units=buf[10], dmin=buf[11])
 
@@ -1101,6 +1101,141 @@ def test_spmm_panel_plan_rectangular_strided_and_declined(cuda, tune):
     tune("spmm_panel", 1)
     got = U.spmm(Bu)                                                 # forced: still correct, whatever the coverage
     assert spmm_error(got, ur, uc, uv, 3000, 3000, Bu.cpu()) <= REL_TOL
+
+
+def _tile_info(A, f, transpose=False):
+    """The tile plan (spmm_tile_kernel) a product of width f uses: panels of 256 / 512 / 1024 rows."""
+    import ctypes
+    from cagnet_amd._lib import check, lib
+    which = 1 + (2 if f <= 64 else 1 if f <= 128 else 0)
+    buf = (ctypes.c_int64 * 12)()
+    check(lib.cg_csr_panel_info(A._handle, int(transpose) | (which << 2), buf), "cg_csr_panel_info")
+    return dict(state=buf[0], covered=buf[1], tiles=buf[2], units=buf[3], split=buf[4], rest=buf[5])
+
+
+@pytest.mark.parametrize("f", [16, 44, 64, 68, 96, 128, 132, 192, 256, 260, 302, 320, 602, 636, 640, 1000])
+def test_spmm_tile_plan_matches_oracle(cuda, tune, f):
+    """Every width class of the tile kernel with its plan forced on: one register per row and panels of 1024 rows
+    (f <= 64), two and 512 (f <= 128), four or five and 256 (wider, in column slices of up to 316: 602 takes two, 1000
+    four).  Both accumulate forms, the transpose side, bit-identical repeats; small units so that panels have several
+    blocks of partial rows as well as units that write C themselves."""
+    from cagnet_amd import ops
+    row, col, val, n = small_graph(13, 400000, seed=3 * f + 1)
+    g = torch.Generator().manual_seed(f)
+    B = torch.randn(n, f, generator=g)
+    C0 = torch.randn(n, f, generator=g)
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n, transpose=True)
+    tune("spmm_tile", 1)
+    for unit in (0, 3000):
+        tune("spmm_panel_unit", unit)
+        got = A.spmm(B.to(cuda))
+        info = _tile_info(A, f)
+        assert info["state"] == 1 and info["covered"] == row.numel() and info["rest"] == 0 and info["tiles"] > 0
+        if unit:
+            assert info["split"] > 0
+        assert spmm_error(got, row, col, val, n, n, B) <= REL_TOL
+        assert torch.equal(got, A.spmm(B.to(cuda)))
+        C = C0.to(cuda).clone()
+        A.spmm(B.to(cuda), out=C, beta=1.0)
+        assert spmm_error(C, row, col, val, n, n, B, C0) <= REL_TOL
+    gotT = A.spmm(B.to(cuda), transpose=True)                        # the graph is symmetric: same product
+    assert _tile_info(A, f, transpose=True)["state"] == 1
+    assert spmm_error(gotT, row, col, val, n, n, B) <= REL_TOL
+
+
+def test_spmm_tile_plan_rectangular_strided_and_refused_operands(cuda, tune):
+    """A rectangular, non-symmetric matrix with empty rows; B and C as column slices of wider buffers.  Operands the
+    tile kernel cannot copy from (rows an odd number of floats apart; a narrow width that is not a multiple of 4)
+    go to the other kernels and give the same product."""
+    from cagnet_amd import ops
+    from tests.util import random_coo
+    n, m = 3000, 5000
+    row, col, val = random_coo(n, m, 150000, seed=21)
+    keep = row % 7 != 3                                              # rows without entries
+    row, col, val = row[keep], col[keep], val[keep]
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, m, transpose=True)
+    tune("spmm_tile", 1)
+    for f, ld in ((300, 308), (602, 610), (128, 136), (64, 72), (48, 64)):
+        Bw = torch.randn(m, ld, generator=torch.Generator().manual_seed(f))
+        B = Bw[:, 4:4 + f]                                           # rows ld floats apart, 16 bytes into the buffer
+        Cd = torch.full((n, f + 5), 3.0, device=cuda)
+        A.spmm(Bw.to(cuda)[:, 4:4 + f], out=Cd[:, 2:2 + f])
+        assert _tile_info(A, f)["state"] == 1
+        assert spmm_error(Cd[:, 2:2 + f], row, col, val, n, m, B) <= REL_TOL
+        assert bool((Cd[:, :2] == 3.0).all()) and bool((Cd[:, 2 + f:] == 3.0).all())
+        Bt = torch.randn(n, f, generator=torch.Generator().manual_seed(f + 1))
+        assert spmm_error(A.spmm(Bt.to(cuda), transpose=True), col, row, val, m, n, Bt) <= REL_TOL
+    for f in (301, 63, 46):                                          # odd leading dimension / narrow and not a multiple of 4
+        B = torch.randn(m, f, generator=torch.Generator().manual_seed(f))
+        assert spmm_error(A.spmm(B.to(cuda)), row, col, val, n, m, B) <= REL_TOL
+
+
+@pytest.mark.parametrize("f", [602, 64])
+def test_non_finite_rows_of_B(cuda, tune, f):
+    """One row of B holds +inf, another NaN.  cusparseSpMM (sparse-extension/sparse_coo_tensor.cu:215-226) and
+    torch.sparse.mm touch only the rows of C that reference them: that is what the row-wise kernels, the tile plans
+    and `spmm_strict_nonfinite` give, exactly.  The panel plan with tiles on the matrix cores is documented to differ:
+    a dense tile multiplies its zeros, so a non-finite row of B reaches every row of the tile (rows that reference
+    neither column come out either untouched or non-finite, never as another finite number), and the zero records
+    that pad odd runs can turn an infinity into a NaN in a row that references it; without dense tiles
+    (`spmm_panel_dmin = -1`) the rows that reference neither column are untouched."""
+    from cagnet_amd import ops
+    row, col, val, n = small_graph(11, 260000, seed=5)               # 127 entries per row: dense and staged tiles
+    deg = torch.bincount(col, minlength=n)
+    order = torch.argsort(deg, descending=True)
+    j_inf, j_nan = int(order[3]), int(order[40])                     # two popular columns
+    refs_inf = torch.zeros(n, dtype=torch.bool)
+    refs_nan = torch.zeros(n, dtype=torch.bool)
+    refs_inf[row[col == j_inf]] = True
+    refs_nan[row[col == j_nan]] = True
+    assert 0 < int(refs_inf.sum()) < n and 0 < int(refs_nan.sum()) < n and int((~refs_inf & ~refs_nan).sum()) > 0
+    B = torch.randn(n, f, generator=torch.Generator().manual_seed(2))
+    Bbad = B.clone()
+    Bbad[j_inf] = float("inf")
+    Bbad[j_nan] = float("nan")
+    ref = torch.sparse.mm(orc.coo_tensor(row, col, val, n, n, torch.float32), Bbad)   # the reference's CPU twin
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n)
+    clean_rows = ~refs_inf & ~refs_nan
+
+    def check_reference_semantics(what):
+        clean = A.spmm(B.to(cuda)).cpu()
+        got = A.spmm(Bbad.to(cuda)).cpu()
+        assert torch.equal(torch.isnan(got), torch.isnan(ref)), what
+        assert torch.equal(torch.isinf(got) & (got > 0), torch.isinf(ref) & (ref > 0)), what
+        assert torch.equal(torch.isinf(got) & (got < 0), torch.isinf(ref) & (ref < 0)), what
+        assert torch.equal(got[clean_rows], clean[clean_rows]), what
+
+    tune("spmm_panel", -1)
+    tune("spmm_panel_narrow", -1)
+    check_reference_semantics("row-wise kernels")
+    tune("spmm_panel", 0)
+    tune("spmm_panel_narrow", 0)
+    tune("spmm_tile", 1)
+    check_reference_semantics("tile plan")
+    assert _tile_info(A, f)["state"] == 1
+    tune("spmm_tile", -1)
+    tune("spmm_panel", 1)
+    tune("spmm_panel_narrow", 1)
+    tune("spmm_strict_nonfinite", 1)                                 # the plans that deviate stand back
+    check_reference_semantics("strict")
+    tune("spmm_strict_nonfinite", 0)
+    clean = A.spmm(B.to(cuda)).cpu()
+    got = A.spmm(Bbad.to(cuda)).cpu()
+    info = _panel_info(A, narrow=(f <= 64)) if f <= 64 else _panel_info(A)
+    assert info["state"] == 1 and info["dense_tiles"] > 0
+    assert not bool(torch.isfinite(got[refs_inf | refs_nan]).all(dim=1).any())       # every referencing row is non-finite
+    untouched = (got[clean_rows] == clean[clean_rows]).all(dim=1)
+    tainted = ~torch.isfinite(got[clean_rows]).all(dim=1)
+    assert bool((untouched | tainted).all())
+    assert bool(tainted.any())                                       # the documented deviation is real on this matrix
+    if f > 64:
+        tune("spmm_panel_dmin", -1)
+        A2 = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n)
+        clean2 = A2.spmm(B.to(cuda)).cpu()
+        got2 = A2.spmm(Bbad.to(cuda)).cpu()
+        assert _panel_info(A2)["state"] == 1 and _panel_info(A2)["dense_tiles"] == 0
+        assert torch.equal(got2[clean_rows], clean2[clean_rows])
+        assert not bool(torch.isfinite(got2[refs_inf | refs_nan]).all(dim=1).any())
 
 
 def test_captured_graph_outlives_plan_eviction_and_scratch_growth(cuda, tune):
