@@ -345,26 +345,30 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
     d.epi_relu = epi->epi_relu;
   }
   // Tile plan: every entry is multiplied out of LDS by spmm_tile_kernel, in panels whose height goes by the width.
-  if (!epi && !fold && allow_panel && want_tile(s, f) &&
-      tile_operands_ok(tile_params(tile_geometry(f)).prows, tile_params(tile_geometry(f)).tcols, B, ldb, f, s.cols)) {
+  // `after_panel`: the second look, for the widths that the panel plan with its matrix-core tiles is tried for first.
+  bool tile_done = false;
+  auto try_tile = [&](bool after_panel) -> int {
+    if (epi || fold || !allow_panel || !want_tile(s, f, after_panel)) return CG_OK;
     const int geom = tile_geometry(f);
     const PanelParams par = tile_params(geom);
-    const bool may_decline = g_tune_tile.load(std::memory_order_relaxed) == 0;
+    if (!tile_operands_ok(par.prows, par.tcols, B, ldb, f, s.cols)) return CG_OK;
     PanelPlan &pp = s.tile[geom];
-    if (!pp.valid || !par.same(pp) || (pp.declined && !may_decline && !pp.failed)) {
-      const int st = build_panel(s, pp, par, may_decline, stream);
+    if (!pp.valid || !par.same(pp)) {
+      const int st = build_panel(s, pp, par, false, stream, 0.0, 0.0);
       if (st == CG_ERR_ALLOC || st == CG_ERR_OVERFLOW) {  // no memory for the plan: remembered as declined
         pp.declined = pp.failed = pp.valid = true;
       } else if (st != CG_OK) {
         return st;
       }
     }
-    if (!pp.declined && pp.rest->nnz == 0) {
-      float *P = nullptr;
-      CG_TRY(launch_panel(pp, B, ldb, f, &P, stream, false, C, ldc, s.rows, beta));
-      return launch_panel_finish(pp, P, C, ldc, f, beta, stream);
-    }
-  }
+    if (pp.declined || pp.rest->nnz != 0) return CG_OK;
+    float *P = nullptr;
+    CG_TRY(launch_panel(pp, B, ldb, f, &P, stream, false, C, ldc, s.rows, beta));
+    tile_done = true;
+    return launch_panel_finish(pp, P, C, ldc, f, beta, stream);
+  };
+  CG_TRY(try_tile(false));
+  if (tile_done) return CG_OK;
   // Panel plan: the entries of dense (row panel, column block) tiles are multiplied out of LDS into
   // partial rows; the row-wise kernels then run over the other entries and add those rows in.
   if (!epi && allow_panel && f <= cap && want_panel(s, f)) {
@@ -393,6 +397,8 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
       return spmm_side(*pp.rest, B, ldb, C, ldc, f, beta, stream, nullptr, &fd, false);
     }
   }
+  CG_TRY(try_tile(true));  // the panel plan stood back (too few entries share their column inside a panel of 128 rows)
+  if (tile_done) return CG_OK;
   // Narrow products: the dense tiles of a panel plan of their own on the matrix cores, the other entries by the
   // row-wise kernels, then the partial rows are added in (a pass over an n x f array, which is small here).
   if (!epi && !fold && allow_panel && want_panel_narrow(s, f)) {

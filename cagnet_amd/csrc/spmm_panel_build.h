@@ -50,11 +50,26 @@ static bool want_panel(const CsrSide &s, int32_t f) {
 //   geometry 0: panels of 256 rows, tiles of 64 columns: widths above 128, in slices of up to 316 columns
 //   geometry 1: 512 x 128: widths 65 .. 128          geometry 2: 1024 x 256: widths up to 64
 static int tile_geometry(int32_t f) { return f <= 64 ? 2 : f <= 128 ? 1 : 0; }
-static bool want_tile(const CsrSide &s, int32_t f) {
+static bool panel_width_ok(int32_t f);
+// Measured, tile plan against the library's other kernels (ms; 232,965 vertices with 492 entries per row | R-MAT
+// scale 20 with 31 | 14,249,639 vertices with 16):
+//   f = 1000  17.0 / 29.7 | 11.5 / 14.0        f = 700  12.6 / 19.6 | 8.2 / 9.5         f = 602  10.6 / 8.2 | 6.7 / 6.1
+//   f = 300   5.4 / 5.8 | 3.3 / 4.1 | 35.8 / 42.9          f = 256  4.3 / 6.4 | 2.7 / 3.4          f = 128  2.5 / 3.3 | 1.4 / 1.8
+//   f = 64    2.1 / 1.4 | 0.90 / 1.14 | 7.5 / 10.7         f = 48   2.1 / 1.5         f = 24   - | - | 6.5 / 5.1        f = 16  2.0 / 0.70 | 0.81 / 0.39
+// So: every width from 65 on except those where the panel plan with its matrix-core tiles is in use (even 318..636,
+// where two column slices visit every record twice), and 48..64 on matrices of under 64 entries per row (denser ones
+// have the narrow plan's matrix-core tiles).  Products under 8e8 multiply-adds or 8 entries per row stay row-wise.
+static bool want_tile(const CsrSide &s, int32_t f, bool after_panel) {
   const int t = g_tune_tile.load(std::memory_order_relaxed);
   if (t < 0 || s.rows == 0 || s.nnz == 0 || s.is_rest || f < 1) return false;
-  if (t > 0) return true;
-  return false;
+  if (t > 0) return !after_panel;
+  if (s.nnz / s.rows < 8 || (double)s.nnz * f < 8e8) return false;
+  const bool panel_first = panel_width_ok(f) && f > 316 && g_tune_panel.load(std::memory_order_relaxed) >= 0 &&
+                           g_tune_strict.load(std::memory_order_relaxed) <= 0;
+  if (panel_first != after_panel) return false;
+  if (after_panel) return s.panel.valid && s.panel.declined;  // the panel plan looked at the matrix and stood back
+  if (f >= 65) return true;
+  return f >= 48 && s.nnz / s.rows < 64;
 }
 
 static int alloc_sort_buffers(DevTemps &tmp, SortBuffers &buf, int64_t count) {
@@ -726,7 +741,7 @@ struct TileShape {
 static bool tile_shape(int32_t prows, int32_t tcols, int32_t f, TileShape &sh) {
   const int32_t R = prows / kPanelWaves;
   int32_t cap = R <= 8 ? 636 : R <= 16 ? 316 : R <= 32 ? 128 : R <= 64 ? 64 : 0;
-  const int32_t lds_cap = (int32_t)((160 * 1024 - 64) / (2 * (size_t)tcols) / 16 * 4);  // columns two tiles leave room for
+  const int32_t lds_cap = (int32_t)((160 * 1024 - 1024 - 256) / (2 * (size_t)tcols) / 16 * 4);  // columns two tiles leave room for
   if (lds_cap < cap) cap = lds_cap;
   if (cap < 4 || f < 1) return false;
   sh.nsl = (f + cap - 1) / cap;
@@ -785,10 +800,9 @@ static int launch_tile(const PanelPlan &pp, const float *B, int64_t ldb, int32_t
   ta.beta = beta;
   // two tiles of staged rows (narrow slices: a wave's staging area is a whole number of 1 KiB pieces) and some room
   // behind them: the lanes of a row read beyond the slice's last column
-  const size_t tlds_max = 160 * 1024 - 64;
-  const size_t rs = (size_t)sh.fsw * 4;
-  const size_t area = sh.nr >= 4 ? (size_t)(pp.tcols / kPanelWaves) * rs
-                                 : (size_t)ceil_div64((int64_t)(pp.tcols / kPanelWaves) * (sh.fsw / 4), kWave) * (kWave * 16);
+  const size_t tlds_max = 160 * 1024 - 1024;  // the kernel's own LDS word lies in front, the buffers start on a multiple of 1024
+  const size_t rs = sh.nr == 1 ? 256 : sh.nr == 2 ? 512 : sh.nr == 4 ? 1024 : (size_t)sh.fsw * 4;  // LROW of the kernel
+  const size_t area = (size_t)(pp.tcols / kPanelWaves) * rs;
   size_t tlds = 2 * (size_t)kPanelWaves * area + 256;
   if (tlds > tlds_max) tlds = tlds_max;
   if (2 * (size_t)kPanelWaves * area > tlds_max) CG_FAIL(CG_ERR_UNSUPPORTED, "tile product: f=%d does not fit the LDS", f);

@@ -57,34 +57,43 @@ __device__ __forceinline__ int tile_col(int k, int lane) {
   return 512 + 2 * lane + (k - 8);
 }
 
+typedef float tile_f2 __attribute__((ext_vector_type(2)));
+typedef float tile_f4 __attribute__((ext_vector_type(4)));
+template <typename T>
+__device__ __forceinline__ T tile_lds_load(uint32_t addr) {  // addr: a byte address in LDS
+  return *(const __attribute__((address_space(3))) T *)addr;
+}
+
+// The lane's registers of a staged row.  a0: LDS address of the lane's first piece (row + lane * 4, 8 or 16 by the
+// layout above); a1: of its piece with the other lane stride (NR 5, 6, 10; unused otherwise).
 template <int NR>
-__device__ __forceinline__ void tile_row_read(const char *src, int lane, float (&b)[NR]) {
+__device__ __forceinline__ void tile_row_read(uint32_t a0, uint32_t a1, float (&b)[NR]) {
   if constexpr (NR == 1) {
-    b[0] = *reinterpret_cast<const float *>(src + lane * 4);
+    b[0] = tile_lds_load<float>(a0);
   } else if constexpr (NR == 2) {
-    const float2 v = *reinterpret_cast<const float2 *>(src + lane * 8);
+    const tile_f2 v = tile_lds_load<tile_f2>(a0);
     b[0] = v.x;
     b[1] = v.y;
   } else {
-    const float4 v = *reinterpret_cast<const float4 *>(src + lane * 16);
+    const tile_f4 v = tile_lds_load<tile_f4>(a0);
     b[0] = v.x;
     b[1] = v.y;
     b[2] = v.z;
     b[3] = v.w;
     if constexpr (NR == 5) {
-      b[4] = *reinterpret_cast<const float *>(src + 1024 + lane * 4);
+      b[4] = tile_lds_load<float>(a1);
     } else if constexpr (NR == 6) {
-      const float2 w = *reinterpret_cast<const float2 *>(src + 1024 + lane * 8);
+      const tile_f2 w = tile_lds_load<tile_f2>(a1);
       b[4] = w.x;
       b[5] = w.y;
     } else if constexpr (NR >= 8) {
-      const float4 w = *reinterpret_cast<const float4 *>(src + 1024 + lane * 16);
+      const tile_f4 w = tile_lds_load<tile_f4>(a0 + 1024u);
       b[4] = w.x;
       b[5] = w.y;
       b[6] = w.z;
       b[7] = w.w;
       if constexpr (NR == 10) {
-        const float2 u = *reinterpret_cast<const float2 *>(src + 2048 + lane * 8);
+        const tile_f2 u = tile_lds_load<tile_f2>(a1);
         b[8] = u.x;
         b[9] = u.y;
       }
@@ -339,8 +348,12 @@ __device__ __forceinline__ int tile_take_item(const int32_t *__restrict__ unit_q
 template <int NR, int R, int TCW>
 __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs a) {
   static_assert(NR * R <= 80, "80 accumulator registers");
-  extern __shared__ __align__(16) char panel_lds[];
+  extern __shared__ __align__(1024) char panel_lds[];  // (the staged rows of narrow slices start on multiples of their stride)
   constexpr int HS = TCW + 2;
+  // Slices of up to 256 columns keep a staged row in a fixed stride of 256, 512 or 1024 bytes, whatever the slice's
+  // width: the row's offset is then a multiple of it, the record's accumulator index fits below it in the same
+  // word, and a lane's LDS address is (word & mask) | the lane's own offset: one instruction.
+  constexpr int LROW = NR == 1 ? 256 : NR == 2 ? 512 : NR == 4 ? 1024 : 0;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int32_t *__restrict__ hdr = a.hdr;
@@ -354,7 +367,7 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
     const float *__restrict__ Bs = a.B + col0;
     const int t0 = a.unit_tile[unit], t1 = a.unit_tile[unit + 1];
     const int c16 = (a.fsw + 3) >> 2;                 // 16-byte pieces of a staged row (every slice alike)
-    const int rs = c16 * 16;                          // bytes of a staged row
+    const int rs = LROW ? LROW : c16 * 16;            // bytes from one staged row to the next
     const uint32_t lim = (uint32_t)fs * 4u;              // bytes of a slice row
     // The last piece of a row may reach up to 12 bytes beyond the slice: into the next slice or the next row of B,
     // which is harmless (those columns of the accumulators are never stored) except behind the last row of B in
@@ -368,8 +381,8 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
     // 64 x 16 bytes from a wave-uniform base address (scalar arithmetic only; the lanes beyond the row's end are
     // switched off inside the copy).  The state below names the next piece; a tile has TCW * ppr of them.
     const int ppr = (c16 + kWave - 1) / kWave;  // pieces of a row
-    const int npieces = NR >= 4 ? TCW * ppr : (TCW * c16 + kWave - 1) / kWave;
-    const int bufsz = kPanelWaves * (NR >= 4 ? TCW * rs : npieces * (kWave * 16));  // bytes of a tile's buffer
+    const int npieces = NR >= 4 ? TCW * ppr : TCW * (LROW / 16) / kWave;  // (narrow slices: 4)
+    const int bufsz = kPanelWaves * TCW * rs;  // bytes of a tile's buffer
     const uint32_t lane16 = (uint32_t)lane * 16u;
     const uint32_t ldb32 = (uint32_t)a.ldb;  // the launch refuses leading dimensions of 2^31 and more
     int st_r = 0, st_j = 0;
@@ -394,25 +407,23 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
       }
     };
     // Narrower slices (NR < 4): a copy instruction covers several rows of B, so every lane has an offset of its own
-    // (32 bits from the slice's base: the launch makes sure that B fits).  A wave's staging area is a whole number
-    // of pieces; piece q = pc * 64 + lane of it is row q / c16, position q % c16.  Nothing is switched off: the
-    // lanes behind the wave's last row, and the positions behind a row's end, copy a valid piece once more into
-    // places nobody reads.  (The launch hands narrow products to this kernel only when f is a multiple of 4, so that
-    // every row of B ends with a whole piece.)
-    constexpr int NPN = NR >= 4 ? 1 : 4;  // pieces of a tile at most: 16 rows of 256 bytes, 8 of 512
+    // (32 bits from the slice's base: the launch makes sure that B fits).  A staged row takes LROW bytes, and piece
+    // q = pc * 64 + lane of the wave's staging area is row q / (LROW / 16), position q % (LROW / 16).  Nothing is
+    // switched off: positions behind the row's end copy the row's last piece once more, into places nobody reads.
+    // (The launch hands narrow products to this kernel only when f is a multiple of 4, so that every row of B ends
+    // with a whole piece.)
+    constexpr int NPN = NR >= 4 ? 1 : 4;  // pieces of a tile: 16 rows of 256 bytes, 8 of 512
     int nsel[NPN];
     uint32_t noff[NPN];
     if constexpr (NR < 4) {
+      constexpr uint32_t C16L = LROW / 16;
       const uint32_t cmax = (lim - 1u) >> 4;  // the last piece that starts inside a row
 #pragma unroll
       for (int pc = 0; pc < NPN; ++pc) {
         const uint32_t q = (uint32_t)(pc * kWave + lane);
-        uint32_t row = q / (uint32_t)c16;
-        uint32_t c = q - row * (uint32_t)c16;
-        row = row < (uint32_t)TCW ? row : (uint32_t)TCW - 1u;
-        c = c < cmax ? c : cmax;
+        const uint32_t row = q / C16L, c = q % C16L;
         nsel[pc] = (int)(row << 2);
-        noff[pc] = c * 16u;
+        noff[pc] = (c < cmax ? c : cmax) * 16u;
       }
     }
     const uint32_t ldb_bytes = ldb32 * 4u;
@@ -440,7 +451,7 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
       idx = idx < b1 ? idx : (b1 > b0 ? b1 - 1 : 0);
       return ent[idx];
     };
-    const int area = NR >= 4 ? TCW * rs : npieces * (kWave * 16);  // bytes of a wave's staging area in a buffer
+    const int area = TCW * rs;  // bytes of a wave's staging area in a buffer
     char *const wave_area = panel_lds + wave * area;
     const uint32_t wave_area32 = (uint32_t)(uintptr_t)wave_area;
 
@@ -481,33 +492,53 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
       }
 
       // cnt records in the lanes of r.  K records at a time: their rows of B are read from LDS, then one stretch of
-      // index mode multiplies them (while a wave waits for its reads the other waves of the SIMD multiply).
+      // index mode multiplies them (while a wave waits for its reads the other waves of the SIMD multiply).  A
+      // record becomes one word: the LDS offset of its row of B and, in the low 8 bits, its first accumulator.
+      const uint32_t lane_off = (uint32_t)lane * (NR == 1 ? 4u : NR == 2 ? 8u : 16u);
+      // the lane's second piece of a row: behind the first 1024 (2048) bytes, 4 (8) bytes per lane
+      const uint32_t lane_off2 = NR == 5 ? 1024u + (uint32_t)lane * 4u : NR == 6 ? 1024u + (uint32_t)lane * 8u
+                                                                                  : 2048u + (uint32_t)lane * 8u;
+      const uint32_t lbase32 = (uint32_t)(uintptr_t)lbase;
       auto process = [&](const uint2 r, int cnt) {
         const uint32_t c = r.x & 0xffu;
-        const uint32_t packed = (((c & 15u) * (uint32_t)area + (c >> 4) * (uint32_t)rs) << 8) | ((r.x >> 8) * (uint32_t)NR);
+        const uint32_t rowoff = lbase32 + (c & 15u) * (uint32_t)area + (c >> 4) * (uint32_t)rs;
+        const uint32_t idx = (r.x >> 8) * (uint32_t)NR;
+        const uint32_t packed = LROW ? (rowoff | idx) : ((rowoff << 8) | idx);
         constexpr int K = NR == 1 ? 8 : NR == 2 ? 4 : 2;
-        int i = 0;
-        for (; i + K <= cnt; i += K) {
+        auto read = [&](uint32_t pk, float (&b)[NR]) {
+          if constexpr (LROW != 0) {
+            uint32_t addr;  // (pk & ~(LROW - 1)) | lane_off: the row's address is a multiple of LROW, the index lies below it
+            asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(addr) : "s"(pk), "v"(~(uint32_t)(LROW - 1)), "v"(lane_off));
+            tile_row_read<NR>(addr, 0u, b);
+          } else {
+            const uint32_t row = pk >> 8;
+            tile_row_read<NR>(row + lane_off, row + lane_off2, b);
+          }
+        };
+        auto step = [&](int first) {  // K records from lane `first` on
           uint32_t pk[K];
           float v[K], b[K][NR];
 #pragma unroll
           for (int k = 0; k < K; ++k) {
-            pk[k] = __builtin_amdgcn_readlane(packed, i + k);
-            v[k] = __uint_as_float(__builtin_amdgcn_readlane(r.y, i + k));
-            tile_row_read<NR>(lbase + (pk[k] >> 8), lane, b[k]);
+            pk[k] = __builtin_amdgcn_readlane(packed, first + k);
+            v[k] = __uint_as_float(__builtin_amdgcn_readlane(r.y, first + k));
+            read(pk[k], b[k]);
           }
           tile_window<NR, K>(acc, pk, v, b);
+          __builtin_amdgcn_sched_barrier(0);  // the next K records' reads stay behind this stretch (registers)
           if (NR >= 4 && pc < npieces) {
             stage_next(hn, dst32);
             ++pc;
           }
-        }
+        };
+        int i = 0;
+        for (; i + K <= cnt; i += K) step(i);
         for (; i < cnt; ++i) {
           uint32_t pk[1];
           float v[1], b[1][NR];
           pk[0] = __builtin_amdgcn_readlane(packed, i);
           v[0] = __uint_as_float(__builtin_amdgcn_readlane(r.y, i));
-          tile_row_read<NR>(lbase + (pk[0] >> 8), lane, b[0]);
+          read(pk[0], b[0]);
           tile_window<NR, 1>(acc, pk, v, b);
         }
       };

@@ -541,11 +541,12 @@ def test_spmm_hub_plan_is_declined_when_columns_are_not_skewed(cuda):
         got = A.spmm(Bd)
         assert torch.equal(got, A.spmm(Bd))
         assert key.numel() * f >= 3e9                                  # large enough for a plan to be considered
-        tiers, panel = A.info()["plan_tiers"], _panel_info(A)["state"]
-        if skewed:                                                     # one of the two plans takes the popular columns
-            assert panel == 1 or tiers >= 1, (panel, tiers)
-        else:                                                          # the hub plan was looked at and declined; the panel
-            assert panel in (0, -1) and tiers == -1, (panel, tiers)    # plan likewise, or not considered at this size
+        tiers, panel, tile = A.info()["plan_tiers"], _panel_info(A)["state"], _tile_info(A, f)["state"]
+        if skewed:                                                     # one of the plans takes the popular columns
+            assert panel == 1 or tile == 1 or tiers >= 1, (panel, tile, tiers)
+        else:                                                          # the panel plan was looked at and declined (or not
+                                                                       # considered at this size); then the tile plan takes
+            assert panel in (0, -1) and (tile == 1 or tiers == -1), (panel, tile, tiers)   # the product, or the hub plan declines too
         keep = torch.isin(r, sample)
         ref_rows = torch.unique(r[keep])
         remap = torch.full((n,), -1, dtype=torch.long)
