@@ -89,6 +89,31 @@ def build_library(jobs: int | None = None, verbose: bool = True) -> Path:
     return LIB_PATH
 
 
+def kernel_resources(source: str = "spmm.hip", match: str = "spmm_tile_kernel") -> dict:
+    """Registers and scratch of the kernels of csrc/<source> whose names contain `match`, from the compiler's own
+    resource notes (the device pass only, to assembly text).  {mangled name: {"vgpr_count", "vgpr_spill_count",
+    "sgpr_spill_count", "private_segment_fixed_size"}}.  The tile kernels keep their accumulators in fixed registers
+    across inline-asm statements; that only holds while the register allocator spills nothing around them."""
+    import re
+    import tempfile
+
+    with tempfile.TemporaryDirectory() as tmp:
+        out = Path(tmp) / "kernels.s"
+        cmd = [_hipcc(), *HIPCC_FLAGS, "--offload-device-only", "-S", str(CSRC_DIR / source), "-o", str(out)]
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"hipcc failed for {source}:\n{proc.stderr}")
+        text = out.read_text()
+    found = {}
+    for block in re.split(r"\n  - \.agpr_count:", text)[1:]:
+        name = re.search(r"\.name:\s+(\S+)", block)
+        if not name or match not in name.group(1):
+            continue
+        keys = ("vgpr_count", "vgpr_spill_count", "sgpr_spill_count", "private_segment_fixed_size")
+        found[name.group(1)] = {k: int(re.search(rf"\.{k}:\s+(\d+)", block).group(1)) for k in keys}
+    return found
+
+
 def build_host_sanitized(jobs: int | None = None) -> Path:
     """The same sources with the host code instrumented by ASan and UBSan, as
     lib/libcagnet_amd_hostsan.so.  It is only ever linked into a sanitized test driver

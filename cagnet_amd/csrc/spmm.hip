@@ -165,7 +165,15 @@ static bool want_hub(int32_t rows, int64_t nnz, int32_t f) {
   if (t > 0) return true;
   return f >= 64 && nnz / rows >= 8 && (double)nnz * f >= 3e9;
 }
-static bool want_hub(const CsrSide &s, int32_t f) { return want_hub(s.rows, s.nnz, f); }
+// The rest matrix of a narrow panel plan (its dense tiles are gone: what is left are the entries of the less
+// popular columns) takes the plan from 40 columns on: measured on 232,965 vertices with 492 entries per row, f = 44
+// (rows of B 192 bytes apart): 1.56 -> 1.37 ms, f = 48: 1.54 -> 1.34 ms; on the whole matrix at those widths the
+// plan does not pay (1.85 -> 1.90 ms).
+static bool want_hub(const CsrSide &s, int32_t f) {
+  if (s.is_rest && f >= 40 && f < 64 && g_tune_hub.load(std::memory_order_relaxed) == 0)
+    return s.rows > 0 && s.nnz / s.rows >= 8 && (double)s.nnz * f >= 1.5e9;
+  return want_hub(s.rows, s.nnz, f);
+}
 
 // *declined: the plan was found not to pay for this matrix and width; nothing was computed.
 static int spmm_hub(CsrSide &s, int vec, const DenseOps &d, hipStream_t stream, bool *declined) {
@@ -913,6 +921,8 @@ int cg_tune_set(const char *key, int value) {
   else if (!strcmp(key, "spmm_panel_share")) cg::g_tune_panel_share.store(value);
   else if (!strcmp(key, "spmm_tile")) cg::g_tune_tile.store(value);
   else if (!strcmp(key, "spmm_strict_nonfinite")) cg::g_tune_strict.store(value);
+  else if (!strcmp(key, "spmm_panel_qskip")) cg::g_tune_panel_qskip.store(value);
+  else if (!strcmp(key, "spmm_panel_qcap")) cg::g_tune_panel_qcap.store(value);
   else if (!strcmp(key, "spmm_panel_narrow")) cg::g_tune_panel_narrow.store(value);
   else if (!strcmp(key, "spmm_panel_narrow_dmin")) cg::g_tune_panel_narrow_dmin.store(value);
   else if (!strcmp(key, "dense_mfma")) cg::g_tune_dense_mfma.store(value);

@@ -43,6 +43,7 @@ constexpr int kDenseTileFloats = kPanelRows * kPanelCols;
 
 static std::atomic<int> g_tune_panel{0}, g_tune_panel_emin{0}, g_tune_panel_cols{0}, g_tune_panel_unit{0};
 static std::atomic<int> g_tune_panel_dmin{0}, g_tune_panel_dwg{0}, g_tune_panel_share{0}, g_tune_tile{0}, g_tune_strict{0};
+static std::atomic<int> g_tune_panel_qskip{0}, g_tune_panel_qcap{0};  // measuring aid: a launch takes units qskip .. qcap - 1 of every queue only
 
 struct CsrSide;
 
@@ -149,14 +150,16 @@ __device__ __forceinline__ void panel_copy4_if(uint32_t lds_addr, const float *b
 // once that queue is empty, from the next XCD's that is not: what an XCD is short of by the estimate's error the
 // others make up.  Returns -1 when every queue is empty.  qhead: eight counters, zero at launch.
 __device__ __forceinline__ int panel_take_unit(const int32_t *__restrict__ unit_queue, const int32_t *__restrict__ qstart,
-                                               int32_t *__restrict__ qhead) {
+                                               int32_t *__restrict__ qhead, int32_t qcap) {
   __shared__ int taken;
   if (threadIdx.x == 0) {
     const int xcd = (int)__builtin_amdgcn_s_getreg((3 << 11) | 20) & 7;  // hardware register XCC_ID, bits 0..3
     int unit = -1;
     for (int k = 0; k < 8 && unit < 0; ++k) {
       const int q = (xcd + k) & 7;
-      const int first = qstart[q], count = qstart[q + 1] - first;
+      const int first = qstart[q];
+      int count = qstart[q + 1] - first;
+      if (qcap > 0 && count > qcap) count = qcap;  // measuring aid (spmm_panel_qcap): only the queue's first units
       if (count <= 0) continue;
       const int pos = atomicAdd(&qhead[q], 1);
       if (pos < count) unit = unit_queue[first + pos];
@@ -173,13 +176,13 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_panel_kernel(
     int32_t *__restrict__ qhead, const int32_t *__restrict__ unit_block,
     const int32_t *__restrict__ hdr, const uint2 *__restrict__ ent, const float *__restrict__ B, int64_t ldb,
     float *__restrict__ P, int32_t f, const int32_t *__restrict__ unit_row0, const int32_t *__restrict__ rank_row,
-    float *__restrict__ C, int64_t ldc, int32_t rows, float beta) {
+    float *__restrict__ C, int64_t ldc, int32_t rows, float beta, int32_t qcap) {
   extern __shared__ __align__(16) char panel_lds[];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   // One workgroup per compute unit, each taking units until the queues are empty (no workgroup waits for another).
   for (;;) {
-  const int unit = panel_take_unit(unit_order, unit_qstart, qhead);
+  const int unit = panel_take_unit(unit_order, unit_qstart, qhead, qcap);
   if (unit < 0) return;
   const int t0 = unit_tile[unit], t1 = unit_tile[unit + 1];
   const int npair = f >> 1;

@@ -62,6 +62,7 @@ static bool panel_width_ok(int32_t f);
 static bool want_tile(const CsrSide &s, int32_t f, bool after_panel) {
   const int t = g_tune_tile.load(std::memory_order_relaxed);
   if (t < 0 || s.rows == 0 || s.nnz == 0 || s.is_rest || f < 1) return false;
+  if (t == 2) return false;  // 2: the panel plan, its staged tiles through spmm_tile_kernel
   if (t > 0) return !after_panel;
   if (s.nnz / s.rows < 8 || (double)s.nnz * f < 8e8) return false;
   const bool panel_first = panel_width_ok(f) && f > 316 && g_tune_panel.load(std::memory_order_relaxed) >= 0 &&
@@ -879,15 +880,17 @@ static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_
     CG_TRY(panel_lds_attr(spmm_panel_kernel<CH>, attr_set, dev, lds_max, lds));                                        \
     spmm_panel_kernel<CH><<<(unsigned)(pp.nunits < cus ? pp.nunits : cus), kPanelThreads, lds, stream>>>(pp.unit_tile, pp.unit_order, pp.unit_qstart, qhead, pp.unit_block, \
                                                                                pp.hdr, pp.ent, B, ldb, P, f, pp.unit_row0, \
-                                                                               pp.rank_row, C_direct, ldc, rows, beta); \
+                                                                               pp.rank_row, C_direct, ldc, rows, beta, \
+                                                                               g_tune_panel_qcap.load(std::memory_order_relaxed)); \
   } break;
     const bool legacy = pp.padded && pp.prows == kPanelRows && pp.tcols == kPanelCols && panel_width_ok(f) &&
-                        g_tune_tile.load(std::memory_order_relaxed) <= 0;
+                        g_tune_tile.load(std::memory_order_relaxed) != 2;
     if (pp.nunits > 0 && !legacy) {
       CG_TRY(fill_u32((uint32_t *)qhead, kXcdQueues, 0u, stream));
       CG_TRY(launch_tile(pp, B, ldb, f, P, qhead, C_direct, ldc, rows, beta, dev, cus, stream));
     } else if (pp.nunits > 0) {
-      CG_TRY(fill_u32((uint32_t *)qhead, kXcdQueues, 0u, stream));
+      const int qskip = g_tune_panel_qskip.load(std::memory_order_relaxed);
+      CG_TRY(fill_u32((uint32_t *)qhead, kXcdQueues, (uint32_t)(qskip > 0 ? qskip : 0), stream));
       switch (chunks) {
         CG_PANEL(3)
         CG_PANEL(4)

@@ -1,6 +1,7 @@
 """Stand-alone measurements of the sparse kernels on one MI355X.
 
-    python -m cagnet_amd.microbench spmm   [--graph rmat20|reddit|amazon] [--widths 16,64,128,602]
+    python -m cagnet_amd.microbench spmm   [--graph rmat20|reddit|amazon] [--widths 16,64,128,602] [--forward-only]
+                                           [--aligned-rows] [--tune KEY=VALUE ...]
     python -m cagnet_amd.microbench grid2d [--grid 4] [--row 1]
     python -m cagnet_amd.microbench prep   [--graph reddit]
 
@@ -88,11 +89,16 @@ def run_spmm(args) -> None:
                       "coo2csr_sorted_ms": round(t_sorted, 3), "coo2csr_plus_transpose_ms": round(t_with_t, 3),
                       "coo2csr_unsorted_radix_ms": round(t_unsorted, 3), "max_degree": A.info()["max_row_degree"]}),
           flush=True)
+    from ._lib import check, lib
+    for item in args.tune:  # tuning keys of cg_tune_set for the products below (measuring runs)
+        key, value = item.split("=")
+        check(lib.cg_tune_set(key.encode(), int(value)), "cg_tune_set")
     for f in args.widths:
-        B = torch.randn(n, f, device=dev)
+        ld = (f + 31) // 32 * 32 if args.aligned_rows else f  # rows of B a whole number of 128-byte lines apart
+        B = torch.randn(n, ld, device=dev)[:, :f]
         C = torch.empty(n, f, device=dev)
         alg = 8 * nnz + 4 * (n + 1) + 4 * n * f + 4 * n * f
-        for name, tr in (("A@H", False), ("A^T@G", True)):
+        for name, tr in ((("A@H", False),) if args.forward_only else (("A@H", False), ("A^T@G", True))):
             ms = _time(lambda: A.spmm(B, out=C, beta=0.0, transpose=tr), args.reps)
             print(json.dumps({"what": "spmm", "graph": args.graph, "product": name, "f": f, "ms": round(ms, 4),
                               "gflops": round(2.0 * nnz * f / ms / 1e6, 1), "algorithmic_gbs": round(alg / ms / 1e6, 1),
@@ -144,15 +150,22 @@ def run_grid2d(args) -> None:
         for k in range(q):
             blocks[k].spmm(H[k], out=z, beta=0.0 if k == 0 else 1.0)
 
-    ms_stage = _time(stages, args.reps)
+    def fused():  # the library's stage loop: one product of the blocks side by side with the stacked operands
+        gcn.broad_func(rows, blocks, x.detach(), r, q, g1.forward, out=z)
+
+    ms_stage = float("nan") if args.stages_only and not args.per_stage else _time(stages, args.reps)
+    ms_fused = float("nan") if args.stages_only and args.per_stage else _time(fused, args.reps)
     flops = 2.0 * sum(nnzs) * feats
     alg = sum(8 * nz + 4 * (rows + 1) + 4 * (b[k + 1] - b[k]) * feats + 4 * rows * feats * (1 if k == 0 else 2)
               for k, nz in enumerate(nnzs))
+    alg_fused = 8 * sum(nnzs) + 4 * (rows + 1) + 4 * n * feats + 4 * rows * feats
     print(json.dumps({"what": "grid2d rank share", "grid": f"{q}x{q}", "process_row": r, "rows": rows, "block_nnz": nnzs,
                       "fwd_bwd_both_layers_ms": None if args.stages_only else round(ms, 3),
-                      "stage_loop_f602_ms": round(ms_stage, 3), "stage_loops_run": args.reps + 1,
-                      "stage_loop_gflops": round(flops / ms_stage / 1e6, 1),
-                      "stage_loop_algorithmic_gbs": round(alg / ms_stage / 1e6, 1)}), flush=True)
+                      "stage_loop_f602_ms": round(ms_fused, 3), "stage_loop_f602_one_product_per_stage_ms": round(ms_stage, 3),
+                      "stage_loops_run": args.reps + 1,
+                      "stage_loop_gflops": round(flops / ms_fused / 1e6, 1),
+                      "stage_loop_algorithmic_gbs": round(alg_fused / ms_fused / 1e6, 1),
+                      "one_product_per_stage_algorithmic_gbs": round(alg / ms_stage / 1e6, 1)}), flush=True)
 
 
 def run_prep(args) -> None:
@@ -198,12 +211,18 @@ def main() -> int:
     s.add_argument("--graph", default="rmat20", choices=sorted(GRAPHS))
     s.add_argument("--widths", default="16,64,128,602", type=lambda t: [int(v) for v in t.split(",")])
     s.add_argument("--reps", type=int, default=5)
+    s.add_argument("--forward-only", action="store_true", help="A @ H only")
+    s.add_argument("--aligned-rows", action="store_true", help="rows of the dense operand a multiple of 128 bytes apart")
+    s.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
+                   help="a tuning key of cg_tune_set for the products (repeatable), e.g. spmm_panel_qcap=128")
     g = sub.add_parser("grid2d")
     g.add_argument("--grid", type=int, default=4)
     g.add_argument("--row", type=int, default=1)
     g.add_argument("--reps", type=int, default=5)
     g.add_argument("--stages-only", action="store_true",
                    help="run the stage loop only (reps + 1 times): what a counter run of the stage loop profiles")
+    g.add_argument("--per-stage", action="store_true",
+                   help="with --stages-only: the loop as one product per stage instead of the fused one")
     pr = sub.add_parser("prep")
     pr.add_argument("--graph", default="reddit", choices=sorted(GRAPHS))
     pr.add_argument("--reps", type=int, default=3)

@@ -87,3 +87,15 @@ def test_stage_schedule_15d_covers_every_block_once(size, c):
         assert sorted(seen) == list(range(size // c))
     with pytest.raises(ValueError):
         gcn.stage_schedule_15d(0, 6, 4)
+
+
+def test_tile_kernels_keep_their_accumulators_in_registers():
+    """spmm_tile_kernel holds 80 accumulators in the physical registers v48..v127 and names them as tied operands of
+    its inline-asm statements; the scheme stands only while the register allocator neither spills nor needs scratch
+    in any instantiation (a spill around the asm statements would move the accumulators through memory)."""
+    from cagnet_amd import build
+    res = build.kernel_resources("spmm.hip", "spmm_tile_kernel")
+    assert len(res) >= 6, sorted(res)
+    for name, r in res.items():
+        assert r["vgpr_count"] == 128, (name, r)
+        assert r["vgpr_spill_count"] == 0 and r["private_segment_fixed_size"] == 0, (name, r)
