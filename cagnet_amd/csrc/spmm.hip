@@ -380,7 +380,10 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
   // Panel plan: the entries of dense (row panel, column block) tiles are multiplied out of LDS into
   // partial rows; the row-wise kernels then run over the other entries and add those rows in.
   if (!epi && allow_panel && f <= cap && want_panel(s, f)) {
-    const PanelParams par = panel_params();
+    PanelParams par = panel_params();
+    // The staged tiles go through spmm_tile_kernel, which takes the records as they are; the older spmm_panel_kernel
+    // (records of a run padded to pairs) serves operands that kernel cannot read and the tuning value.
+    par.padded = g_tune_panel_legacy.load(std::memory_order_relaxed) > 0 || !tile_operands_ok(par.prows, par.tcols, B, ldb, f, s.cols);
     const bool may_decline = g_tune_panel.load(std::memory_order_relaxed) == 0;
     PanelPlan &pp = s.panel;
     if (!pp.valid || !par.same(pp) || (pp.declined && !may_decline && !pp.failed)) {
@@ -920,6 +923,7 @@ int cg_tune_set(const char *key, int value) {
   else if (!strcmp(key, "spmm_panel_dwg")) cg::g_tune_panel_dwg.store(value);
   else if (!strcmp(key, "spmm_panel_share")) cg::g_tune_panel_share.store(value);
   else if (!strcmp(key, "spmm_tile")) cg::g_tune_tile.store(value);
+  else if (!strcmp(key, "spmm_panel_legacy")) cg::g_tune_panel_legacy.store(value);
   else if (!strcmp(key, "spmm_strict_nonfinite")) cg::g_tune_strict.store(value);
   else if (!strcmp(key, "spmm_panel_qskip")) cg::g_tune_panel_qskip.store(value);
   else if (!strcmp(key, "spmm_panel_qcap")) cg::g_tune_panel_qcap.store(value);

@@ -62,7 +62,6 @@ static bool panel_width_ok(int32_t f);
 static bool want_tile(const CsrSide &s, int32_t f, bool after_panel) {
   const int t = g_tune_tile.load(std::memory_order_relaxed);
   if (t < 0 || s.rows == 0 || s.nnz == 0 || s.is_rest || f < 1) return false;
-  if (t == 2) return false;  // 2: the panel plan, its staged tiles through spmm_tile_kernel
   if (t > 0) return !after_panel;
   if (s.nnz / s.rows < 8 || (double)s.nnz * f < 8e8) return false;
   const bool panel_first = panel_width_ok(f) && f > 316 && g_tune_panel.load(std::memory_order_relaxed) >= 0 &&
@@ -352,7 +351,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     if (!padded) {
       if (covered > 0x7fffffffLL) CG_FAIL(CG_ERR_OVERFLOW, "panel plan: records exceed the int32 range");
       pp.nrec = covered;
-      CG_TRY(dev_alloc((void **)&pp.ent, (size_t)(covered > 0 ? covered : 1) * 8));
+      CG_TRY(dev_alloc((void **)&pp.ent, (size_t)(covered + kWave) * 8));  // (the tile kernels load 64 records from any start)
       if (covered > 0) CG_HIP(hipMemcpyAsync(pp.ent, ent_raw, (size_t)covered * 8, hipMemcpyDeviceToDevice, stream));
     } else {
       uint32_t *start = nullptr, *runs_before = nullptr, *run_first = nullptr, *padf = nullptr, *shift = nullptr;
@@ -375,7 +374,7 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
       CG_HIP(hipStreamSynchronize(stream));
       if (covered + (int64_t)npad > 0x7fffffffLL) CG_FAIL(CG_ERR_OVERFLOW, "panel plan: records exceed the int32 range");
       pp.nrec = covered + npad;
-      CG_TRY(dev_alloc((void **)&pp.ent, (size_t)pp.nrec * 8));
+      CG_TRY(dev_alloc((void **)&pp.ent, (size_t)(pp.nrec + kWave) * 8));
       if (covered > 0) {
         panel_pad_write_kernel<<<gc, kSpmmThreads, 0, stream>>>(ent_raw, padf, shift, covered, pp.ent);
         CG_LAUNCH_CHECK();
@@ -883,8 +882,7 @@ static int launch_panel(const PanelPlan &pp, const float *B, int64_t ldb, int32_
                                                                                pp.rank_row, C_direct, ldc, rows, beta, \
                                                                                g_tune_panel_qcap.load(std::memory_order_relaxed)); \
   } break;
-    const bool legacy = pp.padded && pp.prows == kPanelRows && pp.tcols == kPanelCols && panel_width_ok(f) &&
-                        g_tune_tile.load(std::memory_order_relaxed) != 2;
+    const bool legacy = pp.padded && pp.prows == kPanelRows && pp.tcols == kPanelCols && panel_width_ok(f);
     if (pp.nunits > 0 && !legacy) {
       CG_TRY(fill_u32((uint32_t *)qhead, kXcdQueues, 0u, stream));
       CG_TRY(launch_tile(pp, B, ldb, f, P, qhead, C_direct, ldc, rows, beta, dev, cus, stream));

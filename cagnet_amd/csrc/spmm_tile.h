@@ -299,6 +299,48 @@ __device__ __forceinline__ float tile_acc_get(const TileAcc &acc, int e) {
   return e < 32 ? acc.a0[e] : e < 64 ? acc.a1[e - 32] : acc.a2[e - 64];
 }
 
+// A row of a wide slice, global -> LDS, in PPR pieces of 64 x 16 bytes from one wave-uniform base: M0 is set once and the
+// pieces differ in the instruction's immediate offset, which moves the global and the LDS address alike.  The last piece
+// runs under `mask` (the lanes that start inside the row), the others with every lane.
+template <int PPR>
+__device__ __forceinline__ void tile_copy_row(uint32_t lds_addr, const float *base, uint32_t lane16, uint64_t mask) {
+  static_assert(PPR >= 1 && PPR <= 3, "pieces of a row");
+  uint64_t saved;
+  if constexpr (PPR == 3)
+    asm volatile(
+        "s_mov_b32 m0, %1\n\t"
+        "s_mov_b64 %0, exec\n\t"
+        "global_load_lds_dwordx4 %2, %3\n\t"
+        "global_load_lds_dwordx4 %2, %3 offset:1024\n\t"
+        "s_mov_b64 exec, %4\n\t"
+        "global_load_lds_dwordx4 %2, %3 offset:2048\n\t"
+        "s_mov_b64 exec, %0"
+        : "=&s"(saved)
+        : "s"(lds_addr), "v"(lane16), "s"(base), "s"(mask)
+        : "m0", "memory");
+  else if constexpr (PPR == 2)
+    asm volatile(
+        "s_mov_b32 m0, %1\n\t"
+        "s_mov_b64 %0, exec\n\t"
+        "global_load_lds_dwordx4 %2, %3\n\t"
+        "s_mov_b64 exec, %4\n\t"
+        "global_load_lds_dwordx4 %2, %3 offset:1024\n\t"
+        "s_mov_b64 exec, %0"
+        : "=&s"(saved)
+        : "s"(lds_addr), "v"(lane16), "s"(base), "s"(mask)
+        : "m0", "memory");
+  else
+    asm volatile(
+        "s_mov_b32 m0, %1\n\t"
+        "s_mov_b64 %0, exec\n\t"
+        "s_mov_b64 exec, %4\n\t"
+        "global_load_lds_dwordx4 %2, %3\n\t"
+        "s_mov_b64 exec, %0"
+        : "=&s"(saved)
+        : "s"(lds_addr), "v"(lane16), "s"(base), "s"(mask)
+        : "m0", "memory");
+}
+
 struct TileArgs {
   const int32_t *unit_tile, *unit_order, *unit_qstart;
   int32_t *qhead;
@@ -406,6 +448,37 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
         if (++st_r < TCW) stage_row(hrows, st_r);
       }
     };
+    // The usual case: every row of the slice is as long as the slice's width says (all but the last row of B in a last
+    // slice that does not end on a 16-byte piece) and long enough to fill all but the last of its PPR pieces.
+    constexpr int PPR = NR == 10 ? 3 : NR >= 5 ? 2 : 1;
+    const bool whole_rows = NR >= 4 && lim > (uint32_t)(PPR - 1) * 1024u;
+    const uint32_t last_lanes = (lim - (uint32_t)(PPR - 1) * 1024u + 15u) >> 4;  // lanes of the last piece that start inside the row
+    const uint64_t last_mask = last_lanes >= 64u ? ~0ull : (1ull << (last_lanes & 63u)) - 1ull;
+    auto stage_wide = [&](int hrows, uint32_t dst_wave) {  // all rows of a tile
+      if (whole_rows && !tail) {
+#pragma unroll
+        for (int r = 0; r < TCW; ++r) {
+          const uint32_t ridx = (uint32_t)__builtin_amdgcn_readlane(hrows, r);
+          tile_copy_row<PPR>(dst_wave + (uint32_t)(r * rs), Bs + (uint64_t)ridx * ldb32, lane16, last_mask);
+        }
+      } else if (whole_rows) {
+#pragma unroll
+        for (int r = 0; r < TCW; ++r) {
+          const int ridx = __builtin_amdgcn_readlane(hrows, r);
+          const float *base = Bs + (uint64_t)(uint32_t)ridx * ldb32;
+          if (tail && ridx == a.m - 1) {  // the short row: piece by piece, its last piece is left to stage_tail
+            for (int j = 0; j < ppr; ++j)
+              panel_copy16_if(dst_wave + (uint32_t)(r * rs) + (uint32_t)j * (kWave * 16u), base, lane16 + (uint32_t)j * (kWave * 16u),
+                              lim & ~15u);
+          } else {
+            tile_copy_row<PPR>(dst_wave + (uint32_t)(r * rs), base, lane16, last_mask);
+          }
+        }
+      } else {
+        stage_begin(hrows);
+        for (int pc = 0; pc < npieces; ++pc) stage_next(hrows, dst_wave);
+      }
+    };
     // Narrower slices (NR < 4): a copy instruction covers several rows of B, so every lane has an offset of its own
     // (32 bits from the slice's base: the launch makes sure that B fits).  A staged row takes LROW bytes, and piece
     // q = pc * 64 + lane of the wave's staging area is row q / (LROW / 16), position q % (LROW / 16).  Nothing is
@@ -446,11 +519,8 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
             Bs[(int64_t)(a.m - 1) * a.ldb + clast * 4u + lane];
     };
     auto hdr_load = [&](int t) { return hdr[((int64_t)t * kPanelWaves + wave) * HS + (lane < HS ? lane : HS - 1)]; };
-    auto rec_load = [&](int first, int b0, int b1) {
-      int idx = first + lane;
-      idx = idx < b1 ? idx : (b1 > b0 ? b1 - 1 : 0);
-      return ent[idx];
-    };
+    // 64 records from `first` on, one per lane (the plan keeps 64 records of room behind the last one)
+    auto rec_load = [&](int first, int, int) { return ent[(uint32_t)(first + lane)]; };
     const int area = TCW * rs;  // bytes of a wave's staging area in a buffer
     char *const wave_area = panel_lds + wave * area;
     const uint32_t wave_area32 = (uint32_t)(uintptr_t)wave_area;
@@ -461,8 +531,7 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
       const int h0 = hdr_load(t0);
       hn = hdr_load(t0 + 1 < t1 ? t0 + 1 : t0);
       if constexpr (NR >= 4) {
-        stage_begin(h0);
-        for (int pc = 0; pc < npieces; ++pc) stage_next(h0, wave_area32);
+        stage_wide(h0, wave_area32);
       } else {
         stage_narrow(h0, wave_area32);
       }
@@ -483,12 +552,11 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
       const int hn2 = hdr_load(t + 2 < t1 ? t + 2 : t1 - 1);
       const uint2 recn = rec_load(e0n, e0n, e1n);
       const uint32_t dst32 = wave_area32 + (uint32_t)((buf ^ 1) * bufsz);
-      int pc = 0;  // the next tile's copies go out one at a time between the records (the last tile stages itself once more)
+      // the next tile's copies (the last tile stages itself once more)
       if constexpr (NR >= 4) {
-        stage_begin(hn);
+        stage_wide(hn, dst32);
       } else {
         stage_narrow(hn, dst32);
-        pc = npieces;
       }
 
       // cnt records in the lanes of r.  K records at a time: their rows of B are read from LDS, then one stretch of
@@ -526,10 +594,6 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
           }
           tile_window<NR, K>(acc, pk, v, b);
           __builtin_amdgcn_sched_barrier(0);  // the next K records' reads stay behind this stretch (registers)
-          if (NR >= 4 && pc < npieces) {
-            stage_next(hn, dst32);
-            ++pc;
-          }
         };
         int i = 0;
         for (; i + K <= cnt; i += K) step(i);
@@ -550,8 +614,6 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
         process(cur, left > kWave ? kWave : left);
         cur = nxt;
       }
-      if constexpr (NR >= 4)
-        for (; pc < npieces; ++pc) stage_next(hn, dst32);
       if constexpr (NR >= 4) stage_tail(hn, wave_area + (buf ^ 1) * bufsz);
       rec = recn;
       e0 = e0n;
