@@ -66,23 +66,29 @@ def spmm_alg_bytes(nnz: int, n: int, m: int, f: int, reads_c: bool) -> int:
 
 
 def load_traffic() -> dict:
-    """profiles/spmm_traffic.txt: `workload f kernels read_bytes write_bytes` per line (kernels joined by +),
-    HBM-side bytes of one product from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, already scaled."""
+    """profiles/spmm_traffic.txt: `workload f kernels read_bytes write_bytes plan commit` per line (kernels joined
+    by +), HBM-side bytes of one product from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, already scaled; `plan` is
+    plan_signature() of the matrix in the recorded run, `commit` the library's commit of that run."""
     out = {}
     if not TRAFFIC_FILE.exists():
         return out
     for line in TRAFFIC_FILE.read_text().splitlines():
         line = line.split("#", 1)[0].split()
-        if len(line) == 5:
+        if len(line) == 7:
             out[(line[0], int(line[1]))] = dict(kernels=frozenset(line[2].split("+")), read=float(line[3]),
-                                               write=float(line[4]))
+                                               write=float(line[4]), plan=line[5], commit=line[6])
     return out
 
 
-def traffic_of(table: dict, workload: str, f: int, launched: set):
-    """Bytes of the recorded profile run when it launched the same kernels as this run, else None."""
+def plan_signature(A, f: int, launched: set, transpose: bool = False) -> str:
+    """What decides the traffic of a product of width f besides its kernels (ops.CsrMatrix.plan_signature)."""
+    return A.plan_signature(f, launched, transpose=transpose)
+
+
+def traffic_of(table: dict, workload: str, f: int, launched: set, plan: str = None):
+    """Bytes of the recorded profile run when it launched the same kernels on the same plan as this run, else None."""
     rec = table.get((workload, f))
-    if rec is None or rec["kernels"] != frozenset(launched):
+    if rec is None or rec["kernels"] != frozenset(launched) or (plan is not None and rec["plan"] != plan):
         return None
     return rec["read"] + rec["write"]
 
@@ -334,8 +340,10 @@ def extra_rmat20(dev, reps: int, traffic_table: dict) -> dict:
         for name, tr in (("A@H", False), ("A^T@G", True)):
             ms = median_ms(lambda: A.spmm(B, out=C, beta=0.0, transpose=tr), reps)
             launched = launched_spmm_kernels(lambda: A.spmm(B, out=C, beta=0.0, transpose=tr), f)
-            products.append(dict(product=name, f=f, kernels="+".join(sorted(launched)),
-                                 **roofline_fields(alg, 2.0 * nnz * f, ms, traffic_of(traffic_table, "rmat20", f, launched))))
+            plan = plan_signature(A, f, launched, transpose=tr)
+            products.append(dict(product=name, f=f, kernels="+".join(sorted(launched)), plan=plan,
+                                 **roofline_fields(alg, 2.0 * nnz * f, ms,
+                                                   traffic_of(traffic_table, "rmat20", f, launched, plan))))
         del B, C
     return {"workload": "R-MAT scale 20 (1,048,576 vertices, 16,777,216 directed edges), symmetrised, self-loops, "
                         "GCN-normalised; median of %d" % reps,
@@ -399,13 +407,16 @@ def extra_grid_row(prob, spec, dev, reps: int, traffic_table: dict) -> dict:
         gcn.broad_func(rows, blocks, x.detach(), r, q, g1.forward, out=z)
 
     ms_stage = median_ms(fused, reps)
-    traffic = traffic_of(traffic_table, "grid_row", feats, launched_spmm_kernels(fused, feats))
+    launched = launched_spmm_kernels(fused, feats)
+    plan = plan_signature(gcn.stacked_blocks(blocks), feats, launched)
+    traffic = traffic_of(traffic_table, "grid_row", feats, launched, plan)
     alg_per_stage = sum(spmm_alg_bytes(nz, rows, b[k + 1] - b[k], feats, reads_c=k > 0) for k, nz in enumerate(nnzs))
     alg = spmm_alg_bytes(sum(nnzs), rows, prob.n, feats, reads_c=False)
     return {"workload": "last process row of the 4 x 4 grid on the Reddit-shaped graph, four stages resident in HBM; "
                         "median of %d" % reps,
             "rows": rows, "block_cols": [b[k + 1] - b[k] for k in range(q)], "block_nnz": nnzs, "bound": "hbm",
-            "stage_loop_f%d" % feats: roofline_fields(alg, 2.0 * sum(nnzs) * feats, ms_stage, traffic),
+            "stage_loop_f%d" % feats: dict(kernels="+".join(sorted(launched)), plan=plan,
+                                           **roofline_fields(alg, 2.0 * sum(nnzs) * feats, ms_stage, traffic)),
             "stage_loop_f%d_one_product_per_stage" % feats: roofline_fields(alg_per_stage, 2.0 * sum(nnzs) * feats,
                                                                             ms_per_stage, None),
             "fwd_bwd_both_layers_ms": round(ms_epoch, 4)}
@@ -426,13 +437,14 @@ def extra_amazon(dev, traffic_table: dict, steps: int) -> dict:
     parts, dom_ms = dominant_product(rec["kernels"], f_in)
     alg = spmm_alg_bytes(prob.nnz, prob.n, prob.n, f_in, reads_c=False)
     launched = {k.split("/")[0] for k in parts}
+    plan = plan_signature(blk, f_in, launched)
     out = {"workload": spec["desc"] + "; Adam, input gradient on; %d timed epochs" % steps, "n": prob.n, "nnz": prob.nnz,
            "bound": "hbm", "epoch_ms": round(rec["epoch_ms"], 3),
            "epoch_ms_default_fusion_policy": round(rec["epoch_ms_default_fusion_policy"], 3),
            "final_loss": rec["final_loss"],
-           "spmm_f%d" % f_in: dict(kernels="+".join(sorted(launched)),
+           "spmm_f%d" % f_in: dict(kernels="+".join(sorted(launched)), plan=plan,
                                    **roofline_fields(alg, 2.0 * prob.nnz * f_in, dom_ms,
-                                                     traffic_of(traffic_table, "amazon", f_in, launched))),
+                                                     traffic_of(traffic_table, "amazon", f_in, launched, plan))),
            "kernels": {k: {"launches": v["launches"], "avg_ms": round(v["avg_ms"], 5)} for k, v in rec["kernels"].items()}}
     del rec, blk, prob
     torch.cuda.empty_cache()
@@ -551,7 +563,8 @@ def main() -> int:
     alg_bytes = spmm_alg_bytes(nnz, n, n, f_in, reads_c=False)
     achieved = alg_bytes / (dom_ms * 1e-3) / 1e9
     gather_bytes = 8 * nnz + 4 * (n + 1) + 4 * nnz * f_in + 4 * n * f_in
-    traffic = traffic_of(traffic_table, args.workload, f_in, launched)
+    plan = plan_signature(blk, f_in, launched)
+    traffic = traffic_of(traffic_table, args.workload, f_in, launched, plan)
     steps = args.steps
     spmm_total_ms = sum(v["avg_ms"] * v["launches"] for k, v in kernels.items() if k.startswith("spmm")) / steps
     dense_total_ms = sum(v["avg_ms"] * v["launches"] for k, v in kernels.items() if k.startswith("dense")) / steps
@@ -601,9 +614,11 @@ def main() -> int:
             "frac": round(achieved / HBM_PEAK_GBS, 5),
             "traffic": traffic,
             "traffic_source": ("HBM-side bytes of this product from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs recorded "
-                               "in profiles/spmm_traffic.txt (a profile-run figure, not measured by this run)"
+                               "in profiles/spmm_traffic.txt (a profile-run figure, not measured by this run; the recorded "
+                               "run launched the same kernels on a plan of the same parameters and sizes)"
                                if traffic is not None else
-                               "no profile run of these kernels is recorded in profiles/spmm_traffic.txt"),
+                               "no profile run of these kernels on this plan is recorded in profiles/spmm_traffic.txt"),
+            "plan": plan,
             "algorithmic_bytes": alg_bytes,
             "avg_launch_ms": round(dom_ms, 5),
             # the same launch priced on the recorded HBM-side bytes, not a substitute for `achieved`: how

@@ -17,6 +17,7 @@ One JSON object per line.  Timing: HIP events on the current stream, median of `
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import sys
 import time
@@ -57,6 +58,28 @@ def _time(fn, reps: int) -> float:
         times.append(e0.elapsed_time(e1))
     times.sort()
     return times[len(times) // 2]
+
+
+_SPMM_KERNELS = ("spmm_panel_dense", "spmm_panel", "spmm_panel_add", "spmm_hub_hot", "spmm_rowseg", "spmm_reduce",
+                 "spmm_hub_reduce")
+
+
+def _launched(fn, f: int) -> set:
+    """Profiling names of the SpMM kernels one call of fn launches at width f."""
+    from ._lib import lib
+
+    torch.cuda.synchronize()
+    lib.cg_prof_enable(1)
+    fn()
+    torch.cuda.synchronize()
+    lib.cg_prof_enable(0)
+    out = set()
+    for k in _SPMM_KERNELS:
+        t, c = ctypes.c_double(0.0), ctypes.c_int64(0)
+        lib.cg_prof_read(f"{k}/f={f}".encode(), ctypes.byref(t), ctypes.byref(c))
+        if c.value:
+            out.add(k)
+    return out
 
 
 def run_spmm(args) -> None:
@@ -100,7 +123,9 @@ def run_spmm(args) -> None:
         alg = 8 * nnz + 4 * (n + 1) + 4 * n * f + 4 * n * f
         for name, tr in ((("A@H", False),) if args.forward_only else (("A@H", False), ("A^T@G", True))):
             ms = _time(lambda: A.spmm(B, out=C, beta=0.0, transpose=tr), args.reps)
+            launched = _launched(lambda: A.spmm(B, out=C, beta=0.0, transpose=tr), f)
             print(json.dumps({"what": "spmm", "graph": args.graph, "product": name, "f": f, "ms": round(ms, 4),
+                              "kernels": "+".join(sorted(launched)), "plan": A.plan_signature(f, launched, transpose=tr),
                               "gflops": round(2.0 * nnz * f / ms / 1e6, 1), "algorithmic_gbs": round(alg / ms / 1e6, 1),
                               "pct_of_8TBs": round(alg / ms / 1e6 / 80.0, 2)}), flush=True)
         del B, C
@@ -155,6 +180,8 @@ def run_grid2d(args) -> None:
 
     ms_stage = float("nan") if args.stages_only and not args.per_stage else _time(stages, args.reps)
     ms_fused = float("nan") if args.stages_only and args.per_stage else _time(fused, args.reps)
+    launched = set() if ms_fused != ms_fused else _launched(fused, feats)
+    plan = gcn.stacked_blocks(blocks).plan_signature(feats, launched) if launched else None
     flops = 2.0 * sum(nnzs) * feats
     alg = sum(8 * nz + 4 * (rows + 1) + 4 * (b[k + 1] - b[k]) * feats + 4 * rows * feats * (1 if k == 0 else 2)
               for k, nz in enumerate(nnzs))
@@ -162,7 +189,7 @@ def run_grid2d(args) -> None:
     print(json.dumps({"what": "grid2d rank share", "grid": f"{q}x{q}", "process_row": r, "rows": rows, "block_nnz": nnzs,
                       "fwd_bwd_both_layers_ms": None if args.stages_only else round(ms, 3),
                       "stage_loop_f602_ms": round(ms_fused, 3), "stage_loop_f602_one_product_per_stage_ms": round(ms_stage, 3),
-                      "stage_loops_run": args.reps + 1,
+                      "stage_loops_run": args.reps + 1, "kernels": "+".join(sorted(launched)), "plan": plan,
                       "stage_loop_gflops": round(flops / ms_fused / 1e6, 1),
                       "stage_loop_algorithmic_gbs": round(alg_fused / ms_fused / 1e6, 1),
                       "one_product_per_stage_algorithmic_gbs": round(alg / ms_stage / 1e6, 1)}), flush=True)

@@ -374,15 +374,35 @@ class CsrMatrix:
                 # column-popularity plan the last wide product looked up: tiers, -1 declined, 0 none
                 "plan_tiers": buf[6], "plan_tiers_transpose": buf[7]}
 
-    def panel_info(self, transpose: bool = False, narrow: bool = False) -> dict:
-        """Panel plan the last wide (narrow=True: narrow, f <= 64) product of A (transpose=True: of A^T) looked up:
+    def panel_info(self, transpose: bool = False, narrow: bool = False, tile: int = 0) -> dict:
+        """Panel plan the last wide (narrow=True: narrow, f <= 64) product of A (transpose=True: of A^T) looked up, or
+        with tile = 1, 2, 3 the tile plan with panels of 256, 512, 1024 rows:
         state 1 in use / -1 declined / 0 none considered; entries multiplied out of LDS, in dense tiles on the matrix
         cores, left to the row-wise kernels; tile and unit counts; the thresholds the plan was built with."""
         buf = (c_int64 * 12)()
-        check(lib.cg_csr_panel_info(self._handle, int(transpose) | (2 if narrow else 0), buf), "cg_csr_panel_info")
+        which = int(transpose) | (2 if narrow else 0) | ((int(tile) & 3) << 2)
+        check(lib.cg_csr_panel_info(self._handle, which, buf), "cg_csr_panel_info")
         return {"state": buf[0], "staged_entries": buf[1], "staged_tiles": buf[2], "staged_units": buf[3],
                 "split_panels": buf[4], "rest_entries": buf[5], "tile_min_entries": buf[6], "column_ranks": buf[7],
                 "dense_entries": buf[8], "dense_tiles": buf[9], "dense_units": buf[10], "dense_min_entries": buf[11]}
+
+    def plan_signature(self, f: int, launched, transpose: bool = False) -> str:
+        """What decides the memory traffic of a product of width f besides the kernels it launched (`launched`: their
+        profiling names): the parameters and sizes of the plan it ran on - the tile plan of the width's panel height,
+        else the panel plan, else the narrow plan's dense tiles - and the tiers of a hub plan."""
+        parts = []
+        if "spmm_panel" in launched or "spmm_panel_dense" in launched:
+            for name, kw in (("tile", dict(tile=1 if f > 128 else 2 if f > 64 else 3)), ("panel", dict()),
+                             ("narrow", dict(narrow=True))):
+                i = self.panel_info(transpose=transpose, **kw)
+                if i["state"] == 1:
+                    parts.append("%s:e%d.c%d.d%d.t%d.u%d.dt%d.r%d" % (
+                        name, i["tile_min_entries"], i["column_ranks"], i["dense_min_entries"], i["staged_tiles"],
+                        i["staged_units"], i["dense_tiles"], i["rest_entries"]))
+                    break
+        if "spmm_hub_hot" in launched:
+            parts.append("hub:%d" % self.info()["plan_tiers_transpose" if transpose else "plan_tiers"])
+        return ",".join(parts) if parts else "rowwise"
 
     def arrays(self, transpose: bool = False):
         """(rowptr, colind, values) of A, or of A^T, as tensors that alias the handle's memory."""

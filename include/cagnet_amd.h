@@ -208,7 +208,8 @@ int cg_csr_spmm_xw(cg_csr_t *h, int transpose, const float *d_B, int64_t ldb, co
  *                tiers in use, -1 when the column counts declined it, 0 when none was considered } */
 int cg_csr_info(const cg_csr_t *h, int64_t info[8]);
 /* Panel plan a wide product of A (bit 0 of `transpose` set: of A^T) last looked up; with bit 1 of `transpose` set the
- * plan of the narrow products (f <= 64), which has dense tiles only: info[0..11] =
+ * plan of the narrow products (f <= 64), which has dense tiles only; with bits 2..3 holding 1, 2 or 3 the tile plan
+ * with panels of 256, 512 or 1024 rows: info[0..11] =
  * { 1 in use / -1 declined (the tiles hold too few of the entries) / 0 none considered yet,
  *   entries multiplied out of LDS by the vector ALUs, their (active) tiles, their units (workgroups),
  *   row panels with several units of either kind, entries left to the row-wise kernels, entries a tile
@@ -377,6 +378,22 @@ int cg_prof_enable(int on);
  *                     hold at least 64 entries on average, the product has at least 1e9 multiply-adds and the dense
  *                     tiles hold at least a quarter of the entries
  *   "spmm_panel_narrow_dmin" entries from which a tile is dense for narrow products (0: 512)
+ *   "spmm_panel_legacy" 1: the staged tiles of the panel plan go through the older kernel, which keeps a panel's rows
+ *                     in named registers and takes the records of a (tile, wave, row) run in pairs, padded; 0: through
+ *                     the tile kernel (accumulators addressed through the register index, records as they are).  A B
+ *                     that is not 8-byte aligned or has an odd leading dimension goes to the older kernel whatever
+ *                     this says: the tile kernel's copies need 8-byte aligned rows
+ *   "spmm_tile"       tile plans (every entry multiplied out of LDS by the tile kernel; panels of 256 rows and
+ *                     column slices of up to 316 columns for widths above 128, 512 rows for 65..128, 1024 rows up
+ *                     to 64): -1 never, 1 always, 0 by width and matrix: widths from 65 on except the even widths
+ *                     318..636 where the panel plan is in use, and 48..64 on matrices of under 64 entries per row,
+ *                     on products of at least 8e8 multiply-adds with at least 8 entries per row
+ *   "spmm_strict_nonfinite" 1: no plan that multiplies stored zeros (the dense tiles of the panel plans) or padding
+ *                     records: a row of B with an infinity or a NaN then reaches exactly the rows of C that have an
+ *                     entry in that column, as in a product entry by entry (cusparseSpMM in the reference)
+ *   "spmm_panel_qskip", "spmm_panel_qcap" measuring aids for the older staged-tile kernel ("spmm_panel_legacy" 1):
+ *                     a launch takes only the units from position qskip on, or before position qcap, of each of its
+ *                     eight unit queues; the product is then incomplete
  *   "dense_mfma"      -1: dense products on the vector ALU tile kernel only
  *   "coo_cache_blocks" blocks cg_spmm_coo_cached keeps (0: 8; negative: none)
  *   "coo_cache_mib"   device memory those blocks may hold together, in MiB (0: 32768); a block counts as four

@@ -862,6 +862,38 @@ def test_spmm_panel_plan_matches_oracle(cuda, tune, f, emin, unit):
     assert spmm_error(plain, row, col, val, n, n, B) <= REL_TOL
 
 
+@pytest.mark.parametrize("f", [258, 384, 512, 514, 602, 636])
+def test_spmm_panel_staged_tiles_through_either_kernel(cuda, tune, f):
+    """The staged tiles of the panel plan go through the tile kernel (records as they are) or, with spmm_panel_legacy or
+    for a B whose rows are not 8-byte aligned, through the older kernel on padded records: both against the fp64 oracle,
+    each bit-identical on repeats, with accumulation into C."""
+    from cagnet_amd import ops
+    row, col, val, n = small_graph(12, 140000, seed=5 * f)
+    A = ops.CsrMatrix(_i32(row, cuda), _i32(col, cuda), val.to(cuda), n, n)
+    B = torch.randn(n, f, generator=torch.Generator().manual_seed(f))
+    C0 = torch.randn(n, f, generator=torch.Generator().manual_seed(f + 1))
+    tune("spmm_panel", 1)
+    tune("spmm_panel_dmin", 200)
+    results = []
+    for legacy in (0, 1, 0):
+        tune("spmm_panel_legacy", legacy)
+        got = A.spmm(B.to(cuda))
+        info = _panel_info(A)
+        assert info["state"] == 1 and info["covered"] > 0 and info["dense_tiles"] > 0 and info["rest"] == 0
+        assert spmm_error(got, row, col, val, n, n, B) <= REL_TOL
+        assert torch.equal(got, A.spmm(B.to(cuda)))
+        C = C0.to(cuda).clone()
+        A.spmm(B.to(cuda), out=C, beta=1.0)
+        assert spmm_error(C, row, col, val, n, n, B, C0) <= REL_TOL
+        results.append(got)
+    assert torch.equal(results[0], results[2])                       # the plan is rebuilt the same way
+    tune("spmm_panel_legacy", 0)
+    wide = torch.zeros(n, f + 1, device=cuda)                         # rows 4 bytes off an 8-byte boundary when f is even
+    wide[:, 1:] = B.to(cuda)
+    odd = A.spmm(wide[:, 1:])
+    assert spmm_error(odd, row, col, val, n, n, B) <= REL_TOL
+
+
 @pytest.mark.parametrize("f", [258, 320, 384, 448, 512, 576, 602, 636])
 @pytest.mark.parametrize("dmin,dwg", [(40, 3), (200, 0)])
 def test_spmm_panel_dense_tiles_on_matrix_cores(cuda, tune, f, dmin, dwg):
