@@ -924,6 +924,7 @@ int cg_tune_set(const char *key, int value) {
   else if (!strcmp(key, "spmm_panel_share")) cg::g_tune_panel_share.store(value);
   else if (!strcmp(key, "spmm_tile")) cg::g_tune_tile.store(value);
   else if (!strcmp(key, "spmm_panel_legacy")) cg::g_tune_panel_legacy.store(value);
+  else if (!strcmp(key, "spmm_panel_costcap")) cg::g_tune_panel_costcap.store(value);
   else if (!strcmp(key, "spmm_strict_nonfinite")) cg::g_tune_strict.store(value);
   else if (!strcmp(key, "spmm_panel_qskip")) cg::g_tune_panel_qskip.store(value);
   else if (!strcmp(key, "spmm_panel_qcap")) cg::g_tune_panel_qcap.store(value);

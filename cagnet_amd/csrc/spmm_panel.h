@@ -43,6 +43,7 @@ constexpr int kDenseTileFloats = kPanelRows * kPanelCols;
 
 static std::atomic<int> g_tune_panel{0}, g_tune_panel_emin{0}, g_tune_panel_cols{0}, g_tune_panel_unit{0};
 static std::atomic<int> g_tune_panel_dmin{0}, g_tune_panel_dwg{0}, g_tune_panel_share{0}, g_tune_tile{0}, g_tune_strict{0};
+static std::atomic<int> g_tune_panel_costcap{0};  // microseconds of modelled cost from which a unit is cut at the latest (0: 100)
 static std::atomic<int> g_tune_panel_legacy{0};  // > 0: the panel plan's staged tiles through spmm_panel_kernel (padded records)
 static std::atomic<int> g_tune_panel_qskip{0}, g_tune_panel_qcap{0};  // measuring aid: a launch takes units qskip .. qcap - 1 of every queue only
 

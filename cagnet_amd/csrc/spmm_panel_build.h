@@ -425,8 +425,8 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   // What a run of tiles costs, in microseconds: a tile with e records 1.50 + 0.0034 e + 8.7e-6 e^2 (fitted to the
   // durations of the 3744 units of the matrix with 232,965 vertices and 492 entries per row at f = 602: 3.4 % off
   // in the median; a tile costs its copies and its barrier whatever it holds, and the waves' records run the more
-  // unevenly the more of them a tile has).  Only ratios matter.  A unit is also cut when it has an eighth of a
-  // compute unit's share of the whole cost (at least 100 us), so that a small matrix still gets balanced work.
+  // unevenly the more of them a tile has).  Only ratios matter.  A unit is also cut when its cost reaches a cap
+  // (below), so that a small matrix still gets balanced work.
   // (Tiles of other shapes go to spmm_tile_kernel, whose waves take a record in about 60 cycles whatever the tile
   // holds: a fixed part per tile and a linear one.)
   const bool legacy_shape = PR == kPanelRows && TC == kPanelCols;
@@ -434,6 +434,12 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     const double e = (double)(h_base[(size_t)t + 1] - h_base[(size_t)t]);
     return legacy_shape ? 1.50 + 0.0034 * e + 8.7e-6 * e * e : 1.50 + 0.0016 * e;
   };
+  // A unit is cut at the latest when its cost reaches `cost_cap`: an eighth of a compute unit's share of the whole cost,
+  // and at least a third of it within 100 .. 200 us (300 for the tile plans' shapes).  The lower bounds keep the
+  // number of blocks of partial rows down on small matrices, which the pass that sums them pays for: a block row of
+  // a 4 x 4 grid over 232,965 vertices at f = 602 (9.4 M entries) takes 1.54 / 1.47 / 1.39 / 1.50 / 1.54 ms with units of
+  // at most 100 / 150 / 200 / 300 / 400 us; R-MAT scale 20 at f = 64, 128, 256 with 100 us 0.94 / 1.41 / 2.50 ms, with
+  // 300 us 0.87 / 1.30 / 2.40 ms.
   double cost_cap = 100.0;
   {
     int dev = 0, cus = 0;
@@ -444,6 +450,9 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
     }
     double total = 0.0;
     for (int64_t t = 0; t < ntiles; ++t) total += tile_cost(t);
+    const int tuned = g_tune_panel_costcap.load(std::memory_order_relaxed);
+    const double hi = legacy_shape ? 200.0 : 300.0;
+    cost_cap = tuned > 0 ? (double)tuned : std::min(hi, std::max(100.0, total / (3.0 * cus)));
     if (total / (8.0 * cus) > cost_cap) cost_cap = total / (8.0 * cus);
   }
   for (int64_t k = 0; k < ntiles;) {

@@ -135,6 +135,10 @@ def run_grid2d(args) -> None:
     from . import gcn, ops, synth
 
     dev = torch.device("cuda:0")
+    from ._lib import check, lib
+    for item in args.tune:
+        key, value = item.split("=")
+        check(lib.cg_tune_set(key.encode(), int(value)), "cg_tune_set")
     row, col, val, n = _graph("reddit", dev)
     q, r = args.grid, args.row
     b = synth.block_bounds_2d(n, q)
@@ -248,6 +252,8 @@ def main() -> int:
     g.add_argument("--reps", type=int, default=5)
     g.add_argument("--stages-only", action="store_true",
                    help="run the stage loop only (reps + 1 times): what a counter run of the stage loop profiles")
+    g.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
+                   help="cg_tune_set before the products (repeatable)")
     g.add_argument("--per-stage", action="store_true",
                    help="with --stages-only: the loop as one product per stage instead of the fused one")
     pr = sub.add_parser("prep")

@@ -392,8 +392,11 @@ class CsrMatrix:
         else the panel plan, else the narrow plan's dense tiles - and the tiers of a hub plan."""
         parts = []
         if "spmm_panel" in launched or "spmm_panel_dense" in launched:
-            for name, kw in (("tile", dict(tile=1 if f > 128 else 2 if f > 64 else 3)), ("panel", dict()),
-                             ("narrow", dict(narrow=True))):
+            tile = ("tile", dict(tile=1 if f > 128 else 2 if f > 64 else 3))
+            # tiles on the matrix cores: only the panel plan (wide products) and the narrow plan have them
+            order = ((("narrow", dict(narrow=True)),) if f <= 64 else (("panel", dict()),)) if "spmm_panel_dense" in launched \
+                else (tile, ("panel", dict()))
+            for name, kw in order:
                 i = self.panel_info(transpose=transpose, **kw)
                 if i["state"] == 1:
                     parts.append("%s:e%d.c%d.d%d.t%d.u%d.dt%d.r%d" % (
