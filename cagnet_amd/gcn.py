@@ -38,9 +38,17 @@ spmm_first = True
 # product order as the reference; only the summation order inside the small W product differs.
 fused_forward = True
 # ... but only where it pays: the epilogue costs a fixed f_in * f_out multiply-adds per row, the
-# saving is one write and one read of the row.  Measured: Amazon shape (16 entries per row) epoch
-# 77.7 -> 71.4 ms, Reddit shape (492 entries per row) 24.3 -> 24.5 ms.
+# saving is one write and one read of the row.  Measured against the row-wise SpMM kernels: Amazon shape
+# (16 entries per row) epoch 77.7 -> 71.4 ms, Reddit shape (492 entries per row) 24.3 -> 24.5 ms.  Where the
+# library multiplies the block through a tile plan (rows of 8 entries and more, products from 8e8 multiply-adds
+# and 65 columns on: cg_tune_set "spmm_tile"), the plain product wins - Amazon shape at f = 300: fused 39.5 ms,
+# tile plan 33.0 ms + 3.4 ms for the product with W - and the fused form is left to the smaller products.
 fused_forward_max_row_entries = 64
+
+
+def _tile_plan_expected(block: CsrMatrix, width: int) -> bool:
+    """The library's own rule for multiplying `block` at this width through a tile plan (spmm.hip: want_tile)."""
+    return width >= 65 and block.nnz >= 8 * max(block.n, 1) and float(block.nnz) * width >= 8e8
 
 
 # The stage loop reads a wide operand that the caller registered with ops.keep_aligned (the input features, say)
@@ -253,7 +261,8 @@ class GCNFunc(torch.autograd.Function):
         if spmm_first or size != 1 or weight.shape[1] >= inputs.shape[1]:  # reordering only pays when the layer narrows
             out = None
             last = am_partitions[size - 1]
-            short_rows = last.nnz <= fused_forward_max_row_entries * max(last.n, 1)
+            short_rows = (last.nnz <= fused_forward_max_row_entries * max(last.n, 1)
+                          and not _tile_plan_expected(last, inputs.shape[1]))
             if fused_forward and short_rows and weight.shape[1] <= 64 and inputs.shape[1] >= 128:
                 # stages 0 .. size-2 accumulate as usual, the last one also applies W (and ReLU)
                 z = broad_func(node_count, am_partitions[:-1], inputs, rank, size - 1, peers_fwd) if size > 1 else None

@@ -651,7 +651,12 @@ def _aligned_wanted(t: torch.Tensor) -> bool:
 
 def keep_aligned(t: torch.Tensor) -> torch.Tensor:
     """Register `t` (a dense operand that stays the same over many products, e.g. the input features) for a kept
-    copy with line-aligned rows; registering again drops a copy made earlier.  Returns `t`."""
+    copy with line-aligned rows; registering again drops a copy made earlier.  Returns `t`.
+
+    The copy is remade when `t`'s version counter, storage address, shape or strides change, i.e. after every
+    in-place write through torch or this library.  A write that bypasses the version counter (`t.data`, a view of the
+    storage taken under `torch.no_grad()` tricks, another process) is not seen: register only tensors you do not
+    write that way, or call `keep_aligned(t)` again (or `aligned_cache_clear()`) after such a write."""
     import weakref
 
     _aligned_cache[id(t)] = [weakref.ref(t), None, None, None, None]

@@ -372,6 +372,56 @@ def test_graphed_train_matches_eager_epochs(cuda, optimizer):
     assert graphed.epochs_run == warm + 5
 
 
+def test_two_graphed_trainers_over_one_matrix(cuda):
+    """Two `GraphedTrain` objects captured over the same matrix each count as a graph that names its tables: closing the
+    first must leave the second's replays intact (bit-identical to eager epochs, with plans evicted and scratch grown in
+    between), and the parked tables go only when the last one is closed."""
+    from cagnet_amd import gcn, ops
+    p = synth.make_problem(scale=11, n_edges=20000, features=128, hidden=16, classes=8, mask_fraction=0.7, seed=13,
+                           device=cuda)
+    blk = ops.CsrMatrix(p.row.int(), p.col.int(), p.val, p.n, p.n, transpose=True)
+
+    class Data:
+        y = p.y
+        train_mask = p.train_mask
+
+    def model():
+        w1, w2 = p.w1.clone().requires_grad_(True), p.w2.clone().requires_grad_(True)
+        x = p.x.clone().requires_grad_(True)
+        return x, w1, w2, torch.optim.SGD([w1, w2], lr=0.01)
+
+    xa, w1a, w2a, opta = model()
+    xb, w1b, w2b, optb = model()
+    xe, w1e, w2e, opte = model()
+    ga = gcn.GraphedTrain(xa, w1a, w2a, p.n, [blk], opta, Data, warmup=1)
+    gb = gcn.GraphedTrain(xb, w1b, w2b, p.n, [blk], optb, Data, warmup=1)
+    assert blk._graph_refs == 2
+    gcn.train(xe, w1e, w2e, p.n, [blk], opte, Data)
+    xe.grad = None
+    ga.step()
+    gb.step()
+    gcn.train(xe, w1e, w2e, p.n, [blk], opte, Data)
+    xe.grad = None
+    torch.cuda.synchronize()
+    assert torch.equal(w1a, w1e) and torch.equal(w1b, w1e)
+    ga.close()                                                           # one graph gone: the tables must stay
+    assert blk._graph_refs == 1
+    for f in (96, 200, 330):                                             # eager products at other widths: new schedules,
+        blk.spmm(torch.randn(p.n, f, device=cuda))                       # recycled tables, more scratch
+    for epoch in range(3):
+        gb.step()
+        gcn.train(xe, w1e, w2e, p.n, [blk], opte, Data)
+        xe.grad = None
+        torch.cuda.synchronize()
+        assert torch.equal(w1b, w1e) and torch.equal(w2b, w2e), f"epoch {epoch} after the first trainer was closed"
+        assert float(gb.loss) == float(gcn.train.last_loss)
+    gb.close()
+    assert blk._graph_refs == 0
+    assert blk.unpin() == 0                                              # nothing left parked
+    out = gcn.train(xe, w1e, w2e, p.n, [blk], opte, Data)               # and the matrix still works
+    assert torch.isfinite(out).all()
+
+
 def test_activations_off_is_the_plain_linear_model(cuda, monkeypatch):
     """The reference runs with its activations switched off unless asked otherwise (module global,
     gcn_distr.py:57, :284-294): GCNFunc then returns Z itself for every `func`, and backward passes the

@@ -99,3 +99,22 @@ def test_tile_kernels_keep_their_accumulators_in_registers():
     for name, r in res.items():
         assert r["vgpr_count"] == 128, (name, r)
         assert r["vgpr_spill_count"] == 0 and r["private_segment_fixed_size"] == 0, (name, r)
+
+
+def test_recorded_traffic_is_reported_only_for_the_same_kernels_on_the_same_plan():
+    """profiles/spmm_traffic.txt: every record names its kernels, its plan signature and the commit it was measured
+    at; bench.py hands a record out only to a run that launched those kernels on a plan of that signature."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench_for_test", ROOT / "bench.py")
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    table = bench.load_traffic()
+    lines = [l for l in (ROOT / "profiles" / "spmm_traffic.txt").read_text().splitlines() if l and not l.startswith("#")]
+    assert len(table) == len(lines) >= 5
+    for (workload, f), rec in table.items():
+        assert rec["read"] > 0 and rec["write"] > 0 and len(rec["commit"]) >= 7
+        assert rec["plan"] == "rowwise" or rec["plan"].split(":")[0] in ("panel", "tile", "narrow", "hub")
+        assert bench.traffic_of(table, workload, f, set(rec["kernels"]), rec["plan"]) == rec["read"] + rec["write"]
+        assert bench.traffic_of(table, workload, f, set(rec["kernels"]), rec["plan"] + "x") is None
+        assert bench.traffic_of(table, workload, f, set(rec["kernels"]) | {"spmm_hub_hot"}, rec["plan"]) is None
+    assert bench.traffic_of(table, "reddit", 600, {"spmm_panel"}, "rowwise") is None
