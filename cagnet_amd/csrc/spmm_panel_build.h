@@ -289,8 +289,10 @@ static int build_panel_once(CsrSide &s, PanelPlan &pp, int32_t emin, int32_t hot
   panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, tindex, tiles, (uint32_t)emin, (uint32_t)dmin, 1, tbase,
                                                            (int32_t)npanels, tile_panel, tile_kb);
   CG_LAUNCH_CHECK();
-  CG_TRY(dev_alloc((void **)&pp.hdr, (size_t)(ntiles > 0 ? ntiles : 1) * kPanelWaves * HS * 4));
+  // (two tiles' worth of zero headers behind the last: spmm_tile_kernel reads headers two tiles ahead without looking)
+  CG_TRY(dev_alloc((void **)&pp.hdr, (size_t)(ntiles + 2) * kPanelWaves * HS * 4));
   CG_TRY(fill_u32((uint32_t *)pp.hdr, ntiles * kPanelWaves * HS, 0xffffffffu, stream));
+  CG_TRY(fill_u32((uint32_t *)pp.hdr + ntiles * kPanelWaves * HS, 2 * kPanelWaves * HS, 0u, stream));
   if (ndtiles > 0) {
     panel_tile_tables_kernel<<<gt, kSpmmThreads, 0, stream>>>(tcount, dindex, tiles, (uint32_t)emin, (uint32_t)dmin, 2, tbase,
                                                              (int32_t)npanels, dtile_panel, nullptr);
@@ -775,7 +777,7 @@ static bool tile_operands_ok(int32_t prows, int32_t tcols, const float *B, int64
   if (((uintptr_t)B & 7u) != 0 || (ldb & 1) != 0 || ldb > 0x7fffffffLL) return false;
   if (sh.nr < 4) {
     if (f % 4 != 0) return false;
-    if ((int64_t)m * ldb * 4 >= (int64_t)1 << 32) return false;
+    if ((int64_t)m * ldb * 4 >= (int64_t)1 << 31) return false;  // (32-bit offsets that are positive as int32 too)
     if (((uintptr_t)B & 15u) != 0 || (ldb & 3) != 0) return false;  // every piece of a narrow row on a 16-byte boundary
   }
   return true;

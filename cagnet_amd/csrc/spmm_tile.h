@@ -427,6 +427,8 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
     const int bufsz = kPanelWaves * TCW * rs;  // bytes of a tile's buffer
     const uint32_t lane16 = (uint32_t)lane * 16u;
     const uint32_t ldb32 = (uint32_t)a.ldb;  // the launch refuses leading dimensions of 2^31 and more
+    const uint32_t ldb_bytes = ldb32 * 4u;
+    const bool b_small = (uint64_t)(uint32_t)a.m * ldb32 * 4u + 4096u < ((uint64_t)1 << 31);  // (offsets that are positive as int32 too)
     int st_r = 0, st_j = 0;
     const float *st_base = Bs;
     uint32_t st_lim = 0;
@@ -455,7 +457,13 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
     const uint32_t last_lanes = (lim - (uint32_t)(PPR - 1) * 1024u + 15u) >> 4;  // lanes of the last piece that start inside the row
     const uint64_t last_mask = last_lanes >= 64u ? ~0ull : (1ull << (last_lanes & 63u)) - 1ull;
     auto stage_wide = [&](int hrows, uint32_t dst_wave) {  // all rows of a tile
-      if (whole_rows && !tail) {
+      if (whole_rows && !tail && b_small) {  // every byte of B within 2 GB of its start: 32-bit offsets from one base
+#pragma unroll
+        for (int r = 0; r < TCW; ++r) {
+          const uint32_t ridx = (uint32_t)__builtin_amdgcn_readlane(hrows, r);
+          tile_copy_row<PPR>(dst_wave + (uint32_t)(r * rs), Bs, ridx * ldb_bytes + lane16, last_mask);
+        }
+      } else if (whole_rows && !tail) {
 #pragma unroll
         for (int r = 0; r < TCW; ++r) {
           const uint32_t ridx = (uint32_t)__builtin_amdgcn_readlane(hrows, r);
@@ -499,7 +507,6 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
         noff[pc] = (c < cmax ? c : cmax) * 16u;
       }
     }
-    const uint32_t ldb_bytes = ldb32 * 4u;
     auto stage_narrow = [&](int hrows, uint32_t dst_wave) {
 #pragma unroll
       for (int pc = 0; pc < NPN; ++pc) {
@@ -518,7 +525,9 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
         *reinterpret_cast<float *>(dst_wave + j * rs + clast * 16u + lane * 4) =
             Bs[(int64_t)(a.m - 1) * a.ldb + clast * 4u + lane];
     };
-    auto hdr_load = [&](int t) { return hdr[((int64_t)t * kPanelWaves + wave) * HS + (lane < HS ? lane : HS - 1)]; };
+    // the wave's header of a tile: lanes 0 .. HS - 1 (the plan keeps two tiles' worth of zero headers behind the last)
+    const int32_t *hdr_lane = hdr + ((int64_t)t0 * kPanelWaves + wave) * HS + (lane < HS ? lane : HS - 1);
+    auto hdr_load = [&](int dt) { return hdr_lane[(int64_t)dt * (kPanelWaves * HS)]; };  // dt tiles behind the current one
     // 64 records from `first` on, one per lane (the plan keeps 64 records of room behind the last one)
     auto rec_load = [&](int first, int, int) { return ent[(uint32_t)(first + lane)]; };
     const int area = TCW * rs;  // bytes of a wave's staging area in a buffer
@@ -528,8 +537,8 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
     uint2 rec = make_uint2(0u, 0u);
     int e0 = 0, e1 = 0, hn = 0;
     if (t1 > t0) {
-      const int h0 = hdr_load(t0);
-      hn = hdr_load(t0 + 1 < t1 ? t0 + 1 : t0);
+      const int h0 = hdr_load(0);
+      hn = hdr_load(1);
       if constexpr (NR >= 4) {
         stage_wide(h0, wave_area32);
       } else {
@@ -542,17 +551,18 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    uint32_t cur_off = 0u, nxt_off = (uint32_t)bufsz;  // the buffer of the tile in use, of the tile on its way
     for (int t = t0; t < t1; ++t) {
-      const int buf = (t - t0) & 1;
-      const char *lbase = panel_lds + buf * bufsz;
+      const char *lbase = panel_lds + cur_off;
       // The records of this tile and the header of the next arrived before the last barrier.  Touching them
       // here puts the compiler's wait for them ahead of the copies it cannot see.
       asm volatile("" ::"v"(rec.x), "v"(rec.y), "v"(hn));
       const int e0n = __builtin_amdgcn_readlane(hn, TCW), e1n = __builtin_amdgcn_readlane(hn, TCW + 1);
-      const int hn2 = hdr_load(t + 2 < t1 ? t + 2 : t1 - 1);
+      const int hn2 = hdr_load(2);
+      hdr_lane += kPanelWaves * HS;
       const uint2 recn = rec_load(e0n, e0n, e1n);
-      const uint32_t dst32 = wave_area32 + (uint32_t)((buf ^ 1) * bufsz);
-      // the next tile's copies (the last tile stages itself once more)
+      const uint32_t dst32 = wave_area32 + nxt_off;
+      // the next tile's copies (behind the unit's last tile: the tile after it, whatever it is, into the free buffer)
       if constexpr (NR >= 4) {
         stage_wide(hn, dst32);
       } else {
@@ -606,19 +616,23 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
           tile_window<NR, 1>(acc, pk, v, b);
         }
       };
-      uint2 cur = rec;
-      for (int base = e0; base < e1; base += kWave) {
-        const int left = e1 - base;
-        uint2 nxt = cur;
-        if (left > kWave) nxt = rec_load(base + kWave, e0, e1);
-        process(cur, left > kWave ? kWave : left);
-        cur = nxt;
+      // the first 64 records came with the last tile; a (tile, wave) with more loads the others here (few tiles have
+      // that many: the fullest ones are the dense tiles of the panel plan)
+      if (e1 > e0) process(rec, e1 - e0 < kWave ? e1 - e0 : kWave);
+      for (int base = e0 + kWave; base < e1; base += kWave) {
+        const uint2 more = rec_load(base, e0, e1);
+        process(more, e1 - base < kWave ? e1 - base : kWave);
       }
-      if constexpr (NR >= 4) stage_tail(hn, wave_area + (buf ^ 1) * bufsz);
+      if constexpr (NR >= 4) stage_tail(hn, wave_area + nxt_off);
       rec = recn;
       e0 = e0n;
       e1 = e1n;
       hn = hn2;
+      {
+        const uint32_t o = cur_off;
+        cur_off = nxt_off;
+        nxt_off = o;
+      }
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
     }

@@ -166,6 +166,86 @@ def test_spmm_panel_plan_random(cuda, knobs_restored, seed):
             lib.cg_tune_set(key, 0)
 
 
+TILE_KNOBS = [b"spmm_tile", b"spmm_panel", b"spmm_panel_legacy", b"spmm_panel_unit", b"spmm_panel_costcap",
+              b"spmm_strict_nonfinite", b"spmm_panel_dmin"]
+
+
+@pytest.mark.parametrize("seed", [41, 42])
+def test_spmm_tile_plans_random(cuda, knobs_restored, seed):
+    """The tile plans forced on (every entry through the tile kernel: panels of 256, 512 or 1024 rows by width, column
+    slices for wide products) and the panel plan with its staged tiles through either kernel, over random patterns,
+    widths of every register layout (1 .. 10 registers per row, one to four slices), both sides, accumulate forms,
+    leading dimensions that keep or break the alignment the kernel's copies need (such operands must come out right
+    through the other kernels), unit sizes, and a row of B made of infinities."""
+    from cagnet_amd import ops
+    lib = knobs_restored
+    rng = random.Random(seed)
+    try:
+        for case in range(120):
+            n = rng.choice([1, 15, 64, 255, 256, 257, 600, 1100, 2500])
+            m = rng.choice([16, 63, 64, 65, 300, 1000, 3001])
+            g = torch.Generator().manual_seed(rng.randrange(1 << 30))
+            if rng.random() < 0.6:
+                pr = torch.rand(n, 1, generator=g) ** 3
+                pc = torch.rand(1, m, generator=g) ** 3
+                mask = torch.rand(n, m, generator=g) < (pr * pc * rng.choice([0.5, 2.0, 8.0])).clamp(max=1.0)
+            else:
+                mask = torch.rand(n, m, generator=g) < rng.choice([0.01, 0.1, 0.6, 1.0])
+            if rng.random() < 0.5 and n > 2:
+                mask[rng.randrange(n)] = True
+                mask[:, rng.randrange(m)] = True
+            dense = torch.where(mask, torch.randn(n, m, generator=g), torch.zeros(()))
+            idx = mask.nonzero()
+            if idx.shape[0] == 0:
+                continue
+            row, col, val = idx[:, 0].int().to(cuda), idx[:, 1].int().to(cuda), dense[mask].to(cuda)
+            f = rng.choice([4, 8, 16, 44, 48, 64, 65, 66, 96, 100, 128, 130, 192, 256, 258, 300, 316, 320, 384, 500, 512, 514,
+                            602, 636, 640, 700, 950, 1000, 1300])
+            mode = rng.choice(["tile", "tile", "panel", "panel_legacy"])
+            values = {b"spmm_tile": 1 if mode == "tile" else -1, b"spmm_panel": 1 if mode != "tile" else 0,
+                      b"spmm_panel_legacy": 1 if mode == "panel_legacy" else 0,
+                      b"spmm_panel_unit": rng.choice([0, 0, 64, 1000, 20000]), b"spmm_panel_costcap": rng.choice([0, 0, 1, 50]),
+                      b"spmm_strict_nonfinite": 0, b"spmm_panel_dmin": rng.choice([0, 40, -1])}
+            tr = rng.random() < 0.4
+            beta = rng.choice([0.0, 1.0, -0.5])
+            extra_b, extra_c = rng.choice([0, 0, 2, 4, 1, 3]), rng.choice([0, 0, 2, 4])
+            with_inf = rng.random() < 0.15
+            if with_inf:
+                values[b"spmm_strict_nonfinite"] = 1          # entry-by-entry semantics: the fp64 product is the oracle
+            for key, v in values.items():
+                assert lib.cg_tune_set(key, v) == 0
+            what = (f"seed {seed} case {case}: n={n} m={m} nnz={val.numel()} f={f} mode={mode} tr={tr} beta={beta} "
+                    f"ld+{extra_b}/{extra_c} inf={with_inf} knobs={values}")
+            gen = torch.Generator(device=cuda).manual_seed(case)
+            B = _strided(n if tr else m, f, extra_b, gen, cuda)
+            C0 = torch.randn(m if tr else n, f, device=cuda, generator=gen)
+            A64 = dense.double().to(cuda)
+            A64 = A64.t() if tr else A64
+            if with_inf:
+                # a row of B that no entry refers to holds infinities: they must reach no row of C
+                unused = (A64 != 0).sum(0) == 0
+                if bool(unused.any()):
+                    B[int(unused.nonzero()[0])] = float("inf")
+                else:
+                    with_inf = False
+            A = ops.CsrMatrix(row, col, val, n, m, is_sorted=True, transpose=tr)
+            outs = []
+            for _ in range(2):
+                C = torch.empty(C0.shape[0], f + extra_c, device=cuda)[:, :f].copy_(C0)
+                A.spmm(B, out=C, beta=beta, transpose=tr)
+                outs.append(C)
+            Bf = torch.where(torch.isfinite(B), B, torch.zeros((), device=cuda)).double()
+            ref = beta * C0.double() + A64 @ Bf
+            mag = abs(beta) * C0.double().abs() + A64.abs() @ Bf.abs()
+            assert torch.isfinite(outs[0]).all(), what
+            assert _rel(outs[0], ref, mag) <= REL_TOL, what
+            assert torch.equal(outs[0], outs[1]), what
+            del A
+    finally:
+        for key in TILE_KNOBS:
+            lib.cg_tune_set(key, 0)
+
+
 @pytest.mark.parametrize("seed", [21, 22])
 def test_dense_and_rowwise_random(cuda, knobs_restored, seed):
     """The three dense products (both kernel families) on strided operands and outputs, and the
