@@ -32,7 +32,7 @@ HIPCC_FLAGS = [
     "-Wall",
     "-Wno-unused-function",
     "-Wno-unknown-warning-option",
-    "-Wno-inline-asm",  # the asm statements that set m0 name it as clobbered; clang notes that it is a reserved register
+    "-Wno-inline-asm", "-Wno-int-to-pointer-cast",  # the asm statements that set m0 name it as clobbered; clang notes that it is a reserved register
 ]
 
 
