@@ -562,11 +562,17 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
       hdr_lane += kPanelWaves * HS;
       const uint2 recn = rec_load(e0n, e0n, e1n);
       const uint32_t dst32 = wave_area32 + nxt_off;
-      // the next tile's copies (behind the unit's last tile: the tile after it, whatever it is, into the free buffer)
+      // The next tile's copies (behind the unit's last tile: the tile after it, whatever it is, into the free buffer).
+      // A wave cannot go on before the memory pipeline has taken its copy instructions, and that pipeline takes one
+      // (1 KiB) in about 17 cycles: with all 16 waves issuing their copies at the start of a tile nobody multiplied
+      // until the tile's 96 copies were nearly through (cycle counters: 800 cycles per wave in the six copies).  So two
+      // of a SIMD's four waves issue theirs behind their records: they multiply while the other two's copies are
+      // taken, and the other way round.  (Four different points instead of two: no better.)
+      const bool copies_first = ((wave >> 2) & 1) == 0;  // (waves w, w + 4, w + 8, w + 12 share a SIMD)
       if constexpr (NR >= 4) {
-        stage_wide(hn, dst32);
+        if (copies_first) stage_wide(hn, dst32);
       } else {
-        stage_narrow(hn, dst32);
+        if (copies_first) stage_narrow(hn, dst32);
       }
 
       // cnt records in the lanes of r.  K records at a time: their rows of B are read from LDS, then one stretch of
@@ -622,6 +628,11 @@ __global__ __launch_bounds__(kPanelThreads) void spmm_tile_kernel(const TileArgs
       for (int base = e0 + kWave; base < e1; base += kWave) {
         const uint2 more = rec_load(base, e0, e1);
         process(more, e1 - base < kWave ? e1 - base : kWave);
+      }
+      if constexpr (NR >= 4) {
+        if (!copies_first) stage_wide(hn, dst32);
+      } else {
+        if (!copies_first) stage_narrow(hn, dst32);
       }
       if constexpr (NR >= 4) stage_tail(hn, wave_area + nxt_off);
       rec = recn;
