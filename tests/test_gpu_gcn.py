@@ -167,6 +167,45 @@ def test_fused_stage_loop_matches_oracle_stage_loop(cuda, monkeypatch, width):
     assert orc.max_rel_error(out[:, :width], ref, mag) <= REL_TOL and bool((out[:, width:] == 7.0).all())
 
 
+def test_hstack_edge_cases(cuda):
+    """cg_csr_hstack: a single block, blocks without entries, rows without entries, the transpose of the stacked
+    matrix, and the refusals (blocks of different heights, more than 16 blocks)."""
+    from cagnet_amd import ops
+    from cagnet_amd._lib import CagnetError
+    gen = torch.Generator().manual_seed(5)
+    rows = 37
+
+    def block(m, density):
+        mask = torch.rand(rows, m, generator=gen) < density
+        mask[5] = False                                                  # a row without entries in every block
+        idx = mask.nonzero()
+        val = torch.randn(idx.shape[0], generator=gen)
+        d = torch.zeros(rows, m)
+        d[mask] = val
+        return ops.CsrMatrix(idx[:, 0].int().to(cuda), idx[:, 1].int().to(cuda), val.to(cuda), rows, m), d
+
+    parts = [block(11, 0.3), block(1, 0.0), block(64, 0.1), block(7, 1.0)]
+    S = ops.CsrMatrix.hstack([p[0] for p in parts], transpose=True)
+    dense = torch.cat([p[1] for p in parts], dim=1)
+    assert (S.n, S.m, S.nnz) == (rows, 83, int((dense != 0).sum()))
+    B = torch.randn(83, 9, generator=gen)
+    got = S.spmm(B.to(cuda)).cpu()
+    assert torch.allclose(got, dense @ B, atol=1e-5) and bool((got[5] == 0).all())
+    G = torch.randn(rows, 5, generator=gen)
+    assert torch.allclose(S.spmm(G.to(cuda), transpose=True).cpu(), dense.t() @ G, atol=1e-5)
+    one = ops.CsrMatrix.hstack([parts[0][0]])
+    assert torch.equal(one.spmm(B[:11].to(cuda).contiguous()), parts[0][0].spmm(B[:11].to(cuda).contiguous()))
+    other = ops.CsrMatrix(torch.zeros(1, dtype=torch.int32, device=cuda), torch.zeros(1, dtype=torch.int32, device=cuda),
+                          torch.ones(1, device=cuda), rows + 1, 4)
+    with pytest.raises(CagnetError):
+        ops.CsrMatrix.hstack([parts[0][0], other])
+    with pytest.raises(CagnetError):
+        ops.CsrMatrix.hstack([parts[0][0]] * 17)
+    with pytest.raises(ValueError):
+        ops.CsrMatrix.hstack([])
+    assert ops.CsrMatrix.hstack([parts[0][0]] * 16).m == 11 * 16
+
+
 def test_one_rank_share_of_2d_grid(cuda):
     """One rank's share of the 4x4 2D algorithm (gcn_distr_2d.py:333-417) with the broadcast
     operands resident: z = sum_k A(r,k) H_k over 4 stages, both layers, forward and backward."""
