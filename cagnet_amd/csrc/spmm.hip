@@ -383,7 +383,10 @@ static int spmm_side(CsrSide &s, const float *B, int64_t ldb, float *C, int64_t 
     PanelParams par = panel_params();
     // The staged tiles go through spmm_tile_kernel, which takes the records as they are; the older spmm_panel_kernel
     // (records of a run padded to pairs) serves operands that kernel cannot read and the tuning value.
-    par.padded = g_tune_panel_legacy.load(std::memory_order_relaxed) > 0 || !tile_operands_ok(par.prows, par.tcols, B, ldb, f, s.cols);
+    // (also for the last widths two of whose tiles the tile kernel's LDS layout has no room for: it would take them in two slices)
+    TileShape one;
+    par.padded = g_tune_panel_legacy.load(std::memory_order_relaxed) > 0 || !tile_operands_ok(par.prows, par.tcols, B, ldb, f, s.cols) ||
+                 !tile_shape(par.prows, par.tcols, f, one) || one.nsl != 1;
     const bool may_decline = g_tune_panel.load(std::memory_order_relaxed) == 0;
     PanelPlan &pp = s.panel;
     if (!pp.valid || !par.same(pp) || (pp.declined && !may_decline && !pp.failed)) {

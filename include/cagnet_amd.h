@@ -382,7 +382,8 @@ int cg_prof_enable(int on);
  *                     in named registers and takes the records of a (tile, wave, row) run in pairs, padded; 0: through
  *                     the tile kernel (accumulators addressed through the register index, records as they are).  A B
  *                     that is not 8-byte aligned or has an odd leading dimension goes to the older kernel whatever
- *                     this says: the tile kernel's copies need 8-byte aligned rows
+ *                     this says (the tile kernel's copies need 8-byte aligned rows), and so do the widths 634 and 636,
+ *                     two of whose tiles the tile kernel's LDS layout has no room for
  *   "spmm_tile"       tile plans (every entry multiplied out of LDS by the tile kernel; panels of 256 rows and
  *                     column slices of up to 316 columns for widths above 128, 512 rows for 65..128, 1024 rows up
  *                     to 64): -1 never, 1 always, 0 by width and matrix: widths from 65 on except the even widths
